@@ -1,0 +1,448 @@
+// k_ew.hip — fused elementwise programs and last-axis reductions for gfx950.
+//
+// Serves Backend::{add,sub,mul,div,pow,lt,eq,sin,cos,neg,cast,broadcast,zeros,arange} and the
+// materialising forms of reshape/transpose/slice/concat (one strided pass), and
+// Backend::{sum,max,argmax} with an optional elementwise prologue
+// (catgrad/src/interpreter/backend/mod.rs:26-57; semantics: ndarray.rs:97-114, 164-246, 401-493).
+//
+// All of these are HBM-bound.  The kernels therefore (a) read each operand through its own
+// strides so views are never materialised, (b) move 16 bytes per lane whenever the innermost
+// stride allows it, (c) use grid-stride loops sized to the 256 CUs, and (d) evaluate a whole
+// expression tree per element so intermediates never touch memory.
+//
+// The evaluator is a stack machine whose stack lives in VGPRs: every instruction carries the
+// stack depth at which it runs, so register indices are compile-time constants inside a
+// wave-uniform switch (no scratch memory, no divergence).
+#include <hip/hip_runtime.h>
+#include <math.h>
+#include "program.hpp"
+#include "launch.hpp"
+
+namespace cgk {
+
+__device__ __forceinline__ float as_f(uint32_t u) { return __uint_as_float(u); }
+__device__ __forceinline__ uint32_t as_u(float f) { return __float_as_uint(f); }
+
+// Rust `f32 as u32`: truncate toward zero, saturate, NaN -> 0 (ndarray.rs:101)
+__device__ __forceinline__ uint32_t f2u_sat(float v) {
+  if (!(v == v) || v <= 0.f) return 0u;
+  if (v >= 4294967296.f) return 0xFFFFFFFFu;
+  return (uint32_t)v;
+}
+
+__device__ __forceinline__ uint32_t upow(uint32_t a, uint32_t e) {
+  uint32_t r = 1;
+  while (e) {
+    if (e & 1) r *= a;
+    a *= a;
+    e >>= 1;
+  }
+  return r;
+}
+
+__device__ __forceinline__ uint32_t f32_to_bf16_rne(uint32_t u) {
+  if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (u >> 16) | 0x40u;  // quiet NaN
+  return (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
+}
+
+// pow(x, 0.5) with powf's answers at the points where sqrtf differs
+__device__ __forceinline__ float sqrt_like_pow(float x) {
+  if (x == 0.f) return 0.f;
+  if (x == -INFINITY) return INFINITY;
+  return sqrtf(x);
+}
+
+__device__ __forceinline__ uint32_t apply_bin(uint8_t op, uint32_t a, uint32_t b, uint32_t *err) {
+  switch (op) {
+    case E_ADD_F: return as_u(as_f(a) + as_f(b));
+    case E_SUB_F: return as_u(as_f(a) - as_f(b));
+    case E_MUL_F: return as_u(as_f(a) * as_f(b));
+    case E_DIV_F: return as_u(as_f(a) / as_f(b));
+    case E_POW_F: return as_u(powf(as_f(a), as_f(b)));
+    case E_LT_F: return as_u(as_f(a) < as_f(b) ? 1.f : 0.f);
+    case E_EQ_F: return as_u(as_f(a) == as_f(b) ? 1.f : 0.f);
+    case E_ADD_U: return a + b;
+    case E_SUB_U: return a - b;
+    case E_MUL_U: return a * b;
+    case E_DIV_U:
+      if (b == 0u) {
+        atomicOr(err, ERRF_DIV_ZERO);
+        return 0xFFFFFFFFu;
+      }
+      return a / b;
+    case E_POW_U: return upow(a, b);
+    case E_LT_U: return a < b ? 1u : 0u;
+    case E_EQ_U: return a == b ? 1u : 0u;
+    default: return 0u;
+  }
+}
+
+__device__ __forceinline__ uint32_t apply_un(uint8_t op, uint32_t a) {
+  switch (op) {
+    case E_NEG_F: return a ^ 0x80000000u;
+    case E_NEG_U: return 0u - a;
+    case E_SIN_F: return as_u(sinf(as_f(a)));
+    case E_COS_F: return as_u(cosf(as_f(a)));
+    case E_F2U: return f2u_sat(as_f(a));
+    case E_U2F: return as_u((float)a);
+    case E_EXP_F: return as_u(expf(as_f(a)));
+    case E_SQRT_F: return as_u(sqrt_like_pow(as_f(a)));
+    case E_CUBE_F: { float x = as_f(a); return as_u(x * x * x); }
+    case E_RCP_F: return as_u(1.0f / as_f(a));
+    default: return 0u;
+  }
+}
+
+template <int VEC>
+__device__ __forceinline__ void load_operand(const Operand &in, const uint32_t (&idx)[MAX_DIMS],
+                                             int n_dims, uint32_t (&v)[VEC]) {
+  int64_t off = 0;
+#pragma unroll
+  for (int d = 0; d < MAX_DIMS; ++d)
+    if (d < n_dims) off += (int64_t)idx[d] * in.stride[d];
+  const int64_t inner = in.stride[n_dims - 1];
+  if (in.stype == ST_BF16) {
+    const uint16_t *p = (const uint16_t *)in.ptr + off;
+    if (VEC == 4 && in.vec) {
+      uint2 q = *(const uint2 *)p;
+      v[0] = q.x << 16; v[1 % VEC] = q.x & 0xFFFF0000u;
+      v[2 % VEC] = q.y << 16; v[3 % VEC] = q.y & 0xFFFF0000u;
+    } else {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) v[j] = (uint32_t)p[j * inner] << 16;
+    }
+  } else {
+    const uint32_t *p = (const uint32_t *)in.ptr + off;
+    if (VEC == 4 && in.vec) {
+      uint4 q = *(const uint4 *)p;
+      v[0] = q.x; v[1 % VEC] = q.y; v[2 % VEC] = q.z; v[3 % VEC] = q.w;
+    } else if (inner == 0) {
+      uint32_t s = p[0];
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) v[j] = s;
+    } else {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) v[j] = p[j * inner];
+    }
+  }
+}
+
+#define CG_DEPTHS(M) \
+  case 0: M(0) break; case 1: M(1) break; case 2: M(2) break; case 3: M(3) break; \
+  case 4: M(4) break; case 5: M(5) break; case 6: M(6) break; case 7: M(7) break;
+
+// Evaluate the program for VEC consecutive elements along the innermost dim.
+template <int VEC>
+__device__ __forceinline__ void eval_program(const Program &p, const uint32_t (&idx)[MAX_DIMS],
+                                             uint32_t lin, uint32_t *err, uint32_t (&res)[VEC]) {
+  uint32_t r[MAX_STACK][VEC];
+  for (int pc = 0; pc < p.n_instr; ++pc) {
+    const Instr ins = p.code[pc];
+    if (ins.op <= E_IOTA) {
+      uint32_t t[VEC];
+      if (ins.op == E_LOAD) {
+        load_operand<VEC>(p.in[ins.arg], idx, p.n_dims, t);
+      } else if (ins.op == E_CONST) {
+        uint32_t c = p.imm[ins.arg];
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) t[j] = c;
+      } else {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) t[j] = lin + j;
+      }
+      switch (ins.depth) {
+#define M(d) _Pragma("unroll") for (int j = 0; j < VEC; ++j) r[d][j] = t[j];
+        CG_DEPTHS(M)
+#undef M
+      }
+    } else if (ins.op <= E_EQ_U) {
+      uint32_t a[VEC], b[VEC];
+      switch (ins.depth) {
+#define M(d) _Pragma("unroll") for (int j = 0; j < VEC; ++j) { \
+    a[j] = r[(d) >= 2 ? (d)-2 : 0][j]; b[j] = r[(d) >= 1 ? (d)-1 : 0][j]; }
+        CG_DEPTHS(M)
+#undef M
+      }
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) a[j] = apply_bin(ins.op, a[j], b[j], err);
+      switch (ins.depth) {
+#define M(d) _Pragma("unroll") for (int j = 0; j < VEC; ++j) r[(d) >= 2 ? (d)-2 : 0][j] = a[j];
+        CG_DEPTHS(M)
+#undef M
+      }
+    } else {
+      uint32_t a[VEC];
+      switch (ins.depth) {
+#define M(d) _Pragma("unroll") for (int j = 0; j < VEC; ++j) a[j] = r[(d) >= 1 ? (d)-1 : 0][j];
+        CG_DEPTHS(M)
+#undef M
+      }
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) a[j] = apply_un(ins.op, a[j]);
+      switch (ins.depth) {
+#define M(d) _Pragma("unroll") for (int j = 0; j < VEC; ++j) r[(d) >= 1 ? (d)-1 : 0][j] = a[j];
+        CG_DEPTHS(M)
+#undef M
+      }
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) res[j] = r[0][j];
+}
+
+__device__ __forceinline__ void decompose(const Program &p, uint64_t lin,
+                                          uint32_t (&idx)[MAX_DIMS]) {
+  // all programs stay below 2^32 elements (checked on the host)
+  uint32_t rem = (uint32_t)lin;
+#pragma unroll
+  for (int d = MAX_DIMS - 1; d >= 0; --d) {
+    if (d < p.n_dims) {
+      if (d == 0) {
+        idx[d] = rem;
+      } else {
+        uint32_t q = rem / p.dims[d];
+        idx[d] = rem - q * p.dims[d];
+        rem = q;
+      }
+    } else {
+      idx[d] = 0;
+    }
+  }
+}
+
+template <int VEC>
+__global__ void __launch_bounds__(256) ew_kernel(Program p, OutDesc o, uint64_t n_groups,
+                                                 uint32_t *err) {
+  for (uint64_t g = (uint64_t)blockIdx.x * 256 + threadIdx.x; g < n_groups;
+       g += (uint64_t)gridDim.x * 256) {
+    uint32_t idx[MAX_DIMS];
+    const uint64_t lin = g * VEC;
+    decompose(p, lin, idx);
+    uint32_t v[VEC];
+    eval_program<VEC>(p, idx, (uint32_t)lin, err, v);
+    int64_t off = 0;
+#pragma unroll
+    for (int d = 0; d < MAX_DIMS; ++d)
+      if (d < p.n_dims) off += (int64_t)idx[d] * o.stride[d];
+    const int64_t inner = o.stride[p.n_dims - 1];
+    if (o.stype == ST_BF16) {
+      uint16_t *q = (uint16_t *)o.ptr + off;
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) q[j * inner] = (uint16_t)f32_to_bf16_rne(v[j]);
+    } else {
+      uint32_t *q = (uint32_t *)o.ptr + off;
+      if (VEC == 4 && o.vec) {
+        *(uint4 *)q = make_uint4(v[0], v[1 % VEC], v[2 % VEC], v[3 % VEC]);
+      } else {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) q[j * inner] = v[j];
+      }
+    }
+  }
+}
+
+// ---- reductions over the innermost program dim -------------------------------------------------
+
+// f32::total_cmp key (monotone signed integer)
+__device__ __forceinline__ int32_t total_key(uint32_t bits) {
+  int32_t b = (int32_t)bits;
+  return b ^ (int32_t)(((uint32_t)(b >> 31)) >> 1);
+}
+
+template <int KIND> struct Acc;
+// Every accumulator exposes its state as W 32-bit words (for shuffles and LDS), without
+// type punning.
+template <> struct Acc<R_SUM_F> {
+  enum { W = 1 };
+  float v = 0.f;
+  __device__ void add(uint32_t x, uint32_t) { v += as_f(x); }
+  __device__ void merge(const Acc &o) { v += o.v; }
+  __device__ uint32_t result() const { return as_u(v); }
+  __device__ void get(uint32_t *w) const { w[0] = as_u(v); }
+  __device__ void set(const uint32_t *w) { v = as_f(w[0]); }
+};
+template <> struct Acc<R_SUM_U> {
+  enum { W = 1 };
+  uint32_t v = 0;
+  __device__ void add(uint32_t x, uint32_t) { v += x; }
+  __device__ void merge(const Acc &o) { v += o.v; }
+  __device__ uint32_t result() const { return v; }
+  __device__ void get(uint32_t *w) const { w[0] = v; }
+  __device__ void set(const uint32_t *w) { v = w[0]; }
+};
+// fold(f32::MIN, f32::max): NaN ignored, floor at f32::MIN (ndarray.rs:455-460)
+template <> struct Acc<R_MAX_F> {
+  enum { W = 1 };
+  float v = -3.40282347e+38f;
+  __device__ void add(uint32_t x, uint32_t) { v = fmaxf(v, as_f(x)); }
+  __device__ void merge(const Acc &o) { v = fmaxf(v, o.v); }
+  __device__ uint32_t result() const { return as_u(v); }
+  __device__ void get(uint32_t *w) const { w[0] = as_u(v); }
+  __device__ void set(const uint32_t *w) { v = as_f(w[0]); }
+};
+template <> struct Acc<R_MAX_U> {
+  enum { W = 1 };
+  uint32_t v = 0;
+  __device__ void add(uint32_t x, uint32_t) { v = x > v ? x : v; }
+  __device__ void merge(const Acc &o) { v = o.v > v ? o.v : v; }
+  __device__ uint32_t result() const { return v; }
+  __device__ void get(uint32_t *w) const { w[0] = v; }
+  __device__ void set(const uint32_t *w) { v = w[0]; }
+};
+// max_by(total_cmp): the LAST of equal maxima wins (ndarray.rs:469-480).  `any` = 0 marks an
+// accumulator that has seen no element yet.
+template <> struct Acc<R_ARGMAX_F> {
+  enum { W = 3 };
+  int32_t k = INT32_MIN;
+  uint32_t i = 0, any = 0;
+  __device__ void add(uint32_t x, uint32_t col) {
+    int32_t kk = total_key(x);
+    if (!any || kk > k || (kk == k && col > i)) { k = kk; i = col; any = 1; }
+  }
+  __device__ void merge(const Acc &o) {
+    if (o.any && (!any || o.k > k || (o.k == k && o.i > i))) { k = o.k; i = o.i; any = 1; }
+  }
+  __device__ uint32_t result() const { return i; }
+  __device__ void get(uint32_t *w) const { w[0] = (uint32_t)k; w[1] = i; w[2] = any; }
+  __device__ void set(const uint32_t *w) { k = (int32_t)w[0]; i = w[1]; any = w[2]; }
+};
+template <> struct Acc<R_ARGMAX_U> {
+  enum { W = 3 };
+  uint32_t k = 0, i = 0, any = 0;
+  __device__ void add(uint32_t x, uint32_t col) {
+    if (!any || x > k || (x == k && col > i)) { k = x; i = col; any = 1; }
+  }
+  __device__ void merge(const Acc &o) {
+    if (o.any && (!any || o.k > k || (o.k == k && o.i > i))) { k = o.k; i = o.i; any = 1; }
+  }
+  __device__ uint32_t result() const { return i; }
+  __device__ void get(uint32_t *w) const { w[0] = k; w[1] = i; w[2] = any; }
+  __device__ void set(const uint32_t *w) { k = w[0]; i = w[1]; any = w[2]; }
+};
+
+template <int KIND>
+__device__ __forceinline__ Acc<KIND> shfl_xor_acc(const Acc<KIND> &a, int m) {
+  uint32_t w[Acc<KIND>::W];
+  a.get(w);
+#pragma unroll
+  for (int j = 0; j < Acc<KIND>::W; ++j) w[j] = (uint32_t)__shfl_xor((int)w[j], m, 64);
+  Acc<KIND> r;
+  r.set(w);
+  return r;
+}
+
+// One row per workgroup (WAVES_PER_ROW = 4) or per wavefront (WAVES_PER_ROW = 1).
+template <int KIND, int VEC, int WAVES_PER_ROW>
+__global__ void __launch_bounds__(256) reduce_kernel(Program p, uint32_t *out, uint32_t rows,
+                                                     uint32_t n, uint32_t *err) {
+  __shared__ uint32_t part[4][Acc<KIND>::W];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const uint32_t rows_per_block = 4 / WAVES_PER_ROW;
+  const uint32_t tid_in_row = WAVES_PER_ROW == 4 ? threadIdx.x : lane;
+  const uint32_t threads_per_row = WAVES_PER_ROW * 64;
+  for (uint32_t rb = blockIdx.x * rows_per_block; rb < rows; rb += gridDim.x * rows_per_block) {
+    const uint32_t row = rb + (WAVES_PER_ROW == 4 ? 0 : wave);
+    Acc<KIND> acc;
+    if (row < rows) {
+      uint32_t idx[MAX_DIMS];
+      // outer coordinates: decompose the row number over dims[0 .. n_dims-2]
+      uint32_t rem = row;
+#pragma unroll
+      for (int d = MAX_DIMS - 2; d >= 0; --d) {
+        if (d < p.n_dims - 1) {
+          if (d == 0) {
+            idx[d] = rem;
+          } else {
+            uint32_t q = rem / p.dims[d];
+            idx[d] = rem - q * p.dims[d];
+            rem = q;
+          }
+        } else {
+          idx[d] = 0;
+        }
+      }
+      idx[MAX_DIMS - 1] = 0;
+      for (uint32_t c = tid_in_row * VEC; c < n; c += threads_per_row * VEC) {
+        // the innermost coordinate lives at position n_dims-1
+#pragma unroll
+        for (int d = 0; d < MAX_DIMS; ++d)
+          if (d == p.n_dims - 1) idx[d] = c;
+        uint32_t v[VEC];
+        eval_program<VEC>(p, idx, c, err, v);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) acc.add(v[j], c + j);
+      }
+    }
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) acc.merge(shfl_xor_acc<KIND>(acc, m));
+    if (WAVES_PER_ROW == 4) {
+      __syncthreads();
+      if (lane == 0) acc.get(part[wave]);
+      __syncthreads();
+      if (threadIdx.x == 0) {
+        for (int w2 = 1; w2 < 4; ++w2) {
+          Acc<KIND> o;
+          o.set(part[w2]);
+          acc.merge(o);
+        }
+        out[row] = acc.result();
+      }
+    } else if (lane == 0 && row < rows) {
+      out[row] = acc.result();
+    }
+  }
+}
+
+// ---- host launchers --------------------------------------------------------------------------
+
+static inline unsigned grid_for(uint64_t blocks_needed, const LaunchCtx &lc) {
+  uint64_t cap = (uint64_t)lc.n_cus * 8;
+  uint64_t g = blocks_needed < cap ? blocks_needed : cap;
+  return (unsigned)(g ? g : 1);
+}
+
+hipError_t launch_ew(const LaunchCtx &lc, const Program &p, const OutDesc &o, uint64_t n_elems,
+                     bool vec4) {
+  if (n_elems == 0) return hipSuccess;
+  if (vec4) {
+    uint64_t groups = n_elems / 4;
+    ew_kernel<4><<<grid_for((groups + 255) / 256, lc), 256, 0, lc.stream>>>(p, o, groups, lc.err_flag);
+  } else {
+    ew_kernel<1><<<grid_for((n_elems + 255) / 256, lc), 256, 0, lc.stream>>>(p, o, n_elems,
+                                                                             lc.err_flag);
+  }
+  return hipGetLastError();
+}
+
+template <int KIND>
+static hipError_t launch_reduce_kind(const LaunchCtx &lc, const Program &p, uint32_t *out,
+                                     uint32_t rows, uint32_t n, bool vec4) {
+  const bool block_per_row = n >= 2048;
+  if (block_per_row) {
+    unsigned g = grid_for(rows, lc);
+    if (vec4) reduce_kernel<KIND, 4, 4><<<g, 256, 0, lc.stream>>>(p, out, rows, n, lc.err_flag);
+    else reduce_kernel<KIND, 1, 4><<<g, 256, 0, lc.stream>>>(p, out, rows, n, lc.err_flag);
+  } else {
+    unsigned g = grid_for((rows + 3) / 4, lc);
+    if (vec4) reduce_kernel<KIND, 4, 1><<<g, 256, 0, lc.stream>>>(p, out, rows, n, lc.err_flag);
+    else reduce_kernel<KIND, 1, 1><<<g, 256, 0, lc.stream>>>(p, out, rows, n, lc.err_flag);
+  }
+  return hipGetLastError();
+}
+
+hipError_t launch_reduce(const LaunchCtx &lc, int kind, const Program &p, void *out, uint32_t rows,
+                         uint32_t n, bool vec4) {
+  if (rows == 0) return hipSuccess;
+  uint32_t *o = (uint32_t *)out;
+  switch (kind) {
+    case R_SUM_F: return launch_reduce_kind<R_SUM_F>(lc, p, o, rows, n, vec4);
+    case R_SUM_U: return launch_reduce_kind<R_SUM_U>(lc, p, o, rows, n, vec4);
+    case R_MAX_F: return launch_reduce_kind<R_MAX_F>(lc, p, o, rows, n, vec4);
+    case R_MAX_U: return launch_reduce_kind<R_MAX_U>(lc, p, o, rows, n, vec4);
+    case R_ARGMAX_F: return launch_reduce_kind<R_ARGMAX_F>(lc, p, o, rows, n, vec4);
+    case R_ARGMAX_U: return launch_reduce_kind<R_ARGMAX_U>(lc, p, o, rows, n, vec4);
+  }
+  return hipErrorInvalidValue;
+}
+
+}  // namespace cgk

@@ -1,0 +1,469 @@
+// k_gemm.hip — batched matmul for gfx950: MFMA GEMM (LDS-tiled), row-dot and column GEMV.
+//
+// Backend::matmul (mod.rs:41; ndarray.rs:549-615): (N.., A, B) x (N.., B, C) -> (N.., A, C).
+// Operands arrive as strided views, never copies: a `linear` weight W[out, in] reaches matmul
+// as transpose(0,1) + reshape([1, in, out]) (stdlib/nn/mod.rs:182-192), i.e. B[k, n] with
+// stride 1 along k — the "NT" layout both MFMA operands want.  K^T of attention has the same
+// layout; V and rank-2 user matmuls have stride 1 along n.
+//
+//  * gemm_kernel: 128x128 output tile per 256-thread workgroup, four wavefronts in a 2x2 grid,
+//    each owning 64x64 = 2x2 MFMA 32x32 accumulators (64 VGPRs).  Tiles are staged through LDS
+//    k-contiguous for both operands; global loads for step i+1 are issued before the MFMAs of
+//    step i.  bf16 mode: operands rounded to bf16 on the way into LDS, v_mfma_f32_32x32x16_bf16.
+//    f32 mode: v_mfma_f32_32x32x2_f32 (gfx950 has no xf32).  MFMA-bound for M >= 64.
+//  * gemv_rowdot_kernel (M <= 8, B k-contiguous): the decode path.  HBM-bound on the weight
+//    matrix: every lane streams 16 bytes per load, a group of lanes owns one output column,
+//    partial dots meet in a DPP/shuffle reduction; x stays in L2/registers.
+//  * gemv_col_kernel (M <= 8, B n-contiguous): lanes across n, k split over the workgroup.
+#include <hip/hip_runtime.h>
+#include "launch.hpp"
+
+namespace cgk {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+
+__device__ __forceinline__ uint32_t bf16_rne(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (u >> 16) | 0x40u;
+  return (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
+}
+__device__ __forceinline__ float widen(float v) { return v; }
+__device__ __forceinline__ float widen(uint16_t v) { return __uint_as_float((uint32_t)v << 16); }
+
+// ---- tile loading -------------------------------------------------------------------------
+// Eight consecutive elements of a [rows, K] operand tile, either along k (KC) or along the row
+// axis (!KC), zero-filled out of bounds, widened to f32.
+template <typename T, bool KC>
+__device__ __forceinline__ void load8(const T *base, int64_t s_row, int64_t s_k, uint32_t row,
+                                      uint32_t k, uint32_t n_rows, uint32_t K, bool vec,
+                                      float (&v)[8]) {
+  if (KC) {
+    const T *p = base + (int64_t)row * s_row + k;
+    if (row < n_rows && k + 8 <= K && vec) {
+      if (sizeof(T) == 4) {
+        float4 q0 = *(const float4 *)p, q1 = *(const float4 *)(p + 4);
+        v[0] = q0.x; v[1] = q0.y; v[2] = q0.z; v[3] = q0.w;
+        v[4] = q1.x; v[5] = q1.y; v[6] = q1.z; v[7] = q1.w;
+      } else {
+        uint4 q = *(const uint4 *)p;
+        v[0] = __uint_as_float(q.x << 16); v[1] = __uint_as_float(q.x & 0xFFFF0000u);
+        v[2] = __uint_as_float(q.y << 16); v[3] = __uint_as_float(q.y & 0xFFFF0000u);
+        v[4] = __uint_as_float(q.z << 16); v[5] = __uint_as_float(q.z & 0xFFFF0000u);
+        v[6] = __uint_as_float(q.w << 16); v[7] = __uint_as_float(q.w & 0xFFFF0000u);
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v[j] = (row < n_rows && k + j < K) ? widen(p[j]) : 0.f;
+    }
+  } else {
+    const T *p = base + (int64_t)k * s_k + row;
+    if (k < K && row + 8 <= n_rows && vec) {
+      if (sizeof(T) == 4) {
+        float4 q0 = *(const float4 *)p, q1 = *(const float4 *)(p + 4);
+        v[0] = q0.x; v[1] = q0.y; v[2] = q0.z; v[3] = q0.w;
+        v[4] = q1.x; v[5] = q1.y; v[6] = q1.z; v[7] = q1.w;
+      } else {
+        uint4 q = *(const uint4 *)p;
+        v[0] = __uint_as_float(q.x << 16); v[1] = __uint_as_float(q.x & 0xFFFF0000u);
+        v[2] = __uint_as_float(q.y << 16); v[3] = __uint_as_float(q.y & 0xFFFF0000u);
+        v[4] = __uint_as_float(q.z << 16); v[5] = __uint_as_float(q.z & 0xFFFF0000u);
+        v[6] = __uint_as_float(q.w << 16); v[7] = __uint_as_float(q.w & 0xFFFF0000u);
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v[j] = (k < K && row + j < n_rows) ? widen(p[j]) : 0.f;
+    }
+  }
+}
+
+template <bool BF16> struct Tile;
+template <> struct Tile<true> {
+  enum { BK = 32, LD = 40 };  // row pitch 80 bytes: 16-byte aligned, spreads banks
+  typedef uint16_t LT;
+};
+template <> struct Tile<false> {
+  enum { BK = 16, LD = 20 };  // row pitch 80 bytes
+  typedef float LT;
+};
+
+enum { BM = 128, BN = 128 };
+
+template <typename TA, typename TB, bool A_KC, bool B_KC, bool BF16>
+__global__ void __launch_bounds__(256) gemm_kernel(GemmDesc g, int a_vec, int b_vec) {
+  typedef Tile<BF16> TL;
+  typedef typename TL::LT LT;
+  constexpr int BK = TL::BK, LD = TL::LD;
+  constexpr int CPT = BM * BK / 8 / 256;  // 8-element chunks per thread per operand tile
+  __shared__ __attribute__((aligned(16))) LT As[BM * LD];
+  __shared__ __attribute__((aligned(16))) LT Bs[BN * LD];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const uint32_t m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+  const uint32_t bz = blockIdx.z, b0 = bz / g.nb1, b1 = bz - b0 * g.nb1;
+  const TA *A = (const TA *)g.a + b0 * g.sa_b0 + b1 * g.sa_b1;
+  const TB *B = (const TB *)g.b + b0 * g.sb_b0 + b1 * g.sb_b1;
+  float *C = g.c + (uint64_t)bz * g.M * g.N;
+
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  float ra[CPT][8], rb[CPT][8];
+
+  auto fetch = [&](uint32_t k0) {
+#pragma unroll
+    for (int c = 0; c < CPT; ++c) {
+      const int chunk = tid + c * 256;
+      if (A_KC) {
+        const int row = chunk / (BK / 8), kc = (chunk % (BK / 8)) * 8;
+        load8<TA, true>(A, g.sam, g.sak, m0 + row, k0 + kc, g.M, g.K, a_vec, ra[c]);
+      } else {
+        const int kk = chunk / (BM / 8), rc = (chunk % (BM / 8)) * 8;
+        load8<TA, false>(A, g.sam, g.sak, m0 + rc, k0 + kk, g.M, g.K, a_vec, ra[c]);
+      }
+      if (B_KC) {
+        const int row = chunk / (BK / 8), kc = (chunk % (BK / 8)) * 8;
+        load8<TB, true>(B, g.sbn, g.sbk, n0 + row, k0 + kc, g.N, g.K, b_vec, rb[c]);
+      } else {
+        const int kk = chunk / (BN / 8), rc = (chunk % (BN / 8)) * 8;
+        load8<TB, false>(B, g.sbn, g.sbk, n0 + rc, k0 + kk, g.N, g.K, b_vec, rb[c]);
+      }
+    }
+  };
+
+  auto put = [&](LT *S, const float (&v)[8], int chunk, bool kc_layout, int rows_total) {
+    if (kc_layout) {
+      const int row = chunk / (BK / 8), kc = (chunk % (BK / 8)) * 8;
+      LT *d = S + row * LD + kc;
+      if (BF16) {
+        uint4 q;
+        q.x = bf16_rne(v[0]) | (bf16_rne(v[1]) << 16);
+        q.y = bf16_rne(v[2]) | (bf16_rne(v[3]) << 16);
+        q.z = bf16_rne(v[4]) | (bf16_rne(v[5]) << 16);
+        q.w = bf16_rne(v[6]) | (bf16_rne(v[7]) << 16);
+        *(uint4 *)d = q;
+      } else {
+        *(float4 *)d = make_float4(v[0], v[1], v[2], v[3]);
+        *(float4 *)(d + 4) = make_float4(v[4], v[5], v[6], v[7]);
+      }
+    } else {
+      const int kk = chunk / (rows_total / 8), rc = (chunk % (rows_total / 8)) * 8;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        if (BF16) S[(rc + j) * LD + kk] = (LT)bf16_rne(v[j]);
+        else S[(rc + j) * LD + kk] = (LT)v[j];
+      }
+    }
+  };
+
+  auto stash = [&]() {
+#pragma unroll
+    for (int c = 0; c < CPT; ++c) {
+      put(As, ra[c], tid + c * 256, A_KC, BM);
+      put(Bs, rb[c], tid + c * 256, B_KC, BN);
+    }
+  };
+
+  const uint32_t n_steps = (g.K + BK - 1) / BK;
+  if (n_steps) fetch(0);
+  for (uint32_t s = 0; s < n_steps; ++s) {
+    __syncthreads();  // previous step's MFMA reads are done
+    stash();
+    __syncthreads();
+    if (s + 1 < n_steps) fetch((s + 1) * BK);
+    if (BF16) {
+#pragma unroll
+      for (int kk = 0; kk < BK; kk += 16) {
+        bf16x8 af[2], bfr[2];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+          af[i] = *(const bf16x8 *)(&As[(wm * 64 + i * 32 + (lane & 31)) * LD + kk + (lane >> 5) * 8]);
+          bfr[i] = *(const bf16x8 *)(&Bs[(wn * 64 + i * 32 + (lane & 31)) * LD + kk + (lane >> 5) * 8]);
+        }
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+          for (int j = 0; j < 2; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
+      }
+    } else {
+#pragma unroll
+      for (int kk = 0; kk < BK; kk += 2) {
+        float af[2], bfr[2];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+          af[i] = (float)As[(wm * 64 + i * 32 + (lane & 31)) * LD + kk + (lane >> 5)];
+          bfr[i] = (float)Bs[(wn * 64 + i * 32 + (lane & 31)) * LD + kk + (lane >> 5)];
+        }
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+          for (int j = 0; j < 2; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i], bfr[j], acc[i][j], 0, 0, 0);
+      }
+    }
+  }
+
+  // 32x32 accumulator layout: element e of a lane sits at
+  //   row = (e / 4) * 8 + (lane / 32) * 4 + e % 4,  col = lane % 32
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const uint32_t col = n0 + wn * 64 + j * 32 + (lane & 31);
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const uint32_t row = m0 + wm * 64 + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
+        if (row < g.M && col < g.N) C[(uint64_t)row * g.N + col] = acc[i][j][e];
+      }
+    }
+}
+
+// ---- GEMV, B k-contiguous (weights, K^T): y[m, n] = sum_k x[m, k] * B[n, k] ------------------------
+// LPR lanes share one output column; each lane moves 16 bytes of B per step.
+template <typename TB, int LPR, int MROWS>
+__global__ void __launch_bounds__(256) gemv_rowdot_kernel(GemmDesc g, int b_vec, int a_vec) {
+  constexpr int EPL = 16 / sizeof(TB);  // elements per 16-byte load
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int sub = lane % LPR, col_in_wave = lane / LPR;
+  constexpr int CPW = 64 / LPR;  // columns per wave pass
+  const uint32_t bz = blockIdx.y, b0 = bz / g.nb1, b1 = bz - b0 * g.nb1;
+  const float *A = (const float *)g.a + b0 * g.sa_b0 + b1 * g.sa_b1;
+  const TB *B = (const TB *)g.b + b0 * g.sb_b0 + b1 * g.sb_b1;
+  float *C = g.c + (uint64_t)bz * g.M * g.N;
+  const uint32_t n_waves = gridDim.x * 4;
+  for (uint32_t nb = (blockIdx.x * 4 + wave) * CPW; nb < g.N; nb += n_waves * CPW) {
+    const uint32_t n = nb + col_in_wave;
+    float acc[MROWS];
+#pragma unroll
+    for (int m = 0; m < MROWS; ++m) acc[m] = 0.f;
+    if (n < g.N) {
+      const TB *brow = B + (int64_t)n * g.sbn;
+      for (uint32_t k = sub * EPL; k < g.K; k += LPR * EPL) {
+        float w[EPL];
+        if (b_vec && k + EPL <= g.K) {
+          if (sizeof(TB) == 4) {
+            float4 q = *(const float4 *)(brow + k);
+            w[0] = q.x; w[1 % EPL] = q.y; w[2 % EPL] = q.z; w[3 % EPL] = q.w;
+          } else {
+            uint4 q = *(const uint4 *)(brow + k);
+            w[0] = __uint_as_float(q.x << 16); w[1 % EPL] = __uint_as_float(q.x & 0xFFFF0000u);
+            w[2 % EPL] = __uint_as_float(q.y << 16); w[3 % EPL] = __uint_as_float(q.y & 0xFFFF0000u);
+            w[4 % EPL] = __uint_as_float(q.z << 16); w[5 % EPL] = __uint_as_float(q.z & 0xFFFF0000u);
+            w[6 % EPL] = __uint_as_float(q.w << 16); w[7 % EPL] = __uint_as_float(q.w & 0xFFFF0000u);
+          }
+        } else {
+#pragma unroll
+          for (int j = 0; j < EPL; ++j) w[j] = k + j < g.K ? widen(brow[k + j]) : 0.f;
+        }
+#pragma unroll
+        for (int m = 0; m < MROWS; ++m) {
+          if ((uint32_t)m < g.M) {
+            const float *xr = A + (int64_t)m * g.sam + k;
+            if (a_vec && k + EPL <= g.K) {
+#pragma unroll
+              for (int j4 = 0; j4 < EPL; j4 += 4) {
+                float4 xv = *(const float4 *)(xr + j4);
+                acc[m] += w[j4] * xv.x + w[j4 + 1] * xv.y + w[j4 + 2] * xv.z + w[j4 + 3] * xv.w;
+              }
+            } else {
+#pragma unroll
+              for (int j = 0; j < EPL; ++j)
+                if (k + j < g.K) acc[m] += w[j] * xr[(int64_t)j * g.sak];
+            }
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int m = 0; m < MROWS; ++m) {
+#pragma unroll
+      for (int s = LPR / 2; s >= 1; s >>= 1) acc[m] += __shfl_xor(acc[m], s, 64);
+      if (sub == 0 && n < g.N && (uint32_t)m < g.M) C[(uint64_t)m * g.N + n] = acc[m];
+    }
+  }
+}
+
+// ---- GEMV, B n-contiguous (V of attention): y[m, n] = sum_k x[m, k] * B[k, n] ---------------------
+// 16 column groups of 4 x 16 k-slices per workgroup; slices meet in LDS.
+template <typename TB, int MROWS>
+__global__ void __launch_bounds__(256) gemv_col_kernel(GemmDesc g, int b_vec) {
+  __shared__ float part[16][MROWS][64 + 4];
+  const int cg = threadIdx.x & 15, ks = threadIdx.x >> 4;
+  const uint32_t bz = blockIdx.y, b0 = bz / g.nb1, b1 = bz - b0 * g.nb1;
+  const float *A = (const float *)g.a + b0 * g.sa_b0 + b1 * g.sa_b1;
+  const TB *B = (const TB *)g.b + b0 * g.sb_b0 + b1 * g.sb_b1;
+  float *C = g.c + (uint64_t)bz * g.M * g.N;
+  const uint32_t n = blockIdx.x * 64 + cg * 4;
+  float acc[MROWS][4];
+#pragma unroll
+  for (int m = 0; m < MROWS; ++m)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[m][j] = 0.f;
+  for (uint32_t k = ks; k < g.K; k += 16) {
+    const TB *brow = B + (int64_t)k * g.sbk + n;
+    float w[4];
+    if (b_vec && n + 4 <= g.N) {
+      if (sizeof(TB) == 4) {
+        float4 q = *(const float4 *)brow;
+        w[0] = q.x; w[1] = q.y; w[2] = q.z; w[3] = q.w;
+      } else {
+        uint2 q = *(const uint2 *)brow;
+        w[0] = __uint_as_float(q.x << 16); w[1] = __uint_as_float(q.x & 0xFFFF0000u);
+        w[2] = __uint_as_float(q.y << 16); w[3] = __uint_as_float(q.y & 0xFFFF0000u);
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) w[j] = n + j < g.N ? widen(brow[j]) : 0.f;
+    }
+#pragma unroll
+    for (int m = 0; m < MROWS; ++m) {
+      if ((uint32_t)m < g.M) {
+        const float xv = A[(int64_t)m * g.sam + (int64_t)k * g.sak];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[m][j] += xv * w[j];
+      }
+    }
+  }
+#pragma unroll
+  for (int m = 0; m < MROWS; ++m)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) part[ks][m][cg * 4 + j] = acc[m][j];
+  __syncthreads();
+  for (int o = threadIdx.x; o < MROWS * 64; o += 256) {
+    const int m = o / 64, c = o % 64;
+    float s = 0.f;
+#pragma unroll
+    for (int q = 0; q < 16; ++q) s += part[q][m][c];
+    const uint32_t col = blockIdx.x * 64 + c;
+    if ((uint32_t)m < g.M && col < g.N) C[(uint64_t)m * g.N + col] = s;
+  }
+}
+
+// ---- u32 matmul (wrapping), contiguous operands: correctness path only -------------------------
+__global__ void __launch_bounds__(256) matmul_u32_kernel(const uint32_t *a, const uint32_t *b,
+                                                         uint32_t *c, uint32_t batch, uint32_t M,
+                                                         uint32_t N, uint32_t K) {
+  const uint64_t total = (uint64_t)batch * M * N;
+  for (uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x; i < total;
+       i += (uint64_t)gridDim.x * 256) {
+    const uint32_t n = i % N, m = (i / N) % M, bz = i / ((uint64_t)M * N);
+    const uint32_t *ar = a + ((uint64_t)bz * M + m) * K, *bc = b + (uint64_t)bz * K * N + n;
+    uint32_t s = 0;
+    for (uint32_t k = 0; k < K; ++k) s += ar[k] * bc[(uint64_t)k * N];
+    c[i] = s;
+  }
+}
+
+hipError_t launch_matmul_u32(const LaunchCtx &lc, const uint32_t *a, const uint32_t *b, uint32_t *c,
+                             uint32_t batch, uint32_t M, uint32_t N, uint32_t K) {
+  uint64_t total = (uint64_t)batch * M * N;
+  if (!total) return hipSuccess;
+  uint64_t blocks = (total + 255) / 256, cap = (uint64_t)lc.n_cus * 8;
+  matmul_u32_kernel<<<(unsigned)(blocks < cap ? blocks : cap), 256, 0, lc.stream>>>(a, b, c, batch,
+                                                                                   M, N, K);
+  return hipGetLastError();
+}
+
+// ---- dispatch ------------------------------------------------------------------------------
+static bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
+
+// 16-byte loads along the unit-stride axis are legal when the base, the other matrix stride and
+// the batch strides all keep 16-byte alignment
+static int vec_ok(const void *base, int esize, int64_t other_stride, int64_t sb0, int64_t sb1) {
+  const int64_t q = 16 / esize;
+  return aligned16(base) && other_stride % q == 0 && sb0 % q == 0 && sb1 % q == 0;
+}
+
+template <typename TA, typename TB, bool BF16>
+static void launch_gemm_layout(const LaunchCtx &lc, const GemmDesc &g, dim3 grid, int av, int bv) {
+  const bool akc = g.sak == 1 || g.K == 1, bkc = g.sbk == 1 && !(g.sbn == 1 && g.N > 1 && false);
+  if (akc && bkc) gemm_kernel<TA, TB, true, true, BF16><<<grid, 256, 0, lc.stream>>>(g, av, bv);
+  else if (akc) gemm_kernel<TA, TB, true, false, BF16><<<grid, 256, 0, lc.stream>>>(g, av, bv);
+  else if (bkc) gemm_kernel<TA, TB, false, true, BF16><<<grid, 256, 0, lc.stream>>>(g, av, bv);
+  else gemm_kernel<TA, TB, false, false, BF16><<<grid, 256, 0, lc.stream>>>(g, av, bv);
+}
+
+template <typename TB, int MROWS>
+static void launch_rowdot(const LaunchCtx &lc, const GemmDesc &g, int bv, int av) {
+  constexpr int EPL = 16 / sizeof(TB);
+  const uint32_t batch = g.nb0 * g.nb1;
+  uint32_t lanes = (g.K + EPL - 1) / EPL;
+  int lpr = lanes >= 64 ? 64 : lanes >= 32 ? 32 : lanes >= 16 ? 16 : 8;
+  // enough waves to cover the CUs a few times over, at least one column pass per wave
+  uint32_t cpw = 64 / lpr;
+  uint32_t waves_needed = (g.N + cpw - 1) / cpw;
+  uint32_t blocks = (waves_needed + 3) / 4;
+  uint32_t cap = (uint32_t)lc.n_cus * 8;
+  if ((uint64_t)blocks * batch > cap) blocks = (cap + batch - 1) / batch;
+  if (blocks < 1) blocks = 1;
+  dim3 grid(blocks, batch);
+  switch (lpr) {
+    case 64: gemv_rowdot_kernel<TB, 64, MROWS><<<grid, 256, 0, lc.stream>>>(g, bv, av); break;
+    case 32: gemv_rowdot_kernel<TB, 32, MROWS><<<grid, 256, 0, lc.stream>>>(g, bv, av); break;
+    case 16: gemv_rowdot_kernel<TB, 16, MROWS><<<grid, 256, 0, lc.stream>>>(g, bv, av); break;
+    default: gemv_rowdot_kernel<TB, 8, MROWS><<<grid, 256, 0, lc.stream>>>(g, bv, av); break;
+  }
+}
+
+hipError_t launch_matmul(const LaunchCtx &lc, const GemmDesc &g, const char **kernel_name) {
+  const uint32_t batch = g.nb0 * g.nb1;
+  if (!batch || !g.M || !g.N) return hipSuccess;
+  const int asz = g.a_stype == ST_BF16 ? 2 : 4, bsz = g.b_stype == ST_BF16 ? 2 : 4;
+  const bool a_unit_k = g.sak == 1 || g.K == 1, b_unit_k = g.sbk == 1 || g.K == 1;
+  const bool b_unit_n = g.sbn == 1 || g.N == 1;
+  const int av = vec_ok(g.a, asz, a_unit_k ? g.sam : g.sak, g.sa_b0, g.sa_b1);
+  const int bv = vec_ok(g.b, bsz, b_unit_k ? g.sbn : g.sbk, g.sb_b0, g.sb_b1);
+
+  if (g.M <= 8 && g.a_stype == ST_F32 && g.K > 0) {
+    if (b_unit_k) {
+      if (kernel_name) *kernel_name = g.b_stype == ST_BF16 ? "gemv_rowdot_bf16" : "gemv_rowdot_f32";
+      const int avx = av && a_unit_k;
+      if (g.M == 1) {
+        if (g.b_stype == ST_BF16) launch_rowdot<uint16_t, 1>(lc, g, bv, avx);
+        else launch_rowdot<float, 1>(lc, g, bv, avx);
+      } else if (g.M <= 4) {
+        if (g.b_stype == ST_BF16) launch_rowdot<uint16_t, 4>(lc, g, bv, avx);
+        else launch_rowdot<float, 4>(lc, g, bv, avx);
+      } else {
+        if (g.b_stype == ST_BF16) launch_rowdot<uint16_t, 8>(lc, g, bv, avx);
+        else launch_rowdot<float, 8>(lc, g, bv, avx);
+      }
+      return hipGetLastError();
+    }
+    if (b_unit_n) {
+      if (kernel_name) *kernel_name = g.b_stype == ST_BF16 ? "gemv_col_bf16" : "gemv_col_f32";
+      dim3 grid((g.N + 63) / 64, batch);
+      if (g.M == 1) {
+        if (g.b_stype == ST_BF16) gemv_col_kernel<uint16_t, 1><<<grid, 256, 0, lc.stream>>>(g, bv);
+        else gemv_col_kernel<float, 1><<<grid, 256, 0, lc.stream>>>(g, bv);
+      } else {
+        if (g.b_stype == ST_BF16) gemv_col_kernel<uint16_t, 8><<<grid, 256, 0, lc.stream>>>(g, bv);
+        else gemv_col_kernel<float, 8><<<grid, 256, 0, lc.stream>>>(g, bv);
+      }
+      return hipGetLastError();
+    }
+  }
+
+  dim3 grid((g.N + BN - 1) / BN, (g.M + BM - 1) / BM, batch);
+  if (g.bf16_math) {
+    if (kernel_name) *kernel_name = "gemm_mfma_bf16";
+    if (g.a_stype == ST_F32 && g.b_stype == ST_BF16) launch_gemm_layout<float, uint16_t, true>(lc, g, grid, av, bv);
+    else if (g.a_stype == ST_F32 && g.b_stype == ST_F32) launch_gemm_layout<float, float, true>(lc, g, grid, av, bv);
+    else if (g.a_stype == ST_BF16 && g.b_stype == ST_BF16) launch_gemm_layout<uint16_t, uint16_t, true>(lc, g, grid, av, bv);
+    else launch_gemm_layout<uint16_t, float, true>(lc, g, grid, av, bv);
+  } else {
+    if (kernel_name) *kernel_name = "gemm_mfma_f32";
+    if (g.a_stype != ST_F32 || g.b_stype != ST_F32) return hipErrorInvalidValue;
+    launch_gemm_layout<float, float, false>(lc, g, grid, av, bv);
+  }
+  return hipGetLastError();
+}
+
+}  // namespace cgk

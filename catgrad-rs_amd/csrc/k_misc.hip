@@ -1,0 +1,168 @@
+// k_misc.hip — index/gather, top-k, compare and fill kernels for gfx950.
+//
+// Backend::index  (mod.rs:66-71, ndarray.rs:373-381): select(Axis(dim), flattened indices)
+// Backend::topk   (mod.rs:58,    ndarray.rs:495-520): stable sort by descending total_cmp
+// Backend::compare(mod.rs:59,    ndarray.rs:337-343): shape and element equality
+// All HBM- or latency-bound; index moves 16 bytes per lane along the innermost axis.
+#include <hip/hip_runtime.h>
+#include "launch.hpp"
+
+namespace cgk {
+
+template <int VEC>
+__global__ void __launch_bounds__(256) gather_kernel(GatherDesc g, uint64_t n_groups,
+                                                     uint32_t *err) {
+  for (uint64_t t = (uint64_t)blockIdx.x * 256 + threadIdx.x; t < n_groups;
+       t += (uint64_t)gridDim.x * 256) {
+    uint64_t lin = t * VEC;
+    uint64_t rem = lin;
+    int64_t off = 0;
+#pragma unroll
+    for (int d = MAX_DIMS + 1; d >= 0; --d) {
+      if (d < g.n_dims) {
+        uint32_t c;
+        if (d == 0) {
+          c = (uint32_t)rem;
+        } else {
+          uint64_t q = rem / g.out_dims[d];
+          c = (uint32_t)(rem - q * g.out_dims[d]);
+          rem = q;
+        }
+        if (d == g.dim) {
+          uint32_t ix = g.idx[c];
+          if (ix >= g.x_dim_size) {  // the reference panics; flag it and stay in bounds
+            atomicOr(err, ERRF_INDEX_OOB);
+            ix = g.x_dim_size - 1;
+          }
+          c = ix;
+        }
+        off += (int64_t)c * g.x_stride[d];
+      }
+    }
+    const int64_t inner = g.x_stride[g.n_dims - 1];
+    uint32_t v[VEC];
+    if (g.x_stype == ST_BF16) {
+      const uint16_t *p = (const uint16_t *)g.x + off;
+      if (VEC == 4 && g.vec) {
+        uint2 q = *(const uint2 *)p;
+        v[0] = q.x << 16; v[1 % VEC] = q.x & 0xFFFF0000u;
+        v[2 % VEC] = q.y << 16; v[3 % VEC] = q.y & 0xFFFF0000u;
+      } else {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) v[j] = (uint32_t)p[j * inner] << 16;
+      }
+    } else {
+      const uint32_t *p = (const uint32_t *)g.x + off;
+      if (VEC == 4 && g.vec) {
+        uint4 q = *(const uint4 *)p;
+        v[0] = q.x; v[1 % VEC] = q.y; v[2 % VEC] = q.z; v[3 % VEC] = q.w;
+      } else {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) v[j] = p[j * inner];
+      }
+    }
+    uint32_t *o = (uint32_t *)g.out + lin;
+    if (VEC == 4) {
+      *(uint4 *)o = make_uint4(v[0], v[1 % VEC], v[2 % VEC], v[3 % VEC]);
+    } else {
+      o[0] = v[0];
+    }
+  }
+}
+
+hipError_t launch_gather(const LaunchCtx &lc, const GatherDesc &g, uint64_t n_out) {
+  if (!n_out) return hipSuccess;
+  const bool vec = g.vec && g.dim != g.n_dims - 1 && (g.out_dims[g.n_dims - 1] % 4 == 0);
+  uint64_t groups = vec ? n_out / 4 : n_out;
+  uint64_t blocks = (groups + 255) / 256, cap = (uint64_t)lc.n_cus * 8;
+  unsigned grid = (unsigned)(blocks < cap ? blocks : cap);
+  if (vec) gather_kernel<4><<<grid, 256, 0, lc.stream>>>(g, groups, lc.err_flag);
+  else gather_kernel<1><<<grid, 256, 0, lc.stream>>>(g, groups, lc.err_flag);
+  return hipGetLastError();
+}
+
+__device__ __forceinline__ int32_t total_key_f(float v) {
+  int32_t b = __float_as_int(v);
+  return b ^ (int32_t)(((uint32_t)(b >> 31)) >> 1);
+}
+
+// One wavefront per row.  Round t selects the t-th element of the order
+// (key descending, index ascending) = what a stable descending sort yields.
+__global__ void __launch_bounds__(256) topk_kernel(const float *x, float *values, uint32_t *indices,
+                                                   uint32_t rows, uint32_t n, uint32_t k) {
+  const int lane = threadIdx.x & 63;
+  const uint32_t row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const float *lane_x = x + (uint64_t)row * n;
+  int32_t prev_key = 0;
+  uint32_t prev_idx = 0;
+  for (uint32_t t = 0; t < k; ++t) {
+    int32_t bk = 0;
+    uint32_t bi = 0xFFFFFFFFu;  // none
+    for (uint32_t c = lane; c < n; c += 64) {
+      int32_t key = total_key_f(lane_x[c]);
+      bool eligible = t == 0 || key < prev_key || (key == prev_key && c > prev_idx);
+      if (eligible && (bi == 0xFFFFFFFFu || key > bk || (key == bk && c < bi))) {
+        bk = key;
+        bi = c;
+      }
+    }
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) {
+      int32_t ok = __shfl_xor(bk, m, 64);
+      uint32_t oi = (uint32_t)__shfl_xor((int)bi, m, 64);
+      if (oi != 0xFFFFFFFFu && (bi == 0xFFFFFFFFu || ok > bk || (ok == bk && oi < bi))) {
+        bk = ok;
+        bi = oi;
+      }
+    }
+    prev_key = bk;
+    prev_idx = bi;
+    if (lane == 0) {
+      values[(uint64_t)row * k + t] = lane_x[bi];
+      indices[(uint64_t)row * k + t] = bi;
+    }
+  }
+}
+
+hipError_t launch_topk(const LaunchCtx &lc, const float *x, float *values, uint32_t *indices,
+                       uint32_t rows, uint32_t n, uint32_t k) {
+  if (!rows || !k) return hipSuccess;
+  topk_kernel<<<(rows + 3) / 4, 256, 0, lc.stream>>>(x, values, indices, rows, n, k);
+  return hipGetLastError();
+}
+
+__global__ void __launch_bounds__(256) compare_kernel(const uint32_t *a, const uint32_t *b,
+                                                      uint64_t n, int is_f32, uint32_t *flag) {
+  bool diff = false;
+  for (uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x; i < n;
+       i += (uint64_t)gridDim.x * 256) {
+    if (is_f32) diff |= !(__uint_as_float(a[i]) == __uint_as_float(b[i]));
+    else diff |= a[i] != b[i];
+  }
+  if (diff) atomicOr(flag, 1u);
+}
+
+hipError_t launch_compare(const LaunchCtx &lc, const void *a, const void *b, uint64_t n,
+                          int is_f32, uint32_t *flag) {
+  if (!n) return hipSuccess;
+  uint64_t blocks = (n + 255) / 256, cap = (uint64_t)lc.n_cus * 8;
+  compare_kernel<<<(unsigned)(blocks < cap ? blocks : cap), 256, 0, lc.stream>>>(
+      (const uint32_t *)a, (const uint32_t *)b, n, is_f32, flag);
+  return hipGetLastError();
+}
+
+__global__ void __launch_bounds__(256) fill_kernel(uint32_t *dst, uint32_t value, uint64_t n) {
+  for (uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x; i < n;
+       i += (uint64_t)gridDim.x * 256)
+    dst[i] = value;
+}
+
+hipError_t launch_fill_u32(const LaunchCtx &lc, uint32_t *dst, uint32_t value, uint64_t n) {
+  if (!n) return hipSuccess;
+  uint64_t blocks = (n + 255) / 256, cap = (uint64_t)lc.n_cus * 8;
+  fill_kernel<<<(unsigned)(blocks < cap ? blocks : cap), 256, 0, lc.stream>>>(dst, value, n);
+  return hipGetLastError();
+}
+
+}  // namespace cgk

@@ -1,0 +1,65 @@
+// launch.hpp — host-callable launchers of the gfx950 kernels (one per kernel family).
+// Every launcher enqueues on lc.stream and returns the launch status; nothing synchronises.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include "program.hpp"
+
+namespace cgk {
+
+// bits of the device-side error word (checked by the host at synchronisation points)
+enum : uint32_t { ERRF_DIV_ZERO = 1u, ERRF_INDEX_OOB = 2u };
+
+struct LaunchCtx {
+  hipStream_t stream;
+  int n_cus;
+  uint32_t *err_flag;  // device word
+};
+
+// ---- k_ew.hip
+hipError_t launch_ew(const LaunchCtx &lc, const Program &p, const OutDesc &o, uint64_t n_elems,
+                     bool vec4);
+hipError_t launch_reduce(const LaunchCtx &lc, int kind, const Program &p, void *out, uint32_t rows,
+                         uint32_t n, bool vec4);
+
+// ---- k_misc.hip
+// out[o, i, inner] = x[o, idx[i], inner]; x is read through its strides, out is contiguous
+struct GatherDesc {
+  const void *x;
+  const uint32_t *idx;
+  void *out;
+  int32_t x_stype;         // ST_F32 / ST_U32 / ST_BF16 (bf16 is widened to f32)
+  int32_t n_dims;          // rank of x (== rank of out)
+  int32_t dim;             // gathered axis
+  uint32_t out_dims[MAX_DIMS + 2];
+  int64_t x_stride[MAX_DIMS + 2];
+  uint32_t x_dim_size;     // extent of x along `dim`
+  int32_t vec;             // 16-byte moves along the innermost axis are legal
+};
+hipError_t launch_gather(const LaunchCtx &lc, const GatherDesc &g, uint64_t n_out);
+// stable descending top-k per row of a contiguous [rows, n] f32 tensor
+hipError_t launch_topk(const LaunchCtx &lc, const float *x, float *values, uint32_t *indices,
+                       uint32_t rows, uint32_t n, uint32_t k);
+// *flag |= 1 if any element differs (u32: bit compare, f32: IEEE ==, so NaN differs)
+hipError_t launch_compare(const LaunchCtx &lc, const void *a, const void *b, uint64_t n,
+                          int is_f32, uint32_t *flag);
+hipError_t launch_fill_u32(const LaunchCtx &lc, uint32_t *dst, uint32_t value, uint64_t n);
+
+// ---- k_gemm.hip
+struct GemmDesc {
+  const void *a, *b;
+  float *c;                  // contiguous [batch, M, N]
+  int32_t a_stype, b_stype;  // ST_F32 or ST_BF16
+  uint32_t M, N, K;
+  int64_t sam, sak;          // element strides of A[m, k]
+  int64_t sbk, sbn;          // element strides of B[k, n]
+  uint32_t nb0, nb1;         // batch = nb0 * nb1 (row-major)
+  int64_t sa_b0, sa_b1, sb_b0, sb_b1;  // batch strides (0 = broadcast)
+  int32_t bf16_math;         // 1: operands rounded to bf16, bf16 MFMA; 0: f32 MFMA
+};
+hipError_t launch_matmul(const LaunchCtx &lc, const GemmDesc &g, const char **kernel_name);
+// wrapping u32 matmul (ndarray's generic dot); all operands contiguous
+hipError_t launch_matmul_u32(const LaunchCtx &lc, const uint32_t *a, const uint32_t *b, uint32_t *c,
+                             uint32_t batch, uint32_t M, uint32_t N, uint32_t K);
+
+}  // namespace cgk

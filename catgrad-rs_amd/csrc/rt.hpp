@@ -1,0 +1,102 @@
+// rt.hpp — host runtime of the HIP backend: device allocator, ref-counted tensor handles with
+// shape/stride views, deferred op nodes, and the scheduler that turns them into kernel launches.
+//
+// The `Backend` trait is called one op at a time (catgrad/src/interpreter/tensor_op.rs:15-41)
+// and cannot see the graph, so fusion has to happen behind the interface: every call only
+// checks shapes and records a node; kernels run when a value is needed on the host
+// (to_vec / compare / cg_sync).  Views (transpose, slice, broadcast, mergeable reshape) never
+// move data.
+#pragma once
+#include <hip/hip_runtime_api.h>
+
+#include <atomic>
+#include <cstdint>
+#include <map>
+#include <string>
+#include <vector>
+
+#include "../../include/catgrad_hip.h"
+#include "launch.hpp"
+
+namespace cgrt {
+
+struct Storage {
+  std::atomic<int> rc{1};
+  void *ptr = nullptr;
+  size_t bytes = 0;  // size class actually allocated
+  cg_backend *be = nullptr;
+};
+
+enum NodeOp : uint8_t {
+  N_REAL = 0,   // has storage
+  N_CONST,      // every element equals cbits; no storage until someone needs a buffer
+  N_ARANGE,
+  N_BIN,        // ew = EwOp, in[0], in[1]
+  N_UN,         // ew = EwOp, in[0]
+  N_TRANSPOSE,  // p0, p1
+  N_BROADCAST,
+  N_RESHAPE,
+  N_SLICE,      // p0 = dim, p1 = start
+  N_MATMUL,
+  N_REDUCE,     // p0 = ReduceKind
+  N_CONCAT,     // p0 = dim
+  N_INDEX       // p0 = dim; in[0] = x, in[1] = indices
+};
+
+struct TraceRec {
+  uint64_t launches = 0;
+  double ms = 0, bytes = 0, flops = 0;
+};
+
+struct PendingEvent {
+  std::string name;
+  hipEvent_t start, stop;
+  double bytes, flops;
+};
+
+}  // namespace cgrt
+
+struct cg_tensor {
+  std::atomic<int> rc{1};
+  cg_backend *be = nullptr;
+  cg_dtype dtype = CG_F32;
+  int rank = 0;
+  int64_t shape[CG_MAX_RANK] = {};
+  // realised state
+  cgrt::Storage *st = nullptr;
+  int stype = cgk::ST_F32;
+  int64_t strides[CG_MAX_RANK] = {};  // in elements
+  int64_t offset = 0;                 // in elements
+  // deferred state
+  uint8_t op = cgrt::N_REAL;
+  uint8_t ew = 0;
+  cg_tensor *in[2] = {nullptr, nullptr};
+  int64_t p0 = 0, p1 = 0;
+  uint32_t cbits = 0;
+
+  int64_t size() const {
+    int64_t n = 1;
+    for (int i = 0; i < rank; ++i) n *= shape[i];
+    return n;
+  }
+};
+
+struct cg_backend {
+  std::atomic<int> rc{1};
+  int device = 0;
+  uint32_t flags = 0;
+  hipStream_t stream = nullptr;
+  int n_cus = 256;
+  std::string err;
+  uint32_t *d_words = nullptr;  // [0] kernel error flags, [1] compare flag
+  uint32_t *h_words = nullptr;  // pinned mirror
+  // caching allocator
+  std::map<size_t, std::vector<void *>> pool;
+  uint64_t pool_bytes = 0, device_bytes = 0, launches = 0;
+  // tracing
+  bool trace = false;
+  std::map<std::string, cgrt::TraceRec> trace_recs;
+  std::vector<cgrt::PendingEvent> trace_pending;
+
+  cgk::LaunchCtx lc() const { return cgk::LaunchCtx{stream, n_cus, d_words}; }
+};

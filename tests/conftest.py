@@ -1,0 +1,55 @@
+import importlib
+import os
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+ORACLE_LIB = os.path.join(ROOT, "oracle", "liboracle.so")
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
+
+
+@pytest.fixture(scope="session")
+def cg():
+    return importlib.import_module("catgrad-rs_amd")
+
+
+@pytest.fixture(scope="session")
+def oracle_lib(cg):
+    if not os.path.exists(ORACLE_LIB):
+        import subprocess
+        subprocess.check_call(["make", "-C", os.path.join(ROOT, "oracle")])
+    return cg.load_library(ORACLE_LIB)
+
+
+@pytest.fixture(scope="session")
+def oracle(cg, oracle_lib):
+    """The CPU restatement of NdArrayBackend: the checker."""
+    return cg.Backend(oracle_lib)
+
+
+@pytest.fixture(scope="session")
+def hip_lib(cg):
+    return cg.load_library()
+
+
+@pytest.fixture(scope="session")
+def hip(cg, hip_lib):
+    """The product: deferred (fusing) mode, f32."""
+    return cg.Backend(hip_lib)
+
+
+@pytest.fixture(scope="session")
+def hip_eager(cg, hip_lib):
+    return cg.Backend(hip_lib, flags=cg.FLAG_EAGER)
+
+
+@pytest.fixture(scope="session")
+def hip_bf16(cg, hip_lib):
+    return cg.Backend(hip_lib, flags=cg.FLAG_BF16)
