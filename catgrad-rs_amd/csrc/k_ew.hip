@@ -52,13 +52,20 @@ __device__ __forceinline__ float sqrt_like_pow(float x) {
   return sqrtf(x);
 }
 
+// powf / sinf / cosf expand to hundreds of instructions each; kept out of line so that the
+// interpreter loop stays inside the instruction cache (they are rare in model graphs: exp,
+// sqrt, cube and reciprocal have their own cheap opcodes)
+__device__ __noinline__ float nf_pow(float a, float b) { return powf(a, b); }
+__device__ __noinline__ float nf_sin(float a) { return sinf(a); }
+__device__ __noinline__ float nf_cos(float a) { return cosf(a); }
+
 __device__ __forceinline__ uint32_t apply_bin(uint8_t op, uint32_t a, uint32_t b, uint32_t *err) {
   switch (op) {
     case E_ADD_F: return as_u(as_f(a) + as_f(b));
     case E_SUB_F: return as_u(as_f(a) - as_f(b));
     case E_MUL_F: return as_u(as_f(a) * as_f(b));
     case E_DIV_F: return as_u(as_f(a) / as_f(b));
-    case E_POW_F: return as_u(powf(as_f(a), as_f(b)));
+    case E_POW_F: return as_u(nf_pow(as_f(a), as_f(b)));
     case E_LT_F: return as_u(as_f(a) < as_f(b) ? 1.f : 0.f);
     case E_EQ_F: return as_u(as_f(a) == as_f(b) ? 1.f : 0.f);
     case E_ADD_U: return a + b;
@@ -81,8 +88,8 @@ __device__ __forceinline__ uint32_t apply_un(uint8_t op, uint32_t a) {
   switch (op) {
     case E_NEG_F: return a ^ 0x80000000u;
     case E_NEG_U: return 0u - a;
-    case E_SIN_F: return as_u(sinf(as_f(a)));
-    case E_COS_F: return as_u(cosf(as_f(a)));
+    case E_SIN_F: return as_u(nf_sin(as_f(a)));
+    case E_COS_F: return as_u(nf_cos(as_f(a)));
     case E_F2U: return f2u_sat(as_f(a));
     case E_U2F: return as_u((float)a);
     case E_EXP_F: return as_u(expf(as_f(a)));
@@ -93,14 +100,10 @@ __device__ __forceinline__ uint32_t apply_un(uint8_t op, uint32_t a) {
   }
 }
 
+// Load VEC consecutive elements (along the innermost dim) of one operand at element offset off.
 template <int VEC>
-__device__ __forceinline__ void load_operand(const Operand &in, const uint32_t (&idx)[MAX_DIMS],
-                                             int n_dims, uint32_t (&v)[VEC]) {
-  int64_t off = 0;
-#pragma unroll
-  for (int d = 0; d < MAX_DIMS; ++d)
-    if (d < n_dims) off += (int64_t)idx[d] * in.stride[d];
-  const int64_t inner = in.stride[n_dims - 1];
+__device__ __forceinline__ void load_vec(const Operand &in, int64_t off, int64_t inner,
+                                         uint32_t *v) {
   if (in.stype == ST_BF16) {
     const uint16_t *p = (const uint16_t *)in.ptr + off;
     if (VEC == 4 && in.vec) {
@@ -131,63 +134,111 @@ __device__ __forceinline__ void load_operand(const Operand &in, const uint32_t (
   case 0: M(0) break; case 1: M(1) break; case 2: M(2) break; case 3: M(3) break; \
   case 4: M(4) break; case 5: M(5) break; case 6: M(6) break; case 7: M(7) break;
 
-// Evaluate the program for VEC consecutive elements along the innermost dim.
-template <int VEC>
-__device__ __forceinline__ void eval_program(const Program &p, const uint32_t (&idx)[MAX_DIMS],
-                                             uint32_t lin, uint32_t *err, uint32_t (&res)[VEC]) {
-  uint32_t r[MAX_STACK][VEC];
-  for (int pc = 0; pc < p.n_instr; ++pc) {
+// Evaluate code[pc0, pc1) for K chunks of VEC consecutive elements.  Chunk k starts at inner
+// coordinate c0 + k * cstride (idx[] holds the outer coordinates; its innermost entry is
+// ignored); chunk k is skipped when bit k of `valid` is clear.  Running one instruction over
+// K * VEC elements amortises the (wave-uniform) instruction decode.
+// All K chunks of one operand for this thread.
+template <int VEC, int K>
+__device__ __forceinline__ void load_chunks(const Program &p, int slot,
+                                            const uint32_t (&idx)[MAX_DIMS], uint32_t c0,
+                                            uint32_t cstride, uint32_t valid,
+                                            uint32_t (&t)[K * VEC]) {
+  const Operand &in = p.in[slot];
+  int64_t off = 0;
+#pragma unroll
+  for (int d = 0; d < MAX_DIMS - 1; ++d)
+    if (d < p.n_dims - 1) off += (int64_t)idx[d] * in.stride[d];
+  const int64_t inner = in.stride[p.n_dims - 1];
+#pragma unroll
+  for (int k = 0; k < K; ++k) {
+    if (valid & (1u << k)) {
+      load_vec<VEC>(in, off + (int64_t)(c0 + k * cstride) * inner, inner, &t[k * VEC]);
+    } else {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) t[k * VEC + j] = 0u;
+    }
+  }
+}
+
+template <int VEC, int K>
+__device__ __forceinline__ void eval_program(const Program &p, int pc0, int pc1,
+                                             const uint32_t (&idx)[MAX_DIMS], uint32_t c0,
+                                             uint32_t cstride, uint32_t valid, uint32_t row0,
+                                             uint32_t row1, uint32_t *err,
+                                             uint32_t (&res)[K * VEC]) {
+  constexpr int E = K * VEC;
+  uint32_t r[MAX_STACK][E];
+  for (int pc = pc0; pc < pc1; ++pc) {
     const Instr ins = p.code[pc];
-    if (ins.op <= E_IOTA) {
-      uint32_t t[VEC];
+    if (ins.op <= E_ROW1) {
+      uint32_t t[E];
       if (ins.op == E_LOAD) {
-        load_operand<VEC>(p.in[ins.arg], idx, p.n_dims, t);
-      } else if (ins.op == E_CONST) {
-        uint32_t c = p.imm[ins.arg];
+        load_chunks<VEC, K>(p, ins.arg, idx, c0, cstride, valid, t);
+      } else if (ins.op == E_IOTA) {
 #pragma unroll
-        for (int j = 0; j < VEC; ++j) t[j] = c;
+        for (int k = 0; k < K; ++k)
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) t[k * VEC + j] = c0 + k * cstride + j;
       } else {
+        uint32_t c = ins.op == E_CONST ? p.imm[ins.arg] : (ins.op == E_ROW0 ? row0 : row1);
 #pragma unroll
-        for (int j = 0; j < VEC; ++j) t[j] = lin + j;
+        for (int j = 0; j < E; ++j) t[j] = c;
       }
       switch (ins.depth) {
-#define M(d) _Pragma("unroll") for (int j = 0; j < VEC; ++j) r[d][j] = t[j];
+#define M(d) _Pragma("unroll") for (int j = 0; j < E; ++j) r[d][j] = t[j];
         CG_DEPTHS(M)
 #undef M
       }
     } else if (ins.op <= E_EQ_U) {
-      uint32_t a[VEC], b[VEC];
+      uint32_t a[E], b[E];
       switch (ins.depth) {
-#define M(d) _Pragma("unroll") for (int j = 0; j < VEC; ++j) { \
+#define M(d) _Pragma("unroll") for (int j = 0; j < E; ++j) { \
     a[j] = r[(d) >= 2 ? (d)-2 : 0][j]; b[j] = r[(d) >= 1 ? (d)-1 : 0][j]; }
         CG_DEPTHS(M)
 #undef M
+        case 8:
+#pragma unroll
+          for (int j = 0; j < E; ++j) { a[j] = r[6][j]; b[j] = r[7][j]; }
+          break;
       }
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) a[j] = apply_bin(ins.op, a[j], b[j], err);
+      for (int j = 0; j < E; ++j) a[j] = apply_bin(ins.op, a[j], b[j], err);
       switch (ins.depth) {
-#define M(d) _Pragma("unroll") for (int j = 0; j < VEC; ++j) r[(d) >= 2 ? (d)-2 : 0][j] = a[j];
+#define M(d) _Pragma("unroll") for (int j = 0; j < E; ++j) r[(d) >= 2 ? (d)-2 : 0][j] = a[j];
         CG_DEPTHS(M)
 #undef M
+        case 8:
+#pragma unroll
+          for (int j = 0; j < E; ++j) r[6][j] = a[j];
+          break;
       }
     } else {
-      uint32_t a[VEC];
+      uint32_t a[E];
       switch (ins.depth) {
-#define M(d) _Pragma("unroll") for (int j = 0; j < VEC; ++j) a[j] = r[(d) >= 1 ? (d)-1 : 0][j];
+#define M(d) _Pragma("unroll") for (int j = 0; j < E; ++j) a[j] = r[(d) >= 1 ? (d)-1 : 0][j];
         CG_DEPTHS(M)
 #undef M
+        case 8:
+#pragma unroll
+          for (int j = 0; j < E; ++j) a[j] = r[7][j];
+          break;
       }
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) a[j] = apply_un(ins.op, a[j]);
+      for (int j = 0; j < E; ++j) a[j] = apply_un(ins.op, a[j]);
       switch (ins.depth) {
-#define M(d) _Pragma("unroll") for (int j = 0; j < VEC; ++j) r[(d) >= 1 ? (d)-1 : 0][j] = a[j];
+#define M(d) _Pragma("unroll") for (int j = 0; j < E; ++j) r[(d) >= 1 ? (d)-1 : 0][j] = a[j];
         CG_DEPTHS(M)
 #undef M
+        case 8:
+#pragma unroll
+          for (int j = 0; j < E; ++j) r[7][j] = a[j];
+          break;
       }
     }
   }
 #pragma unroll
-  for (int j = 0; j < VEC; ++j) res[j] = r[0][j];
+  for (int j = 0; j < E; ++j) res[j] = r[0][j];
 }
 
 __device__ __forceinline__ void decompose(const Program &p, uint64_t lin,
@@ -211,7 +262,7 @@ __device__ __forceinline__ void decompose(const Program &p, uint64_t lin,
 }
 
 template <int VEC>
-__global__ void __launch_bounds__(256) ew_kernel(Program p, OutDesc o, uint64_t n_groups,
+__global__ void __launch_bounds__(256) ew_kernel(const Program p, OutDesc o, uint64_t n_groups,
                                                  uint32_t *err) {
   for (uint64_t g = (uint64_t)blockIdx.x * 256 + threadIdx.x; g < n_groups;
        g += (uint64_t)gridDim.x * 256) {
@@ -219,7 +270,12 @@ __global__ void __launch_bounds__(256) ew_kernel(Program p, OutDesc o, uint64_t 
     const uint64_t lin = g * VEC;
     decompose(p, lin, idx);
     uint32_t v[VEC];
-    eval_program<VEC>(p, idx, (uint32_t)lin, err, v);
+    uint32_t c0 = 0;
+#pragma unroll
+    for (int d = 0; d < MAX_DIMS; ++d)
+      if (d == p.n_dims - 1) c0 = idx[d];
+    // rank-1 programs (the only ones with E_IOTA) have c0 == lin
+    eval_program<VEC, 1>(p, 0, p.n_instr, idx, c0, 0u, 1u, 0u, 0u, err, v);
     int64_t off = 0;
 #pragma unroll
     for (int d = 0; d < MAX_DIMS; ++d)
@@ -333,7 +389,7 @@ __device__ __forceinline__ Acc<KIND> shfl_xor_acc(const Acc<KIND> &a, int m) {
 
 // One row per workgroup (WAVES_PER_ROW = 4) or per wavefront (WAVES_PER_ROW = 1).
 template <int KIND, int VEC, int WAVES_PER_ROW>
-__global__ void __launch_bounds__(256) reduce_kernel(Program p, uint32_t *out, uint32_t rows,
+__global__ void __launch_bounds__(256) reduce_kernel(const Program p, uint32_t *out, uint32_t rows,
                                                      uint32_t n, uint32_t *err) {
   __shared__ uint32_t part[4][Acc<KIND>::W];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -368,7 +424,7 @@ __global__ void __launch_bounds__(256) reduce_kernel(Program p, uint32_t *out, u
         for (int d = 0; d < MAX_DIMS; ++d)
           if (d == p.n_dims - 1) idx[d] = c;
         uint32_t v[VEC];
-        eval_program<VEC>(p, idx, c, err, v);
+        eval_program<VEC, 1>(p, 0, p.n_instr, idx, c, 0u, 1u, 0u, 0u, err, v);
 #pragma unroll
         for (int j = 0; j < VEC; ++j) acc.add(v[j], c + j);
       }
@@ -391,6 +447,187 @@ __global__ void __launch_bounds__(256) reduce_kernel(Program p, uint32_t *out, u
       out[row] = acc.result();
     }
   }
+}
+
+// ---- row programs: reduction stages + a final elementwise segment in one kernel --------------------
+__device__ __forceinline__ uint32_t red_init(int kind) {
+  switch (kind) {
+    case R_MAX_F: return 0xFF7FFFFFu;  // f32::MIN
+    default: return 0u;                // 0.0f and 0u share the bit pattern
+  }
+}
+__device__ __forceinline__ uint32_t red_combine(int kind, uint32_t a, uint32_t b) {
+  switch (kind) {
+    case R_SUM_F: return as_u(as_f(a) + as_f(b));
+    case R_SUM_U: return a + b;
+    case R_MAX_F: return as_u(fmaxf(as_f(a), as_f(b)));
+    default: return a > b ? a : b;
+  }
+}
+
+// One row per workgroup (WPR = 4 waves) or per wavefront (WPR = 1).  A thread owns K chunks of
+// VEC elements per pass, so a row of up to WPR * 64 * K * VEC elements is one pass per segment.
+// Every stage re-reads the row through the program; rows come back from L2.
+template <int VEC, int K, int WPR>
+__global__ void __launch_bounds__(256) row_kernel(const Program p, OutDesc o, uint32_t rows,
+                                                  uint32_t n, uint32_t *err) {
+  __shared__ uint32_t part[4];
+  constexpr int E = K * VEC;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const uint32_t rows_per_block = 4 / WPR;
+  const uint32_t tid_in_row = WPR == 4 ? threadIdx.x : lane;
+  const uint32_t cstride = WPR * 64 * VEC;    // distance between a thread's chunks
+  const uint32_t pass = cstride * K;          // elements per pass
+  for (uint32_t rb = blockIdx.x * rows_per_block; rb < rows; rb += gridDim.x * rows_per_block) {
+    const uint32_t row = rb + (WPR == 4 ? 0 : wave);
+    const bool active = row < rows;
+    uint32_t idx[MAX_DIMS];
+    uint32_t rem = active ? row : 0;
+#pragma unroll
+    for (int d = MAX_DIMS - 2; d >= 0; --d) {
+      if (d < p.n_dims - 1) {
+        if (d == 0) {
+          idx[d] = rem;
+        } else {
+          uint32_t q = rem / p.dims[d];
+          idx[d] = rem - q * p.dims[d];
+          rem = q;
+        }
+      } else {
+        idx[d] = 0;
+      }
+    }
+    idx[MAX_DIMS - 1] = 0;
+    uint32_t rv0 = 0, rv1 = 0;
+    int64_t obase = 0;
+#pragma unroll
+    for (int d = 0; d < MAX_DIMS - 1; ++d)
+      if (d < p.n_dims - 1) obase += (int64_t)idx[d] * o.stride[d];
+    const int64_t oinner = o.stride[p.n_dims - 1];
+    int pc = 0;
+    // segments 0 .. n_stages-1 feed a reduction, segment n_stages is stored
+    for (int s = 0; s <= p.n_stages; ++s) {
+      const bool final_seg = s == p.n_stages;
+      const int kind = final_seg ? 0 : p.red_kind[s];
+      const int pc_end = p.seg_end[s];
+      uint32_t acc = red_init(kind);
+      if (active) {
+        for (uint32_t base = 0; base < n; base += pass) {
+          const uint32_t c0 = base + tid_in_row * VEC;
+          uint32_t valid = 0;
+#pragma unroll
+          for (int k = 0; k < K; ++k)
+            if (c0 + k * cstride < n) valid |= 1u << k;
+          if (!valid) continue;
+          uint32_t v[E];
+          eval_program<VEC, K>(p, pc, pc_end, idx, c0, cstride, valid, rv0, rv1, err, v);
+          if (!final_seg) {
+#pragma unroll
+            for (int k = 0; k < K; ++k)
+              if (valid & (1u << k))
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) acc = red_combine(kind, acc, v[k * VEC + j]);
+          } else {
+#pragma unroll
+            for (int k = 0; k < K; ++k) {
+              if (valid & (1u << k)) {
+                uint32_t *q = (uint32_t *)o.ptr + obase + (int64_t)(c0 + k * cstride) * oinner;
+                if (VEC == 4 && o.vec) {
+                  *(uint4 *)q = make_uint4(v[k * VEC], v[k * VEC + 1 % VEC], v[k * VEC + 2 % VEC],
+                                           v[k * VEC + 3 % VEC]);
+                } else {
+#pragma unroll
+                  for (int j = 0; j < VEC; ++j) q[j * oinner] = v[k * VEC + j];
+                }
+              }
+            }
+          }
+        }
+      }
+      if (!final_seg) {
+#pragma unroll
+        for (int m = 32; m >= 1; m >>= 1)
+          acc = red_combine(kind, acc, (uint32_t)__shfl_xor((int)acc, m, 64));
+        if (WPR == 4) {
+          __syncthreads();
+          if (lane == 0) part[wave] = acc;
+          __syncthreads();
+          acc = red_combine(kind, red_combine(kind, part[0], part[1]),
+                            red_combine(kind, part[2], part[3]));
+        }
+        if (s == 0) rv0 = acc; else rv1 = acc;
+      }
+      pc = pc_end;
+    }
+  }
+}
+
+// ---- split-row reductions: few, very long rows (argmax over a vocabulary) ---------------------------
+// Stage A: chunk c of row r -> accumulator words in scratch[(r * chunks + c) * W].
+template <int KIND, int VEC>
+__global__ void __launch_bounds__(256) reduce_split_kernel(const Program p, uint32_t *scratch,
+                                                           uint32_t rows, uint32_t n,
+                                                           uint32_t chunks, uint32_t chunk_len,
+                                                           uint32_t *err) {
+  __shared__ uint32_t part[4][Acc<KIND>::W];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const uint32_t row = blockIdx.x / chunks, chunk = blockIdx.x - row * chunks;
+  uint32_t idx[MAX_DIMS];
+  uint32_t rem = row;
+#pragma unroll
+  for (int d = MAX_DIMS - 2; d >= 0; --d) {
+    if (d < p.n_dims - 1) {
+      if (d == 0) {
+        idx[d] = rem;
+      } else {
+        uint32_t q = rem / p.dims[d];
+        idx[d] = rem - q * p.dims[d];
+        rem = q;
+      }
+    } else {
+      idx[d] = 0;
+    }
+  }
+  idx[MAX_DIMS - 1] = 0;
+  Acc<KIND> acc;
+  const uint32_t c0 = chunk * chunk_len, c1 = min(n, c0 + chunk_len);
+  for (uint32_t c = c0 + threadIdx.x * VEC; c < c1; c += 256 * VEC) {
+#pragma unroll
+    for (int d = 0; d < MAX_DIMS; ++d)
+      if (d == p.n_dims - 1) idx[d] = c;
+    uint32_t v[VEC];
+    eval_program<VEC, 1>(p, 0, p.n_instr, idx, c, 0u, 1u, 0u, 0u, err, v);
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) acc.add(v[j], c + j);
+  }
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) acc.merge(shfl_xor_acc<KIND>(acc, m));
+  if (lane == 0) acc.get(part[wave]);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w2 = 1; w2 < 4; ++w2) {
+      Acc<KIND> o;
+      o.set(part[w2]);
+      acc.merge(o);
+    }
+    acc.get(scratch + (uint64_t)blockIdx.x * Acc<KIND>::W);
+  }
+}
+
+// Stage B: one wavefront per row merges the chunk accumulators.
+template <int KIND>
+__global__ void __launch_bounds__(64) reduce_merge_kernel(const uint32_t *scratch, uint32_t *out,
+                                                          uint32_t rows, uint32_t chunks) {
+  const uint32_t row = blockIdx.x;
+  Acc<KIND> acc;
+  for (uint32_t c = threadIdx.x; c < chunks; c += 64) {
+    Acc<KIND> o;
+    o.set(scratch + ((uint64_t)row * chunks + c) * Acc<KIND>::W);
+    acc.merge(o);
+  }
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) acc.merge(shfl_xor_acc<KIND>(acc, m));
+  if (threadIdx.x == 0) out[row] = acc.result();
 }
 
 // ---- host launchers --------------------------------------------------------------------------
@@ -416,7 +653,20 @@ hipError_t launch_ew(const LaunchCtx &lc, const Program &p, const OutDesc &o, ui
 
 template <int KIND>
 static hipError_t launch_reduce_kind(const LaunchCtx &lc, const Program &p, uint32_t *out,
-                                     uint32_t rows, uint32_t n, bool vec4) {
+                                     uint32_t rows, uint32_t n, bool vec4, uint32_t *scratch,
+                                     uint32_t chunks) {
+  if (scratch && chunks > 1) {
+    uint32_t chunk_len = (n + chunks - 1) / chunks;
+    chunk_len = (chunk_len + 3) / 4 * 4;  // keep vector groups inside one chunk
+    if (vec4)
+      reduce_split_kernel<KIND, 4><<<rows * chunks, 256, 0, lc.stream>>>(p, scratch, rows, n, chunks,
+                                                                         chunk_len, lc.err_flag);
+    else
+      reduce_split_kernel<KIND, 1><<<rows * chunks, 256, 0, lc.stream>>>(p, scratch, rows, n, chunks,
+                                                                         chunk_len, lc.err_flag);
+    reduce_merge_kernel<KIND><<<rows, 64, 0, lc.stream>>>(scratch, out, rows, chunks);
+    return hipGetLastError();
+  }
   const bool block_per_row = n >= 2048;
   if (block_per_row) {
     unsigned g = grid_for(rows, lc);
@@ -430,19 +680,44 @@ static hipError_t launch_reduce_kind(const LaunchCtx &lc, const Program &p, uint
   return hipGetLastError();
 }
 
+uint32_t reduce_split_chunks(const LaunchCtx &lc, uint32_t rows, uint32_t n) {
+  // worth splitting when the rows alone cannot fill the CUs and each row is long
+  if (rows == 0 || n < 16384 || rows * 2 > (uint32_t)lc.n_cus) return 1;
+  uint32_t chunks = (uint32_t)lc.n_cus * 2 / rows;
+  uint32_t max_chunks = n / 2048;
+  if (chunks > max_chunks) chunks = max_chunks;
+  return chunks < 2 ? 1 : chunks;
+}
+
 hipError_t launch_reduce(const LaunchCtx &lc, int kind, const Program &p, void *out, uint32_t rows,
-                         uint32_t n, bool vec4) {
+                         uint32_t n, bool vec4, uint32_t *scratch, uint32_t chunks) {
   if (rows == 0) return hipSuccess;
   uint32_t *o = (uint32_t *)out;
   switch (kind) {
-    case R_SUM_F: return launch_reduce_kind<R_SUM_F>(lc, p, o, rows, n, vec4);
-    case R_SUM_U: return launch_reduce_kind<R_SUM_U>(lc, p, o, rows, n, vec4);
-    case R_MAX_F: return launch_reduce_kind<R_MAX_F>(lc, p, o, rows, n, vec4);
-    case R_MAX_U: return launch_reduce_kind<R_MAX_U>(lc, p, o, rows, n, vec4);
-    case R_ARGMAX_F: return launch_reduce_kind<R_ARGMAX_F>(lc, p, o, rows, n, vec4);
-    case R_ARGMAX_U: return launch_reduce_kind<R_ARGMAX_U>(lc, p, o, rows, n, vec4);
+    case R_SUM_F: return launch_reduce_kind<R_SUM_F>(lc, p, o, rows, n, vec4, scratch, chunks);
+    case R_SUM_U: return launch_reduce_kind<R_SUM_U>(lc, p, o, rows, n, vec4, scratch, chunks);
+    case R_MAX_F: return launch_reduce_kind<R_MAX_F>(lc, p, o, rows, n, vec4, scratch, chunks);
+    case R_MAX_U: return launch_reduce_kind<R_MAX_U>(lc, p, o, rows, n, vec4, scratch, chunks);
+    case R_ARGMAX_F: return launch_reduce_kind<R_ARGMAX_F>(lc, p, o, rows, n, vec4, scratch, chunks);
+    case R_ARGMAX_U: return launch_reduce_kind<R_ARGMAX_U>(lc, p, o, rows, n, vec4, scratch, chunks);
   }
   return hipErrorInvalidValue;
+}
+
+hipError_t launch_row(const LaunchCtx &lc, const Program &p, const OutDesc &o, uint32_t rows,
+                      uint32_t n, bool vec4) {
+  if (rows == 0 || n == 0) return hipSuccess;
+  // one pass per segment when the row fits: 64 lanes x K chunks x VEC per wave, x4 per workgroup
+  if (vec4) {
+    const bool block_per_row = n > 64 * 2 * 4 || rows * 8 <= (uint32_t)lc.n_cus;
+    if (block_per_row) row_kernel<4, 2, 4><<<grid_for(rows, lc), 256, 0, lc.stream>>>(p, o, rows, n, lc.err_flag);
+    else row_kernel<4, 2, 1><<<grid_for((rows + 3) / 4, lc), 256, 0, lc.stream>>>(p, o, rows, n, lc.err_flag);
+  } else {
+    const bool block_per_row = n > 64 * 4 || rows * 8 <= (uint32_t)lc.n_cus;
+    if (block_per_row) row_kernel<1, 4, 4><<<grid_for(rows, lc), 256, 0, lc.stream>>>(p, o, rows, n, lc.err_flag);
+    else row_kernel<1, 4, 1><<<grid_for((rows + 3) / 4, lc), 256, 0, lc.stream>>>(p, o, rows, n, lc.err_flag);
+  }
+  return hipGetLastError();
 }
 
 }  // namespace cgk

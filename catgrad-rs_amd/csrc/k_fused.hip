@@ -1,0 +1,266 @@
+// k_fused.hip — hand-written fused kernels for the op patterns catgrad-llm emits.
+//
+// The deferred graph behind the Backend interface is matched (rt.cpp) against the exact op
+// sequences of the reference's emitters and, on a match, one of these kernels replaces the
+// generic program interpreter:
+//   softmax  (+ the scale and additive mask attention puts in front of it)
+//            catgrad/src/stdlib/nn/mod.rs:162-171, catgrad-llm/src/models/llama.rs:97-107
+//   rmsnorm  catgrad-llm/src/helpers.rs:120-145 (and the (1 + gamma) form of gemma3.rs:41-68)
+//   rope     catgrad-llm/src/helpers.rs:195-221 (half-split rotate, tables sliced at `pos`)
+//   swiglu   silu(gate) * up, catgrad/src/stdlib/nn/mod.rs:130-148, models/llama.rs:26
+//   geglu    gelu(gate) * up, nn/mod.rs:150-160, models/gemma3.rs
+//   binary   a single add/sub/mul/div over contiguous operands (the residual adds)
+// All are HBM- or latency-bound: one read of every operand, one write, 16-byte accesses,
+// short straight-line code (a decode step runs each of them on a few KB, where instruction
+// fetch and launch latency dominate).
+#include <hip/hip_runtime.h>
+#include <math.h>
+#include "launch.hpp"
+
+namespace cgk {
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, 64);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) v = fmaxf(v, __shfl_xor(v, m, 64));
+  return v;
+}
+
+// Reduce across the workgroup (BLOCK threads, a multiple of 64); every thread gets the result.
+template <int BLOCK, bool IS_MAX>
+__device__ __forceinline__ float block_reduce(float v, float *lds) {
+  v = IS_MAX ? wave_max(v) : wave_sum(v);
+  if (BLOCK == 64) return v;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  __syncthreads();
+  if (lane == 0) lds[wave] = v;
+  __syncthreads();
+  float r = lds[0];
+#pragma unroll
+  for (int w = 1; w < BLOCK / 64; ++w) r = IS_MAX ? fmaxf(r, lds[w]) : r + lds[w];
+  return r;
+}
+
+// ---- rmsnorm ----------------------------------------------------------------------------------
+// y = x / sqrt(sum(x*x) / n + eps) * (gamma_offset + gamma), rows contiguous along the last axis.
+// One workgroup per row; the row lives in registers between the two phases.
+template <int BLOCK, int EPT>  // EPT = float4 chunks per thread
+__global__ void __launch_bounds__(BLOCK) rmsnorm_kernel(RmsNormDesc d) {
+  __shared__ float lds[BLOCK / 64];
+  const uint32_t row = blockIdx.x;
+  const float *x = d.x + (int64_t)row * d.x_row_stride;
+  float *y = d.y + (int64_t)row * d.n;
+  float4 v[EPT];
+  float ss = 0.f;
+#pragma unroll
+  for (int e = 0; e < EPT; ++e) {
+    const uint32_t c = (threadIdx.x + e * BLOCK) * 4;
+    if (c < d.n) {
+      v[e] = *(const float4 *)(x + c);
+      ss += v[e].x * v[e].x + v[e].y * v[e].y + v[e].z * v[e].z + v[e].w * v[e].w;
+    }
+  }
+  ss = block_reduce<BLOCK, false>(ss, lds);
+  // the reference divides by sqrt (pow(.., 0.5)); keep a true division for the 1e-4 bar
+  const float rms = sqrtf(ss / d.n_as_float + d.eps);
+#pragma unroll
+  for (int e = 0; e < EPT; ++e) {
+    const uint32_t c = (threadIdx.x + e * BLOCK) * 4;
+    if (c < d.n) {
+      float4 o;
+      o.x = v[e].x / rms; o.y = v[e].y / rms; o.z = v[e].z / rms; o.w = v[e].w / rms;
+      if (d.gamma) {
+        const float4 g = *(const float4 *)(d.gamma + c);
+        o.x *= d.gamma_offset + g.x; o.y *= d.gamma_offset + g.y;
+        o.z *= d.gamma_offset + g.z; o.w *= d.gamma_offset + g.w;
+      }
+      *(float4 *)(y + c) = o;
+    }
+  }
+}
+
+hipError_t launch_rmsnorm(const LaunchCtx &lc, const RmsNormDesc &d) {
+  if (!d.rows || !d.n) return hipSuccess;
+  // n % 4 == 0 and n <= 16384 are checked by the caller
+  if (d.n <= 256) rmsnorm_kernel<64, 1><<<d.rows, 64, 0, lc.stream>>>(d);
+  else if (d.n <= 1024) rmsnorm_kernel<256, 1><<<d.rows, 256, 0, lc.stream>>>(d);
+  else if (d.n <= 2048) rmsnorm_kernel<256, 2><<<d.rows, 256, 0, lc.stream>>>(d);
+  else if (d.n <= 4096) rmsnorm_kernel<256, 4><<<d.rows, 256, 0, lc.stream>>>(d);
+  else rmsnorm_kernel<1024, 4><<<d.rows, 1024, 0, lc.stream>>>(d);
+  return hipGetLastError();
+}
+
+// ---- softmax(x / scale + mask) ------------------------------------------------------------------------
+// x rows contiguous; mask (optional) is read through (row-group, row, col) strides so that the
+// [S, S] causal mask broadcast over batch and heads is never materialised.  The row is kept in
+// registers: EPT elements per thread, lanes strided for coalescing.
+template <int BLOCK, int EPT>
+__global__ void __launch_bounds__(BLOCK == 64 ? 256 : BLOCK) softmax_kernel(SoftmaxDesc d) {
+  __shared__ float lds[BLOCK / 64];
+  constexpr int RPB = BLOCK == 64 ? 4 : 1;  // rows per workgroup (one wave each) for short rows
+  const uint32_t row = blockIdx.x * RPB + (RPB == 4 ? threadIdx.y : 0);
+  if (row >= d.rows) return;  // whole wave exits together (RPB == 4) or never (RPB == 1)
+  const uint32_t tid = threadIdx.x;
+  const float *x = d.x + (int64_t)row * d.x_row_stride;
+  float *y = d.y + (int64_t)row * d.n;
+  const float *mk = nullptr;
+  if (d.mask) {
+    const uint32_t r_in = row % d.mask_rows, grp = row / d.mask_rows;
+    mk = d.mask + (int64_t)grp * d.mask_group_stride + (int64_t)r_in * d.mask_row_stride;
+  }
+  float v[EPT];
+  float mx = -3.40282347e+38f;  // max folds from f32::MIN (ndarray.rs:455-460)
+#pragma unroll
+  for (int e = 0; e < EPT; ++e) {
+    const uint32_t c = tid + e * BLOCK;
+    if (c < d.n) {
+      float t = x[c];
+      if (d.has_scale) t = t / d.scale;
+      if (mk) t = t + mk[(int64_t)c * d.mask_col_stride];
+      else if (d.has_mask_const) t = t + d.mask_const;
+      v[e] = t;
+      mx = fmaxf(mx, t);
+    }
+  }
+  mx = block_reduce<BLOCK, true>(mx, lds);
+  float sum = 0.f;
+#pragma unroll
+  for (int e = 0; e < EPT; ++e) {
+    const uint32_t c = tid + e * BLOCK;
+    if (c < d.n) {
+      v[e] = expf(v[e] - mx);
+      sum += v[e];
+    }
+  }
+  sum = block_reduce<BLOCK, false>(sum, lds);
+#pragma unroll
+  for (int e = 0; e < EPT; ++e) {
+    const uint32_t c = tid + e * BLOCK;
+    if (c < d.n) y[c] = v[e] / sum;
+  }
+}
+
+hipError_t launch_softmax(const LaunchCtx &lc, const SoftmaxDesc &d) {
+  if (!d.rows || !d.n) return hipSuccess;
+  // n <= 16384 checked by the caller
+  if (d.n <= 64) softmax_kernel<64, 1><<<(d.rows + 3) / 4, dim3(64, 4), 0, lc.stream>>>(d);
+  else if (d.n <= 256) softmax_kernel<64, 4><<<(d.rows + 3) / 4, dim3(64, 4), 0, lc.stream>>>(d);
+  else if (d.n <= 512) softmax_kernel<64, 8><<<(d.rows + 3) / 4, dim3(64, 4), 0, lc.stream>>>(d);
+  else if (d.n <= 1024) softmax_kernel<256, 4><<<d.rows, 256, 0, lc.stream>>>(d);
+  else if (d.n <= 4096) softmax_kernel<256, 16><<<d.rows, 256, 0, lc.stream>>>(d);
+  else softmax_kernel<1024, 16><<<d.rows, 1024, 0, lc.stream>>>(d);
+  return hipGetLastError();
+}
+
+// ---- rope -------------------------------------------------------------------------------------------
+// out[b,h,s,j] = cos[s,j] * x[b,h,s,j] + sin[s,j] * rot, rot = j < half ? -x[..,j+half] : x[..,j-half]
+// x is read through (b, h, s) strides with a unit stride along j, so the transposed view of the
+// q/k projection is consumed in place; out is contiguous.  One thread per 4 consecutive j.
+__global__ void __launch_bounds__(256) rope_kernel(RopeDesc d) {
+  const uint32_t q4 = d.dim / 4;
+  const uint64_t total = (uint64_t)d.b * d.h * d.s * q4;
+  for (uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x; i < total;
+       i += (uint64_t)gridDim.x * 256) {
+    const uint32_t j = (uint32_t)(i % q4) * 4;
+    uint64_t r = i / q4;
+    const uint32_t s = (uint32_t)(r % d.s);
+    r /= d.s;
+    const uint32_t h = (uint32_t)(r % d.h), b = (uint32_t)(r / d.h);
+    const float *xr = d.x + (int64_t)b * d.x_sb + (int64_t)h * d.x_sh + (int64_t)s * d.x_ss;
+    const float4 xv = *(const float4 *)(xr + j);
+    const bool lo = j < d.half;
+    float4 pv = *(const float4 *)(xr + (lo ? j + d.half : j - d.half));
+    if (lo) { pv.x = -pv.x; pv.y = -pv.y; pv.z = -pv.z; pv.w = -pv.w; }
+    const float4 c = *(const float4 *)(d.cos + (int64_t)s * d.cs_ss + j);
+    const float4 sn = *(const float4 *)(d.sin + (int64_t)s * d.cs_ss + j);
+    float4 o;
+    o.x = c.x * xv.x + sn.x * pv.x; o.y = c.y * xv.y + sn.y * pv.y;
+    o.z = c.z * xv.z + sn.z * pv.z; o.w = c.w * xv.w + sn.w * pv.w;
+    *(float4 *)(d.out + i * 4) = o;
+  }
+}
+
+hipError_t launch_rope(const LaunchCtx &lc, const RopeDesc &d) {
+  const uint64_t total = (uint64_t)d.b * d.h * d.s * (d.dim / 4);
+  if (!total) return hipSuccess;
+  uint64_t blocks = (total + 255) / 256, cap = (uint64_t)lc.n_cus * 8;
+  rope_kernel<<<(unsigned)(blocks < cap ? blocks : cap), 256, 0, lc.stream>>>(d);
+  return hipGetLastError();
+}
+
+// ---- gated activations --------------------------------------------------------------------------------
+__device__ __forceinline__ float sigmoid_ref(float x) { return 1.0f / (1.0f + expf(-x)); }
+// nn::gelu: 0.5 x (1 + tanh(c (x + k x^3))), tanh(t) = 2 sigmoid(2 t) - 1 (nn/mod.rs:138-160)
+__device__ __forceinline__ float gelu_ref(float x) {
+  const float t = __uint_as_float(0x3F4C4229u) * (x + 0.044715f * (x * x * x));  // f32 sqrt(2/pi)
+  const float th = 2.0f * sigmoid_ref(2.0f * t) - 1.0f;
+  return 0.5f * x * (1.0f + th);
+}
+
+template <bool GELU>
+__global__ void __launch_bounds__(256) glu_kernel(const float *gate, const float *up, float *out,
+                                                  uint64_t n4) {
+  for (uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x; i < n4;
+       i += (uint64_t)gridDim.x * 256) {
+    const float4 g = ((const float4 *)gate)[i], u = ((const float4 *)up)[i];
+    float4 o;
+    if (GELU) {
+      o.x = gelu_ref(g.x) * u.x; o.y = gelu_ref(g.y) * u.y;
+      o.z = gelu_ref(g.z) * u.z; o.w = gelu_ref(g.w) * u.w;
+    } else {
+      o.x = g.x * sigmoid_ref(g.x) * u.x; o.y = g.y * sigmoid_ref(g.y) * u.y;
+      o.z = g.z * sigmoid_ref(g.z) * u.z; o.w = g.w * sigmoid_ref(g.w) * u.w;
+    }
+    ((float4 *)out)[i] = o;
+  }
+}
+
+hipError_t launch_glu(const LaunchCtx &lc, int gelu, const float *gate, const float *up, float *out,
+                      uint64_t n) {
+  if (!n) return hipSuccess;
+  const uint64_t n4 = n / 4;
+  uint64_t blocks = (n4 + 255) / 256, cap = (uint64_t)lc.n_cus * 8;
+  const unsigned grid = (unsigned)(blocks < cap ? blocks : cap);
+  if (gelu) glu_kernel<true><<<grid, 256, 0, lc.stream>>>(gate, up, out, n4);
+  else glu_kernel<false><<<grid, 256, 0, lc.stream>>>(gate, up, out, n4);
+  return hipGetLastError();
+}
+
+// ---- one f32 binary op, a contiguous, b contiguous or a row vector repeated over rows ---------------
+template <int OP>
+__global__ void __launch_bounds__(256) binary_kernel(const float *a, const float *b, float *out,
+                                                     uint64_t n4, uint32_t b_period4) {
+  for (uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x; i < n4;
+       i += (uint64_t)gridDim.x * 256) {
+    const float4 x = ((const float4 *)a)[i];
+    const float4 y = ((const float4 *)b)[b_period4 ? i % b_period4 : i];
+    float4 o;
+    if (OP == 0) { o.x = x.x + y.x; o.y = x.y + y.y; o.z = x.z + y.z; o.w = x.w + y.w; }
+    if (OP == 1) { o.x = x.x - y.x; o.y = x.y - y.y; o.z = x.z - y.z; o.w = x.w - y.w; }
+    if (OP == 2) { o.x = x.x * y.x; o.y = x.y * y.y; o.z = x.z * y.z; o.w = x.w * y.w; }
+    if (OP == 3) { o.x = x.x / y.x; o.y = x.y / y.y; o.z = x.z / y.z; o.w = x.w / y.w; }
+    ((float4 *)out)[i] = o;
+  }
+}
+
+hipError_t launch_binary_f32(const LaunchCtx &lc, int op, const float *a, const float *b, float *out,
+                             uint64_t n, uint32_t b_period) {
+  if (!n) return hipSuccess;
+  const uint64_t n4 = n / 4;
+  uint64_t blocks = (n4 + 255) / 256, cap = (uint64_t)lc.n_cus * 16;
+  const unsigned grid = (unsigned)(blocks < cap ? blocks : cap);
+  const uint32_t p4 = b_period / 4;
+  switch (op) {
+    case 0: binary_kernel<0><<<grid, 256, 0, lc.stream>>>(a, b, out, n4, p4); break;
+    case 1: binary_kernel<1><<<grid, 256, 0, lc.stream>>>(a, b, out, n4, p4); break;
+    case 2: binary_kernel<2><<<grid, 256, 0, lc.stream>>>(a, b, out, n4, p4); break;
+    default: binary_kernel<3><<<grid, 256, 0, lc.stream>>>(a, b, out, n4, p4); break;
+  }
+  return hipGetLastError();
+}
+
+}  // namespace cgk

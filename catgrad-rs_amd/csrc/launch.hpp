@@ -19,8 +19,14 @@ struct LaunchCtx {
 // ---- k_ew.hip
 hipError_t launch_ew(const LaunchCtx &lc, const Program &p, const OutDesc &o, uint64_t n_elems,
                      bool vec4);
+// chunks > 1 (from reduce_split_chunks) splits every row over several workgroups; scratch then
+// needs rows * chunks * 3 words
+uint32_t reduce_split_chunks(const LaunchCtx &lc, uint32_t rows, uint32_t n);
 hipError_t launch_reduce(const LaunchCtx &lc, int kind, const Program &p, void *out, uint32_t rows,
-                         uint32_t n, bool vec4);
+                         uint32_t n, bool vec4, uint32_t *scratch, uint32_t chunks);
+// reduction stages + final segment of a row program in one launch
+hipError_t launch_row(const LaunchCtx &lc, const Program &p, const OutDesc &o, uint32_t rows,
+                      uint32_t n, bool vec4);
 
 // ---- k_misc.hip
 // out[o, i, inner] = x[o, idx[i], inner]; x is read through its strides, out is contiguous
@@ -44,6 +50,43 @@ hipError_t launch_topk(const LaunchCtx &lc, const float *x, float *values, uint3
 hipError_t launch_compare(const LaunchCtx &lc, const void *a, const void *b, uint64_t n,
                           int is_f32, uint32_t *flag);
 hipError_t launch_fill_u32(const LaunchCtx &lc, uint32_t *dst, uint32_t value, uint64_t n);
+
+// ---- k_fused.hip
+struct RmsNormDesc {
+  const float *x;        // rows of n contiguous floats, row r at x + r * x_row_stride
+  const float *gamma;    // n floats or null
+  float *y;              // contiguous [rows, n]
+  int64_t x_row_stride;
+  uint32_t rows, n;
+  float n_as_float, eps, gamma_offset;  // gamma_offset: 0 (llama) or 1 (gemma's 1 + gamma)
+};
+hipError_t launch_rmsnorm(const LaunchCtx &lc, const RmsNormDesc &d);
+
+struct SoftmaxDesc {
+  const float *x;        // row r at x + r * x_row_stride, unit stride along the row
+  const float *mask;     // or null; row r reads mask + (r / mask_rows) * group + (r % mask_rows) * row
+  float *y;              // contiguous [rows, n]
+  int64_t x_row_stride, mask_group_stride, mask_row_stride, mask_col_stride;
+  uint32_t rows, n, mask_rows;
+  int32_t has_scale, has_mask_const;
+  float scale, mask_const;
+};
+hipError_t launch_softmax(const LaunchCtx &lc, const SoftmaxDesc &d);
+
+struct RopeDesc {
+  const float *x, *cos, *sin;
+  float *out;            // contiguous [b, h, s, dim]
+  int64_t x_sb, x_sh, x_ss, cs_ss;  // element strides (unit stride along dim everywhere)
+  uint32_t b, h, s, dim, half;
+};
+hipError_t launch_rope(const LaunchCtx &lc, const RopeDesc &d);
+// out = silu(gate) * up (gelu = 0) or gelu(gate) * up (gelu = 1); contiguous, n % 4 == 0
+hipError_t launch_glu(const LaunchCtx &lc, int gelu, const float *gate, const float *up, float *out,
+                      uint64_t n);
+// op: 0 add, 1 sub, 2 mul, 3 div; b is contiguous (b_period = 0) or a vector of b_period floats
+// repeated; n % 4 == 0, b_period % 4 == 0
+hipError_t launch_binary_f32(const LaunchCtx &lc, int op, const float *a, const float *b, float *out,
+                             uint64_t n, uint32_t b_period);
 
 // ---- k_gemm.hip
 struct GemmDesc {

@@ -267,106 +267,281 @@ int alloc_result(cg_backend *be, cg_tensor *n, int stype) {
 
 void *data_ptr(const cg_tensor *t) { return (char *)t->st->ptr + t->offset * esize(t->stype); }
 
-bool ew_inlineable(const cg_tensor *n) {
-  return (n->op == N_BIN || n->op == N_UN) && n->rc.load() == 1;
+// ---- fusion regions ------------------------------------------------------------------------
+// A region is the set of deferred nodes that one kernel evaluates: the elementwise tree under a
+// root and, when `rows` is on, the row values it reads through a last-axis broadcast:
+//     root <- BIN/UN ... <- BROADCAST <- (BIN/UN on [.., 1])* <- REDUCE(sum|max) <- BIN/UN ...
+// A node may be evaluated inside the region (instead of being materialised) iff every reference
+// to it comes from inside the region; a node referenced k times is simply evaluated k times.
+bool same_shape(const cg_tensor *a, const cg_tensor *b) {
+  return a->rank == b->rank && std::equal(a->shape, a->shape + a->rank, b->shape);
 }
 
-struct Cost {
-  int instr = 0, inputs = 0, depth = 0;
-};
+// `b` broadcasts a [.., 1] tensor along the last axis only, to the shape of `root`
+bool is_row_broadcast(const cg_tensor *b, const cg_tensor *root) {
+  if (b->op != N_BROADCAST || !same_shape(b, root) || b->rank == 0) return false;
+  const cg_tensor *r = b->in[0];
+  if (r->rank != b->rank || r->shape[r->rank - 1] != 1) return false;
+  for (int i = 0; i + 1 < r->rank; ++i)
+    if (r->shape[i] != b->shape[i]) return false;
+  return true;
+}
 
-Cost measure(const cg_tensor *n) {
-  Cost c;
-  if (n->op == N_CONST || (n->op == N_ARANGE && n->rank == 1)) {
-    c.instr = 1;
-    c.depth = 1;
-  } else if (n->op == N_BIN) {
-    Cost a = ew_inlineable(n->in[0]) || n->in[0]->op == N_CONST ? measure(n->in[0]) : Cost{1, 1, 1};
-    Cost b = ew_inlineable(n->in[1]) || n->in[1]->op == N_CONST ? measure(n->in[1]) : Cost{1, 1, 1};
-    c.instr = a.instr + b.instr + 1;
-    c.inputs = a.inputs + b.inputs;
-    c.depth = std::max(a.depth, b.depth + 1);
-  } else if (n->op == N_UN) {
-    Cost a = ew_inlineable(n->in[0]) || n->in[0]->op == N_CONST ? measure(n->in[0]) : Cost{1, 1, 1};
-    c.instr = a.instr + 1;
-    c.inputs = a.inputs;
-    c.depth = a.depth;
-  } else {
-    c = Cost{1, 1, 1};
+// every leaf under the row value `r` is a constant or a fusable reduction of a root-shaped tensor
+bool row_chain_ok(const cg_tensor *r, const cg_tensor *root, int depth = 0) {
+  if (depth > 32) return false;
+  if (r->op == N_CONST) return true;
+  if (r->op == N_BIN) return row_chain_ok(r->in[0], root, depth + 1) && row_chain_ok(r->in[1], root, depth + 1);
+  if (r->op == N_UN) return row_chain_ok(r->in[0], root, depth + 1);
+  if (r->op == N_REDUCE && r->p0 <= R_MAX_U) return same_shape(r->in[0], root);
+  return false;
+}
+
+struct Region {
+  const cg_tensor *root = nullptr;
+  bool rows = false;
+  std::vector<std::pair<const cg_tensor *, int>> refs;  // internal reference counts
+  std::vector<cg_tensor *> order;                        // children before parents
+
+  int *count(const cg_tensor *n) {
+    for (auto &kv : refs)
+      if (kv.first == n) return &kv.second;
+    return nullptr;
   }
-  return c;
-}
+  // true the first time `n` is seen
+  bool edge(const cg_tensor *n) {
+    if (int *c = count(n)) {
+      ++*c;
+      return false;
+    }
+    refs.emplace_back(n, 1);
+    return true;
+  }
+  bool qualified(const cg_tensor *n) const {
+    for (const cg_tensor *o : order)
+      if (o == n) return true;
+    return false;
+  }
+  // evaluated inside the kernel: a walked node all of whose readers are in the region
+  bool inside(const cg_tensor *n) {
+    if (n == root) return true;
+    int *c = count(n);
+    return c && n->op != N_REAL && n->rc.load() == *c && qualified(n);
+  }
+
+  void walk_full(cg_tensor *n) {
+    if (n->op == N_BIN || n->op == N_UN) {
+      for (int i = 0; i < 2; ++i)
+        if (cg_tensor *c = n->in[i])
+          if (edge(c)) walk_full(c);
+      order.push_back(n);
+    } else if (rows && is_row_broadcast(n, root) && row_chain_ok(n->in[0], root)) {
+      if (edge(n->in[0])) walk_row(n->in[0]);
+      order.push_back(n);
+    }
+  }
+  void walk_row(cg_tensor *r) {
+    if (r->op == N_BIN || r->op == N_UN) {
+      for (int i = 0; i < 2; ++i)
+        if (cg_tensor *c = r->in[i])
+          if (edge(c)) walk_row(c);
+      order.push_back(r);
+    } else if (r->op == N_REDUCE) {
+      if (edge(r->in[0])) walk_full(r->in[0]);
+      order.push_back(r);
+    }
+  }
+  void build(cg_tensor *root_, bool rows_) {
+    root = root_;
+    rows = rows_;
+    refs.clear();
+    order.clear();
+    walk_full(root_);
+  }
+  // a deferred node of the region that somebody outside also reads: it has to exist in memory
+  cg_tensor *shared_node() {
+    for (cg_tensor *n : order)
+      if (n != root && !inside(n)) return n;
+    return nullptr;
+  }
+};
 
 struct EwCompiler {
   cg_backend *be;
+  Region *reg;
   Program p;
   std::vector<cg_tensor *> ins;
-  EwCompiler(cg_backend *b) : be(b) { std::memset(&p, 0, sizeof(p)); }
+  std::vector<uint32_t> imms;
+  struct Stage {
+    const cg_tensor *reduce;
+    std::vector<Instr> code;
+  };
+  std::vector<Stage> stages;
+  std::vector<Instr> final_code;
+  bool overflow = false;  // a limit was hit: the caller retries with a smaller region
 
-  int push(uint8_t op, int depth, uint16_t arg) {
-    if (p.n_instr >= MAX_INSTR || depth > MAX_STACK)
+  EwCompiler(cg_backend *b, Region *r) : be(b), reg(r) { std::memset(&p, 0, sizeof(p)); }
+
+  int total_instr() const {
+    size_t n = final_code.size();
+    for (auto &s : stages) n += s.code.size();
+    return (int)n;
+  }
+  int push(std::vector<Instr> &code, uint8_t op, int depth, uint16_t arg) {
+    // a push writes slot `depth`; an operator reads the slots below `depth`
+    const bool is_push = op <= E_ROW1;
+    if (total_instr() >= MAX_INSTR || depth > MAX_STACK || (is_push && depth >= MAX_STACK)) {
+      overflow = true;
       return fail(be, CG_ERR_INTERNAL, "elementwise program overflow");
-    p.code[p.n_instr].op = op;
-    p.code[p.n_instr].depth = (uint8_t)depth;
-    p.code[p.n_instr].arg = arg;
-    p.n_instr++;
+    }
+    Instr i;
+    i.op = op;
+    i.depth = (uint8_t)depth;
+    i.arg = arg;
+    code.push_back(i);
     return CG_OK;
   }
-  int push_const(uint32_t bits, int depth) {
-    if (p.n_instr >= MAX_INSTR) return fail(be, CG_ERR_INTERNAL, "elementwise program overflow");
-    p.imm[p.n_instr] = bits;
-    return push(E_CONST, depth, (uint16_t)p.n_instr);
+  int push_const(std::vector<Instr> &code, uint32_t bits, int depth) {
+    size_t k = 0;
+    for (; k < imms.size(); ++k)
+      if (imms[k] == bits) break;
+    if (k == imms.size()) imms.push_back(bits);
+    return push(code, E_CONST, depth, (uint16_t)k);
   }
-  int load(cg_tensor *n, int depth) {
+  int load(std::vector<Instr> &code, cg_tensor *n, int depth) {
     if (n->op != N_REAL) TRY(realize(be, n));
     size_t slot = 0;
     for (; slot < ins.size(); ++slot)
       if (ins[slot] == n) break;
     if (slot == ins.size()) {
-      if (ins.size() >= MAX_IN) return fail(be, CG_ERR_INTERNAL, "elementwise program: too many inputs");
+      if (ins.size() >= MAX_IN) {
+        overflow = true;
+        return fail(be, CG_ERR_INTERNAL, "elementwise program: too many inputs");
+      }
       ins.push_back(n);
     }
-    return push(E_LOAD, depth, (uint16_t)slot);
+    return push(code, E_LOAD, depth, (uint16_t)slot);
   }
   static bool is_const(const cg_tensor *n, uint32_t bits) { return n->op == N_CONST && n->cbits == bits; }
 
-  // emit code leaving the value of `n` at stack slot `depth`
-  int emit(cg_tensor *n, int depth, int pend_instr, int pend_in, bool root) {
-    if (n->op == N_CONST) return push_const(n->cbits, depth);
-    if (n->op == N_ARANGE && n->rank == 1) return push(E_IOTA, depth, 0);
-    if (!(root || ew_inlineable(n)) || (n->op != N_BIN && n->op != N_UN)) return load(n, depth);
-    if (!root) {
-      Cost c = measure(n);
-      if (p.n_instr + c.instr + pend_instr > MAX_INSTR ||
-          (int)ins.size() + c.inputs + pend_in > MAX_IN || depth + c.depth > MAX_STACK)
-        return load(n, depth);
+  // stack slots needed to evaluate `n` (capped), mirroring emit/emit_op
+  int need(cg_tensor *n, bool row, int budget = 64) {
+    if (budget <= 0) return MAX_STACK + 1;
+    if (n->op == N_CONST) return 1;
+    if (!row) {
+      if (!reg->inside(n)) return 1;
+      if (n->op == N_BROADCAST) return need(n->in[0], true, budget - 1);
+    } else if (n->op == N_REDUCE) {
+      return 1;
     }
+    if (n->op == N_UN) return need(n->in[0], row, budget - 1);
+    if (n->op != N_BIN) return 1;
+    cg_tensor *a = n->in[0], *b = n->in[1];
+    if (n->ew == E_POW_F && is_const(a, 0x402DF854u)) return need(b, row, budget - 1);
+    if (n->ew == E_POW_F && (is_const(b, 0x3F000000u) || is_const(b, 0x40400000u))) return need(a, row, budget - 1);
+    if (n->ew == E_DIV_F && is_const(a, 0x3F800000u)) return need(b, row, budget - 1);
+    const int na = need(a, row, budget / 2), nb = need(b, row, budget / 2);
+    const int fwd = std::max(na, nb + 1), rev = std::max(nb, na + 1);
+    return commutative(n->ew) ? std::min(fwd, rev) : fwd;
+  }
+  static bool commutative(uint8_t op) {
+    return op == E_ADD_F || op == E_MUL_F || op == E_EQ_F || op == E_ADD_U || op == E_MUL_U || op == E_EQ_U;
+  }
+
+  int emit_op(std::vector<Instr> &code, cg_tensor *n, int depth, bool row) {
+    auto sub = [&](cg_tensor *c, int d) { return row ? emit_row(code, c, d) : emit(code, c, d); };
     if (n->op == N_UN) {
-      TRY(emit(n->in[0], depth, pend_instr + 1, pend_in, false));
-      return push(n->ew, depth + 1, 0);
+      TRY(sub(n->in[0], depth));
+      return push(code, n->ew, depth + 1, 0);
     }
     cg_tensor *a = n->in[0], *b = n->in[1];
     if (n->ew == E_POW_F) {
       // nn::exp = pow(broadcast(E), x); nn::sqrt = pow(x, broadcast(0.5)); gelu: pow(x, 3)
       // (catgrad/src/stdlib/nn/mod.rs:117-128, 157)
       if (is_const(a, 0x402DF854u)) {
-        TRY(emit(b, depth, pend_instr + 1, pend_in, false));
-        return push(E_EXP_F, depth + 1, 0);
+        TRY(sub(b, depth));
+        return push(code, E_EXP_F, depth + 1, 0);
       }
       if (is_const(b, 0x3F000000u) || is_const(b, 0x40400000u)) {
-        TRY(emit(a, depth, pend_instr + 1, pend_in, false));
-        return push(is_const(b, 0x3F000000u) ? E_SQRT_F : E_CUBE_F, depth + 1, 0);
+        TRY(sub(a, depth));
+        return push(code, is_const(b, 0x3F000000u) ? E_SQRT_F : E_CUBE_F, depth + 1, 0);
       }
     }
     if (n->ew == E_DIV_F && is_const(a, 0x3F800000u)) {
-      TRY(emit(b, depth, pend_instr + 1, pend_in, false));
-      return push(E_RCP_F, depth + 1, 0);
+      TRY(sub(b, depth));
+      return push(code, E_RCP_F, depth + 1, 0);
     }
-    TRY(emit(a, depth, pend_instr + 2, pend_in + 1, false));
-    TRY(emit(b, depth + 1, pend_instr + 1, pend_in, false));
-    return push(n->ew, depth + 2, 0);
+    // commutative ops evaluate the deeper operand first (fewer live stack slots)
+    if (commutative(n->ew) && need(b, row) > need(a, row)) std::swap(a, b);
+    TRY(sub(a, depth));
+    TRY(sub(b, depth + 1));
+    return push(code, n->ew, depth + 2, 0);
+  }
+
+  // value of the root-shaped node `n` at stack slot `depth`
+  int emit(std::vector<Instr> &code, cg_tensor *n, int depth) {
+    if (n->op == N_CONST) return push_const(code, n->cbits, depth);
+    if (n->op == N_ARANGE && n->rank == 1) return push(code, E_IOTA, depth, 0);
+    if (reg->inside(n)) {
+      if (n->op == N_BIN || n->op == N_UN) return emit_op(code, n, depth, false);
+      if (n->op == N_BROADCAST) return emit_row(code, n->in[0], depth);
+    }
+    return load(code, n, depth);
+  }
+
+  // value of the row-shaped node `r`
+  int emit_row(std::vector<Instr> &code, cg_tensor *r, int depth) {
+    if (r->op == N_CONST) return push_const(code, r->cbits, depth);
+    if (!reg->inside(r)) {
+      overflow = true;  // cannot happen in a prepared region
+      return fail(be, CG_ERR_INTERNAL, "row value escaped its region");
+    }
+    if (r->op == N_BIN || r->op == N_UN) return emit_op(code, r, depth, true);
+    // N_REDUCE: its input becomes (or already is) a reduction stage
+    size_t sid = 0;
+    for (; sid < stages.size(); ++sid)
+      if (stages[sid].reduce == r) break;
+    if (sid == stages.size()) {
+      std::vector<Instr> sc;
+      TRY(emit(sc, r->in[0], 0));  // may add earlier stages first
+      if (stages.size() >= MAX_STAGES) {
+        overflow = true;
+        return fail(be, CG_ERR_INTERNAL, "row program: too many reduction stages");
+      }
+      sid = stages.size();
+      stages.push_back(Stage{r, std::move(sc)});
+    }
+    return push(code, sid == 0 ? E_ROW0 : E_ROW1, depth, 0);
+  }
+
+  int compile_root(cg_tensor *root) { return emit(final_code, root, 0); }
+
+  void flatten() {
+    int k = 0;
+    p.n_stages = (int)stages.size();
+    for (size_t s = 0; s < stages.size(); ++s) {
+      for (const Instr &i : stages[s].code) p.code[k++] = i;
+      p.seg_end[s] = k;
+      p.red_kind[s] = (int)stages[s].reduce->p0;
+    }
+    for (const Instr &i : final_code) p.code[k++] = i;
+    p.seg_end[stages.size()] = k;
+    p.n_instr = k;
+    for (size_t i = 0; i < imms.size() && i < (size_t)MAX_INSTR; ++i) p.imm[i] = imms[i];
   }
 };
+
+// Realise every node of the region that is also read from outside it, until the region is
+// closed.  Returns the prepared region.
+int prepare_region(cg_backend *be, cg_tensor *root, bool rows, Region &reg) {
+  for (int guard = 0; guard < 4096; ++guard) {
+    reg.build(root, rows);
+    cg_tensor *victim = reg.shared_node();
+    if (!victim) return CG_OK;
+    TRY(realize(be, victim));
+  }
+  return fail(be, CG_ERR_INTERNAL, "prepare_region did not converge");
+}
 
 // Collapse the logical dims shared by all operands: drop extent-1 dims, merge neighbours that
 // every operand walks contiguously.  strides[o] are per-operand stride arrays of length rank.
@@ -441,16 +616,14 @@ int finish_program(cg_backend *be, EwCompiler &c, int rank, const int64_t *shape
   return CG_OK;
 }
 
-// Evaluate the elementwise tree rooted at `root` into (dst storage, dst strides, dst stype).
-int run_ew(cg_backend *be, cg_tensor *root, bool root_is_value, void *dst, const int64_t *dst_strides,
-           int dst_stype, const char *name) {
-  if (root->size() == 0) return CG_OK;
-  EwCompiler c(be);
-  if (root_is_value) TRY(c.load(root, 0));
-  else TRY(c.emit(root, 0, 0, 0, true));
+// Launch the compiled program of `c` into (dst, dst_strides, dst_stype).
+int launch_compiled(cg_backend *be, EwCompiler &c, cg_tensor *root, void *dst,
+                    const int64_t *dst_strides, int dst_stype, const char *name) {
+  c.flatten();
+  const bool rowprog = c.p.n_stages > 0;
   std::vector<int64_t> ostr;
   double bytes_in = 0;
-  TRY(finish_program(be, c, root->rank, root->shape, dst_strides, false, ostr, &bytes_in));
+  TRY(finish_program(be, c, root->rank, root->shape, dst_strides, rowprog, ostr, &bytes_in));
   const int64_t n = root->size();
   if (n >= (int64_t)1 << 32) return fail(be, CG_ERR_INTERNAL, "tensor above 2^32 elements");
   OutDesc o;
@@ -459,10 +632,50 @@ int run_ew(cg_backend *be, cg_tensor *root, bool root_is_value, void *dst, const
   o.stype = dst_stype;
   for (int d = 0; d < c.p.n_dims; ++d) o.stride[d] = ostr[d];
   o.vec = dst_stype != ST_BF16 && operand_vec_ok(dst, dst_stype, ostr);
-  const bool vec4 = c.p.dims[c.p.n_dims - 1] % 4 == 0;
+  const uint32_t inner = c.p.dims[c.p.n_dims - 1];
+  const bool vec4 = inner % 4 == 0;
+  if (rowprog) {
+    if (dst_stype == ST_BF16) return fail(be, CG_ERR_INTERNAL, "row program into bf16 storage");
+    const int64_t cols = root->shape[root->rank - 1];
+    KernelScope ks(be, "row_fused", bytes_in + (double)n * 4, 0);
+    HIPCHK(be, launch_row(be->lc(), c.p, o, (uint32_t)(n / cols), (uint32_t)cols, vec4));
+    return CG_OK;
+  }
   KernelScope ks(be, name, bytes_in + (double)n * esize(dst_stype), 0);
   HIPCHK(be, launch_ew(be->lc(), c.p, o, (uint64_t)n, vec4));
   return CG_OK;
+}
+
+// Evaluate the elementwise tree rooted at `root` into (dst storage, dst strides, dst stype).
+// root_is_value: just copy the (realised) value of root through its strides.
+int run_ew(cg_backend *be, cg_tensor *root, bool root_is_value, void *dst, const int64_t *dst_strides,
+           int dst_stype, const char *name) {
+  if (root->size() == 0) return CG_OK;
+  if (root_is_value) {
+    Region reg;
+    EwCompiler c(be, &reg);
+    TRY(c.load(c.final_code, root, 0));
+    return launch_compiled(be, c, root, dst, dst_strides, dst_stype, name);
+  }
+  // first with row values fused in, then without, then cutting the tree at its children
+  for (int attempt = 0; attempt < 64; ++attempt) {
+    const bool rows = attempt == 0 && root->rank > 0 && dst_stype != ST_BF16;
+    Region reg;
+    TRY(prepare_region(be, root, rows, reg));
+    EwCompiler c(be, &reg);
+    int st = c.compile_root(root);
+    if (!st) return launch_compiled(be, c, root, dst, dst_strides, dst_stype, name);
+    if (!c.overflow) return st;
+    if (attempt >= 1) {
+      // still too large: materialise the biggest deferred child and try again
+      cg_tensor *victim = nullptr;
+      for (cg_tensor *n : reg.order)
+        if (n != root && (n->op == N_BIN || n->op == N_UN)) victim = n;  // last = closest to root
+      if (!victim) return st;
+      TRY(realize(be, victim));
+    }
+  }
+  return fail(be, CG_ERR_INTERNAL, "elementwise program does not fit");
 }
 
 // A fresh contiguous tensor holding the value of `src` (f32/u32 storage unless keep_bf16).
@@ -498,7 +711,435 @@ int realize_const(cg_backend *be, cg_tensor *n) {
   return CG_OK;
 }
 
+// ---- pattern kernels --------------------------------------------------------------------------
+// The emitters of the reference produce fixed op sequences for softmax, RMSNorm, RoPE and the
+// gated activations (cited in k_fused.hip).  When the deferred graph under a root is exactly one
+// of those sequences, and nothing outside reads its interior, a hand-written kernel runs it.
+// Everything else (and every near miss) goes to the generic program path below.
+bool is_bin(const cg_tensor *n, uint8_t ew) { return n->op == N_BIN && n->ew == ew; }
+bool is_un(const cg_tensor *n, uint8_t ew) { return n->op == N_UN && n->ew == ew; }
+bool is_constf(const cg_tensor *n, uint32_t bits) { return n->op == N_CONST && n->cbits == bits; }
+int refs(const cg_tensor *n) { return n->rc.load(); }
+float bits_f(uint32_t b) {
+  float f;
+  std::memcpy(&f, &b, 4);
+  return f;
+}
+enum : uint32_t { F_ONE = 0x3F800000u, F_HALF = 0x3F000000u, F_E = 0x402DF854u, F_TWO = 0x40000000u };
+
+// t (realised, f32 storage) seen as rows of `n` unit-stride elements with one row stride
+bool rows_view(const cg_tensor *t, int64_t *row_stride) {
+  if (t->op != N_REAL || t->stype != ST_F32 || t->rank == 0) return false;
+  const int r = t->rank;
+  if (t->shape[r - 1] != 1 && t->strides[r - 1] != 1) return false;
+  int64_t expect = -1;  // stride the next outer dim must have
+  bool any = false;
+  for (int i = r - 2; i >= 0; --i) {
+    if (t->shape[i] == 1) continue;
+    if (!any) {
+      *row_stride = t->strides[i];
+      expect = t->strides[i] * t->shape[i];
+      any = true;
+    } else {
+      if (t->strides[i] != expect) return false;
+      expect *= t->shape[i];
+    }
+  }
+  if (!any) *row_stride = t->shape[r - 1];
+  return true;
+}
+
+// a realised f32 tensor usable as contiguous rows: itself or a contiguous copy
+int as_rows(cg_backend *be, cg_tensor *t, cg_tensor **out, int64_t *row_stride) {
+  TRY(realize(be, t));
+  if (rows_view(t, row_stride) && (*row_stride % 4 == 0) &&
+      ((uintptr_t)data_ptr(t) % 16 == 0)) {
+    *out = retain(t);
+    return CG_OK;
+  }
+  TRY(materialize(be, t, out));
+  *row_stride = t->shape[t->rank - 1];
+  return CG_OK;
+}
+
+void finish_fused(cg_tensor *n) {
+  n->op = N_REAL;
+  drop_inputs(n);
+}
+
+// nn::softmax (stdlib/nn/mod.rs:162-171) with attention's `/ sqrt(d)` and `+ mask` in front
+int try_softmax(cg_backend *be, cg_tensor *root, bool *done) {
+  if (root->dtype != CG_F32 || root->rank == 0 || !is_bin(root, E_DIV_F)) return CG_OK;
+  cg_tensor *ex = root->in[0], *bs = root->in[1];
+  if (!is_bin(ex, E_POW_F) || refs(ex) != 2 || !is_constf(ex->in[0], F_E)) return CG_OK;
+  if (bs->op != N_BROADCAST || refs(bs) != 1 || !is_row_broadcast(bs, root)) return CG_OK;
+  cg_tensor *sm = bs->in[0];
+  if (sm->op != N_REDUCE || sm->p0 != R_SUM_F || refs(sm) != 1 || sm->in[0] != ex) return CG_OK;
+  cg_tensor *sb = ex->in[1];
+  if (!is_bin(sb, E_SUB_F) || refs(sb) != 1) return CG_OK;
+  cg_tensor *x = sb->in[0], *bm = sb->in[1];
+  if (bm->op != N_BROADCAST || refs(bm) != 1 || !is_row_broadcast(bm, root)) return CG_OK;
+  cg_tensor *mx = bm->in[0];
+  if (mx->op != N_REDUCE || mx->p0 != R_MAX_F || refs(mx) != 1 || mx->in[0] != x) return CG_OK;
+  const int64_t n = root->shape[root->rank - 1];
+  if (n == 0 || n > 16384 || root->size() >= ((int64_t)1 << 31)) return CG_OK;
+
+  SoftmaxDesc d;
+  std::memset(&d, 0, sizeof(d));
+  cg_tensor *src = x, *mask = nullptr;
+  if (x->op != N_REAL && refs(x) == 2) {
+    cg_tensor *y = x;
+    if (is_bin(x, E_ADD_F)) {  // attn + mask
+      cg_tensor *mk = x->in[1];
+      if (mk->op == N_CONST) {
+        d.has_mask_const = 1;
+        d.mask_const = bits_f(mk->cbits);
+      } else {
+        mask = mk;
+      }
+      y = x->in[0];
+      src = y;
+    }
+    if (is_bin(y, E_DIV_F) && y->in[1]->op == N_CONST && (y == x || refs(y) == 1)) {  // attn / sqrt(d)
+      d.has_scale = 1;
+      d.scale = bits_f(y->in[1]->cbits);
+      src = y->in[0];
+    }
+  }
+  cg_tensor *xs = nullptr, *ms = nullptr;
+  int64_t row_stride = 0;
+  TRY(as_rows(be, src, &xs, &row_stride));
+  int st = CG_OK;
+  if (mask) {
+    st = realize(be, mask);
+    if (!st) {
+      // rows of the mask: the leading dims must fold into (group, row)
+      const int r = mask->rank;
+      std::vector<int64_t> sz, sd;
+      for (int i = 0; i + 1 < r; ++i) {
+        if (mask->shape[i] == 1) continue;
+        if (!sz.empty() && sd.back() == mask->strides[i] * mask->shape[i]) {
+          sz.back() *= mask->shape[i];
+          sd.back() = mask->strides[i];
+        } else {
+          sz.push_back(mask->shape[i]);
+          sd.push_back(mask->strides[i]);
+        }
+      }
+      if (mask->stype != ST_F32 || sz.size() > 2) {
+        st = materialize(be, mask, &ms);
+        if (!st) {
+          d.mask = (const float *)data_ptr(ms);
+          d.mask_rows = (uint32_t)(root->size() / n);
+          d.mask_row_stride = n;
+          d.mask_col_stride = 1;
+        }
+      } else {
+        d.mask = (const float *)data_ptr(mask);
+        d.mask_col_stride = mask->strides[r - 1];
+        if (sz.size() == 2) {
+          d.mask_rows = (uint32_t)sz[1];
+          d.mask_row_stride = sd[1];
+          d.mask_group_stride = sd[0];
+        } else if (sz.size() == 1) {
+          d.mask_rows = (uint32_t)sz[0];
+          d.mask_row_stride = sd[0];
+        } else {
+          d.mask_rows = 1;
+        }
+      }
+    }
+  }
+  if (!st) st = alloc_result(be, root, ST_F32);
+  if (!st) {
+    d.x = (const float *)data_ptr(xs);
+    d.y = (float *)root->st->ptr;
+    d.x_row_stride = row_stride;
+    d.rows = (uint32_t)(root->size() / n);
+    d.n = (uint32_t)n;
+    KernelScope ks(be, "softmax_fused", (double)root->size() * 8, 0);
+    hipError_t e = launch_softmax(be->lc(), d);
+    if (e != hipSuccess) st = fail(be, CG_ERR_DEVICE, hipGetErrorString(e));
+  }
+  node_release(xs);
+  node_release(ms);
+  if (st) return st;
+  finish_fused(root);
+  *done = true;
+  return CG_OK;
+}
+
+// rmsnorm_raw / rmsnorm (catgrad-llm/src/helpers.rs:120-145; gemma3.rs:41-68)
+int try_rmsnorm(cg_backend *be, cg_tensor *root, bool *done) {
+  if (root->dtype != CG_F32 || root->rank == 0) return CG_OK;
+  cg_tensor *dv = root, *gb = nullptr;
+  float gamma_offset = 0.f;
+  if (is_bin(root, E_MUL_F) && is_bin(root->in[0], E_DIV_F) && refs(root->in[0]) == 1) {
+    dv = root->in[0];
+    gb = root->in[1];
+    if (is_bin(gb, E_ADD_F) && refs(gb) == 1 && is_constf(gb->in[0], F_ONE)) {  // (1 + gamma)
+      gamma_offset = 1.f;
+      gb = gb->in[1];
+    }
+  }
+  if (!is_bin(dv, E_DIV_F)) return CG_OK;
+  cg_tensor *x = dv->in[0], *br = dv->in[1];
+  if (br->op != N_BROADCAST || refs(br) != 1 || !is_row_broadcast(br, root)) return CG_OK;
+  cg_tensor *r = br->in[0];
+  if (!is_bin(r, E_POW_F) || refs(r) != 1 || !is_constf(r->in[1], F_HALF)) return CG_OK;
+  cg_tensor *a = r->in[0];
+  if (!is_bin(a, E_ADD_F) || refs(a) != 1 || a->in[1]->op != N_CONST) return CG_OK;
+  cg_tensor *mn = a->in[0];
+  if (!is_bin(mn, E_DIV_F) || refs(mn) != 1 || mn->in[1]->op != N_CONST) return CG_OK;
+  cg_tensor *sm = mn->in[0];
+  if (sm->op != N_REDUCE || sm->p0 != R_SUM_F || refs(sm) != 1) return CG_OK;
+  cg_tensor *sq = sm->in[0];
+  if (!is_bin(sq, E_MUL_F) || refs(sq) != 1 || sq->in[0] != x || sq->in[1] != x) return CG_OK;
+  const int64_t n = root->shape[root->rank - 1];
+  if (n == 0 || n % 4 || n > 16384) return CG_OK;
+
+  RmsNormDesc d;
+  std::memset(&d, 0, sizeof(d));
+  d.eps = bits_f(a->in[1]->cbits);
+  d.n_as_float = bits_f(mn->in[1]->cbits);
+  d.gamma_offset = gamma_offset;
+  cg_tensor *gs = nullptr;
+  if (gb) {
+    TRY(realize(be, gb));
+    bool vec = gb->stype == ST_F32 && (gb->shape[gb->rank - 1] == 1 || gb->strides[gb->rank - 1] == 1) &&
+               ((uintptr_t)data_ptr(gb) % 16 == 0);
+    for (int i = 0; i + 1 < gb->rank; ++i)
+      if (gb->shape[i] != 1 && gb->strides[i] != 0) vec = false;
+    if (!vec) return CG_OK;  // gamma is not a broadcast row vector: generic path
+    gs = gb;
+  }
+  cg_tensor *xs = nullptr;
+  int64_t row_stride = 0;
+  TRY(as_rows(be, x, &xs, &row_stride));
+  int st = alloc_result(be, root, ST_F32);
+  if (!st) {
+    d.x = (const float *)data_ptr(xs);
+    d.gamma = gs ? (const float *)data_ptr(gs) : nullptr;
+    d.y = (float *)root->st->ptr;
+    d.x_row_stride = row_stride;
+    d.rows = (uint32_t)(root->size() / n);
+    d.n = (uint32_t)n;
+    KernelScope ks(be, "rmsnorm_fused", (double)root->size() * 8 + n * 4, 0);
+    hipError_t e = launch_rmsnorm(be->lc(), d);
+    if (e != hipSuccess) st = fail(be, CG_ERR_DEVICE, hipGetErrorString(e));
+  }
+  node_release(xs);
+  if (st) return st;
+  finish_fused(root);
+  *done = true;
+  return CG_OK;
+}
+
+// apply_rope_embedding (catgrad-llm/src/helpers.rs:195-221): cos * x + sin * rotate_half(x)
+int try_rope(cg_backend *be, cg_tensor *root, bool *done) {
+  if (root->dtype != CG_F32 || root->rank != 4 || !is_bin(root, E_ADD_F)) return CG_OK;
+  cg_tensor *m1 = root->in[0], *m2 = root->in[1];
+  if (!is_bin(m1, E_MUL_F) || !is_bin(m2, E_MUL_F) || refs(m1) != 1 || refs(m2) != 1) return CG_OK;
+  cg_tensor *cb = m1->in[0], *x = m1->in[1], *sb = m2->in[0], *rot = m2->in[1];
+  if (rot->op != N_CONCAT || rot->p0 != 3 || refs(rot) != 1) return CG_OK;
+  cg_tensor *ng = rot->in[0], *lo = rot->in[1];
+  if (!is_un(ng, E_NEG_F) || refs(ng) != 1) return CG_OK;
+  cg_tensor *hi = ng->in[0];
+  const int64_t dim = root->shape[3], half = dim / 2;
+  if (dim % 8 || hi->shape[3] != half || lo->shape[3] != half) return CG_OK;
+  // the two halves are slices of x along the last axis: still deferred, or (x already in
+  // memory) views created on the spot
+  auto half_of = [&](const cg_tensor *t, int64_t start) {
+    if (t->op == N_SLICE) return t->in[0] == x && t->p0 == 3 && t->p1 == start && refs(t) == 1;
+    if (t->op != N_REAL || x->op != N_REAL || t->st != x->st) return false;
+    for (int i = 0; i < 4; ++i)
+      if (t->strides[i] != x->strides[i] && t->shape[i] != 1) return false;
+    return t->offset == x->offset + start * x->strides[3];
+  };
+  if (!half_of(hi, half) || !half_of(lo, 0)) return CG_OK;
+  if (root->size() >= ((int64_t)1 << 31)) return CG_OK;
+
+  TRY(realize(be, cb));
+  TRY(realize(be, sb));
+  TRY(realize(be, x));
+  auto table_ok = [&](const cg_tensor *t) {
+    return t->stype == ST_F32 && t->strides[0] * (t->shape[0] != 1) == 0 &&
+           t->strides[1] * (t->shape[1] != 1) == 0 && t->strides[3] == 1 && t->strides[2] % 4 == 0 &&
+           (uintptr_t)data_ptr(t) % 16 == 0;
+  };
+  if (!table_ok(cb) || !table_ok(sb) || cb->strides[2] != sb->strides[2]) return CG_OK;
+  cg_tensor *xs = retain(x);
+  bool ok = x->stype == ST_F32 && x->strides[3] == 1 && (uintptr_t)data_ptr(x) % 16 == 0;
+  for (int i = 0; i < 3; ++i)
+    if (x->strides[i] % 4) ok = false;
+  if (!ok) {
+    node_release(xs);
+    xs = nullptr;
+    TRY(materialize(be, x, &xs));
+  }
+  int st = alloc_result(be, root, ST_F32);
+  if (!st) {
+    RopeDesc d;
+    std::memset(&d, 0, sizeof(d));
+    d.x = (const float *)data_ptr(xs);
+    d.cos = (const float *)data_ptr(cb);
+    d.sin = (const float *)data_ptr(sb);
+    d.out = (float *)root->st->ptr;
+    d.x_sb = xs->strides[0];
+    d.x_sh = xs->strides[1];
+    d.x_ss = xs->strides[2];
+    d.cs_ss = root->shape[2] == 1 ? 0 : cb->strides[2];
+    d.b = (uint32_t)root->shape[0];
+    d.h = (uint32_t)root->shape[1];
+    d.s = (uint32_t)root->shape[2];
+    d.dim = (uint32_t)dim;
+    d.half = (uint32_t)half;
+    KernelScope ks(be, "rope_fused", (double)root->size() * 8, 0);
+    hipError_t e = launch_rope(be->lc(), d);
+    if (e != hipSuccess) st = fail(be, CG_ERR_DEVICE, hipGetErrorString(e));
+  }
+  node_release(xs);
+  if (st) return st;
+  finish_fused(root);
+  *done = true;
+  return CG_OK;
+}
+
+// nn::sigmoid as emitted: one / (one + exp(-g)) (stdlib/nn/mod.rs:130-136)
+bool is_sigmoid_of(const cg_tensor *s, const cg_tensor **arg) {
+  if (!is_bin(s, E_DIV_F) || refs(s) != 1 || !is_constf(s->in[0], F_ONE)) return false;
+  const cg_tensor *ad = s->in[1];
+  if (!is_bin(ad, E_ADD_F) || refs(ad) != 1 || !is_constf(ad->in[0], F_ONE)) return false;
+  const cg_tensor *pw = ad->in[1];
+  if (!is_bin(pw, E_POW_F) || refs(pw) != 1 || !is_constf(pw->in[0], F_E)) return false;
+  const cg_tensor *ng = pw->in[1];
+  if (!is_un(ng, E_NEG_F) || refs(ng) != 1) return false;
+  *arg = ng->in[0];
+  return true;
+}
+
+// nn::gelu as emitted (stdlib/nn/mod.rs:138-160):
+//   half * x * (one + (two * sigmoid(two * (c * (x + k * pow(x, three)))) - one))
+bool is_gelu_of(const cg_tensor *g, const cg_tensor **arg) {
+  if (!is_bin(g, E_MUL_F) || refs(g) != 1) return false;
+  const cg_tensor *hx = g->in[0], *op = g->in[1];
+  if (!is_bin(hx, E_MUL_F) || refs(hx) != 1 || !is_constf(hx->in[0], F_HALF)) return false;
+  const cg_tensor *x = hx->in[1];
+  if (!is_bin(op, E_ADD_F) || refs(op) != 1 || !is_constf(op->in[0], F_ONE)) return false;
+  const cg_tensor *th = op->in[1];
+  if (!is_bin(th, E_SUB_F) || refs(th) != 1 || !is_constf(th->in[1], F_ONE)) return false;
+  const cg_tensor *ts = th->in[0];
+  if (!is_bin(ts, E_MUL_F) || refs(ts) != 1 || !is_constf(ts->in[0], F_TWO)) return false;
+  const cg_tensor *sa = nullptr;
+  if (!is_sigmoid_of(ts->in[1], &sa)) return false;
+  if (!is_bin(sa, E_MUL_F) || refs(sa) != 1 || !is_constf(sa->in[0], F_TWO)) return false;
+  const cg_tensor *ct = sa->in[1];
+  if (!is_bin(ct, E_MUL_F) || refs(ct) != 1 || (!is_constf(ct->in[0], 0x3F4C4229u) && !is_constf(ct->in[0], 0x3F4C422Au))) return false;  // sqrt(2/pi)
+  const cg_tensor *in = ct->in[1];
+  if (!is_bin(in, E_ADD_F) || refs(in) != 1 || in->in[0] != x) return false;
+  const cg_tensor *kx = in->in[1];
+  if (!is_bin(kx, E_MUL_F) || refs(kx) != 1 || !is_constf(kx->in[0], 0x3D372713u)) return false;  // 0.044715
+  const cg_tensor *pw = kx->in[1];
+  if (!is_bin(pw, E_POW_F) || refs(pw) != 1 || pw->in[0] != x || !is_constf(pw->in[1], 0x40400000u)) return false;
+  *arg = x;
+  return true;
+}
+
+// silu(gate) * up (models/llama.rs:26) and gelu(gate) * up (models/gemma3.rs:28)
+int try_glu(cg_backend *be, cg_tensor *root, bool *done) {
+  if (root->dtype != CG_F32 || !is_bin(root, E_MUL_F) || root->size() % 4) return CG_OK;
+  cg_tensor *act = root->in[0], *up = root->in[1];
+  const cg_tensor *g = nullptr;
+  int gelu = 0;
+  if (is_bin(act, E_MUL_F) && refs(act) == 1 && is_sigmoid_of(act->in[1], &g) && g == act->in[0]) {
+    gelu = 0;
+  } else if (is_gelu_of(act, &g)) {
+    gelu = 1;
+  } else {
+    return CG_OK;
+  }
+  cg_tensor *gate = const_cast<cg_tensor *>(g);
+  cg_tensor *gc = nullptr, *uc = nullptr;
+  TRY(contiguous(be, gate, &gc));
+  int st = contiguous(be, up, &uc);
+  if (!st) st = alloc_result(be, root, ST_F32);
+  if (!st) {
+    KernelScope ks(be, gelu ? "geglu_fused" : "swiglu_fused", (double)root->size() * 12, 0);
+    hipError_t e = launch_glu(be->lc(), gelu, (const float *)data_ptr(gc), (const float *)data_ptr(uc),
+                              (float *)root->st->ptr, (uint64_t)root->size());
+    if (e != hipSuccess) st = fail(be, CG_ERR_DEVICE, hipGetErrorString(e));
+  }
+  node_release(gc);
+  node_release(uc);
+  if (st) return st;
+  finish_fused(root);
+  *done = true;
+  return CG_OK;
+}
+
+// a single f32 add/sub/mul/div of two tensors that are (or will be) in memory anyway
+int try_binary(cg_backend *be, cg_tensor *root, bool *done) {
+  if (root->dtype != CG_F32 || root->op != N_BIN || root->size() % 4 || root->rank == 0) return CG_OK;
+  int op;
+  switch (root->ew) {
+    case E_ADD_F: op = 0; break;
+    case E_SUB_F: op = 1; break;
+    case E_MUL_F: op = 2; break;
+    case E_DIV_F: op = 3; break;
+    default: return CG_OK;
+  }
+  cg_tensor *a = root->in[0], *b = root->in[1];
+  auto leaf = [](const cg_tensor *t) {
+    return t->op != N_CONST && !((t->op == N_BIN || t->op == N_UN) && t->rc.load() == 1);
+  };
+  if (!leaf(a) || !leaf(b)) return CG_OK;
+  TRY(realize(be, a));
+  TRY(realize(be, b));
+  if (a->stype != ST_F32 || b->stype != ST_F32 || !is_contiguous(a) || (uintptr_t)data_ptr(a) % 16 ||
+      (uintptr_t)data_ptr(b) % 16)
+    return CG_OK;
+  uint32_t period = 0;
+  if (!is_contiguous(b)) {
+    // b = a trailing block repeated over the leading dims (a bias / row-vector broadcast)
+    int k = b->rank;
+    int64_t inner = 1;
+    while (k > 0 && (b->shape[k - 1] == 1 || b->strides[k - 1] == inner)) {
+      inner *= b->shape[k - 1];
+      --k;
+    }
+    for (int i = 0; i < k; ++i)
+      if (b->shape[i] != 1 && b->strides[i] != 0) return CG_OK;
+    if (inner % 4 || inner >= ((int64_t)1 << 31)) return CG_OK;
+    period = (uint32_t)inner;
+  }
+  TRY(alloc_result(be, root, ST_F32));
+  {
+    KernelScope ks(be, "binary_f32", (double)root->size() * (period ? 8 : 12) + period * 4.0, 0);
+    HIPCHK(be, launch_binary_f32(be->lc(), op, (const float *)data_ptr(a), (const float *)data_ptr(b),
+                                 (float *)root->st->ptr, (uint64_t)root->size(), period));
+  }
+  finish_fused(root);
+  *done = true;
+  return CG_OK;
+}
+
+int try_patterns(cg_backend *be, cg_tensor *root, bool *done) {
+  if (be->flags & CG_FLAG_NO_PATTERNS) return CG_OK;
+  TRY(try_softmax(be, root, done));
+  if (*done) return CG_OK;
+  TRY(try_rmsnorm(be, root, done));
+  if (*done) return CG_OK;
+  TRY(try_rope(be, root, done));
+  if (*done) return CG_OK;
+  TRY(try_glu(be, root, done));
+  if (*done) return CG_OK;
+  return try_binary(be, root, done);
+}
+
 int realize_ew(cg_backend *be, cg_tensor *n) {
+  bool done = false;
+  TRY(try_patterns(be, n, &done));
+  if (done) return CG_OK;
   int stype = n->dtype == CG_F32 ? ST_F32 : ST_U32;
   int64_t cnt = std::max<int64_t>(n->size(), 1);
   Storage *s = nullptr;
@@ -579,9 +1220,21 @@ int realize_view(cg_backend *be, cg_tensor *n) {
 int realize_reduce(cg_backend *be, cg_tensor *n) {
   cg_tensor *x = n->in[0];
   const int kind = (int)n->p0;
-  EwCompiler c(be);
-  if (ew_inlineable(x)) TRY(c.emit(x, 0, 0, 0, true));
-  else TRY(c.load(x, 0));
+  // the input tree is evaluated inside the reduction when nobody else reads it
+  Region reg;
+  EwCompiler c(be, &reg);
+  bool fused = false;
+  if ((x->op == N_BIN || x->op == N_UN) && x->rc.load() == 1) {
+    TRY(prepare_region(be, x, false, reg));
+    int st = c.compile_root(x);
+    if (!st) fused = true;
+    else if (!c.overflow) return st;
+  }
+  if (!fused) {
+    c = EwCompiler(be, &reg);
+    TRY(c.load(c.final_code, x, 0));
+  }
+  c.flatten();
   std::vector<int64_t> ostr;
   double bytes_in = 0;
   TRY(finish_program(be, c, x->rank, x->shape, nullptr, true, ostr, &bytes_in));
@@ -591,10 +1244,17 @@ int realize_reduce(cg_backend *be, cg_tensor *n) {
   TRY(alloc_result(be, n, n->dtype == CG_F32 ? ST_F32 : ST_U32));
   const bool vec4 = cols % 4 == 0 && cols >= 4;
   const char *name = kind <= R_SUM_U ? "reduce_sum" : kind <= R_MAX_U ? "reduce_max" : "reduce_argmax";
+  const uint32_t chunks = reduce_split_chunks(be->lc(), (uint32_t)rows, (uint32_t)cols);
+  Storage *scratch = nullptr;
+  if (chunks > 1) TRY(dev_alloc(be, (size_t)rows * chunks * 3 * 4, &scratch));
+  hipError_t e;
   {
     KernelScope ks(be, name, bytes_in + (double)rows * 4, 0);
-    HIPCHK(be, launch_reduce(be->lc(), kind, c.p, n->st->ptr, (uint32_t)rows, (uint32_t)cols, vec4));
+    e = launch_reduce(be->lc(), kind, c.p, n->st->ptr, (uint32_t)rows, (uint32_t)cols, vec4,
+                      scratch ? (uint32_t *)scratch->ptr : nullptr, chunks);
   }
+  storage_release(scratch);
+  HIPCHK(be, e);
   n->op = N_REAL;
   drop_inputs(n);
   return CG_OK;
@@ -798,17 +1458,20 @@ int realize_index(cg_backend *be, cg_tensor *n) {
 
 int realize_arange(cg_backend *be, cg_tensor *n) {
   TRY(alloc_result(be, n, ST_U32));
-  EwCompiler c(be);
-  TRY(c.push(E_IOTA, 0, 0));
-  c.p.n_dims = 1;
-  c.p.dims[0] = (uint32_t)n->shape[0];
+  Program p;
+  std::memset(&p, 0, sizeof(p));
+  p.n_instr = 1;
+  p.seg_end[0] = 1;
+  p.code[0].op = E_IOTA;
+  p.n_dims = 1;
+  p.dims[0] = (uint32_t)n->shape[0];
   OutDesc o;
   std::memset(&o, 0, sizeof(o));
   o.ptr = n->st->ptr;
   o.stype = ST_U32;
   o.stride[0] = 1;
   KernelScope ks(be, "ew_arange", (double)n->size() * 4, 0);
-  HIPCHK(be, launch_ew(be->lc(), c.p, o, (uint64_t)n->size(), false));
+  HIPCHK(be, launch_ew(be->lc(), p, o, (uint64_t)n->size(), false));
   n->op = N_REAL;
   return CG_OK;
 }
@@ -869,6 +1532,44 @@ int to_shape(cg_backend *be, const size_t *dims, int rank, int64_t *shape) {
   return CG_OK;
 }
 
+uint32_t host_upow(uint32_t a, uint32_t e) {
+  uint32_t r = 1;
+  while (e) {
+    if (e & 1) r *= a;
+    a *= a;
+    e >>= 1;
+  }
+  return r;
+}
+
+// Exactly specified scalar ops on two host-known constants (IEEE-754 basic operations and
+// comparisons, wrapping integer arithmetic).  pow/sin/cos are left to the device.
+bool fold_binary(EwOp op, uint32_t a, uint32_t b, uint32_t *out) {
+  float x, y, r;
+  std::memcpy(&x, &a, 4);
+  std::memcpy(&y, &b, 4);
+  switch (op) {
+    case E_ADD_F: r = x + y; break;
+    case E_SUB_F: r = x - y; break;
+    case E_MUL_F: r = x * y; break;
+    case E_DIV_F: r = x / y; break;
+    case E_LT_F: r = x < y ? 1.f : 0.f; break;
+    case E_EQ_F: r = x == y ? 1.f : 0.f; break;
+    case E_ADD_U: *out = a + b; return true;
+    case E_SUB_U: *out = a - b; return true;
+    case E_MUL_U: *out = a * b; return true;
+    case E_DIV_U: if (!b) return false; *out = a / b; return true;
+    case E_POW_U: *out = host_upow(a, b); return true;
+    case E_LT_U: *out = a < b ? 1u : 0u; return true;
+    case E_EQ_U: *out = a == b ? 1u : 0u; return true;
+    default: return false;
+  }
+  std::memcpy(out, &r, 4);
+  return true;
+}
+
+cg_tensor *const_node(cg_backend *be, cg_dtype dt, int rank, const int64_t *shape, uint32_t bits);
+
 int binary(cg_backend *be, cg_tensor *a, cg_tensor *b, cg_tensor **out, EwOp f_op, EwOp u_op) {
   TRY(check_args(be, a, b, out));
   if (!b) return fail(be, CG_ERR_ARG, "null argument");
@@ -876,6 +1577,10 @@ int binary(cg_backend *be, cg_tensor *a, cg_tensor *b, cg_tensor **out, EwOp f_o
   if (a->rank != b->rank || !std::equal(a->shape, a->shape + a->rank, b->shape))
     return fail(be, CG_ERR_SHAPE, "Shape mismatch in operation: " + shape_str(a->shape, a->rank) +
                                       " vs " + shape_str(b->shape, b->rank));
+  uint32_t folded;
+  if (a->op == N_CONST && b->op == N_CONST &&
+      fold_binary(a->dtype == CG_F32 ? f_op : u_op, a->cbits, b->cbits, &folded))
+    return finish(be, const_node(be, a->dtype, a->rank, a->shape, folded), out);
   cg_tensor *n = new_node(be, a->dtype, a->rank, a->shape);
   n->op = N_BIN;
   n->ew = a->dtype == CG_F32 ? f_op : u_op;
@@ -939,6 +1644,7 @@ int upload(cg_backend *be, const void *data, size_t n, const int64_t *shape, int
       Program p;
       std::memset(&p, 0, sizeof(p));
       p.n_instr = 1;
+      p.seg_end[0] = 1;
       p.code[0].op = E_LOAD;
       p.n_in = 1;
       p.n_dims = 1;
@@ -1130,6 +1836,9 @@ int cg_cos(cg_backend *be, cg_tensor *x, cg_tensor **out) {
 }
 int cg_neg(cg_backend *be, cg_tensor *x, cg_tensor **out) {
   TRY(check_args(be, x, nullptr, out));
+  if (x->op == N_CONST)
+    return finish(be, const_node(be, x->dtype, x->rank, x->shape,
+                                 x->dtype == CG_F32 ? x->cbits ^ 0x80000000u : 0u - x->cbits), out);
   return unary(be, x, out, x->dtype == CG_F32 ? E_NEG_F : E_NEG_U, x->dtype);
 }
 
@@ -1330,6 +2039,7 @@ int cg_slice(cg_backend *be, cg_tensor *x, size_t dim, size_t start, size_t len,
 int cg_arange(cg_backend *be, size_t end, cg_tensor **out) {
   if (!be || !out) return CG_ERR_ARG;
   int64_t shape[1] = {(int64_t)end};
+  if (end == 1) return finish(be, const_node(be, CG_U32, 1, shape, 0u), out);
   cg_tensor *n = new_node(be, CG_U32, 1, shape);
   n->op = N_ARANGE;
   return finish(be, n, out);

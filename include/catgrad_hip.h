@@ -62,7 +62,10 @@ enum {
    * matmul rounds its operands to bf16 (f32 accumulation).  Everything else stays f32. */
   CG_FLAG_BF16 = 1u,
   /* run every op when it is issued instead of deferring and fusing */
-  CG_FLAG_EAGER = 2u
+  CG_FLAG_EAGER = 2u,
+  /* keep deferring, but never dispatch to the hand-written pattern kernels (softmax, RMSNorm,
+   * RoPE, gated activations): everything goes through the generic fused-program kernels */
+  CG_FLAG_NO_PATTERNS = 4u
 };
 
 #define CG_MAX_RANK 8

@@ -53,3 +53,9 @@ def hip_eager(cg, hip_lib):
 @pytest.fixture(scope="session")
 def hip_bf16(cg, hip_lib):
     return cg.Backend(hip_lib, flags=cg.FLAG_BF16)
+
+
+@pytest.fixture(scope="session")
+def hip_nopat(cg, hip_lib):
+    """Deferred mode with the hand-written pattern kernels switched off (generic programs only)."""
+    return cg.Backend(hip_lib, flags=4)

@@ -48,9 +48,9 @@ def assert_close(ref, got, rtol, scale=None):
     assert not bad.any(), f"max rel err {np.max(err[finite] / (scale[finite] + 1e-30))}"
 
 
-@pytest.fixture(params=["lazy", "eager"])
-def dev(request, hip, hip_eager):
-    return hip if request.param == "lazy" else hip_eager
+@pytest.fixture(params=["lazy", "eager", "nopat"])
+def dev(request, hip, hip_eager, hip_nopat):
+    return {"lazy": hip, "eager": hip_eager, "nopat": hip_nopat}[request.param]
 
 
 SHAPES = [(7,), (4, 4), (3, 5, 8), (2, 3, 4, 5), (1, 1), (257, 3), (64, 128)]
@@ -244,7 +244,8 @@ def test_arange_zeros(cg, oracle, dev):
         assert_bits(d[0], np.zeros((3, 5), npdt))
 
 
-@pytest.mark.parametrize("shape", [(2, 3), (2, 2, 3), (5, 64), (3, 257), (2, 4096), (1, 9000), (7, 1)])
+@pytest.mark.parametrize("shape", [(2, 3), (2, 2, 3), (5, 64), (3, 257), (2, 4096), (1, 9000), (7, 1),
+                                   (1, 128256), (3, 40002)])
 def test_sum_max_argmax(oracle, dev, shape):
     g = rng(sum(shape))
     a = g.standard_normal(shape).astype(np.float32)
@@ -411,3 +412,27 @@ def test_bf16_mode_matmul(cg, oracle, hip_bf16):
     idx = np.array([3, 0, 7, 3], np.uint32)
     got = hip_bf16.numpy(hip_bf16.index(hip_bf16.tensor(w), 0, hip_bf16.tensor(idx)))
     assert_bits(got, rne[idx])
+
+
+def test_row_fusion_layernorm_and_softmax_views(oracle, hip, hip_eager):
+    """Row programs (reduction stages + final segment in one kernel) on strided inputs: softmax of
+    a transposed view, layernorm with gamma/beta broadcasts, and a row value read twice."""
+    import vectors
+    lang, nn, helpers = vectors.lang, vectors.nn, vectors.helpers
+    g = rng(70)
+    x = (g.standard_normal((2, 24, 40)) * 3).astype(np.float32)
+    gamma = g.standard_normal((40,)).astype(np.float32)
+
+    def f(b, x, gamma):
+        xt = lang.transpose(b, 1, 2, x)                         # [2, 40, 24] view
+        sm = nn.softmax(b, xt)
+        ln = helpers.layernorm_raw(b, 1e-5, x)
+        ln = ln * lang.broadcast(b, gamma, lang.shape(b, ln))
+        m = lang.max(b, x)
+        twice = (x - lang.broadcast(b, m, lang.shape(b, x))) * lang.broadcast(b, m, lang.shape(b, x))
+        return sm, ln, twice
+    ref = vectors.run(oracle, f, 3, x, gamma)
+    for dev in (hip, hip_eager):
+        got = vectors.run(dev, f, 3, x, gamma)
+        for r, d in zip(ref, got):
+            assert np.allclose(d, r, rtol=1e-4, atol=2e-6)

@@ -1,0 +1,142 @@
+"""The hand-written pattern kernels (softmax, RMSNorm, RoPE, SwiGLU/GeGLU, single binary op):
+each is checked against the oracle, against the generic program path on the same device, and
+for having actually been dispatched (by kernel name in the backend's trace)."""
+import numpy as np
+import pytest
+
+import vectors
+
+pytestmark = pytest.mark.gpu
+lang, nn, helpers = vectors.lang, vectors.nn, vectors.helpers
+
+
+def run_traced(be, fn, n_out, *arrays, params=None):
+    be.trace(True)
+    be.trace_reset()
+    out = vectors.run(be, fn, n_out, *arrays, params=params)
+    rep = be.trace_report()
+    be.trace(False)
+    return out, set(rep)
+
+
+def check(oracle, hip, hip_nopat, fn, n_out, arrays, kernel, params=None, rtol=1e-4, atol=1e-6):
+    ref = vectors.run(oracle, fn, n_out, *arrays, params=params)
+    got, names = run_traced(hip, fn, n_out, *arrays, params=params)
+    gen, gnames = run_traced(hip_nopat, fn, n_out, *arrays, params=params)
+    assert kernel in names, f"{kernel} not dispatched: {sorted(names)}"
+    assert kernel not in gnames
+    for r, g, h in zip(ref, got, gen):
+        assert np.allclose(g, r, rtol=rtol, atol=atol), np.abs(g - r).max()
+        assert np.allclose(h, r, rtol=rtol, atol=atol), np.abs(h - r).max()
+
+
+@pytest.mark.parametrize("shape", [(1, 1, 2048), (1, 7, 64), (2, 33, 1152), (1, 3, 8192), (5, 16)])
+def test_rmsnorm(oracle, hip, hip_nopat, shape):
+    g = np.random.default_rng(sum(shape))
+    x = (g.standard_normal(shape) * 3).astype(np.float32)
+    if len(shape) == 2:
+        x = x.reshape((1,) + shape)
+    gamma = g.standard_normal(shape[-1]).astype(np.float32)
+    p = {"n.weight": gamma}
+    check(oracle, hip, hip_nopat, lambda b, v: helpers.rmsnorm(b, 1e-5, lang.path(["n"]), v), 1, [x],
+          "rmsnorm_fused", params=p)
+    check(oracle, hip, hip_nopat, lambda b, v: helpers.rmsnorm_raw(b, 1e-6, v), 1, [x], "rmsnorm_fused")
+
+    def gemma(b, v):  # lr * (one + gamma), catgrad-llm/src/models/gemma3.rs:60-68
+        gm = lang.param(b, lang.path(["n", "weight"]))
+        lr = helpers.rmsnorm_raw(b, 1e-6, v)
+        gm = lang.broadcast(b, gm, lang.shape(b, lr))
+        one = lang.constant(b, 1.0, lang.shape(b, gm))
+        return lr * (one + gm)
+    check(oracle, hip, hip_nopat, gemma, 1, [x], "rmsnorm_fused", params=p)
+
+
+def test_rmsnorm_of_strided_rows(oracle, hip, hip_nopat):
+    g = np.random.default_rng(3)
+    x = g.standard_normal((1, 6, 40, 32)).astype(np.float32)
+
+    def f(b, v):  # QK-norm style: rows are slices of a wider tensor
+        s = lang.slice(b, 3, 0, 16, v)
+        s = lang.reshape(b, lang.make_shape(b, 1, 240, 16), s)
+        return helpers.rmsnorm_raw(b, 1e-6, s)
+    check(oracle, hip, hip_nopat, f, 1, [x], "rmsnorm_fused")
+
+
+@pytest.mark.parametrize("shape", [(1, 32, 1, 530), (1, 4, 19, 19), (2, 3, 64, 512), (1, 2, 5, 1500),
+                                   (1, 1, 3, 5000), (3, 60)])
+def test_softmax(oracle, hip, hip_nopat, shape):
+    g = np.random.default_rng(sum(shape))
+    x = (g.standard_normal(shape) * 4).astype(np.float32)
+    check(oracle, hip, hip_nopat, nn.softmax, 1, [x], "softmax_fused", atol=1e-7)
+
+    def scaled(b, a):
+        return nn.softmax(b, a / lang.constant(b, 8.0, lang.shape(b, a)))
+    check(oracle, hip, hip_nopat, scaled, 1, [x], "softmax_fused", atol=1e-7)
+
+
+@pytest.mark.parametrize("s,t", [(19, 19), (64, 64), (1, 530)])
+def test_softmax_scale_and_causal_mask(oracle, hip, hip_nopat, s, t):
+    """attention's `attn / sqrt(d) + broadcast(causal_mask)` (models/llama.rs:97-107); with s = 1
+    the mask folds to the constant -0.0."""
+    g = np.random.default_rng(s * t)
+    x = (g.standard_normal((1, 6, s, t)) * 5).astype(np.float32)
+
+    def f(b, a):
+        sh = lang.shape(b, a)
+        _, _, n, _ = lang.unpack(b, 4, sh)
+        a = a / lang.constant(b, 8.0, sh)
+        mask = lang.broadcast(b, helpers.causal_mask(b, n), sh)
+        return nn.softmax(b, a + mask)
+    check(oracle, hip, hip_nopat, f, 1, [x], "softmax_fused", atol=1e-7)
+
+
+@pytest.mark.parametrize("b,h,s,d,pos", [(1, 32, 1, 64, 17), (1, 8, 24, 64, 0), (2, 4, 9, 256, 3)])
+def test_rope(oracle, hip, hip_nopat, b, h, s, d, pos):
+    g = np.random.default_rng(b + h + s + d)
+    x = g.standard_normal((b, s, h, d)).astype(np.float32)     # as the q projection leaves it
+
+    def f(bl, v):
+        cos, sin = helpers.rope_tables(bl, 500000.0, lang.to_nat(bl, pos + s + 5), d)
+        q = lang.transpose(bl, 1, 2, v)                         # [b, h, s, d] view
+        return helpers.apply_rope_embedding(bl, pos, d, cos, sin, q)
+    check(oracle, hip, hip_nopat, f, 1, [x], "rope_fused", atol=2e-6)
+
+
+@pytest.mark.parametrize("shape", [(1, 1, 8192), (1, 37, 256), (2, 5, 6912)])
+def test_swiglu_geglu(oracle, hip, hip_nopat, shape):
+    g = np.random.default_rng(shape[-1])
+    gate = (g.standard_normal(shape) * 3).astype(np.float32)
+    up = g.standard_normal(shape).astype(np.float32)
+    check(oracle, hip, hip_nopat, lambda b, x, y: nn.silu(b, x) * y, 1, [gate, up], "swiglu_fused")
+    check(oracle, hip, hip_nopat, lambda b, x, y: nn.gelu(b, x) * y, 1, [gate, up], "geglu_fused",
+          atol=2e-6)
+
+
+def test_single_binary_op(oracle, hip, hip_nopat):
+    g = np.random.default_rng(9)
+    x = g.standard_normal((4, 96, 128)).astype(np.float32)
+    y = g.standard_normal((4, 96, 128)).astype(np.float32)
+    bias = g.standard_normal((128,)).astype(np.float32)
+    check(oracle, hip, hip_nopat, lambda b, p, q: p + q, 1, [x, y], "binary_f32", rtol=0, atol=0)
+    check(oracle, hip, hip_nopat, lambda b, p, q: p / q, 1, [x, y], "binary_f32", rtol=0, atol=0)
+    check(oracle, hip, hip_nopat, lambda b, p, v: p + lang.broadcast(b, v, lang.shape(b, p)), 1, [x, bias],
+          "binary_f32", rtol=0, atol=0)
+
+
+def test_near_misses_take_the_generic_path(oracle, hip):
+    """A softmax whose max is read elsewhere, an rmsnorm with a different exponent: same results
+    through the generic programs."""
+    g = np.random.default_rng(10)
+    x = (g.standard_normal((2, 9, 40)) * 2).astype(np.float32)
+
+    def f(b, v):
+        sh = lang.shape(b, v)
+        m = lang.max(b, v)
+        e = nn.exp(b, v - lang.broadcast(b, m, sh))
+        s = lang.sum(b, e)
+        return e / lang.broadcast(b, s, sh), m          # m escapes
+    ref = vectors.run(oracle, f, 2, x)
+    got, names = run_traced(hip, f, 2, x)
+    assert "softmax_fused" not in names
+    for r, d in zip(ref, got):
+        assert np.allclose(d, r, rtol=1e-4, atol=1e-7)

@@ -8,9 +8,9 @@ import vectors
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(params=["lazy", "eager"])
-def dev(request, hip, hip_eager):
-    return hip if request.param == "lazy" else hip_eager
+@pytest.fixture(params=["lazy", "eager", "nopat"])
+def dev(request, hip, hip_eager, hip_nopat):
+    return {"lazy": hip, "eager": hip_eager, "nopat": hip_nopat}[request.param]
 
 
 def test_reference_backend_vectors(dev):
