@@ -226,75 +226,160 @@ __global__ void __launch_bounds__(256) gemm_kernel(GemmDesc g, int a_vec, int b_
 }
 
 // ---- GEMV, B k-contiguous (weights, K^T): y[m, n] = sum_k x[m, k] * B[n, k] ------------------------
-// LPR lanes share one output column; each lane moves 16 bytes of B per step.
-template <typename TB, int LPR, int MROWS>
+// LPR lanes share one output column; each lane moves 16 bytes of B per load and keeps UNROLL
+// loads in flight (HBM latency x bandwidth needs tens of KB outstanding per CU); B is streamed
+// with non-temporal loads, x comes back from L1/L2.
+typedef float f32x4n __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4n __attribute__((ext_vector_type(4)));
+template <typename TB> struct WVec;
+template <> struct WVec<float> {
+  typedef f32x4n type;
+  enum { EPL = 4 };
+  static __device__ __forceinline__ void widen(const f32x4n &q, float (&w)[4]) {
+    w[0] = q.x; w[1] = q.y; w[2] = q.z; w[3] = q.w;
+  }
+};
+template <> struct WVec<uint16_t> {
+  typedef u32x4n type;
+  enum { EPL = 8 };
+  static __device__ __forceinline__ void widen(const u32x4n &q, float (&w)[8]) {
+    w[0] = __uint_as_float(q.x << 16); w[1] = __uint_as_float(q.x & 0xFFFF0000u);
+    w[2] = __uint_as_float(q.y << 16); w[3] = __uint_as_float(q.y & 0xFFFF0000u);
+    w[4] = __uint_as_float(q.z << 16); w[5] = __uint_as_float(q.z & 0xFFFF0000u);
+    w[6] = __uint_as_float(q.w << 16); w[7] = __uint_as_float(q.w & 0xFFFF0000u);
+  }
+};
+
+// R: column groups a wave keeps in flight at once; KSPLIT: waves of a workgroup that share one
+// column group, each taking a contiguous 1/KSPLIT of k (for deep, narrow matrices).
+template <typename TB, int LPR, int MROWS, int R, int KSPLIT>
 __global__ void __launch_bounds__(256) gemv_rowdot_kernel(GemmDesc g, int b_vec, int a_vec) {
-  constexpr int EPL = 16 / sizeof(TB);  // elements per 16-byte load
+  typedef typename WVec<TB>::type VT;
+  constexpr int EPL = WVec<TB>::EPL;  // elements per 16-byte load
+  constexpr int UNROLL = 4;
+  constexpr int CPW = 64 / LPR;       // columns per wave per group
+  __shared__ float red[KSPLIT > 1 ? 4 : 1][R][MROWS][CPW];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int sub = lane % LPR, col_in_wave = lane / LPR;
-  constexpr int CPW = 64 / LPR;  // columns per wave pass
   const uint32_t bz = blockIdx.y, b0 = bz / g.nb1, b1 = bz - b0 * g.nb1;
   const float *A = (const float *)g.a + b0 * g.sa_b0 + b1 * g.sa_b1;
   const TB *B = (const TB *)g.b + b0 * g.sb_b0 + b1 * g.sb_b1;
   float *C = g.c + (uint64_t)bz * g.M * g.N;
-  const uint32_t n_waves = gridDim.x * 4;
-  for (uint32_t nb = (blockIdx.x * 4 + wave) * CPW; nb < g.N; nb += n_waves * CPW) {
-    const uint32_t n = nb + col_in_wave;
-    float acc[MROWS];
+  // a "slot" is one wave (KSPLIT == 1) or one workgroup (KSPLIT == 4)
+  const uint32_t slot = KSPLIT == 1 ? blockIdx.x * 4 + wave : blockIdx.x;
+  const uint32_t n_slots = KSPLIT == 1 ? gridDim.x * 4 : gridDim.x;
+  // this wave's share of k (multiples of the load width)
+  uint32_t k_begin = 0, k_end = g.K;
+  if (KSPLIT > 1) {
+    const uint32_t per = ((g.K + KSPLIT - 1) / KSPLIT + EPL - 1) / EPL * EPL;
+    k_begin = min(g.K, wave * per);
+    k_end = min(g.K, k_begin + per);
+  }
+  const bool fast = b_vec && a_vec && (g.K % EPL == 0);
+  for (uint32_t nb = slot * CPW * R; nb < g.N; nb += n_slots * CPW * R) {
+    float acc[R][MROWS];
 #pragma unroll
-    for (int m = 0; m < MROWS; ++m) acc[m] = 0.f;
-    if (n < g.N) {
-      const TB *brow = B + (int64_t)n * g.sbn;
-      for (uint32_t k = sub * EPL; k < g.K; k += LPR * EPL) {
-        float w[EPL];
-        if (b_vec && k + EPL <= g.K) {
-          if (sizeof(TB) == 4) {
-            float4 q = *(const float4 *)(brow + k);
-            w[0] = q.x; w[1 % EPL] = q.y; w[2 % EPL] = q.z; w[3 % EPL] = q.w;
-          } else {
-            uint4 q = *(const uint4 *)(brow + k);
-            w[0] = __uint_as_float(q.x << 16); w[1 % EPL] = __uint_as_float(q.x & 0xFFFF0000u);
-            w[2 % EPL] = __uint_as_float(q.y << 16); w[3 % EPL] = __uint_as_float(q.y & 0xFFFF0000u);
-            w[4 % EPL] = __uint_as_float(q.z << 16); w[5 % EPL] = __uint_as_float(q.z & 0xFFFF0000u);
-            w[6 % EPL] = __uint_as_float(q.w << 16); w[7 % EPL] = __uint_as_float(q.w & 0xFFFF0000u);
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+      for (int m = 0; m < MROWS; ++m) acc[r][m] = 0.f;
+    if (fast) {
+      for (uint32_t k0 = k_begin + sub * EPL; k0 < k_end; k0 += LPR * EPL * UNROLL) {
+        VT q[R][UNROLL];
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          const uint32_t n = nb + r * CPW + col_in_wave;
+#pragma unroll
+          for (int u = 0; u < UNROLL; ++u) {
+            const uint32_t k = k0 + u * LPR * EPL;
+            if (k < k_end && n < g.N)
+              q[r][u] = __builtin_nontemporal_load((const VT *)(B + (int64_t)n * g.sbn + k));
           }
-        } else {
-#pragma unroll
-          for (int j = 0; j < EPL; ++j) w[j] = k + j < g.K ? widen(brow[k + j]) : 0.f;
         }
 #pragma unroll
-        for (int m = 0; m < MROWS; ++m) {
-          if ((uint32_t)m < g.M) {
-            const float *xr = A + (int64_t)m * g.sam + k;
-            if (a_vec && k + EPL <= g.K) {
+        for (int u = 0; u < UNROLL; ++u) {
+          const uint32_t k = k0 + u * LPR * EPL;
+          if (k < k_end) {
 #pragma unroll
-              for (int j4 = 0; j4 < EPL; j4 += 4) {
-                float4 xv = *(const float4 *)(xr + j4);
-                acc[m] += w[j4] * xv.x + w[j4 + 1] * xv.y + w[j4 + 2] * xv.z + w[j4 + 3] * xv.w;
+            for (int m = 0; m < MROWS; ++m) {
+              if ((uint32_t)m < g.M) {
+                const float *xr = A + (int64_t)m * g.sam + k;
+                float xs[EPL];
+#pragma unroll
+                for (int j4 = 0; j4 < EPL; j4 += 4) {
+                  const float4 xv = *(const float4 *)(xr + j4);
+                  xs[j4] = xv.x; xs[j4 + 1] = xv.y; xs[j4 + 2] = xv.z; xs[j4 + 3] = xv.w;
+                }
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                  if (nb + r * CPW + col_in_wave < g.N) {
+                    float w[EPL];
+                    WVec<TB>::widen(q[r][u], w);
+#pragma unroll
+                    for (int j = 0; j < EPL; ++j) acc[r][m] += w[j] * xs[j];
+                  }
+                }
               }
-            } else {
-#pragma unroll
-              for (int j = 0; j < EPL; ++j)
-                if (k + j < g.K) acc[m] += w[j] * xr[(int64_t)j * g.sak];
             }
+          }
+        }
+      }
+    } else {
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        const uint32_t n = nb + r * CPW + col_in_wave;
+        if (n < g.N) {
+          const TB *brow = B + (int64_t)n * g.sbn;
+          for (uint32_t k = k_begin + sub; k < k_end; k += LPR) {
+            const float w = widen(brow[(int64_t)k * g.sbk]);
+#pragma unroll
+            for (int m = 0; m < MROWS; ++m)
+              if ((uint32_t)m < g.M) acc[r][m] += w * A[(int64_t)m * g.sam + (int64_t)k * g.sak];
           }
         }
       }
     }
 #pragma unroll
-    for (int m = 0; m < MROWS; ++m) {
+    for (int r = 0; r < R; ++r)
 #pragma unroll
-      for (int s = LPR / 2; s >= 1; s >>= 1) acc[m] += __shfl_xor(acc[m], s, 64);
-      if (sub == 0 && n < g.N && (uint32_t)m < g.M) C[(uint64_t)m * g.N + n] = acc[m];
+      for (int m = 0; m < MROWS; ++m)
+#pragma unroll
+        for (int s = LPR / 2; s >= 1; s >>= 1) acc[r][m] += __shfl_xor(acc[r][m], s, 64);
+    if (KSPLIT > 1) {
+      __syncthreads();
+      if (sub == 0)
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+          for (int m = 0; m < MROWS; ++m) red[wave][r][m][col_in_wave] = acc[r][m];
+      __syncthreads();
+      if (wave == 0 && sub == 0) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          const uint32_t n = nb + r * CPW + col_in_wave;
+#pragma unroll
+          for (int m = 0; m < MROWS; ++m)
+            if (n < g.N && (uint32_t)m < g.M)
+              C[(uint64_t)m * g.N + n] = (red[0][r][m][col_in_wave] + red[1][r][m][col_in_wave]) +
+                                         (red[2][r][m][col_in_wave] + red[3][r][m][col_in_wave]);
+        }
+      }
+    } else if (sub == 0) {
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        const uint32_t n = nb + r * CPW + col_in_wave;
+#pragma unroll
+        for (int m = 0; m < MROWS; ++m)
+          if (n < g.N && (uint32_t)m < g.M) C[(uint64_t)m * g.N + n] = acc[r][m];
+      }
     }
   }
 }
 
 // ---- GEMV, B n-contiguous (V of attention): y[m, n] = sum_k x[m, k] * B[k, n] ---------------------
-// 16 column groups of 4 x 16 k-slices per workgroup; slices meet in LDS.
-template <typename TB, int MROWS>
-__global__ void __launch_bounds__(256) gemv_col_kernel(GemmDesc g, int b_vec) {
-  __shared__ float part[16][MROWS][64 + 4];
+// 16 column groups of 4 columns x KS k-slices per workgroup; slices meet in LDS.
+template <typename TB, int MROWS, int KS>
+__global__ void __launch_bounds__(16 * KS) gemv_col_kernel(GemmDesc g, int b_vec) {
+  __shared__ float part[KS][MROWS][64 + 4];
   const int cg = threadIdx.x & 15, ks = threadIdx.x >> 4;
   const uint32_t bz = blockIdx.y, b0 = bz / g.nb1, b1 = bz - b0 * g.nb1;
   const float *A = (const float *)g.a + b0 * g.sa_b0 + b1 * g.sa_b1;
@@ -306,7 +391,7 @@ __global__ void __launch_bounds__(256) gemv_col_kernel(GemmDesc g, int b_vec) {
   for (int m = 0; m < MROWS; ++m)
 #pragma unroll
     for (int j = 0; j < 4; ++j) acc[m][j] = 0.f;
-  for (uint32_t k = ks; k < g.K; k += 16) {
+  for (uint32_t k = ks; k < g.K; k += KS) {
     const TB *brow = B + (int64_t)k * g.sbk + n;
     float w[4];
     if (b_vec && n + 4 <= g.N) {
@@ -336,11 +421,11 @@ __global__ void __launch_bounds__(256) gemv_col_kernel(GemmDesc g, int b_vec) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) part[ks][m][cg * 4 + j] = acc[m][j];
   __syncthreads();
-  for (int o = threadIdx.x; o < MROWS * 64; o += 256) {
+  for (int o = threadIdx.x; o < MROWS * 64; o += 16 * KS) {
     const int m = o / 64, c = o % 64;
     float s = 0.f;
 #pragma unroll
-    for (int q = 0; q < 16; ++q) s += part[q][m][c];
+    for (int q = 0; q < KS; ++q) s += part[q][m][c];
     const uint32_t col = blockIdx.x * 64 + c;
     if ((uint32_t)m < g.M && col < g.N) C[(uint64_t)m * g.N + col] = s;
   }
@@ -393,22 +478,28 @@ static void launch_gemm_layout(const LaunchCtx &lc, const GemmDesc &g, dim3 grid
 template <typename TB, int MROWS>
 static void launch_rowdot(const LaunchCtx &lc, const GemmDesc &g, int bv, int av) {
   constexpr int EPL = 16 / sizeof(TB);
+  constexpr int R = MROWS == 1 ? 2 : 1;
   const uint32_t batch = g.nb0 * g.nb1;
   uint32_t lanes = (g.K + EPL - 1) / EPL;
   int lpr = lanes >= 64 ? 64 : lanes >= 32 ? 32 : lanes >= 16 ? 16 : 8;
-  // enough waves to cover the CUs a few times over, at least one column pass per wave
-  uint32_t cpw = 64 / lpr;
-  uint32_t waves_needed = (g.N + cpw - 1) / cpw;
-  uint32_t blocks = (waves_needed + 3) / 4;
-  uint32_t cap = (uint32_t)lc.n_cus * 8;
+  const uint32_t cpw = 64 / lpr;
+  const uint32_t groups = (g.N + cpw * R - 1) / (cpw * R);  // column groups of one wave-pass
+  // deep and narrow (down_proj: K = 8192, N = 2048): four waves share a column group
+  const bool ksplit = lpr == 64 && g.K >= 4096 && (uint64_t)groups * batch <= (uint64_t)lc.n_cus * 16;
+  uint32_t blocks = ksplit ? groups : (groups + 3) / 4;
+  const uint32_t cap = (uint32_t)lc.n_cus * 16;
   if ((uint64_t)blocks * batch > cap) blocks = (cap + batch - 1) / batch;
   if (blocks < 1) blocks = 1;
   dim3 grid(blocks, batch);
+  if (ksplit) {
+    gemv_rowdot_kernel<TB, 64, MROWS, R, 4><<<grid, 256, 0, lc.stream>>>(g, bv, av);
+    return;
+  }
   switch (lpr) {
-    case 64: gemv_rowdot_kernel<TB, 64, MROWS><<<grid, 256, 0, lc.stream>>>(g, bv, av); break;
-    case 32: gemv_rowdot_kernel<TB, 32, MROWS><<<grid, 256, 0, lc.stream>>>(g, bv, av); break;
-    case 16: gemv_rowdot_kernel<TB, 16, MROWS><<<grid, 256, 0, lc.stream>>>(g, bv, av); break;
-    default: gemv_rowdot_kernel<TB, 8, MROWS><<<grid, 256, 0, lc.stream>>>(g, bv, av); break;
+    case 64: gemv_rowdot_kernel<TB, 64, MROWS, R, 1><<<grid, 256, 0, lc.stream>>>(g, bv, av); break;
+    case 32: gemv_rowdot_kernel<TB, 32, MROWS, R, 1><<<grid, 256, 0, lc.stream>>>(g, bv, av); break;
+    case 16: gemv_rowdot_kernel<TB, 16, MROWS, R, 1><<<grid, 256, 0, lc.stream>>>(g, bv, av); break;
+    default: gemv_rowdot_kernel<TB, 8, MROWS, R, 1><<<grid, 256, 0, lc.stream>>>(g, bv, av); break;
   }
 }
 
@@ -441,11 +532,12 @@ hipError_t launch_matmul(const LaunchCtx &lc, const GemmDesc &g, const char **ke
       if (kernel_name) *kernel_name = g.b_stype == ST_BF16 ? "gemv_col_bf16" : "gemv_col_f32";
       dim3 grid((g.N + 63) / 64, batch);
       if (g.M == 1) {
-        if (g.b_stype == ST_BF16) gemv_col_kernel<uint16_t, 1><<<grid, 256, 0, lc.stream>>>(g, bv);
-        else gemv_col_kernel<float, 1><<<grid, 256, 0, lc.stream>>>(g, bv);
+        // one output row: 64 k-slices per workgroup keep enough loads in flight
+        if (g.b_stype == ST_BF16) gemv_col_kernel<uint16_t, 1, 64><<<grid, 1024, 0, lc.stream>>>(g, bv);
+        else gemv_col_kernel<float, 1, 64><<<grid, 1024, 0, lc.stream>>>(g, bv);
       } else {
-        if (g.b_stype == ST_BF16) gemv_col_kernel<uint16_t, 8><<<grid, 256, 0, lc.stream>>>(g, bv);
-        else gemv_col_kernel<float, 8><<<grid, 256, 0, lc.stream>>>(g, bv);
+        if (g.b_stype == ST_BF16) gemv_col_kernel<uint16_t, 8, 16><<<grid, 256, 0, lc.stream>>>(g, bv);
+        else gemv_col_kernel<float, 8, 16><<<grid, 256, 0, lc.stream>>>(g, bv);
       }
       return hipGetLastError();
     }

@@ -1289,29 +1289,87 @@ bool collapse_batch(int nb, const int64_t *bshape, const int64_t *sa, const int6
   return true;
 }
 
-bool matrix_ok(const cg_tensor *t) {
-  const int r = t->rank;
-  const int64_t rows = t->shape[r - 2], cols = t->shape[r - 1];
-  const int64_t sr = t->strides[r - 2], sc = t->strides[r - 1];
-  return sc == 1 || cols == 1 || sr == 1 || rows == 1;
+// A matmul operand as the kernels see it: a realised tensor plus the shape/strides to read it
+// with (which may differ from the tensor's own when a repeat_kv chain was peeled off).
+struct MatOperand {
+  cg_tensor *t = nullptr;  // retained
+  int rank = 0;
+  int64_t shape[CG_MAX_RANK + 1], strides[CG_MAX_RANK + 1];
+  void set(cg_tensor *x) {
+    node_release(t);
+    t = x;
+    rank = x->rank;
+    std::copy(x->shape, x->shape + rank, shape);
+    std::copy(x->strides, x->strides + rank, strides);
+  }
+  ~MatOperand() { node_release(t); }
+};
+
+// repeat_kv (catgrad-llm/src/helpers.rs:147-161) leaves K and V as
+//   reshape([b, kv*rep, s, d]) <- broadcast([b, kv, rep, s, d]) <- reshape([b, kv, 1, s, d]) <- x
+// optionally under transpose(2, 3).  Instead of materialising rep copies, the 5-d broadcast
+// view (stride 0 along rep) is handed to the GEMM as three batch dims.
+int peel_repeat_kv(cg_backend *be, cg_tensor *t, MatOperand *out, bool *peeled) {
+  *peeled = false;
+  bool tr = false;
+  if (t->op == N_TRANSPOSE && refs(t) == 1 && t->rank == 4 &&
+      ((t->p0 == 2 && t->p1 == 3) || (t->p0 == 3 && t->p1 == 2))) {
+    tr = true;
+    t = t->in[0];
+  }
+  if (t->op != N_RESHAPE || refs(t) != 1 || t->rank != 4) return CG_OK;
+  cg_tensor *u = t->in[0];
+  if (u->rank != 5 || u->shape[0] != t->shape[0] || u->shape[1] * u->shape[2] != t->shape[1] ||
+      u->shape[3] != t->shape[2] || u->shape[4] != t->shape[3])
+    return CG_OK;
+  TRY(realize(be, u));
+  out->set(retain(u));
+  if (tr) {
+    std::swap(out->shape[3], out->shape[4]);
+    std::swap(out->strides[3], out->strides[4]);
+  }
+  *peeled = true;
+  return CG_OK;
+}
+
+// view a rank-4 operand [b, h, r, c] as [b, h / rep, rep, r, c]
+void split_heads(MatOperand *o, int64_t rep) {
+  for (int i = 4; i >= 2; --i) {
+    o->shape[i] = o->shape[i - 1];
+    o->strides[i] = o->strides[i - 1];
+  }
+  o->shape[2] = rep;
+  o->shape[1] = o->shape[1] / rep;
+  o->strides[2] = o->strides[1];  // one head
+  o->strides[1] = o->strides[2] * rep;
+  o->rank = 5;
+}
+
+bool matrix_ok(const MatOperand &o) {
+  const int r = o.rank;
+  return o.strides[r - 1] == 1 || o.shape[r - 1] == 1 || o.strides[r - 2] == 1 || o.shape[r - 2] == 1;
 }
 
 int realize_matmul(cg_backend *be, cg_tensor *n) {
-  cg_tensor *a = nullptr, *b = nullptr;
-  TRY(realize(be, n->in[0]));
-  TRY(realize(be, n->in[1]));
-  a = retain(n->in[0]);
-  b = retain(n->in[1]);
-  struct Guard {
-    cg_tensor *&a, *&b;
-    ~Guard() {
-      node_release(a);
-      node_release(b);
-    }
-  } guard{a, b};
-  const int r = a->rank;
-  const uint32_t M = (uint32_t)a->shape[r - 2], K = (uint32_t)a->shape[r - 1],
-                 N = (uint32_t)b->shape[r - 1];
+  MatOperand A, B;
+  bool pa = false, pb = false;
+  if (n->dtype == CG_F32 && n->rank == 4) {
+    TRY(peel_repeat_kv(be, n->in[1], &B, &pb));
+    if (!pb) TRY(peel_repeat_kv(be, n->in[0], &A, &pa));
+  }
+  if (!pa) {
+    TRY(realize(be, n->in[0]));
+    A.set(retain(n->in[0]));
+  }
+  if (!pb) {
+    TRY(realize(be, n->in[1]));
+    B.set(retain(n->in[1]));
+  }
+  if (pb) split_heads(&A, B.shape[2]);
+  if (pa) split_heads(&B, A.shape[2]);
+  const int r = n->rank;
+  const uint32_t M = (uint32_t)n->shape[r - 2], N = (uint32_t)n->shape[r - 1],
+                 K = (uint32_t)A.shape[A.rank - 1];
   TRY(alloc_result(be, n, n->dtype == CG_F32 ? ST_F32 : ST_U32));
   const int64_t batch = (int64_t)M * N ? n->size() / ((int64_t)M * N) : 0;
   if (n->size() == 0) {
@@ -1321,56 +1379,56 @@ int realize_matmul(cg_backend *be, cg_tensor *n) {
   }
   if (n->dtype == CG_U32) {
     cg_tensor *ac = nullptr, *bc = nullptr;
-    TRY(contiguous(be, a, &ac));
-    node_release(a);
-    a = ac;
-    TRY(contiguous(be, b, &bc));
-    node_release(b);
-    b = bc;
+    TRY(contiguous(be, A.t, &ac));
+    A.set(ac);
+    TRY(contiguous(be, B.t, &bc));
+    B.set(bc);
     KernelScope ks(be, "matmul_u32", 0, 2.0 * batch * M * N * K);
-    HIPCHK(be, launch_matmul_u32(be->lc(), (const uint32_t *)data_ptr(a), (const uint32_t *)data_ptr(b),
+    HIPCHK(be, launch_matmul_u32(be->lc(), (const uint32_t *)data_ptr(A.t), (const uint32_t *)data_ptr(B.t),
                                  (uint32_t *)n->st->ptr, (uint32_t)batch, M, N, K));
   } else {
     GemmDesc g;
     std::memset(&g, 0, sizeof(g));
-    if (!matrix_ok(a)) {
+    // an operand with no unit stride in its matrix dims is laid out once (a peeled operand
+    // always has one: it is a view of the cache)
+    if (!matrix_ok(A) && !pa && !pb) {
       cg_tensor *c = nullptr;
-      TRY(materialize(be, a, &c, true));
-      node_release(a);
-      a = c;
+      TRY(materialize(be, A.t, &c, true));
+      A.set(c);
     }
-    if (!matrix_ok(b)) {
+    if (!matrix_ok(B) && !pa && !pb) {
       cg_tensor *c = nullptr;
-      TRY(materialize(be, b, &c, true));
-      node_release(b);
-      b = c;
+      TRY(materialize(be, B.t, &c, true));
+      B.set(c);
     }
     uint32_t nbo[2];
     int64_t sao[2], sbo[2];
-    if (!collapse_batch(r - 2, a->shape, a->strides, b->strides, nbo, sao, sbo)) {
+    bool ok = matrix_ok(A) && matrix_ok(B) &&
+              collapse_batch(A.rank - 2, A.shape, A.strides, B.strides, nbo, sao, sbo);
+    if (!ok) {
+      // fall back to plain contiguous operands of the logical shapes
       cg_tensor *c = nullptr;
-      TRY(materialize(be, a, &c, true));
-      node_release(a);
-      a = c;
+      TRY(materialize(be, n->in[0], &c, true));
+      A.set(c);
       c = nullptr;
-      TRY(materialize(be, b, &c, true));
-      node_release(b);
-      b = c;
-      if (!collapse_batch(r - 2, a->shape, a->strides, b->strides, nbo, sao, sbo))
+      TRY(materialize(be, n->in[1], &c, true));
+      B.set(c);
+      if (!collapse_batch(A.rank - 2, A.shape, A.strides, B.strides, nbo, sao, sbo))
         return fail(be, CG_ERR_INTERNAL, "matmul: batch dims do not collapse");
     }
-    g.a = data_ptr(a);
-    g.b = data_ptr(b);
+    const int ra = A.rank;
+    g.a = data_ptr(A.t);
+    g.b = data_ptr(B.t);
     g.c = (float *)n->st->ptr;
-    g.a_stype = a->stype;
-    g.b_stype = b->stype;
+    g.a_stype = A.t->stype;
+    g.b_stype = B.t->stype;
     g.M = M;
     g.N = N;
     g.K = K;
-    g.sam = a->strides[r - 2];
-    g.sak = a->strides[r - 1];
-    g.sbk = b->strides[r - 2];
-    g.sbn = b->strides[r - 1];
+    g.sam = A.strides[ra - 2];
+    g.sak = A.strides[ra - 1];
+    g.sbk = B.strides[ra - 2];
+    g.sbn = B.strides[ra - 1];
     // a unit extent makes its stride irrelevant: normalise so the kernels see a unit stride
     if (K == 1) g.sak = 1, g.sbk = 1;
     if (M == 1 && g.sak != 1) g.sam = 1;
@@ -1382,17 +1440,17 @@ int realize_matmul(cg_backend *be, cg_tensor *n) {
     g.sb_b0 = sbo[0];
     g.sb_b1 = sbo[1];
     g.bf16_math = (be->flags & CG_FLAG_BF16) ? 1 : 0;
-    if (!g.bf16_math && (a->stype == ST_BF16 || b->stype == ST_BF16))
+    if (!g.bf16_math && (g.a_stype == ST_BF16 || g.b_stype == ST_BF16))
       return fail(be, CG_ERR_INTERNAL, "matmul: bf16 storage without CG_FLAG_BF16");
     // bytes: each operand once (batch-broadcast operands once), output once
-    auto uniq = [&](const cg_tensor *t, const int64_t *sb) {
-      double e = (double)t->shape[r - 2] * t->shape[r - 1];
+    auto uniq = [&](const MatOperand &o, const int64_t *sb) {
+      double e = (double)o.shape[ra - 2] * o.shape[ra - 1];
       if (sb[0]) e *= nbo[0];
       if (sb[1]) e *= nbo[1];
-      return e * esize(t->stype);
+      return e * esize(o.t->stype);
     };
     const char *kname = "gemm";
-    KernelScope ks(be, kname, uniq(a, sao) + uniq(b, sbo) + (double)n->size() * 4,
+    KernelScope ks(be, kname, uniq(A, sao) + uniq(B, sbo) + (double)n->size() * 4,
                    2.0 * batch * M * N * K);
     hipError_t e = launch_matmul(be->lc(), g, &kname);
     ks.rename(kname);
@@ -1403,18 +1461,62 @@ int realize_matmul(cg_backend *be, cg_tensor *n) {
   return CG_OK;
 }
 
+// concat(x, y, dim).  The KV cache grows by `concat(2, cached, new)` once per decode step
+// (catgrad-llm/src/legacy/models/utils.rs:210-228): copying the whole cache every step would cost
+// O(T) traffic per layer, so a small y appended to a large x gets storage with room to grow along
+// `dim`, and when the next concat finds that x is owned by nobody else it writes y in place.
 int realize_concat(cg_backend *be, cg_tensor *n) {
   cg_tensor *x = n->in[0], *y = n->in[1];
   TRY(realize(be, x));
   TRY(realize(be, y));
-  const int keep = (x->stype == ST_BF16 && y->stype == ST_BF16) ? ST_BF16
-                   : (n->dtype == CG_F32 ? ST_F32 : ST_U32);
-  TRY(alloc_result(be, n, keep));
   const int dim = (int)n->p0;
+  const int64_t xd = x->shape[dim], yd = y->shape[dim];
+  const int plain = n->dtype == CG_F32 ? ST_F32 : ST_U32;
+  // (1) append in place
+  if (xd > 0 && yd > 0 && refs(x) == 1 && x->st->rc.load() == 1 && x->st->grow_dim == dim &&
+      xd + yd <= x->st->grow_cap && x->offset == 0 && x->stype == plain) {
+    n->st = x->st;
+    n->st->rc.fetch_add(1);
+    n->stype = plain;
+    n->offset = 0;
+    std::memcpy(n->strides, x->strides, sizeof(n->strides));
+    char *dst = (char *)n->st->ptr + xd * n->strides[dim] * 4;
+    TRY(run_ew(be, y, true, dst, n->strides, plain, "kv_append"));
+    n->op = N_REAL;
+    drop_inputs(n);
+    return CG_OK;
+  }
+  // (2) an append-shaped concat: allocate with capacity along dim
+  if (xd > 0 && yd > 0 && yd * 4 <= xd && x->stype != ST_BF16 && y->stype != ST_BF16 &&
+      n->size() < ((int64_t)1 << 30)) {
+    int64_t cap = 64;
+    while (cap < 2 * (xd + yd)) cap <<= 1;
+    int64_t cshape[CG_MAX_RANK];
+    std::copy(n->shape, n->shape + n->rank, cshape);
+    cshape[dim] = cap;
+    int64_t total = 1;
+    for (int i = 0; i < n->rank; ++i) total *= cshape[i];
+    Storage *s = nullptr;
+    TRY(dev_alloc(be, (size_t)total * 4, &s));
+    s->grow_dim = dim;
+    s->grow_cap = cap;
+    n->st = s;
+    n->stype = plain;
+    n->offset = 0;
+    contiguous_strides(n->rank, cshape, n->strides);
+    TRY(run_ew(be, x, true, s->ptr, n->strides, plain, "ew_concat"));
+    char *dst = (char *)s->ptr + xd * n->strides[dim] * 4;
+    TRY(run_ew(be, y, true, dst, n->strides, plain, "ew_concat"));
+    n->op = N_REAL;
+    drop_inputs(n);
+    return CG_OK;
+  }
+  const int keep = (x->stype == ST_BF16 && y->stype == ST_BF16) ? ST_BF16 : plain;
+  TRY(alloc_result(be, n, keep));
   if (x->size())
     TRY(run_ew(be, x, true, n->st->ptr, n->strides, keep, "ew_concat"));
   if (y->size()) {
-    char *dst = (char *)n->st->ptr + x->shape[dim] * n->strides[dim] * esize(keep);
+    char *dst = (char *)n->st->ptr + xd * n->strides[dim] * esize(keep);
     TRY(run_ew(be, y, true, dst, n->strides, keep, "ew_concat"));
   }
   n->op = N_REAL;

@@ -25,6 +25,9 @@ struct Storage {
   void *ptr = nullptr;
   size_t bytes = 0;  // size class actually allocated
   cg_backend *be = nullptr;
+  // set by concat when the buffer was laid out with spare room along one axis (KV cache)
+  int grow_dim = -1;
+  int64_t grow_cap = 0;
 };
 
 enum NodeOp : uint8_t {

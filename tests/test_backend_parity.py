@@ -436,3 +436,49 @@ def test_row_fusion_layernorm_and_softmax_views(oracle, hip, hip_eager):
         got = vectors.run(dev, f, 3, x, gamma)
         for r, d in zip(ref, got):
             assert np.allclose(d, r, rtol=1e-4, atol=2e-6)
+
+
+def test_concat_append_in_place_keeps_values(dev):
+    """The KV-cache pattern: repeated concat of one row onto a growing tensor.  Storage may be
+    reused in place only when nobody else holds the old value."""
+    g = rng(80)
+    cur = g.standard_normal((1, 2, 8, 4)).astype(np.float32)
+    t = dev.tensor(cur)
+    held = []
+    for step in range(40):
+        y = g.standard_normal((1, 2, 1, 4)).astype(np.float32)
+        new = dev.concat(t, dev.tensor(y), 2)
+        cur = np.concatenate([cur, y], axis=2)
+        if step % 3 == 0:
+            held.append((t, cur[:, :, :-1].copy()))     # an old value somebody still reads
+        t = new
+        if step % 5 == 0:
+            assert_bits(dev.numpy(t), cur)
+    assert_bits(dev.numpy(t), cur)
+    for old, exp in held:
+        assert_bits(dev.numpy(old), exp)
+    # the grown tensor is an ordinary value: views and matmuls read it through its strides
+    w = g.standard_normal((1, 2, 4, 3)).astype(np.float32)
+    out = dev.numpy(dev.matmul(t, dev.tensor(w)))
+    assert np.allclose(out, np.matmul(cur, w), rtol=1e-5, atol=1e-5)
+
+
+def test_repeat_kv_matmul(oracle, dev):
+    """q @ repeat_kv(k)^T and p @ repeat_kv(v) (helpers.rs:147-161, models/llama.rs:95-108)."""
+    import vectors
+    lang, helpers = vectors.lang, vectors.helpers
+    g = rng(81)
+    for s, t in ((1, 37), (5, 5), (70, 70)):
+        q = g.standard_normal((1, 8, s, 16)).astype(np.float32)
+        k = g.standard_normal((1, 2, t, 16)).astype(np.float32)
+        p = g.standard_normal((1, 8, s, t)).astype(np.float32)
+
+        def f(b, q, k, p):
+            kr = helpers.repeat_kv(b, 4, k)
+            return lang.matmul(b, q, lang.transpose(b, 2, 3, kr)), lang.matmul(b, p, kr)
+        ref = vectors.run(oracle, f, 2, q, k, p)
+        got = vectors.run(dev, f, 2, q, k, p)
+        kr = np.repeat(k, 4, axis=1)
+        assert np.allclose(ref[0], q @ kr.transpose(0, 1, 3, 2), rtol=1e-4, atol=1e-4)
+        for r, d in zip(ref, got):
+            assert np.allclose(d, r, rtol=1e-4, atol=1e-4)
