@@ -643,9 +643,9 @@ hipError_t launch_ew(const LaunchCtx &lc, const Program &p, const OutDesc &o, ui
   if (n_elems == 0) return hipSuccess;
   if (vec4) {
     uint64_t groups = n_elems / 4;
-    ew_kernel<4><<<grid_for((groups + 255) / 256, lc), 256, 0, lc.stream>>>(p, o, groups, lc.err_flag);
+    CG_LAUNCH(lc, (ew_kernel<4>), grid_for((groups + 255) / 256, lc), 256, p, o, groups, lc.err_flag);
   } else {
-    ew_kernel<1><<<grid_for((n_elems + 255) / 256, lc), 256, 0, lc.stream>>>(p, o, n_elems,
+    CG_LAUNCH(lc, (ew_kernel<1>), grid_for((n_elems + 255) / 256, lc), 256, p, o, n_elems,
                                                                              lc.err_flag);
   }
   return hipGetLastError();
@@ -659,23 +659,25 @@ static hipError_t launch_reduce_kind(const LaunchCtx &lc, const Program &p, uint
     uint32_t chunk_len = (n + chunks - 1) / chunks;
     chunk_len = (chunk_len + 3) / 4 * 4;  // keep vector groups inside one chunk
     if (vec4)
-      reduce_split_kernel<KIND, 4><<<rows * chunks, 256, 0, lc.stream>>>(p, scratch, rows, n, chunks,
+      CG_LAUNCH(lc, (reduce_split_kernel<KIND, 4>), rows * chunks, 256, p, scratch, rows, n, chunks,
                                                                          chunk_len, lc.err_flag);
     else
-      reduce_split_kernel<KIND, 1><<<rows * chunks, 256, 0, lc.stream>>>(p, scratch, rows, n, chunks,
+      CG_LAUNCH(lc, (reduce_split_kernel<KIND, 1>), rows * chunks, 256, p, scratch, rows, n, chunks,
                                                                          chunk_len, lc.err_flag);
-    reduce_merge_kernel<KIND><<<rows, 64, 0, lc.stream>>>(scratch, out, rows, chunks);
+    LaunchCtx untimed = lc;  // the events stay with the (dominant) split pass
+    untimed.ev_start = untimed.ev_stop = nullptr;
+    CG_LAUNCH(untimed, (reduce_merge_kernel<KIND>), rows, 64, scratch, out, rows, chunks);
     return hipGetLastError();
   }
   const bool block_per_row = n >= 2048;
   if (block_per_row) {
     unsigned g = grid_for(rows, lc);
-    if (vec4) reduce_kernel<KIND, 4, 4><<<g, 256, 0, lc.stream>>>(p, out, rows, n, lc.err_flag);
-    else reduce_kernel<KIND, 1, 4><<<g, 256, 0, lc.stream>>>(p, out, rows, n, lc.err_flag);
+    if (vec4) CG_LAUNCH(lc, (reduce_kernel<KIND, 4, 4>), g, 256, p, out, rows, n, lc.err_flag);
+    else CG_LAUNCH(lc, (reduce_kernel<KIND, 1, 4>), g, 256, p, out, rows, n, lc.err_flag);
   } else {
     unsigned g = grid_for((rows + 3) / 4, lc);
-    if (vec4) reduce_kernel<KIND, 4, 1><<<g, 256, 0, lc.stream>>>(p, out, rows, n, lc.err_flag);
-    else reduce_kernel<KIND, 1, 1><<<g, 256, 0, lc.stream>>>(p, out, rows, n, lc.err_flag);
+    if (vec4) CG_LAUNCH(lc, (reduce_kernel<KIND, 4, 1>), g, 256, p, out, rows, n, lc.err_flag);
+    else CG_LAUNCH(lc, (reduce_kernel<KIND, 1, 1>), g, 256, p, out, rows, n, lc.err_flag);
   }
   return hipGetLastError();
 }
@@ -710,12 +712,12 @@ hipError_t launch_row(const LaunchCtx &lc, const Program &p, const OutDesc &o, u
   // one pass per segment when the row fits: 64 lanes x K chunks x VEC per wave, x4 per workgroup
   if (vec4) {
     const bool block_per_row = n > 64 * 2 * 4 || rows * 8 <= (uint32_t)lc.n_cus;
-    if (block_per_row) row_kernel<4, 2, 4><<<grid_for(rows, lc), 256, 0, lc.stream>>>(p, o, rows, n, lc.err_flag);
-    else row_kernel<4, 2, 1><<<grid_for((rows + 3) / 4, lc), 256, 0, lc.stream>>>(p, o, rows, n, lc.err_flag);
+    if (block_per_row) CG_LAUNCH(lc, (row_kernel<4, 2, 4>), grid_for(rows, lc), 256, p, o, rows, n, lc.err_flag);
+    else CG_LAUNCH(lc, (row_kernel<4, 2, 1>), grid_for((rows + 3) / 4, lc), 256, p, o, rows, n, lc.err_flag);
   } else {
     const bool block_per_row = n > 64 * 4 || rows * 8 <= (uint32_t)lc.n_cus;
-    if (block_per_row) row_kernel<1, 4, 4><<<grid_for(rows, lc), 256, 0, lc.stream>>>(p, o, rows, n, lc.err_flag);
-    else row_kernel<1, 4, 1><<<grid_for((rows + 3) / 4, lc), 256, 0, lc.stream>>>(p, o, rows, n, lc.err_flag);
+    if (block_per_row) CG_LAUNCH(lc, (row_kernel<1, 4, 4>), grid_for(rows, lc), 256, p, o, rows, n, lc.err_flag);
+    else CG_LAUNCH(lc, (row_kernel<1, 4, 1>), grid_for((rows + 3) / 4, lc), 256, p, o, rows, n, lc.err_flag);
   }
   return hipGetLastError();
 }

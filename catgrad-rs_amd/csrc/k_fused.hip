@@ -86,11 +86,11 @@ __global__ void __launch_bounds__(BLOCK) rmsnorm_kernel(RmsNormDesc d) {
 hipError_t launch_rmsnorm(const LaunchCtx &lc, const RmsNormDesc &d) {
   if (!d.rows || !d.n) return hipSuccess;
   // n % 4 == 0 and n <= 16384 are checked by the caller
-  if (d.n <= 256) rmsnorm_kernel<64, 1><<<d.rows, 64, 0, lc.stream>>>(d);
-  else if (d.n <= 1024) rmsnorm_kernel<256, 1><<<d.rows, 256, 0, lc.stream>>>(d);
-  else if (d.n <= 2048) rmsnorm_kernel<256, 2><<<d.rows, 256, 0, lc.stream>>>(d);
-  else if (d.n <= 4096) rmsnorm_kernel<256, 4><<<d.rows, 256, 0, lc.stream>>>(d);
-  else rmsnorm_kernel<1024, 4><<<d.rows, 1024, 0, lc.stream>>>(d);
+  if (d.n <= 256) CG_LAUNCH(lc, (rmsnorm_kernel<64, 1>), d.rows, 64, d);
+  else if (d.n <= 1024) CG_LAUNCH(lc, (rmsnorm_kernel<256, 1>), d.rows, 256, d);
+  else if (d.n <= 2048) CG_LAUNCH(lc, (rmsnorm_kernel<256, 2>), d.rows, 256, d);
+  else if (d.n <= 4096) CG_LAUNCH(lc, (rmsnorm_kernel<256, 4>), d.rows, 256, d);
+  else CG_LAUNCH(lc, (rmsnorm_kernel<1024, 4>), d.rows, 1024, d);
   return hipGetLastError();
 }
 
@@ -147,12 +147,12 @@ __global__ void __launch_bounds__(BLOCK == 64 ? 256 : BLOCK) softmax_kernel(Soft
 hipError_t launch_softmax(const LaunchCtx &lc, const SoftmaxDesc &d) {
   if (!d.rows || !d.n) return hipSuccess;
   // n <= 16384 checked by the caller
-  if (d.n <= 64) softmax_kernel<64, 1><<<(d.rows + 3) / 4, dim3(64, 4), 0, lc.stream>>>(d);
-  else if (d.n <= 256) softmax_kernel<64, 4><<<(d.rows + 3) / 4, dim3(64, 4), 0, lc.stream>>>(d);
-  else if (d.n <= 512) softmax_kernel<64, 8><<<(d.rows + 3) / 4, dim3(64, 4), 0, lc.stream>>>(d);
-  else if (d.n <= 1024) softmax_kernel<256, 4><<<d.rows, 256, 0, lc.stream>>>(d);
-  else if (d.n <= 4096) softmax_kernel<256, 16><<<d.rows, 256, 0, lc.stream>>>(d);
-  else softmax_kernel<1024, 16><<<d.rows, 1024, 0, lc.stream>>>(d);
+  if (d.n <= 64) CG_LAUNCH(lc, (softmax_kernel<64, 1>), (d.rows + 3) / 4, dim3(64, 4), d);
+  else if (d.n <= 256) CG_LAUNCH(lc, (softmax_kernel<64, 4>), (d.rows + 3) / 4, dim3(64, 4), d);
+  else if (d.n <= 512) CG_LAUNCH(lc, (softmax_kernel<64, 8>), (d.rows + 3) / 4, dim3(64, 4), d);
+  else if (d.n <= 1024) CG_LAUNCH(lc, (softmax_kernel<256, 4>), d.rows, 256, d);
+  else if (d.n <= 4096) CG_LAUNCH(lc, (softmax_kernel<256, 16>), d.rows, 256, d);
+  else CG_LAUNCH(lc, (softmax_kernel<1024, 16>), d.rows, 1024, d);
   return hipGetLastError();
 }
 
@@ -188,7 +188,7 @@ hipError_t launch_rope(const LaunchCtx &lc, const RopeDesc &d) {
   const uint64_t total = (uint64_t)d.b * d.h * d.s * (d.dim / 4);
   if (!total) return hipSuccess;
   uint64_t blocks = (total + 255) / 256, cap = (uint64_t)lc.n_cus * 8;
-  rope_kernel<<<(unsigned)(blocks < cap ? blocks : cap), 256, 0, lc.stream>>>(d);
+  CG_LAUNCH(lc, (rope_kernel), (unsigned)(blocks < cap ? blocks : cap), 256, d);
   return hipGetLastError();
 }
 
@@ -225,8 +225,8 @@ hipError_t launch_glu(const LaunchCtx &lc, int gelu, const float *gate, const fl
   const uint64_t n4 = n / 4;
   uint64_t blocks = (n4 + 255) / 256, cap = (uint64_t)lc.n_cus * 8;
   const unsigned grid = (unsigned)(blocks < cap ? blocks : cap);
-  if (gelu) glu_kernel<true><<<grid, 256, 0, lc.stream>>>(gate, up, out, n4);
-  else glu_kernel<false><<<grid, 256, 0, lc.stream>>>(gate, up, out, n4);
+  if (gelu) CG_LAUNCH(lc, (glu_kernel<true>), grid, 256, gate, up, out, n4);
+  else CG_LAUNCH(lc, (glu_kernel<false>), grid, 256, gate, up, out, n4);
   return hipGetLastError();
 }
 
@@ -255,10 +255,10 @@ hipError_t launch_binary_f32(const LaunchCtx &lc, int op, const float *a, const 
   const unsigned grid = (unsigned)(blocks < cap ? blocks : cap);
   const uint32_t p4 = b_period / 4;
   switch (op) {
-    case 0: binary_kernel<0><<<grid, 256, 0, lc.stream>>>(a, b, out, n4, p4); break;
-    case 1: binary_kernel<1><<<grid, 256, 0, lc.stream>>>(a, b, out, n4, p4); break;
-    case 2: binary_kernel<2><<<grid, 256, 0, lc.stream>>>(a, b, out, n4, p4); break;
-    default: binary_kernel<3><<<grid, 256, 0, lc.stream>>>(a, b, out, n4, p4); break;
+    case 0: CG_LAUNCH(lc, (binary_kernel<0>), grid, 256, a, b, out, n4, p4); break;
+    case 1: CG_LAUNCH(lc, (binary_kernel<1>), grid, 256, a, b, out, n4, p4); break;
+    case 2: CG_LAUNCH(lc, (binary_kernel<2>), grid, 256, a, b, out, n4, p4); break;
+    default: CG_LAUNCH(lc, (binary_kernel<3>), grid, 256, a, b, out, n4, p4); break;
   }
   return hipGetLastError();
 }

@@ -225,6 +225,178 @@ __global__ void __launch_bounds__(256) gemm_kernel(GemmDesc g, int a_vec, int b_
     }
 }
 
+// ---- bf16 x bf16 "NT" GEMM: the prefill fast path --------------------------------------------------
+// A[M, K] and B[N, K] both bf16 with unit stride along k (activations are narrowed once by
+// cast_bf16_kernel and the copy is shared by every GEMM that reads them; weights are stored
+// bf16).  BM x BN tile per 256-thread workgroup, 2 x 2 waves, BK = 64.  LDS is double buffered:
+// the global loads of step s+1 are issued before the MFMAs of step s and land in the other
+// buffer after them, one barrier per step.  16-byte global loads, 16-byte LDS reads feeding
+// v_mfma_f32_32x32x16_bf16 directly.
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+typedef __attribute__((ext_vector_type(2))) float f32x2_t;
+
+template <int BM_, int BN_, bool B_KC>
+__global__ void __launch_bounds__(256) gemm_bf16_nt_kernel(GemmDesc g) {
+  constexpr int BK = 64, LD = BK + 8;          // row pitch 144 bytes
+  constexpr int WM = BM_ / 2, WN = BN_ / 2;    // wave tile
+  constexpr int TM = WM / 32, TN = WN / 32;    // MFMA tiles per wave
+  constexpr int ACH = BM_ * BK / 8 / 256, BCH = BN_ * BK / 8 / 256;  // 16-byte chunks per thread
+  __shared__ __attribute__((aligned(16))) uint16_t As[2][BM_ * LD];
+  __shared__ __attribute__((aligned(16))) uint16_t Bs[2][BN_ * LD];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const uint32_t m0 = blockIdx.y * BM_, n0 = blockIdx.x * BN_;
+  // blockIdx.z = split * batch + batch index; split s covers k in [s * k_per, (s + 1) * k_per)
+  const uint32_t batch = g.nb0 * g.nb1;
+  const uint32_t split = blockIdx.z / batch, bz = blockIdx.z - split * batch;
+  const uint32_t b0 = bz / g.nb1, b1 = bz - b0 * g.nb1;
+  const uint16_t *A = (const uint16_t *)g.a + b0 * g.sa_b0 + b1 * g.sa_b1;
+  const uint16_t *B = (const uint16_t *)g.b + b0 * g.sb_b0 + b1 * g.sb_b1;
+  float *C = (g.splits > 1 ? g.workspace + (uint64_t)split * batch * g.M * g.N : g.c) +
+             (uint64_t)bz * g.M * g.N;
+  const uint32_t k_begin = split * g.k_per_split;
+  const uint32_t k_end = min(g.K, k_begin + g.k_per_split);
+
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  uint4 ra[ACH], rb[BCH];
+  auto fetch = [&](uint32_t k0) {
+#pragma unroll
+    for (int c = 0; c < ACH; ++c) {
+      const int chunk = tid + c * 256, row = chunk >> 3, kc = (chunk & 7) * 8;
+      ra[c] = (m0 + row < g.M && k0 + kc < k_end)
+                  ? *(const uint4 *)(A + (int64_t)(m0 + row) * g.sam + k0 + kc)
+                  : make_uint4(0, 0, 0, 0);
+    }
+#pragma unroll
+    for (int c = 0; c < BCH; ++c) {
+      const int chunk = tid + c * 256;
+      if (B_KC) {
+        const int row = chunk >> 3, kc = (chunk & 7) * 8;
+        rb[c] = (n0 + row < g.N && k0 + kc < k_end)
+                    ? *(const uint4 *)(B + (int64_t)(n0 + row) * g.sbn + k0 + kc)
+                    : make_uint4(0, 0, 0, 0);
+      } else {  // B[k, n] with unit stride along n: 8 columns of one k row
+        const int kk = chunk / (BN_ / 8), nc = (chunk % (BN_ / 8)) * 8;
+        rb[c] = (k0 + kk < k_end && n0 + nc < g.N)
+                    ? *(const uint4 *)(B + (int64_t)(k0 + kk) * g.sbk + n0 + nc)
+                    : make_uint4(0, 0, 0, 0);
+      }
+    }
+  };
+  auto stash = [&](int buf) {
+#pragma unroll
+    for (int c = 0; c < ACH; ++c) {
+      const int chunk = tid + c * 256, row = chunk >> 3, kc = (chunk & 7) * 8;
+      *(uint4 *)(&As[buf][row * LD + kc]) = ra[c];
+    }
+#pragma unroll
+    for (int c = 0; c < BCH; ++c) {
+      const int chunk = tid + c * 256;
+      if (B_KC) {
+        const int row = chunk >> 3, kc = (chunk & 7) * 8;
+        *(uint4 *)(&Bs[buf][row * LD + kc]) = rb[c];
+      } else {  // transpose on the way into LDS
+        const int kk = chunk / (BN_ / 8), nc = (chunk % (BN_ / 8)) * 8;
+        const uint32_t w[4] = {rb[c].x, rb[c].y, rb[c].z, rb[c].w};
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+          Bs[buf][(nc + j) * LD + kk] = (uint16_t)(w[j >> 1] >> ((j & 1) * 16));
+      }
+    }
+  };
+
+  const uint32_t n_steps = k_end > k_begin ? (k_end - k_begin + BK - 1) / BK : 0;
+  if (n_steps) {
+    fetch(k_begin);
+    stash(0);
+  }
+  __syncthreads();
+  for (uint32_t s = 0; s < n_steps; ++s) {
+    const int buf = s & 1;
+    if (s + 1 < n_steps) fetch(k_begin + (s + 1) * BK);
+#pragma unroll
+    for (int kk = 0; kk < BK; kk += 16) {
+      bf16x8 af[TM], bfr[TN];
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+        af[i] = *(const bf16x8 *)(&As[buf][(wm * WM + i * 32 + (lane & 31)) * LD + kk + (lane >> 5) * 8]);
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        bfr[j] = *(const bf16x8 *)(&Bs[buf][(wn * WN + j * 32 + (lane & 31)) * LD + kk + (lane >> 5) * 8]);
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
+    }
+    if (s + 1 < n_steps) stash(buf ^ 1);
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const uint32_t col = n0 + wn * WN + j * 32 + (lane & 31);
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const uint32_t row = m0 + wm * WM + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
+        if (row < g.M && col < g.N) C[(uint64_t)row * g.N + col] = acc[i][j][e];
+      }
+    }
+}
+
+// C = sum over splits of workspace[split] (float4 per thread; sizes are multiples of 4 or the
+// tail is handled scalar)
+__global__ void __launch_bounds__(256) splitk_reduce_kernel(const float *ws, float *c, uint64_t n,
+                                                            uint32_t splits) {
+  const uint64_t n4 = n / 4;
+  for (uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x; i < n4;
+       i += (uint64_t)gridDim.x * 256) {
+    float4 s = ((const float4 *)ws)[i];
+    for (uint32_t k = 1; k < splits; ++k) {
+      const float4 v = ((const float4 *)(ws + (uint64_t)k * n))[i];
+      s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+    }
+    ((float4 *)c)[i] = s;
+  }
+  if (blockIdx.x == 0 && threadIdx.x < (n & 3)) {
+    const uint64_t i = n4 * 4 + threadIdx.x;
+    float s = ws[i];
+    for (uint32_t k = 1; k < splits; ++k) s += ws[(uint64_t)k * n + i];
+    c[i] = s;
+  }
+}
+
+// f32 -> bf16 (round to nearest even, v_cvt_pk_bf16_f32), contiguous, 8 elements per thread
+__global__ void __launch_bounds__(256) cast_bf16_kernel(const float *in, uint16_t *out, uint64_t n8) {
+  for (uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x; i < n8;
+       i += (uint64_t)gridDim.x * 256) {
+    const float4 a = ((const float4 *)in)[2 * i], b = ((const float4 *)in)[2 * i + 1];
+    bf16x2_t h0 = __builtin_convertvector((f32x2_t){a.x, a.y}, bf16x2_t);
+    bf16x2_t h1 = __builtin_convertvector((f32x2_t){a.z, a.w}, bf16x2_t);
+    bf16x2_t h2 = __builtin_convertvector((f32x2_t){b.x, b.y}, bf16x2_t);
+    bf16x2_t h3 = __builtin_convertvector((f32x2_t){b.z, b.w}, bf16x2_t);
+    uint4 q;
+    q.x = *(uint32_t *)&h0; q.y = *(uint32_t *)&h1; q.z = *(uint32_t *)&h2; q.w = *(uint32_t *)&h3;
+    ((uint4 *)out)[i] = q;
+  }
+}
+
+hipError_t launch_cast_bf16(const LaunchCtx &lc, const float *in, void *out, uint64_t n) {
+  if (!n) return hipSuccess;
+  const uint64_t n8 = n / 8;
+  uint64_t blocks = (n8 + 255) / 256, cap = (uint64_t)lc.n_cus * 16;
+  CG_LAUNCH(lc, (cast_bf16_kernel), (unsigned)(blocks < cap ? blocks : cap), 256, in, (uint16_t *)out, n8);
+  return hipGetLastError();
+}
+
 // ---- GEMV, B k-contiguous (weights, K^T): y[m, n] = sum_k x[m, k] * B[n, k] ------------------------
 // LPR lanes share one output column; each lane moves 16 bytes of B per load and keeps UNROLL
 // loads in flight (HBM latency x bandwidth needs tens of KB outstanding per CU); B is streamed
@@ -375,6 +547,76 @@ __global__ void __launch_bounds__(256) gemv_rowdot_kernel(GemmDesc g, int b_vec,
   }
 }
 
+// ---- several GEMVs sharing x in one launch (q/k/v and gate/up of a decode step) -------------------
+// Same streaming scheme as gemv_rowdot_kernel<.., 64, 1, 2, 1>; blockIdx.y selects the problem.
+template <typename TB>
+__global__ void __launch_bounds__(256) gemv_multi_kernel(GemvMultiDesc g) {
+  typedef typename WVec<TB>::type VT;
+  constexpr int EPL = WVec<TB>::EPL, UNROLL = 4, R = 2;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const uint32_t N = g.p[blockIdx.y].N;
+  const TB *B = (const TB *)g.p[blockIdx.y].b;
+  const int64_t sbn = g.p[blockIdx.y].sbn;
+  float *C = g.p[blockIdx.y].c;
+  const uint32_t n_waves = gridDim.x * 4;
+  for (uint32_t nb = (blockIdx.x * 4 + wave) * R; nb < N; nb += n_waves * R) {
+    float acc[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) acc[r] = 0.f;
+    for (uint32_t k0 = lane * EPL; k0 < g.K; k0 += 64 * EPL * UNROLL) {
+      VT q[R][UNROLL];
+#pragma unroll
+      for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+          const uint32_t k = k0 + u * 64 * EPL;
+          if (k < g.K && nb + r < N)
+            q[r][u] = __builtin_nontemporal_load((const VT *)(B + (int64_t)(nb + r) * sbn + k));
+        }
+#pragma unroll
+      for (int u = 0; u < UNROLL; ++u) {
+        const uint32_t k = k0 + u * 64 * EPL;
+        if (k < g.K) {
+          float xs[EPL];
+#pragma unroll
+          for (int j4 = 0; j4 < EPL; j4 += 4) {
+            const float4 xv = *(const float4 *)(g.x + k + j4);
+            xs[j4] = xv.x; xs[j4 + 1] = xv.y; xs[j4 + 2] = xv.z; xs[j4 + 3] = xv.w;
+          }
+#pragma unroll
+          for (int r = 0; r < R; ++r) {
+            if (nb + r < N) {
+              float w[EPL];
+              WVec<TB>::widen(q[r][u], w);
+#pragma unroll
+              for (int j = 0; j < EPL; ++j) acc[r] += w[j] * xs[j];
+            }
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+#pragma unroll
+      for (int s = 32; s >= 1; s >>= 1) acc[r] += __shfl_xor(acc[r], s, 64);
+      if (lane == 0 && nb + r < N) C[nb + r] = acc[r];
+    }
+  }
+}
+
+hipError_t launch_gemv_multi(const LaunchCtx &lc, const GemvMultiDesc &g) {
+  uint32_t max_n = 0;
+  for (int i = 0; i < g.n_prob; ++i) max_n = g.p[i].N > max_n ? g.p[i].N : max_n;
+  if (!max_n || !g.n_prob) return hipSuccess;
+  uint32_t blocks = (max_n + 7) / 8;  // 4 waves x 2 columns per workgroup pass
+  const uint32_t cap = (uint32_t)lc.n_cus * 16 / g.n_prob;
+  if (blocks > cap) blocks = cap;
+  dim3 grid(blocks, g.n_prob);
+  if (g.b_stype == ST_BF16) CG_LAUNCH(lc, (gemv_multi_kernel<uint16_t>), grid, 256, g);
+  else CG_LAUNCH(lc, (gemv_multi_kernel<float>), grid, 256, g);
+  return hipGetLastError();
+}
+
 // ---- GEMV, B n-contiguous (V of attention): y[m, n] = sum_k x[m, k] * B[k, n] ---------------------
 // 16 column groups of 4 columns x KS k-slices per workgroup; slices meet in LDS.
 template <typename TB, int MROWS, int KS>
@@ -451,7 +693,7 @@ hipError_t launch_matmul_u32(const LaunchCtx &lc, const uint32_t *a, const uint3
   uint64_t total = (uint64_t)batch * M * N;
   if (!total) return hipSuccess;
   uint64_t blocks = (total + 255) / 256, cap = (uint64_t)lc.n_cus * 8;
-  matmul_u32_kernel<<<(unsigned)(blocks < cap ? blocks : cap), 256, 0, lc.stream>>>(a, b, c, batch,
+  CG_LAUNCH(lc, (matmul_u32_kernel), (unsigned)(blocks < cap ? blocks : cap), 256, a, b, c, batch,
                                                                                    M, N, K);
   return hipGetLastError();
 }
@@ -469,10 +711,10 @@ static int vec_ok(const void *base, int esize, int64_t other_stride, int64_t sb0
 template <typename TA, typename TB, bool BF16>
 static void launch_gemm_layout(const LaunchCtx &lc, const GemmDesc &g, dim3 grid, int av, int bv) {
   const bool akc = g.sak == 1 || g.K == 1, bkc = g.sbk == 1 && !(g.sbn == 1 && g.N > 1 && false);
-  if (akc && bkc) gemm_kernel<TA, TB, true, true, BF16><<<grid, 256, 0, lc.stream>>>(g, av, bv);
-  else if (akc) gemm_kernel<TA, TB, true, false, BF16><<<grid, 256, 0, lc.stream>>>(g, av, bv);
-  else if (bkc) gemm_kernel<TA, TB, false, true, BF16><<<grid, 256, 0, lc.stream>>>(g, av, bv);
-  else gemm_kernel<TA, TB, false, false, BF16><<<grid, 256, 0, lc.stream>>>(g, av, bv);
+  if (akc && bkc) CG_LAUNCH(lc, (gemm_kernel<TA, TB, true, true, BF16>), grid, 256, g, av, bv);
+  else if (akc) CG_LAUNCH(lc, (gemm_kernel<TA, TB, true, false, BF16>), grid, 256, g, av, bv);
+  else if (bkc) CG_LAUNCH(lc, (gemm_kernel<TA, TB, false, true, BF16>), grid, 256, g, av, bv);
+  else CG_LAUNCH(lc, (gemm_kernel<TA, TB, false, false, BF16>), grid, 256, g, av, bv);
 }
 
 template <typename TB, int MROWS>
@@ -492,15 +734,34 @@ static void launch_rowdot(const LaunchCtx &lc, const GemmDesc &g, int bv, int av
   if (blocks < 1) blocks = 1;
   dim3 grid(blocks, batch);
   if (ksplit) {
-    gemv_rowdot_kernel<TB, 64, MROWS, R, 4><<<grid, 256, 0, lc.stream>>>(g, bv, av);
+    CG_LAUNCH(lc, (gemv_rowdot_kernel<TB, 64, MROWS, R, 4>), grid, 256, g, bv, av);
     return;
   }
   switch (lpr) {
-    case 64: gemv_rowdot_kernel<TB, 64, MROWS, R, 1><<<grid, 256, 0, lc.stream>>>(g, bv, av); break;
-    case 32: gemv_rowdot_kernel<TB, 32, MROWS, R, 1><<<grid, 256, 0, lc.stream>>>(g, bv, av); break;
-    case 16: gemv_rowdot_kernel<TB, 16, MROWS, R, 1><<<grid, 256, 0, lc.stream>>>(g, bv, av); break;
-    default: gemv_rowdot_kernel<TB, 8, MROWS, R, 1><<<grid, 256, 0, lc.stream>>>(g, bv, av); break;
+    case 64: CG_LAUNCH(lc, (gemv_rowdot_kernel<TB, 64, MROWS, R, 1>), grid, 256, g, bv, av); break;
+    case 32: CG_LAUNCH(lc, (gemv_rowdot_kernel<TB, 32, MROWS, R, 1>), grid, 256, g, bv, av); break;
+    case 16: CG_LAUNCH(lc, (gemv_rowdot_kernel<TB, 16, MROWS, R, 1>), grid, 256, g, bv, av); break;
+    default: CG_LAUNCH(lc, (gemv_rowdot_kernel<TB, 8, MROWS, R, 1>), grid, 256, g, bv, av); break;
   }
+}
+
+static bool gemm_fast_path(const GemmDesc &g, int av, int bv) {
+  return g.bf16_math && g.M > 8 && g.a_stype == ST_BF16 && g.b_stype == ST_BF16 && g.sak == 1 &&
+         (g.sbk == 1 || g.sbn == 1) && g.K % 8 == 0 && (g.sbk == 1 || g.N % 8 == 0) && av && bv;
+}
+
+// Split-K factor for a problem too small to fill the CUs with 128x128 tiles (0/1 = none).
+// The caller provides g.workspace of splits * batch * M * N floats and sets g.splits/k_per_split.
+uint32_t gemm_split_k(const LaunchCtx &lc, const GemmDesc &g) {
+  const uint32_t batch = g.nb0 * g.nb1;
+  const int asz = g.a_stype == ST_BF16 ? 2 : 4, bsz = g.b_stype == ST_BF16 ? 2 : 4;
+  const int av = vec_ok(g.a, asz, g.sak == 1 ? g.sam : g.sak, g.sa_b0, g.sa_b1);
+  const int bv = vec_ok(g.b, bsz, g.sbk == 1 ? g.sbn : g.sbk, g.sb_b0, g.sb_b1);
+  if (!gemm_fast_path(g, av, bv) || g.N <= 64) return 1;
+  const uint64_t tiles = (uint64_t)((g.M + 127) / 128) * ((g.N + 127) / 128) * batch;
+  uint32_t splits = 1;
+  while (tiles * splits * 2 <= (uint64_t)lc.n_cus && g.K / (splits * 2) >= 512 && splits < 8) splits *= 2;
+  return splits;
 }
 
 hipError_t launch_matmul(const LaunchCtx &lc, const GemmDesc &g, const char **kernel_name) {
@@ -533,16 +794,43 @@ hipError_t launch_matmul(const LaunchCtx &lc, const GemmDesc &g, const char **ke
       dim3 grid((g.N + 63) / 64, batch);
       if (g.M == 1) {
         // one output row: 64 k-slices per workgroup keep enough loads in flight
-        if (g.b_stype == ST_BF16) gemv_col_kernel<uint16_t, 1, 64><<<grid, 1024, 0, lc.stream>>>(g, bv);
-        else gemv_col_kernel<float, 1, 64><<<grid, 1024, 0, lc.stream>>>(g, bv);
+        if (g.b_stype == ST_BF16) CG_LAUNCH(lc, (gemv_col_kernel<uint16_t, 1, 64>), grid, 1024, g, bv);
+        else CG_LAUNCH(lc, (gemv_col_kernel<float, 1, 64>), grid, 1024, g, bv);
       } else {
-        if (g.b_stype == ST_BF16) gemv_col_kernel<uint16_t, 8, 16><<<grid, 256, 0, lc.stream>>>(g, bv);
-        else gemv_col_kernel<float, 8, 16><<<grid, 256, 0, lc.stream>>>(g, bv);
+        if (g.b_stype == ST_BF16) CG_LAUNCH(lc, (gemv_col_kernel<uint16_t, 8, 16>), grid, 256, g, bv);
+        else CG_LAUNCH(lc, (gemv_col_kernel<float, 8, 16>), grid, 256, g, bv);
       }
       return hipGetLastError();
     }
   }
 
+  if (gemm_fast_path(g, av, bv)) {
+    if (kernel_name) *kernel_name = "gemm_mfma_bf16";
+    const bool bkc = g.sbk == 1;
+    const uint32_t splits = g.splits > 1 ? g.splits : 1;
+    GemmDesc gg = g;
+    gg.splits = splits;
+    if (splits == 1) gg.k_per_split = g.K;
+    const uint64_t big_tiles = (uint64_t)((g.M + 127) / 128) * ((g.N + 127) / 128) * batch * splits;
+    if (big_tiles * 2 >= (uint64_t)lc.n_cus && g.N > 64) {
+      dim3 gr((g.N + 127) / 128, (g.M + 127) / 128, batch * splits);
+      if (bkc) CG_LAUNCH(lc, (gemm_bf16_nt_kernel<128, 128, true>), gr, 256, gg);
+      else CG_LAUNCH(lc, (gemm_bf16_nt_kernel<128, 128, false>), gr, 256, gg);
+    } else {
+      dim3 gr((g.N + 63) / 64, (g.M + 63) / 64, batch * splits);
+      if (bkc) CG_LAUNCH(lc, (gemm_bf16_nt_kernel<64, 64, true>), gr, 256, gg);
+      else CG_LAUNCH(lc, (gemm_bf16_nt_kernel<64, 64, false>), gr, 256, gg);
+    }
+    if (splits > 1) {
+      LaunchCtx untimed = lc;
+      untimed.ev_start = untimed.ev_stop = nullptr;
+      const uint64_t n = (uint64_t)batch * g.M * g.N;
+      uint64_t blocks = (n / 4 + 255) / 256, cap = (uint64_t)lc.n_cus * 16;
+      CG_LAUNCH(untimed, (splitk_reduce_kernel), (unsigned)(blocks < cap ? (blocks ? blocks : 1) : cap), 256,
+                (const float *)g.workspace, g.c, n, splits);
+    }
+    return hipGetLastError();
+  }
   dim3 grid((g.N + BN - 1) / BN, (g.M + BM - 1) / BM, batch);
   if (g.bf16_math) {
     if (kernel_name) *kernel_name = "gemm_mfma_bf16";

@@ -76,8 +76,8 @@ hipError_t launch_gather(const LaunchCtx &lc, const GatherDesc &g, uint64_t n_ou
   uint64_t groups = vec ? n_out / 4 : n_out;
   uint64_t blocks = (groups + 255) / 256, cap = (uint64_t)lc.n_cus * 8;
   unsigned grid = (unsigned)(blocks < cap ? blocks : cap);
-  if (vec) gather_kernel<4><<<grid, 256, 0, lc.stream>>>(g, groups, lc.err_flag);
-  else gather_kernel<1><<<grid, 256, 0, lc.stream>>>(g, groups, lc.err_flag);
+  if (vec) CG_LAUNCH(lc, (gather_kernel<4>), grid, 256, g, groups, lc.err_flag);
+  else CG_LAUNCH(lc, (gather_kernel<1>), grid, 256, g, groups, lc.err_flag);
   return hipGetLastError();
 }
 
@@ -128,7 +128,7 @@ __global__ void __launch_bounds__(256) topk_kernel(const float *x, float *values
 hipError_t launch_topk(const LaunchCtx &lc, const float *x, float *values, uint32_t *indices,
                        uint32_t rows, uint32_t n, uint32_t k) {
   if (!rows || !k) return hipSuccess;
-  topk_kernel<<<(rows + 3) / 4, 256, 0, lc.stream>>>(x, values, indices, rows, n, k);
+  CG_LAUNCH(lc, (topk_kernel), (rows + 3) / 4, 256, x, values, indices, rows, n, k);
   return hipGetLastError();
 }
 
@@ -147,7 +147,7 @@ hipError_t launch_compare(const LaunchCtx &lc, const void *a, const void *b, uin
                           int is_f32, uint32_t *flag) {
   if (!n) return hipSuccess;
   uint64_t blocks = (n + 255) / 256, cap = (uint64_t)lc.n_cus * 8;
-  compare_kernel<<<(unsigned)(blocks < cap ? blocks : cap), 256, 0, lc.stream>>>(
+  CG_LAUNCH(lc, (compare_kernel), (unsigned)(blocks < cap ? blocks : cap), 256, 
       (const uint32_t *)a, (const uint32_t *)b, n, is_f32, flag);
   return hipGetLastError();
 }
@@ -161,7 +161,7 @@ __global__ void __launch_bounds__(256) fill_kernel(uint32_t *dst, uint32_t value
 hipError_t launch_fill_u32(const LaunchCtx &lc, uint32_t *dst, uint32_t value, uint64_t n) {
   if (!n) return hipSuccess;
   uint64_t blocks = (n + 255) / 256, cap = (uint64_t)lc.n_cus * 8;
-  fill_kernel<<<(unsigned)(blocks < cap ? blocks : cap), 256, 0, lc.stream>>>(dst, value, n);
+  CG_LAUNCH(lc, (fill_kernel), (unsigned)(blocks < cap ? blocks : cap), 256, dst, value, n);
   return hipGetLastError();
 }
 

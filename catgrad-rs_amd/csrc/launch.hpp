@@ -2,6 +2,7 @@
 // Every launcher enqueues on lc.stream and returns the launch status; nothing synchronises.
 #pragma once
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 #include <stdint.h>
 #include "program.hpp"
 
@@ -14,7 +15,15 @@ struct LaunchCtx {
   hipStream_t stream;
   int n_cus;
   uint32_t *err_flag;  // device word
+  // when tracing: events that receive the kernel's own begin / end timestamps
+  hipEvent_t ev_start, ev_stop;
 };
+
+// Every kernel is launched through this: with null events it is an ordinary launch; with events
+// the runtime stamps them at the kernel's start and end (what a profiler reports as duration).
+#define CG_LAUNCH(lc, kernel, grid, block, ...)                                            \
+  hipExtLaunchKernelGGL(kernel, dim3(grid), dim3(block), 0, (lc).stream, (lc).ev_start, \
+                        (lc).ev_stop, 0, __VA_ARGS__)
 
 // ---- k_ew.hip
 hipError_t launch_ew(const LaunchCtx &lc, const Program &p, const OutDesc &o, uint64_t n_elems,
@@ -99,8 +108,29 @@ struct GemmDesc {
   uint32_t nb0, nb1;         // batch = nb0 * nb1 (row-major)
   int64_t sa_b0, sa_b1, sb_b0, sb_b1;  // batch strides (0 = broadcast)
   int32_t bf16_math;         // 1: operands rounded to bf16, bf16 MFMA; 0: f32 MFMA
+  // split-K (bf16 fast path only): partial products go to workspace[split][batch][M][N]
+  float *workspace;
+  uint32_t splits, k_per_split;
 };
+// split factor launch_matmul should be given for this problem (1 = none)
+uint32_t gemm_split_k(const LaunchCtx &lc, const GemmDesc &g);
 hipError_t launch_matmul(const LaunchCtx &lc, const GemmDesc &g, const char **kernel_name);
+// contiguous f32 -> bf16 (RNE); n % 8 == 0, 16-byte aligned
+hipError_t launch_cast_bf16(const LaunchCtx &lc, const float *in, void *out, uint64_t n);
+// Several GEMVs y_p = x . B_p^T that share x (M == 1, B_p k-contiguous, 16-byte aligned rows):
+// one launch, problem p on grid.y
+struct GemvMultiDesc {
+  const float *x;
+  uint32_t K;
+  int32_t n_prob, b_stype;
+  struct {
+    const void *b;
+    float *c;
+    int64_t sbn;
+    uint32_t N;
+  } p[4];
+};
+hipError_t launch_gemv_multi(const LaunchCtx &lc, const GemvMultiDesc &g);
 // wrapping u32 matmul (ndarray's generic dot); all operands contiguous
 hipError_t launch_matmul_u32(const LaunchCtx &lc, const uint32_t *a, const uint32_t *b, uint32_t *c,
                              uint32_t batch, uint32_t M, uint32_t N, uint32_t K);

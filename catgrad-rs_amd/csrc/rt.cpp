@@ -95,6 +95,7 @@ void backend_release(cg_backend *be);
 
 void storage_release(Storage *s) {
   if (!s || s->rc.fetch_sub(1) != 1) return;
+  storage_release(s->shadow);
   cg_backend *be = s->be;
   // Safe to recycle at once: every consumer was enqueued on the backend's only stream.
   be->pool[s->bytes].push_back(s->ptr);
@@ -129,6 +130,17 @@ cg_tensor *new_node(cg_backend *be, cg_dtype dt, int rank, const int64_t *shape)
   return t;
 }
 
+void forget_gemv_candidate(cg_tensor *n) {
+  auto &v = n->be->gemv_candidates;
+  for (size_t i = 0; i < v.size(); ++i)
+    if (v[i] == n) {
+      v[i] = v.back();
+      v.pop_back();
+      break;
+    }
+  n->gemv_candidate = false;
+}
+
 void node_release(cg_tensor *t) {
   if (!t) return;
   std::vector<cg_tensor *> stack{t};
@@ -136,6 +148,7 @@ void node_release(cg_tensor *t) {
     cg_tensor *n = stack.back();
     stack.pop_back();
     if (n->rc.fetch_sub(1) != 1) continue;
+    if (n->gemv_candidate) forget_gemv_candidate(n);
     if (n->in[0]) stack.push_back(n->in[0]);
     if (n->in[1]) stack.push_back(n->in[1]);
     storage_release(n->st);
@@ -210,6 +223,8 @@ bool try_reshape_view(int ornk, const int64_t *oshape, const int64_t *ostr, int 
 }
 
 // ---- tracing -------------------------------------------------------------------------------
+// Accounts one kernel launch.  When tracing, the launch (issued through CG_LAUNCH with the
+// backend's current events) gets its own begin/end timestamps from the runtime.
 struct KernelScope {
   cg_backend *be;
   PendingEvent pe;
@@ -222,14 +237,15 @@ struct KernelScope {
     pe.flops = flops;
     (void)hipEventCreate(&pe.start);
     (void)hipEventCreate(&pe.stop);
-    (void)hipEventRecord(pe.start, be->stream);
+    be->cur_start = pe.start;
+    be->cur_stop = pe.stop;
   }
   void rename(const char *name) {
     if (on && name) pe.name = name;
   }
   ~KernelScope() {
     if (!on) return;
-    (void)hipEventRecord(pe.stop, be->stream);
+    be->cur_start = be->cur_stop = nullptr;
     be->trace_pending.push_back(pe);
   }
 };
@@ -239,12 +255,15 @@ void trace_collect(cg_backend *be) {
   (void)hipStreamSynchronize(be->stream);
   for (auto &pe : be->trace_pending) {
     float ms = 0.f;
-    (void)hipEventElapsedTime(&ms, pe.start, pe.stop);
-    TraceRec &r = be->trace_recs[pe.name];
-    r.launches++;
-    r.ms += ms;
-    r.bytes += pe.bytes;
-    r.flops += pe.flops;
+    if (hipEventElapsedTime(&ms, pe.start, pe.stop) == hipSuccess) {  // fails if nothing was launched
+      TraceRec &r = be->trace_recs[pe.name];
+      r.launches++;
+      r.ms += ms;
+      r.bytes += pe.bytes;
+      r.flops += pe.flops;
+    } else {
+      (void)hipGetLastError();
+    }
     (void)hipEventDestroy(pe.start);
     (void)hipEventDestroy(pe.stop);
   }
@@ -1350,6 +1369,23 @@ bool matrix_ok(const MatOperand &o) {
   return o.strides[r - 1] == 1 || o.shape[r - 1] == 1 || o.strides[r - 2] == 1 || o.shape[r - 2] == 1;
 }
 
+// bf16 twin of an f32 storage (whole buffer, so any view of it maps onto the twin unchanged)
+int bf16_shadow(cg_backend *be, Storage *st, Storage **out) {
+  if (!st->shadow) {
+    Storage *sh = nullptr;
+    TRY(dev_alloc(be, st->bytes / 2, &sh));
+    KernelScope ks(be, "cast_bf16", (double)st->bytes * 1.5, 0);
+    hipError_t e = launch_cast_bf16(be->lc(), (const float *)st->ptr, sh->ptr, st->bytes / 4);
+    if (e != hipSuccess) {
+      storage_release(sh);
+      return fail(be, CG_ERR_DEVICE, hipGetErrorString(e));
+    }
+    st->shadow = sh;
+  }
+  *out = st->shadow;
+  return CG_OK;
+}
+
 int realize_matmul(cg_backend *be, cg_tensor *n) {
   MatOperand A, B;
   bool pa = false, pb = false;
@@ -1422,6 +1458,21 @@ int realize_matmul(cg_backend *be, cg_tensor *n) {
     g.c = (float *)n->st->ptr;
     g.a_stype = A.t->stype;
     g.b_stype = B.t->stype;
+    // MFMA path in bf16 mode: f32 operands with a unit k stride are read from the bf16 twin of
+    // their storage (narrowed once, shared by every GEMM on the same activations)
+    if ((be->flags & CG_FLAG_BF16) && M >= 32 && K % 8 == 0) {
+      auto twin = [&](MatOperand &o, bool unit_k, const void **ptr, int32_t *stype) -> int {
+        Storage *st = o.t->st;
+        if (o.t->stype != ST_F32 || !unit_k || st->grow_dim >= 0 || st->bytes % 32) return CG_OK;
+        Storage *sh = nullptr;
+        TRY(bf16_shadow(be, st, &sh));
+        *ptr = (const char *)sh->ptr + o.t->offset * 2;
+        *stype = ST_BF16;
+        return CG_OK;
+      };
+      TRY(twin(A, A.strides[ra - 1] == 1, &g.a, &g.a_stype));
+      TRY(twin(B, B.strides[ra - 2] == 1 || B.strides[ra - 1] == 1, &g.b, &g.b_stype));
+    }
     g.M = M;
     g.N = N;
     g.K = K;
@@ -1449,13 +1500,84 @@ int realize_matmul(cg_backend *be, cg_tensor *n) {
       if (sb[1]) e *= nbo[1];
       return e * esize(o.t->stype);
     };
+    // q/k/v and gate/up: other deferred one-row matmuls on the same left operand go out in the
+    // same launch (weights are read once either way; the launch ramp is paid once)
+    if (M == 1 && batch == 1 && n->gemv_candidate && g.a_stype == ST_F32 && g.sak == 1 && g.sbk == 1 &&
+        K % 8 == 0 && K >= 512 && (uintptr_t)g.a % 16 == 0) {
+      auto weight_ok = [&](const void *ptr, int stype, int64_t sbn) {
+        return (uintptr_t)ptr % 16 == 0 && sbn % (16 / esize(stype)) == 0;
+      };
+      GemvMultiDesc md;
+      std::memset(&md, 0, sizeof(md));
+      std::vector<cg_tensor *> members;
+      if (weight_ok(g.b, g.b_stype, g.sbn)) {
+        for (cg_tensor *c : std::vector<cg_tensor *>(be->gemv_candidates)) {
+          if (c == n || members.size() >= 3 || c->op != N_MATMUL || c->in[0] != n->in[0]) continue;
+          cg_tensor *w = c->in[1];
+          if (w->op != N_REAL || w->rank != n->rank || w->stype != g.b_stype) continue;
+          if (w->shape[w->rank - 2] != (int64_t)K || w->strides[w->rank - 2] != 1) continue;
+          bool one_batch = true;
+          for (int i = 0; i + 2 < w->rank; ++i) one_batch = one_batch && w->shape[i] == 1;
+          if (!one_batch || !weight_ok(data_ptr(w), w->stype, w->strides[w->rank - 1])) continue;
+          members.push_back(c);
+        }
+      }
+      if (!members.empty()) {
+        md.x = (const float *)g.a;
+        md.K = K;
+        md.b_stype = g.b_stype;
+        md.p[0].b = g.b;
+        md.p[0].c = g.c;
+        md.p[0].sbn = g.sbn;
+        md.p[0].N = N;
+        md.n_prob = 1;
+        double bytes = uniq(A, sao) + uniq(B, sbo) + (double)n->size() * 4, flops = 2.0 * N * K;
+        for (cg_tensor *c : members) {
+          cg_tensor *w = c->in[1];
+          TRY(alloc_result(be, c, ST_F32));
+          auto &pr = md.p[md.n_prob++];
+          pr.b = data_ptr(w);
+          pr.c = (float *)c->st->ptr;
+          pr.sbn = w->strides[w->rank - 1];
+          pr.N = (uint32_t)w->shape[w->rank - 1];
+          bytes += (double)pr.N * K * esize(w->stype) + (double)pr.N * 4;
+          flops += 2.0 * pr.N * K;
+        }
+        {
+          KernelScope ks(be, g.b_stype == ST_BF16 ? "gemv_rowdot_bf16" : "gemv_rowdot_f32", bytes, flops);
+          HIPCHK(be, launch_gemv_multi(be->lc(), md));
+        }
+        for (cg_tensor *c : members) {
+          forget_gemv_candidate(c);
+          c->op = N_REAL;
+          drop_inputs(c);
+        }
+        forget_gemv_candidate(n);
+        n->op = N_REAL;
+        drop_inputs(n);
+        return CG_OK;
+      }
+    }
+    Storage *ws = nullptr;
+    const uint32_t splits = gemm_split_k(be->lc(), g);
+    if (splits > 1) {
+      TRY(dev_alloc(be, (size_t)splits * n->size() * 4, &ws));
+      g.workspace = (float *)ws->ptr;
+      g.splits = splits;
+      g.k_per_split = ((K + splits - 1) / splits + 63) / 64 * 64;
+    }
     const char *kname = "gemm";
-    KernelScope ks(be, kname, uniq(A, sao) + uniq(B, sbo) + (double)n->size() * 4,
-                   2.0 * batch * M * N * K);
-    hipError_t e = launch_matmul(be->lc(), g, &kname);
-    ks.rename(kname);
+    hipError_t e;
+    {
+      KernelScope ks(be, kname, uniq(A, sao) + uniq(B, sbo) + (double)n->size() * 4,
+                     2.0 * batch * M * N * K);
+      e = launch_matmul(be->lc(), g, &kname);
+      ks.rename(kname);
+    }
+    storage_release(ws);
     HIPCHK(be, e);
   }
+  if (n->gemv_candidate) forget_gemv_candidate(n);
   n->op = N_REAL;
   drop_inputs(n);
   return CG_OK;
@@ -1477,6 +1599,8 @@ int realize_concat(cg_backend *be, cg_tensor *n) {
       xd + yd <= x->st->grow_cap && x->offset == 0 && x->stype == plain) {
     n->st = x->st;
     n->st->rc.fetch_add(1);
+    storage_release(n->st->shadow);  // contents change: any bf16 twin is stale
+    n->st->shadow = nullptr;
     n->stype = plain;
     n->offset = 0;
     std::memcpy(n->strides, x->strides, sizeof(n->strides));
@@ -1913,6 +2037,11 @@ int cg_matmul(cg_backend *be, cg_tensor *a, cg_tensor *b, cg_tensor **out) {
   n->op = N_MATMUL;
   n->in[0] = retain(a);
   n->in[1] = retain(b);
+  if (a->dtype == CG_F32 && shape[a->rank - 2] == 1 && !(be->flags & CG_FLAG_EAGER)) {
+    if (be->gemv_candidates.size() >= 4096) forget_gemv_candidate(be->gemv_candidates.front());
+    be->gemv_candidates.push_back(n);
+    n->gemv_candidate = true;
+  }
   return finish(be, n, out);
 }
 

@@ -28,6 +28,9 @@ struct Storage {
   // set by concat when the buffer was laid out with spare room along one axis (KV cache)
   int grow_dim = -1;
   int64_t grow_cap = 0;
+  // bf16 copy of this (f32) storage, element for element, made on demand for the MFMA GEMM and
+  // shared by every matmul that reads a view of it (q/k/v, gate/up read the same activations)
+  Storage *shadow = nullptr;
 };
 
 enum NodeOp : uint8_t {
@@ -76,6 +79,7 @@ struct cg_tensor {
   cg_tensor *in[2] = {nullptr, nullptr};
   int64_t p0 = 0, p1 = 0;
   uint32_t cbits = 0;
+  bool gemv_candidate = false;  // listed in cg_backend::gemv_candidates (a weak reference)
 
   int64_t size() const {
     int64_t n = 1;
@@ -101,5 +105,10 @@ struct cg_backend {
   std::map<std::string, cgrt::TraceRec> trace_recs;
   std::vector<cgrt::PendingEvent> trace_pending;
 
-  cgk::LaunchCtx lc() const { return cgk::LaunchCtx{stream, n_cus, d_words}; }
+  // deferred small-M matmuls, so that those sharing their left operand (q/k/v, gate/up) can be
+  // issued as one launch; weak references, removed when a node is realised or deleted
+  std::vector<cg_tensor *> gemv_candidates;
+  hipEvent_t cur_start = nullptr, cur_stop = nullptr;  // set while a traced launch is issued
+
+  cgk::LaunchCtx lc() const { return cgk::LaunchCtx{stream, n_cus, d_words, cur_start, cur_stop}; }
 };

@@ -63,10 +63,14 @@ class CachedRunner:
         self.decode_term = llama.LlamaDecode(cfg).term()
         self.kv = None
         self.pos = 0
+        self._prefill_terms = {}
 
     def prefill(self, ids):
         ids = np.asarray(ids, np.uint32).reshape(1, -1)
-        term = llama.LlamaPrefill(self.cfg, ids.shape[1]).term()
+        n = ids.shape[1]
+        if n not in self._prefill_terms:      # the term depends on the prompt length only
+            self._prefill_terms[n] = llama.LlamaPrefill(self.cfg, n).term()
+        term = self._prefill_terms[n]
         out = self.it.run(term, [self.be.tensor(ids), self.cos, self.sin])
         self.kv = out[2:]
         self.pos = ids.shape[1]

@@ -482,3 +482,26 @@ def test_repeat_kv_matmul(oracle, dev):
         assert np.allclose(ref[0], q @ kr.transpose(0, 1, 3, 2), rtol=1e-4, atol=1e-4)
         for r, d in zip(ref, got):
             assert np.allclose(d, r, rtol=1e-4, atol=1e-4)
+
+
+def test_one_row_matmuls_sharing_x_go_out_together(oracle, hip, hip_bf16):
+    """q/k/v- and gate/up-style linears on one activation row: one launch, same results."""
+    g = rng(82)
+    k = 1024
+    x = g.standard_normal((1, 1, k)).astype(np.float32)
+    ws = [(g.standard_normal((n, k)) * 0.05).astype(np.float32) for n in (96, 40, 1024)]
+
+    def f(be, x, *w):
+        x = be.reshape(x, (1, 1, k))      # uploaded as rank 1: an activation, kept f32 in bf16 mode
+        outs = [be.matmul(x, be.reshape(be.transpose(wi, 0, 1), (1, k, wi.shape[0]))) for wi in w]
+        return tuple(outs)
+    for dev, tol in ((hip, RTOL_F32), (hip_bf16, RTOL_BF16)):
+        dev.trace(True)
+        dev.trace_reset()
+        r, d = both(oracle, dev, f, x.reshape(k), *ws)
+        rep = dev.trace_report()
+        dev.trace(False)
+        name = "gemv_rowdot_f32" if dev is hip else "gemv_rowdot_bf16"
+        assert rep[name]["launches"] == 1, rep
+        for ref, got, w in zip(r, d, ws):
+            assert_close(ref, got, tol, scale=np.abs(x) @ np.abs(w.T) + 1e-6)
