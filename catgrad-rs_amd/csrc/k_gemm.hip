@@ -31,6 +31,19 @@ __device__ __forceinline__ uint32_t bf16_rne(float f) {
 __device__ __forceinline__ float widen(float v) { return v; }
 __device__ __forceinline__ float widen(uint16_t v) { return __uint_as_float((uint32_t)v << 16); }
 
+// element offset of batch (b0, b1)'s B matrix
+__device__ __forceinline__ int64_t b_batch_offset(const GemmDesc &g, uint32_t bz, uint32_t b0, uint32_t b1) {
+  if (g.b_index) {
+    uint32_t ix = g.b_index[(int64_t)bz * g.b_index_stride];
+    if (ix >= g.b_index_limit) {  // the reference's select() panics; flag it and stay in bounds
+      atomicOr(g.err, ERRF_INDEX_OOB);
+      ix = g.b_index_limit - 1;
+    }
+    return (int64_t)ix * g.sb_index;
+  }
+  return b0 * g.sb_b0 + b1 * g.sb_b1;
+}
+
 // ---- tile loading -------------------------------------------------------------------------
 // Eight consecutive elements of a [rows, K] operand tile, either along k (KC) or along the row
 // axis (!KC), zero-filled out of bounds, widened to f32.
@@ -435,7 +448,7 @@ __global__ void __launch_bounds__(256) gemv_rowdot_kernel(GemmDesc g, int b_vec,
   const int sub = lane % LPR, col_in_wave = lane / LPR;
   const uint32_t bz = blockIdx.y, b0 = bz / g.nb1, b1 = bz - b0 * g.nb1;
   const float *A = (const float *)g.a + b0 * g.sa_b0 + b1 * g.sa_b1;
-  const TB *B = (const TB *)g.b + b0 * g.sb_b0 + b1 * g.sb_b1;
+  const TB *B = (const TB *)g.b + b_batch_offset(g, bz, b0, b1);
   float *C = g.c + (uint64_t)bz * g.M * g.N;
   // a "slot" is one wave (KSPLIT == 1) or one workgroup (KSPLIT == 4)
   const uint32_t slot = KSPLIT == 1 ? blockIdx.x * 4 + wave : blockIdx.x;
@@ -625,7 +638,7 @@ __global__ void __launch_bounds__(16 * KS) gemv_col_kernel(GemmDesc g, int b_vec
   const int cg = threadIdx.x & 15, ks = threadIdx.x >> 4;
   const uint32_t bz = blockIdx.y, b0 = bz / g.nb1, b1 = bz - b0 * g.nb1;
   const float *A = (const float *)g.a + b0 * g.sa_b0 + b1 * g.sa_b1;
-  const TB *B = (const TB *)g.b + b0 * g.sb_b0 + b1 * g.sb_b1;
+  const TB *B = (const TB *)g.b + b_batch_offset(g, bz, b0, b1);
   float *C = g.c + (uint64_t)bz * g.M * g.N;
   const uint32_t n = blockIdx.x * 64 + cg * 4;
   float acc[MROWS][4];
@@ -771,7 +784,10 @@ hipError_t launch_matmul(const LaunchCtx &lc, const GemmDesc &g, const char **ke
   const bool a_unit_k = g.sak == 1 || g.K == 1, b_unit_k = g.sbk == 1 || g.K == 1;
   const bool b_unit_n = g.sbn == 1 || g.N == 1;
   const int av = vec_ok(g.a, asz, a_unit_k ? g.sam : g.sak, g.sa_b0, g.sa_b1);
-  const int bv = vec_ok(g.b, bsz, b_unit_k ? g.sbn : g.sbk, g.sb_b0, g.sb_b1);
+  const int bv = vec_ok(g.b, bsz, b_unit_k ? g.sbn : g.sbk, g.b_index ? g.sb_index : g.sb_b0, g.sb_b1);
+  // only the one-row kernels follow b_index
+  if (g.b_index && !(g.M <= 8 && g.a_stype == ST_F32 && g.K > 0 && (b_unit_k || b_unit_n)))
+    return hipErrorInvalidValue;
 
   if (g.M <= 8 && g.a_stype == ST_F32 && g.K > 0) {
     if (b_unit_k) {

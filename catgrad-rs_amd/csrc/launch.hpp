@@ -111,6 +111,13 @@ struct GemmDesc {
   // split-K (bf16 fast path only): partial products go to workspace[split][batch][M][N]
   float *workspace;
   uint32_t splits, k_per_split;
+  // expert-indirect batches (one-row kernels only): when b_index is set, batch z reads its B
+  // matrix at b + b_index[z * b_index_stride] * sb_index instead of the batch strides; an
+  // index >= b_index_limit raises ERRF_INDEX_OOB in *err and is clamped
+  const uint32_t *b_index;
+  int64_t b_index_stride, sb_index;
+  uint32_t b_index_limit;
+  uint32_t *err;
 };
 // split factor launch_matmul should be given for this problem (1 = none)
 uint32_t gemm_split_k(const LaunchCtx &lc, const GemmDesc &g);

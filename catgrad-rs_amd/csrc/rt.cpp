@@ -1386,10 +1386,61 @@ int bf16_shadow(cg_backend *be, Storage *st, Storage **out) {
   return CG_OK;
 }
 
+// Routed experts (catgrad-llm/src/models/qwen3.rs:104-123) multiply each token by the matrix of
+// its expert:  matmul(x[S, 1, K], transpose(1, 2, index(0, idx[S], W[E, N, K]))).  Gathering S
+// whole matrices first would move S*N*K elements twice; instead the one-row kernels are given
+// the index vector and read W[idx[s]] in place.
+struct ExpertPeel {
+  cg_tensor *w = nullptr, *idx = nullptr;  // retained, realised
+  ~ExpertPeel() {
+    node_release(w);
+    node_release(idx);
+  }
+};
+
+int peel_expert_index(cg_backend *be, cg_tensor *n, ExpertPeel *out) {
+  if (be->flags & CG_FLAG_NO_PATTERNS) return CG_OK;
+  cg_tensor *t = n->in[1];
+  if (n->rank != 3 || n->shape[1] > 8 || n->size() == 0) return CG_OK;
+  if (t->op != N_TRANSPOSE || refs(t) != 1 || !((t->p0 == 1 && t->p1 == 2) || (t->p0 == 2 && t->p1 == 1)))
+    return CG_OK;
+  cg_tensor *g = t->in[0];
+  if (g->op != N_INDEX || refs(g) != 1 || g->p0 != 0 || g->rank != 3) return CG_OK;
+  cg_tensor *w = g->in[0], *idx = g->in[1];
+  if (idx->size() != n->shape[0] || w->shape[0] == 0) return CG_OK;
+  TRY(realize(be, n->in[0]));
+  if (n->in[0]->stype != ST_F32) return CG_OK;  // the one-row kernels take f32 activations
+  TRY(realize(be, w));
+  if (w->strides[2] != 1 && w->strides[1] != 1) return CG_OK;
+  // indices of any rank are read flattened (ndarray.rs:373-381); a strided view needs one stride
+  TRY(realize(be, idx));
+  cg_tensor *flat = nullptr;
+  if (idx->rank == 1) {
+    flat = retain(idx);
+  } else {
+    TRY(contiguous(be, idx, &flat));
+  }
+  out->w = retain(w);
+  out->idx = flat;
+  return CG_OK;
+}
+
 int realize_matmul(cg_backend *be, cg_tensor *n) {
   MatOperand A, B;
   bool pa = false, pb = false;
-  if (n->dtype == CG_F32 && n->rank == 4) {
+  ExpertPeel ex;
+  if (n->dtype == CG_F32) TRY(peel_expert_index(be, n, &ex));
+  if (ex.w) {
+    // B as the kernels see it: [S, K, N] = W[.]^T with the expert axis resolved per batch
+    B.set(retain(ex.w));
+    B.shape[0] = n->shape[0];
+    B.strides[0] = 0;
+    B.shape[1] = ex.w->shape[2];
+    B.shape[2] = ex.w->shape[1];
+    B.strides[1] = ex.w->strides[2];
+    B.strides[2] = ex.w->strides[1];
+    pb = true;
+  } else if (n->dtype == CG_F32 && n->rank == 4) {
     TRY(peel_repeat_kv(be, n->in[1], &B, &pb));
     if (!pb) TRY(peel_repeat_kv(be, n->in[0], &A, &pa));
   }
@@ -1401,7 +1452,7 @@ int realize_matmul(cg_backend *be, cg_tensor *n) {
     TRY(realize(be, n->in[1]));
     B.set(retain(n->in[1]));
   }
-  if (pb) split_heads(&A, B.shape[2]);
+  if (pb && !ex.w) split_heads(&A, B.shape[2]);
   if (pa) split_heads(&B, A.shape[2]);
   const int r = n->rank;
   const uint32_t M = (uint32_t)n->shape[r - 2], N = (uint32_t)n->shape[r - 1],
@@ -1443,6 +1494,8 @@ int realize_matmul(cg_backend *be, cg_tensor *n) {
               collapse_batch(A.rank - 2, A.shape, A.strides, B.strides, nbo, sao, sbo);
     if (!ok) {
       // fall back to plain contiguous operands of the logical shapes
+      node_release(ex.w);
+      ex.w = nullptr;
       cg_tensor *c = nullptr;
       TRY(materialize(be, n->in[0], &c, true));
       A.set(c);
@@ -1491,6 +1544,13 @@ int realize_matmul(cg_backend *be, cg_tensor *n) {
     g.sb_b0 = sbo[0];
     g.sb_b1 = sbo[1];
     g.bf16_math = (be->flags & CG_FLAG_BF16) ? 1 : 0;
+    if (ex.w) {
+      g.b_index = (const uint32_t *)data_ptr(ex.idx);
+      g.b_index_stride = ex.idx->rank == 1 ? ex.idx->strides[0] : 1;
+      g.sb_index = ex.w->strides[0];
+      g.b_index_limit = (uint32_t)ex.w->shape[0];
+      g.err = be->d_words;
+    }
     if (!g.bf16_math && (g.a_stype == ST_BF16 || g.b_stype == ST_BF16))
       return fail(be, CG_ERR_INTERNAL, "matmul: bf16 storage without CG_FLAG_BF16");
     // bytes: each operand once (batch-broadcast operands once), output once
@@ -1502,7 +1562,7 @@ int realize_matmul(cg_backend *be, cg_tensor *n) {
     };
     // q/k/v and gate/up: other deferred one-row matmuls on the same left operand go out in the
     // same launch (weights are read once either way; the launch ramp is paid once)
-    if (M == 1 && batch == 1 && n->gemv_candidate && g.a_stype == ST_F32 && g.sak == 1 && g.sbk == 1 &&
+    if (M == 1 && batch == 1 && !g.b_index && n->gemv_candidate && g.a_stype == ST_F32 && g.sak == 1 && g.sbk == 1 &&
         K % 8 == 0 && K >= 512 && (uintptr_t)g.a % 16 == 0) {
       auto weight_ok = [&](const void *ptr, int stype, int64_t sbn) {
         return (uintptr_t)ptr % 16 == 0 && sbn % (16 / esize(stype)) == 0;
@@ -1569,7 +1629,7 @@ int realize_matmul(cg_backend *be, cg_tensor *n) {
     const char *kname = "gemm";
     hipError_t e;
     {
-      KernelScope ks(be, kname, uniq(A, sao) + uniq(B, sbo) + (double)n->size() * 4,
+      KernelScope ks(be, kname, uniq(A, sao) + uniq(B, sbo) * (ex.w ? (double)batch : 1.0) + (double)n->size() * 4,
                      2.0 * batch * M * N * K);
       e = launch_matmul(be->lc(), g, &kname);
       ks.rename(kname);

@@ -1,3 +1,3 @@
 """LLM building blocks and model definitions as catgrad `Module`s (mirror of catgrad-llm)."""
-from . import helpers, llama  # noqa: F401
+from . import helpers, llama, qwen_moe, gemma3  # noqa: F401
 from .helpers import Config  # noqa: F401

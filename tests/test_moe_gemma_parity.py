@@ -1,0 +1,178 @@
+"""Qwen-MoE-layout and Gemma-3 decoders at reduced shapes (BASELINE configs 4 and 5): the oracle
+against independent numpy statements of the two build-authored pieces (top-k routed experts with
+a gated shared expert; sliding-window mask), then HIP vs oracle."""
+import numpy as np
+import pytest
+
+import llama_util as U
+import model_util as MU
+
+cg, llm = U.cg, U.llm
+
+
+def run_model(be, module, arrays, ids):
+    it = U.interpreter(be, arrays)
+    tok, logits = it.run(module.term(), [be.tensor(np.asarray(ids, np.uint32))])
+    return be.numpy(tok), be.numpy(logits)
+
+
+def test_moe_block_matches_numpy(oracle):
+    """The routed + shared expert block against a direct numpy statement of the same maths."""
+    cfg = MU.qwen_moe_config(num_hidden_layers=1)
+    P = MU.qwen_moe_params(cfg, seed=3, std=0.3)
+    model = llm.qwen_moe.QwenMoeModel(cfg, 8)
+    g = np.random.default_rng(4)
+    x = g.standard_normal((1, 6, cfg.hidden_size)).astype(np.float32)
+    pre = "qwen_moe.model.layers.0.mlp."
+
+    import vectors
+    (y,) = vectors.run(oracle, lambda b, v: model.moe(b, vectors.lang.path(["qwen_moe", "model", "layers", 0, "mlp"]), v),
+                       1, x, params={k: v for k, v in P.items() if k.startswith(pre)})
+
+    def silu(a):
+        return a / (1 + np.exp(-a))
+    t = x[0].astype(np.float64)
+    logits = t @ P[pre + "gate.weight"].T.astype(np.float64)
+    pr = np.exp(logits - logits.max(-1, keepdims=True))
+    pr /= pr.sum(-1, keepdims=True)
+    ref = np.zeros_like(t)
+    for i in range(t.shape[0]):
+        order = sorted(range(cfg.num_experts), key=lambda e: (-pr[i, e], e))[:cfg.num_experts_per_tok]
+        for e in order:
+            gw = P[pre + "experts.gate_proj.weight"][e].astype(np.float64)
+            uw = P[pre + "experts.up_proj.weight"][e].astype(np.float64)
+            dw = P[pre + "experts.down_proj.weight"][e].astype(np.float64)
+            ref[i] += pr[i, e] * ((silu(t[i] @ gw.T) * (t[i] @ uw.T)) @ dw.T)
+    sg = P[pre + "shared_expert.gate_proj.weight"].astype(np.float64)
+    su = P[pre + "shared_expert.up_proj.weight"].astype(np.float64)
+    sd = P[pre + "shared_expert.down_proj.weight"].astype(np.float64)
+    shared = (silu(t @ sg.T) * (t @ su.T)) @ sd.T
+    gate = 1 / (1 + np.exp(-(t @ P[pre + "shared_expert_gate.weight"].T.astype(np.float64))))
+    ref += shared * gate
+    assert np.allclose(y[0], ref, rtol=1e-4, atol=1e-5)
+
+
+def test_window_mask_matches_numpy(oracle):
+    import vectors
+    lang = vectors.lang
+    cfg = MU.gemma_config()
+    model = llm.gemma3.Gemma3Model(cfg, 9)
+
+    def f(b, v):
+        (n,) = lang.unpack(b, 1, lang.shape(b, v))
+        return model.window_mask(b, n, 4)
+    (m,) = vectors.run(oracle, f, 1, np.zeros(9, np.float32))
+    i, j = np.meshgrid(np.arange(9), np.arange(9), indexing="ij")
+    masked = (j > i) | (i - j >= 4)
+    assert np.array_equal(m != 0, masked)
+    assert np.all(m[masked] <= np.finfo(np.float32).min)
+
+
+def test_batch_folding_equals_per_sequence(oracle):
+    """[B, S] ids give the same logits as running each sequence alone (batch-1, as the reference)."""
+    cfg = MU.gemma_config()
+    P = MU.gemma_params(cfg, seed=5, std=0.2)
+    ids = np.random.default_rng(6).integers(0, cfg.vocab_size, (3, 7))
+    model = llm.gemma3.Gemma3Model(cfg, 7)
+    _, both = run_model(oracle, model, P, ids)
+    for r in range(3):
+        _, one = run_model(oracle, model, P, ids[r:r + 1])
+        assert np.allclose(both[r], one[0], rtol=1e-5, atol=1e-6)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("mode", ["f32", "nopat", "bf16"])
+def test_qwen_moe_hip_vs_oracle(oracle, hip, hip_nopat, hip_bf16, mode):
+    cfg = MU.qwen_moe_config()
+    P = MU.qwen_moe_params(cfg, seed=7, std=0.15)
+    ids = np.random.default_rng(8).integers(0, cfg.vocab_size, (2, 9))
+    model = llm.qwen_moe.QwenMoeModel(cfg, 9)
+    dev = {"f32": hip, "nopat": hip_nopat, "bf16": hip_bf16}[mode]
+    if mode == "bf16":
+        P_ref = {k: (U_round(v) if v.ndim >= 2 else v) for k, v in P.items()}
+    else:
+        P_ref = P
+    rt, rl = run_model(oracle, model, P_ref, ids)
+    gt, gl = run_model(dev, model, P, ids)
+    tol = 4e-2 if mode == "bf16" else 2e-4
+    assert np.max(np.abs(rl - gl)) <= tol * np.abs(rl).max()
+    if mode != "bf16":
+        assert np.array_equal(rt, gt)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("mode", ["f32", "nopat", "bf16"])
+def test_gemma3_hip_vs_oracle(oracle, hip, hip_nopat, hip_bf16, mode):
+    cfg = MU.gemma_config()
+    P = MU.gemma_params(cfg, seed=9, std=0.2)
+    ids = np.random.default_rng(10).integers(0, cfg.vocab_size, (2, 11))
+    model = llm.gemma3.Gemma3Model(cfg, 11, last_position_only=True)
+    dev = {"f32": hip, "nopat": hip_nopat, "bf16": hip_bf16}[mode]
+    P_ref = {k: (U_round(v) if v.ndim >= 2 else v) for k, v in P.items()} if mode == "bf16" else P
+    rt, rl = run_model(oracle, model, P_ref, ids)
+    gt, gl = run_model(dev, model, P, ids)
+    assert rl.shape == (2, 1, cfg.vocab_size)
+    tol = 4e-2 if mode == "bf16" else 2e-4
+    assert np.max(np.abs(rl - gl)) <= tol * np.abs(rl).max()
+    if mode != "bf16":
+        assert np.array_equal(rt, gt)
+
+
+def U_round(a):
+    u = a.view(np.uint32).astype(np.uint64)
+    return (((u + 0x7FFF + ((u >> 16) & 1)) >> 16) << 16).astype(np.uint32).view(np.float32)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dev_name", ["hip", "hip_bf16"])
+@pytest.mark.parametrize("shape", [(5, 8, 24, 64), (1, 4, 96, 1024), (33, 6, 40, 72)])  # S, E, N, K
+def test_expert_indirect_matmul(request, oracle, hip_nopat, dev_name, shape):
+    """matmul(x[S,1,K], transpose(1,2, index(0, idx, W[E,N,K]))) reads the expert matrices in place
+    (no gather launch), with the same result as the oracle and as the gathering path."""
+    import vectors
+    lang = vectors.lang
+    dev = request.getfixturevalue(dev_name)
+    S, E, N, K = shape
+    g = np.random.default_rng(S * 7 + E)
+    x = g.standard_normal((S, 1, K)).astype(np.float32)
+    w = g.standard_normal((E, N, K)).astype(np.float32)
+    idx2 = g.integers(0, E, (S, 3)).astype(np.uint32)     # the model slices one slot of [S, k]
+    if dev_name == "hip_bf16":
+        w = U_round(w)
+
+    def f(b, xv, iv, wv):
+        xv = xv + xv - xv          # activations are computed values (f32), never bf16 uploads
+        slot = lang.get(b, 1, 1, iv)
+        sel = lang.transpose(b, 1, 2, lang.index(b, 0, slot, wv))
+        return lang.matmul(b, xv, sel)
+    (ref,) = vectors.run(oracle, f, 1, x, idx2, w)
+    dev.trace(True)
+    dev.trace_reset()
+    (got,) = vectors.run(dev, f, 1, x, idx2, w)
+    names = set(dev.trace_report())
+    dev.trace(False)
+    (gen,) = vectors.run(hip_nopat, f, 1, x, idx2, w)
+    assert "gather" not in names, sorted(names)
+    expect = np.einsum("sk,snk->sn", x[:, 0].astype(np.float64), w[idx2[:, 1]].astype(np.float64))
+    assert np.allclose(ref[:, 0], expect, rtol=1e-4, atol=1e-3)
+    tol = 2e-2 if dev_name == "hip_bf16" else 1e-4
+    assert np.max(np.abs(got - ref)) <= tol * np.abs(ref).max()
+    assert np.max(np.abs(gen - ref)) <= 1e-4 * np.abs(ref).max()
+
+
+@pytest.mark.gpu
+def test_expert_index_out_of_bounds_is_reported(hip):
+    """ndarray's select panics on an index past the axis; the in-place expert read reports it."""
+    import vectors
+    lang = vectors.lang
+    x = np.ones((2, 1, 16), np.float32)
+    w = np.ones((3, 8, 16), np.float32)
+    idx = np.array([1, 3], np.uint32)
+
+    def f(b, xv, iv, wv):
+        return lang.matmul(b, xv, lang.transpose(b, 1, 2, lang.index(b, 0, iv, wv)))
+    with pytest.raises(cg.abi.BackendPanic, match="index out of bounds"):
+        vectors.run(hip, f, 1, x, idx, w)
+    # the flag is cleared: the next evaluation is clean
+    (ok,) = vectors.run(hip, f, 1, x, np.array([1, 2], np.uint32), w)
+    assert np.array_equal(ok, np.full((2, 1, 8), 16.0, np.float32))
