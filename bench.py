@@ -47,6 +47,9 @@ def main():
     ap.add_argument("--layers", type=int, default=16)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-steps", type=int, default=3)
+    ap.add_argument("--workload", choices=["llama", "ops"], default="llama",
+                    help="ops: the single-op microbenchmarks (one JSON line with a table) instead of "
+                         "the decoder")
     ap.add_argument("--profile-only", action="store_true",
                     help="skip the CPU baseline and the traced pass (for rocprofv3 runs)")
     args = ap.parse_args()
@@ -61,6 +64,13 @@ def main():
 
     cfg = llama_1b_config(llm, args.layers)
     lib = cg.load_library()
+    if args.workload == "ops":
+        opbench = importlib.import_module("catgrad-rs_amd.opbench")
+        recs = opbench.run_all(lib, iters=max(args.steps, 10))
+        print(json.dumps({"metric": "single-op microbenchmarks through the evaluator (BASELINE configs[0], [1])",
+                          "n_gpus": 1, "data": "synthetic", "hbm_peak_gbs": HBM_PEAK_GBS,
+                          "mfma_peak_tflops": MFMA_PEAK_TFLOPS, "ops": recs}))
+        return
     be = cg.Backend(lib, flags=cg.FLAG_BF16 if args.dtype == "bf16" else 0)
     t0 = time.time()
     arrays = U.param_arrays(cfg, seed=0, std=0.02)

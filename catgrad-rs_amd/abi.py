@@ -62,6 +62,7 @@ _SIGNATURES = {
     "cg_backend_destroy": (None, [_P]),
     "cg_last_error": (C.c_char_p, [_P]),
     "cg_sync": (C.c_int, [_P]),
+    "cg_tensor_realize": (C.c_int, [_P, _P]),
     "cg_backend_name": (C.c_char_p, [_P]),
     "cg_tensor_retain": (_P, [_P]),
     "cg_tensor_release": (None, [_P]),
@@ -203,6 +204,11 @@ class Backend:
 
     def sync(self):
         self._check(self.lib.cg_sync(self.ptr))
+
+    def realize(self, x):
+        """Issue the kernels a deferred tensor still needs (no wait)."""
+        self._check(self.lib.cg_tensor_realize(self.ptr, x.ptr))
+        return x
 
     # -- trait methods -----------------------------------------------------------------
     def zeros(self, shape, target_dtype):

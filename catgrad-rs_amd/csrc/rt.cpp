@@ -2013,6 +2013,12 @@ int cg_sync(cg_backend *be) {
   return sync_and_check(be);
 }
 
+int cg_tensor_realize(cg_backend *be, cg_tensor *t) {
+  if (!be || !t || t->be != be) return CG_ERR_ARG;
+  HIPCHK(be, hipSetDevice(be->device));
+  return realize(be, t);
+}
+
 cg_tensor *cg_tensor_retain(cg_tensor *t) { return t ? retain(t) : t; }
 void cg_tensor_release(cg_tensor *t) { node_release(t); }
 int cg_tensor_rank(const cg_tensor *t) { return t->rank; }

@@ -1,0 +1,144 @@
+"""Single-op microbenchmarks through the native evaluator (BASELINE.json configs[0] and [1]).
+
+Every case builds a term holding one op (or one stdlib definition), keeps its inputs resident on
+the device, runs it `iters` times through `Interpreter.run`, and reports
+  * wall time per run between two stream waits (evaluator + launch + kernel, pipelined), and
+  * kernel time from the backend's own start/stop events per launch,
+next to the algorithmic bytes / flops of the op (inputs read once, output written once; a
+broadcast operand counts at its own size, not at the broadcast size).
+"""
+import time
+
+import numpy as np
+
+from . import abi, lang, nn
+from .interpreter import Interpreter, Parameters, stdlib
+
+HBM_PEAK_GBS = 8000.0
+MFMA_PEAK_TFLOPS = {"bf16": 2500.0, "f32": 157.3}
+
+
+class _Fn(lang.Module):
+    def __init__(self, name, n_in, n_out, fn):
+        self.name, self.n_in, self.n_out, self.fn = name, n_in, n_out, fn
+
+    def path(self):
+        return lang.path(["opbench", self.name])
+
+    def sort(self):
+        return [lang.TENSOR] * self.n_in, [lang.TENSOR] * self.n_out
+
+    def def_(self, builder, args):
+        out = self.fn(builder, *args)
+        return list(out) if isinstance(out, (list, tuple)) else [out]
+
+
+def _softmax(b, x):
+    return nn.softmax(b, x)
+
+
+def _bcast_add(b, x, y):
+    return x + lang.broadcast(b, y, lang.shape(b, x))
+
+
+def _transpose_materialised(b, x):
+    # the reference's transpose is a lazy axis swap; the reshape forces the row-major result
+    d0, d1, d2 = lang.unpack(b, 3, lang.shape(b, x))
+    return lang.reshape(b, lang.make_shape(b, d0, d2 * d1), lang.transpose(b, 1, 2, x))
+
+
+def _mlp(b, x, w1, w2):
+    h = nn.sigmoid(b, lang.matmul(b, x, w1))
+    return lang.matmul(b, h, w2)
+
+
+def cases(dtype, scale=1):
+    """(name, fn, inputs, algorithmic bytes, flops).  `scale` divides the big extents (tests)."""
+    g = np.random.default_rng(2)
+    es = 2 if dtype == "bf16" else 4     # storage bytes of an uploaded rank>=2 f32 tensor
+    n = 4096 // scale
+    nb, nm = 8, 1024 // scale
+    rows, tab, width = 4096 // scale, 32000 // scale, 2048 // scale
+
+    def rnd(*shape):
+        return g.standard_normal(shape, dtype=np.float32)
+    out = []
+    a, bm = rnd(nb, nm, nm), rnd(nb, nm, nm)
+    out.append(("bmm", lang.matmul, [a, bm], 2 * a.size * es + a.size * 4, 2.0 * nb * nm ** 3))
+    x, y = rnd(n, n), rnd(n)
+    out.append(("broadcast_add", _bcast_add, [x, y], x.size * es + y.size * 4 + x.size * 4, 0))
+    out.append(("softmax", _softmax, [x], x.size * es + x.size * 4, 0))
+    out.append(("sum", lang.sum, [x], x.size * es + n * 4, 0))
+    out.append(("max", lang.max, [x], x.size * es + n * 4, 0))
+    out.append(("argmax", lang.argmax, [x], x.size * es + n * 4, 0))
+    t = rnd(64, 512 // scale, 512 // scale)
+    out.append(("transpose", _transpose_materialised, [t], t.size * es + t.size * 4, 0))
+    table = rnd(tab, width)
+    ids = g.integers(0, tab, rows).astype(np.uint32)
+    out.append(("gather", lambda b, tb, iv: lang.index(b, 0, iv, tb), [table, ids],
+                rows * width * (es + 4) + rows * 4, 0))
+    return out
+
+
+def mlp_case():
+    """hidden.rs-shaped MLP: x [64,128] U[-1,1]; W1 [128,256], W2 [256,10] ~ N(0, 0.05); seed 0."""
+    g = np.random.default_rng(0)
+    x = g.uniform(-1, 1, (64, 128)).astype(np.float32)
+    w1 = (g.standard_normal((128, 256)) * 0.05).astype(np.float32)
+    w2 = (g.standard_normal((256, 10)) * 0.05).astype(np.float32)
+    return ("mlp_64x128x256x10", _mlp, [x, w1, w2], 0, 2.0 * 64 * 128 * 256 + 2.0 * 64 * 256 * 10)
+
+
+def run_case(be, case, iters=50, warmup=5):
+    name, fn, arrays, nbytes, flops = case
+    it = Interpreter(be, stdlib(), Parameters())
+    term = _Fn(name, len(arrays), 1, fn).term()
+    args = [be.tensor(a) for a in arrays]
+    for a in args:
+        be.realize(a)
+    for _ in range(warmup):
+        be.realize(it.run(term, args)[0])
+    be.sync()
+    t = time.perf_counter()
+    for _ in range(iters):
+        be.realize(it.run(term, args)[0])
+    be.sync()
+    wall_us = (time.perf_counter() - t) / iters * 1e6
+    be.trace(True)
+    be.trace_reset()
+    n_tr = min(iters, 20)
+    for _ in range(n_tr):
+        be.realize(it.run(term, args)[0])
+    be.sync()
+    rep = be.trace_report()
+    be.trace(False)
+    kern_us = sum(v["ms"] for v in rep.values()) * 1e3 / n_tr
+    rec = {"op": name, "wall_us": wall_us, "kernel_us": kern_us,
+           "kernels": {k: v["launches"] // n_tr for k, v in rep.items()}}
+    if flops and nbytes:
+        rec.update(bound="mfma", algorithmic_flops=flops, tflops=flops / (kern_us * 1e-6) / 1e12)
+    elif nbytes:
+        rec.update(bound="hbm", algorithmic_bytes=nbytes, gbs=nbytes / (kern_us * 1e-6) / 1e9)
+    else:
+        rec.update(bound="latency", algorithmic_flops=flops)
+    return rec
+
+
+def run_all(lib, dtypes=("f32", "bf16"), iters=50):
+    out = []
+    for dtype in dtypes:
+        be = abi.Backend(lib, flags=abi.FLAG_BF16 if dtype == "bf16" else 0)
+        for case in cases(dtype):
+            rec = run_case(be, case, iters)
+            rec["dtype"] = dtype
+            if rec["bound"] == "hbm":
+                rec["frac"] = rec["gbs"] / HBM_PEAK_GBS
+            elif rec["bound"] == "mfma":
+                rec["frac"] = rec["tflops"] / MFMA_PEAK_TFLOPS[dtype]
+            out.append(rec)
+        if dtype == "f32":
+            rec = run_case(be, mlp_case(), iters=200, warmup=20)
+            rec["dtype"] = dtype
+            out.append(rec)
+        del be
+    return out

@@ -75,8 +75,13 @@ int cg_backend_create(int device, uint32_t flags, cg_backend **out);
 void cg_backend_destroy(cg_backend *be);
 /* message of the last failed call on this backend (never NULL) */
 const char *cg_last_error(const cg_backend *be);
-/* run everything deferred and wait for the stream */
+/* wait for the stream; reports errors only the data can reveal (u32 division by zero, gather index
+ * out of bounds) raised by kernels since the last wait */
 int cg_sync(cg_backend *be);
+/* issue the kernels a deferred tensor still needs, without waiting.  No counterpart in the reference,
+ * whose backends compute inside every call: the HIP backend records calls and computes when a value
+ * is read (cg_to_f32 / cg_to_u32 / cg_compare) or here; a no-op for the oracle */
+int cg_tensor_realize(cg_backend *be, cg_tensor *t);
 /* "hip-gfx950" or "ndarray-oracle" */
 const char *cg_backend_name(const cg_backend *be);
 
