@@ -365,6 +365,144 @@ __global__ void __launch_bounds__(256) gemm_bf16_nt_kernel(GemmDesc g) {
     }
 }
 
+// ---- bf16 NT GEMM with direct-to-LDS loads: the large-problem path --------------------------------
+// Same operands as above with K a multiple of 64 (per split).  Tiles travel HBM/L2 -> LDS with
+// global_load_lds_dwordx4 (16 bytes per lane, no VGPR staging, no ds_write): a wave's load lands
+// as 1 KB contiguous in LDS, so a tile row is 128 bytes unpadded and bank conflicts are avoided
+// by an XOR swizzle applied on the global side (the lane that fills physical 16-byte slot p of
+// row r fetches logical chunk p ^ ((r >> 1) & 7), which spreads any 16 consecutive rows over
+// all 64 banks).  Two stages: the loads of step s+1 are issued right after the barrier of step
+// s and complete under its MFMAs; the compiler does not know the asm writes LDS, so the waits
+// are explicit (s_waitcnt vmcnt + barrier before the stage is read).  Rows past M / N are
+// clamped on the load side and masked at the store.  Fragment reads of k-slice ks+1 are issued
+// before the MFMAs of slice ks (sched_barrier keeps the order).
+__device__ __forceinline__ void lds_dma16(const void *gptr, uint32_t lds_byte_off) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_byte_off), "v"(gptr)
+               : "memory", "m0");
+}
+template <int N> __device__ __forceinline__ void wait_vmcnt() {
+  __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
+}
+
+template <int BM_, int BN_, int WR, int WC>
+__global__ void __launch_bounds__(WR *WC * 64) gemm_bf16_dma_kernel(GemmDesc g) {
+  constexpr int NW = WR * WC, BK = 64, S = 2;
+  constexpr int WM = BM_ / WR, WN = BN_ / WC, TM = WM / 32, TN = WN / 32;
+  constexpr int LPW = (BM_ + BN_) / 8 / NW;   // 1 KB loads per wave per stage
+  constexpr int STAGE = (BM_ + BN_) * BK * 2;  // bytes
+  extern __shared__ __attribute__((aligned(16))) uint16_t dma_smem[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / WC, wn = wave % WC;
+  const uint32_t tiles_m = (g.M + BM_ - 1) / BM_, tiles_n = (g.N + BN_ - 1) / BN_;
+  const uint32_t per_batch = tiles_m * tiles_n, batch = g.nb0 * g.nb1;
+  // Workgroups are dealt round-robin to the 8 XCDs (one L2 each): give every XCD a contiguous
+  // range of logical tiles, and walk tiles in groups of 4 tile rows so that the ~32 tiles an
+  // XCD works on at once share their A and B panels in that L2.
+  uint32_t id = blockIdx.x;
+  if (gridDim.x % 8 == 0) id = (id % 8) * (gridDim.x / 8) + id / 8;
+  const uint32_t zz = id / per_batch;  // split * batch + batch index
+  const uint32_t t = id - zz * per_batch;
+  const uint32_t split = zz / batch, bz = zz - split * batch;
+  const uint32_t b0 = bz / g.nb1, b1 = bz - b0 * g.nb1;
+  constexpr uint32_t GM = 4;
+  const uint32_t first_m = t / (GM * tiles_n) * GM, gsz = min(tiles_m - first_m, GM);
+  const uint32_t tg = t % (GM * tiles_n);
+  const uint32_t m0 = (first_m + tg % gsz) * BM_, n0 = tg / gsz * BN_;
+  const uint16_t *A = (const uint16_t *)g.a + b0 * g.sa_b0 + b1 * g.sa_b1;
+  const uint16_t *B = (const uint16_t *)g.b + b0 * g.sb_b0 + b1 * g.sb_b1;
+  float *C = (g.splits > 1 ? g.workspace + (uint64_t)split * batch * g.M * g.N : g.c) +
+             (uint64_t)bz * g.M * g.N;
+  const uint32_t k_begin = split * g.k_per_split;
+  const uint32_t k_end = min(g.K, k_begin + g.k_per_split);
+
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint16_t *)dma_smem;
+  const uint16_t *gp[LPW];  // per-lane source of each of this wave's loads; advances by BK per stage
+#pragma unroll
+  for (int i = 0; i < LPW; ++i) {
+    const int q = wave * LPW + i;  // 8-row block of the stacked [A; B] tile
+    const int R = q * 8 + (lane >> 3);
+    const int c = (lane & 7) ^ ((R >> 1) & 7);
+    if (q * 8 < BM_) gp[i] = A + (int64_t)min(m0 + R, g.M - 1) * g.sam + k_begin + c * 8;
+    else gp[i] = B + (int64_t)min(n0 + (R - BM_), g.N - 1) * g.sbn + k_begin + c * 8;
+  }
+  auto issue = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < LPW; ++i) {
+      lds_dma16(gp[i], lds0 + buf * STAGE + (wave * LPW + i) * 1024);
+      gp[i] += BK;
+    }
+  };
+  const int sw = (lane >> 1) & 7, half = lane >> 5;
+  auto compute = [&](int buf) {
+    const uint16_t *As = dma_smem + buf * (STAGE / 2), *Bs = As + BM_ * BK;
+    bf16x8 af[2][TM], bfr[2][TN];
+    auto frags = [&](int ks, int set) {
+      const int p = ((ks * 2 + half) ^ sw) * 8;
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+        af[set][i] = *(const bf16x8 *)(&As[(wm * WM + i * 32 + (lane & 31)) * BK + p]);
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        bfr[set][j] = *(const bf16x8 *)(&Bs[(wn * WN + j * 32 + (lane & 31)) * BK + p]);
+    };
+    frags(0, 0);
+#pragma unroll
+    for (int ks = 0; ks < BK / 16; ++ks) {
+      if (ks + 1 < BK / 16) frags(ks + 1, (ks + 1) & 1);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[ks & 1][i], bfr[ks & 1][j], acc[i][j], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  const int n_steps = k_end > k_begin ? (int)((k_end - k_begin) / BK) : 0;
+  if (n_steps > 0) issue(0);
+  for (int step = 0; step < n_steps; ++step) {
+    wait_vmcnt<0>();   // stage `step` has landed (this wave's part) ...
+    __syncthreads();   // ... and everyone's; all waves are done reading the other buffer
+    if (step + 1 < n_steps) issue((step + 1) & 1);
+    compute(step & 1);
+  }
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const uint32_t col = n0 + wn * WN + j * 32 + (lane & 31);
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const uint32_t row = m0 + wm * WM + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
+        if (row < g.M && col < g.N) C[(uint64_t)row * g.N + col] = acc[i][j][e];
+      }
+    }
+}
+
+template <int BM_, int BN_, int WR, int WC>
+static hipError_t launch_gemm_dma(const LaunchCtx &lc, const GemmDesc &g, uint32_t grid) {
+  constexpr int smem = 2 * (BM_ + BN_) * 64 * 2;
+  static bool configured = false;  // one attribute call per kernel and process
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute((const void *)gemm_bf16_dma_kernel<BM_, BN_, WR, WC>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    if (e != hipSuccess) return e;
+    configured = true;
+  }
+  hipExtLaunchKernelGGL((gemm_bf16_dma_kernel<BM_, BN_, WR, WC>), dim3(grid), dim3(WR * WC * 64), smem,
+                        lc.stream, lc.ev_start, lc.ev_stop, 0, g);
+  return hipGetLastError();
+}
+
 // C = sum over splits of workspace[split] (float4 per thread; sizes are multiples of 4 or the
 // tail is handled scalar)
 __global__ void __launch_bounds__(256) splitk_reduce_kernel(const float *ws, float *c, uint64_t n,
@@ -450,6 +588,7 @@ __global__ void __launch_bounds__(256) gemv_rowdot_kernel(GemmDesc g, int b_vec,
   const float *A = (const float *)g.a + b0 * g.sa_b0 + b1 * g.sa_b1;
   const TB *B = (const TB *)g.b + b_batch_offset(g, bz, b0, b1);
   float *C = g.c + (uint64_t)bz * g.M * g.N;
+  const float *Cadd = g.c_add ? g.c_add + (uint64_t)bz * g.M * g.N : nullptr;
   // a "slot" is one wave (KSPLIT == 1) or one workgroup (KSPLIT == 4)
   const uint32_t slot = KSPLIT == 1 ? blockIdx.x * 4 + wave : blockIdx.x;
   const uint32_t n_slots = KSPLIT == 1 ? gridDim.x * 4 : gridDim.x;
@@ -544,8 +683,9 @@ __global__ void __launch_bounds__(256) gemv_rowdot_kernel(GemmDesc g, int b_vec,
 #pragma unroll
           for (int m = 0; m < MROWS; ++m)
             if (n < g.N && (uint32_t)m < g.M)
-              C[(uint64_t)m * g.N + n] = (red[0][r][m][col_in_wave] + red[1][r][m][col_in_wave]) +
-                                         (red[2][r][m][col_in_wave] + red[3][r][m][col_in_wave]);
+              C[(uint64_t)m * g.N + n] = ((red[0][r][m][col_in_wave] + red[1][r][m][col_in_wave]) +
+                                          (red[2][r][m][col_in_wave] + red[3][r][m][col_in_wave])) +
+                                         (Cadd ? Cadd[(uint64_t)m * g.N + n] : 0.f);
         }
       }
     } else if (sub == 0) {
@@ -554,7 +694,8 @@ __global__ void __launch_bounds__(256) gemv_rowdot_kernel(GemmDesc g, int b_vec,
         const uint32_t n = nb + r * CPW + col_in_wave;
 #pragma unroll
         for (int m = 0; m < MROWS; ++m)
-          if (n < g.N && (uint32_t)m < g.M) C[(uint64_t)m * g.N + n] = acc[r][m];
+          if (n < g.N && (uint32_t)m < g.M)
+            C[(uint64_t)m * g.N + n] = acc[r][m] + (Cadd ? Cadd[(uint64_t)m * g.N + n] : 0.f);
       }
     }
   }
@@ -571,6 +712,7 @@ __global__ void __launch_bounds__(256) gemv_multi_kernel(GemvMultiDesc g) {
   const TB *B = (const TB *)g.p[blockIdx.y].b;
   const int64_t sbn = g.p[blockIdx.y].sbn;
   float *C = g.p[blockIdx.y].c;
+  const float *Cadd = g.p[blockIdx.y].c_add;
   const uint32_t n_waves = gridDim.x * 4;
   for (uint32_t nb = (blockIdx.x * 4 + wave) * R; nb < N; nb += n_waves * R) {
     float acc[R];
@@ -612,7 +754,7 @@ __global__ void __launch_bounds__(256) gemv_multi_kernel(GemvMultiDesc g) {
     for (int r = 0; r < R; ++r) {
 #pragma unroll
       for (int s = 32; s >= 1; s >>= 1) acc[r] += __shfl_xor(acc[r], s, 64);
-      if (lane == 0 && nb + r < N) C[nb + r] = acc[r];
+      if (lane == 0 && nb + r < N) C[nb + r] = acc[r] + (Cadd ? Cadd[nb + r] : 0.f);
     }
   }
 }
@@ -640,6 +782,7 @@ __global__ void __launch_bounds__(16 * KS) gemv_col_kernel(GemmDesc g, int b_vec
   const float *A = (const float *)g.a + b0 * g.sa_b0 + b1 * g.sa_b1;
   const TB *B = (const TB *)g.b + b_batch_offset(g, bz, b0, b1);
   float *C = g.c + (uint64_t)bz * g.M * g.N;
+  const float *Cadd = g.c_add ? g.c_add + (uint64_t)bz * g.M * g.N : nullptr;
   const uint32_t n = blockIdx.x * 64 + cg * 4;
   float acc[MROWS][4];
 #pragma unroll
@@ -682,7 +825,8 @@ __global__ void __launch_bounds__(16 * KS) gemv_col_kernel(GemmDesc g, int b_vec
 #pragma unroll
     for (int q = 0; q < KS; ++q) s += part[q][m][c];
     const uint32_t col = blockIdx.x * 64 + c;
-    if ((uint32_t)m < g.M && col < g.N) C[(uint64_t)m * g.N + col] = s;
+    if ((uint32_t)m < g.M && col < g.N)
+      C[(uint64_t)m * g.N + col] = s + (Cadd ? Cadd[(uint64_t)m * g.N + col] : 0.f);
   }
 }
 
@@ -758,6 +902,11 @@ static void launch_rowdot(const LaunchCtx &lc, const GemmDesc &g, int bv, int av
   }
 }
 
+// the direct-to-LDS kernel: both operands unit-stride along k, K (and each split) a multiple of 64
+static bool gemm_dma_ok(const GemmDesc &g) {
+  return g.sak == 1 && g.sbk == 1 && g.K % 64 == 0 && g.K >= 64 && g.M >= 64 && g.N >= 64;
+}
+
 static bool gemm_fast_path(const GemmDesc &g, int av, int bv) {
   return g.bf16_math && g.M > 8 && g.a_stype == ST_BF16 && g.b_stype == ST_BF16 && g.sak == 1 &&
          (g.sbk == 1 || g.sbn == 1) && g.K % 8 == 0 && (g.sbk == 1 || g.N % 8 == 0) && av && bv;
@@ -785,8 +934,8 @@ hipError_t launch_matmul(const LaunchCtx &lc, const GemmDesc &g, const char **ke
   const bool b_unit_n = g.sbn == 1 || g.N == 1;
   const int av = vec_ok(g.a, asz, a_unit_k ? g.sam : g.sak, g.sa_b0, g.sa_b1);
   const int bv = vec_ok(g.b, bsz, b_unit_k ? g.sbn : g.sbk, g.b_index ? g.sb_index : g.sb_b0, g.sb_b1);
-  // only the one-row kernels follow b_index
-  if (g.b_index && !(g.M <= 8 && g.a_stype == ST_F32 && g.K > 0 && (b_unit_k || b_unit_n)))
+  // only the one-row kernels follow b_index and c_add
+  if ((g.b_index || g.c_add) && !(g.M <= 8 && g.a_stype == ST_F32 && g.K > 0 && (b_unit_k || b_unit_n)))
     return hipErrorInvalidValue;
 
   if (g.M <= 8 && g.a_stype == ST_F32 && g.K > 0) {
@@ -827,6 +976,17 @@ hipError_t launch_matmul(const LaunchCtx &lc, const GemmDesc &g, const char **ke
     GemmDesc gg = g;
     gg.splits = splits;
     if (splits == 1) gg.k_per_split = g.K;
+    if (gemm_dma_ok(g)) {
+      const uint64_t t256 = (uint64_t)((g.M + 255) / 256) * ((g.N + 255) / 256) * batch * splits;
+      hipError_t e;
+      if (t256 >= (uint64_t)lc.n_cus) {
+        e = launch_gemm_dma<256, 256, 2, 4>(lc, gg, (uint32_t)t256);
+      } else {
+        const uint64_t t128 = (uint64_t)((g.M + 127) / 128) * ((g.N + 127) / 128) * batch * splits;
+        e = launch_gemm_dma<128, 128, 2, 2>(lc, gg, (uint32_t)t128);
+      }
+      if (e != hipSuccess) return e;
+    } else {
     const uint64_t big_tiles = (uint64_t)((g.M + 127) / 128) * ((g.N + 127) / 128) * batch * splits;
     if (big_tiles * 2 >= (uint64_t)lc.n_cus && g.N > 64) {
       dim3 gr((g.N + 127) / 128, (g.M + 127) / 128, batch * splits);
@@ -836,6 +996,7 @@ hipError_t launch_matmul(const LaunchCtx &lc, const GemmDesc &g, const char **ke
       dim3 gr((g.N + 63) / 64, (g.M + 63) / 64, batch * splits);
       if (bkc) CG_LAUNCH(lc, (gemm_bf16_nt_kernel<64, 64, true>), gr, 256, gg);
       else CG_LAUNCH(lc, (gemm_bf16_nt_kernel<64, 64, false>), gr, 256, gg);
+    }
     }
     if (splits > 1) {
       LaunchCtx untimed = lc;

@@ -111,6 +111,8 @@ struct GemmDesc {
   // split-K (bf16 fast path only): partial products go to workspace[split][batch][M][N]
   float *workspace;
   uint32_t splits, k_per_split;
+  // optional epilogue of the one-row kernels: C = A . B + c_add (c_add laid out like C)
+  const float *c_add;
   // expert-indirect batches (one-row kernels only): when b_index is set, batch z reads its B
   // matrix at b + b_index[z * b_index_stride] * sb_index instead of the batch strides; an
   // index >= b_index_limit raises ERRF_INDEX_OOB in *err and is clamped
@@ -133,6 +135,7 @@ struct GemvMultiDesc {
   struct {
     const void *b;
     float *c;
+    const float *c_add;  // optional: c = x . b^T + c_add
     int64_t sbn;
     uint32_t N;
   } p[4];

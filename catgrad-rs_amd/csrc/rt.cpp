@@ -240,8 +240,8 @@ struct KernelScope {
     be->cur_start = pe.start;
     be->cur_stop = pe.stop;
   }
-  void rename(const char *name) {
-    if (on && name) pe.name = name;
+  void rename(const std::string &name) {
+    if (on && !name.empty()) pe.name = name;
   }
   ~KernelScope() {
     if (!on) return;
@@ -1097,6 +1097,34 @@ int try_glu(cg_backend *be, cg_tensor *root, bool *done) {
 }
 
 // a single f32 add/sub/mul/div of two tensors that are (or will be) in memory anyway
+int realize_matmul(cg_backend *be, cg_tensor *n, cg_tensor *addend, bool *added);
+
+// residual + linear(x) on a decode step (models/llama.rs:166-186: `res + attention`, `res + mlp`):
+// the add rides in the epilogue of the one-row matmul kernel instead of a launch of its own.
+int try_gemv_add(cg_backend *be, cg_tensor *root, bool *done) {
+  if (root->dtype != CG_F32 || !is_bin(root, E_ADD_F)) return CG_OK;
+  for (int side = 0; side < 2; ++side) {
+    cg_tensor *mm = root->in[side], *other = root->in[1 - side];
+    if (mm->op != N_MATMUL || refs(mm) != 1 || !mm->gemv_candidate || mm->dtype != CG_F32) continue;
+    if (other->op == N_CONST || ((other->op == N_BIN || other->op == N_UN) && refs(other) == 1)) continue;
+    TRY(realize(be, other));
+    if (other->stype != ST_F32 || !is_contiguous(other)) return CG_OK;
+    bool added = false;
+    TRY(realize_matmul(be, mm, other, &added));
+    if (!added) return CG_OK;  // the product is realised; the generic add takes it from here
+    // mm now holds the sum and nobody else can see it: root takes over its storage
+    root->st = mm->st;
+    root->st->rc.fetch_add(1);
+    root->stype = mm->stype;
+    root->offset = mm->offset;
+    std::copy(mm->strides, mm->strides + mm->rank, root->strides);
+    finish_fused(root);
+    *done = true;
+    return CG_OK;
+  }
+  return CG_OK;
+}
+
 int try_binary(cg_backend *be, cg_tensor *root, bool *done) {
   if (root->dtype != CG_F32 || root->op != N_BIN || root->size() % 4 || root->rank == 0) return CG_OK;
   int op;
@@ -1151,6 +1179,8 @@ int try_patterns(cg_backend *be, cg_tensor *root, bool *done) {
   TRY(try_rope(be, root, done));
   if (*done) return CG_OK;
   TRY(try_glu(be, root, done));
+  if (*done) return CG_OK;
+  TRY(try_gemv_add(be, root, done));
   if (*done) return CG_OK;
   return try_binary(be, root, done);
 }
@@ -1425,7 +1455,9 @@ int peel_expert_index(cg_backend *be, cg_tensor *n, ExpertPeel *out) {
   return CG_OK;
 }
 
-int realize_matmul(cg_backend *be, cg_tensor *n) {
+// `addend` (optional; realised, f32, contiguous, shaped like n) is added in the epilogue when a
+// one-row kernel runs the product; *added tells the caller whether that happened.
+int realize_matmul(cg_backend *be, cg_tensor *n, cg_tensor *addend = nullptr, bool *added = nullptr) {
   MatOperand A, B;
   bool pa = false, pb = false;
   ExpertPeel ex;
@@ -1544,6 +1576,10 @@ int realize_matmul(cg_backend *be, cg_tensor *n) {
     g.sb_b0 = sbo[0];
     g.sb_b1 = sbo[1];
     g.bf16_math = (be->flags & CG_FLAG_BF16) ? 1 : 0;
+    if (addend && M <= 8 && g.a_stype == ST_F32 && K > 0 && (g.sbk == 1 || g.sbn == 1 || K == 1 || N == 1)) {
+      g.c_add = (const float *)data_ptr(addend);
+      *added = true;
+    }
     if (ex.w) {
       g.b_index = (const uint32_t *)data_ptr(ex.idx);
       g.b_index_stride = ex.idx->rank == 1 ? ex.idx->strides[0] : 1;
@@ -1588,6 +1624,7 @@ int realize_matmul(cg_backend *be, cg_tensor *n) {
         md.b_stype = g.b_stype;
         md.p[0].b = g.b;
         md.p[0].c = g.c;
+        md.p[0].c_add = g.c_add;
         md.p[0].sbn = g.sbn;
         md.p[0].N = N;
         md.n_prob = 1;
@@ -1596,6 +1633,7 @@ int realize_matmul(cg_backend *be, cg_tensor *n) {
           cg_tensor *w = c->in[1];
           TRY(alloc_result(be, c, ST_F32));
           auto &pr = md.p[md.n_prob++];
+          pr.c_add = nullptr;
           pr.b = data_ptr(w);
           pr.c = (float *)c->st->ptr;
           pr.sbn = w->strides[w->rank - 1];
@@ -1633,6 +1671,11 @@ int realize_matmul(cg_backend *be, cg_tensor *n) {
                      2.0 * batch * M * N * K);
       e = launch_matmul(be->lc(), g, &kname);
       ks.rename(kname);
+      if (be->trace_shapes) {  // per-shape records: gemm_mfma_bf16[b32,512x512x64,s1]
+        char buf[96];
+        snprintf(buf, sizeof buf, "%s[b%lld,%ux%ux%u,s%u]", kname, (long long)batch, M, N, K, splits);
+        ks.rename(buf);
+      }
     }
     storage_release(ws);
     HIPCHK(be, e);
@@ -2350,6 +2393,7 @@ int cg_trace_enable(cg_backend *be, int on) {
   if (!be) return CG_ERR_ARG;
   trace_collect(be);
   be->trace = on != 0;
+  be->trace_shapes = on == 2;
   return CG_OK;
 }
 int cg_trace_reset(cg_backend *be) {

@@ -102,6 +102,7 @@ struct cg_backend {
   uint64_t pool_bytes = 0, device_bytes = 0, launches = 0;
   // tracing
   bool trace = false;
+  bool trace_shapes = false;  // cg_trace_enable(be, 2): matmul records carry their shape
   std::map<std::string, cgrt::TraceRec> trace_recs;
   std::vector<cgrt::PendingEvent> trace_pending;
 

@@ -143,6 +143,7 @@ int cg_to_u32(cg_backend *be, cg_tensor *x, uint32_t *dst, size_t n);
 /* ---- tracing (no counterpart in the reference) -------------------------------------
  * When enabled every kernel launch is bracketed by two events on the backend's stream.
  * cg_trace_report writes one line per kernel name: "name launches total_ms bytes flops".
+ * on = 2 additionally keys matmul records by problem shape ("gemm_mfma_bf16[b1,512x2048x2048,s4]").
  */
 int cg_trace_enable(cg_backend *be, int on);
 int cg_trace_reset(cg_backend *be);

@@ -140,3 +140,27 @@ def test_near_misses_take_the_generic_path(oracle, hip):
     assert "softmax_fused" not in names
     for r, d in zip(ref, got):
         assert np.allclose(d, r, rtol=1e-4, atol=1e-7)
+
+
+@pytest.mark.parametrize("shape", [(1, 2048, 2048), (1, 8192, 2048), (1, 72, 40), (3, 512, 64)])  # M, K, N
+@pytest.mark.parametrize("order", ["res_first", "mm_first"])
+def test_residual_add_in_gemv_epilogue(oracle, hip, hip_nopat, shape, order):
+    """res + linear(x) on one-row activations: no separate add launch, same values."""
+    M, K, N = shape
+    g = np.random.default_rng(K + N)
+    x = g.standard_normal((1, M, K)).astype(np.float32)
+    w = (g.standard_normal((N, K)) * 0.05).astype(np.float32)
+    res = g.standard_normal((1, M, N)).astype(np.float32)
+
+    def f(b, xv, rv):
+        xv = xv + xv - xv
+        y = nn.linear_no_bias(b, K, N, lang.path(["l"]), xv)
+        return rv + y if order == "res_first" else y + rv
+    p = {"l.weight": w}
+    (ref,) = vectors.run(oracle, f, 1, x, res, params=p)
+    got, names = run_traced(hip, f, 1, x, res, params=p)
+    (gen,) = vectors.run(hip_nopat, f, 1, x, res, params=p)
+    if M == 1:
+        assert "binary_f32" not in names, sorted(names)
+    assert np.allclose(got[0], ref, rtol=1e-4, atol=1e-5)
+    assert np.allclose(gen, ref, rtol=1e-4, atol=1e-5)
