@@ -50,6 +50,8 @@ def main():
     ap.add_argument("--workload", choices=["llama", "ops"], default="llama",
                     help="ops: the single-op microbenchmarks (one JSON line with a table) instead of "
                          "the decoder")
+    ap.add_argument("--sync-each-step", action="store_true",
+                    help="read every token on the host before starting the next step")
     ap.add_argument("--profile-only", action="store_true",
                     help="skip the CPU baseline and the traced pass (for rocprofv3 runs)")
     args = ap.parse_args()
@@ -90,19 +92,38 @@ def main():
     prefill_s = time.perf_counter() - t
 
     # ---- decode: W warm-up steps, then exactly K timed steps -------------------------------
-    token = first
-    for _ in range(args.warmup):
-        tok, _ = runner.step(token)
-        token = int(be.to_vec(tok)[0])
+    # Default loop: the sampled token stays on the device as the next step's input and the host
+    # reads it one step behind (cg_tensor_prefetch), so recording and issuing step t+1 overlap
+    # the device's work on step t.  --sync-each-step reads every token before the next step
+    # starts, like the reference's driver (catgrad-llm/examples/llama/main.rs:114-169).
+    def decode(n, tok_tensor):
+        toks = []
+        if args.sync_each_step:
+            token = int(be.to_vec(tok_tensor)[0])
+            for _ in range(n):
+                tok_tensor, _ = runner.step(token)
+                token = int(be.to_vec(tok_tensor)[0])
+                toks.append(token)
+            return toks, tok_tensor
+        prev = tok_tensor
+        for _ in range(n):
+            cur, _ = runner.step(prev)
+            be.prefetch(cur)
+            if prev is not tok_tensor:
+                toks.append(int(be.to_vec(prev)[0]))
+            prev = cur
+        toks.append(int(be.to_vec(prev)[0]))
+        return toks, prev
+
+    _, tok = decode(args.warmup, tok) if args.warmup else ([], tok)
     be.sync()
     runner.it.backend_calls()
     launches0 = be.stats()["launches"]
     t = time.perf_counter()
-    for _ in range(args.steps):
-        tok, _ = runner.step(token)
-        token = int(be.to_vec(tok)[0])
+    toks, tok = decode(args.steps, tok)
     be.sync()
     decode_s = time.perf_counter() - t
+    token = toks[-1]
     calls_per_step = runner.it.backend_calls() / max(args.steps, 1)
     launches_per_step = (be.stats()["launches"] - launches0) / max(args.steps, 1)
     ms_per_step = decode_s / args.steps * 1e3
@@ -121,7 +142,9 @@ def main():
         "dtype": args.dtype, "data": "synthetic",
         "config": {"workload": "BASELINE configs[2]: Llama-3.2-1B shape, random init N(0,0.02), "
                                f"{cfg.num_hidden_layers} layers, batch 1, {args.prompt}-token prompt, "
-                               "greedy decode with KV cache through the catgrad evaluator",
+                               "greedy decode with KV cache through the catgrad evaluator; "
+                               + ("token read back before every step" if args.sync_each_step else
+                                  "token fed back on the device, read by the host one step behind"),
                    "prompt_tokens": args.prompt, "layers": cfg.num_hidden_layers},
         "prefill_tokens_per_s": args.prompt / prefill_s,
         "prefill_ms": prefill_s * 1e3,

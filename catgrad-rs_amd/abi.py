@@ -63,6 +63,7 @@ _SIGNATURES = {
     "cg_last_error": (C.c_char_p, [_P]),
     "cg_sync": (C.c_int, [_P]),
     "cg_tensor_realize": (C.c_int, [_P, _P]),
+    "cg_tensor_prefetch": (C.c_int, [_P, _P]),
     "cg_backend_name": (C.c_char_p, [_P]),
     "cg_tensor_retain": (_P, [_P]),
     "cg_tensor_release": (None, [_P]),
@@ -204,6 +205,12 @@ class Backend:
 
     def sync(self):
         self._check(self.lib.cg_sync(self.ptr))
+
+    def prefetch(self, x):
+        """Realize and start an asynchronous copy of a small tensor to the host; `to_vec(x)` then
+        waits for that copy alone."""
+        self._check(self.lib.cg_tensor_prefetch(self.ptr, x.ptr))
+        return x
 
     def realize(self, x):
         """Issue the kernels a deferred tensor still needs (no wait)."""

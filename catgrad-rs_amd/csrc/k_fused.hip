@@ -156,6 +156,100 @@ hipError_t launch_softmax(const LaunchCtx &lc, const SoftmaxDesc &d) {
   return hipGetLastError();
 }
 
+// ---- one-query attention ----------------------------------------------------------------------------------
+// The decode step of models/llama.rs:77-112: scores = q . K^T, / sqrt(d), + mask, softmax, . V, for one
+// query row per head.  One workgroup per (batch, head); LPK lanes share a key/value row (16 bytes
+// each), so a wave covers 64 / LPK rows per load.  Scores live in LDS between the three phases
+// (dot products + max, exp + sum, weighted sum of V rows); nothing of size T goes to HBM.
+template <int LPK>
+__global__ void __launch_bounds__(512) attn_decode_kernel(AttnDecodeDesc a) {
+  constexpr int BLOCK = 512, NW = BLOCK / 64;
+  constexpr int KPW = 64 / LPK;       // rows per wave per load
+  constexpr int STRIDE = NW * KPW;    // rows per workgroup per load
+  constexpr int U = 4;                // independent row loads in flight per lane
+  __shared__ float sc[ATTN_DECODE_MAX_T];
+  __shared__ float red[STRIDE][LPK * 4];
+  __shared__ float lds[NW];
+  const uint32_t h = blockIdx.x, b = blockIdx.y;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int sub = lane % LPK, kg = lane / LPK;
+  const uint32_t kv = h / a.rep, rp = h % a.rep;
+  const float *q = a.q + (int64_t)b * a.q_sb + (int64_t)h * a.q_sh;
+  const float *K = a.k + (int64_t)b * a.k_sb + (int64_t)kv * a.k_skv + (int64_t)rp * a.k_srep;
+  const float *V = a.v + (int64_t)b * a.v_sb + (int64_t)kv * a.v_skv + (int64_t)rp * a.v_srep;
+  const bool live = (uint32_t)sub * 4 < a.d;
+  float4 qv = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (live) qv = *(const float4 *)(q + sub * 4);
+  const uint32_t first = wave * KPW + kg;
+  // phase 1: scores and their maximum
+  float mx = -3.40282347e+38f;
+  for (uint32_t t0 = first; t0 < a.t; t0 += STRIDE * U) {
+    float4 kr[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const uint32_t t = t0 + u * STRIDE;
+      kr[u] = (live && t < a.t) ? *(const float4 *)(K + (int64_t)t * a.k_st + sub * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const uint32_t t = t0 + u * STRIDE;
+      float s = qv.x * kr[u].x + qv.y * kr[u].y + qv.z * kr[u].z + qv.w * kr[u].w;
+#pragma unroll
+      for (int m = LPK / 2; m >= 1; m >>= 1) s += __shfl_xor(s, m, 64);
+      if (a.has_scale) s = s / a.scale;
+      if (a.has_mask_const) s = s + a.mask_const;
+      if (t < a.t) {
+        if (sub == 0) sc[t] = s;
+        mx = fmaxf(mx, s);
+      }
+    }
+  }
+  mx = block_reduce<BLOCK, true>(mx, lds);  // its barrier also publishes sc[]
+  // phase 2: exponentials and their sum
+  float sum = 0.f;
+  for (uint32_t t = tid; t < a.t; t += BLOCK) {
+    const float e = expf(sc[t] - mx);
+    sc[t] = e;
+    sum += e;
+  }
+  sum = block_reduce<BLOCK, false>(sum, lds);
+  // phase 3: weighted sum of V rows
+  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (uint32_t t0 = first; t0 < a.t; t0 += STRIDE * U) {
+    float4 vr[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const uint32_t t = t0 + u * STRIDE;
+      vr[u] = (live && t < a.t) ? *(const float4 *)(V + (int64_t)t * a.v_st + sub * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const uint32_t t = t0 + u * STRIDE;
+      if (t < a.t) {
+        const float p = sc[t] / sum;
+        acc.x += p * vr[u].x; acc.y += p * vr[u].y; acc.z += p * vr[u].z; acc.w += p * vr[u].w;
+      }
+    }
+  }
+  *(float4 *)(&red[wave * KPW + kg][sub * 4]) = acc;
+  __syncthreads();
+  if ((uint32_t)tid < a.d) {
+    float o = 0.f;
+#pragma unroll
+    for (int g = 0; g < STRIDE; ++g) o += red[g][tid];
+    a.out[((uint64_t)b * a.heads + h) * a.d + tid] = o;
+  }
+}
+
+hipError_t launch_attn_decode(const LaunchCtx &lc, const AttnDecodeDesc &d) {
+  if (!d.b || !d.heads || !d.d) return hipSuccess;
+  dim3 grid(d.heads, d.b);
+  if (d.d <= 64) CG_LAUNCH(lc, (attn_decode_kernel<16>), grid, 512, d);
+  else if (d.d <= 128) CG_LAUNCH(lc, (attn_decode_kernel<32>), grid, 512, d);
+  else CG_LAUNCH(lc, (attn_decode_kernel<64>), grid, 512, d);
+  return hipGetLastError();
+}
+
 // ---- rope -------------------------------------------------------------------------------------------
 // out[b,h,s,j] = cos[s,j] * x[b,h,s,j] + sin[s,j] * rot, rot = j < half ? -x[..,j+half] : x[..,j-half]
 // x is read through (b, h, s) strides with a unit stride along j, so the transposed view of the

@@ -97,6 +97,22 @@ hipError_t launch_glu(const LaunchCtx &lc, int gelu, const float *gate, const fl
 hipError_t launch_binary_f32(const LaunchCtx &lc, int op, const float *a, const float *b, float *out,
                              uint64_t n, uint32_t b_period);
 
+// One-query attention (a decode step): out[b, h, :] = softmax(q[b, h, :] . K[b, h, t, :] / scale + mask_const) . V
+// K and V rows are read in place from the (growable) cache through strides; head h of a
+// grouped-query model reads kv head h / rep (stride 0 along the repeat axis).
+struct AttnDecodeDesc {
+  const float *q, *k, *v;
+  float *out;                       // contiguous [b, heads, d]
+  int64_t q_sb, q_sh;               // q strides (unit stride along d)
+  int64_t k_sb, k_skv, k_srep, k_st;  // K[b, kv, rep, t, :] strides (unit stride along d)
+  int64_t v_sb, v_skv, v_srep, v_st;
+  uint32_t b, heads, rep, t, d;
+  int32_t has_scale, has_mask_const;
+  float scale, mask_const;
+};
+enum { ATTN_DECODE_MAX_T = 8192, ATTN_DECODE_MAX_D = 256 };
+hipError_t launch_attn_decode(const LaunchCtx &lc, const AttnDecodeDesc &d);
+
 // ---- k_gemm.hip
 struct GemmDesc {
   const void *a, *b;

@@ -112,6 +112,8 @@ void backend_release(cg_backend *be) {
     (void)hipEventDestroy(pe.stop);
   }
   trim_pool(be);
+  for (void *p : be->pinned_pool) (void)hipHostFree(p);
+  for (hipEvent_t ev : be->event_pool) (void)hipEventDestroy(ev);
   if (be->d_words) (void)hipFree(be->d_words);
   if (be->h_words) (void)hipHostFree(be->h_words);
   if (be->stream) (void)hipStreamDestroy(be->stream);
@@ -141,18 +143,26 @@ void forget_gemv_candidate(cg_tensor *n) {
   n->gemv_candidate = false;
 }
 
+enum { PREFETCH_BYTES = 4096 };  // pinned buffer of a prefetched tensor: data + 8 bytes of error words
+
 void node_release(cg_tensor *t) {
-  if (!t) return;
+  if (!t || t->rc.fetch_sub(1) != 1) return;  // the common case takes no allocation
   std::vector<cg_tensor *> stack{t};
   while (!stack.empty()) {
     cg_tensor *n = stack.back();
     stack.pop_back();
-    if (n->rc.fetch_sub(1) != 1) continue;
+    if (n != t && n->rc.fetch_sub(1) != 1) continue;
     if (n->gemv_candidate) forget_gemv_candidate(n);
     if (n->in[0]) stack.push_back(n->in[0]);
     if (n->in[1]) stack.push_back(n->in[1]);
     storage_release(n->st);
     cg_backend *be = n->be;
+    if (n->host_copy) {
+      // the copy may still be in flight: the buffer is only reused after its event has completed
+      (void)hipEventSynchronize(n->host_ev);
+      be->pinned_pool.push_back(n->host_copy);
+      be->event_pool.push_back(n->host_ev);
+    }
     delete n;
     backend_release(be);
   }
@@ -786,45 +796,65 @@ void finish_fused(cg_tensor *n) {
   drop_inputs(n);
 }
 
-// nn::softmax (stdlib/nn/mod.rs:162-171) with attention's `/ sqrt(d)` and `+ mask` in front
-int try_softmax(cg_backend *be, cg_tensor *root, bool *done) {
-  if (root->dtype != CG_F32 || root->rank == 0 || !is_bin(root, E_DIV_F)) return CG_OK;
-  cg_tensor *ex = root->in[0], *bs = root->in[1];
-  if (!is_bin(ex, E_POW_F) || refs(ex) != 2 || !is_constf(ex->in[0], F_E)) return CG_OK;
-  if (bs->op != N_BROADCAST || refs(bs) != 1 || !is_row_broadcast(bs, root)) return CG_OK;
-  cg_tensor *sm = bs->in[0];
-  if (sm->op != N_REDUCE || sm->p0 != R_SUM_F || refs(sm) != 1 || sm->in[0] != ex) return CG_OK;
-  cg_tensor *sb = ex->in[1];
-  if (!is_bin(sb, E_SUB_F) || refs(sb) != 1) return CG_OK;
-  cg_tensor *x = sb->in[0], *bm = sb->in[1];
-  if (bm->op != N_BROADCAST || refs(bm) != 1 || !is_row_broadcast(bm, root)) return CG_OK;
-  cg_tensor *mx = bm->in[0];
-  if (mx->op != N_REDUCE || mx->p0 != R_MAX_F || refs(mx) != 1 || mx->in[0] != x) return CG_OK;
-  const int64_t n = root->shape[root->rank - 1];
-  if (n == 0 || n > 16384 || root->size() >= ((int64_t)1 << 31)) return CG_OK;
+// nn::softmax (stdlib/nn/mod.rs:162-171) with attention's `/ sqrt(d)` and `+ mask` in front:
+// pure matching, nothing is realised.  src is the tensor the scale / mask / softmax apply to.
+struct SoftmaxMatch {
+  cg_tensor *src = nullptr, *mask = nullptr;
+  cg_tensor *x = nullptr;  // what max / sub / exp are applied to (src after scale and mask)
+  bool has_scale = false, has_mask_const = false;
+  float scale = 1.f, mask_const = 0.f;
+};
 
-  SoftmaxDesc d;
-  std::memset(&d, 0, sizeof(d));
-  cg_tensor *src = x, *mask = nullptr;
+bool match_softmax(cg_tensor *root, SoftmaxMatch *m) {
+  if (root->dtype != CG_F32 || root->rank == 0 || !is_bin(root, E_DIV_F)) return false;
+  cg_tensor *ex = root->in[0], *bs = root->in[1];
+  if (!is_bin(ex, E_POW_F) || refs(ex) != 2 || !is_constf(ex->in[0], F_E)) return false;
+  if (bs->op != N_BROADCAST || refs(bs) != 1 || !is_row_broadcast(bs, root)) return false;
+  cg_tensor *sm = bs->in[0];
+  if (sm->op != N_REDUCE || sm->p0 != R_SUM_F || refs(sm) != 1 || sm->in[0] != ex) return false;
+  cg_tensor *sb = ex->in[1];
+  if (!is_bin(sb, E_SUB_F) || refs(sb) != 1) return false;
+  cg_tensor *x = sb->in[0], *bm = sb->in[1];
+  if (bm->op != N_BROADCAST || refs(bm) != 1 || !is_row_broadcast(bm, root)) return false;
+  cg_tensor *mx = bm->in[0];
+  if (mx->op != N_REDUCE || mx->p0 != R_MAX_F || refs(mx) != 1 || mx->in[0] != x) return false;
+  const int64_t n = root->shape[root->rank - 1];
+  if (n == 0 || n > 16384 || root->size() >= ((int64_t)1 << 31)) return false;
+  m->src = x;
+  m->x = x;
   if (x->op != N_REAL && refs(x) == 2) {
     cg_tensor *y = x;
     if (is_bin(x, E_ADD_F)) {  // attn + mask
       cg_tensor *mk = x->in[1];
       if (mk->op == N_CONST) {
-        d.has_mask_const = 1;
-        d.mask_const = bits_f(mk->cbits);
+        m->has_mask_const = true;
+        m->mask_const = bits_f(mk->cbits);
       } else {
-        mask = mk;
+        m->mask = mk;
       }
       y = x->in[0];
-      src = y;
+      m->src = y;
     }
     if (is_bin(y, E_DIV_F) && y->in[1]->op == N_CONST && (y == x || refs(y) == 1)) {  // attn / sqrt(d)
-      d.has_scale = 1;
-      d.scale = bits_f(y->in[1]->cbits);
-      src = y->in[0];
+      m->has_scale = true;
+      m->scale = bits_f(y->in[1]->cbits);
+      m->src = y->in[0];
     }
   }
+  return true;
+}
+
+int try_softmax(cg_backend *be, cg_tensor *root, bool *done) {
+  SoftmaxMatch sm_;
+  if (!match_softmax(root, &sm_)) return CG_OK;
+  const int64_t n = root->shape[root->rank - 1];
+  SoftmaxDesc d;
+  std::memset(&d, 0, sizeof(d));
+  cg_tensor *src = sm_.src, *mask = sm_.mask;
+  d.has_scale = sm_.has_scale;
+  d.scale = sm_.scale;
+  d.has_mask_const = sm_.has_mask_const;
+  d.mask_const = sm_.mask_const;
   cg_tensor *xs = nullptr, *ms = nullptr;
   int64_t row_stride = 0;
   TRY(as_rows(be, src, &xs, &row_stride));
@@ -1455,9 +1485,93 @@ int peel_expert_index(cg_backend *be, cg_tensor *n, ExpertPeel *out) {
   return CG_OK;
 }
 
+// Attention of a decode step (models/llama.rs:77-112 with one query row):
+//   matmul(softmax(matmul(q, K^T) / sqrt(d) + mask), V)
+// in one launch that reads K and V rows in place from the cache; the [b, h, 1, T] scores and
+// probabilities never exist in HBM.
+int try_attn_decode(cg_backend *be, cg_tensor *n, bool *done) {
+  cg_tensor *P = n->in[0];
+  if (P->op == N_REAL || refs(P) != 1 || P->rank != 4) return CG_OK;
+  SoftmaxMatch m;
+  if (!match_softmax(P, &m) || m.mask) return CG_OK;
+  cg_tensor *S = m.src;
+  if (S->op != N_MATMUL || S->rank != 4 || S->shape[2] != 1 || refs(S) != (S == m.x ? 2 : 1)) return CG_OK;
+  const int64_t T = S->shape[3], d = n->shape[3], heads = n->shape[1], nb = n->shape[0];
+  if (T < 1 || T > ATTN_DECODE_MAX_T || d > ATTN_DECODE_MAX_D || d % 4 || n->in[1]->shape[2] != T) return CG_OK;
+  if (S->in[0]->shape[3] != d) return CG_OK;
+  MatOperand Kop, Vop;
+  bool pk = false, pv = false;
+  TRY(peel_repeat_kv(be, S->in[1], &Kop, &pk));
+  TRY(peel_repeat_kv(be, n->in[1], &Vop, &pv));
+  auto unpeeled = [&](cg_tensor *t, MatOperand *o) -> int {  // [b, h, r, c] as [b, h, 1, r, c]
+    TRY(realize(be, t));
+    o->set(retain(t));
+    for (int i = 4; i >= 3; --i) {
+      o->shape[i] = o->shape[i - 1];
+      o->strides[i] = o->strides[i - 1];
+    }
+    o->shape[2] = 1;
+    o->strides[2] = 0;
+    o->rank = 5;
+    return CG_OK;
+  };
+  if (!pk) TRY(unpeeled(S->in[1], &Kop));
+  if (!pv) TRY(unpeeled(n->in[1], &Vop));
+  cg_tensor *q = S->in[0];
+  TRY(realize(be, q));
+  auto rows_ok = [](const void *ptr, int64_t unit, std::initializer_list<int64_t> strides) {
+    if (unit != 1 || (uintptr_t)ptr % 16) return false;
+    for (int64_t st : strides)
+      if (st % 4) return false;
+    return true;
+  };
+  // K as [b, kv, rep, d, T] (the transposed view), V as [b, kv, rep, T, d]
+  if (Kop.shape[2] != Vop.shape[2] || Kop.shape[1] != Vop.shape[1] || Kop.shape[1] * Kop.shape[2] != heads) return CG_OK;
+  if (q->stype != ST_F32 || Kop.t->stype != ST_F32 || Vop.t->stype != ST_F32) return CG_OK;
+  if (!rows_ok(data_ptr(q), q->strides[3], {q->strides[0], q->strides[1]}) ||
+      !rows_ok(data_ptr(Kop.t), Kop.strides[3], {Kop.strides[0], Kop.strides[1], Kop.strides[2], Kop.strides[4]}) ||
+      !rows_ok(data_ptr(Vop.t), Vop.strides[4], {Vop.strides[0], Vop.strides[1], Vop.strides[2], Vop.strides[3]}))
+    return CG_OK;
+  TRY(alloc_result(be, n, ST_F32));
+  AttnDecodeDesc a;
+  std::memset(&a, 0, sizeof(a));
+  a.q = (const float *)data_ptr(q);
+  a.k = (const float *)data_ptr(Kop.t);
+  a.v = (const float *)data_ptr(Vop.t);
+  a.out = (float *)n->st->ptr;
+  a.q_sb = q->strides[0];
+  a.q_sh = q->strides[1];
+  a.k_sb = Kop.strides[0]; a.k_skv = Kop.strides[1]; a.k_srep = Kop.strides[2]; a.k_st = Kop.strides[4];
+  a.v_sb = Vop.strides[0]; a.v_skv = Vop.strides[1]; a.v_srep = Vop.strides[2]; a.v_st = Vop.strides[3];
+  a.b = (uint32_t)nb;
+  a.heads = (uint32_t)heads;
+  a.rep = (uint32_t)Kop.shape[2];
+  a.t = (uint32_t)T;
+  a.d = (uint32_t)d;
+  a.has_scale = m.has_scale;
+  a.scale = m.scale;
+  a.has_mask_const = m.has_mask_const;
+  a.mask_const = m.mask_const;
+  {
+    const double kv_bytes = 2.0 * nb * Kop.shape[1] * T * d * 4;
+    KernelScope ks(be, "attn_decode", kv_bytes + 2.0 * nb * heads * d * 4, 4.0 * nb * heads * T * d);
+    HIPCHK(be, launch_attn_decode(be->lc(), a));
+  }
+  if (n->gemv_candidate) forget_gemv_candidate(n);
+  n->op = N_REAL;
+  drop_inputs(n);
+  *done = true;
+  return CG_OK;
+}
+
 // `addend` (optional; realised, f32, contiguous, shaped like n) is added in the epilogue when a
 // one-row kernel runs the product; *added tells the caller whether that happened.
 int realize_matmul(cg_backend *be, cg_tensor *n, cg_tensor *addend = nullptr, bool *added = nullptr) {
+  if (!addend && n->dtype == CG_F32 && n->rank == 4 && n->shape[2] == 1 && !(be->flags & CG_FLAG_NO_PATTERNS)) {
+    bool done = false;
+    TRY(try_attn_decode(be, n, &done));
+    if (done) return CG_OK;
+  }
   MatOperand A, B;
   bool pa = false, pb = false;
   ExpertPeel ex;
@@ -1643,6 +1757,12 @@ int realize_matmul(cg_backend *be, cg_tensor *n, cg_tensor *addend = nullptr, bo
         }
         {
           KernelScope ks(be, g.b_stype == ST_BF16 ? "gemv_rowdot_bf16" : "gemv_rowdot_f32", bytes, flops);
+          if (be->trace_shapes) {
+            char buf[96];
+            snprintf(buf, sizeof buf, "%s[multi%d,K%u,N%.0f]", g.b_stype == ST_BF16 ? "gemv_rowdot_bf16" : "gemv_rowdot_f32",
+                     md.n_prob, K, flops / (2.0 * K));
+            ks.rename(buf);
+          }
           HIPCHK(be, launch_gemv_multi(be->lc(), md));
         }
         for (cg_tensor *c : members) {
@@ -2006,6 +2126,15 @@ int download(cg_backend *be, cg_tensor *x, void *dst, size_t n, cg_dtype want) {
   if (x->dtype != want) return fail(be, CG_ERR_DTYPE, "to_vec: wrong dtype for this accessor");
   if ((int64_t)n != x->size()) return fail(be, CG_ERR_SHAPE, "to_vec: size mismatch");
   HIPCHK(be, hipSetDevice(be->device));
+  if (x->host_copy) {  // prefetched: wait for that copy only, not for work queued behind it
+    HIPCHK(be, hipEventSynchronize(x->host_ev));
+    const uint32_t *words = (const uint32_t *)((const char *)x->host_copy + PREFETCH_BYTES - 8);
+    if (words[0] == 0) {
+      std::memcpy(dst, x->host_copy, n * 4);
+      return CG_OK;
+    }
+    // a kernel flagged an error: take the synchronising path, which reports it
+  }
   cg_tensor *c = nullptr;
   TRY(contiguous(be, x, &c));
   int st = CG_OK;
@@ -2054,6 +2183,42 @@ int cg_sync(cg_backend *be) {
   if (!be) return CG_ERR_ARG;
   HIPCHK(be, hipSetDevice(be->device));
   return sync_and_check(be);
+}
+
+int cg_tensor_prefetch(cg_backend *be, cg_tensor *t) {
+  if (!be || !t || t->be != be) return CG_ERR_ARG;
+  HIPCHK(be, hipSetDevice(be->device));
+  TRY(realize(be, t));
+  const size_t bytes = (size_t)t->size() * 4;
+  if (t->host_copy || bytes == 0 || bytes > PREFETCH_BYTES - 8 || esize(t->stype) != 4 || !is_contiguous(t))
+    return CG_OK;  // the read will take the synchronising path
+  void *buf = nullptr;
+  hipEvent_t ev = nullptr;
+  if (!be->pinned_pool.empty()) {
+    buf = be->pinned_pool.back();
+    be->pinned_pool.pop_back();
+  } else {
+    HIPCHK(be, hipHostMalloc(&buf, PREFETCH_BYTES, hipHostMallocDefault));
+  }
+  if (!be->event_pool.empty()) {
+    ev = be->event_pool.back();
+    be->event_pool.pop_back();
+  } else if (hipEventCreateWithFlags(&ev, hipEventDisableTiming) != hipSuccess) {
+    be->pinned_pool.push_back(buf);
+    return fail(be, CG_ERR_DEVICE, "hipEventCreate failed");
+  }
+  hipError_t e = hipMemcpyAsync(buf, data_ptr(t), bytes, hipMemcpyDeviceToHost, be->stream);
+  if (e == hipSuccess)
+    e = hipMemcpyAsync((char *)buf + PREFETCH_BYTES - 8, be->d_words, 8, hipMemcpyDeviceToHost, be->stream);
+  if (e == hipSuccess) e = hipEventRecord(ev, be->stream);
+  if (e != hipSuccess) {
+    be->pinned_pool.push_back(buf);
+    be->event_pool.push_back(ev);
+    return fail(be, CG_ERR_DEVICE, hipGetErrorString(e));
+  }
+  t->host_copy = buf;
+  t->host_ev = ev;
+  return CG_OK;
 }
 
 int cg_tensor_realize(cg_backend *be, cg_tensor *t) {

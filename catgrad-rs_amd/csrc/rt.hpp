@@ -80,6 +80,10 @@ struct cg_tensor {
   int64_t p0 = 0, p1 = 0;
   uint32_t cbits = 0;
   bool gemv_candidate = false;  // listed in cg_backend::gemv_candidates (a weak reference)
+  // cg_tensor_prefetch: a pinned host copy in flight (data, then the backend's error words) and the
+  // event recorded behind the copy
+  void *host_copy = nullptr;
+  hipEvent_t host_ev = nullptr;
 
   int64_t size() const {
     int64_t n = 1;
@@ -110,6 +114,9 @@ struct cg_backend {
   // issued as one launch; weak references, removed when a node is realised or deleted
   std::vector<cg_tensor *> gemv_candidates;
   hipEvent_t cur_start = nullptr, cur_stop = nullptr;  // set while a traced launch is issued
+  // recycled pinned buffers (PREFETCH_BYTES each) and events of cg_tensor_prefetch
+  std::vector<void *> pinned_pool;
+  std::vector<hipEvent_t> event_pool;
 
   cgk::LaunchCtx lc() const { return cgk::LaunchCtx{stream, n_cus, d_words, cur_start, cur_stop}; }
 };

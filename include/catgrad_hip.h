@@ -82,6 +82,12 @@ int cg_sync(cg_backend *be);
  * whose backends compute inside every call: the HIP backend records calls and computes when a value
  * is read (cg_to_f32 / cg_to_u32 / cg_compare) or here; a no-op for the oracle */
 int cg_tensor_realize(cg_backend *be, cg_tensor *t);
+/* cg_tensor_realize, then start copying a small tensor (<= 4088 bytes, e.g. the sampled token) to
+ * pinned host memory behind the work queued so far.  A later cg_to_f32 / cg_to_u32 of the same
+ * handle waits for that copy only, so the caller can keep the device busy with the next step while
+ * it reads this one.  Larger or strided tensors are left alone (their read synchronises as usual).
+ * No counterpart in the reference, whose to_vec is the only way out of a tensor. */
+int cg_tensor_prefetch(cg_backend *be, cg_tensor *t);
 /* "hip-gfx950" or "ndarray-oracle" */
 const char *cg_backend_name(const cg_backend *be);
 

@@ -89,6 +89,7 @@ void cg_backend_destroy(cg_backend *be) { delete be; }
 const char *cg_last_error(const cg_backend *be) { return be ? be->err.c_str() : ""; }
 int cg_sync(cg_backend *) { return CG_OK; }
 int cg_tensor_realize(cg_backend *, cg_tensor *) { return CG_OK; }
+int cg_tensor_prefetch(cg_backend *, cg_tensor *) { return CG_OK; }
 const char *cg_backend_name(const cg_backend *) { return "ndarray-oracle"; }
 
 cg_tensor *cg_tensor_retain(cg_tensor *t) {

@@ -77,11 +77,29 @@ class CachedRunner:
         return out[0], out[1]
 
     def step(self, token):
-        ids = self.be.tensor(np.asarray([[token]], np.uint32))
+        """`token`: an int, or the [1, 1, 1] token tensor of the previous step (stays on the device)."""
+        if isinstance(token, cg.Tensor):
+            ids = self.be.reshape(token, [1, 1])
+        else:
+            ids = self.be.tensor(np.asarray([[token]], np.uint32))
         out = self.it.run(self.decode_term, [ids, self.pos, self.cos, self.sin] + self.kv)
         self.kv = out[2:]
         self.pos += 1
         return out[0], out[1]
+
+    def generate_pipelined(self, prompt, steps):
+        """Greedy tokens with the sampled token fed back on the device and read one step behind:
+        the host records and issues step t+1 while the device still runs step t."""
+        tok, _ = self.prefill(prompt)
+        self.be.prefetch(tok)
+        toks, prev = [], tok
+        for _ in range(steps - 1):
+            tok, _ = self.step(prev)
+            self.be.prefetch(tok)
+            toks.append(int(self.be.to_vec(prev)[0]))
+            prev = tok
+        toks.append(int(self.be.to_vec(prev)[0]))
+        return toks
 
     def generate(self, prompt, steps):
         """Returns (tokens, logits per step as numpy)."""

@@ -164,3 +164,36 @@ def test_residual_add_in_gemv_epilogue(oracle, hip, hip_nopat, shape, order):
         assert "binary_f32" not in names, sorted(names)
     assert np.allclose(got[0], ref, rtol=1e-4, atol=1e-5)
     assert np.allclose(gen, ref, rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize("cfg", [(1, 32, 8, 513, 64), (1, 4, 4, 7, 16), (2, 8, 2, 100, 128), (1, 4, 1, 33, 256),
+                                 (1, 16, 16, 1, 64)])  # b, heads, kv heads, T, d
+def test_attention_decode(oracle, hip, hip_nopat, cfg):
+    """One-query attention over a cache (q . K^T / sqrt(d) + mask, softmax, . V) as one launch."""
+    nb, H, KV, T, d = cfg
+    g = np.random.default_rng(T * 3 + d)
+    q = g.standard_normal((nb, H, 1, d)).astype(np.float32)
+    k = g.standard_normal((nb, KV, T, d)).astype(np.float32)
+    v = g.standard_normal((nb, KV, T, d)).astype(np.float32)
+
+    def f(b, qv, kv, vv):
+        qv, kv, vv = qv + qv - qv, kv + kv - kv, vv + vv - vv      # computed f32 values
+        kr = helpers.repeat_kv(b, H // KV, kv)
+        vr = helpers.repeat_kv(b, H // KV, vv)
+        attn = lang.matmul(b, qv, lang.transpose(b, 2, 3, kr))
+        sh = lang.shape(b, attn)
+        attn = attn / lang.constant(b, float(np.sqrt(np.float32(d))), sh)
+        attn = attn + lang.broadcast(b, helpers.causal_mask(b, lang.to_nat(b, 1)), sh)
+        return lang.matmul(b, nn.softmax(b, attn), vr)
+    (ref,) = vectors.run(oracle, f, 1, q, k, v)
+    got, names = run_traced(hip, f, 1, q, k, v)
+    gen, gnames = run_traced(hip_nopat, f, 1, q, k, v)
+    assert "attn_decode" in names and "softmax_fused" not in names, sorted(names)
+    assert "attn_decode" not in gnames
+    s = np.einsum("bhd,bhtd->bht", q[:, :, 0].astype(np.float64), np.repeat(k, H // KV, 1).astype(np.float64)) / np.sqrt(d)
+    p = np.exp(s - s.max(-1, keepdims=True))
+    p /= p.sum(-1, keepdims=True)
+    expect = np.einsum("bht,bhtd->bhd", p, np.repeat(v, H // KV, 1).astype(np.float64))[:, :, None]
+    assert np.allclose(ref, expect, rtol=1e-4, atol=1e-5)
+    assert np.allclose(got[0], ref, rtol=1e-4, atol=1e-5), np.abs(got[0] - ref).max()
+    assert np.allclose(gen[0], ref, rtol=1e-4, atol=1e-5)

@@ -106,3 +106,26 @@ def test_llama_bf16_logits(oracle, hip_bf16):
     _, gl = g.step(tok)
     rl, gl = oracle.to_vec(rl), hip_bf16.to_vec(gl)
     assert np.max(np.abs(rl - gl)) <= 2e-2 * np.abs(rl).max()
+
+
+@pytest.mark.gpu
+def test_pipelined_decode_gives_the_same_tokens(hip, hip_bf16):
+    """Token fed back on the device and read one step behind (cg_tensor_prefetch) == the loop that
+    reads every token before the next step; also that a prefetched read returns the right data."""
+    cfg = U.tiny_config(hidden_size=128, intermediate_size=256, num_hidden_layers=3, num_attention_heads=8,
+                        num_key_value_heads=2, vocab_size=509)
+    arrays = U.param_arrays(cfg, seed=5, std=0.1)
+    prompt = list(np.random.default_rng(6).integers(0, cfg.vocab_size, 17))
+    for be in (hip, hip_bf16):
+        sync_tokens, _ = U.CachedRunner(be, cfg, arrays, 64).generate(prompt, 24)
+        piped = U.CachedRunner(be, cfg, arrays, 64).generate_pipelined(prompt, 24)
+        assert piped == sync_tokens
+    x = np.arange(1000, dtype=np.float32)
+    t = hip.add(hip.tensor(x), hip.tensor(x))
+    hip.prefetch(t)
+    later = hip.mul(t, t)                       # more work queued behind the copy
+    assert np.array_equal(hip.to_vec(t), x + x)
+    assert np.array_equal(hip.to_vec(later), (x + x) * (x + x))
+    big = hip.add(hip.tensor(np.ones(5000, np.float32)), hip.tensor(np.ones(5000, np.float32)))
+    hip.prefetch(big)                           # too large for the pinned slot: falls back to the plain read
+    assert np.array_equal(hip.to_vec(big), np.full(5000, 2.0, np.float32))
