@@ -1,0 +1,44 @@
+// dev_common.hpp — device helpers shared by the kernel files: wavefront / workgroup reductions and
+// the activation formulas of the stdlib definitions.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <math.h>
+
+namespace cgk {
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, 64);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) v = fmaxf(v, __shfl_xor(v, m, 64));
+  return v;
+}
+
+// Reduce across the workgroup (BLOCK threads, a multiple of 64); every thread gets the result.
+template <int BLOCK, bool IS_MAX>
+__device__ __forceinline__ float block_reduce(float v, float *lds) {
+  v = IS_MAX ? wave_max(v) : wave_sum(v);
+  if (BLOCK == 64) return v;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  __syncthreads();
+  if (lane == 0) lds[wave] = v;
+  __syncthreads();
+  float r = lds[0];
+#pragma unroll
+  for (int w = 1; w < BLOCK / 64; ++w) r = IS_MAX ? fmaxf(r, lds[w]) : r + lds[w];
+  return r;
+}
+
+__device__ __forceinline__ float sigmoid_ref(float x) { return 1.0f / (1.0f + expf(-x)); }
+// nn::gelu: 0.5 x (1 + tanh(c (x + k x^3))), tanh(t) = 2 sigmoid(2 t) - 1 (nn/mod.rs:138-160)
+__device__ __forceinline__ float gelu_ref(float x) {
+  const float t = __uint_as_float(0x3F4C4229u) * (x + 0.044715f * (x * x * x));  // f32 sqrt(2/pi)
+  const float th = 2.0f * sigmoid_ref(2.0f * t) - 1.0f;
+  return 0.5f * x * (1.0f + th);
+}
+
+
+}  // namespace cgk

@@ -17,6 +17,7 @@
 //  * gemv_col_kernel (M <= 8, B n-contiguous): lanes across n, k split over the workgroup.
 #include <hip/hip_runtime.h>
 #include "launch.hpp"
+#include "dev_common.hpp"
 
 namespace cgk {
 
@@ -769,6 +770,153 @@ hipError_t launch_gemv_multi(const LaunchCtx &lc, const GemvMultiDesc &g) {
   dim3 grid(blocks, g.n_prob);
   if (g.b_stype == ST_BF16) CG_LAUNCH(lc, (gemv_multi_kernel<uint16_t>), grid, 256, g);
   else CG_LAUNCH(lc, (gemv_multi_kernel<float>), grid, 256, g);
+  return hipGetLastError();
+}
+
+// ---- GEMVs whose input row is computed in the kernel --------------------------------------------------
+// A decode step spends as much time launching its small kernels as running them.  The RMSNorm in
+// front of q/k/v and gate/up, and the SwiGLU in front of down_proj, produce a single row of K
+// floats: every workgroup recomputes that row into LDS (a few KB from L2, microseconds of ALU
+// spread over all CUs) and then streams its share of the weight rows exactly like
+// gemv_multi_kernel, reading x from LDS.  KSPLIT: the four waves of a workgroup share a column
+// pair and take a quarter of k each (deep, narrow matrices).
+template <typename TB, bool KSPLIT>
+__global__ void __launch_bounds__(256) gemv_pro_kernel(GemvProDesc g) {
+  typedef typename WVec<TB>::type VT;
+  constexpr int EPL = WVec<TB>::EPL, UNROLL = 4, R = 2;
+  __shared__ __attribute__((aligned(16))) float xs[GEMV_PRO_MAX_K];
+  __shared__ float lds[4];
+  __shared__ float part[4][R];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const uint32_t K = g.m.K;
+  // ---- prologue: the input row
+  if (g.pro == PRO_RMSNORM) {
+    float ss = 0.f;
+    for (uint32_t k = tid * 4; k < K; k += 1024) {
+      const float4 v = *(const float4 *)(g.a + k);
+      ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+    }
+    ss = block_reduce<256, false>(ss, lds);
+    const float rms = sqrtf(ss / g.n_as_float + g.eps);
+    for (uint32_t k = tid * 4; k < K; k += 1024) {
+      const float4 v = *(const float4 *)(g.a + k);
+      float4 o;
+      o.x = v.x / rms; o.y = v.y / rms; o.z = v.z / rms; o.w = v.w / rms;
+      if (g.aux) {
+        const float4 gm = *(const float4 *)(g.aux + k);
+        o.x *= g.gamma_offset + gm.x; o.y *= g.gamma_offset + gm.y;
+        o.z *= g.gamma_offset + gm.z; o.w *= g.gamma_offset + gm.w;
+      }
+      *(float4 *)(xs + k) = o;
+    }
+  } else {
+    for (uint32_t k = tid * 4; k < K; k += 1024) {
+      const float4 a = *(const float4 *)(g.a + k), u = *(const float4 *)(g.aux + k);
+      float4 o;
+      if (g.pro == PRO_GEGLU) {
+        o.x = gelu_ref(a.x) * u.x; o.y = gelu_ref(a.y) * u.y;
+        o.z = gelu_ref(a.z) * u.z; o.w = gelu_ref(a.w) * u.w;
+      } else {
+        o.x = a.x * sigmoid_ref(a.x) * u.x; o.y = a.y * sigmoid_ref(a.y) * u.y;
+        o.z = a.z * sigmoid_ref(a.z) * u.z; o.w = a.w * sigmoid_ref(a.w) * u.w;
+      }
+      *(float4 *)(xs + k) = o;
+    }
+  }
+  __syncthreads();
+  // ---- the products
+  const uint32_t N = g.m.p[blockIdx.y].N;
+  const TB *B = (const TB *)g.m.p[blockIdx.y].b;
+  const int64_t sbn = g.m.p[blockIdx.y].sbn;
+  float *C = g.m.p[blockIdx.y].c;
+  const float *Cadd = g.m.p[blockIdx.y].c_add;
+  const uint32_t slot = KSPLIT ? blockIdx.x : blockIdx.x * 4 + wave;
+  const uint32_t n_slots = KSPLIT ? gridDim.x : gridDim.x * 4;
+  uint32_t k_begin = 0, k_end = K;
+  if (KSPLIT) {
+    const uint32_t per = ((K + 3) / 4 + EPL - 1) / EPL * EPL;
+    k_begin = min(K, wave * per);
+    k_end = min(K, k_begin + per);
+  }
+  for (uint32_t nb = slot * R; nb < N; nb += n_slots * R) {  // uniform per workgroup when KSPLIT
+    float acc[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) acc[r] = 0.f;
+    for (uint32_t k0 = k_begin + lane * EPL; k0 < k_end; k0 += 64 * EPL * UNROLL) {
+      VT q[R][UNROLL];
+#pragma unroll
+      for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+          const uint32_t k = k0 + u * 64 * EPL;
+          if (k < k_end && nb + r < N)
+            q[r][u] = __builtin_nontemporal_load((const VT *)(B + (int64_t)(nb + r) * sbn + k));
+        }
+#pragma unroll
+      for (int u = 0; u < UNROLL; ++u) {
+        const uint32_t k = k0 + u * 64 * EPL;
+        if (k < k_end) {
+          float xv[EPL];
+#pragma unroll
+          for (int j4 = 0; j4 < EPL; j4 += 4) {
+            const float4 t = *(const float4 *)(xs + k + j4);
+            xv[j4] = t.x; xv[j4 + 1] = t.y; xv[j4 + 2] = t.z; xv[j4 + 3] = t.w;
+          }
+#pragma unroll
+          for (int r = 0; r < R; ++r) {
+            if (nb + r < N) {
+              float w[EPL];
+              WVec<TB>::widen(q[r][u], w);
+#pragma unroll
+              for (int j = 0; j < EPL; ++j) acc[r] += w[j] * xv[j];
+            }
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) acc[r] = wave_sum(acc[r]);
+    if (KSPLIT) {
+      __syncthreads();
+      if (lane == 0)
+#pragma unroll
+        for (int r = 0; r < R; ++r) part[wave][r] = acc[r];
+      __syncthreads();
+      if (tid < R && nb + tid < N)
+        C[nb + tid] = ((part[0][tid] + part[1][tid]) + (part[2][tid] + part[3][tid])) + (Cadd ? Cadd[nb + tid] : 0.f);
+    } else if (lane == 0) {
+#pragma unroll
+      for (int r = 0; r < R; ++r)
+        if (nb + r < N) C[nb + r] = acc[r] + (Cadd ? Cadd[nb + r] : 0.f);
+    }
+  }
+}
+
+template <typename TB, bool KSPLIT>
+static void launch_gemv_pro_block(const LaunchCtx &lc, const GemvProDesc &g, uint32_t slots) {
+  // `slots` = column pairs per problem; 256-thread workgroups (wider ones stream worse).  Long input
+  // rows cost more to recompute, so fewer workgroups each take several column pairs.
+  const uint32_t per_wg = KSPLIT ? 1 : 4;
+  uint32_t blocks = (slots + per_wg - 1) / per_wg;
+  const uint32_t cap = (uint32_t)lc.n_cus * (g.m.K >= 4096 ? 2 : 4) / g.m.n_prob;
+  if (blocks > cap) blocks = cap ? cap : 1;
+  dim3 grid(blocks, g.m.n_prob);
+  CG_LAUNCH(lc, (gemv_pro_kernel<TB, KSPLIT>), grid, 256, g);
+}
+
+hipError_t launch_gemv_pro(const LaunchCtx &lc, const GemvProDesc &g) {
+  uint32_t max_n = 0;
+  for (int i = 0; i < g.m.n_prob; ++i) max_n = g.m.p[i].N > max_n ? g.m.p[i].N : max_n;
+  if (!max_n || !g.m.n_prob) return hipSuccess;
+  const uint32_t slots = (max_n + 1) / 2;
+  const bool ksplit = g.m.K >= 4096 && slots * (uint32_t)g.m.n_prob <= (uint32_t)lc.n_cus * 8;
+  if (g.m.b_stype == ST_BF16) {
+    if (ksplit) launch_gemv_pro_block<uint16_t, true>(lc, g, slots);
+    else launch_gemv_pro_block<uint16_t, false>(lc, g, slots);
+  } else {
+    if (ksplit) launch_gemv_pro_block<float, true>(lc, g, slots);
+    else launch_gemv_pro_block<float, false>(lc, g, slots);
+  }
   return hipGetLastError();
 }
 

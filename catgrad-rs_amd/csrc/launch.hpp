@@ -157,6 +157,19 @@ struct GemvMultiDesc {
   } p[4];
 };
 hipError_t launch_gemv_multi(const LaunchCtx &lc, const GemvMultiDesc &g);
+// The same, with x produced inside the kernel (once per workgroup, kept in LDS) from the op that
+// feeds these projections in a decoder layer, so that op needs no launch of its own:
+//   PRO_RMSNORM: x = a / sqrt(sum(a*a) / n + eps) * (gamma_offset + gamma)   (gamma may be null)
+//   PRO_SWIGLU / PRO_GEGLU: x = silu(a) * aux  /  gelu(a) * aux
+// K <= GEMV_PRO_MAX_K, K % 8 == 0; a, aux, gamma contiguous, 16-byte aligned
+enum { PRO_RMSNORM = 1, PRO_SWIGLU = 2, PRO_GEGLU = 3, GEMV_PRO_MAX_K = 8192 };
+struct GemvProDesc {
+  GemvMultiDesc m;  // m.x is ignored
+  int32_t pro;
+  const float *a, *aux;
+  float n_as_float, eps, gamma_offset;
+};
+hipError_t launch_gemv_pro(const LaunchCtx &lc, const GemvProDesc &g);
 // wrapping u32 matmul (ndarray's generic dot); all operands contiguous
 hipError_t launch_matmul_u32(const LaunchCtx &lc, const uint32_t *a, const uint32_t *b, uint32_t *c,
                              uint32_t batch, uint32_t M, uint32_t N, uint32_t K);

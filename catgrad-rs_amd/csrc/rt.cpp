@@ -919,8 +919,14 @@ int try_softmax(cg_backend *be, cg_tensor *root, bool *done) {
 }
 
 // rmsnorm_raw / rmsnorm (catgrad-llm/src/helpers.rs:120-145; gemma3.rs:41-68)
-int try_rmsnorm(cg_backend *be, cg_tensor *root, bool *done) {
-  if (root->dtype != CG_F32 || root->rank == 0) return CG_OK;
+struct RmsNormMatch {
+  cg_tensor *x = nullptr, *gamma = nullptr;  // gamma: the broadcast node or null
+  float eps = 0.f, n_as_float = 1.f, gamma_offset = 0.f;
+};
+
+// pure matching; nothing is realised
+bool match_rmsnorm(cg_tensor *root, RmsNormMatch *m) {
+  if (root->dtype != CG_F32 || root->rank == 0) return false;
   cg_tensor *dv = root, *gb = nullptr;
   float gamma_offset = 0.f;
   if (is_bin(root, E_MUL_F) && is_bin(root->in[0], E_DIV_F) && refs(root->in[0]) == 1) {
@@ -931,34 +937,54 @@ int try_rmsnorm(cg_backend *be, cg_tensor *root, bool *done) {
       gb = gb->in[1];
     }
   }
-  if (!is_bin(dv, E_DIV_F)) return CG_OK;
+  if (!is_bin(dv, E_DIV_F)) return false;
   cg_tensor *x = dv->in[0], *br = dv->in[1];
-  if (br->op != N_BROADCAST || refs(br) != 1 || !is_row_broadcast(br, root)) return CG_OK;
+  if (br->op != N_BROADCAST || refs(br) != 1 || !is_row_broadcast(br, root)) return false;
   cg_tensor *r = br->in[0];
-  if (!is_bin(r, E_POW_F) || refs(r) != 1 || !is_constf(r->in[1], F_HALF)) return CG_OK;
+  if (!is_bin(r, E_POW_F) || refs(r) != 1 || !is_constf(r->in[1], F_HALF)) return false;
   cg_tensor *a = r->in[0];
-  if (!is_bin(a, E_ADD_F) || refs(a) != 1 || a->in[1]->op != N_CONST) return CG_OK;
+  if (!is_bin(a, E_ADD_F) || refs(a) != 1 || a->in[1]->op != N_CONST) return false;
   cg_tensor *mn = a->in[0];
-  if (!is_bin(mn, E_DIV_F) || refs(mn) != 1 || mn->in[1]->op != N_CONST) return CG_OK;
+  if (!is_bin(mn, E_DIV_F) || refs(mn) != 1 || mn->in[1]->op != N_CONST) return false;
   cg_tensor *sm = mn->in[0];
-  if (sm->op != N_REDUCE || sm->p0 != R_SUM_F || refs(sm) != 1) return CG_OK;
+  if (sm->op != N_REDUCE || sm->p0 != R_SUM_F || refs(sm) != 1) return false;
   cg_tensor *sq = sm->in[0];
-  if (!is_bin(sq, E_MUL_F) || refs(sq) != 1 || sq->in[0] != x || sq->in[1] != x) return CG_OK;
+  if (!is_bin(sq, E_MUL_F) || refs(sq) != 1 || sq->in[0] != x || sq->in[1] != x) return false;
   const int64_t n = root->shape[root->rank - 1];
-  if (n == 0 || n % 4 || n > 16384) return CG_OK;
+  if (n == 0 || n % 4 || n > 16384) return false;
+  m->x = x;
+  m->gamma = gb;
+  m->eps = bits_f(a->in[1]->cbits);
+  m->n_as_float = bits_f(mn->in[1]->cbits);
+  m->gamma_offset = gamma_offset;
+  return true;
+}
 
+// gamma as a row vector broadcast over the rows (realises it); false: some other layout
+int gamma_row_vector(cg_backend *be, cg_tensor *gb, bool *ok) {
+  TRY(realize(be, gb));
+  bool vec = gb->stype == ST_F32 && (gb->shape[gb->rank - 1] == 1 || gb->strides[gb->rank - 1] == 1) &&
+             ((uintptr_t)data_ptr(gb) % 16 == 0);
+  for (int i = 0; i + 1 < gb->rank; ++i)
+    if (gb->shape[i] != 1 && gb->strides[i] != 0) vec = false;
+  *ok = vec;
+  return CG_OK;
+}
+
+int try_rmsnorm(cg_backend *be, cg_tensor *root, bool *done) {
+  RmsNormMatch rm;
+  if (!match_rmsnorm(root, &rm)) return CG_OK;
+  cg_tensor *x = rm.x, *gb = rm.gamma;
+  const int64_t n = root->shape[root->rank - 1];
   RmsNormDesc d;
   std::memset(&d, 0, sizeof(d));
-  d.eps = bits_f(a->in[1]->cbits);
-  d.n_as_float = bits_f(mn->in[1]->cbits);
-  d.gamma_offset = gamma_offset;
+  d.eps = rm.eps;
+  d.n_as_float = rm.n_as_float;
+  d.gamma_offset = rm.gamma_offset;
   cg_tensor *gs = nullptr;
   if (gb) {
-    TRY(realize(be, gb));
-    bool vec = gb->stype == ST_F32 && (gb->shape[gb->rank - 1] == 1 || gb->strides[gb->rank - 1] == 1) &&
-               ((uintptr_t)data_ptr(gb) % 16 == 0);
-    for (int i = 0; i + 1 < gb->rank; ++i)
-      if (gb->shape[i] != 1 && gb->strides[i] != 0) vec = false;
+    bool vec = false;
+    TRY(gamma_row_vector(be, gb, &vec));
     if (!vec) return CG_OK;  // gamma is not a broadcast row vector: generic path
     gs = gb;
   }
@@ -1095,19 +1121,26 @@ bool is_gelu_of(const cg_tensor *g, const cg_tensor **arg) {
 }
 
 // silu(gate) * up (models/llama.rs:26) and gelu(gate) * up (models/gemma3.rs:28)
-int try_glu(cg_backend *be, cg_tensor *root, bool *done) {
-  if (root->dtype != CG_F32 || !is_bin(root, E_MUL_F) || root->size() % 4) return CG_OK;
-  cg_tensor *act = root->in[0], *up = root->in[1];
+bool match_glu(cg_tensor *root, cg_tensor **gate, cg_tensor **up, int *gelu) {
+  if (root->dtype != CG_F32 || !is_bin(root, E_MUL_F) || root->size() % 4) return false;
+  cg_tensor *act = root->in[0];
   const cg_tensor *g = nullptr;
-  int gelu = 0;
   if (is_bin(act, E_MUL_F) && refs(act) == 1 && is_sigmoid_of(act->in[1], &g) && g == act->in[0]) {
-    gelu = 0;
+    *gelu = 0;
   } else if (is_gelu_of(act, &g)) {
-    gelu = 1;
+    *gelu = 1;
   } else {
-    return CG_OK;
+    return false;
   }
-  cg_tensor *gate = const_cast<cg_tensor *>(g);
+  *gate = const_cast<cg_tensor *>(g);
+  *up = root->in[1];
+  return true;
+}
+
+int try_glu(cg_backend *be, cg_tensor *root, bool *done) {
+  cg_tensor *gate = nullptr, *up = nullptr;
+  int gelu = 0;
+  if (!match_glu(root, &gate, &up, &gelu)) return CG_OK;
   cg_tensor *gc = nullptr, *uc = nullptr;
   TRY(contiguous(be, gate, &gc));
   int st = contiguous(be, up, &uc);
@@ -1564,12 +1597,124 @@ int try_attn_decode(cg_backend *be, cg_tensor *n, bool *done) {
   return CG_OK;
 }
 
+// q/k/v, gate/up and down_proj of a decode step: one-row products whose input row is an RMSNorm
+// or a SwiGLU/GeGLU of earlier values.  When every consumer of that row is such a product, the
+// row is computed inside the product kernel (launch_gemv_pro) and its node is never realised.
+int try_gemv_prologue(cg_backend *be, cg_tensor *n, cg_tensor *addend, bool *added, bool *done) {
+  cg_tensor *A = n->in[0];
+  if (A->op == N_REAL || A->dtype != CG_F32 || !n->gemv_candidate || A->rank < 1) return CG_OK;
+  const int64_t K = A->shape[A->rank - 1];
+  if (A->size() != K || K % 8 || K < 256 || K > GEMV_PRO_MAX_K) return CG_OK;
+  RmsNormMatch rm;
+  cg_tensor *gate = nullptr, *up = nullptr;
+  int gelu = 0, pro = 0;
+  if (match_rmsnorm(A, &rm)) pro = PRO_RMSNORM;
+  else if (match_glu(A, &gate, &up, &gelu)) pro = gelu ? PRO_GEGLU : PRO_SWIGLU;
+  else return CG_OK;
+  // the group: every deferred one-row product reading A (n first)
+  std::vector<cg_tensor *> members{n};
+  for (cg_tensor *c : be->gemv_candidates)
+    if (c != n && c->op == N_MATMUL && c->in[0] == A) members.push_back(c);
+  if ((int)members.size() != refs(A) || members.size() > 4) return CG_OK;
+  GemvProDesc d;
+  std::memset(&d, 0, sizeof(d));
+  int b_stype = -1;
+  for (cg_tensor *c : members) {
+    cg_tensor *w = c->in[1];
+    if (c->rank != A->rank || c->size() != c->shape[c->rank - 1]) return CG_OK;
+    TRY(realize(be, w));
+    if (w->rank < 2 || w->shape[w->rank - 2] != K || w->strides[w->rank - 2] != 1) return CG_OK;
+    for (int i = 0; i + 2 < w->rank; ++i)
+      if (w->shape[i] != 1) return CG_OK;
+    if (w->stype != ST_F32 && w->stype != ST_BF16) return CG_OK;
+    if (b_stype >= 0 && w->stype != b_stype) return CG_OK;
+    b_stype = w->stype;
+    if ((uintptr_t)data_ptr(w) % 16 || w->strides[w->rank - 1] % (16 / esize(w->stype))) return CG_OK;
+  }
+  // operands of the row
+  cg_tensor *a0 = nullptr, *a1 = nullptr;
+  if (pro == PRO_RMSNORM) {
+    if (rm.gamma) {
+      bool vec = false;
+      TRY(gamma_row_vector(be, rm.gamma, &vec));
+      if (!vec) return CG_OK;
+    }
+    TRY(realize(be, rm.x));
+    if (rm.x->stype != ST_F32 || !is_contiguous(rm.x) || (uintptr_t)data_ptr(rm.x) % 16) return CG_OK;
+    a0 = retain(rm.x);
+    if (rm.gamma) a1 = retain(rm.gamma);
+  } else {
+    TRY(contiguous(be, gate, &a0));
+    int st = contiguous(be, up, &a1);
+    if (st) {
+      node_release(a0);
+      return st;
+    }
+    if (a0->stype != ST_F32 || a1->stype != ST_F32 || (uintptr_t)data_ptr(a0) % 16 || (uintptr_t)data_ptr(a1) % 16) {
+      node_release(a0);
+      node_release(a1);
+      return CG_OK;
+    }
+  }
+  d.pro = pro;
+  d.a = (const float *)data_ptr(a0);
+  d.aux = a1 ? (const float *)data_ptr(a1) : nullptr;
+  d.n_as_float = rm.n_as_float;
+  d.eps = rm.eps;
+  d.gamma_offset = rm.gamma_offset;
+  d.m.K = (uint32_t)K;
+  d.m.b_stype = b_stype;
+  double bytes = (double)K * 8, flops = 0;
+  int st = CG_OK;
+  for (cg_tensor *c : members) {
+    cg_tensor *w = c->in[1];
+    st = alloc_result(be, c, ST_F32);
+    if (st) break;
+    auto &pr = d.m.p[d.m.n_prob++];
+    pr.b = data_ptr(w);
+    pr.c = (float *)c->st->ptr;
+    pr.c_add = (c == n && addend) ? (const float *)data_ptr(addend) : nullptr;
+    pr.sbn = w->strides[w->rank - 1];
+    pr.N = (uint32_t)w->shape[w->rank - 1];
+    bytes += (double)pr.N * K * esize(w->stype) + (double)pr.N * 4;
+    flops += 2.0 * pr.N * K;
+  }
+  if (!st) {
+    const char *base = b_stype == ST_BF16 ? "gemv_rowdot_bf16" : "gemv_rowdot_f32";
+    KernelScope ks(be, base, bytes, flops);
+    if (be->trace_shapes) {
+      char buf[96];
+      snprintf(buf, sizeof buf, "%s[%s%d,K%lld,N%.0f]", base, pro == PRO_RMSNORM ? "rmsnorm+multi" : "glu+multi",
+               d.m.n_prob, (long long)K, flops / (2.0 * K));
+      ks.rename(buf);
+    }
+    hipError_t e = launch_gemv_pro(be->lc(), d);
+    if (e != hipSuccess) st = fail(be, CG_ERR_DEVICE, hipGetErrorString(e));
+  }
+  node_release(a0);
+  node_release(a1);
+  if (st) return st;
+  if (addend) *added = true;
+  for (cg_tensor *c : members) {
+    forget_gemv_candidate(c);
+    c->op = N_REAL;
+    drop_inputs(c);
+  }
+  *done = true;
+  return CG_OK;
+}
+
 // `addend` (optional; realised, f32, contiguous, shaped like n) is added in the epilogue when a
 // one-row kernel runs the product; *added tells the caller whether that happened.
 int realize_matmul(cg_backend *be, cg_tensor *n, cg_tensor *addend = nullptr, bool *added = nullptr) {
   if (!addend && n->dtype == CG_F32 && n->rank == 4 && n->shape[2] == 1 && !(be->flags & CG_FLAG_NO_PATTERNS)) {
     bool done = false;
     TRY(try_attn_decode(be, n, &done));
+    if (done) return CG_OK;
+  }
+  if (n->dtype == CG_F32 && n->gemv_candidate && !(be->flags & CG_FLAG_NO_PATTERNS)) {
+    bool done = false;
+    TRY(try_gemv_prologue(be, n, addend, added, &done));
     if (done) return CG_OK;
   }
   MatOperand A, B;

@@ -197,3 +197,70 @@ def test_attention_decode(oracle, hip, hip_nopat, cfg):
     assert np.allclose(ref, expect, rtol=1e-4, atol=1e-5)
     assert np.allclose(got[0], ref, rtol=1e-4, atol=1e-5), np.abs(got[0] - ref).max()
     assert np.allclose(gen[0], ref, rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize("K", [2048, 256, 1152])
+@pytest.mark.parametrize("variant", ["llama", "gemma", "extra_consumer"])
+def test_rmsnorm_in_projection_prologue(oracle, hip, hip_bf16, hip_nopat, K, variant):
+    """rmsnorm(x) feeding q/k/v-style one-row projections: the norm runs inside the product launch
+    (no rmsnorm launch) unless something else also reads the normed row."""
+    g = np.random.default_rng(K)
+    x = (g.standard_normal((1, 1, K)) * 2).astype(np.float32)
+    p = {"n.weight": g.standard_normal(K).astype(np.float32)}
+    outs = [K, 512, 264]
+    for i, o in enumerate(outs):
+        p[f"l{i}.weight"] = (g.standard_normal((o, K)) * 0.05).astype(np.float32)
+
+    def f(b, xv):
+        xv = xv + xv - xv
+        if variant == "gemma":
+            gm = lang.param(b, lang.path(["n", "weight"]))
+            raw = helpers.rmsnorm_raw(b, 1e-6, xv)
+            gm = lang.broadcast(b, gm, lang.shape(b, raw))
+            h = raw * (lang.constant(b, 1.0, lang.shape(b, gm)) + gm)
+        else:
+            h = helpers.rmsnorm(b, 1e-5, lang.path(["n"]), xv)
+        ys = [nn.linear_no_bias(b, K, o, lang.path([f"l{i}"]), h) for i, o in enumerate(outs)]
+        if variant == "extra_consumer":
+            ys.append(h + h)
+        return ys
+    n_out = len(outs) + (variant == "extra_consumer")
+    ref = vectors.run(oracle, f, n_out, x, params=p)
+    got, names = run_traced(hip, f, n_out, x, params=p)
+    gen = vectors.run(hip_nopat, f, n_out, x, params=p)
+    if variant == "extra_consumer":
+        assert "rmsnorm_fused" in names
+    else:
+        assert "rmsnorm_fused" not in names and "gemv_rowdot_f32" in names, sorted(names)
+    for r, a, c in zip(ref, got, gen):
+        assert np.allclose(a, r, rtol=1e-4, atol=1e-5), np.abs(a - r).max()
+        assert np.allclose(c, r, rtol=1e-4, atol=1e-5)
+    p16 = {k: (vectors.bf16_round(v) if v.ndim >= 2 else v) for k, v in p.items()}
+    ref16 = vectors.run(oracle, f, n_out, x, params=p16)
+    got16, names16 = run_traced(hip_bf16, f, n_out, x, params=p)
+    if variant != "extra_consumer":
+        assert "rmsnorm_fused" not in names16 and "gemv_rowdot_bf16" in names16, sorted(names16)
+    for r, a in zip(ref16, got16):
+        assert np.max(np.abs(a - r)) <= 2e-2 * np.abs(r).max()
+
+
+@pytest.mark.parametrize("K,N", [(8192, 2048), (512, 96), (6912, 1152)])
+@pytest.mark.parametrize("act", ["silu", "gelu"])
+def test_glu_in_projection_prologue(oracle, hip, hip_nopat, K, N, act):
+    """down_proj(silu(gate) * up) + residual as one launch."""
+    g = np.random.default_rng(K + N)
+    gate = g.standard_normal((1, 1, K)).astype(np.float32)
+    up = g.standard_normal((1, 1, K)).astype(np.float32)
+    res = g.standard_normal((1, 1, N)).astype(np.float32)
+    p = {"d.weight": (g.standard_normal((N, K)) * 0.02).astype(np.float32)}
+
+    def f(b, gv, uv, rv):
+        gv, uv = gv + gv - gv, uv + uv - uv
+        h = (nn.silu(b, gv) if act == "silu" else nn.gelu(b, gv)) * uv
+        return nn.linear_no_bias(b, K, N, lang.path(["d"]), h) + rv
+    (ref,) = vectors.run(oracle, f, 1, gate, up, res, params=p)
+    got, names = run_traced(hip, f, 1, gate, up, res, params=p)
+    (gen,) = vectors.run(hip_nopat, f, 1, gate, up, res, params=p)
+    assert not ({"swiglu_fused", "geglu_fused", "binary_f32"} & names), sorted(names)
+    assert np.allclose(got[0], ref, rtol=1e-4, atol=1e-5), np.abs(got[0] - ref).max()
+    assert np.allclose(gen, ref, rtol=1e-4, atol=1e-5)

@@ -167,3 +167,9 @@ def check_nn_vectors(be):
     fmin = np.finfo(np.float32).min
     assert m.shape == (3, 3)
     assert np.array_equal(m.ravel(), f32(g["pattern"]) * fmin)       # 0 * MIN = -0.0 == 0
+
+
+def bf16_round(a):
+    """f32 array rounded to the nearest bf16 (ties to even), as f32."""
+    u = np.ascontiguousarray(a, np.float32).view(np.uint32).astype(np.uint64)
+    return (((u + 0x7FFF + ((u >> 16) & 1)) >> 16) << 16).astype(np.uint32).view(np.float32)
