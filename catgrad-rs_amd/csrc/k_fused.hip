@@ -154,7 +154,18 @@ __global__ void __launch_bounds__(512) attn_decode_kernel(AttnDecodeDesc a) {
   const float *V = a.v + (int64_t)b * a.v_sb + (int64_t)kv * a.v_skv + (int64_t)rp * a.v_srep;
   const bool live = (uint32_t)sub * 4 < a.d;
   float4 qv = make_float4(0.f, 0.f, 0.f, 0.f);
-  if (live) qv = *(const float4 *)(q + sub * 4);
+  if (live) {
+    qv = *(const float4 *)(q + sub * 4);
+    if (a.q_cos) {  // apply_rope_embedding on the fly, same arithmetic as rope_kernel
+      const uint32_t j = sub * 4, half = a.d / 2;
+      const bool lo = j < half;
+      float4 pv = *(const float4 *)(q + (lo ? j + half : j - half));
+      if (lo) { pv.x = -pv.x; pv.y = -pv.y; pv.z = -pv.z; pv.w = -pv.w; }
+      const float4 c = *(const float4 *)(a.q_cos + j), sn = *(const float4 *)(a.q_sin + j);
+      qv.x = c.x * qv.x + sn.x * pv.x; qv.y = c.y * qv.y + sn.y * pv.y;
+      qv.z = c.z * qv.z + sn.z * pv.z; qv.w = c.w * qv.w + sn.w * pv.w;
+    }
+  }
   const uint32_t first = wave * KPW + kg;
   // phase 1: scores and their maximum
   float mx = -3.40282347e+38f;
@@ -249,7 +260,7 @@ __global__ void __launch_bounds__(256) rope_kernel(RopeDesc d) {
     float4 o;
     o.x = c.x * xv.x + sn.x * pv.x; o.y = c.y * xv.y + sn.y * pv.y;
     o.z = c.z * xv.z + sn.z * pv.z; o.w = c.w * xv.w + sn.w * pv.w;
-    *(float4 *)(d.out + i * 4) = o;
+    *(float4 *)(d.out + (int64_t)b * d.o_sb + (int64_t)h * d.o_sh + (int64_t)s * d.o_ss + j) = o;
   }
 }
 

@@ -84,8 +84,9 @@ hipError_t launch_softmax(const LaunchCtx &lc, const SoftmaxDesc &d);
 
 struct RopeDesc {
   const float *x, *cos, *sin;
-  float *out;            // contiguous [b, h, s, dim]
+  float *out;            // [b, h, s, dim] through o_sb / o_sh / o_ss (e.g. a slot of the KV cache)
   int64_t x_sb, x_sh, x_ss, cs_ss;  // element strides (unit stride along dim everywhere)
+  int64_t o_sb, o_sh, o_ss;
   uint32_t b, h, s, dim, half;
 };
 hipError_t launch_rope(const LaunchCtx &lc, const RopeDesc &d);
@@ -109,6 +110,9 @@ struct AttnDecodeDesc {
   uint32_t b, heads, rep, t, d;
   int32_t has_scale, has_mask_const;
   float scale, mask_const;
+  // optional: q is the projection before apply_rope_embedding; the kernel rotates it with this
+  // position's cos / sin rows (d floats each, half-split) as it loads it
+  const float *q_cos, *q_sin;
 };
 enum { ATTN_DECODE_MAX_T = 8192, ATTN_DECODE_MAX_D = 256 };
 hipError_t launch_attn_decode(const LaunchCtx &lc, const AttnDecodeDesc &d);

@@ -1011,17 +1011,22 @@ int try_rmsnorm(cg_backend *be, cg_tensor *root, bool *done) {
 }
 
 // apply_rope_embedding (catgrad-llm/src/helpers.rs:195-221): cos * x + sin * rotate_half(x)
-int try_rope(cg_backend *be, cg_tensor *root, bool *done) {
-  if (root->dtype != CG_F32 || root->rank != 4 || !is_bin(root, E_ADD_F)) return CG_OK;
+struct RopeMatch {
+  cg_tensor *cb = nullptr, *sb = nullptr, *x = nullptr;  // cos / sin broadcasts, the rotated tensor
+};
+
+// pure matching; nothing is realised
+bool match_rope(cg_tensor *root, RopeMatch *m) {
+  if (root->dtype != CG_F32 || root->rank != 4 || !is_bin(root, E_ADD_F)) return false;
   cg_tensor *m1 = root->in[0], *m2 = root->in[1];
-  if (!is_bin(m1, E_MUL_F) || !is_bin(m2, E_MUL_F) || refs(m1) != 1 || refs(m2) != 1) return CG_OK;
+  if (!is_bin(m1, E_MUL_F) || !is_bin(m2, E_MUL_F) || refs(m1) != 1 || refs(m2) != 1) return false;
   cg_tensor *cb = m1->in[0], *x = m1->in[1], *sb = m2->in[0], *rot = m2->in[1];
-  if (rot->op != N_CONCAT || rot->p0 != 3 || refs(rot) != 1) return CG_OK;
+  if (rot->op != N_CONCAT || rot->p0 != 3 || refs(rot) != 1) return false;
   cg_tensor *ng = rot->in[0], *lo = rot->in[1];
-  if (!is_un(ng, E_NEG_F) || refs(ng) != 1) return CG_OK;
+  if (!is_un(ng, E_NEG_F) || refs(ng) != 1) return false;
   cg_tensor *hi = ng->in[0];
   const int64_t dim = root->shape[3], half = dim / 2;
-  if (dim % 8 || hi->shape[3] != half || lo->shape[3] != half) return CG_OK;
+  if (dim % 8 || hi->shape[3] != half || lo->shape[3] != half) return false;
   // the two halves are slices of x along the last axis: still deferred, or (x already in
   // memory) views created on the spot
   auto half_of = [&](const cg_tensor *t, int64_t start) {
@@ -1031,18 +1036,36 @@ int try_rope(cg_backend *be, cg_tensor *root, bool *done) {
       if (t->strides[i] != x->strides[i] && t->shape[i] != 1) return false;
     return t->offset == x->offset + start * x->strides[3];
   };
-  if (!half_of(hi, half) || !half_of(lo, 0)) return CG_OK;
-  if (root->size() >= ((int64_t)1 << 31)) return CG_OK;
+  if (!half_of(hi, half) || !half_of(lo, 0)) return false;
+  if (root->size() >= ((int64_t)1 << 31)) return false;
+  m->cb = cb;
+  m->sb = sb;
+  m->x = x;
+  return true;
+}
 
-  TRY(realize(be, cb));
-  TRY(realize(be, sb));
-  TRY(realize(be, x));
+// realises the operands of a matched rope; *ok = the kernel's layout requirements hold
+int rope_operands(cg_backend *be, const RopeMatch &m, bool *ok) {
+  TRY(realize(be, m.cb));
+  TRY(realize(be, m.sb));
+  TRY(realize(be, m.x));
   auto table_ok = [&](const cg_tensor *t) {
     return t->stype == ST_F32 && t->strides[0] * (t->shape[0] != 1) == 0 &&
            t->strides[1] * (t->shape[1] != 1) == 0 && t->strides[3] == 1 && t->strides[2] % 4 == 0 &&
            (uintptr_t)data_ptr(t) % 16 == 0;
   };
-  if (!table_ok(cb) || !table_ok(sb) || cb->strides[2] != sb->strides[2]) return CG_OK;
+  *ok = table_ok(m.cb) && table_ok(m.sb) && m.cb->strides[2] == m.sb->strides[2];
+  return CG_OK;
+}
+
+// Launches the rope kernel for `root` (matched as m) into `out` with the given element strides.
+// *done = false: layout requirements not met, nothing was launched.
+int rope_into(cg_backend *be, cg_tensor *root, const RopeMatch &m, float *out, const int64_t *o_strides,
+              const char *name, bool *done) {
+  bool tables = false;
+  TRY(rope_operands(be, m, &tables));
+  if (!tables) return CG_OK;
+  cg_tensor *x = m.x, *cb = m.cb, *sb = m.sb;
   cg_tensor *xs = retain(x);
   bool ok = x->stype == ST_F32 && x->strides[3] == 1 && (uintptr_t)data_ptr(x) % 16 == 0;
   for (int i = 0; i < 3; ++i)
@@ -1052,29 +1075,52 @@ int try_rope(cg_backend *be, cg_tensor *root, bool *done) {
     xs = nullptr;
     TRY(materialize(be, x, &xs));
   }
-  int st = alloc_result(be, root, ST_F32);
-  if (!st) {
-    RopeDesc d;
-    std::memset(&d, 0, sizeof(d));
-    d.x = (const float *)data_ptr(xs);
-    d.cos = (const float *)data_ptr(cb);
-    d.sin = (const float *)data_ptr(sb);
-    d.out = (float *)root->st->ptr;
-    d.x_sb = xs->strides[0];
-    d.x_sh = xs->strides[1];
-    d.x_ss = xs->strides[2];
-    d.cs_ss = root->shape[2] == 1 ? 0 : cb->strides[2];
-    d.b = (uint32_t)root->shape[0];
-    d.h = (uint32_t)root->shape[1];
-    d.s = (uint32_t)root->shape[2];
-    d.dim = (uint32_t)dim;
-    d.half = (uint32_t)half;
-    KernelScope ks(be, "rope_fused", (double)root->size() * 8, 0);
+  const int64_t dim = root->shape[3];
+  RopeDesc d;
+  std::memset(&d, 0, sizeof(d));
+  d.x = (const float *)data_ptr(xs);
+  d.cos = (const float *)data_ptr(cb);
+  d.sin = (const float *)data_ptr(sb);
+  d.out = out;
+  d.x_sb = xs->strides[0];
+  d.x_sh = xs->strides[1];
+  d.x_ss = xs->strides[2];
+  d.o_sb = o_strides[0];
+  d.o_sh = o_strides[1];
+  d.o_ss = o_strides[2];
+  d.cs_ss = root->shape[2] == 1 ? 0 : cb->strides[2];
+  d.b = (uint32_t)root->shape[0];
+  d.h = (uint32_t)root->shape[1];
+  d.s = (uint32_t)root->shape[2];
+  d.dim = (uint32_t)dim;
+  d.half = (uint32_t)(dim / 2);
+  int st = CG_OK;
+  {
+    KernelScope ks(be, name, (double)root->size() * 8, 0);
     hipError_t e = launch_rope(be->lc(), d);
     if (e != hipSuccess) st = fail(be, CG_ERR_DEVICE, hipGetErrorString(e));
   }
   node_release(xs);
   if (st) return st;
+  *done = true;
+  return CG_OK;
+}
+
+// apply_rope_embedding (catgrad-llm/src/helpers.rs:195-221): cos * x + sin * rotate_half(x)
+int try_rope(cg_backend *be, cg_tensor *root, bool *done) {
+  RopeMatch m;
+  if (!match_rope(root, &m)) return CG_OK;
+  bool tables = false;
+  TRY(rope_operands(be, m, &tables));
+  if (!tables) return CG_OK;
+  TRY(alloc_result(be, root, ST_F32));
+  bool launched = false;
+  int st = rope_into(be, root, m, (float *)root->st->ptr, root->strides, "rope_fused", &launched);
+  if (st || !launched) {
+    storage_release(root->st);
+    root->st = nullptr;
+    return st;
+  }
   finish_fused(root);
   *done = true;
   return CG_OK;
@@ -1551,6 +1597,20 @@ int try_attn_decode(cg_backend *be, cg_tensor *n, bool *done) {
   if (!pk) TRY(unpeeled(S->in[1], &Kop));
   if (!pv) TRY(unpeeled(n->in[1], &Vop));
   cg_tensor *q = S->in[0];
+  // q straight from apply_rope_embedding and read by nobody else: rotate it inside the kernel
+  RopeMatch qrope;
+  const float *q_cos = nullptr, *q_sin = nullptr;
+  if (q->op != N_REAL && refs(q) == 1 && match_rope(q, &qrope)) {
+    bool tables = false;
+    TRY(rope_operands(be, qrope, &tables));
+    cg_tensor *qx = qrope.x;
+    if (tables && qx->stype == ST_F32 && qx->strides[3] == 1 && (uintptr_t)data_ptr(qx) % 16 == 0 &&
+        qx->strides[0] % 4 == 0 && qx->strides[1] % 4 == 0) {
+      q_cos = (const float *)data_ptr(qrope.cb);
+      q_sin = (const float *)data_ptr(qrope.sb);
+      q = qx;
+    }
+  }
   TRY(realize(be, q));
   auto rows_ok = [](const void *ptr, int64_t unit, std::initializer_list<int64_t> strides) {
     if (unit != 1 || (uintptr_t)ptr % 16) return false;
@@ -1585,6 +1645,8 @@ int try_attn_decode(cg_backend *be, cg_tensor *n, bool *done) {
   a.scale = m.scale;
   a.has_mask_const = m.has_mask_const;
   a.mask_const = m.mask_const;
+  a.q_cos = q_cos;
+  a.q_sin = q_sin;
   {
     const double kv_bytes = 2.0 * nb * Kop.shape[1] * T * d * 4;
     KernelScope ks(be, "attn_decode", kv_bytes + 2.0 * nb * heads * d * 4, 4.0 * nb * heads * T * d);
@@ -1958,13 +2020,18 @@ int realize_matmul(cg_backend *be, cg_tensor *n, cg_tensor *addend = nullptr, bo
 int realize_concat(cg_backend *be, cg_tensor *n) {
   cg_tensor *x = n->in[0], *y = n->in[1];
   TRY(realize(be, x));
-  TRY(realize(be, y));
   const int dim = (int)n->p0;
   const int64_t xd = x->shape[dim], yd = y->shape[dim];
   const int plain = n->dtype == CG_F32 ? ST_F32 : ST_U32;
+  const bool in_place = xd > 0 && yd > 0 && refs(x) == 1 && x->st->rc.load() == 1 && x->st->grow_dim == dim &&
+                        xd + yd <= x->st->grow_cap && x->offset == 0 && x->stype == plain;
+  // the new key rows arrive through apply_rope_embedding: rotate them straight into the cache slot
+  RopeMatch rope;
+  const bool rope_y = in_place && !(be->flags & CG_FLAG_NO_PATTERNS) && y->op != N_REAL && refs(y) == 1 &&
+                      n->rank == 4 && dim == 2 && match_rope(y, &rope);
+  if (!rope_y) TRY(realize(be, y));
   // (1) append in place
-  if (xd > 0 && yd > 0 && refs(x) == 1 && x->st->rc.load() == 1 && x->st->grow_dim == dim &&
-      xd + yd <= x->st->grow_cap && x->offset == 0 && x->stype == plain) {
+  if (in_place) {
     n->st = x->st;
     n->st->rc.fetch_add(1);
     storage_release(n->st->shadow);  // contents change: any bf16 twin is stale
@@ -1973,7 +2040,12 @@ int realize_concat(cg_backend *be, cg_tensor *n) {
     n->offset = 0;
     std::memcpy(n->strides, x->strides, sizeof(n->strides));
     char *dst = (char *)n->st->ptr + xd * n->strides[dim] * 4;
-    TRY(run_ew(be, y, true, dst, n->strides, plain, "kv_append"));
+    bool roped = false;
+    if (rope_y) {
+      TRY(rope_into(be, y, rope, (float *)dst, n->strides, "rope_kv_append", &roped));
+      if (!roped) TRY(realize(be, y));
+    }
+    if (!roped) TRY(run_ew(be, y, true, dst, n->strides, plain, "kv_append"));
     n->op = N_REAL;
     drop_inputs(n);
     return CG_OK;
