@@ -21,6 +21,11 @@ sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per launch of the decode GEMV kernels at the default workload (bf16, 16 layers), from two
+# rocprofv3 --pmc runs of this file (FETCH_SIZE, WRITE_SIZE), each scaled by what the same counter
+# read for the 1 GiB peak_copy_kernel in the same run (x2.000 and x1.000); a profiler cannot run
+# inside this process, so the figure is carried here and reported only for that workload
+PMC_TRAFFIC_BYTES_PER_LAUNCH = {("bf16", 16, "gemv_rowdot_bf16"): 38382778.0}
 MFMA_PEAK_TFLOPS = {"bf16": 2500.0, "f32": 157.3}
 
 
@@ -155,6 +160,11 @@ def main():
         "setup_s": setup_s,
     }
 
+    # ---- what this device gives the simplest code (denominators next to the data-sheet peaks) ----
+    out["measured_peaks"] = {"copy_gbs_read_plus_write": be.peak_copy_gbs(1 << 30, 10),
+                             "mfma_bf16_tflops": be.peak_mfma_tflops(cg.abi.U32, 20000),
+                             "mfma_f32_tflops": be.peak_mfma_tflops(cg.abi.F32, 20000)}
+
     if not args.profile_only:
         # ---- traced pass: per-kernel durations from events on the backend's own stream ---------
         be.trace(True)
@@ -169,7 +179,8 @@ def main():
             r = rep[gemv]
             achieved = r["bytes"] / (r["ms"] * 1e-3) / 1e9
             out["roofline"] = {"bound": "hbm", "kernel": gemv, "achieved": achieved, "peak": HBM_PEAK_GBS,
-                               "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                               "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
+                               "traffic": PMC_TRAFFIC_BYTES_PER_LAUNCH.get((args.dtype, args.layers, gemv)),
                                "launches_per_step": r["launches"] / n_tr,
                                "avg_us": r["ms"] * 1e3 / r["launches"],
                                "algorithmic_bytes_per_launch": r["bytes"] / r["launches"]}

@@ -64,6 +64,8 @@ _SIGNATURES = {
     "cg_sync": (C.c_int, [_P]),
     "cg_tensor_realize": (C.c_int, [_P, _P]),
     "cg_tensor_prefetch": (C.c_int, [_P, _P]),
+    "cg_peak_copy_gbs": (C.c_int, [_P, _SZ, C.c_int, C.POINTER(C.c_double)]),
+    "cg_peak_mfma_tflops": (C.c_int, [_P, C.c_int, C.c_int, C.POINTER(C.c_double)]),
     "cg_backend_name": (C.c_char_p, [_P]),
     "cg_tensor_retain": (_P, [_P]),
     "cg_tensor_release": (None, [_P]),
@@ -205,6 +207,16 @@ class Backend:
 
     def sync(self):
         self._check(self.lib.cg_sync(self.ptr))
+
+    def peak_copy_gbs(self, nbytes=1 << 30, iters=10):
+        out = C.c_double()
+        self._check(self.lib.cg_peak_copy_gbs(self.ptr, nbytes, iters, C.byref(out)))
+        return out.value
+
+    def peak_mfma_tflops(self, operand=None, iters=20000):
+        out = C.c_double()
+        self._check(self.lib.cg_peak_mfma_tflops(self.ptr, U32 if operand is None else operand, iters, C.byref(out)))
+        return out.value
 
     def prefetch(self, x):
         """Realize and start an asynchronous copy of a small tensor to the host; `to_vec(x)` then

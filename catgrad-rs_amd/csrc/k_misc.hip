@@ -165,4 +165,51 @@ hipError_t launch_fill_u32(const LaunchCtx &lc, uint32_t *dst, uint32_t value, u
   return hipGetLastError();
 }
 
+// ---- peak probes --------------------------------------------------------------------------------------
+// What the machine gives to the simplest possible code, as denominators next to the data-sheet
+// numbers: a grid-stride 16-byte copy (HBM read + write) and a register-resident MFMA issue loop.
+__global__ void __launch_bounds__(256) peak_copy_kernel(const uint4 *in, uint4 *out, uint64_t n) {
+  for (uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (uint64_t)gridDim.x * 256)
+    out[i] = in[i];
+}
+
+hipError_t launch_peak_copy(const LaunchCtx &lc, const void *in, void *out, uint64_t bytes) {
+  CG_LAUNCH(lc, (peak_copy_kernel), (unsigned)lc.n_cus * 8, 256, (const uint4 *)in, (uint4 *)out, bytes / 16);
+  return hipGetLastError();
+}
+
+typedef __attribute__((ext_vector_type(8))) __bf16 pk_bf16x8;
+typedef __attribute__((ext_vector_type(16))) float pk_f32x16;
+
+template <bool BF16>
+__global__ void __launch_bounds__(256) peak_mfma_kernel(float *out, int iters) {
+  pk_f32x16 acc[4];
+  for (int i = 0; i < 4; ++i)
+    for (int e = 0; e < 16; ++e) acc[i][e] = 0.f;
+  pk_bf16x8 a, b;
+  for (int e = 0; e < 8; ++e) {
+    a[e] = (__bf16)(float)((threadIdx.x + e) & 3);
+    b[e] = (__bf16)(float)(e & 1);
+  }
+  const float fa = (float)(threadIdx.x & 3), fb = 1.0f;
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if (BF16) acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc[i], 0, 0, 0);
+      else acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa, fb, acc[i], 0, 0, 0);
+    }
+  }
+  float s = 0.f;
+  for (int i = 0; i < 4; ++i)
+    for (int e = 0; e < 16; ++e) s += acc[i][e];
+  out[(uint64_t)blockIdx.x * 256 + threadIdx.x] = s;
+}
+
+// flops issued: grid * 4 waves * iters * 4 MFMAs * (2 * 32 * 32 * k), k = 16 (bf16) or 2 (f32)
+hipError_t launch_peak_mfma(const LaunchCtx &lc, int bf16, float *out, unsigned grid, int iters) {
+  if (bf16) CG_LAUNCH(lc, (peak_mfma_kernel<true>), grid, 256, out, iters);
+  else CG_LAUNCH(lc, (peak_mfma_kernel<false>), grid, 256, out, iters);
+  return hipGetLastError();
+}
+
 }  // namespace cgk

@@ -59,6 +59,9 @@ hipError_t launch_topk(const LaunchCtx &lc, const float *x, float *values, uint3
 hipError_t launch_compare(const LaunchCtx &lc, const void *a, const void *b, uint64_t n,
                           int is_f32, uint32_t *flag);
 hipError_t launch_fill_u32(const LaunchCtx &lc, uint32_t *dst, uint32_t value, uint64_t n);
+// peak probes: plain 16-byte copy; MFMA issue loop (out: grid * 256 floats)
+hipError_t launch_peak_copy(const LaunchCtx &lc, const void *in, void *out, uint64_t bytes);
+hipError_t launch_peak_mfma(const LaunchCtx &lc, int bf16, float *out, unsigned grid, int iters);
 
 // ---- k_fused.hip
 struct RmsNormDesc {

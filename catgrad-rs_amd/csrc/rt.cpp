@@ -2771,6 +2771,68 @@ int cg_arange(cg_backend *be, size_t end, cg_tensor **out) {
 int cg_to_f32(cg_backend *be, cg_tensor *x, float *dst, size_t n) { return download(be, x, dst, n, CG_F32); }
 int cg_to_u32(cg_backend *be, cg_tensor *x, uint32_t *dst, size_t n) { return download(be, x, dst, n, CG_U32); }
 
+// ---- peak probes (measured denominators; nothing in the product depends on them) ------------------
+int cg_peak_copy_gbs(cg_backend *be, size_t bytes, int iters, double *gbs) {
+  if (!be || !gbs || bytes < 4096 || iters < 1) return CG_ERR_ARG;
+  HIPCHK(be, hipSetDevice(be->device));
+  bytes &= ~(size_t)4095;
+  Storage *a = nullptr, *b = nullptr;
+  TRY(dev_alloc(be, bytes, &a));
+  int st = dev_alloc(be, bytes, &b);
+  if (st) {
+    storage_release(a);
+    return st;
+  }
+  hipEvent_t e0 = nullptr, e1 = nullptr;
+  hipError_t e = hipEventCreate(&e0);
+  if (e == hipSuccess) e = hipEventCreate(&e1);
+  LaunchCtx lc = be->lc();
+  lc.ev_start = lc.ev_stop = nullptr;
+  if (e == hipSuccess) e = launch_fill_u32(lc, (uint32_t *)a->ptr, 0x3F800000u, bytes / 4);
+  if (e == hipSuccess) e = launch_peak_copy(lc, a->ptr, b->ptr, bytes);  // warm-up
+  if (e == hipSuccess) e = hipEventRecord(e0, be->stream);
+  for (int i = 0; i < iters && e == hipSuccess; ++i) e = launch_peak_copy(lc, a->ptr, b->ptr, bytes);
+  if (e == hipSuccess) e = hipEventRecord(e1, be->stream);
+  if (e == hipSuccess) e = hipStreamSynchronize(be->stream);
+  float ms = 0.f;
+  if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
+  if (e0) (void)hipEventDestroy(e0);
+  if (e1) (void)hipEventDestroy(e1);
+  storage_release(a);
+  storage_release(b);
+  if (e != hipSuccess) return fail(be, CG_ERR_DEVICE, hipGetErrorString(e));
+  *gbs = 2.0 * (double)bytes * iters / (ms * 1e-3) / 1e9;  // read + write
+  return CG_OK;
+}
+
+int cg_peak_mfma_tflops(cg_backend *be, cg_dtype operand, int iters, double *tflops) {
+  if (!be || !tflops || iters < 1) return CG_ERR_ARG;
+  HIPCHK(be, hipSetDevice(be->device));
+  const int bf16 = operand != CG_F32;  // CG_F32: v_mfma_f32_32x32x2_f32; otherwise bf16 32x32x16
+  const unsigned grid = (unsigned)be->n_cus * 8;
+  Storage *o = nullptr;
+  TRY(dev_alloc(be, (size_t)grid * 256 * 4, &o));
+  hipEvent_t e0 = nullptr, e1 = nullptr;
+  hipError_t e = hipEventCreate(&e0);
+  if (e == hipSuccess) e = hipEventCreate(&e1);
+  LaunchCtx lc = be->lc();
+  lc.ev_start = lc.ev_stop = nullptr;
+  if (e == hipSuccess) e = launch_peak_mfma(lc, bf16, (float *)o->ptr, grid, 64);
+  if (e == hipSuccess) e = hipEventRecord(e0, be->stream);
+  if (e == hipSuccess) e = launch_peak_mfma(lc, bf16, (float *)o->ptr, grid, iters);
+  if (e == hipSuccess) e = hipEventRecord(e1, be->stream);
+  if (e == hipSuccess) e = hipStreamSynchronize(be->stream);
+  float ms = 0.f;
+  if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
+  if (e0) (void)hipEventDestroy(e0);
+  if (e1) (void)hipEventDestroy(e1);
+  storage_release(o);
+  if (e != hipSuccess) return fail(be, CG_ERR_DEVICE, hipGetErrorString(e));
+  const double k = bf16 ? 16.0 : 2.0;
+  *tflops = (double)grid * 4 * iters * 4 * (2.0 * 32 * 32 * k) / (ms * 1e-3) / 1e12;
+  return CG_OK;
+}
+
 int cg_trace_enable(cg_backend *be, int on) {
   if (!be) return CG_ERR_ARG;
   trace_collect(be);

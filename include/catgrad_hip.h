@@ -152,6 +152,12 @@ int cg_to_u32(cg_backend *be, cg_tensor *x, uint32_t *dst, size_t n);
  * on = 2 additionally keys matmul records by problem shape ("gemm_mfma_bf16[b1,512x2048x2048,s4]").
  */
 int cg_trace_enable(cg_backend *be, int on);
+/* Peak probes (no counterpart in the reference): what this device gives a plain 16-byte grid-stride
+ * copy of `bytes` (GB/s, read + write counted) and a register-resident MFMA issue loop
+ * (operand CG_F32: v_mfma_f32_32x32x2_f32, otherwise bf16 v_mfma_f32_32x32x16_bf16; TFLOP/s).
+ * Benchmarks report them beside the data-sheet peaks. */
+int cg_peak_copy_gbs(cg_backend *be, size_t bytes, int iters, double *gbs);
+int cg_peak_mfma_tflops(cg_backend *be, cg_dtype operand, int iters, double *tflops);
 int cg_trace_reset(cg_backend *be);
 /* returns the number of bytes needed (including the NUL); writes at most cap bytes */
 size_t cg_trace_report(cg_backend *be, char *buf, size_t cap);

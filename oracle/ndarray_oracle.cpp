@@ -90,6 +90,9 @@ const char *cg_last_error(const cg_backend *be) { return be ? be->err.c_str() : 
 int cg_sync(cg_backend *) { return CG_OK; }
 int cg_tensor_realize(cg_backend *, cg_tensor *) { return CG_OK; }
 int cg_tensor_prefetch(cg_backend *, cg_tensor *) { return CG_OK; }
+// the probes measure a device; the oracle has none
+int cg_peak_copy_gbs(cg_backend *, size_t, int, double *) { return CG_ERR_DEVICE; }
+int cg_peak_mfma_tflops(cg_backend *, cg_dtype, int, double *) { return CG_ERR_DEVICE; }
 const char *cg_backend_name(const cg_backend *) { return "ndarray-oracle"; }
 
 cg_tensor *cg_tensor_retain(cg_tensor *t) {
