@@ -387,6 +387,92 @@ __device__ __forceinline__ Acc<KIND> shfl_xor_acc(const Acc<KIND> &a, int m) {
   return r;
 }
 
+// ---- reductions of a tensor that is already in memory ------------------------------------------------
+// No program to interpret: rows of n unit-stride elements (f32 / u32 words, or bf16 widened to f32)
+// streamed with 16-byte (8-byte for bf16) loads, four in flight per lane.  One row per workgroup
+// (WPR = 4) or per wavefront (WPR = 1).
+template <int KIND, typename T, int WPR>
+__global__ void __launch_bounds__(256) reduce_plain_kernel(const T *x, int64_t row_stride, uint32_t *out,
+                                                           uint32_t rows, uint32_t n) {
+  __shared__ uint32_t part[4][Acc<KIND>::W];
+  constexpr int U = 4;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const uint32_t row = WPR == 4 ? blockIdx.x : blockIdx.x * 4 + wave;
+  const uint32_t t_in_row = WPR == 4 ? threadIdx.x : lane, tpr = WPR * 64;
+  Acc<KIND> acc;
+  if (row < rows) {
+    const T *r = x + (int64_t)row * row_stride;
+    for (uint32_t c0 = t_in_row * 4; c0 < n; c0 += tpr * 4 * U) {
+      uint32_t v[U][4];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const uint32_t c = c0 + u * tpr * 4;
+        if (c < n) {
+          if (sizeof(T) == 4) {
+            const uint4 q = *(const uint4 *)(r + c);
+            v[u][0] = q.x; v[u][1] = q.y; v[u][2] = q.z; v[u][3] = q.w;
+          } else {
+            const uint2 q = *(const uint2 *)(r + c);
+            v[u][0] = q.x << 16; v[u][1] = q.x & 0xFFFF0000u; v[u][2] = q.y << 16; v[u][3] = q.y & 0xFFFF0000u;
+          }
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const uint32_t c = c0 + u * tpr * 4;
+        if (c < n) {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) acc.add(v[u][j], c + j);
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) acc.merge(shfl_xor_acc<KIND>(acc, m));
+  if (WPR == 4) {
+    if (lane == 0) acc.get(part[wave]);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      for (int w2 = 1; w2 < 4; ++w2) {
+        Acc<KIND> o;
+        o.set(part[w2]);
+        acc.merge(o);
+      }
+      out[row] = acc.result();
+    }
+  } else if (lane == 0 && row < rows) {
+    out[row] = acc.result();
+  }
+}
+
+template <int KIND>
+static void launch_reduce_plain_kind(const LaunchCtx &lc, const void *x, int bf16, int64_t row_stride, uint32_t *out,
+                                     uint32_t rows, uint32_t n) {
+  if (n >= 1024) {
+    if (bf16) CG_LAUNCH(lc, (reduce_plain_kernel<KIND, uint16_t, 4>), rows, 256, (const uint16_t *)x, row_stride, out, rows, n);
+    else CG_LAUNCH(lc, (reduce_plain_kernel<KIND, uint32_t, 4>), rows, 256, (const uint32_t *)x, row_stride, out, rows, n);
+  } else {
+    if (bf16) CG_LAUNCH(lc, (reduce_plain_kernel<KIND, uint16_t, 1>), (rows + 3) / 4, 256, (const uint16_t *)x, row_stride, out, rows, n);
+    else CG_LAUNCH(lc, (reduce_plain_kernel<KIND, uint32_t, 1>), (rows + 3) / 4, 256, (const uint32_t *)x, row_stride, out, rows, n);
+  }
+}
+
+hipError_t launch_reduce_plain(const LaunchCtx &lc, int kind, const void *x, int bf16, int64_t row_stride, void *out,
+                               uint32_t rows, uint32_t n) {
+  if (!rows) return hipSuccess;
+  uint32_t *o = (uint32_t *)out;
+  switch (kind) {
+    case R_SUM_F: launch_reduce_plain_kind<R_SUM_F>(lc, x, bf16, row_stride, o, rows, n); break;
+    case R_SUM_U: launch_reduce_plain_kind<R_SUM_U>(lc, x, bf16, row_stride, o, rows, n); break;
+    case R_MAX_F: launch_reduce_plain_kind<R_MAX_F>(lc, x, bf16, row_stride, o, rows, n); break;
+    case R_MAX_U: launch_reduce_plain_kind<R_MAX_U>(lc, x, bf16, row_stride, o, rows, n); break;
+    case R_ARGMAX_F: launch_reduce_plain_kind<R_ARGMAX_F>(lc, x, bf16, row_stride, o, rows, n); break;
+    case R_ARGMAX_U: launch_reduce_plain_kind<R_ARGMAX_U>(lc, x, bf16, row_stride, o, rows, n); break;
+    default: return hipErrorInvalidValue;
+  }
+  return hipGetLastError();
+}
+
 // One row per workgroup (WAVES_PER_ROW = 4) or per wavefront (WAVES_PER_ROW = 1).
 template <int KIND, int VEC, int WAVES_PER_ROW>
 __global__ void __launch_bounds__(256) reduce_kernel(const Program p, uint32_t *out, uint32_t rows,

@@ -119,9 +119,82 @@ __global__ void __launch_bounds__(BLOCK == 64 ? 256 : BLOCK) softmax_kernel(Soft
   }
 }
 
+// Same, 16 bytes per access (n % 4 == 0, rows and mask rows 16-byte aligned, unit mask column stride);
+// the row stays in registers between the passes: CH float4 chunks per thread.
+template <int BLOCK, int CH>
+__global__ void __launch_bounds__(BLOCK) softmax_vec_kernel(SoftmaxDesc d) {
+  __shared__ float lds[BLOCK / 64];
+  const uint32_t row = blockIdx.x, tid = threadIdx.x;
+  const float *x = d.x + (int64_t)row * d.x_row_stride;
+  float *y = d.y + (int64_t)row * d.n;
+  const float *mk = nullptr;
+  if (d.mask) {
+    const uint32_t r_in = row % d.mask_rows, grp = row / d.mask_rows;
+    mk = d.mask + (int64_t)grp * d.mask_group_stride + (int64_t)r_in * d.mask_row_stride;
+  }
+  float4 v[CH];
+  float mx = -3.40282347e+38f;
+#pragma unroll
+  for (int e = 0; e < CH; ++e) {
+    const uint32_t c = (tid + e * BLOCK) * 4;
+    if (c < d.n) v[e] = *(const float4 *)(x + c);
+  }
+#pragma unroll
+  for (int e = 0; e < CH; ++e) {
+    const uint32_t c = (tid + e * BLOCK) * 4;
+    if (c < d.n) {
+      float4 t = v[e];
+      if (d.has_scale) { t.x = t.x / d.scale; t.y = t.y / d.scale; t.z = t.z / d.scale; t.w = t.w / d.scale; }
+      if (mk) {
+        const float4 m = *(const float4 *)(mk + c);
+        t.x += m.x; t.y += m.y; t.z += m.z; t.w += m.w;
+      } else if (d.has_mask_const) {
+        t.x += d.mask_const; t.y += d.mask_const; t.z += d.mask_const; t.w += d.mask_const;
+      }
+      v[e] = t;
+      mx = fmaxf(fmaxf(mx, t.x), fmaxf(t.y, fmaxf(t.z, t.w)));
+    }
+  }
+  mx = block_reduce<BLOCK, true>(mx, lds);
+  float sum = 0.f;
+#pragma unroll
+  for (int e = 0; e < CH; ++e) {
+    const uint32_t c = (tid + e * BLOCK) * 4;
+    if (c < d.n) {
+      float4 t = v[e];
+      t.x = expf(t.x - mx); t.y = expf(t.y - mx); t.z = expf(t.z - mx); t.w = expf(t.w - mx);
+      v[e] = t;
+      sum += (t.x + t.y) + (t.z + t.w);
+    }
+  }
+  sum = block_reduce<BLOCK, false>(sum, lds);
+#pragma unroll
+  for (int e = 0; e < CH; ++e) {
+    const uint32_t c = (tid + e * BLOCK) * 4;
+    if (c < d.n) {
+      float4 t = v[e];
+      t.x = t.x / sum; t.y = t.y / sum; t.z = t.z / sum; t.w = t.w / sum;
+      *(float4 *)(y + c) = t;
+    }
+  }
+}
+
 hipError_t launch_softmax(const LaunchCtx &lc, const SoftmaxDesc &d) {
   if (!d.rows || !d.n) return hipSuccess;
   // n <= 16384 checked by the caller
+  const bool vec = d.n % 4 == 0 && d.n >= 256 && (uintptr_t)d.x % 16 == 0 && d.x_row_stride % 4 == 0 &&
+                   (uintptr_t)d.y % 16 == 0 &&
+                   (!d.mask || (d.mask_col_stride == 1 && (uintptr_t)d.mask % 16 == 0 && d.mask_row_stride % 4 == 0 &&
+                                d.mask_group_stride % 4 == 0));
+  if (vec) {
+    if (d.n <= 512) CG_LAUNCH(lc, (softmax_vec_kernel<64, 2>), d.rows, 64, d);
+    else if (d.n <= 1024) CG_LAUNCH(lc, (softmax_vec_kernel<256, 1>), d.rows, 256, d);
+    else if (d.n <= 2048) CG_LAUNCH(lc, (softmax_vec_kernel<256, 2>), d.rows, 256, d);
+    else if (d.n <= 4096) CG_LAUNCH(lc, (softmax_vec_kernel<256, 4>), d.rows, 256, d);
+    else if (d.n <= 8192) CG_LAUNCH(lc, (softmax_vec_kernel<512, 4>), d.rows, 512, d);
+    else CG_LAUNCH(lc, (softmax_vec_kernel<1024, 4>), d.rows, 1024, d);
+    return hipGetLastError();
+  }
   if (d.n <= 64) CG_LAUNCH(lc, (softmax_kernel<64, 1>), (d.rows + 3) / 4, dim3(64, 4), d);
   else if (d.n <= 256) CG_LAUNCH(lc, (softmax_kernel<64, 4>), (d.rows + 3) / 4, dim3(64, 4), d);
   else if (d.n <= 512) CG_LAUNCH(lc, (softmax_kernel<64, 8>), (d.rows + 3) / 4, dim3(64, 4), d);

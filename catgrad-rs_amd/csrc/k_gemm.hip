@@ -541,6 +541,77 @@ __global__ void __launch_bounds__(256) cast_bf16_kernel(const float *in, uint16_
   }
 }
 
+// B[k, n] with unit stride along n (f32 or bf16)  ->  bf16 [batch][n][k], k-contiguous: the layout
+// the direct-to-LDS GEMM wants.  64 x 64 tiles through LDS: reads run along n, writes along k.
+template <typename TB, bool VEC>
+__global__ void __launch_bounds__(256) transpose_cast_bf16_kernel(const TB *b, uint16_t *out, uint32_t K,
+                                                                  uint32_t N, int64_t sbk, uint32_t nb1,
+                                                                  int64_t sb_b0, int64_t sb_b1) {
+  __shared__ __attribute__((aligned(8))) uint16_t tile[64][68];  // pitch 136 bytes keeps 8-byte alignment
+  const uint32_t bz = blockIdx.z, b0 = bz / nb1, b1 = bz - b0 * nb1;
+  const TB *src = b + b0 * sb_b0 + b1 * sb_b1;
+  uint16_t *dst = out + (uint64_t)bz * N * K;
+  const uint32_t n0 = blockIdx.x * 64, k0 = blockIdx.y * 64;
+  const int r = threadIdx.x >> 4, c4 = (threadIdx.x & 15) * 4;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const uint32_t k = k0 + r + i * 16, n = n0 + c4;
+    uint16_t v[4] = {0, 0, 0, 0};
+    if (VEC) {  // N % 4 == 0, 4-element groups aligned: all four in range or none
+      if (k < K && n < N) {
+        if (sizeof(TB) == 4) {
+          const float4 q = *(const float4 *)((const float *)src + (int64_t)k * sbk + n);
+          v[0] = (uint16_t)bf16_rne(q.x); v[1] = (uint16_t)bf16_rne(q.y);
+          v[2] = (uint16_t)bf16_rne(q.z); v[3] = (uint16_t)bf16_rne(q.w);
+        } else {
+          const uint2 q = *(const uint2 *)((const uint16_t *)src + (int64_t)k * sbk + n);
+          v[0] = (uint16_t)q.x; v[1] = (uint16_t)(q.x >> 16); v[2] = (uint16_t)q.y; v[3] = (uint16_t)(q.y >> 16);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if (k < K && n + j < N) {
+          if (sizeof(TB) == 4) v[j] = (uint16_t)bf16_rne(widen(src[(int64_t)k * sbk + n + j]));
+          else v[j] = (uint16_t)src[(int64_t)k * sbk + n + j];
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) tile[c4 + j][r + i * 16] = v[j];  // stored transposed: tile[n][k]
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const uint32_t n = n0 + r + i * 16, k = k0 + c4;
+    const uint16_t *t = &tile[r + i * 16][c4];
+    if (VEC) {
+      if (n < N && k < K) *(uint2 *)(dst + (uint64_t)n * K + k) = *(const uint2 *)t;
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if (n < N && k + j < K) dst[(uint64_t)n * K + k + j] = t[j];
+    }
+  }
+}
+
+hipError_t launch_transpose_cast_bf16(const LaunchCtx &lc, const void *b, int b_stype, void *out, uint32_t K,
+                                      uint32_t N, int64_t sbk, uint32_t nb0, uint32_t nb1, int64_t sb_b0,
+                                      int64_t sb_b1) {
+  if (!K || !N || !nb0 || !nb1) return hipSuccess;
+  dim3 grid((N + 63) / 64, (K + 63) / 64, nb0 * nb1);
+  const int es = b_stype == ST_BF16 ? 2 : 4;
+  const bool vec = N % 4 == 0 && K % 4 == 0 && sbk % 4 == 0 && sb_b0 % 4 == 0 && sb_b1 % 4 == 0 &&
+                   ((uintptr_t)b % (4 * es)) == 0 && ((uintptr_t)out % 8) == 0;
+  if (b_stype == ST_BF16) {
+    if (vec) CG_LAUNCH(lc, (transpose_cast_bf16_kernel<uint16_t, true>), grid, 256, (const uint16_t *)b, (uint16_t *)out, K, N, sbk, nb1, sb_b0, sb_b1);
+    else CG_LAUNCH(lc, (transpose_cast_bf16_kernel<uint16_t, false>), grid, 256, (const uint16_t *)b, (uint16_t *)out, K, N, sbk, nb1, sb_b0, sb_b1);
+  } else {
+    if (vec) CG_LAUNCH(lc, (transpose_cast_bf16_kernel<float, true>), grid, 256, (const float *)b, (uint16_t *)out, K, N, sbk, nb1, sb_b0, sb_b1);
+    else CG_LAUNCH(lc, (transpose_cast_bf16_kernel<float, false>), grid, 256, (const float *)b, (uint16_t *)out, K, N, sbk, nb1, sb_b0, sb_b1);
+  }
+  return hipGetLastError();
+}
+
 hipError_t launch_cast_bf16(const LaunchCtx &lc, const float *in, void *out, uint64_t n) {
   if (!n) return hipSuccess;
   const uint64_t n8 = n / 8;

@@ -165,6 +165,55 @@ hipError_t launch_fill_u32(const LaunchCtx &lc, uint32_t *dst, uint32_t value, u
   return hipGetLastError();
 }
 
+// ---- materialised transpose ------------------------------------------------------------------------------
+// T: input element (uint16_t = bf16); OUT16: bf16 stays bf16, otherwise 4-byte output (bf16 widened)
+template <typename T, bool OUT16>
+__global__ void __launch_bounds__(256) transpose_copy_kernel(TransposeDesc d) {
+  __shared__ uint32_t tile[64][65];
+  // blockIdx.z enumerates the other axes
+  uint32_t rem = blockIdx.z;
+  int64_t xo = 0, oo = 0;
+  for (int i = d.n_other - 1; i >= 0; --i) {
+    const uint32_t c = rem % d.odims[i];
+    rem /= d.odims[i];
+    xo += (int64_t)c * d.x_so[i];
+    oo += (int64_t)c * d.o_so[i];
+  }
+  const T *x = (const T *)d.x + xo;
+  uint32_t *out = (uint32_t *)d.out + (OUT16 ? 0 : oo);
+  uint16_t *out16 = (uint16_t *)d.out + oo;
+  const uint32_t c0 = blockIdx.x * 64, j0 = blockIdx.y * 64;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const uint32_t c = c0 + ty + i * 4, j = j0 + tx;
+    if (c < d.C && j < d.R) {
+      const T v = x[(int64_t)c * d.x_sc + j];
+      tile[ty + i * 4][tx] = (sizeof(T) == 2 && !OUT16) ? (uint32_t)v << 16 : (uint32_t)v;
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const uint32_t j = j0 + ty + i * 4, c = c0 + tx;
+    if (j < d.R && c < d.C) {
+      if (OUT16) out16[(int64_t)j * d.o_sj + c] = (uint16_t)tile[tx][ty + i * 4];
+      else out[(int64_t)j * d.o_sj + c] = tile[tx][ty + i * 4];
+    }
+  }
+}
+
+hipError_t launch_transpose_copy(const LaunchCtx &lc, const TransposeDesc &d) {
+  uint64_t other = 1;
+  for (int i = 0; i < d.n_other; ++i) other *= d.odims[i];
+  if (!d.R || !d.C || !other) return hipSuccess;
+  dim3 grid((d.C + 63) / 64, (d.R + 63) / 64, (unsigned)other);
+  if (d.x_stype == ST_BF16 && d.out_bf16) CG_LAUNCH(lc, (transpose_copy_kernel<uint16_t, true>), grid, 256, d);
+  else if (d.x_stype == ST_BF16) CG_LAUNCH(lc, (transpose_copy_kernel<uint16_t, false>), grid, 256, d);
+  else CG_LAUNCH(lc, (transpose_copy_kernel<uint32_t, false>), grid, 256, d);
+  return hipGetLastError();
+}
+
 // ---- peak probes --------------------------------------------------------------------------------------
 // What the machine gives to the simplest possible code, as denominators next to the data-sheet
 // numbers: a grid-stride 16-byte copy (HBM read + write) and a register-resident MFMA issue loop.

@@ -33,6 +33,10 @@ hipError_t launch_ew(const LaunchCtx &lc, const Program &p, const OutDesc &o, ui
 uint32_t reduce_split_chunks(const LaunchCtx &lc, uint32_t rows, uint32_t n);
 hipError_t launch_reduce(const LaunchCtx &lc, int kind, const Program &p, void *out, uint32_t rows,
                          uint32_t n, bool vec4, uint32_t *scratch, uint32_t chunks);
+// last-axis reduction of rows already in memory (unit stride along the row, n % 4 == 0, rows 16-byte
+// aligned; bf16 rows are widened); kind = ReduceKind
+hipError_t launch_reduce_plain(const LaunchCtx &lc, int kind, const void *x, int bf16, int64_t row_stride, void *out,
+                               uint32_t rows, uint32_t n);
 // reduction stages + final segment of a row program in one launch
 hipError_t launch_row(const LaunchCtx &lc, const Program &p, const OutDesc &o, uint32_t rows,
                       uint32_t n, bool vec4);
@@ -59,6 +63,21 @@ hipError_t launch_topk(const LaunchCtx &lc, const float *x, float *values, uint3
 hipError_t launch_compare(const LaunchCtx &lc, const void *a, const void *b, uint64_t n,
                           int is_f32, uint32_t *flag);
 hipError_t launch_fill_u32(const LaunchCtx &lc, uint32_t *dst, uint32_t value, uint64_t n);
+// Contiguous copy of a strided view whose unit-stride axis is not the last one (a materialised
+// transpose): 64 x 64 tiles through LDS, reads along the input's unit-stride axis `j`, writes
+// along the output's last axis.  4-byte output elements (bf16 input widened), or bf16 to bf16.
+struct TransposeDesc {
+  const void *x;
+  void *out;
+  int32_t x_stype, out_bf16;  // out_bf16: bf16 in, bf16 out (otherwise 4-byte output)
+  uint32_t R, C;            // extents of axis j and of the last axis
+  int64_t x_sc;             // input stride of the last axis (axis j has input stride 1)
+  int64_t o_sj;             // output stride of axis j (the last axis has output stride 1)
+  int32_t n_other;          // remaining axes, outermost first
+  uint32_t odims[MAX_DIMS + 2];
+  int64_t x_so[MAX_DIMS + 2], o_so[MAX_DIMS + 2];
+};
+hipError_t launch_transpose_copy(const LaunchCtx &lc, const TransposeDesc &d);
 // peak probes: plain 16-byte copy; MFMA issue loop (out: grid * 256 floats)
 hipError_t launch_peak_copy(const LaunchCtx &lc, const void *in, void *out, uint64_t bytes);
 hipError_t launch_peak_mfma(const LaunchCtx &lc, int bf16, float *out, unsigned grid, int iters);
@@ -149,6 +168,11 @@ uint32_t gemm_split_k(const LaunchCtx &lc, const GemmDesc &g);
 hipError_t launch_matmul(const LaunchCtx &lc, const GemmDesc &g, const char **kernel_name);
 // contiguous f32 -> bf16 (RNE); n % 8 == 0, 16-byte aligned
 hipError_t launch_cast_bf16(const LaunchCtx &lc, const float *in, void *out, uint64_t n);
+// B[k, n] (unit stride along n, row stride sbk, f32 or bf16, nb0 x nb1 batches through sb_b0 / sb_b1)
+// -> contiguous bf16 [nb0 * nb1][N][K]
+hipError_t launch_transpose_cast_bf16(const LaunchCtx &lc, const void *b, int b_stype, void *out, uint32_t K,
+                                      uint32_t N, int64_t sbk, uint32_t nb0, uint32_t nb1, int64_t sb_b0,
+                                      int64_t sb_b1);
 // Several GEMVs y_p = x . B_p^T that share x (M == 1, B_p k-contiguous, 16-byte aligned rows):
 // one launch, problem p on grid.y
 struct GemvMultiDesc {

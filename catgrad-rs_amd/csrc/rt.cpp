@@ -708,12 +708,54 @@ int run_ew(cg_backend *be, cg_tensor *root, bool root_is_value, void *dst, const
 }
 
 // A fresh contiguous tensor holding the value of `src` (f32/u32 storage unless keep_bf16).
+// src (realised) -> dst (contiguous, 4-byte elements) when src's unit-stride axis is not its last
+// one: the tiled transpose kernel instead of a strided elementwise pass.
+int try_transpose_copy(cg_backend *be, const cg_tensor *src, cg_tensor *dst, bool *done) {
+  const int r = src->rank;
+  if (r < 2 || src->size() == 0 || (dst->stype == ST_BF16 && src->stype != ST_BF16)) return CG_OK;
+  const int64_t C = src->shape[r - 1];
+  if (C < 16 || src->strides[r - 1] == 1 || src->strides[r - 1] == 0) return CG_OK;
+  int j = -1;
+  for (int i = r - 2; i >= 0; --i)
+    if (src->strides[i] == 1 && src->shape[i] >= 16) {
+      j = i;
+      break;
+    }
+  if (j < 0) return CG_OK;
+  TransposeDesc d;
+  std::memset(&d, 0, sizeof(d));
+  d.x = data_ptr(src);
+  d.out = data_ptr(dst);
+  d.x_stype = src->stype;
+  d.out_bf16 = dst->stype == ST_BF16;
+  d.R = (uint32_t)src->shape[j];
+  d.C = (uint32_t)C;
+  d.x_sc = src->strides[r - 1];
+  d.o_sj = dst->strides[j];
+  uint64_t other = 1;
+  for (int i = 0; i < r - 1; ++i) {
+    if (i == j || src->shape[i] == 1) continue;
+    d.odims[d.n_other] = (uint32_t)src->shape[i];
+    d.x_so[d.n_other] = src->strides[i];
+    d.o_so[d.n_other] = dst->strides[i];
+    d.n_other++;
+    other *= (uint64_t)src->shape[i];
+  }
+  if (other > 65535) return CG_OK;  // grid.z
+  KernelScope ks(be, "transpose_copy", (double)src->size() * (esize(src->stype) + esize(dst->stype)), 0);
+  HIPCHK(be, launch_transpose_copy(be->lc(), d));
+  *done = true;
+  return CG_OK;
+}
+
 int materialize(cg_backend *be, cg_tensor *src, cg_tensor **out, bool keep_bf16 = false) {
   TRY(realize(be, src));
   cg_tensor *t = new_node(be, src->dtype, src->rank, src->shape);
   int stype = (keep_bf16 && src->stype == ST_BF16) ? ST_BF16 : (src->dtype == CG_F32 ? ST_F32 : ST_U32);
   int st = alloc_result(be, t, stype);
-  if (!st) st = run_ew(be, src, true, data_ptr(t), t->strides, stype, "ew_copy");
+  bool transposed = false;
+  if (!st && !(be->flags & CG_FLAG_NO_PATTERNS)) st = try_transpose_copy(be, src, t, &transposed);
+  if (!st && !transposed) st = run_ew(be, src, true, data_ptr(t), t->strides, stype, "ew_copy");
   if (st) {
     node_release(t);
     return st;
@@ -1375,9 +1417,51 @@ int realize_view(cg_backend *be, cg_tensor *n) {
   return CG_OK;
 }
 
+// t (realised) as rows of unit-stride elements with one stride between rows
+bool rows_layout(const cg_tensor *t, int64_t *row_stride) {
+  const int r = t->rank;
+  if (r == 0 || (t->shape[r - 1] != 1 && t->strides[r - 1] != 1)) return false;
+  int64_t rs = -1, expect = 0;
+  for (int i = r - 2; i >= 0; --i) {
+    if (t->shape[i] == 1) continue;
+    if (rs < 0) {
+      rs = t->strides[i];
+      expect = rs * t->shape[i];
+    } else {
+      if (t->strides[i] != expect) return false;
+      expect *= t->shape[i];
+    }
+  }
+  *row_stride = rs < 0 ? t->shape[r - 1] : rs;
+  return true;
+}
+
 int realize_reduce(cg_backend *be, cg_tensor *n) {
   cg_tensor *x = n->in[0];
   const int kind = (int)n->p0;
+  // a tensor that is (or has to be) in memory anyway, with enough rows to fill the device: stream it
+  if (!(be->flags & CG_FLAG_NO_PATTERNS) && !((x->op == N_BIN || x->op == N_UN) && x->rc.load() == 1) &&
+      x->rank >= 1 && x->size() > 0 && x->size() < ((int64_t)1 << 32)) {
+    const int64_t cols = x->shape[x->rank - 1], rows = x->size() / cols;
+    if (cols % 4 == 0 && cols >= 64 && rows >= be->n_cus) {
+      TRY(realize(be, x));
+      int64_t rs = 0;
+      const int es = esize(x->stype);
+      if (rows_layout(x, &rs) && (uintptr_t)data_ptr(x) % (4 * es) == 0 && rs % 4 == 0 &&
+          !(x->stype == ST_BF16 && (kind == R_SUM_U || kind == R_MAX_U || kind == R_ARGMAX_U))) {
+        TRY(alloc_result(be, n, n->dtype == CG_F32 ? ST_F32 : ST_U32));
+        const char *name = kind <= R_SUM_U ? "reduce_sum" : kind <= R_MAX_U ? "reduce_max" : "reduce_argmax";
+        {
+          KernelScope ks(be, name, (double)x->size() * es + (double)rows * 4, 0);
+          HIPCHK(be, launch_reduce_plain(be->lc(), kind, data_ptr(x), x->stype == ST_BF16, rs, n->st->ptr,
+                                         (uint32_t)rows, (uint32_t)cols));
+        }
+        n->op = N_REAL;
+        drop_inputs(n);
+        return CG_OK;
+      }
+    }
+  }
   // the input tree is evaluated inside the reduction when nobody else reads it
   Region reg;
   EwCompiler c(be, &reg);
@@ -1897,6 +1981,30 @@ int realize_matmul(cg_backend *be, cg_tensor *n, cg_tensor *addend = nullptr, bo
     g.sb_b0 = sbo[0];
     g.sb_b1 = sbo[1];
     g.bf16_math = (be->flags & CG_FLAG_BF16) ? 1 : 0;
+    // B with unit stride along n (bmm of row-major matrices, p . V): re-laid out once as bf16 [N, K]
+    // so that the product takes the direct-to-LDS kernel (one pass over B against K/64 strided ones)
+    Storage *bt = nullptr;
+    if (g.bf16_math && M >= 64 && N >= 64 && K % 64 == 0 && g.a_stype == ST_BF16 && g.sak == 1 && g.sbn == 1 &&
+        g.sbk != 1 && !ex.w && (g.b_stype == ST_F32 || g.b_stype == ST_BF16)) {
+      // batches that only repeat (stride 0) are transposed once
+      const uint32_t tb0 = g.sb_b0 ? g.nb0 : 1, tb1 = g.sb_b1 ? g.nb1 : 1;
+      TRY(dev_alloc(be, (size_t)tb0 * tb1 * N * K * 2, &bt));
+      hipError_t te;
+      {
+        KernelScope ks(be, "transpose_cast_bf16", (double)tb0 * tb1 * N * K * (esize(g.b_stype) + 2), 0);
+        te = launch_transpose_cast_bf16(be->lc(), g.b, g.b_stype, bt->ptr, K, N, g.sbk, tb0, tb1, g.sb_b0, g.sb_b1);
+      }
+      if (te != hipSuccess) {
+        storage_release(bt);
+        return fail(be, CG_ERR_DEVICE, hipGetErrorString(te));
+      }
+      g.b = bt->ptr;
+      g.b_stype = ST_BF16;
+      g.sbk = 1;
+      g.sbn = K;
+      g.sb_b1 = g.sb_b1 ? (int64_t)N * K : 0;
+      g.sb_b0 = g.sb_b0 ? (int64_t)tb1 * N * K : 0;
+    }
     if (addend && M <= 8 && g.a_stype == ST_F32 && K > 0 && (g.sbk == 1 || g.sbn == 1 || K == 1 || N == 1)) {
       g.c_add = (const float *)data_ptr(addend);
       *added = true;
@@ -2005,6 +2113,7 @@ int realize_matmul(cg_backend *be, cg_tensor *n, cg_tensor *addend = nullptr, bo
       }
     }
     storage_release(ws);
+    storage_release(bt);
     HIPCHK(be, e);
   }
   if (n->gemv_candidate) forget_gemv_candidate(n);
