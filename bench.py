@@ -49,12 +49,12 @@ def main():
     ap.add_argument("--warmup", type=int, default=4)
     ap.add_argument("--dtype", choices=["bf16", "f32"], default="bf16")
     ap.add_argument("--prompt", type=int, default=512)
-    ap.add_argument("--layers", type=int, default=16)
+    ap.add_argument("--layers", type=int, default=None)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-steps", type=int, default=3)
-    ap.add_argument("--workload", choices=["llama", "ops"], default="llama",
-                    help="ops: the single-op microbenchmarks (one JSON line with a table) instead of "
-                         "the decoder")
+    ap.add_argument("--workload", choices=["llama", "ops", "qwen_moe", "gemma3"], default="llama",
+                    help="ops: the single-op microbenchmarks (one JSON line with a table); qwen_moe / gemma3: "
+                         "BASELINE configs[3] / [4] at full shape (--layers to shorten)")
     ap.add_argument("--sync-each-step", action="store_true",
                     help="read every token on the host before starting the next step")
     ap.add_argument("--profile-only", action="store_true",
@@ -69,8 +69,17 @@ def main():
     llm = importlib.import_module("catgrad-rs_amd.llm")
     import llama_util as U
 
-    cfg = llama_1b_config(llm, args.layers)
     lib = cg.load_library()
+    if args.workload in ("qwen_moe", "gemma3"):
+        mb = importlib.import_module("catgrad-rs_amd.modelbench")
+        if args.workload == "qwen_moe":
+            rec = mb.run_qwen_moe(lib, layers=args.layers or 24, steps=args.steps, warmup=args.warmup)
+        else:
+            rec = mb.run_gemma3(lib, layers=args.layers or 26)
+        print(json.dumps({"metric": rec.pop("workload"), "n_gpus": 1, "dtype": "bf16", "data": "synthetic", **rec}))
+        return
+    args.layers = args.layers or 16
+    cfg = llama_1b_config(llm, args.layers)
     if args.workload == "ops":
         opbench = importlib.import_module("catgrad-rs_amd.opbench")
         recs = opbench.run_all(lib, iters=max(args.steps, 10))

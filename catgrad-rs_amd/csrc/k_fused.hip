@@ -53,6 +53,10 @@ __global__ void __launch_bounds__(BLOCK) rmsnorm_kernel(RmsNormDesc d) {
         o.x *= d.gamma_offset + g.x; o.y *= d.gamma_offset + g.y;
         o.z *= d.gamma_offset + g.z; o.w *= d.gamma_offset + g.w;
       }
+      if (d.residual) {
+        const float4 r = *(const float4 *)(d.residual + (int64_t)row * d.n + c);
+        o.x += r.x; o.y += r.y; o.z += r.z; o.w += r.w;
+      }
       *(float4 *)(y + c) = o;
     }
   }

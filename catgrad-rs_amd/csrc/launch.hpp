@@ -86,6 +86,7 @@ hipError_t launch_peak_mfma(const LaunchCtx &lc, int bf16, float *out, unsigned 
 struct RmsNormDesc {
   const float *x;        // rows of n contiguous floats, row r at x + r * x_row_stride
   const float *gamma;    // n floats or null
+  const float *residual; // contiguous [rows, n] added to the result, or null
   float *y;              // contiguous [rows, n]
   int64_t x_row_stride;
   uint32_t rows, n;

@@ -667,6 +667,12 @@ int launch_compiled(cg_backend *be, EwCompiler &c, cg_tensor *root, void *dst,
     if (dst_stype == ST_BF16) return fail(be, CG_ERR_INTERNAL, "row program into bf16 storage");
     const int64_t cols = root->shape[root->rank - 1];
     KernelScope ks(be, "row_fused", bytes_in + (double)n * 4, 0);
+    if (be->trace_shapes) {
+      char buf[96];
+      snprintf(buf, sizeof buf, "row_fused[%lldx%lld,i%d,in%d,st%d]", (long long)(n / cols), (long long)cols,
+               (int)c.p.n_instr, (int)c.p.n_in, (int)c.p.n_stages);
+      ks.rename(buf);
+    }
     HIPCHK(be, launch_row(be->lc(), c.p, o, (uint32_t)(n / cols), (uint32_t)cols, vec4));
     return CG_OK;
   }
@@ -1013,11 +1019,35 @@ int gamma_row_vector(cg_backend *be, cg_tensor *gb, bool *ok) {
   return CG_OK;
 }
 
+// also `res + rmsnorm(..)` / `rmsnorm(..) + res` (gemma3.rs:198-240 adds the residual right after the
+// post-attention and post-feedforward norms): the addend rides along in the same kernel
 int try_rmsnorm(cg_backend *be, cg_tensor *root, bool *done) {
   RmsNormMatch rm;
-  if (!match_rmsnorm(root, &rm)) return CG_OK;
+  cg_tensor *residual = nullptr;
+  if (!match_rmsnorm(root, &rm)) {
+    if (root->dtype != CG_F32 || !is_bin(root, E_ADD_F)) return CG_OK;
+    int side = -1;
+    for (int i = 0; i < 2 && side < 0; ++i)
+      if (root->in[i]->op != N_REAL && refs(root->in[i]) == 1 && match_rmsnorm(root->in[i], &rm)) side = i;
+    if (side < 0) return CG_OK;
+    residual = root->in[1 - side];
+    if (residual->op == N_CONST || ((residual->op == N_BIN || residual->op == N_UN) && refs(residual) == 1))
+      return CG_OK;  // the addend is itself an unrealised expression: leave it to the generic fusion
+  }
   cg_tensor *x = rm.x, *gb = rm.gamma;
   const int64_t n = root->shape[root->rank - 1];
+  cg_tensor *rs = nullptr;
+  if (residual) {
+    TRY(contiguous(be, residual, &rs));
+    if ((uintptr_t)data_ptr(rs) % 16) {
+      node_release(rs);
+      return CG_OK;
+    }
+  }
+  struct Rel {
+    cg_tensor *t;
+    ~Rel() { node_release(t); }
+  } rel{rs};
   RmsNormDesc d;
   std::memset(&d, 0, sizeof(d));
   d.eps = rm.eps;
@@ -1041,7 +1071,8 @@ int try_rmsnorm(cg_backend *be, cg_tensor *root, bool *done) {
     d.x_row_stride = row_stride;
     d.rows = (uint32_t)(root->size() / n);
     d.n = (uint32_t)n;
-    KernelScope ks(be, "rmsnorm_fused", (double)root->size() * 8 + n * 4, 0);
+    d.residual = rs ? (const float *)data_ptr(rs) : nullptr;
+    KernelScope ks(be, "rmsnorm_fused", (double)root->size() * (rs ? 12 : 8) + n * 4, 0);
     hipError_t e = launch_rmsnorm(be->lc(), d);
     if (e != hipSuccess) st = fail(be, CG_ERR_DEVICE, hipGetErrorString(e));
   }

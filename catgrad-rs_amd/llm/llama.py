@@ -13,7 +13,7 @@ import numpy as np
 
 from ..lang import (Module, NAT, TENSOR, argmax, broadcast, concat, constant, matmul, make_shape,
                     path, reshape, shape, slice, transpose, unpack)
-from ..nn import linear_no_bias, silu, softmax
+from ..nn import linear_b, silu, softmax
 from .helpers import (Cache, apply_rope_embedding, causal_mask, embeddings, repeat_kv, rmsnorm,
                       rope_tables)
 
@@ -29,13 +29,23 @@ class LlamaModel(Module):
     def sort(self):
         return [TENSOR], [TENSOR]
 
+    # Two seams for the decoders built on this layer (qwen_moe.py): how a linear is applied (the
+    # reference's is batch-1, stdlib/nn/mod.rs:182-192) and how ids become the first activations.
+    qkv_bias = False
+
+    def linear(self, builder, in_dim, out_dim, p, x, bias=False):
+        return linear_b(builder, in_dim, out_dim, bias, p, x)
+
+    def embed(self, builder, ids):
+        return embeddings(builder, self.path().extend(["model", "embed_tokens"]), ids)
+
     # models/llama.rs:11-35
     def mlp(self, builder, p, x):
         c = self.config
-        gate = linear_no_bias(builder, c.hidden_size, c.intermediate_size, p.extend(["gate_proj"]), x)
-        up = linear_no_bias(builder, c.hidden_size, c.intermediate_size, p.extend(["up_proj"]), x)
+        gate = self.linear(builder, c.hidden_size, c.intermediate_size, p.extend(["gate_proj"]), x)
+        up = self.linear(builder, c.hidden_size, c.intermediate_size, p.extend(["up_proj"]), x)
         x = silu(builder, gate) * up
-        return linear_no_bias(builder, c.intermediate_size, c.hidden_size, p.extend(["down_proj"]), x)
+        return self.linear(builder, c.intermediate_size, c.hidden_size, p.extend(["down_proj"]), x)
 
     def qkv(self, builder, p, x):
         c = self.config
@@ -44,9 +54,9 @@ class LlamaModel(Module):
         head_dim = c.hidden_size // num_heads
         rep = num_heads // num_kv_heads
         b, s, _ = unpack(builder, 3, shape(builder, x))
-        q = linear_no_bias(builder, dim, dim, p.extend(["q_proj"]), x)
-        k = linear_no_bias(builder, dim, dim // rep, p.extend(["k_proj"]), x)
-        v = linear_no_bias(builder, dim, dim // rep, p.extend(["v_proj"]), x)
+        q = self.linear(builder, dim, dim, p.extend(["q_proj"]), x, bias=self.qkv_bias)
+        k = self.linear(builder, dim, dim // rep, p.extend(["k_proj"]), x, bias=self.qkv_bias)
+        v = self.linear(builder, dim, dim // rep, p.extend(["v_proj"]), x, bias=self.qkv_bias)
         sh = make_shape(builder, b, s, num_kv_heads, head_dim)
         k = reshape(builder, sh, k)
         v = reshape(builder, sh, v)
@@ -74,7 +84,7 @@ class LlamaModel(Module):
         attn = matmul(builder, attn, v)
         attn = transpose(builder, 1, 2, attn)
         attn = reshape(builder, make_shape(builder, b, s, dim), attn)
-        return linear_no_bias(builder, dim, dim, p.extend(["o_proj"]), attn)
+        return self.linear(builder, dim, dim, p.extend(["o_proj"]), attn)
 
     # models/llama.rs:37-112
     def attention(self, builder, layer_id, cache, pos, p, x):
@@ -104,7 +114,7 @@ class LlamaModel(Module):
         c = self.config
         root = self.path()
         w = ["model", "embed_tokens"] if c.tie_word_embeddings else ["lm_head"]
-        return linear_no_bias(builder, c.hidden_size, c.vocab_size, root.extend(w), x)
+        return self.linear(builder, c.hidden_size, c.vocab_size, root.extend(w), x)
 
     # models/llama.rs:150-204
     def def_(self, builder, args):
@@ -112,7 +122,7 @@ class LlamaModel(Module):
         c = self.config
         root = self.path()
         cache = Cache.init(builder, c, self.max_sequence_length)
-        x = embeddings(builder, root.extend(["model", "embed_tokens"]), x)
+        x = self.embed(builder, x)
         for i in range(c.num_hidden_layers):
             x = self.layer(builder, i, cache, 0, root.extend(["model", "layers", i]), x)
         x = rmsnorm(builder, c.rms_norm_eps, root.extend(["model", "norm"]), x)
@@ -128,7 +138,7 @@ class RopeTables(Module):
         self.config = config
 
     def path(self):
-        return path(["llama", "rope_tables"])
+        return path(["rope_tables"])
 
     def sort(self):
         return [NAT], [TENSOR, TENSOR]
@@ -164,7 +174,7 @@ class _LlamaCached(LlamaModel):
             vr = repeat_kv(builder, rep, v)
             return self.scores(builder, b, s, q, kr, vr, p)
 
-        x = embeddings(builder, root.extend(["model", "embed_tokens"]), ids)
+        x = self.embed(builder, ids)
         for i in range(c.num_hidden_layers):
             x = self.layer(builder, i, cache, pos, root.extend(["model", "layers", i]), x,
                            attention=attention)

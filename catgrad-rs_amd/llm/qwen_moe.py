@@ -31,24 +31,16 @@ def unfold_batch(builder, b, s, x):
     return reshape(builder, make_shape(builder, b, s, h), x)
 
 
-class QwenMoeModel(Module):
-    def __init__(self, config, max_sequence_length, last_position_only=False):
-        self.config = config
-        self.max_sequence_length = max_sequence_length
-        self.last_position_only = last_position_only
-
-    def path(self):
-        return path(["qwen_moe"])
-
-    def sort(self):
-        return [TENSOR], [TENSOR, TENSOR]
+class QwenMoeParts:
+    """The pieces shared by the full-recompute model below and the KV-cached terms: batch-folding
+    linear, routed experts + gated shared expert."""
 
     def linear(self, builder, i, o, p, x, bias=False):
         f, b, s = fold_batch(builder, x)
         y = linear_b(builder, i, o, bias, p, f)
         return unfold_batch(builder, b, s, y)
 
-    def mlp(self, builder, ffn, p, x):
+    def dense_mlp(self, builder, ffn, p, x):
         c = self.config
         gate = linear_no_bias(builder, c.hidden_size, ffn, p.extend(["gate_proj"]), x)
         up = linear_no_bias(builder, c.hidden_size, ffn, p.extend(["up_proj"]), x)
@@ -91,10 +83,24 @@ class QwenMoeModel(Module):
             sumk = sumk + h * v
         sumk = transpose(builder, 0, 1, sumk)
         # shared expert (deepseek.rs:163-165) with Qwen1.5-MoE's sigmoid gate
-        shared = self.mlp(builder, c.shared_expert_intermediate_size, p.extend(["shared_expert"]), x)
+        shared = self.dense_mlp(builder, c.shared_expert_intermediate_size, p.extend(["shared_expert"]), x)
         sg = linear_no_bias(builder, c.hidden_size, 1, p.extend(["shared_expert_gate"]), x)
         sg = broadcast(builder, sigmoid(builder, sg), shape(builder, shared))
         return sumk + shared * sg
+
+
+
+class QwenMoeModel(QwenMoeParts, Module):
+    def __init__(self, config, max_sequence_length, last_position_only=False):
+        self.config = config
+        self.max_sequence_length = max_sequence_length
+        self.last_position_only = last_position_only
+
+    def path(self):
+        return path(["qwen_moe"])
+
+    def sort(self):
+        return [TENSOR], [TENSOR, TENSOR]
 
     def attention(self, builder, cache, pos, p, x):
         c = self.config
@@ -147,3 +153,34 @@ class QwenMoeModel(Module):
             x = slice_(builder, 1, self.max_sequence_length - 1, 1, x)
         logits = self.linear(builder, c.hidden_size, c.vocab_size, root.extend(["lm_head"]), x)
         return [argmax(builder, logits), logits]
+
+
+# ---- KV-cached terms (BASELINE config 4: batch 4 x 256-token prompts, 64 greedy steps) -----------------
+# The same cached layer as llama.LlamaPrefill / LlamaDecode (rope, concat(2, cached, new), repeat_kv,
+# last-position lm_head), with this model's linear (q/k/v bias, batch folded into the sequence
+# axis) and the MoE block in place of the dense MLP.
+from . import llama as _llama  # noqa: E402
+
+
+class _QwenMoeCachedParts(QwenMoeParts):
+    qkv_bias = True
+
+    def path(self):
+        return path(["qwen_moe"])
+
+    def embed(self, builder, ids):
+        b, s = unpack(builder, 2, shape(builder, ids))
+        x = embeddings(builder, self.path().extend(["model", "embed_tokens"]), ids)
+        return reshape(builder, make_shape(builder, b, s, self.config.hidden_size), x)
+
+    def mlp(self, builder, p, x):
+        f, b, s = fold_batch(builder, x)
+        return unfold_batch(builder, b, s, self.moe(builder, p, f))
+
+
+class QwenMoePrefill(_QwenMoeCachedParts, _llama.LlamaPrefill):
+    """ids[B,S], cos, sin -> token[B,1,1], logits[B,1,V], k0, v0, ..."""
+
+
+class QwenMoeDecode(_QwenMoeCachedParts, _llama.LlamaDecode):
+    """ids[B,1], pos: Nat, cos, sin, k0, v0, ... -> token, logits, k0', v0', ..."""

@@ -56,20 +56,25 @@ def interpreter(be, arrays):
 class CachedRunner:
     """Greedy decoding with the KV-cached terms (prefill once, then one token per run)."""
 
-    def __init__(self, be, cfg, arrays, max_positions):
+    def __init__(self, be, cfg, arrays, max_positions, prefill_cls=None, decode_cls=None):
+        """prefill_cls / decode_cls: the KV-cached term classes (default Llama's; the Qwen-MoE-layout
+        ones take ids of shape [B, S])."""
         self.be, self.cfg = be, cfg
+        self.prefill_cls = prefill_cls or llama.LlamaPrefill
         self.it = interpreter(be, arrays)
         self.cos, self.sin = self.it.run(llama.RopeTables(cfg).term(), [max_positions])
-        self.decode_term = llama.LlamaDecode(cfg).term()
+        self.decode_term = (decode_cls or llama.LlamaDecode)(cfg).term()
         self.kv = None
         self.pos = 0
         self._prefill_terms = {}
 
     def prefill(self, ids):
-        ids = np.asarray(ids, np.uint32).reshape(1, -1)
+        ids = np.asarray(ids, np.uint32)
+        ids = ids.reshape(1, -1) if ids.ndim == 1 else ids
         n = ids.shape[1]
+        self.batch = ids.shape[0]
         if n not in self._prefill_terms:      # the term depends on the prompt length only
-            self._prefill_terms[n] = llama.LlamaPrefill(self.cfg, n).term()
+            self._prefill_terms[n] = self.prefill_cls(self.cfg, n).term()
         term = self._prefill_terms[n]
         out = self.it.run(term, [self.be.tensor(ids), self.cos, self.sin])
         self.kv = out[2:]
@@ -79,9 +84,9 @@ class CachedRunner:
     def step(self, token):
         """`token`: an int, or the [1, 1, 1] token tensor of the previous step (stays on the device)."""
         if isinstance(token, cg.Tensor):
-            ids = self.be.reshape(token, [1, 1])
+            ids = self.be.reshape(token, [self.batch, 1])
         else:
-            ids = self.be.tensor(np.asarray([[token]], np.uint32))
+            ids = self.be.tensor(np.asarray(token, np.uint32).reshape(self.batch, 1))
         out = self.it.run(self.decode_term, [ids, self.pos, self.cos, self.sin] + self.kv)
         self.kv = out[2:]
         self.pos += 1

@@ -9,7 +9,8 @@ llm = importlib.import_module("catgrad-rs_amd.llm")
 def qwen_moe_config(**kw):
     c = dict(hidden_size=64, num_hidden_layers=2, num_attention_heads=4, num_key_value_heads=4, head_dim=16,
              vocab_size=97, rms_norm_eps=1e-6, rope_theta=1000000.0, num_experts=8, num_experts_per_tok=2,
-             moe_intermediate_size=48, shared_expert_intermediate_size=96, norm_topk_prob=False)
+             moe_intermediate_size=48, shared_expert_intermediate_size=96, norm_topk_prob=False,
+             tie_word_embeddings=False)
     c.update(kw)
     return llm.Config(**c)
 

@@ -264,3 +264,22 @@ def test_glu_in_projection_prologue(oracle, hip, hip_nopat, K, N, act):
     assert not ({"swiglu_fused", "geglu_fused", "binary_f32"} & names), sorted(names)
     assert np.allclose(got[0], ref, rtol=1e-4, atol=1e-5), np.abs(got[0] - ref).max()
     assert np.allclose(gen, ref, rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize("order", ["res_first", "norm_first"])
+@pytest.mark.parametrize("shape", [(2, 33, 1152), (1, 7, 64)])
+def test_rmsnorm_plus_residual(oracle, hip, hip_nopat, shape, order):
+    """gemma3.rs:198-240: res + rmsnorm(x) (1 + gamma form) in the RMSNorm kernel."""
+    g = np.random.default_rng(shape[1])
+    x = (g.standard_normal(shape) * 2).astype(np.float32)
+    res = g.standard_normal(shape).astype(np.float32)
+    p = {"n.weight": (g.standard_normal(shape[-1]) * 0.1).astype(np.float32)}
+
+    def f(b, xv, rv):
+        xv = xv + xv - xv           # the residual stream is a value in memory; the normed branch is computed
+        gm = lang.param(b, lang.path(["n", "weight"]))
+        raw = helpers.rmsnorm_raw(b, 1e-6, xv)
+        gm = lang.broadcast(b, gm, lang.shape(b, raw))
+        h = raw * (lang.constant(b, 1.0, lang.shape(b, gm)) + gm)
+        return rv + h if order == "res_first" else h + rv
+    check(oracle, hip, hip_nopat, f, 1, [x, res], "rmsnorm_fused", params=p, rtol=1e-4, atol=1e-5)

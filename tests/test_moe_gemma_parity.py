@@ -176,3 +176,50 @@ def test_expert_index_out_of_bounds_is_reported(hip):
     # the flag is cleared: the next evaluation is clean
     (ok,) = vectors.run(hip, f, 1, x, np.array([1, 2], np.uint32), w)
     assert np.array_equal(ok, np.full((2, 1, 8), 16.0, np.float32))
+
+
+def moe_cached_generate(be, cfg, arrays, prompts, steps):
+    """Greedy tokens [steps, B] and last logits per step with the KV-cached Qwen-MoE terms."""
+    r = U.CachedRunner(be, cfg, arrays, prompts.shape[1] + steps + 4,
+                       prefill_cls=llm.qwen_moe.QwenMoePrefill, decode_cls=llm.qwen_moe.QwenMoeDecode)
+    tok, logits = r.prefill(prompts)
+    toks, lg = [], []
+    for _ in range(steps):
+        t = be.to_vec(tok).reshape(-1)
+        toks.append(t.copy())
+        lg.append(be.numpy(logits))
+        tok, logits = r.step(t)
+    return np.stack(toks), lg
+
+
+def test_moe_cached_equals_full_recompute_on_oracle(oracle):
+    """Batch of 2 prompts: the KV-cached terms give the logits of the full-recompute model."""
+    cfg = MU.qwen_moe_config()
+    P = MU.qwen_moe_params(cfg, seed=11, std=0.15)
+    prompts = np.random.default_rng(12).integers(0, cfg.vocab_size, (2, 6))
+    toks, lg = moe_cached_generate(oracle, cfg, P, prompts, 3)
+    seqs = prompts.copy()
+    for i in range(3):
+        _, full = run_model(oracle, llm.qwen_moe.QwenMoeModel(cfg, seqs.shape[1]), P, seqs)
+        assert np.allclose(lg[i][:, 0], full[:, -1], rtol=2e-4, atol=2e-5), i
+        assert np.array_equal(toks[i], full[:, -1].argmax(-1))
+        seqs = np.concatenate([seqs, toks[i][:, None]], axis=1)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("mode", ["f32", "bf16"])
+def test_moe_cached_decode_hip_vs_oracle(oracle, hip, hip_bf16, mode):
+    cfg = MU.qwen_moe_config()
+    P = MU.qwen_moe_params(cfg, seed=13, std=0.15)
+    prompts = np.random.default_rng(14).integers(0, cfg.vocab_size, (3, 9))
+    dev = hip if mode == "f32" else hip_bf16
+    P_ref = {k: (U_round(v) if v.ndim >= 2 else v) for k, v in P.items()} if mode == "bf16" else P
+    rt, rl = moe_cached_generate(oracle, cfg, P_ref, prompts, 6)
+    gt, gl = moe_cached_generate(dev, cfg, P, prompts, 6)
+    tol = 4e-2 if mode == "bf16" else 2e-4
+    for i in range(6):
+        if not np.array_equal(rt[i], gt[i]):
+            break   # sequences diverged on a near tie: later steps are not comparable
+        assert np.max(np.abs(rl[i] - gl[i])) <= tol * np.abs(rl[i]).max(), i
+    if mode == "f32":
+        assert np.array_equal(rt, gt)
