@@ -32,6 +32,16 @@ __device__ __forceinline__ float block_reduce(float v, float *lds) {
   return r;
 }
 
+// f32 -> bf16, round to nearest even (NaN stays NaN); two values packed low / high
+__device__ __forceinline__ uint32_t bf16_bits(float f) {
+  const uint32_t u = __float_as_uint(f);
+  if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (u >> 16) | 0x40u;
+  return (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
+}
+__device__ __forceinline__ uint2 bf16_pack4(float4 v) {
+  return make_uint2(bf16_bits(v.x) | (bf16_bits(v.y) << 16), bf16_bits(v.z) | (bf16_bits(v.w) << 16));
+}
+
 __device__ __forceinline__ float sigmoid_ref(float x) { return 1.0f / (1.0f + expf(-x)); }
 // nn::gelu: 0.5 x (1 + tanh(c (x + k x^3))), tanh(t) = 2 sigmoid(2 t) - 1 (nn/mod.rs:138-160)
 __device__ __forceinline__ float gelu_ref(float x) {

@@ -58,6 +58,7 @@ __global__ void __launch_bounds__(BLOCK) rmsnorm_kernel(RmsNormDesc d) {
         o.x += r.x; o.y += r.y; o.z += r.z; o.w += r.w;
       }
       *(float4 *)(y + c) = o;
+      if (d.y16) *(uint2 *)(d.y16 + (int64_t)row * d.n + c) = bf16_pack4(o);
     }
   }
 }
@@ -119,7 +120,11 @@ __global__ void __launch_bounds__(BLOCK == 64 ? 256 : BLOCK) softmax_kernel(Soft
 #pragma unroll
   for (int e = 0; e < EPT; ++e) {
     const uint32_t c = tid + e * BLOCK;
-    if (c < d.n) y[c] = v[e] / sum;
+    if (c < d.n) {
+      const float o = v[e] / sum;
+      y[c] = o;
+      if (d.y16) d.y16[(int64_t)row * d.n + c] = (uint16_t)bf16_bits(o);
+    }
   }
 }
 
@@ -179,6 +184,7 @@ __global__ void __launch_bounds__(BLOCK) softmax_vec_kernel(SoftmaxDesc d) {
       float4 t = v[e];
       t.x = t.x / sum; t.y = t.y / sum; t.z = t.z / sum; t.w = t.w / sum;
       *(float4 *)(y + c) = t;
+      if (d.y16) *(uint2 *)(d.y16 + (int64_t)row * d.n + c) = bf16_pack4(t);
     }
   }
 }
@@ -337,7 +343,9 @@ __global__ void __launch_bounds__(256) rope_kernel(RopeDesc d) {
     float4 o;
     o.x = c.x * xv.x + sn.x * pv.x; o.y = c.y * xv.y + sn.y * pv.y;
     o.z = c.z * xv.z + sn.z * pv.z; o.w = c.w * xv.w + sn.w * pv.w;
-    *(float4 *)(d.out + (int64_t)b * d.o_sb + (int64_t)h * d.o_sh + (int64_t)s * d.o_ss + j) = o;
+    const int64_t oo = (int64_t)b * d.o_sb + (int64_t)h * d.o_sh + (int64_t)s * d.o_ss + j;
+    *(float4 *)(d.out + oo) = o;
+    if (d.out16) *(uint2 *)(d.out16 + oo) = bf16_pack4(o);
   }
 }
 
@@ -352,7 +360,7 @@ hipError_t launch_rope(const LaunchCtx &lc, const RopeDesc &d) {
 // ---- gated activations --------------------------------------------------------------------------------
 template <bool GELU>
 __global__ void __launch_bounds__(256) glu_kernel(const float *gate, const float *up, float *out,
-                                                  uint64_t n4) {
+                                                  uint64_t n4, uint16_t *out16) {
   for (uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x; i < n4;
        i += (uint64_t)gridDim.x * 256) {
     const float4 g = ((const float4 *)gate)[i], u = ((const float4 *)up)[i];
@@ -365,17 +373,18 @@ __global__ void __launch_bounds__(256) glu_kernel(const float *gate, const float
       o.z = g.z * sigmoid_ref(g.z) * u.z; o.w = g.w * sigmoid_ref(g.w) * u.w;
     }
     ((float4 *)out)[i] = o;
+    if (out16) ((uint2 *)out16)[i] = bf16_pack4(o);
   }
 }
 
 hipError_t launch_glu(const LaunchCtx &lc, int gelu, const float *gate, const float *up, float *out,
-                      uint64_t n) {
+                      uint64_t n, uint16_t *out16) {
   if (!n) return hipSuccess;
   const uint64_t n4 = n / 4;
   uint64_t blocks = (n4 + 255) / 256, cap = (uint64_t)lc.n_cus * 8;
   const unsigned grid = (unsigned)(blocks < cap ? blocks : cap);
-  if (gelu) CG_LAUNCH(lc, (glu_kernel<true>), grid, 256, gate, up, out, n4);
-  else CG_LAUNCH(lc, (glu_kernel<false>), grid, 256, gate, up, out, n4);
+  if (gelu) CG_LAUNCH(lc, (glu_kernel<true>), grid, 256, gate, up, out, n4, out16);
+  else CG_LAUNCH(lc, (glu_kernel<false>), grid, 256, gate, up, out, n4, out16);
   return hipGetLastError();
 }
 

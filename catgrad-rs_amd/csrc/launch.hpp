@@ -87,6 +87,7 @@ struct RmsNormDesc {
   const float *x;        // rows of n contiguous floats, row r at x + r * x_row_stride
   const float *gamma;    // n floats or null
   const float *residual; // contiguous [rows, n] added to the result, or null
+  uint16_t *y16;         // optional bf16 copy of y (the operand of the GEMMs that follow), or null
   float *y;              // contiguous [rows, n]
   int64_t x_row_stride;
   uint32_t rows, n;
@@ -98,6 +99,7 @@ struct SoftmaxDesc {
   const float *x;        // row r at x + r * x_row_stride, unit stride along the row
   const float *mask;     // or null; row r reads mask + (r / mask_rows) * group + (r % mask_rows) * row
   float *y;              // contiguous [rows, n]
+  uint16_t *y16;         // optional bf16 copy of y (vector kernels only), or null
   int64_t x_row_stride, mask_group_stride, mask_row_stride, mask_col_stride;
   uint32_t rows, n, mask_rows;
   int32_t has_scale, has_mask_const;
@@ -110,12 +112,13 @@ struct RopeDesc {
   float *out;            // [b, h, s, dim] through o_sb / o_sh / o_ss (e.g. a slot of the KV cache)
   int64_t x_sb, x_sh, x_ss, cs_ss;  // element strides (unit stride along dim everywhere)
   int64_t o_sb, o_sh, o_ss;
+  uint16_t *out16;       // optional bf16 copy, same layout as out, or null
   uint32_t b, h, s, dim, half;
 };
 hipError_t launch_rope(const LaunchCtx &lc, const RopeDesc &d);
 // out = silu(gate) * up (gelu = 0) or gelu(gate) * up (gelu = 1); contiguous, n % 4 == 0
 hipError_t launch_glu(const LaunchCtx &lc, int gelu, const float *gate, const float *up, float *out,
-                      uint64_t n);
+                      uint64_t n, uint16_t *out16 = nullptr);  // out16: optional bf16 copy of out
 // op: 0 add, 1 sub, 2 mul, 3 div; b is contiguous (b_period = 0) or a vector of b_period floats
 // repeated; n % 4 == 0, b_period % 4 == 0
 hipError_t launch_binary_f32(const LaunchCtx &lc, int op, const float *a, const float *b, float *out,

@@ -844,6 +844,21 @@ void finish_fused(cg_tensor *n) {
   drop_inputs(n);
 }
 
+// In bf16 mode the results of the pattern kernels of a prefill (many rows) are the operands of
+// the GEMMs that follow: the kernel writes the bf16 copy the GEMM would otherwise make with a
+// pass of its own.  The copy becomes the twin of n's freshly allocated storage.
+int twin_for_result(cg_backend *be, cg_tensor *n, uint16_t **out) {
+  *out = nullptr;
+  if (!(be->flags & CG_FLAG_BF16) || n->rank < 2 || n->stype != ST_F32 || n->offset != 0) return CG_OK;
+  const int64_t cols = n->shape[n->rank - 1];
+  if (cols % 8 || n->size() / std::max<int64_t>(cols, 1) < 32 || n->st->shadow || n->st->bytes % 32) return CG_OK;
+  Storage *sh = nullptr;
+  if (dev_alloc(be, n->st->bytes / 2, &sh) != CG_OK) return CG_OK;  // no room: the GEMM will narrow it later
+  n->st->shadow = sh;
+  *out = (uint16_t *)sh->ptr;
+  return CG_OK;
+}
+
 // nn::softmax (stdlib/nn/mod.rs:162-171) with attention's `/ sqrt(d)` and `+ mask` in front:
 // pure matching, nothing is realised.  src is the tensor the scale / mask / softmax apply to.
 struct SoftmaxMatch {
@@ -951,10 +966,11 @@ int try_softmax(cg_backend *be, cg_tensor *root, bool *done) {
   if (!st) {
     d.x = (const float *)data_ptr(xs);
     d.y = (float *)root->st->ptr;
+    st = twin_for_result(be, root, &d.y16);
     d.x_row_stride = row_stride;
     d.rows = (uint32_t)(root->size() / n);
     d.n = (uint32_t)n;
-    KernelScope ks(be, "softmax_fused", (double)root->size() * 8, 0);
+    KernelScope ks(be, "softmax_fused", (double)root->size() * (d.y16 ? 10 : 8), 0);
     hipError_t e = launch_softmax(be->lc(), d);
     if (e != hipSuccess) st = fail(be, CG_ERR_DEVICE, hipGetErrorString(e));
   }
@@ -1072,7 +1088,8 @@ int try_rmsnorm(cg_backend *be, cg_tensor *root, bool *done) {
     d.rows = (uint32_t)(root->size() / n);
     d.n = (uint32_t)n;
     d.residual = rs ? (const float *)data_ptr(rs) : nullptr;
-    KernelScope ks(be, "rmsnorm_fused", (double)root->size() * (rs ? 12 : 8) + n * 4, 0);
+    if (!residual) st = twin_for_result(be, root, &d.y16);  // a residual stream feeds no GEMM directly
+    KernelScope ks(be, "rmsnorm_fused", (double)root->size() * (rs ? 12 : 8) + (d.y16 ? 2.0 * root->size() : 0.0) + n * 4, 0);
     hipError_t e = launch_rmsnorm(be->lc(), d);
     if (e != hipSuccess) st = fail(be, CG_ERR_DEVICE, hipGetErrorString(e));
   }
@@ -1134,7 +1151,7 @@ int rope_operands(cg_backend *be, const RopeMatch &m, bool *ok) {
 // Launches the rope kernel for `root` (matched as m) into `out` with the given element strides.
 // *done = false: layout requirements not met, nothing was launched.
 int rope_into(cg_backend *be, cg_tensor *root, const RopeMatch &m, float *out, const int64_t *o_strides,
-              const char *name, bool *done) {
+              const char *name, bool *done, uint16_t *out16 = nullptr) {
   bool tables = false;
   TRY(rope_operands(be, m, &tables));
   if (!tables) return CG_OK;
@@ -1155,6 +1172,7 @@ int rope_into(cg_backend *be, cg_tensor *root, const RopeMatch &m, float *out, c
   d.cos = (const float *)data_ptr(cb);
   d.sin = (const float *)data_ptr(sb);
   d.out = out;
+  d.out16 = out16;
   d.x_sb = xs->strides[0];
   d.x_sh = xs->strides[1];
   d.x_ss = xs->strides[2];
@@ -1188,7 +1206,9 @@ int try_rope(cg_backend *be, cg_tensor *root, bool *done) {
   if (!tables) return CG_OK;
   TRY(alloc_result(be, root, ST_F32));
   bool launched = false;
-  int st = rope_into(be, root, m, (float *)root->st->ptr, root->strides, "rope_fused", &launched);
+  uint16_t *y16 = nullptr;
+  TRY(twin_for_result(be, root, &y16));
+  int st = rope_into(be, root, m, (float *)root->st->ptr, root->strides, "rope_fused", &launched, y16);
   if (st || !launched) {
     storage_release(root->st);
     root->st = nullptr;
@@ -1266,8 +1286,10 @@ int try_glu(cg_backend *be, cg_tensor *root, bool *done) {
   if (!st) st = alloc_result(be, root, ST_F32);
   if (!st) {
     KernelScope ks(be, gelu ? "geglu_fused" : "swiglu_fused", (double)root->size() * 12, 0);
+    uint16_t *y16 = nullptr;
+    (void)twin_for_result(be, root, &y16);
     hipError_t e = launch_glu(be->lc(), gelu, (const float *)data_ptr(gc), (const float *)data_ptr(uc),
-                              (float *)root->st->ptr, (uint64_t)root->size());
+                              (float *)root->st->ptr, (uint64_t)root->size(), y16);
     if (e != hipSuccess) st = fail(be, CG_ERR_DEVICE, hipGetErrorString(e));
   }
   node_release(gc);
@@ -2532,7 +2554,14 @@ int cg_backend_create(int device, uint32_t flags, cg_backend **out) {
   return CG_OK;
 }
 
-void cg_backend_destroy(cg_backend *be) { backend_release(be); }
+void cg_backend_destroy(cg_backend *be) {
+  if (!be) return;
+  // cached nodes hold references to the backend: drop them first
+  std::map<int64_t, cg_tensor *> cache;
+  cache.swap(be->arange_cache);
+  for (auto &kv : cache) node_release(kv.second);
+  backend_release(be);
+}
 const char *cg_last_error(const cg_backend *be) { return be ? be->err.c_str() : ""; }
 const char *cg_backend_name(const cg_backend *) { return "hip-gfx950"; }
 
@@ -2902,6 +2931,19 @@ int cg_arange(cg_backend *be, size_t end, cg_tensor **out) {
   if (!be || !out) return CG_ERR_ARG;
   int64_t shape[1] = {(int64_t)end};
   if (end == 1) return finish(be, const_node(be, CG_U32, 1, shape, 0u), out);
+  if (!(be->flags & CG_FLAG_EAGER) && end <= ((size_t)1 << 20)) {
+    auto it = be->arange_cache.find((int64_t)end);
+    if (it != be->arange_cache.end()) {
+      *out = retain(it->second);
+      return CG_OK;
+    }
+    if (be->arange_cache.size() < 32) {
+      cg_tensor *n = new_node(be, CG_U32, 1, shape);
+      n->op = N_ARANGE;
+      be->arange_cache[(int64_t)end] = retain(n);
+      return finish(be, n, out);
+    }
+  }
   cg_tensor *n = new_node(be, CG_U32, 1, shape);
   n->op = N_ARANGE;
   return finish(be, n, out);

@@ -114,6 +114,9 @@ struct cg_backend {
   // issued as one launch; weak references, removed when a node is realised or deleted
   std::vector<cg_tensor *> gemv_candidates;
   hipEvent_t cur_start = nullptr, cur_stop = nullptr;  // set while a traced launch is issued
+  // arange(n) is immutable and models ask for the same few n over and over (masks, RoPE tables of
+  // every layer): one node per n, realised once
+  std::map<int64_t, cg_tensor *> arange_cache;
   // recycled pinned buffers (PREFETCH_BYTES each) and events of cg_tensor_prefetch
   std::vector<void *> pinned_pool;
   std::vector<hipEvent_t> event_pool;
