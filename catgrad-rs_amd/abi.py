@@ -105,6 +105,7 @@ _SIGNATURES = {
     "cg_params_destroy": (None, [_P]),
     "cg_params_set": (C.c_int, [_P, C.c_char_p, _P]),
     "cg_interp_eval": (C.c_int, [_P, _P, _P, _P, C.POINTER(cg_value), _SZ, C.POINTER(cg_value), _SZ, _U32P]),
+    "cg_interp_eval_owned": (C.c_int, [_P, _P, _P, _P, C.POINTER(cg_value), _SZ, C.POINTER(cg_value), _SZ, _U32P]),
     "cg_interp_last_error": (C.c_char_p, []),
     "cg_interp_backend_calls": (C.c_uint64, [C.c_int]),
 }

@@ -602,12 +602,22 @@ int cg_params_set(cg_params *p, const char *path, cg_tensor *t) {
   return CG_OK;
 }
 
-int cg_interp_eval(cg_backend *be, const cg_env *env, const cg_params *params, cg_term *term,
-                   const cg_value *args, size_t n_args, cg_value *results, size_t n_results,
-                   uint32_t *err_id) {
-  if (!be || !term) return ierr(CG_ERR_ARG, "eval: null backend or term");
-  if (n_results != term->targets.size())
+static int eval_entry(cg_backend *be, const cg_env *env, const cg_params *params, cg_term *term,
+                      const cg_value *args, size_t n_args, cg_value *results, size_t n_results,
+                      uint32_t *err_id, bool owned) {
+  auto give_back = [&]() {  // an owned call consumes its tensor arguments on every path
+    if (owned)
+      for (size_t i = 0; i < n_args; ++i)
+        if (args[i].kind == CG_VAL_TENSOR && args[i].tensor) cg_tensor_release(args[i].tensor);
+  };
+  if (!be || !term) {
+    give_back();
+    return ierr(CG_ERR_ARG, "eval: null backend or term");
+  }
+  if (n_results != term->targets.size()) {
+    give_back();
     return ierr(CG_ERR_ARITY, "eval: result buffer does not match the term's targets");
+  }
   std::vector<Value> a(n_args), r;
   for (size_t i = 0; i < n_args; ++i) {
     a[i].kind = args[i].kind;
@@ -615,12 +625,17 @@ int cg_interp_eval(cg_backend *be, const cg_env *env, const cg_params *params, c
     a[i].dtype = args[i].dtype;
     a[i].rank = args[i].rank;
     std::memcpy(a[i].dims, args[i].dims, sizeof(a[i].dims));
-    a[i].tensor = args[i].kind == CG_VAL_TENSOR ? cg_tensor_retain(args[i].tensor) : nullptr;
+    a[i].tensor = args[i].kind != CG_VAL_TENSOR ? nullptr
+                  : owned                       ? args[i].tensor
+                                                : cg_tensor_retain(args[i].tensor);
   }
   Ctx cx{be, env, params};
   int st = eval_term(cx, term, a, r);
   if (err_id) *err_id = cx.err_id;
-  if (st) return st;
+  if (st) {
+    for (Value &v : a) drop(v);  // whatever the failed run did not consume
+    return st;
+  }
   for (size_t i = 0; i < n_results; ++i) {
     std::memset(&results[i], 0, sizeof(cg_value));
     results[i].kind = r[i].kind;
@@ -631,6 +646,18 @@ int cg_interp_eval(cg_backend *be, const cg_env *env, const cg_params *params, c
     results[i].tensor = r[i].tensor;
   }
   return CG_OK;
+}
+
+int cg_interp_eval(cg_backend *be, const cg_env *env, const cg_params *params, cg_term *term,
+                   const cg_value *args, size_t n_args, cg_value *results, size_t n_results,
+                   uint32_t *err_id) {
+  return eval_entry(be, env, params, term, args, n_args, results, n_results, err_id, false);
+}
+
+int cg_interp_eval_owned(cg_backend *be, const cg_env *env, const cg_params *params, cg_term *term,
+                         const cg_value *args, size_t n_args, cg_value *results, size_t n_results,
+                         uint32_t *err_id) {
+  return eval_entry(be, env, params, term, args, n_args, results, n_results, err_id, true);
 }
 
 const char *cg_interp_last_error(void) { return g_err.c_str(); }

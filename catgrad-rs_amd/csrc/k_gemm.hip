@@ -859,30 +859,34 @@ __global__ void __launch_bounds__(256) gemv_pro_kernel(GemvProDesc g) {
   __shared__ float lds[4];
   __shared__ float part[4][R];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const uint32_t K = g.m.K;
+  const uint32_t K = g.m.K, bz = blockIdx.z;
+  const float *ga = g.a + (int64_t)bz * g.a_bstride;
+  const float *gaux = g.aux ? g.aux + (int64_t)bz * g.aux_bstride : nullptr;
   // ---- prologue: the input row
   if (g.pro == PRO_RMSNORM) {
     float ss = 0.f;
     for (uint32_t k = tid * 4; k < K; k += 1024) {
-      const float4 v = *(const float4 *)(g.a + k);
+      const float4 v = *(const float4 *)(ga + k);
       ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
     }
     ss = block_reduce<256, false>(ss, lds);
     const float rms = sqrtf(ss / g.n_as_float + g.eps);
     for (uint32_t k = tid * 4; k < K; k += 1024) {
-      const float4 v = *(const float4 *)(g.a + k);
+      const float4 v = *(const float4 *)(ga + k);
       float4 o;
       o.x = v.x / rms; o.y = v.y / rms; o.z = v.z / rms; o.w = v.w / rms;
-      if (g.aux) {
-        const float4 gm = *(const float4 *)(g.aux + k);
+      if (gaux) {
+        const float4 gm = *(const float4 *)(gaux + k);
         o.x *= g.gamma_offset + gm.x; o.y *= g.gamma_offset + gm.y;
         o.z *= g.gamma_offset + gm.z; o.w *= g.gamma_offset + gm.w;
       }
       *(float4 *)(xs + k) = o;
     }
+  } else if (g.pro == PRO_NONE) {
+    for (uint32_t k = tid * 4; k < K; k += 1024) *(float4 *)(xs + k) = *(const float4 *)(ga + k);
   } else {
     for (uint32_t k = tid * 4; k < K; k += 1024) {
-      const float4 a = *(const float4 *)(g.a + k), u = *(const float4 *)(g.aux + k);
+      const float4 a = *(const float4 *)(ga + k), u = *(const float4 *)(gaux + k);
       float4 o;
       if (g.pro == PRO_GEGLU) {
         o.x = gelu_ref(a.x) * u.x; o.y = gelu_ref(a.y) * u.y;
@@ -898,9 +902,17 @@ __global__ void __launch_bounds__(256) gemv_pro_kernel(GemvProDesc g) {
   // ---- the products
   const uint32_t N = g.m.p[blockIdx.y].N;
   const TB *B = (const TB *)g.m.p[blockIdx.y].b;
+  if (g.b_index) {
+    uint32_t ix = g.b_index[(int64_t)bz * g.b_index_stride];
+    if (ix >= g.b_index_limit) {  // the reference's select() panics; flag it and stay in bounds
+      atomicOr(g.err, ERRF_INDEX_OOB);
+      ix = g.b_index_limit - 1;
+    }
+    B += (int64_t)ix * g.sb_index;
+  }
   const int64_t sbn = g.m.p[blockIdx.y].sbn;
-  float *C = g.m.p[blockIdx.y].c;
-  const float *Cadd = g.m.p[blockIdx.y].c_add;
+  float *C = g.m.p[blockIdx.y].c + (uint64_t)bz * N;
+  const float *Cadd = g.m.p[blockIdx.y].c_add ? g.m.p[blockIdx.y].c_add + (uint64_t)bz * N : nullptr;
   const uint32_t slot = KSPLIT ? blockIdx.x : blockIdx.x * 4 + wave;
   const uint32_t n_slots = KSPLIT ? gridDim.x : gridDim.x * 4;
   uint32_t k_begin = 0, k_end = K;
@@ -969,9 +981,10 @@ static void launch_gemv_pro_block(const LaunchCtx &lc, const GemvProDesc &g, uin
   // rows cost more to recompute, so fewer workgroups each take several column pairs.
   const uint32_t per_wg = KSPLIT ? 1 : 4;
   uint32_t blocks = (slots + per_wg - 1) / per_wg;
-  const uint32_t cap = (uint32_t)lc.n_cus * (g.m.K >= 4096 ? 2 : 4) / g.m.n_prob;
+  const uint32_t batch = g.batch ? g.batch : 1;
+  const uint32_t cap = (uint32_t)lc.n_cus * (g.m.K >= 4096 ? 2 : 4) / (g.m.n_prob * batch);
   if (blocks > cap) blocks = cap ? cap : 1;
-  dim3 grid(blocks, g.m.n_prob);
+  dim3 grid(blocks, g.m.n_prob, batch);
   CG_LAUNCH(lc, (gemv_pro_kernel<TB, KSPLIT>), grid, 256, g);
 }
 

@@ -197,12 +197,23 @@ hipError_t launch_gemv_multi(const LaunchCtx &lc, const GemvMultiDesc &g);
 //   PRO_RMSNORM: x = a / sqrt(sum(a*a) / n + eps) * (gamma_offset + gamma)   (gamma may be null)
 //   PRO_SWIGLU / PRO_GEGLU: x = silu(a) * aux  /  gelu(a) * aux
 // K <= GEMV_PRO_MAX_K, K % 8 == 0; a, aux, gamma contiguous, 16-byte aligned
-enum { PRO_RMSNORM = 1, PRO_SWIGLU = 2, PRO_GEGLU = 3, GEMV_PRO_MAX_K = 8192 };
+//   PRO_NONE: x = a (staged once per workgroup)
+// Batched form (the routed experts of a MoE layer, models/qwen3.rs:104-123): batch z has its own
+// input row (a + z * a_bstride, aux + z * aux_bstride), its own output rows (c + z * N) and reads
+// the weight matrices of expert b_index[z * b_index_stride] (b + index * sb_index); an index >=
+// b_index_limit raises ERRF_INDEX_OOB in *err and is clamped.
+enum { PRO_NONE = 0, PRO_RMSNORM = 1, PRO_SWIGLU = 2, PRO_GEGLU = 3, GEMV_PRO_MAX_K = 8192 };
 struct GemvProDesc {
   GemvMultiDesc m;  // m.x is ignored
   int32_t pro;
   const float *a, *aux;
   float n_as_float, eps, gamma_offset;
+  uint32_t batch;   // 0 or 1: a single row
+  int64_t a_bstride, aux_bstride;
+  const uint32_t *b_index;
+  int64_t b_index_stride, sb_index;
+  uint32_t b_index_limit;
+  uint32_t *err;
 };
 hipError_t launch_gemv_pro(const LaunchCtx &lc, const GemvProDesc &g);
 // wrapping u32 matmul (ndarray's generic dot); all operands contiguous

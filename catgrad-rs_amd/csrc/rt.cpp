@@ -1668,6 +1668,7 @@ int bf16_shadow(cg_backend *be, Storage *st, Storage **out) {
 // the index vector and read W[idx[s]] in place.
 struct ExpertPeel {
   cg_tensor *w = nullptr, *idx = nullptr;  // retained, realised
+  int64_t idx_stride = 1;                  // elements between consecutive indices
   ~ExpertPeel() {
     node_release(w);
     node_release(idx);
@@ -1690,14 +1691,25 @@ int peel_expert_index(cg_backend *be, cg_tensor *n, ExpertPeel *out) {
   if (w->strides[2] != 1 && w->strides[1] != 1) return CG_OK;
   // indices of any rank are read flattened (ndarray.rs:373-381); a strided view needs one stride
   TRY(realize(be, idx));
+  // one stride between consecutive (flattened) indices: a column of the [S, k] top-k result
+  int64_t stride = 1, expect = -1;
+  bool uniform = true;
+  for (int i = idx->rank - 1; i >= 0; --i) {
+    if (idx->shape[i] == 1) continue;
+    if (expect < 0) stride = idx->strides[i];
+    else if (idx->strides[i] != expect) uniform = false;
+    expect = idx->strides[i] * idx->shape[i];
+  }
   cg_tensor *flat = nullptr;
-  if (idx->rank == 1) {
+  if (uniform) {
     flat = retain(idx);
   } else {
     TRY(contiguous(be, idx, &flat));
+    stride = 1;
   }
   out->w = retain(w);
   out->idx = flat;
+  out->idx_stride = stride;
   return CG_OK;
 }
 
@@ -1903,6 +1915,142 @@ int try_gemv_prologue(cg_backend *be, cg_tensor *n, cg_tensor *addend, bool *add
   return CG_OK;
 }
 
+// The routed experts of a MoE layer as the reference emits them (models/qwen3.rs:104-123), per slot:
+//   g = matmul(x[S,1,H], T(index(0, idx, Wg)));  u = matmul(x, T(index(0, idx, Wu)))
+//   y = matmul(silu(g) * u, T(index(0, idx, Wd)))
+// g and u go out as one launch (two problems sharing the staged input rows); the SwiGLU runs in the
+// prologue of the down product.  Every workgroup stages the row of its token in LDS once and
+// reads the weight rows of that token's expert in place (no gather of expert matrices).
+struct ExpertOperand {
+  cg_tensor *w = nullptr, *idx = nullptr;  // the stacked matrices [E, N, K] and the index tensor
+};
+
+bool match_expert_operand(const cg_tensor *t, int64_t S, ExpertOperand *o) {
+  if (t->op != N_TRANSPOSE || refs(t) != 1 || t->rank != 3 ||
+      !((t->p0 == 1 && t->p1 == 2) || (t->p0 == 2 && t->p1 == 1)))
+    return false;
+  const cg_tensor *g = t->in[0];
+  if (g->op != N_INDEX || refs(g) != 1 || g->p0 != 0 || g->rank != 3) return false;
+  if (g->in[1]->size() != S || g->in[0]->shape[0] == 0) return false;
+  o->w = g->in[0];
+  o->idx = g->in[1];
+  return true;
+}
+
+int try_moe_gemv(cg_backend *be, cg_tensor *n, bool *done) {
+  if (n->rank != 3 || n->shape[1] != 1 || !n->gemv_candidate || n->size() == 0) return CG_OK;
+  const int64_t S = n->shape[0];
+  ExpertOperand eo;
+  if (!match_expert_operand(n->in[1], S, &eo)) return CG_OK;
+  cg_tensor *A = n->in[0];
+  const int64_t K = A->shape[2];
+  if (A->rank != 3 || K % 8 || K < 64 || K > GEMV_PRO_MAX_K || S > 65535) return CG_OK;
+  cg_tensor *gate = nullptr, *up = nullptr;
+  int gelu = 0, pro = PRO_NONE;
+  if (A->op != N_REAL && refs(A) == 1 && match_glu(A, &gate, &up, &gelu)) pro = gelu ? PRO_GEGLU : PRO_SWIGLU;
+  // siblings: other deferred expert products of the same rows by the same indices (gate and up)
+  std::vector<cg_tensor *> members{n};
+  std::vector<ExpertOperand> ops{eo};
+  if (pro == PRO_NONE)
+    for (cg_tensor *c : be->gemv_candidates) {
+      if (c == n || c->op != N_MATMUL || c->in[0] != A || c->rank != 3 || c->shape[0] != S || members.size() >= 4) continue;
+      ExpertOperand co;
+      if (!match_expert_operand(c->in[1], S, &co) || co.idx != eo.idx) continue;
+      members.push_back(c);
+      ops.push_back(co);
+    }
+  // index vector: one stride between consecutive indices
+  cg_tensor *idx = eo.idx;
+  TRY(realize(be, idx));
+  int64_t istride = 1, expect = -1;
+  for (int i = idx->rank - 1; i >= 0; --i) {
+    if (idx->shape[i] == 1) continue;
+    if (expect < 0) istride = idx->strides[i];
+    else if (idx->strides[i] != expect) return CG_OK;
+    expect = idx->strides[i] * idx->shape[i];
+  }
+  if (idx->dtype != CG_U32) return CG_OK;
+  int b_stype = -1;
+  for (auto &o : ops) {
+    cg_tensor *w = o.w;
+    TRY(realize(be, w));
+    if (w->shape[2] != K || w->strides[2] != 1 || (w->stype != ST_F32 && w->stype != ST_BF16)) return CG_OK;
+    if (b_stype >= 0 && (w->stype != b_stype || w->shape[0] != ops[0].w->shape[0] || w->strides[0] != ops[0].w->strides[0]))
+      return CG_OK;
+    b_stype = w->stype;
+    const int q = 16 / esize(w->stype);
+    if ((uintptr_t)data_ptr(w) % 16 || w->strides[1] % q || w->strides[0] % q) return CG_OK;
+  }
+  // input rows
+  cg_tensor *a0 = nullptr, *a1 = nullptr;
+  int64_t a_bs = 0, aux_bs = 0;
+  if (pro == PRO_NONE) {
+    TRY(realize(be, A));
+    if (A->stype != ST_F32 || A->strides[2] != 1 || A->strides[0] % 4 || (uintptr_t)data_ptr(A) % 16) return CG_OK;
+    a0 = retain(A);
+    a_bs = A->strides[0];
+  } else {
+    TRY(contiguous(be, gate, &a0));
+    int st = contiguous(be, up, &a1);
+    if (st) {
+      node_release(a0);
+      return st;
+    }
+    if (a0->stype != ST_F32 || a1->stype != ST_F32 || (uintptr_t)data_ptr(a0) % 16 || (uintptr_t)data_ptr(a1) % 16) {
+      node_release(a0);
+      node_release(a1);
+      return CG_OK;
+    }
+    a_bs = aux_bs = K;
+  }
+  GemvProDesc d;
+  std::memset(&d, 0, sizeof(d));
+  d.pro = pro;
+  d.a = (const float *)data_ptr(a0);
+  d.aux = a1 ? (const float *)data_ptr(a1) : nullptr;
+  d.batch = (uint32_t)S;
+  d.a_bstride = a_bs;
+  d.aux_bstride = aux_bs;
+  d.b_index = (const uint32_t *)data_ptr(idx);
+  d.b_index_stride = istride;
+  d.sb_index = ops[0].w->strides[0];
+  d.b_index_limit = (uint32_t)ops[0].w->shape[0];
+  d.err = be->d_words;
+  d.m.K = (uint32_t)K;
+  d.m.b_stype = b_stype;
+  double bytes = (double)S * K * 4 * (pro == PRO_NONE ? 1 : 2), flops = 0;
+  int st = CG_OK;
+  for (size_t i = 0; i < members.size() && !st; ++i) {
+    cg_tensor *w = ops[i].w, *c = members[i];
+    st = alloc_result(be, c, ST_F32);
+    if (st) break;
+    auto &pr = d.m.p[d.m.n_prob++];
+    pr.b = data_ptr(w);
+    pr.c = (float *)c->st->ptr;
+    pr.c_add = nullptr;
+    pr.sbn = w->strides[1];
+    pr.N = (uint32_t)w->shape[1];
+    bytes += (double)S * pr.N * K * esize(w->stype) + (double)S * pr.N * 4;
+    flops += 2.0 * S * pr.N * K;
+  }
+  if (!st) {
+    const char *base = b_stype == ST_BF16 ? "gemv_experts_bf16" : "gemv_experts_f32";
+    KernelScope ks(be, base, bytes, flops);
+    hipError_t e = launch_gemv_pro(be->lc(), d);
+    if (e != hipSuccess) st = fail(be, CG_ERR_DEVICE, hipGetErrorString(e));
+  }
+  node_release(a0);
+  node_release(a1);
+  if (st) return st;
+  for (cg_tensor *c : members) {
+    forget_gemv_candidate(c);
+    c->op = N_REAL;
+    drop_inputs(c);
+  }
+  *done = true;
+  return CG_OK;
+}
+
 // `addend` (optional; realised, f32, contiguous, shaped like n) is added in the epilogue when a
 // one-row kernel runs the product; *added tells the caller whether that happened.
 int realize_matmul(cg_backend *be, cg_tensor *n, cg_tensor *addend = nullptr, bool *added = nullptr) {
@@ -1913,6 +2061,8 @@ int realize_matmul(cg_backend *be, cg_tensor *n, cg_tensor *addend = nullptr, bo
   }
   if (n->dtype == CG_F32 && n->gemv_candidate && !(be->flags & CG_FLAG_NO_PATTERNS)) {
     bool done = false;
+    if (!addend) TRY(try_moe_gemv(be, n, &done));
+    if (done) return CG_OK;
     TRY(try_gemv_prologue(be, n, addend, added, &done));
     if (done) return CG_OK;
   }
@@ -2064,7 +2214,7 @@ int realize_matmul(cg_backend *be, cg_tensor *n, cg_tensor *addend = nullptr, bo
     }
     if (ex.w) {
       g.b_index = (const uint32_t *)data_ptr(ex.idx);
-      g.b_index_stride = ex.idx->rank == 1 ? ex.idx->strides[0] : 1;
+      g.b_index_stride = ex.idx_stride;
       g.sb_index = ex.w->strides[0];
       g.b_index_limit = (uint32_t)ex.w->shape[0];
       g.err = be->d_words;
@@ -2187,6 +2337,10 @@ int realize_concat(cg_backend *be, cg_tensor *n) {
   const int plain = n->dtype == CG_F32 ? ST_F32 : ST_U32;
   const bool in_place = xd > 0 && yd > 0 && refs(x) == 1 && x->st->rc.load() == 1 && x->st->grow_dim == dim &&
                         xd + yd <= x->st->grow_cap && x->offset == 0 && x->stype == plain;
+  if (getenv("CG_DEBUG_CONCAT"))
+    fprintf(stderr, "concat dim %d xd %lld yd %lld refs(x) %d st.rc %d grow_dim %d cap %lld off %lld stype %d in_place %d\n", dim,
+            (long long)xd, (long long)yd, refs(x), x->st->rc.load(), x->st->grow_dim, (long long)x->st->grow_cap,
+            (long long)x->offset, x->stype, (int)in_place);
   // the new key rows arrive through apply_rope_embedding: rotate them straight into the cache slot
   RopeMatch rope;
   const bool rope_y = in_place && !(be->flags & CG_FLAG_NO_PATTERNS) && y->op != N_REAL && refs(y) == 1 &&

@@ -111,8 +111,11 @@ class Interpreter:
             self._params_len = len(self.parameters)
         return self._params_handle
 
-    def run(self, term, args):
-        """Interpreter::run: `args` are Tensor / Nat / Dtype / Shape values; returns the same."""
+    def run(self, term, args, moved=()):
+        """Interpreter::run: `args` are Tensor / Nat / Dtype / Shape values; returns the same.
+        `moved`: positions of tensor arguments given away, as the Rust `run` takes its values by
+        value: those Tensor objects are empty afterwards (KV-cache tensors are passed this way so
+        that the step may append to them in place)."""
         assert isinstance(term, Term)
         lib = self.backend.lib
         h = term.compile(lib)
@@ -122,6 +125,10 @@ class Interpreter:
             v = cargs[i]
             if isinstance(a, abi.Tensor):
                 v.kind, v.tensor = VAL_TENSOR, a.ptr
+                if i in moved:
+                    a.ptr = None                    # the evaluator takes over this reference
+                else:
+                    lib.cg_tensor_retain(v.tensor)  # the owned call consumes one reference per tensor
             elif isinstance(a, Shape) or isinstance(a, (tuple, list)):
                 v.kind, v.rank = VAL_SHAPE, len(a)
                 for j, d in enumerate(a):
@@ -132,7 +139,8 @@ class Interpreter:
                 v.kind, v.nat = VAL_NAT, int(a)
         res = (abi.cg_value * max(n_out, 1))()
         err_id = C.c_uint32(0)
-        st = lib.cg_interp_eval(self.backend.ptr, self.environment.handle(lib).ptr,
+        moved = frozenset(moved)
+        st = lib.cg_interp_eval_owned(self.backend.ptr, self.environment.handle(lib).ptr,
                                 self._params().ptr, h.ptr, cargs, len(args), res, n_out,
                                 C.byref(err_id))
         if st:

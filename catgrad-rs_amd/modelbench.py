@@ -86,7 +86,10 @@ class _Runner:
 
     def step(self, tok):
         ids = self.be.reshape(tok, [self.batch, 1])
-        out = self.it.run(self.decode_term, [ids, self.pos, self.cos, self.sin] + self.kv)
+        # the cache tensors are given away (Interpreter::run takes its values by value): the step may
+        # then append to them in place
+        out = self.it.run(self.decode_term, [ids, self.pos, self.cos, self.sin] + self.kv,
+                          moved=range(4, 4 + len(self.kv)))
         self.kv = out[2:]
         self.pos += 1
         return out[0], out[1]

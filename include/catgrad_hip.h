@@ -238,6 +238,13 @@ int cg_params_set(cg_params *p, const char *path, cg_tensor *t);
 int cg_interp_eval(cg_backend *be, const cg_env *env, const cg_params *params, cg_term *term,
                    const cg_value *args, size_t n_args, cg_value *results, size_t n_results,
                    uint32_t *err_id);
+/* The same, taking its values by value as Interpreter::run does (interpreter.rs:33-37): the caller's
+ * reference to every tensor argument passes to the evaluator, on success and on failure.  A cache
+ * tensor handed over this way is owned by nobody else while the term runs, which is what lets
+ * `concat(2, cache, new)` append in place even when an op inside the term forces evaluation. */
+int cg_interp_eval_owned(cg_backend *be, const cg_env *env, const cg_params *params, cg_term *term,
+                         const cg_value *args, size_t n_args, cg_value *results, size_t n_results,
+                         uint32_t *err_id);
 /* message of the last failed cg_interp_eval / cg_term_* call in this thread */
 const char *cg_interp_last_error(void);
 /* counts Backend calls issued by cg_interp_eval since the last reset (per thread) */
