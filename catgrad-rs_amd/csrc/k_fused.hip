@@ -249,6 +249,29 @@ __global__ void __launch_bounds__(512) attn_decode_kernel(AttnDecodeDesc a) {
       qv.z = c.z * qv.z + sn.z * pv.z; qv.w = c.w * qv.w + sn.w * pv.w;
     }
   }
+  // this step's own key / value row: from the projections, not from the cache
+  const bool has_new = a.k_new != nullptr;
+  const uint32_t t_new = has_new ? a.t_new : 0xFFFFFFFFu;
+  float4 knew = make_float4(0.f, 0.f, 0.f, 0.f), vnew = knew;
+  if (has_new && live) {
+    const float *kn = a.k_new + (int64_t)b * a.kn_sb + (int64_t)kv * a.kn_skv;
+    const uint32_t j = sub * 4;
+    knew = *(const float4 *)(kn + j);
+    if (a.kn_cos) {
+      const uint32_t half = a.d / 2;
+      const bool lo = j < half;
+      float4 pv = *(const float4 *)(kn + (lo ? j + half : j - half));
+      if (lo) { pv.x = -pv.x; pv.y = -pv.y; pv.z = -pv.z; pv.w = -pv.w; }
+      const float4 c = *(const float4 *)(a.kn_cos + j), sn = *(const float4 *)(a.kn_sin + j);
+      knew.x = c.x * knew.x + sn.x * pv.x; knew.y = c.y * knew.y + sn.y * pv.y;
+      knew.z = c.z * knew.z + sn.z * pv.z; knew.w = c.w * knew.w + sn.w * pv.w;
+    }
+    vnew = *(const float4 *)(a.v_new + (int64_t)b * a.vn_sb + (int64_t)kv * a.vn_skv + j);
+    if (rp == 0 && wave == 0 && kg == 0) {  // one writer per (batch, kv head)
+      *(float4 *)(const_cast<float *>(K) + (int64_t)t_new * a.k_st + j) = knew;
+      *(float4 *)(const_cast<float *>(V) + (int64_t)t_new * a.v_st + j) = vnew;
+    }
+  }
   const uint32_t first = wave * KPW + kg;
   // phase 1: scores and their maximum
   float mx = -3.40282347e+38f;
@@ -257,7 +280,9 @@ __global__ void __launch_bounds__(512) attn_decode_kernel(AttnDecodeDesc a) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const uint32_t t = t0 + u * STRIDE;
-      kr[u] = (live && t < a.t) ? *(const float4 *)(K + (int64_t)t * a.k_st + sub * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
+      kr[u] = (t == t_new) ? knew
+              : (live && t < a.t) ? *(const float4 *)(K + (int64_t)t * a.k_st + sub * 4)
+                                  : make_float4(0.f, 0.f, 0.f, 0.f);
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -289,7 +314,9 @@ __global__ void __launch_bounds__(512) attn_decode_kernel(AttnDecodeDesc a) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const uint32_t t = t0 + u * STRIDE;
-      vr[u] = (live && t < a.t) ? *(const float4 *)(V + (int64_t)t * a.v_st + sub * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
+      vr[u] = (t == t_new) ? vnew
+              : (live && t < a.t) ? *(const float4 *)(V + (int64_t)t * a.v_st + sub * 4)
+                                  : make_float4(0.f, 0.f, 0.f, 0.f);
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {

@@ -139,6 +139,13 @@ struct AttnDecodeDesc {
   // optional: q is the projection before apply_rope_embedding; the kernel rotates it with this
   // position's cos / sin rows (d floats each, half-split) as it loads it
   const float *q_cos, *q_sin;
+  // optional: the key / value rows of this step are not in the cache yet.  Row t_new (= t - 1) of
+  // K and V is taken from k_new / v_new ([b, kv, d] through the strides; k_new is rotated with
+  // kn_cos / kn_sin when those are set) and the first head of every kv group also stores both rows
+  // into the cache (k and v are written through in that case).
+  const float *k_new, *v_new, *kn_cos, *kn_sin;
+  int64_t kn_sb, kn_skv, vn_sb, vn_skv;
+  uint32_t t_new;
 };
 enum { ATTN_DECODE_MAX_T = 8192, ATTN_DECODE_MAX_D = 256 };
 hipError_t launch_attn_decode(const LaunchCtx &lc, const AttnDecodeDesc &d);

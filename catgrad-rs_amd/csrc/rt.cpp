@@ -1717,6 +1717,87 @@ int peel_expert_index(cg_backend *be, cg_tensor *n, ExpertPeel *out) {
 //   matmul(softmax(matmul(q, K^T) / sqrt(d) + mask), V)
 // in one launch that reads K and V rows in place from the cache; the [b, h, 1, T] scores and
 // probabilities never exist in HBM.
+// The cache update of a decode step, `concat(2, cached, new)` (legacy/models/utils.rs:222-223), seen
+// from the attention that reads it: the node under the repeat_kv chain of a K or V operand.
+cg_tensor *kv_concat_under(cg_tensor *t) {
+  if (t->op == N_TRANSPOSE && refs(t) == 1 && t->rank == 4 &&
+      ((t->p0 == 2 && t->p1 == 3) || (t->p0 == 3 && t->p1 == 2)))
+    t = t->in[0];
+  if (t->op != N_RESHAPE || refs(t) != 1 || t->rank != 4) return nullptr;
+  cg_tensor *u = t->in[0];
+  if (u->op != N_BROADCAST || refs(u) != 1 || u->rank != 5) return nullptr;
+  cg_tensor *r5 = u->in[0];
+  if (r5->op != N_RESHAPE || refs(r5) != 1 || r5->rank != 5 || r5->shape[2] != 1) return nullptr;
+  cg_tensor *c = r5->in[0];
+  if (c->op != N_CONCAT || c->p0 != 2 || c->rank != 4 || c->dtype != CG_F32) return nullptr;
+  return c;
+}
+
+// One new row per (batch, kv head) to be appended in place by the attention kernel itself.
+struct RowAppend {
+  cg_tensor *concat = nullptr;
+  cg_tensor *src = nullptr;  // retained: the tensor the rows are read from
+  const float *cos = nullptr, *sin = nullptr;
+  cg_tensor *cos_t = nullptr, *sin_t = nullptr;  // retained
+  ~RowAppend() {
+    node_release(src);
+    node_release(cos_t);
+    node_release(sin_t);
+  }
+};
+
+// Checks that `c` can be appended to in place and that its new rows can be read by the kernel;
+// realises what has to exist for that (the cache, the projection) but changes nothing.
+int row_append_candidate(cg_backend *be, cg_tensor *c, bool allow_rope, RowAppend *out, bool *ok) {
+  *ok = false;
+  cg_tensor *x = c->in[0], *y = c->in[1];
+  if (y->shape[2] != 1 || x->shape[2] < 1) return CG_OK;
+  TRY(realize(be, x));
+  const int64_t xd = x->shape[2];
+  if (!(refs(x) == 1 && x->st->rc.load() == 1 && x->st->grow_dim == 2 && xd + 1 <= x->st->grow_cap &&
+        x->offset == 0 && x->stype == ST_F32))
+    return CG_OK;
+  if (x->strides[3] != 1 || x->strides[0] % 4 || x->strides[1] % 4 || x->strides[2] % 4 ||
+      (uintptr_t)data_ptr(x) % 16)
+    return CG_OK;
+  cg_tensor *src = y;
+  RopeMatch rm;
+  if (allow_rope && y->op != N_REAL && refs(y) == 1 && match_rope(y, &rm)) {
+    bool tables = false;
+    TRY(rope_operands(be, rm, &tables));
+    if (!tables) return CG_OK;
+    src = rm.x;
+    out->cos_t = retain(rm.cb);
+    out->sin_t = retain(rm.sb);
+    out->cos = (const float *)data_ptr(rm.cb);
+    out->sin = (const float *)data_ptr(rm.sb);
+  } else {
+    TRY(realize(be, y));
+  }
+  if (src->stype != ST_F32 || src->strides[3] != 1 || src->strides[0] % 4 || src->strides[1] % 4 ||
+      (uintptr_t)data_ptr(src) % 16)
+    return CG_OK;
+  out->concat = c;
+  out->src = retain(src);
+  *ok = true;
+  return CG_OK;
+}
+
+// The bookkeeping half of realize_concat's in-place append; the rows themselves are stored by
+// the kernel launched right after.
+void commit_row_append(cg_tensor *c) {
+  cg_tensor *x = c->in[0];
+  c->st = x->st;
+  c->st->rc.fetch_add(1);
+  storage_release(c->st->shadow);
+  c->st->shadow = nullptr;
+  c->stype = ST_F32;
+  c->offset = 0;
+  std::memcpy(c->strides, x->strides, sizeof(c->strides));
+  c->op = N_REAL;
+  drop_inputs(c);
+}
+
 int try_attn_decode(cg_backend *be, cg_tensor *n, bool *done) {
   cg_tensor *P = n->in[0];
   if (P->op == N_REAL || refs(P) != 1 || P->rank != 4) return CG_OK;
@@ -1727,6 +1808,29 @@ int try_attn_decode(cg_backend *be, cg_tensor *n, bool *done) {
   const int64_t T = S->shape[3], d = n->shape[3], heads = n->shape[1], nb = n->shape[0];
   if (T < 1 || T > ATTN_DECODE_MAX_T || d > ATTN_DECODE_MAX_D || d % 4 || n->in[1]->shape[2] != T) return CG_OK;
   if (S->in[0]->shape[3] != d) return CG_OK;
+  // This step's cache update, when both K and V are `concat(2, cached, new)` that can be done in
+  // place: the kernel takes the new rows from the projections and stores them itself.
+  RowAppend ka, va;
+  bool fused_append = false;
+  {
+    cg_tensor *ck = kv_concat_under(S->in[1]), *cv = kv_concat_under(n->in[1]);
+    if (ck && cv && ck != cv && ck->shape[2] == T && cv->shape[2] == T && T >= 2) {
+      bool okk = false, okv = false;
+      TRY(row_append_candidate(be, ck, true, &ka, &okk));
+      if (okk) TRY(row_append_candidate(be, cv, false, &va, &okv));
+      if (okk && okv) {
+        commit_row_append(ck);
+        commit_row_append(cv);
+        fused_append = true;
+      }
+    }
+  }
+  // from here on a fused append must end in the launch: its rows exist nowhere else
+#define ATTN_BAIL()                                                                            \
+  do {                                                                                         \
+    if (fused_append) return fail(be, CG_ERR_INTERNAL, "attention: cache rows left unwritten"); \
+    return CG_OK;                                                                              \
+  } while (0)
   MatOperand Kop, Vop;
   bool pk = false, pv = false;
   TRY(peel_repeat_kv(be, S->in[1], &Kop, &pk));
@@ -1743,6 +1847,7 @@ int try_attn_decode(cg_backend *be, cg_tensor *n, bool *done) {
     o->rank = 5;
     return CG_OK;
   };
+  if (fused_append && (!pk || !pv)) ATTN_BAIL();
   if (!pk) TRY(unpeeled(S->in[1], &Kop));
   if (!pv) TRY(unpeeled(n->in[1], &Vop));
   cg_tensor *q = S->in[0];
@@ -1768,12 +1873,13 @@ int try_attn_decode(cg_backend *be, cg_tensor *n, bool *done) {
     return true;
   };
   // K as [b, kv, rep, d, T] (the transposed view), V as [b, kv, rep, T, d]
-  if (Kop.shape[2] != Vop.shape[2] || Kop.shape[1] != Vop.shape[1] || Kop.shape[1] * Kop.shape[2] != heads) return CG_OK;
-  if (q->stype != ST_F32 || Kop.t->stype != ST_F32 || Vop.t->stype != ST_F32) return CG_OK;
+  if (Kop.shape[2] != Vop.shape[2] || Kop.shape[1] != Vop.shape[1] || Kop.shape[1] * Kop.shape[2] != heads) ATTN_BAIL();
+  if (q->stype != ST_F32 || Kop.t->stype != ST_F32 || Vop.t->stype != ST_F32) ATTN_BAIL();
   if (!rows_ok(data_ptr(q), q->strides[3], {q->strides[0], q->strides[1]}) ||
       !rows_ok(data_ptr(Kop.t), Kop.strides[3], {Kop.strides[0], Kop.strides[1], Kop.strides[2], Kop.strides[4]}) ||
       !rows_ok(data_ptr(Vop.t), Vop.strides[4], {Vop.strides[0], Vop.strides[1], Vop.strides[2], Vop.strides[3]}))
-    return CG_OK;
+    ATTN_BAIL();
+#undef ATTN_BAIL
   TRY(alloc_result(be, n, ST_F32));
   AttnDecodeDesc a;
   std::memset(&a, 0, sizeof(a));
@@ -1796,6 +1902,17 @@ int try_attn_decode(cg_backend *be, cg_tensor *n, bool *done) {
   a.mask_const = m.mask_const;
   a.q_cos = q_cos;
   a.q_sin = q_sin;
+  if (fused_append) {
+    a.k_new = (const float *)data_ptr(ka.src);
+    a.v_new = (const float *)data_ptr(va.src);
+    a.kn_cos = ka.cos;
+    a.kn_sin = ka.sin;
+    a.kn_sb = ka.src->strides[0];
+    a.kn_skv = ka.src->strides[1];
+    a.vn_sb = va.src->strides[0];
+    a.vn_skv = va.src->strides[1];
+    a.t_new = (uint32_t)(T - 1);
+  }
   {
     const double kv_bytes = 2.0 * nb * Kop.shape[1] * T * d * 4;
     KernelScope ks(be, "attn_decode", kv_bytes + 2.0 * nb * heads * d * 4, 4.0 * nb * heads * T * d);
