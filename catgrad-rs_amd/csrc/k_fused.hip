@@ -219,9 +219,9 @@ hipError_t launch_softmax(const LaunchCtx &lc, const SoftmaxDesc &d) {
 // query row per head.  One workgroup per (batch, head); LPK lanes share a key/value row (16 bytes
 // each), so a wave covers 64 / LPK rows per load.  Scores live in LDS between the three phases
 // (dot products + max, exp + sum, weighted sum of V rows); nothing of size T goes to HBM.
-template <int LPK>
-__global__ void __launch_bounds__(512) attn_decode_kernel(AttnDecodeDesc a) {
-  constexpr int BLOCK = 512, NW = BLOCK / 64;
+template <int LPK, int BLOCK>
+__global__ void __launch_bounds__(BLOCK) attn_decode_kernel(AttnDecodeDesc a) {
+  constexpr int NW = BLOCK / 64;
   constexpr int KPW = 64 / LPK;       // rows per wave per load
   constexpr int STRIDE = NW * KPW;    // rows per workgroup per load
   constexpr int U = 4;                // independent row loads in flight per lane
@@ -340,9 +340,16 @@ __global__ void __launch_bounds__(512) attn_decode_kernel(AttnDecodeDesc a) {
 hipError_t launch_attn_decode(const LaunchCtx &lc, const AttnDecodeDesc &d) {
   if (!d.b || !d.heads || !d.d) return hipSuccess;
   dim3 grid(d.heads, d.b);
-  if (d.d <= 64) CG_LAUNCH(lc, (attn_decode_kernel<16>), grid, 512, d);
-  else if (d.d <= 128) CG_LAUNCH(lc, (attn_decode_kernel<32>), grid, 512, d);
-  else CG_LAUNCH(lc, (attn_decode_kernel<64>), grid, 512, d);
+  // long caches: more rows in flight per workgroup
+  if (d.t > 256) {
+    if (d.d <= 64) CG_LAUNCH(lc, (attn_decode_kernel<16, 1024>), grid, 1024, d);
+    else if (d.d <= 128) CG_LAUNCH(lc, (attn_decode_kernel<32, 1024>), grid, 1024, d);
+    else CG_LAUNCH(lc, (attn_decode_kernel<64, 1024>), grid, 1024, d);
+  } else {
+    if (d.d <= 64) CG_LAUNCH(lc, (attn_decode_kernel<16, 512>), grid, 512, d);
+    else if (d.d <= 128) CG_LAUNCH(lc, (attn_decode_kernel<32, 512>), grid, 512, d);
+    else CG_LAUNCH(lc, (attn_decode_kernel<64, 512>), grid, 512, d);
+  }
   return hipGetLastError();
 }
 

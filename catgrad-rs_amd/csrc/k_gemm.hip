@@ -851,7 +851,9 @@ hipError_t launch_gemv_multi(const LaunchCtx &lc, const GemvMultiDesc &g) {
 // spread over all CUs) and then streams its share of the weight rows exactly like
 // gemv_multi_kernel, reading x from LDS.  KSPLIT: the four waves of a workgroup share a column
 // pair and take a quarter of k each (deep, narrow matrices).
-template <typename TB, bool KSPLIT>
+// GLUEPI (two problems of equal N, no k-split): a wave computes column n of both and stores
+// act(first) * second, i.e. gate_proj, up_proj and the SwiGLU / GeGLU between them in one pass.
+template <typename TB, bool KSPLIT, bool GLUEPI>
 __global__ void __launch_bounds__(256) gemv_pro_kernel(GemvProDesc g) {
   typedef typename WVec<TB>::type VT;
   constexpr int EPL = WVec<TB>::EPL, UNROLL = 4, R = 2;
@@ -902,6 +904,8 @@ __global__ void __launch_bounds__(256) gemv_pro_kernel(GemvProDesc g) {
   // ---- the products
   const uint32_t N = g.m.p[blockIdx.y].N;
   const TB *B = (const TB *)g.m.p[blockIdx.y].b;
+  const TB *B2 = GLUEPI ? (const TB *)g.m.p[1].b : nullptr;
+  const int64_t sbn2 = GLUEPI ? g.m.p[1].sbn : 0;
   if (g.b_index) {
     uint32_t ix = g.b_index[(int64_t)bz * g.b_index_stride];
     if (ix >= g.b_index_limit) {  // the reference's select() panics; flag it and stay in bounds
@@ -921,7 +925,8 @@ __global__ void __launch_bounds__(256) gemv_pro_kernel(GemvProDesc g) {
     k_begin = min(K, wave * per);
     k_end = min(K, k_begin + per);
   }
-  for (uint32_t nb = slot * R; nb < N; nb += n_slots * R) {  // uniform per workgroup when KSPLIT
+  constexpr int CPS = GLUEPI ? 1 : R;  // output columns per slot
+  for (uint32_t nb = slot * CPS; nb < N; nb += n_slots * CPS) {  // uniform per workgroup when KSPLIT
     float acc[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) acc[r] = 0.f;
@@ -932,8 +937,13 @@ __global__ void __launch_bounds__(256) gemv_pro_kernel(GemvProDesc g) {
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
           const uint32_t k = k0 + u * 64 * EPL;
-          if (k < k_end && nb + r < N)
+          if (GLUEPI) {
+            if (k < k_end)
+              q[r][u] = __builtin_nontemporal_load(
+                  (const VT *)((r == 0 ? B + (int64_t)nb * sbn : B2 + (int64_t)nb * sbn2) + k));
+          } else if (k < k_end && nb + r < N) {
             q[r][u] = __builtin_nontemporal_load((const VT *)(B + (int64_t)(nb + r) * sbn + k));
+          }
         }
 #pragma unroll
       for (int u = 0; u < UNROLL; ++u) {
@@ -947,7 +957,7 @@ __global__ void __launch_bounds__(256) gemv_pro_kernel(GemvProDesc g) {
           }
 #pragma unroll
           for (int r = 0; r < R; ++r) {
-            if (nb + r < N) {
+            if (GLUEPI || nb + r < N) {
               float w[EPL];
               WVec<TB>::widen(q[r][u], w);
 #pragma unroll
@@ -959,7 +969,10 @@ __global__ void __launch_bounds__(256) gemv_pro_kernel(GemvProDesc g) {
     }
 #pragma unroll
     for (int r = 0; r < R; ++r) acc[r] = wave_sum(acc[r]);
-    if (KSPLIT) {
+    if (GLUEPI) {
+      if (lane == 0)
+        C[nb] = (g.glu_epilogue == PRO_GEGLU ? gelu_ref(acc[0]) : acc[0] * sigmoid_ref(acc[0])) * acc[1];
+    } else if (KSPLIT) {
       __syncthreads();
       if (lane == 0)
 #pragma unroll
@@ -985,13 +998,28 @@ static void launch_gemv_pro_block(const LaunchCtx &lc, const GemvProDesc &g, uin
   const uint32_t cap = (uint32_t)lc.n_cus * (g.m.K >= 4096 ? 2 : 4) / (g.m.n_prob * batch);
   if (blocks > cap) blocks = cap ? cap : 1;
   dim3 grid(blocks, g.m.n_prob, batch);
-  CG_LAUNCH(lc, (gemv_pro_kernel<TB, KSPLIT>), grid, 256, g);
+  CG_LAUNCH(lc, (gemv_pro_kernel<TB, KSPLIT, false>), grid, 256, g);
+}
+
+template <typename TB>
+static void launch_gemv_pro_glu(const LaunchCtx &lc, const GemvProDesc &g) {
+  const uint32_t slots = g.m.p[0].N;  // one (gate, up) column pair per wave pass
+  uint32_t blocks = (slots + 3) / 4;
+  const uint32_t cap = (uint32_t)lc.n_cus * 4;
+  if (blocks > cap) blocks = cap;
+  CG_LAUNCH(lc, (gemv_pro_kernel<TB, false, true>), dim3(blocks, 1, 1), 256, g);
 }
 
 hipError_t launch_gemv_pro(const LaunchCtx &lc, const GemvProDesc &g) {
   uint32_t max_n = 0;
   for (int i = 0; i < g.m.n_prob; ++i) max_n = g.m.p[i].N > max_n ? g.m.p[i].N : max_n;
   if (!max_n || !g.m.n_prob) return hipSuccess;
+  if (g.glu_epilogue) {
+    if (g.m.n_prob != 2 || g.m.p[0].N != g.m.p[1].N || g.batch > 1 || g.b_index) return hipErrorInvalidValue;
+    if (g.m.b_stype == ST_BF16) launch_gemv_pro_glu<uint16_t>(lc, g);
+    else launch_gemv_pro_glu<float>(lc, g);
+    return hipGetLastError();
+  }
   const uint32_t slots = (max_n + 1) / 2;
   const bool ksplit = g.m.K >= 4096 && slots * (uint32_t)g.m.n_prob <= (uint32_t)lc.n_cus * 8;
   if (g.m.b_stype == ST_BF16) {

@@ -215,6 +215,9 @@ struct GemvProDesc {
   int32_t pro;
   const float *a, *aux;
   float n_as_float, eps, gamma_offset;
+  // 0, or PRO_SWIGLU / PRO_GEGLU: two problems of equal N (gate, up); a single output
+  // p[0].c[n] = act(x . gate_n) * (x . up_n) replaces the two product vectors
+  int32_t glu_epilogue;
   uint32_t batch;   // 0 or 1: a single row
   int64_t a_bstride, aux_bstride;
   const uint32_t *b_index;

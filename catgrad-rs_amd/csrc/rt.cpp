@@ -1925,6 +1925,83 @@ int try_attn_decode(cg_backend *be, cg_tensor *n, bool *done) {
   return CG_OK;
 }
 
+// h = act(gate_proj(x)) * up_proj(x) with one input row (models/llama.rs:11-35): both products and the
+// activation in one launch, a wave computing column n of gate and of up (and x itself from its
+// RMSNorm when nothing else reads the normed row).  `glu` is the deferred act(g) * u node; on
+// success it becomes a realised tensor and g, u are never materialised.
+int try_gate_up_glu(cg_backend *be, cg_tensor *glu, cg_tensor *g, cg_tensor *u, int gelu, bool *done) {
+  if (g->op != N_MATMUL || u->op != N_MATMUL || !g->gemv_candidate || !u->gemv_candidate) return CG_OK;
+  if (refs(g) != (gelu ? 3 : 2) || refs(u) != 1 || g->in[0] != u->in[0] || g->size() != u->size()) return CG_OK;
+  cg_tensor *X = g->in[0];
+  const int64_t K = X->shape[X->rank - 1], N = g->shape[g->rank - 1];
+  if (X->size() != K || g->size() != N || K % 8 || K < 256 || K > GEMV_PRO_MAX_K || glu->size() != N) return CG_OK;
+  cg_tensor *ws[2] = {g->in[1], u->in[1]};
+  for (cg_tensor *w : ws) {
+    TRY(realize(be, w));
+    if (w->rank < 2 || w->shape[w->rank - 2] != K || w->strides[w->rank - 2] != 1) return CG_OK;
+    for (int i = 0; i + 2 < w->rank; ++i)
+      if (w->shape[i] != 1) return CG_OK;
+    if ((w->stype != ST_F32 && w->stype != ST_BF16) || w->stype != ws[0]->stype) return CG_OK;
+    if ((uintptr_t)data_ptr(w) % 16 || w->strides[w->rank - 1] % (16 / esize(w->stype))) return CG_OK;
+  }
+  GemvProDesc d;
+  std::memset(&d, 0, sizeof(d));
+  RmsNormMatch rm;
+  cg_tensor *a0 = nullptr, *a1 = nullptr;
+  if (X->op != N_REAL && refs(X) == 2 && match_rmsnorm(X, &rm)) {
+    bool vec = true;
+    if (rm.gamma) TRY(gamma_row_vector(be, rm.gamma, &vec));
+    TRY(realize(be, rm.x));
+    if (vec && rm.x->stype == ST_F32 && is_contiguous(rm.x) && (uintptr_t)data_ptr(rm.x) % 16 == 0) {
+      d.pro = PRO_RMSNORM;
+      a0 = retain(rm.x);
+      if (rm.gamma) a1 = retain(rm.gamma);
+      d.n_as_float = rm.n_as_float;
+      d.eps = rm.eps;
+      d.gamma_offset = rm.gamma_offset;
+    }
+  }
+  if (!a0) {
+    TRY(contiguous(be, X, &a0));
+    if (a0->stype != ST_F32 || (uintptr_t)data_ptr(a0) % 16) {
+      node_release(a0);
+      return CG_OK;
+    }
+    d.pro = PRO_NONE;
+  }
+  int st = alloc_result(be, glu, ST_F32);
+  if (!st) {
+    d.a = (const float *)data_ptr(a0);
+    d.aux = a1 ? (const float *)data_ptr(a1) : nullptr;
+    d.glu_epilogue = gelu ? PRO_GEGLU : PRO_SWIGLU;
+    d.m.K = (uint32_t)K;
+    d.m.b_stype = ws[0]->stype;
+    d.m.n_prob = 2;
+    for (int i = 0; i < 2; ++i) {
+      d.m.p[i].b = data_ptr(ws[i]);
+      d.m.p[i].c = (float *)glu->st->ptr;
+      d.m.p[i].sbn = ws[i]->strides[ws[i]->rank - 1];
+      d.m.p[i].N = (uint32_t)N;
+    }
+    const char *base = ws[0]->stype == ST_BF16 ? "gemv_rowdot_bf16" : "gemv_rowdot_f32";
+    KernelScope ks(be, base, 2.0 * N * K * esize(ws[0]->stype) + (double)K * 8 + (double)N * 4, 4.0 * N * K);
+    if (be->trace_shapes) {
+      char buf[96];
+      snprintf(buf, sizeof buf, "%s[%sgate*up,K%lld,N%lld]", base, d.pro == PRO_RMSNORM ? "rmsnorm+" : "", (long long)K,
+               (long long)(2 * N));
+      ks.rename(buf);
+    }
+    hipError_t e = launch_gemv_pro(be->lc(), d);
+    if (e != hipSuccess) st = fail(be, CG_ERR_DEVICE, hipGetErrorString(e));
+  }
+  node_release(a0);
+  node_release(a1);
+  if (st) return st;
+  finish_fused(glu);  // releases the activation chain and with it g and u
+  *done = true;
+  return CG_OK;
+}
+
 // q/k/v, gate/up and down_proj of a decode step: one-row products whose input row is an RMSNorm
 // or a SwiGLU/GeGLU of earlier values.  When every consumer of that row is such a product, the
 // row is computed inside the product kernel (launch_gemv_pro) and its node is never realised.
@@ -1939,6 +2016,13 @@ int try_gemv_prologue(cg_backend *be, cg_tensor *n, cg_tensor *addend, bool *add
   if (match_rmsnorm(A, &rm)) pro = PRO_RMSNORM;
   else if (match_glu(A, &gate, &up, &gelu)) pro = gelu ? PRO_GEGLU : PRO_SWIGLU;
   else return CG_OK;
+  if (pro != PRO_RMSNORM) {
+    // better still: the activation in the epilogue of the gate / up products themselves; A is
+    // then a row in memory and this product runs without a prologue
+    bool fused = false;
+    TRY(try_gate_up_glu(be, A, gate, up, gelu, &fused));
+    if (fused) return CG_OK;
+  }
   // the group: every deferred one-row product reading A (n first)
   std::vector<cg_tensor *> members{n};
   for (cg_tensor *c : be->gemv_candidates)
