@@ -12,7 +12,7 @@ import os
 import numpy as np
 
 F32, U32 = 0, 1
-FLAG_BF16, FLAG_EAGER, FLAG_NO_PATTERNS = 1, 2, 4
+FLAG_BF16, FLAG_EAGER, FLAG_NO_PATTERNS, FLAG_ATTN_ONE_PASS = 1, 2, 4, 8
 MAX_RANK = 8
 
 OK, ERR_SHAPE, ERR_DTYPE, ERR_ARG, ERR_DEVICE, ERR_OOM, ERR_ARITH, ERR_INTERNAL = range(8)

@@ -1,0 +1,269 @@
+// k_attn.hip — attention over many query rows (prefill) in one pass, bf16 MFMA, f32 accumulation.
+//
+// The op sequence of catgrad-llm/src/models/llama.rs:95-107 (also gemma3.rs:153-186):
+//   scores = matmul(q, transpose(k));  scores / sqrt(d);  + mask;  softmax;  matmul(., v)
+// materialises [b, h, S, T] twice on the generic path.  Here a workgroup takes 128 query rows of one
+// (batch, head) and walks the keys 64 at a time with the running maximum / sum of the row
+// (online softmax); scores and probabilities only ever exist in registers.
+//
+// Everything is computed transposed so that a lane owns one query for the whole kernel:
+//   S^T[key, query]   = K[key, :] . Q[query, :]       A = K tile (LDS), B = Q rows (registers)
+//   O^T[dim, query]  += V^T[dim, key] . P^T[key, query]  A = V^T tile (LDS), B = P^T (registers)
+// In the 32x32 MFMA result layout a lane holds column (lane & 31) = its query, so the row
+// statistics are in-lane reductions plus one exchange with lane ^ 32, the rescaling of O by
+// exp(m_old - m_new) is a per-lane scalar, and P^T feeds the second product straight from the
+// registers of the first: the key order inside each 16-key block is permuted the same way for
+// both operands (a lane's eight values are keys {4h..4h+3, 8+4h..8+4h+3}, h = lane >> 5), which
+// the V^T fragment mirrors with two 8-byte LDS reads.
+#include <hip/hip_runtime.h>
+#include <math.h>
+#include "launch.hpp"
+#include "dev_common.hpp"
+
+namespace cgk {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 a_bf16x8;
+typedef __attribute__((ext_vector_type(16))) float a_f32x16;
+
+__device__ __forceinline__ a_bf16x8 pack8(const float *v) {
+  union {
+    uint32_t u[4];
+    a_bf16x8 h;
+  } r;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) r.u[i] = bf16_bits(v[2 * i]) | (bf16_bits(v[2 * i + 1]) << 16);
+  return r.h;
+}
+
+// BN keys per step; the K / V rows and the mask values of step i+1 are fetched into registers while
+// step i is being computed, so global latency is paid once per workgroup, not once per step.
+template <int D, int BN>
+__global__ void __launch_bounds__(256) attn_prefill_kernel(AttnPrefillDesc a) {
+  constexpr int KP = D + 8;              // K tile row pitch (bf16 elements)
+  constexpr int VP = BN + 8;             // V^T tile row pitch
+  constexpr int DT = D / 32;             // 32-row tiles of O^T
+  constexpr int KT = BN / 32;            // 32-key tiles of S^T
+  constexpr int KCH = BN * D / 4 / 256;  // float4 chunks of the K tile per thread
+  constexpr int VBL = (BN / 4) * (D / 4) / 256;  // 4 x 4 blocks of the V tile per thread
+  __shared__ __attribute__((aligned(16))) uint16_t Ks[BN * KP];
+  __shared__ __attribute__((aligned(16))) uint16_t Vt[D * VP];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int col = lane & 31, half = lane >> 5;
+  const uint32_t h = blockIdx.y, b = blockIdx.z;
+  const uint32_t kvh = h / a.rep, rp = h % a.rep;
+  const uint32_t query = blockIdx.x * 128 + wave * 32 + col;
+  const bool q_ok = query < a.s;
+  const uint32_t qc = q_ok ? query : a.s - 1;  // loads of lanes past the end go to a valid row
+  const float *Q = a.q + (int64_t)b * a.q_sb + (int64_t)h * a.q_sh + (int64_t)qc * a.q_ss;
+  const float *K = a.k + (int64_t)b * a.k_sb + (int64_t)kvh * a.k_skv + (int64_t)rp * a.k_srep;
+  const float *V = a.v + (int64_t)b * a.v_sb + (int64_t)kvh * a.v_skv + (int64_t)rp * a.v_srep;
+  const float *M = a.mask ? a.mask + (int64_t)b * a.m_sb + (int64_t)h * a.m_sh + (int64_t)qc * a.m_ss : nullptr;
+
+  // this lane's query row as B fragments: k-step ks covers dims 16 ks .. 16 ks + 15, half h takes 8
+  a_bf16x8 qf[D / 16];
+#pragma unroll
+  for (int ks = 0; ks < D / 16; ++ks) {
+    float v[8];
+    if (q_ok) {
+      const float4 x0 = *(const float4 *)(Q + ks * 16 + half * 8), x1 = *(const float4 *)(Q + ks * 16 + half * 8 + 4);
+      v[0] = x0.x; v[1] = x0.y; v[2] = x0.z; v[3] = x0.w; v[4] = x1.x; v[5] = x1.y; v[6] = x1.z; v[7] = x1.w;
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) v[i] = 0.f;
+    }
+    qf[ks] = pack8(v);
+  }
+  a_f32x16 o[DT];
+#pragma unroll
+  for (int t = 0; t < DT; ++t)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) o[t][e] = 0.f;
+  float m_run = -3.40282347e+38f, l_run = 0.f;
+  const float inv_scale = a.has_scale ? 1.0f / a.scale : 1.0f;  // bf16 mode: a product, not the reference's quotient
+
+  // registers of the step in flight
+  float4 kreg[KCH], vreg[VBL][4], mreg[KT][4];
+  // All loads are unconditional (indices clamped into range) so that they are issued back to back;
+  // rows past the end are zeroed when the registers are consumed.
+  auto fetch = [&](uint32_t t0) {
+#pragma unroll
+    for (int c = 0; c < KCH; ++c) {
+      const int ch = tid + c * 256, key = ch / (D / 4), d4 = (ch % (D / 4)) * 4;
+      kreg[c] = *(const float4 *)(K + (int64_t)min(t0 + key, a.t - 1) * a.k_st + d4);
+    }
+#pragma unroll
+    for (int c = 0; c < VBL; ++c) {
+      const int bl = tid + c * 256, k4 = (bl / (D / 4)) * 4, d4 = (bl % (D / 4)) * 4;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) vreg[c][i] = *(const float4 *)(V + (int64_t)min(t0 + k4 + i, a.t - 1) * a.v_st + d4);
+    }
+    if (M) {  // mask rows allow 16-byte loads and T % 4 == 0 (checked by the host)
+#pragma unroll
+      for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          mreg[kt][j] = *(const float4 *)(M + min(t0 + kt * 32 + j * 8 + half * 4, a.t - 4));
+    }
+  };
+  fetch(0);
+  for (uint32_t t0 = 0; t0 < a.t; t0 += BN) {
+    // ---- is any (query, key) pair of this step unmasked?  A causal or sliding-window mask kills
+    // most steps; a dead step only adds terms that the first live step rescales to zero.
+    bool live_pair = !M;
+    float4 mcur[KT][4];
+    if (M) {
+#pragma unroll
+      for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          mcur[kt][j] = mreg[kt][j];
+          const uint32_t key = t0 + kt * 32 + j * 8 + half * 4;
+          const float4 mk = mcur[kt][j];
+          if (q_ok && ((key < a.t && mk.x > -3.0e38f) || (key + 1 < a.t && mk.y > -3.0e38f) ||
+                       (key + 2 < a.t && mk.z > -3.0e38f) || (key + 3 < a.t && mk.w > -3.0e38f)))
+            live_pair = true;
+        }
+    }
+    const bool live = __syncthreads_or(live_pair);  // also: the previous step's fragments have been read
+    if (live) {
+      // ---- registers -> LDS: K [BN, D] and V^T [D, BN] as bf16 (V through a 4 x 4 register transpose)
+#pragma unroll
+      for (int c = 0; c < KCH; ++c) {
+        const int ch = tid + c * 256, key = ch / (D / 4), d4 = (ch % (D / 4)) * 4;
+        *(uint2 *)(&Ks[key * KP + d4]) = (t0 + key < a.t) ? bf16_pack4(kreg[c]) : make_uint2(0u, 0u);
+      }
+#pragma unroll
+      for (int c = 0; c < VBL; ++c) {
+        const int bl = tid + c * 256, k4 = (bl / (D / 4)) * 4, d4 = (bl % (D / 4)) * 4;
+        float4 r[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) r[i] = (t0 + k4 + i < a.t) ? vreg[c][i] : make_float4(0.f, 0.f, 0.f, 0.f);
+        *(uint2 *)(&Vt[(d4 + 0) * VP + k4]) = bf16_pack4(make_float4(r[0].x, r[1].x, r[2].x, r[3].x));
+        *(uint2 *)(&Vt[(d4 + 1) * VP + k4]) = bf16_pack4(make_float4(r[0].y, r[1].y, r[2].y, r[3].y));
+        *(uint2 *)(&Vt[(d4 + 2) * VP + k4]) = bf16_pack4(make_float4(r[0].z, r[1].z, r[2].z, r[3].z));
+        *(uint2 *)(&Vt[(d4 + 3) * VP + k4]) = bf16_pack4(make_float4(r[0].w, r[1].w, r[2].w, r[3].w));
+      }
+    }
+    __syncthreads();
+    if (t0 + BN < a.t) fetch(t0 + BN);  // in flight during the arithmetic below
+    if (!live) continue;
+    // ---- S^T = K . Q^T
+    a_f32x16 st[KT];
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt) {
+#pragma unroll
+      for (int e = 0; e < 16; ++e) st[kt][e] = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < D / 16; ++ks) {
+        const a_bf16x8 kf = *(const a_bf16x8 *)(&Ks[(kt * 32 + col) * KP + ks * 16 + half * 8]);
+        st[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ks], st[kt], 0, 0, 0);
+      }
+    }
+    // ---- scale, mask, running maximum.  Register e of tile kt is key t0 + kt*32 + (e>>2)*8 + half*4 + (e&3)
+    float tmax = -3.40282347e+38f;
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const uint32_t key = t0 + kt * 32 + j * 8 + half * 4;
+        float mv[4] = {0.f, 0.f, 0.f, 0.f};
+        if (M) { mv[0] = mcur[kt][j].x; mv[1] = mcur[kt][j].y; mv[2] = mcur[kt][j].z; mv[3] = mcur[kt][j].w; }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          float s = st[kt][j * 4 + i];
+          if (a.has_scale) s = s * inv_scale;
+          if (M) s = s + mv[i];
+          else if (a.has_mask_const) s = s + a.mask_const;
+          if (key + i >= a.t) s = -3.40282347e+38f;  // past the end: contributes exp(..) = 0
+          st[kt][j * 4 + i] = s;
+          tmax = fmaxf(tmax, s);
+        }
+      }
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+    const float m_new = fmaxf(m_run, tmax);
+    const float alpha = __expf(m_run - m_new);
+    float psum = 0.f;
+    a_bf16x8 pf[KT * 2];  // P^T as B fragments of the 16-key blocks
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+      for (int blk = 0; blk < 2; ++blk) {
+        float p[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const uint32_t key = t0 + kt * 32 + (blk * 2 + (i >> 2)) * 8 + half * 4 + (i & 3);
+          p[i] = key < a.t ? __expf(st[kt][blk * 8 + i] - m_new) : 0.f;
+          psum += p[i];
+        }
+        pf[kt * 2 + blk] = pack8(p);
+      }
+    psum += __shfl_xor(psum, 32, 64);
+    l_run = l_run * alpha + psum;
+    m_run = m_new;
+    // ---- O^T = O^T * alpha + V^T . P^T
+#pragma unroll
+    for (int t = 0; t < DT; ++t) {
+#pragma unroll
+      for (int e = 0; e < 16; ++e) o[t][e] *= alpha;
+#pragma unroll
+      for (int blk = 0; blk < KT * 2; ++blk) {
+        // A fragment: row = dim t*32 + col, the lane's eight keys of this block in the permuted order
+        const uint16_t *vr = &Vt[(t * 32 + col) * VP + blk * 16 + half * 4];
+        union {
+          uint2 u[2];
+          a_bf16x8 hv;
+        } vf;
+        vf.u[0] = *(const uint2 *)vr;
+        vf.u[1] = *(const uint2 *)(vr + 8);
+        o[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf.hv, pf[blk], o[t], 0, 0, 0);
+      }
+    }
+  }
+  // A row whose every key is masked has all scores equal to f32::MIN on the reference path:
+  // uniform weights, i.e. the mean of V.  Dead steps were skipped above, so rebuild that here.
+  if (M && q_ok && m_run <= -3.0e38f) {
+    l_run = (float)a.t;
+#pragma unroll
+    for (int t = 0; t < DT; ++t)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) o[t][e] = 0.f;
+    for (uint32_t key = 0; key < a.t; ++key)
+#pragma unroll
+      for (int t = 0; t < DT; ++t)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float4 vv = *(const float4 *)(V + (int64_t)key * a.v_st + t * 32 + j * 8 + half * 4);
+          o[t][j * 4 + 0] += vv.x; o[t][j * 4 + 1] += vv.y; o[t][j * 4 + 2] += vv.z; o[t][j * 4 + 3] += vv.w;
+        }
+  }
+  // ---- normalise and store: O^T register e of tile t is dim t*32 + (e>>2)*8 + half*4 + (e&3)
+  if (q_ok) {
+    float *out = a.out + (((int64_t)b * a.heads + h) * a.s + query) * D;
+    uint16_t *out16 = a.out16 ? a.out16 + (((int64_t)b * a.heads + h) * a.s + query) * D : nullptr;
+#pragma unroll
+    for (int t = 0; t < DT; ++t)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        float4 r;
+        r.x = o[t][j * 4 + 0] / l_run; r.y = o[t][j * 4 + 1] / l_run;
+        r.z = o[t][j * 4 + 2] / l_run; r.w = o[t][j * 4 + 3] / l_run;
+        const int dim = t * 32 + j * 8 + half * 4;
+        *(float4 *)(out + dim) = r;
+        if (out16) *(uint2 *)(out16 + dim) = bf16_pack4(r);
+      }
+  }
+}
+
+hipError_t launch_attn_prefill(const LaunchCtx &lc, const AttnPrefillDesc &d) {
+  if (!d.b || !d.heads || !d.s) return hipSuccess;
+  dim3 grid((d.s + 127) / 128, d.heads, d.b);
+  switch (d.d) {
+    case 64: CG_LAUNCH(lc, (attn_prefill_kernel<64, 64>), grid, 256, d); break;
+    case 128: CG_LAUNCH(lc, (attn_prefill_kernel<128, 64>), grid, 256, d); break;
+    case 256: CG_LAUNCH(lc, (attn_prefill_kernel<256, 32>), grid, 256, d); break;
+    default: return hipErrorInvalidValue;
+  }
+  return hipGetLastError();
+}
+
+}  // namespace cgk

@@ -150,6 +150,25 @@ struct AttnDecodeDesc {
 enum { ATTN_DECODE_MAX_T = 8192, ATTN_DECODE_MAX_D = 256 };
 hipError_t launch_attn_decode(const LaunchCtx &lc, const AttnDecodeDesc &d);
 
+// ---- k_attn.hip
+// Attention over s query rows per head (bf16 MFMA, online softmax):
+//   out[b, h, i, :] = softmax_j(q[b,h,i,:] . k[b,h,j,:] / scale + mask[b,h,i,j]) . v[b,h,j,:]
+// q, k, v: f32 with unit stride along d (k, v through the kv-head strides as in AttnDecodeDesc);
+// mask: additive f32 through its strides (0 = broadcast) or a constant; out contiguous [b, heads, s, d].
+struct AttnPrefillDesc {
+  const float *q, *k, *v, *mask;
+  float *out;
+  uint16_t *out16;                     // optional bf16 copy of out
+  int64_t q_sb, q_sh, q_ss;
+  int64_t k_sb, k_skv, k_srep, k_st;
+  int64_t v_sb, v_skv, v_srep, v_st;
+  int64_t m_sb, m_sh, m_ss, m_st;
+  uint32_t b, heads, rep, s, t, d;
+  int32_t has_scale, has_mask_const, m_vec;  // m_vec: mask rows allow 16-byte loads
+  float scale, mask_const;
+};
+hipError_t launch_attn_prefill(const LaunchCtx &lc, const AttnPrefillDesc &d);
+
 // ---- k_gemm.hip
 struct GemmDesc {
   const void *a, *b;

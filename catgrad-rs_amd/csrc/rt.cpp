@@ -1717,6 +1717,90 @@ int peel_expert_index(cg_backend *be, cg_tensor *n, ExpertPeel *out) {
 //   matmul(softmax(matmul(q, K^T) / sqrt(d) + mask), V)
 // in one launch that reads K and V rows in place from the cache; the [b, h, 1, T] scores and
 // probabilities never exist in HBM.
+// Attention over many query rows (prefill; models/llama.rs:95-107, gemma3.rs:153-186) in bf16 mode:
+//   matmul(softmax(matmul(q, K^T) / sqrt(d) + mask), V)
+// as one pass with online softmax (k_attn.hip); the [b, h, S, T] scores and probabilities are
+// never written.  f32 mode keeps the generic path (the 1e-4 bar wants f32 products).
+int try_attn_prefill(cg_backend *be, cg_tensor *n, bool *done) {
+  if (!(be->flags & CG_FLAG_BF16)) return CG_OK;
+  cg_tensor *P = n->in[0];
+  if (P->op == N_REAL || refs(P) != 1 || P->rank != 4) return CG_OK;
+  SoftmaxMatch m;
+  if (!match_softmax(P, &m)) return CG_OK;
+  cg_tensor *S = m.src;
+  if (S->op != N_MATMUL || S->rank != 4 || refs(S) != (S == m.x ? 2 : 1)) return CG_OK;
+  const int64_t Sq = S->shape[2], T = S->shape[3], d = n->shape[3], heads = n->shape[1], nb = n->shape[0];
+  if (Sq < 16 || T < 1 || (d != 64 && d != 128 && d != 256) || n->in[1]->shape[2] != T || S->in[0]->shape[3] != d)
+    return CG_OK;
+  // Below this the three-launch path (GEMM, softmax, GEMM) is as fast and the scores are small;
+  // above it the scores of one layer run to hundreds of MB.  CG_FLAG_ATTN_ONE_PASS lifts the threshold.
+  if (T < 1024 && !(be->flags & CG_FLAG_ATTN_ONE_PASS)) return CG_OK;
+  if (nb > 65535 || heads > 65535) return CG_OK;
+  MatOperand Kop, Vop;
+  bool pk = false, pv = false;
+  TRY(peel_repeat_kv(be, S->in[1], &Kop, &pk));
+  TRY(peel_repeat_kv(be, n->in[1], &Vop, &pv));
+  if (!pk || !pv) return CG_OK;  // operands get realised by the generic path below
+  cg_tensor *q = S->in[0];
+  TRY(realize(be, q));
+  cg_tensor *mask = m.mask;
+  if (mask) TRY(realize(be, mask));
+  auto ok4 = [](const void *ptr, int64_t unit, std::initializer_list<int64_t> strides) {
+    if (unit != 1 || (uintptr_t)ptr % 16) return false;
+    for (int64_t st : strides)
+      if (st % 4) return false;
+    return true;
+  };
+  if (Kop.shape[2] != Vop.shape[2] || Kop.shape[1] != Vop.shape[1] || Kop.shape[1] * Kop.shape[2] != heads) return CG_OK;
+  if (q->stype != ST_F32 || Kop.t->stype != ST_F32 || Vop.t->stype != ST_F32 || (mask && mask->stype != ST_F32)) return CG_OK;
+  if (!ok4(data_ptr(q), q->strides[3], {q->strides[0], q->strides[1], q->strides[2]}) ||
+      !ok4(data_ptr(Kop.t), Kop.strides[3], {Kop.strides[0], Kop.strides[1], Kop.strides[2], Kop.strides[4]}) ||
+      !ok4(data_ptr(Vop.t), Vop.strides[4], {Vop.strides[0], Vop.strides[1], Vop.strides[2], Vop.strides[3]}))
+    return CG_OK;
+  TRY(alloc_result(be, n, ST_F32));
+  AttnPrefillDesc a;
+  std::memset(&a, 0, sizeof(a));
+  a.q = (const float *)data_ptr(q);
+  a.k = (const float *)data_ptr(Kop.t);
+  a.v = (const float *)data_ptr(Vop.t);
+  a.out = (float *)n->st->ptr;
+  a.q_sb = q->strides[0]; a.q_sh = q->strides[1]; a.q_ss = q->strides[2];
+  a.k_sb = Kop.strides[0]; a.k_skv = Kop.strides[1]; a.k_srep = Kop.strides[2]; a.k_st = Kop.strides[4];
+  a.v_sb = Vop.strides[0]; a.v_skv = Vop.strides[1]; a.v_srep = Vop.strides[2]; a.v_st = Vop.strides[3];
+  if (mask) {
+    a.mask = (const float *)data_ptr(mask);
+    a.m_sb = mask->shape[0] == 1 ? 0 : mask->strides[0];
+    a.m_sh = mask->shape[1] == 1 ? 0 : mask->strides[1];
+    a.m_ss = mask->shape[2] == 1 ? 0 : mask->strides[2];
+    a.m_st = mask->shape[3] == 1 ? 0 : mask->strides[3];
+    a.m_vec = a.m_st == 1 && (uintptr_t)a.mask % 16 == 0 && a.m_sb % 4 == 0 && a.m_sh % 4 == 0 && a.m_ss % 4 == 0;
+  }
+  if (mask && (!a.m_vec || T % 4)) {  // the kernel reads mask rows 16 bytes at a time: generic path instead
+    storage_release(n->st);
+    n->st = nullptr;
+    return CG_OK;
+  }
+  a.b = (uint32_t)nb;
+  a.heads = (uint32_t)heads;
+  a.rep = (uint32_t)Kop.shape[2];
+  a.s = (uint32_t)Sq;
+  a.t = (uint32_t)T;
+  a.d = (uint32_t)d;
+  a.has_scale = m.has_scale;
+  a.scale = m.scale;
+  a.has_mask_const = m.has_mask_const;
+  a.mask_const = m.mask_const;
+  {
+    const double qo = 2.0 * nb * heads * Sq * d * 4, kvb = 2.0 * nb * Kop.shape[1] * T * d * 4;
+    KernelScope ks(be, "attn_prefill", qo + kvb + (mask ? (double)Sq * T * 4 : 0.0), 4.0 * nb * heads * Sq * T * d);
+    HIPCHK(be, launch_attn_prefill(be->lc(), a));
+  }
+  n->op = N_REAL;
+  drop_inputs(n);
+  *done = true;
+  return CG_OK;
+}
+
 // The cache update of a decode step, `concat(2, cached, new)` (legacy/models/utils.rs:222-223), seen
 // from the attention that reads it: the node under the repeat_kv chain of a K or V operand.
 cg_tensor *kv_concat_under(cg_tensor *t) {
@@ -2258,6 +2342,11 @@ int realize_matmul(cg_backend *be, cg_tensor *n, cg_tensor *addend = nullptr, bo
   if (!addend && n->dtype == CG_F32 && n->rank == 4 && n->shape[2] == 1 && !(be->flags & CG_FLAG_NO_PATTERNS)) {
     bool done = false;
     TRY(try_attn_decode(be, n, &done));
+    if (done) return CG_OK;
+  }
+  if (!addend && n->dtype == CG_F32 && n->rank == 4 && n->shape[2] >= 16 && !(be->flags & CG_FLAG_NO_PATTERNS)) {
+    bool done = false;
+    TRY(try_attn_prefill(be, n, &done));
     if (done) return CG_OK;
   }
   if (n->dtype == CG_F32 && n->gemv_candidate && !(be->flags & CG_FLAG_NO_PATTERNS)) {

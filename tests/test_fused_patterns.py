@@ -283,3 +283,51 @@ def test_rmsnorm_plus_residual(oracle, hip, hip_nopat, shape, order):
         h = raw * (lang.constant(b, 1.0, lang.shape(b, gm)) + gm)
         return rv + h if order == "res_first" else h + rv
     check(oracle, hip, hip_nopat, f, 1, [x, res], "rmsnorm_fused", params=p, rtol=1e-4, atol=1e-5)
+
+
+@pytest.fixture(scope="module")
+def hip_bf16_flash():
+    """bf16 mode with the one-pass attention kernel enabled for every length."""
+    import importlib
+    cg = importlib.import_module("catgrad-rs_amd")
+    return cg.Backend(cg.load_library(), flags=cg.abi.FLAG_BF16 | cg.abi.FLAG_ATTN_ONE_PASS)
+
+
+@pytest.mark.parametrize("cfg", [(1, 32, 8, 512, 64), (2, 4, 2, 100, 128), (1, 4, 1, 200, 256), (1, 8, 8, 33, 64),
+                                 (1, 2, 1, 1024, 64)])
+@pytest.mark.parametrize("mask_kind", ["causal", "window"])
+def test_attention_prefill_bf16(oracle, hip_bf16_flash, hip_bf16, hip_nopat, cfg, mask_kind):
+    """Attention over many query rows in bf16 mode: one launch with online softmax, scores never
+    stored; against the oracle (f32) at the bf16 bar and against the generic f32 path."""
+    import importlib
+    gemma3 = importlib.import_module("catgrad-rs_amd.llm.gemma3")
+    nb, H, KV, S, d = cfg
+    g = np.random.default_rng(S + d)
+    q = g.standard_normal((nb, H, S, d)).astype(np.float32)
+    k = g.standard_normal((nb, KV, S, d)).astype(np.float32)
+    v = g.standard_normal((nb, KV, S, d)).astype(np.float32)
+    model = gemma3.Gemma3Model(importlib.import_module("catgrad-rs_amd.llm").Config(), S)
+
+    def f(b, qv, kv, vv):
+        qv, kv, vv = qv + qv - qv, kv + kv - kv, vv + vv - vv      # computed f32 values
+        kr = helpers.repeat_kv(b, H // KV, kv)
+        vr = helpers.repeat_kv(b, H // KV, vv)
+        attn = lang.matmul(b, qv, lang.transpose(b, 2, 3, kr))
+        sh = lang.shape(b, attn)
+        attn = attn / lang.constant(b, float(np.sqrt(np.float32(d))), sh)
+        n = lang.to_nat(b, S)
+        mask = helpers.causal_mask(b, n) if mask_kind == "causal" else model.window_mask(b, n, 17)
+        attn = attn + lang.broadcast(b, mask, sh)
+        return lang.matmul(b, nn.softmax(b, attn), vr)
+    (ref,) = vectors.run(oracle, f, 1, q, k, v)
+    got, names = run_traced(hip_bf16_flash, f, 1, q, k, v)
+    (gen,) = vectors.run(hip_nopat, f, 1, q, k, v)
+    _, default_names = run_traced(hip_bf16, f, 1, q, k, v)
+    assert ("attn_prefill" in default_names) == (S >= 1024)
+    if S % 4 == 0:
+        assert "attn_prefill" in names and "softmax_fused" not in names, sorted(names)
+    else:       # mask rows are read 16 bytes at a time: other lengths take the three-launch path
+        assert "attn_prefill" not in names
+    scale = np.abs(ref).max()
+    assert np.max(np.abs(got[0] - ref)) <= 2e-2 * scale, np.max(np.abs(got[0] - ref)) / scale
+    assert np.max(np.abs(gen - ref)) <= 1e-4 * scale
