@@ -43,8 +43,7 @@ __global__ void __launch_bounds__(256) attn_prefill_kernel(AttnPrefillDesc a) {
   constexpr int VP = BN + 8;             // V^T tile row pitch
   constexpr int DT = D / 32;             // 32-row tiles of O^T
   constexpr int KT = BN / 32;            // 32-key tiles of S^T
-  constexpr int KCH = BN * D / 4 / 256;  // float4 chunks of the K tile per thread
-  constexpr int VBL = (BN / 4) * (D / 4) / 256;  // 4 x 4 blocks of the V tile per thread
+  constexpr int KCH = BN * D / 8 / 256;  // 16-byte chunks of the K tile / of the V^T tile per thread
   __shared__ __attribute__((aligned(16))) uint16_t Ks[BN * KP];
   __shared__ __attribute__((aligned(16))) uint16_t Vt[D * VP];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -55,7 +54,10 @@ __global__ void __launch_bounds__(256) attn_prefill_kernel(AttnPrefillDesc a) {
   const bool q_ok = query < a.s;
   const uint32_t qc = q_ok ? query : a.s - 1;  // loads of lanes past the end go to a valid row
   const float *Q = a.q + (int64_t)b * a.q_sb + (int64_t)h * a.q_sh + (int64_t)qc * a.q_ss;
-  const float *K = a.k + (int64_t)b * a.k_sb + (int64_t)kvh * a.k_skv + (int64_t)rp * a.k_srep;
+  // K rows as bf16 (the twin of the rotated keys), V as bf16 V^T [b, kv, d, T]: both were narrowed
+  // once, not once per query block
+  const uint16_t *K = a.k16 + (int64_t)b * a.k_sb + (int64_t)kvh * a.k_skv + (int64_t)rp * a.k_srep;
+  const uint16_t *VT = a.vt16 + ((int64_t)b * (a.heads / a.rep) + kvh) * D * (int64_t)a.t;
   const float *V = a.v + (int64_t)b * a.v_sb + (int64_t)kvh * a.v_skv + (int64_t)rp * a.v_srep;
   const float *M = a.mask ? a.mask + (int64_t)b * a.m_sb + (int64_t)h * a.m_sh + (int64_t)qc * a.m_ss : nullptr;
 
@@ -82,22 +84,22 @@ __global__ void __launch_bounds__(256) attn_prefill_kernel(AttnPrefillDesc a) {
   const float inv_scale = a.has_scale ? 1.0f / a.scale : 1.0f;  // bf16 mode: a product, not the reference's quotient
 
   // registers of the step in flight
-  float4 kreg[KCH], vreg[VBL][4], mreg[KT][4];
+  uint4 kreg[KCH], vreg[KCH];
+  float4 mreg[KT][4];
   // All loads are unconditional (indices clamped into range) so that they are issued back to back;
-  // rows past the end are zeroed when the registers are consumed.
+  // chunks past the end are zeroed when the registers are consumed.
   auto fetch = [&](uint32_t t0) {
 #pragma unroll
     for (int c = 0; c < KCH; ++c) {
-      const int ch = tid + c * 256, key = ch / (D / 4), d4 = (ch % (D / 4)) * 4;
-      kreg[c] = *(const float4 *)(K + (int64_t)min(t0 + key, a.t - 1) * a.k_st + d4);
+      const int ch = tid + c * 256, key = ch / (D / 8), d8 = (ch % (D / 8)) * 8;
+      kreg[c] = *(const uint4 *)(K + (int64_t)min(t0 + key, a.t - 1) * a.k_st + d8);
     }
 #pragma unroll
-    for (int c = 0; c < VBL; ++c) {
-      const int bl = tid + c * 256, k4 = (bl / (D / 4)) * 4, d4 = (bl % (D / 4)) * 4;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) vreg[c][i] = *(const float4 *)(V + (int64_t)min(t0 + k4 + i, a.t - 1) * a.v_st + d4);
+    for (int c = 0; c < KCH; ++c) {
+      const int ch = tid + c * 256, dim = ch / (BN / 8), k8 = (ch % (BN / 8)) * 8;
+      vreg[c] = *(const uint4 *)(VT + (int64_t)dim * a.t + min(t0 + k8, a.t - 8));
     }
-    if (M) {  // mask rows allow 16-byte loads and T % 4 == 0 (checked by the host)
+    if (M) {  // mask rows allow 16-byte loads and T % 8 == 0 (checked by the host)
 #pragma unroll
       for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
@@ -126,22 +128,16 @@ __global__ void __launch_bounds__(256) attn_prefill_kernel(AttnPrefillDesc a) {
     }
     const bool live = __syncthreads_or(live_pair);  // also: the previous step's fragments have been read
     if (live) {
-      // ---- registers -> LDS: K [BN, D] and V^T [D, BN] as bf16 (V through a 4 x 4 register transpose)
+      // ---- registers -> LDS: K [BN, D] and V^T [D, BN]
 #pragma unroll
       for (int c = 0; c < KCH; ++c) {
-        const int ch = tid + c * 256, key = ch / (D / 4), d4 = (ch % (D / 4)) * 4;
-        *(uint2 *)(&Ks[key * KP + d4]) = (t0 + key < a.t) ? bf16_pack4(kreg[c]) : make_uint2(0u, 0u);
+        const int ch = tid + c * 256, key = ch / (D / 8), d8 = (ch % (D / 8)) * 8;
+        *(uint4 *)(&Ks[key * KP + d8]) = (t0 + key < a.t) ? kreg[c] : make_uint4(0u, 0u, 0u, 0u);
       }
 #pragma unroll
-      for (int c = 0; c < VBL; ++c) {
-        const int bl = tid + c * 256, k4 = (bl / (D / 4)) * 4, d4 = (bl % (D / 4)) * 4;
-        float4 r[4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) r[i] = (t0 + k4 + i < a.t) ? vreg[c][i] : make_float4(0.f, 0.f, 0.f, 0.f);
-        *(uint2 *)(&Vt[(d4 + 0) * VP + k4]) = bf16_pack4(make_float4(r[0].x, r[1].x, r[2].x, r[3].x));
-        *(uint2 *)(&Vt[(d4 + 1) * VP + k4]) = bf16_pack4(make_float4(r[0].y, r[1].y, r[2].y, r[3].y));
-        *(uint2 *)(&Vt[(d4 + 2) * VP + k4]) = bf16_pack4(make_float4(r[0].z, r[1].z, r[2].z, r[3].z));
-        *(uint2 *)(&Vt[(d4 + 3) * VP + k4]) = bf16_pack4(make_float4(r[0].w, r[1].w, r[2].w, r[3].w));
+      for (int c = 0; c < KCH; ++c) {
+        const int ch = tid + c * 256, dim = ch / (BN / 8), k8 = (ch % (BN / 8)) * 8;
+        *(uint4 *)(&Vt[dim * VP + k8]) = (t0 + k8 < a.t) ? vreg[c] : make_uint4(0u, 0u, 0u, 0u);
       }
     }
     __syncthreads();
@@ -201,10 +197,14 @@ __global__ void __launch_bounds__(256) attn_prefill_kernel(AttnPrefillDesc a) {
     l_run = l_run * alpha + psum;
     m_run = m_new;
     // ---- O^T = O^T * alpha + V^T . P^T
+    if (__any(alpha != 1.0f)) {  // the running maximum moved for some query of this wave
+#pragma unroll
+      for (int t = 0; t < DT; ++t)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) o[t][e] *= alpha;
+    }
 #pragma unroll
     for (int t = 0; t < DT; ++t) {
-#pragma unroll
-      for (int e = 0; e < 16; ++e) o[t][e] *= alpha;
 #pragma unroll
       for (int blk = 0; blk < KT * 2; ++blk) {
         // A fragment: row = dim t*32 + col, the lane's eight keys of this block in the permuted order

@@ -153,10 +153,13 @@ hipError_t launch_attn_decode(const LaunchCtx &lc, const AttnDecodeDesc &d);
 // ---- k_attn.hip
 // Attention over s query rows per head (bf16 MFMA, online softmax):
 //   out[b, h, i, :] = softmax_j(q[b,h,i,:] . k[b,h,j,:] / scale + mask[b,h,i,j]) . v[b,h,j,:]
-// q, k, v: f32 with unit stride along d (k, v through the kv-head strides as in AttnDecodeDesc);
+// q, v: f32 with unit stride along d (v through the kv-head strides as in AttnDecodeDesc; only read for
+// rows whose every key is masked); k16: the keys as bf16 through the same kind of strides; vt16: the
+// values as bf16, transposed, contiguous [b, kv heads, d, t]; t % 8 == 0;
 // mask: additive f32 through its strides (0 = broadcast) or a constant; out contiguous [b, heads, s, d].
 struct AttnPrefillDesc {
-  const float *q, *k, *v, *mask;
+  const float *q, *v, *mask;
+  const uint16_t *k16, *vt16;
   float *out;
   uint16_t *out16;                     // optional bf16 copy of out
   int64_t q_sb, q_sh, q_ss;

@@ -1734,7 +1734,7 @@ int try_attn_prefill(cg_backend *be, cg_tensor *n, bool *done) {
     return CG_OK;
   // Below this the three-launch path (GEMM, softmax, GEMM) is as fast and the scores are small;
   // above it the scores of one layer run to hundreds of MB.  CG_FLAG_ATTN_ONE_PASS lifts the threshold.
-  if (T < 1024 && !(be->flags & CG_FLAG_ATTN_ONE_PASS)) return CG_OK;
+  if (T < 512 && !(be->flags & CG_FLAG_ATTN_ONE_PASS)) return CG_OK;
   if (nb > 65535 || heads > 65535) return CG_OK;
   MatOperand Kop, Vop;
   bool pk = false, pv = false;
@@ -1757,11 +1757,12 @@ int try_attn_prefill(cg_backend *be, cg_tensor *n, bool *done) {
       !ok4(data_ptr(Kop.t), Kop.strides[3], {Kop.strides[0], Kop.strides[1], Kop.strides[2], Kop.strides[4]}) ||
       !ok4(data_ptr(Vop.t), Vop.strides[4], {Vop.strides[0], Vop.strides[1], Vop.strides[2], Vop.strides[3]}))
     return CG_OK;
+  // the bf16 keys are read eight at a time
+  if (Kop.t->offset % 8 || Kop.strides[0] % 8 || Kop.strides[1] % 8 || Kop.strides[2] % 8 || Kop.strides[4] % 8) return CG_OK;
   TRY(alloc_result(be, n, ST_F32));
   AttnPrefillDesc a;
   std::memset(&a, 0, sizeof(a));
   a.q = (const float *)data_ptr(q);
-  a.k = (const float *)data_ptr(Kop.t);
   a.v = (const float *)data_ptr(Vop.t);
   a.out = (float *)n->st->ptr;
   a.q_sb = q->strides[0]; a.q_sh = q->strides[1]; a.q_ss = q->strides[2];
@@ -1775,11 +1776,29 @@ int try_attn_prefill(cg_backend *be, cg_tensor *n, bool *done) {
     a.m_st = mask->shape[3] == 1 ? 0 : mask->strides[3];
     a.m_vec = a.m_st == 1 && (uintptr_t)a.mask % 16 == 0 && a.m_sb % 4 == 0 && a.m_sh % 4 == 0 && a.m_ss % 4 == 0;
   }
-  if (mask && (!a.m_vec || T % 4)) {  // the kernel reads mask rows 16 bytes at a time: generic path instead
+  // the kernel reads mask rows and value columns 16 bytes at a time, and the keys from their bf16 twin
+  Storage *ksh = nullptr;
+  const bool twin_ok = Kop.t->st->grow_dim < 0 && Kop.t->st->bytes % 32 == 0;
+  if ((mask && !a.m_vec) || T % 8 || !twin_ok) {
     storage_release(n->st);
     n->st = nullptr;
     return CG_OK;
   }
+  TRY(bf16_shadow(be, Kop.t->st, &ksh));
+  a.k16 = (const uint16_t *)ksh->ptr + Kop.t->offset;
+  Storage *vt = nullptr;
+  const int64_t kvh = Kop.shape[1];
+  TRY(dev_alloc(be, (size_t)nb * kvh * d * T * 2, &vt));
+  {
+    KernelScope ks(be, "transpose_cast_bf16", (double)nb * kvh * d * T * 6, 0);
+    hipError_t te = launch_transpose_cast_bf16(be->lc(), data_ptr(Vop.t), ST_F32, vt->ptr, (uint32_t)T, (uint32_t)d,
+                                               Vop.strides[3], (uint32_t)nb, (uint32_t)kvh, Vop.strides[0], Vop.strides[1]);
+    if (te != hipSuccess) {
+      storage_release(vt);
+      return fail(be, CG_ERR_DEVICE, hipGetErrorString(te));
+    }
+  }
+  a.vt16 = (const uint16_t *)vt->ptr;
   a.b = (uint32_t)nb;
   a.heads = (uint32_t)heads;
   a.rep = (uint32_t)Kop.shape[2];
@@ -1793,7 +1812,9 @@ int try_attn_prefill(cg_backend *be, cg_tensor *n, bool *done) {
   {
     const double qo = 2.0 * nb * heads * Sq * d * 4, kvb = 2.0 * nb * Kop.shape[1] * T * d * 4;
     KernelScope ks(be, "attn_prefill", qo + kvb + (mask ? (double)Sq * T * 4 : 0.0), 4.0 * nb * heads * Sq * T * d);
-    HIPCHK(be, launch_attn_prefill(be->lc(), a));
+    hipError_t ae = launch_attn_prefill(be->lc(), a);
+    storage_release(vt);
+    HIPCHK(be, ae);
   }
   n->op = N_REAL;
   drop_inputs(n);
@@ -2627,10 +2648,6 @@ int realize_concat(cg_backend *be, cg_tensor *n) {
   const int plain = n->dtype == CG_F32 ? ST_F32 : ST_U32;
   const bool in_place = xd > 0 && yd > 0 && refs(x) == 1 && x->st->rc.load() == 1 && x->st->grow_dim == dim &&
                         xd + yd <= x->st->grow_cap && x->offset == 0 && x->stype == plain;
-  if (getenv("CG_DEBUG_CONCAT"))
-    fprintf(stderr, "concat dim %d xd %lld yd %lld refs(x) %d st.rc %d grow_dim %d cap %lld off %lld stype %d in_place %d\n", dim,
-            (long long)xd, (long long)yd, refs(x), x->st->rc.load(), x->st->grow_dim, (long long)x->st->grow_cap,
-            (long long)x->offset, x->stype, (int)in_place);
   // the new key rows arrive through apply_rope_embedding: rotate them straight into the cache slot
   RopeMatch rope;
   const bool rope_y = in_place && !(be->flags & CG_FLAG_NO_PATTERNS) && y->op != N_REAL && refs(y) == 1 &&
