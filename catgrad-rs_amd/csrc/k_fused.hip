@@ -337,8 +337,188 @@ __global__ void __launch_bounds__(BLOCK) attn_decode_kernel(AttnDecodeDesc a) {
   }
 }
 
+// The same attention with the keys of one (batch, head) divided over `splits` workgroups, for caches
+// long enough that one compute unit's load path is the limit.  Every group of LPK lanes keeps a
+// running maximum / sum / weighted value row over the rows it visits (all K and V rows of an
+// iteration are requested before any is used); the groups of a workgroup are merged through LDS
+// into one partial result (max, sum, d values) in `part`, and the workgroup that finds the counter
+// of its (batch, head) at splits - 1 merges the partials and writes the output row.  The counters
+// are zero between launches: the merging workgroup puts its counter back.
+template <int LPK>
+__global__ void __launch_bounds__(256) attn_decode_split_kernel(AttnDecodeDesc a) {
+  constexpr int KPW = 64 / LPK, STRIDE = 4 * KPW, U = 8;
+  constexpr float FMIN = -3.40282347e+38f;
+  __shared__ float red[STRIDE][LPK * 4];
+  __shared__ float red_m[STRIDE], red_l[STRIDE];
+  __shared__ float cm[64], cl[64];  // partial maxima and sums while merging (splits <= 64)
+  __shared__ uint32_t last_flag;
+  const uint32_t h = blockIdx.x, b = blockIdx.y, c = blockIdx.z;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int sub = lane % LPK, kg = lane / LPK, grp = wave * KPW + kg;
+  const uint32_t kv = h / a.rep, rp = h % a.rep;
+  const float *q = a.q + (int64_t)b * a.q_sb + (int64_t)h * a.q_sh;
+  const float *K = a.k + (int64_t)b * a.k_sb + (int64_t)kv * a.k_skv + (int64_t)rp * a.k_srep;
+  const float *V = a.v + (int64_t)b * a.v_sb + (int64_t)kv * a.v_skv + (int64_t)rp * a.v_srep;
+  const bool live = (uint32_t)sub * 4 < a.d;
+  const uint32_t t_begin = c * a.chunk, t_end = min(a.t, t_begin + a.chunk);
+  float4 qv = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (live) {
+    qv = *(const float4 *)(q + sub * 4);
+    if (a.q_cos) {  // apply_rope_embedding on the fly, same arithmetic as rope_kernel
+      const uint32_t j = sub * 4, half = a.d / 2;
+      const bool lo = j < half;
+      float4 pv = *(const float4 *)(q + (lo ? j + half : j - half));
+      if (lo) { pv.x = -pv.x; pv.y = -pv.y; pv.z = -pv.z; pv.w = -pv.w; }
+      const float4 cs = *(const float4 *)(a.q_cos + j), sn = *(const float4 *)(a.q_sin + j);
+      qv.x = cs.x * qv.x + sn.x * pv.x; qv.y = cs.y * qv.y + sn.y * pv.y;
+      qv.z = cs.z * qv.z + sn.z * pv.z; qv.w = cs.w * qv.w + sn.w * pv.w;
+    }
+  }
+  // this step's own key / value row comes from the projections, not from the cache
+  const bool has_new = a.k_new != nullptr && a.t_new >= t_begin && a.t_new < t_end;
+  const uint32_t t_new = has_new ? a.t_new : 0xFFFFFFFFu;
+  float4 knew = make_float4(0.f, 0.f, 0.f, 0.f), vnew = knew;
+  if (has_new && live) {
+    const float *kn = a.k_new + (int64_t)b * a.kn_sb + (int64_t)kv * a.kn_skv;
+    const uint32_t j = sub * 4;
+    knew = *(const float4 *)(kn + j);
+    if (a.kn_cos) {
+      const uint32_t half = a.d / 2;
+      const bool lo = j < half;
+      float4 pv = *(const float4 *)(kn + (lo ? j + half : j - half));
+      if (lo) { pv.x = -pv.x; pv.y = -pv.y; pv.z = -pv.z; pv.w = -pv.w; }
+      const float4 cs = *(const float4 *)(a.kn_cos + j), sn = *(const float4 *)(a.kn_sin + j);
+      knew.x = cs.x * knew.x + sn.x * pv.x; knew.y = cs.y * knew.y + sn.y * pv.y;
+      knew.z = cs.z * knew.z + sn.z * pv.z; knew.w = cs.w * knew.w + sn.w * pv.w;
+    }
+    vnew = *(const float4 *)(a.v_new + (int64_t)b * a.vn_sb + (int64_t)kv * a.vn_skv + j);
+    if (rp == 0 && grp == 0) {  // one writer per (batch, kv head)
+      *(float4 *)(const_cast<float *>(K) + (int64_t)t_new * a.k_st + j) = knew;
+      *(float4 *)(const_cast<float *>(V) + (int64_t)t_new * a.v_st + j) = vnew;
+    }
+  }
+  float m_run = FMIN, l_run = 0.f;
+  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (uint32_t t0 = t_begin + grp; t0 < t_end; t0 += STRIDE * U) {
+    float4 kr[U], vr[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const uint32_t t = t0 + u * STRIDE;
+      const bool in = live && t < t_end && t != t_new;
+      const uint32_t tc = min(t, t_end - 1);
+      kr[u] = *(const float4 *)(K + (int64_t)tc * a.k_st + (live ? sub * 4 : 0));
+      vr[u] = *(const float4 *)(V + (int64_t)tc * a.v_st + (live ? sub * 4 : 0));
+      if (t == t_new) { kr[u] = knew; vr[u] = vnew; }
+      else if (!in) { kr[u] = make_float4(0.f, 0.f, 0.f, 0.f); vr[u] = kr[u]; }
+    }
+    float sv[U], mx = FMIN;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      float s = qv.x * kr[u].x + qv.y * kr[u].y + qv.z * kr[u].z + qv.w * kr[u].w;
+#pragma unroll
+      for (int m = LPK / 2; m >= 1; m >>= 1) s += __shfl_xor(s, m, 64);
+      if (a.has_scale) s = s / a.scale;
+      if (a.has_mask_const) s = s + a.mask_const;
+      sv[u] = s;
+      if (t0 + u * STRIDE < t_end) mx = fmaxf(mx, s);
+    }
+    const float m_new = fmaxf(m_run, mx);
+    const float alpha = expf(m_run - m_new);
+    l_run *= alpha;
+    acc.x *= alpha; acc.y *= alpha; acc.z *= alpha; acc.w *= alpha;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (t0 + u * STRIDE < t_end) {
+        const float p = expf(sv[u] - m_new);
+        l_run += p;
+        acc.x += p * vr[u].x; acc.y += p * vr[u].y; acc.z += p * vr[u].z; acc.w += p * vr[u].w;
+      }
+    }
+    m_run = m_new;
+  }
+  // merge the lane groups of this workgroup
+  *(float4 *)(&red[grp][sub * 4]) = acc;
+  if (sub == 0) { red_m[grp] = m_run; red_l[grp] = l_run; }
+  __syncthreads();
+  const uint32_t pw = a.d + 2;  // floats per partial: max, sum, d values
+  float *mine = a.part + (((uint64_t)b * a.heads + h) * a.splits + c) * pw;
+  if ((uint32_t)tid < a.d) {
+    float M = FMIN;
+#pragma unroll
+    for (int g = 0; g < STRIDE; ++g) M = fmaxf(M, red_m[g]);
+    float L = 0.f, o = 0.f;
+#pragma unroll
+    for (int g = 0; g < STRIDE; ++g) {
+      const float w = expf(red_m[g] - M);
+      L += w * red_l[g];
+      o += w * red[g][tid];
+    }
+    if (a.splits == 1) {
+      a.out[((uint64_t)b * a.heads + h) * a.d + tid] = o / L;
+      return;
+    }
+    // agent-scope stores go through to where every compute unit sees them; no cache write-back
+    // or invalidation is needed around the counter below
+    __hip_atomic_store(mine + 2 + tid, o, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (tid == 0) {
+      __hip_atomic_store(mine, M, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(mine + 1, L, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
+  if (a.splits == 1) return;
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // the stores above have completed ...
+  __syncthreads();                                        // ... in every wave before the counter moves
+  uint32_t *counter = a.count + (uint64_t)b * a.heads + h;
+  if (tid == 0)
+    last_flag = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == a.splits - 1 ? 1u : 0u;
+  __syncthreads();
+  if (!last_flag) return;
+  const float *base = a.part + ((uint64_t)b * a.heads + h) * a.splits * pw;
+  if ((uint32_t)tid < a.splits) {
+    cm[tid] = __hip_atomic_load(base + tid * pw, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    cl[tid] = __hip_atomic_load(base + tid * pw + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  __syncthreads();
+  if ((uint32_t)tid < a.d) {
+    float M = FMIN;
+    for (uint32_t s = 0; s < a.splits; ++s) M = fmaxf(M, cm[s]);
+    float L = 0.f, o = 0.f;
+    uint32_t s = 0;
+    for (; s + 8 <= a.splits; s += 8) {
+      float pv[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        pv[u] = __hip_atomic_load(base + (s + u) * pw + 2 + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const float w = expf(cm[s + u] - M);
+        L += w * cl[s + u];
+        o += w * pv[u];
+      }
+    }
+    for (; s < a.splits; ++s) {
+      const float w = expf(cm[s] - M);
+      L += w * cl[s];
+      o += w * __hip_atomic_load(base + s * pw + 2 + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    a.out[((uint64_t)b * a.heads + h) * a.d + tid] = o / L;
+  }
+  if (tid == 0) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+uint32_t attn_decode_rows_per_pass(uint32_t d) { return d <= 64 ? 128 : d <= 128 ? 64 : 32; }
+
 hipError_t launch_attn_decode(const LaunchCtx &lc, const AttnDecodeDesc &d) {
   if (!d.b || !d.heads || !d.d) return hipSuccess;
+  if (d.splits) {
+    if (!d.part || !d.count || !d.chunk || (uint64_t)d.chunk * d.splits < d.t || d.splits > 64) return hipErrorInvalidValue;
+    dim3 grid(d.heads, d.b, d.splits);
+    if (d.d <= 64) CG_LAUNCH(lc, (attn_decode_split_kernel<16>), grid, 256, d);
+    else if (d.d <= 128) CG_LAUNCH(lc, (attn_decode_split_kernel<32>), grid, 256, d);
+    else CG_LAUNCH(lc, (attn_decode_split_kernel<64>), grid, 256, d);
+    return hipGetLastError();
+  }
+  if (d.t > ATTN_DECODE_MAX_T) return hipErrorInvalidValue;
   dim3 grid(d.heads, d.b);
   // long caches: more rows in flight per workgroup
   if (d.t > 256) {

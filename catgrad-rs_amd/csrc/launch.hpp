@@ -146,8 +146,17 @@ struct AttnDecodeDesc {
   const float *k_new, *v_new, *kn_cos, *kn_sin;
   int64_t kn_sb, kn_skv, vn_sb, vn_skv;
   uint32_t t_new;
+  // optional: the keys of one (batch, head) divided over `splits` workgroups of `chunk` keys each
+  // (splits * chunk >= t).  part: b * heads * splits * (d + 2) floats of scratch; count: b * heads
+  // words that are zero before the launch and zero again after it.  splits = 0: one workgroup per
+  // (batch, head), t <= ATTN_DECODE_MAX_T.
+  uint32_t splits, chunk;
+  float *part;
+  uint32_t *count;
 };
 enum { ATTN_DECODE_MAX_T = 8192, ATTN_DECODE_MAX_D = 256 };
+// keys one workgroup of the split form visits per pass over its chunk
+uint32_t attn_decode_rows_per_pass(uint32_t d);
 hipError_t launch_attn_decode(const LaunchCtx &lc, const AttnDecodeDesc &d);
 
 // ---- k_attn.hip

@@ -115,6 +115,8 @@ void backend_release(cg_backend *be) {
   for (void *p : be->pinned_pool) (void)hipHostFree(p);
   for (hipEvent_t ev : be->event_pool) (void)hipEventDestroy(ev);
   if (be->d_words) (void)hipFree(be->d_words);
+  if (be->attn_part) (void)hipFree(be->attn_part);
+  if (be->attn_count) (void)hipFree(be->attn_count);
   if (be->h_words) (void)hipHostFree(be->h_words);
   if (be->stream) (void)hipStreamDestroy(be->stream);
   delete be;
@@ -1822,6 +1824,33 @@ int try_attn_prefill(cg_backend *be, cg_tensor *n, bool *done) {
   return CG_OK;
 }
 
+// Scratch of the split decode attention, grown as needed (the stream is drained before the old
+// buffers go, and new counters start at zero).
+int attn_decode_scratch(cg_backend *be, size_t part_floats, size_t count_words) {
+  if (part_floats > be->attn_part_floats) {
+    size_t want = 1 << 16;
+    while (want < part_floats) want <<= 1;
+    HIPCHK(be, hipStreamSynchronize(be->stream));
+    if (be->attn_part) (void)hipFree(be->attn_part);
+    be->attn_part = nullptr;
+    be->attn_part_floats = 0;
+    HIPCHK(be, hipMalloc((void **)&be->attn_part, want * sizeof(float)));
+    be->attn_part_floats = want;
+  }
+  if (count_words > be->attn_count_words) {
+    size_t want = 1 << 10;
+    while (want < count_words) want <<= 1;
+    HIPCHK(be, hipStreamSynchronize(be->stream));
+    if (be->attn_count) (void)hipFree(be->attn_count);
+    be->attn_count = nullptr;
+    be->attn_count_words = 0;
+    HIPCHK(be, hipMalloc((void **)&be->attn_count, want * sizeof(uint32_t)));
+    HIPCHK(be, hipMemsetAsync(be->attn_count, 0, want * sizeof(uint32_t), be->stream));
+    be->attn_count_words = want;
+  }
+  return CG_OK;
+}
+
 // The cache update of a decode step, `concat(2, cached, new)` (legacy/models/utils.rs:222-223), seen
 // from the attention that reads it: the node under the repeat_kv chain of a K or V operand.
 cg_tensor *kv_concat_under(cg_tensor *t) {
@@ -1911,7 +1940,7 @@ int try_attn_decode(cg_backend *be, cg_tensor *n, bool *done) {
   cg_tensor *S = m.src;
   if (S->op != N_MATMUL || S->rank != 4 || S->shape[2] != 1 || refs(S) != (S == m.x ? 2 : 1)) return CG_OK;
   const int64_t T = S->shape[3], d = n->shape[3], heads = n->shape[1], nb = n->shape[0];
-  if (T < 1 || T > ATTN_DECODE_MAX_T || d > ATTN_DECODE_MAX_D || d % 4 || n->in[1]->shape[2] != T) return CG_OK;
+  if (T < 1 || T > 0x7FFFFFFF || d > ATTN_DECODE_MAX_D || d % 4 || n->in[1]->shape[2] != T) return CG_OK;
   if (S->in[0]->shape[3] != d) return CG_OK;
   // This step's cache update, when both K and V are `concat(2, cached, new)` that can be done in
   // place: the kernel takes the new rows from the projections and stores them itself.
@@ -2019,6 +2048,19 @@ int try_attn_decode(cg_backend *be, cg_tensor *n, bool *done) {
     a.t_new = (uint32_t)(T - 1);
   }
   {
+    // long caches: the keys of a (batch, head) go to several workgroups, enough of them to occupy
+    // every compute unit, each with at most a few passes over its chunk
+    const int64_t bh = nb * heads, rpp = attn_decode_rows_per_pass((uint32_t)d);
+    int64_t ns = std::max((T + rpp - 1) / rpp, std::min((be->n_cus + bh - 1) / bh, (T + 31) / 32));
+    ns = std::min<int64_t>(ns, 64);
+    if (ns >= 2 || T > ATTN_DECODE_MAX_T) {
+      const int64_t chunk = (T + ns - 1) / ns;
+      a.chunk = (uint32_t)chunk;
+      a.splits = (uint32_t)((T + chunk - 1) / chunk);
+      TRY(attn_decode_scratch(be, (size_t)bh * a.splits * (d + 2), (size_t)bh));
+      a.part = be->attn_part;
+      a.count = be->attn_count;
+    }
     const double kv_bytes = 2.0 * nb * Kop.shape[1] * T * d * 4;
     KernelScope ks(be, "attn_decode", kv_bytes + 2.0 * nb * heads * d * 4, 4.0 * nb * heads * T * d);
     HIPCHK(be, launch_attn_decode(be->lc(), a));

@@ -120,6 +120,11 @@ struct cg_backend {
   // recycled pinned buffers (PREFETCH_BYTES each) and events of cg_tensor_prefetch
   std::vector<void *> pinned_pool;
   std::vector<hipEvent_t> event_pool;
+  // scratch of the decode attention that divides the keys over several workgroups: partial results
+  // and one counter per (batch, head); the counters are zero whenever no launch is running
+  float *attn_part = nullptr;
+  uint32_t *attn_count = nullptr;
+  size_t attn_part_floats = 0, attn_count_words = 0;
 
   cgk::LaunchCtx lc() const { return cgk::LaunchCtx{stream, n_cus, d_words, cur_start, cur_stop}; }
 };

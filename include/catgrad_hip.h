@@ -67,7 +67,7 @@ enum {
    * RoPE, gated activations): everything goes through the generic fused-program kernels */
   CG_FLAG_NO_PATTERNS = 4u,
   /* bf16 mode: use the one-pass attention kernel for every sequence length (by default only from
-   * 1024 keys on, where the score tensor it avoids is large) */
+   * 512 keys on, where the score tensor it avoids is large) */
   CG_FLAG_ATTN_ONE_PASS = 8u
 };
 

@@ -167,7 +167,8 @@ def test_residual_add_in_gemv_epilogue(oracle, hip, hip_nopat, shape, order):
 
 
 @pytest.mark.parametrize("cfg", [(1, 32, 8, 513, 64), (1, 4, 4, 7, 16), (2, 8, 2, 100, 128), (1, 4, 1, 33, 256),
-                                 (1, 16, 16, 1, 64)])  # b, heads, kv heads, T, d
+                                 (1, 16, 16, 1, 64), (1, 2, 1, 9000, 64), (1, 32, 8, 2049, 128),
+                                 (3, 4, 2, 700, 256)])  # b, heads, kv heads, T, d
 def test_attention_decode(oracle, hip, hip_nopat, cfg):
     """One-query attention over a cache (q . K^T / sqrt(d) + mask, softmax, . V) as one launch."""
     nb, H, KV, T, d = cfg
