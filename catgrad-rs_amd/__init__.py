@@ -8,4 +8,5 @@ values for the native evaluator, `llm` holds the model definitions.
 from . import abi, lang, nn, interpreter  # noqa: F401
 from .abi import (Backend, Tensor, BackendPanic, ShapeError, InterpreterError, load_library,
                   F32, U32, FLAG_BF16, FLAG_EAGER, FLAG_NO_PATTERNS)  # noqa: F401
-from .interpreter import Interpreter, Environment, Parameters, stdlib, tensor  # noqa: F401
+from .interpreter import (Interpreter, Environment, Parameters, WeightFile, WeightsError, stdlib,  # noqa: F401
+                          tensor)

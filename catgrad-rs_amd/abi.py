@@ -104,6 +104,22 @@ _SIGNATURES = {
     "cg_params_create": (C.c_int, [_PP]),
     "cg_params_destroy": (None, [_P]),
     "cg_params_set": (C.c_int, [_P, C.c_char_p, _P]),
+    "cg_params_len": (_SZ, [_P]),
+    "cg_params_key": (C.c_char_p, [_P, _SZ]),
+    "cg_params_get": (C.c_int, [_P, C.c_char_p, _PP]),
+    "cg_params_remove": (C.c_int, [_P, C.c_char_p]),
+    "cg_from_bf16": (C.c_int, [_P, _P, _SZ, _SZP, C.c_int, _PP]),
+    "cg_stack": (C.c_int, [_P, _PP, _SZ, _PP]),
+    "cg_weights_open": (C.c_int, [C.c_char_p, _PP]),
+    "cg_weights_close": (None, [_P]),
+    "cg_weights_count": (_SZ, [_P]),
+    "cg_weights_name": (C.c_char_p, [_P, _SZ]),
+    "cg_weights_info": (C.c_int, [_P, _SZ, C.POINTER(C.c_int), C.POINTER(C.c_char_p), C.POINTER(C.c_int), _SZP,
+                                  C.POINTER(C.c_uint64)]),
+    "cg_weights_tensor": (C.c_int, [_P, _P, _SZ, _PP]),
+    "cg_params_load": (C.c_int, [_P, _P, C.c_char_p, C.c_char_p, _SZP]),
+    "cg_params_stack_experts": (C.c_int, [_P, _P, C.c_char_p, _SZ, _SZ]),
+    "cg_weights_last_error": (C.c_char_p, []),
     "cg_interp_eval": (C.c_int, [_P, _P, _P, _P, C.POINTER(cg_value), _SZ, C.POINTER(cg_value), _SZ, _U32P]),
     "cg_interp_eval_owned": (C.c_int, [_P, _P, _P, _P, C.POINTER(cg_value), _SZ, C.POINTER(cg_value), _SZ, _U32P]),
     "cg_interp_last_error": (C.c_char_p, []),
@@ -244,6 +260,17 @@ class Backend:
         a = np.ascontiguousarray(data, dtype=np.uint32).reshape(-1)
         d, r = _dims(shape)
         return self._out(self.lib.cg_from_u32, a.ctypes.data, a.size, d, r)
+
+    def from_bf16_bits(self, bits, shape):
+        """An F32 tensor from bf16 bit patterns (uint16), widened by the backend."""
+        a = np.ascontiguousarray(bits, dtype=np.uint16).reshape(-1)
+        d, r = _dims(shape)
+        return self._out(self.lib.cg_from_bf16, a.ctypes.data, a.size, d, r)
+
+    def stack(self, parts):
+        """[n, ...] from n tensors of one shape."""
+        arr = (C.c_void_p * len(parts))(*[t.ptr for t in parts])
+        return self._out(self.lib.cg_stack, arr, len(parts))
 
     def cast(self, x, target_dtype):
         return self._out(self.lib.cg_cast, x.ptr, target_dtype)

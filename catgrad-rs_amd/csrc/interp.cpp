@@ -19,6 +19,7 @@
 
 #include <cstring>
 #include <map>
+#include <iterator>
 #include <string>
 #include <unordered_map>
 #include <vector>
@@ -599,6 +600,29 @@ int cg_params_set(cg_params *p, const char *path, cg_tensor *t) {
   } else {
     p->values.emplace(path, t);
   }
+  return CG_OK;
+}
+
+size_t cg_params_len(const cg_params *p) { return p ? p->values.size() : 0; }
+const char *cg_params_key(const cg_params *p, size_t i) {
+  if (!p || i >= p->values.size()) return nullptr;
+  auto it = p->values.begin();
+  std::advance(it, (std::ptrdiff_t)i);
+  return it->first.c_str();
+}
+int cg_params_get(const cg_params *p, const char *path, cg_tensor **out) {
+  if (!p || !path || !out) return CG_ERR_ARG;
+  auto it = p->values.find(path);
+  if (it == p->values.end()) return CG_ERR_LOAD;
+  *out = cg_tensor_retain(it->second);
+  return CG_OK;
+}
+int cg_params_remove(cg_params *p, const char *path) {
+  if (!p || !path) return CG_ERR_ARG;
+  auto it = p->values.find(path);
+  if (it == p->values.end()) return CG_OK;
+  cg_tensor_release(it->second);
+  p->values.erase(it);
   return CG_OK;
 }
 

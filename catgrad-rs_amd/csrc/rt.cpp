@@ -3159,6 +3159,131 @@ int cg_from_u32(cg_backend *be, const uint32_t *d, size_t n, const size_t *dims,
   return from_host(be, d, n, dims, rank, CG_U32, out);
 }
 
+// An F32 tensor from bf16 bit patterns (the widening of examples/llama/main.rs:309-312 done on the
+// device).  In bf16 mode a tensor of rank >= 2 keeps the bits as its storage.
+int cg_from_bf16(cg_backend *be, const uint16_t *bits, size_t n, const size_t *dims, int rank, cg_tensor **out) {
+  if (!be || !out || (!bits && n)) return fail(be, CG_ERR_ARG, "null argument");
+  int64_t shape[CG_MAX_RANK];
+  TRY(to_shape(be, dims, rank, shape));
+  int64_t sz = 1;
+  for (int i = 0; i < rank; ++i) sz *= shape[i];
+  if ((int64_t)n != sz) return fail(be, CG_ERR_SHAPE, "ShapeError");
+  if (n == 1) return finish(be, const_node(be, CG_F32, rank, shape, (uint32_t)bits[0] << 16), out);
+  HIPCHK(be, hipSetDevice(be->device));
+  cg_tensor *t = new_node(be, CG_F32, rank, shape);
+  const bool keep = rank >= 2 && (be->flags & CG_FLAG_BF16);
+  int st = alloc_result(be, t, keep ? ST_BF16 : ST_F32);
+  if (st) {
+    node_release(t);
+    return st;
+  }
+  hipError_t e = hipSuccess;
+  if (n == 0) {
+  } else if (keep) {
+    e = hipMemcpyAsync(t->st->ptr, bits, n * 2, hipMemcpyHostToDevice, be->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(be->stream);
+  } else {
+    const size_t chunk = (size_t)16 << 20;  // elements per staged piece
+    Storage *stage = nullptr;
+    st = dev_alloc(be, std::min(n, chunk) * 2, &stage);
+    if (st) {
+      node_release(t);
+      return st;
+    }
+    for (size_t o = 0; o < n && e == hipSuccess; o += chunk) {
+      const size_t c = std::min(chunk, n - o);
+      e = hipMemcpyAsync(stage->ptr, bits + o, c * 2, hipMemcpyHostToDevice, be->stream);
+      if (e != hipSuccess) break;
+      Program p;
+      std::memset(&p, 0, sizeof(p));
+      p.n_instr = 1;
+      p.seg_end[0] = 1;
+      p.code[0].op = E_LOAD;
+      p.n_in = 1;
+      p.n_dims = 1;
+      p.dims[0] = (uint32_t)c;
+      p.in[0].ptr = stage->ptr;
+      p.in[0].stride[0] = 1;
+      p.in[0].stype = ST_BF16;
+      p.in[0].vec = 1;
+      OutDesc od;
+      std::memset(&od, 0, sizeof(od));
+      od.ptr = (char *)t->st->ptr + o * 4;
+      od.stype = ST_F32;
+      od.stride[0] = 1;
+      KernelScope ks(be, "ew_from_bf16", (double)c * 6, 0);
+      e = launch_ew(be->lc(), p, od, c, c % 4 == 0);
+      if (e == hipSuccess) e = hipStreamSynchronize(be->stream);
+    }
+    storage_release(stage);
+  }
+  if (e != hipSuccess) {
+    node_release(t);
+    return fail(be, CG_ERR_DEVICE, std::string("upload: ") + hipGetErrorString(e));
+  }
+  *out = t;
+  return CG_OK;
+}
+
+// [n, ...] from n tensors of one shape (the stacked experts of examples/llama/main.rs:217-236): one
+// allocation, n device copies.  Parts that are all dense in one storage type keep it (bf16 weights
+// stay bf16); otherwise every part is first written out as plain f32 / u32.
+int cg_stack(cg_backend *be, cg_tensor *const *parts, size_t n, cg_tensor **out) {
+  if (!be || !parts || !out || n == 0) return fail(be, CG_ERR_ARG, "null argument or nothing to stack");
+  for (size_t i = 0; i < n; ++i) {
+    if (!parts[i] || parts[i]->be != be) return fail(be, CG_ERR_ARG, "null tensor or tensor of another backend");
+    if (parts[i]->dtype != parts[0]->dtype) return fail(be, CG_ERR_DTYPE, "stack: mixed dtypes");
+    if (parts[i]->rank != parts[0]->rank) return fail(be, CG_ERR_SHAPE, "stack: Shape mismatch");
+    for (int d = 0; d < parts[0]->rank; ++d)
+      if (parts[i]->shape[d] != parts[0]->shape[d]) return fail(be, CG_ERR_SHAPE, "stack: Shape mismatch");
+  }
+  if (parts[0]->rank + 1 > CG_MAX_RANK) return fail(be, CG_ERR_SHAPE, "stack: rank too large");
+  HIPCHK(be, hipSetDevice(be->device));
+  std::vector<cg_tensor *> dense(n, nullptr);
+  auto drop = [&]() {
+    for (cg_tensor *t : dense)
+      if (t) node_release(t);
+  };
+  bool same = true;
+  for (size_t i = 0; i < n; ++i) {
+    int st = realize(be, parts[i]);
+    if (st) return st;
+    same = same && is_contiguous(parts[i]) && parts[i]->stype == parts[0]->stype;
+  }
+  for (size_t i = 0; i < n; ++i) {
+    if (same) {
+      dense[i] = retain(parts[i]);
+    } else {
+      int st = contiguous(be, parts[i], &dense[i]);
+      if (st) {
+        drop();
+        return st;
+      }
+    }
+  }
+  int64_t shape[CG_MAX_RANK];
+  shape[0] = (int64_t)n;
+  for (int d = 0; d < parts[0]->rank; ++d) shape[d + 1] = parts[0]->shape[d];
+  cg_tensor *t = new_node(be, parts[0]->dtype, parts[0]->rank + 1, shape);
+  int st = alloc_result(be, t, dense[0]->stype);
+  if (st) {
+    node_release(t);
+    drop();
+    return st;
+  }
+  const size_t each = (size_t)parts[0]->size() * esize(dense[0]->stype);
+  hipError_t e = hipSuccess;
+  for (size_t i = 0; i < n && e == hipSuccess && each; ++i)
+    e = hipMemcpyAsync((char *)t->st->ptr + i * each, data_ptr(dense[i]), each, hipMemcpyDeviceToDevice, be->stream);
+  drop();
+  if (e != hipSuccess) {
+    node_release(t);
+    return fail(be, CG_ERR_DEVICE, std::string("stack: ") + hipGetErrorString(e));
+  }
+  *out = t;
+  return CG_OK;
+}
+
 // ndarray.rs:97-114
 int cg_cast(cg_backend *be, cg_tensor *x, cg_dtype target, cg_tensor **out) {
   TRY(check_args(be, x, nullptr, out));

@@ -4,6 +4,7 @@ Mirror of catgrad/src/interpreter/{interpreter,types,mod}.rs.  Evaluation itself
 (csrc/interp.cpp behind cg_interp_eval); this module only marshals values.
 """
 import ctypes as C
+import os
 
 import numpy as np
 
@@ -64,6 +65,14 @@ def stdlib():
     return Environment(stdlib_definitions())
 
 
+class WeightsError(RuntimeError):
+    """A weight file could not be read (the reference's loader returns Err or panics)."""
+
+    def __init__(self, status, message):
+        super().__init__(f"[{status}] {message}")
+        self.status, self.message = status, message
+
+
 class Parameters(dict):
     """abstract_interpreter::parameters::Parameters: path -> tensor Value."""
 
@@ -73,6 +82,80 @@ class Parameters(dict):
         for k, v in self.items():
             lib.cg_params_set(p, str(k).encode(), v.ptr)
         return _Owned(lib.cg_params_destroy, p, None)
+
+    def _take(self, backend, native):
+        """Replace the contents by those of a native table."""
+        lib = backend.lib
+        self.clear()
+        for i in range(lib.cg_params_len(native.ptr)):
+            key = lib.cg_params_key(native.ptr, i)
+            t = C.c_void_p()
+            lib.cg_params_get(native.ptr, key, C.byref(t))
+            self[key.decode()] = abi.Tensor(backend, t.value)
+
+    def load_safetensors(self, backend, files, prefix=""):
+        """The loading loop of catgrad-llm/examples/llama/main.rs:288-333, natively: every tensor of
+        every file becomes the parameter prefix + name (F32 and BF16 files only)."""
+        lib = backend.lib
+        native = self.handle(lib)
+        for f in ([files] if isinstance(files, (str, bytes, os.PathLike)) else files):
+            n = C.c_size_t()
+            st = lib.cg_params_load(backend.ptr, native.ptr, str(f).encode(), prefix.encode(), C.byref(n))
+            if st:
+                raise WeightsError(st, lib.cg_weights_last_error().decode(errors="replace"))
+        self._take(backend, native)
+        return self
+
+    def stack_experts(self, backend, num_layers, num_experts, prefix=""):
+        """concat_moe_experts (main.rs:171-262): per layer and projection, the experts' matrices
+        become one [E, ...] parameter."""
+        lib = backend.lib
+        native = self.handle(lib)
+        st = lib.cg_params_stack_experts(backend.ptr, native.ptr, prefix.encode(), num_layers, num_experts)
+        if st:
+            raise WeightsError(st, lib.cg_weights_last_error().decode(errors="replace"))
+        self._take(backend, native)
+        return self
+
+
+class WeightFile:
+    """An open safetensors file: names, dtypes and shapes from the header (host only)."""
+
+    def __init__(self, lib, path):
+        self.lib, self.ptr = lib, None
+        w = C.c_void_p()
+        st = lib.cg_weights_open(str(path).encode(), C.byref(w))
+        if st:
+            raise WeightsError(st, lib.cg_weights_last_error().decode(errors="replace"))
+        self.ptr = w
+
+    def close(self):
+        if self.ptr:
+            self.lib.cg_weights_close(self.ptr)
+            self.ptr = None
+
+    __del__ = close
+
+    def __len__(self):
+        return self.lib.cg_weights_count(self.ptr)
+
+    def entries(self):
+        """[(name, dtype string, shape tuple, byte count)] in header order."""
+        out = []
+        for i in range(len(self)):
+            dt, name, rank, nbytes = C.c_int(), C.c_char_p(), C.c_int(), C.c_uint64()
+            dims = (C.c_size_t * 8)()
+            self.lib.cg_weights_info(self.ptr, i, C.byref(dt), C.byref(name), C.byref(rank), dims, C.byref(nbytes))
+            out.append((self.lib.cg_weights_name(self.ptr, i).decode(), name.value.decode(),
+                        tuple(dims[d] for d in range(rank.value)), nbytes.value))
+        return out
+
+    def tensor(self, backend, i):
+        t = C.c_void_p()
+        st = self.lib.cg_weights_tensor(backend.ptr, self.ptr, i, C.byref(t))
+        if st:
+            raise WeightsError(st, self.lib.cg_weights_last_error().decode(errors="replace"))
+        return abi.Tensor(backend, t.value)
 
 
 class _Owned:

@@ -53,7 +53,10 @@ enum {
   CG_ERR_TYPE = 23,
   CG_ERR_ARITY = 24,
   CG_ERR_LOAD = 25,
-  CG_ERR_APPLY = 26
+  CG_ERR_APPLY = 26,
+  /* weight files */
+  CG_ERR_IO = 40,      /* open / stat / mmap failed */
+  CG_ERR_FORMAT = 41   /* not a well-formed safetensors file */
 };
 
 /* cg_backend_create flags */
@@ -111,6 +114,16 @@ int cg_from_f32(cg_backend *be, const float *data, size_t n, const size_t *dims,
                 cg_tensor **out);
 int cg_from_u32(cg_backend *be, const uint32_t *data, size_t n, const size_t *dims, int rank,
                 cg_tensor **out);
+/* An F32 tensor from bf16 bit patterns: what the weight loader of
+ * catgrad-llm/examples/llama/main.rs:309-312 does on the host (widen every bf16 to f32, then
+ * ndarray_from_vec_f32), with the widening left to the device.  With CG_FLAG_BF16 a tensor of
+ * rank >= 2 keeps the file's bits as its storage: nothing is widened or rounded. */
+int cg_from_bf16(cg_backend *be, const uint16_t *bits, size_t n, const size_t *dims, int rank,
+                 cg_tensor **out);
+/* `n` tensors of one shape and dtype as one tensor of shape [n, ...]: the value of the chain
+ * reshape([1, ...]) + concat(.., 0) in concat_moe_experts (catgrad-llm/examples/llama/main.rs:217-236),
+ * built with one allocation and n copies instead of n - 1 growing concatenations. */
+int cg_stack(cg_backend *be, cg_tensor *const *parts, size_t n, cg_tensor **out);
 /* cast (mod.rs:40, ndarray.rs:97-114): f32->u32 is Rust `as` (truncate, saturate, NaN->0) */
 int cg_cast(cg_backend *be, cg_tensor *x, cg_dtype target, cg_tensor **out);
 /* matmul (mod.rs:41, ndarray.rs:116-122, 549-615) */
@@ -235,6 +248,13 @@ int cg_params_create(cg_params **out);
 void cg_params_destroy(cg_params *p);
 int cg_params_set(cg_params *p, const char *path, cg_tensor *t);
 
+/* the table itself: number of entries, the i-th path (valid until the table changes), lookup
+ * (*out is a new reference; CG_ERR_LOAD when the path is absent), removal (0 or 1 entries go) */
+size_t cg_params_len(const cg_params *p);
+const char *cg_params_key(const cg_params *p, size_t i);
+int cg_params_get(const cg_params *p, const char *path, cg_tensor **out);
+int cg_params_remove(cg_params *p, const char *path);
+
 /* Interpreter::eval (interpreter.rs:29-31).  args are borrowed; results[i].tensor are new
  * references.  n_results must equal the number of term targets.  On failure *err_id holds the
  * offending node or edge id (may be NULL). */
@@ -252,6 +272,43 @@ int cg_interp_eval_owned(cg_backend *be, const cg_env *env, const cg_params *par
 const char *cg_interp_last_error(void);
 /* counts Backend calls issued by cg_interp_eval since the last reset (per thread) */
 uint64_t cg_interp_backend_calls(int reset);
+
+/* ==================================================================================
+ * Weight files: safetensors -> Parameters
+ * (the loading loop of catgrad-llm/examples/llama/main.rs:288-333 and its post-processing,
+ *  concat_moe_experts, main.rs:171-262)
+ * ================================================================================== */
+typedef struct cg_weights cg_weights;
+typedef enum { CG_WDT_F32 = 0, CG_WDT_BF16 = 1, CG_WDT_OTHER = 2 } cg_weight_dtype;
+
+/* Map a safetensors file and parse its header (main.rs:290-292: File::open, Mmap::map,
+ * SafeTensors::deserialize).  Host only: no backend, no device.  CG_ERR_IO / CG_ERR_FORMAT with
+ * the reason in cg_weights_last_error(). */
+int cg_weights_open(const char *path, cg_weights **out);
+void cg_weights_close(cg_weights *w);
+size_t cg_weights_count(const cg_weights *w);
+/* name, dtype, shape (up to 8 dims) and byte count of the i-th tensor, in file order of the header;
+ * dtype_name receives the header's dtype string ("F32", "BF16", "F16", ...) */
+const char *cg_weights_name(const cg_weights *w, size_t i);
+int cg_weights_info(const cg_weights *w, size_t i, cg_weight_dtype *dtype, const char **dtype_name,
+                    int *rank, size_t *dims, uint64_t *nbytes);
+/* The i-th tensor on the device as an F32-tagged tensor (main.rs:297-321): F32 bytes as they are,
+ * BF16 through cg_from_bf16; any other dtype is CG_ERR_DTYPE ("Unsupported dtype", main.rs:314-316). */
+int cg_weights_tensor(cg_backend *be, const cg_weights *w, size_t i, cg_tensor **out);
+/* Every tensor of `file` into `params` under the path prefix + name (main.rs:294-333);
+ * *n_loaded (may be NULL) receives their number. */
+int cg_params_load(cg_backend *be, cg_params *params, const char *file, const char *prefix,
+                   size_t *n_loaded);
+/* concat_moe_experts (main.rs:171-262): for every layer l < num_layers and every projection in
+ * {down_proj, gate_proj, up_proj}, the entries prefix + "model.layers.{l}.mlp.experts.{e}.{proj}.weight",
+ * e < num_experts, become one entry prefix + "model.layers.{l}.mlp.experts.{proj}.weight" of shape
+ * [num_experts, ...] and are removed.  A (layer, projection) with no expert entry is skipped; one
+ * with some but not all is CG_ERR_LOAD ("Expected {} experts for layer {} {}, found {}"). */
+int cg_params_stack_experts(cg_backend *be, cg_params *params, const char *prefix,
+                            size_t num_layers, size_t num_experts);
+/* message of the last failed cg_weights_* / cg_params_load / cg_params_stack_experts call in
+ * this thread */
+const char *cg_weights_last_error(void);
 
 #ifdef __cplusplus
 }

@@ -137,6 +137,15 @@ int cg_from_u32(cg_backend *be, const uint32_t *d, size_t n, const size_t *dims,
   return from_bits(be, d, n, dims, rank, CG_U32, out);
 }
 
+// The weight loader's BF16 arm (catgrad-llm/examples/llama/main.rs:309-312): every bf16 widened to
+// f32 on the host (half::bf16::to_f32 = the bits in the upper half of the word), then from_vec.
+int cg_from_bf16(cg_backend *be, const uint16_t *bits, size_t n, const size_t *dims, int rank,
+                 cg_tensor **out) {
+  std::vector<uint32_t> wide(n);
+  for (size_t i = 0; i < n; ++i) wide[i] = (uint32_t)bits[i] << 16;
+  return from_bits(be, wide.data(), n, dims, rank, CG_F32, out);
+}
+
 // Rust `f32 as u32`: truncate toward zero, saturate, NaN -> 0 (ndarray.rs:101)
 static inline uint32_t f32_as_u32(float v) {
   if (!(v == v)) return 0u;
@@ -595,6 +604,39 @@ int cg_concat(cg_backend *be, cg_tensor *x, cg_tensor *y, size_t dim, cg_tensor 
     if (ya) std::memcpy(&t->bits[o * (xa + ya) + xa], &y->bits[o * ya], ya * 4);
   }
   *out = t;
+  return CG_OK;
+}
+
+// The expert stacking of catgrad-llm/examples/llama/main.rs:217-236 as written there: every part
+// reshaped to [1, ...], then concatenated one by one along axis 0.
+int cg_stack(cg_backend *be, cg_tensor *const *parts, size_t n, cg_tensor **out) {
+  if (!parts || !out || n == 0) return fail(be, CG_ERR_ARG, "nothing to stack");
+  std::vector<size_t> one{1};
+  one.insert(one.end(), parts[0]->shape.begin(), parts[0]->shape.end());
+  if (one.size() > CG_MAX_RANK) return fail(be, CG_ERR_SHAPE, "stack: rank too large");
+  cg_tensor *acc = nullptr;
+  for (size_t i = 0; i < n; ++i) {
+    if (parts[i]->shape != parts[0]->shape) {
+      if (acc) cg_tensor_release(acc);
+      return fail(be, CG_ERR_SHAPE, "stack: Shape mismatch");
+    }
+    cg_tensor *r = nullptr;
+    int st = cg_reshape(be, parts[i], one.data(), (int)one.size(), &r);
+    if (st == CG_OK && acc) {
+      cg_tensor *c = nullptr;
+      st = cg_concat(be, acc, r, 0, &c);
+      cg_tensor_release(acc);
+      cg_tensor_release(r);
+      acc = c;
+    } else if (st == CG_OK) {
+      acc = r;
+    }
+    if (st != CG_OK) {
+      if (acc) cg_tensor_release(acc);
+      return st;
+    }
+  }
+  *out = acc;
   return CG_OK;
 }
 
