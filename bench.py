@@ -25,7 +25,7 @@ HBM_PEAK_GBS = 8000.0
 # rocprofv3 --pmc runs of this file (FETCH_SIZE, WRITE_SIZE), each scaled by what the same counter
 # read for the 1 GiB peak_copy_kernel in the same run (x2.000 and x1.000); a profiler cannot run
 # inside this process, so the figure is carried here and reported only for that workload
-PMC_TRAFFIC_BYTES_PER_LAUNCH = {("bf16", 16, "gemv_rowdot_bf16"): 38382778.0}
+PMC_TRAFFIC_BYTES_PER_LAUNCH = {("bf16", 16, "gemv_rowdot_bf16"): 38325390.0}
 MFMA_PEAK_TFLOPS = {"bf16": 2500.0, "f32": 157.3}
 
 

@@ -864,6 +864,51 @@ __global__ void __launch_bounds__(256) gemv_pro_kernel(GemvProDesc g) {
   const uint32_t K = g.m.K, bz = blockIdx.z;
   const float *ga = g.a + (int64_t)bz * g.a_bstride;
   const float *gaux = g.aux ? g.aux + (int64_t)bz * g.aux_bstride : nullptr;
+  // ---- which rows of which matrix
+  const uint32_t N = g.m.p[blockIdx.y].N;
+  const TB *B = (const TB *)g.m.p[blockIdx.y].b;
+  const TB *B2 = GLUEPI ? (const TB *)g.m.p[1].b : nullptr;
+  const int64_t sbn2 = GLUEPI ? g.m.p[1].sbn : 0;
+  if (g.b_index) {
+    uint32_t ix = g.b_index[(int64_t)bz * g.b_index_stride];
+    if (ix >= g.b_index_limit) {  // the reference's select() panics; flag it and stay in bounds
+      atomicOr(g.err, ERRF_INDEX_OOB);
+      ix = g.b_index_limit - 1;
+    }
+    B += (int64_t)ix * g.sb_index;
+  }
+  const int64_t sbn = g.m.p[blockIdx.y].sbn;
+  float *C = g.m.p[blockIdx.y].c + (uint64_t)bz * N;
+  const float *Cadd = g.m.p[blockIdx.y].c_add ? g.m.p[blockIdx.y].c_add + (uint64_t)bz * N : nullptr;
+  const uint32_t slot = KSPLIT ? blockIdx.x : blockIdx.x * 4 + wave;
+  const uint32_t n_slots = KSPLIT ? gridDim.x : gridDim.x * 4;
+  uint32_t k_begin = 0, k_end = K;
+  if (KSPLIT) {
+    const uint32_t per = ((K + 3) / 4 + EPL - 1) / EPL * EPL;
+    k_begin = min(K, wave * per);
+    k_end = min(K, k_begin + per);
+  }
+  constexpr int CPS = GLUEPI ? 1 : R;  // output columns per slot
+  // The weight rows of the first pass do not depend on the input row: request them before the
+  // prologue so that their latency overlaps it.
+  VT q[R][UNROLL];
+  auto request = [&](uint32_t nb, uint32_t k0) {
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+      for (int u = 0; u < UNROLL; ++u) {
+        const uint32_t k = k0 + u * 64 * EPL;
+        if (GLUEPI) {
+          if (k < k_end)
+            q[r][u] = __builtin_nontemporal_load(
+                (const VT *)((r == 0 ? B + (int64_t)nb * sbn : B2 + (int64_t)nb * sbn2) + k));
+        } else if (k < k_end && nb + r < N) {
+          q[r][u] = __builtin_nontemporal_load((const VT *)(B + (int64_t)(nb + r) * sbn + k));
+        }
+      }
+  };
+  bool requested = slot * CPS < N;
+  if (requested) request(slot * CPS, k_begin + lane * EPL);
   // ---- prologue: the input row
   if (g.pro == PRO_RMSNORM) {
     float ss = 0.f;
@@ -902,49 +947,13 @@ __global__ void __launch_bounds__(256) gemv_pro_kernel(GemvProDesc g) {
   }
   __syncthreads();
   // ---- the products
-  const uint32_t N = g.m.p[blockIdx.y].N;
-  const TB *B = (const TB *)g.m.p[blockIdx.y].b;
-  const TB *B2 = GLUEPI ? (const TB *)g.m.p[1].b : nullptr;
-  const int64_t sbn2 = GLUEPI ? g.m.p[1].sbn : 0;
-  if (g.b_index) {
-    uint32_t ix = g.b_index[(int64_t)bz * g.b_index_stride];
-    if (ix >= g.b_index_limit) {  // the reference's select() panics; flag it and stay in bounds
-      atomicOr(g.err, ERRF_INDEX_OOB);
-      ix = g.b_index_limit - 1;
-    }
-    B += (int64_t)ix * g.sb_index;
-  }
-  const int64_t sbn = g.m.p[blockIdx.y].sbn;
-  float *C = g.m.p[blockIdx.y].c + (uint64_t)bz * N;
-  const float *Cadd = g.m.p[blockIdx.y].c_add ? g.m.p[blockIdx.y].c_add + (uint64_t)bz * N : nullptr;
-  const uint32_t slot = KSPLIT ? blockIdx.x : blockIdx.x * 4 + wave;
-  const uint32_t n_slots = KSPLIT ? gridDim.x : gridDim.x * 4;
-  uint32_t k_begin = 0, k_end = K;
-  if (KSPLIT) {
-    const uint32_t per = ((K + 3) / 4 + EPL - 1) / EPL * EPL;
-    k_begin = min(K, wave * per);
-    k_end = min(K, k_begin + per);
-  }
-  constexpr int CPS = GLUEPI ? 1 : R;  // output columns per slot
   for (uint32_t nb = slot * CPS; nb < N; nb += n_slots * CPS) {  // uniform per workgroup when KSPLIT
     float acc[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) acc[r] = 0.f;
     for (uint32_t k0 = k_begin + lane * EPL; k0 < k_end; k0 += 64 * EPL * UNROLL) {
-      VT q[R][UNROLL];
-#pragma unroll
-      for (int r = 0; r < R; ++r)
-#pragma unroll
-        for (int u = 0; u < UNROLL; ++u) {
-          const uint32_t k = k0 + u * 64 * EPL;
-          if (GLUEPI) {
-            if (k < k_end)
-              q[r][u] = __builtin_nontemporal_load(
-                  (const VT *)((r == 0 ? B + (int64_t)nb * sbn : B2 + (int64_t)nb * sbn2) + k));
-          } else if (k < k_end && nb + r < N) {
-            q[r][u] = __builtin_nontemporal_load((const VT *)(B + (int64_t)(nb + r) * sbn + k));
-          }
-        }
+      if (!requested) request(nb, k0);
+      requested = false;
 #pragma unroll
       for (int u = 0; u < UNROLL; ++u) {
         const uint32_t k = k0 + u * 64 * EPL;
