@@ -238,8 +238,9 @@ __global__ void __launch_bounds__(256) attn_prefill_kernel(AttnPrefillDesc a) {
   }
   // ---- normalise and store: O^T register e of tile t is dim t*32 + (e>>2)*8 + half*4 + (e&3)
   if (q_ok) {
-    float *out = a.out + (((int64_t)b * a.heads + h) * a.s + query) * D;
-    uint16_t *out16 = a.out16 ? a.out16 + (((int64_t)b * a.heads + h) * a.s + query) * D : nullptr;
+    const int64_t o_off = (int64_t)b * a.o_sb + (int64_t)h * a.o_sh + (int64_t)query * a.o_ss;
+    float *out = a.out + o_off;
+    uint16_t *out16 = a.out16 ? a.out16 + o_off : nullptr;
 #pragma unroll
     for (int t = 0; t < DT; ++t)
 #pragma unroll

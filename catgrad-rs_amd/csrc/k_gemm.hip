@@ -385,7 +385,9 @@ template <int N> __device__ __forceinline__ void wait_vmcnt() {
   __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
 }
 
-template <int BM_, int BN_, int WR, int WC>
+// EPI: the product goes through LDS on its way out, so that the optional gate (C = act(gate) * product)
+// is read, and C and its bf16 copy are written, 16 bytes per lane along rows.
+template <int BM_, int BN_, int WR, int WC, bool EPI>
 __global__ void __launch_bounds__(WR *WC * 64) gemm_bf16_dma_kernel(GemmDesc g) {
   constexpr int NW = WR * WC, BK = 64, S = 2;
   constexpr int WM = BM_ / WR, WN = BN_ / WC, TM = WM / 32, TN = WN / 32;
@@ -414,6 +416,8 @@ __global__ void __launch_bounds__(WR *WC * 64) gemm_bf16_dma_kernel(GemmDesc g) 
   const uint16_t *B = (const uint16_t *)g.b + b0 * g.sb_b0 + b1 * g.sb_b1;
   float *C = (g.splits > 1 ? g.workspace + (uint64_t)split * batch * g.M * g.N : g.c) +
              (uint64_t)bz * g.M * g.N;
+  const float *Gate = g.glu_gate ? g.glu_gate + (uint64_t)bz * g.M * g.N : nullptr;  // only without split-K
+  uint16_t *C16 = g.c16 ? g.c16 + (uint64_t)bz * g.M * g.N : nullptr;
   const uint32_t k_begin = split * g.k_per_split;
   const uint32_t k_end = min(g.K, k_begin + g.k_per_split);
 
@@ -476,6 +480,40 @@ __global__ void __launch_bounds__(WR *WC * 64) gemm_bf16_dma_kernel(GemmDesc g) 
     if (step + 1 < n_steps) issue((step + 1) & 1);
     compute(step & 1);
   }
+  if constexpr (EPI) {
+    constexpr int TP = BN_ + 4;  // row pitch of the staged tile (floats)
+    float *T = (float *)dma_smem;
+    __syncthreads();  // every wave is done with the operand stages
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e)
+          T[(wm * WM + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3)) * TP + wn * WN + j * 32 + (lane & 31)] =
+              acc[i][j][e];
+    __syncthreads();
+    for (int idx = tid; idx < BM_ * BN_ / 4; idx += NW * 64) {
+      const int r = idx / (BN_ / 4), c4 = (idx % (BN_ / 4)) * 4;
+      const uint32_t row = m0 + r, col = n0 + c4;
+      if (row < g.M && col < g.N) {  // N % 4 == 0: a group of four columns is inside or outside
+        const uint64_t at = (uint64_t)row * g.N + col;
+        float4 v = *(const float4 *)(&T[r * TP + c4]);
+        if (Gate) {
+          const float4 gt = *(const float4 *)(Gate + at);
+          if (g.glu_kind) {
+            v.x *= gelu_ref(gt.x); v.y *= gelu_ref(gt.y); v.z *= gelu_ref(gt.z); v.w *= gelu_ref(gt.w);
+          } else {
+            v.x *= gt.x * sigmoid_ref(gt.x); v.y *= gt.y * sigmoid_ref(gt.y);
+            v.z *= gt.z * sigmoid_ref(gt.z); v.w *= gt.w * sigmoid_ref(gt.w);
+          }
+        }
+        *(float4 *)(C + at) = v;
+        if (C16) *(uint2 *)(C16 + at) = bf16_pack4(v);
+      }
+    }
+    return;
+  }
 #pragma unroll
   for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -489,17 +527,18 @@ __global__ void __launch_bounds__(WR *WC * 64) gemm_bf16_dma_kernel(GemmDesc g) 
     }
 }
 
-template <int BM_, int BN_, int WR, int WC>
+template <int BM_, int BN_, int WR, int WC, bool EPI = false>
 static hipError_t launch_gemm_dma(const LaunchCtx &lc, const GemmDesc &g, uint32_t grid) {
-  constexpr int smem = 2 * (BM_ + BN_) * 64 * 2;
+  constexpr int stages = 2 * (BM_ + BN_) * 64 * 2, staged_tile = EPI ? BM_ * (BN_ + 4) * 4 : 0;
+  constexpr int smem = stages > staged_tile ? stages : staged_tile;
   static bool configured = false;  // one attribute call per kernel and process
   if (!configured) {
-    hipError_t e = hipFuncSetAttribute((const void *)gemm_bf16_dma_kernel<BM_, BN_, WR, WC>,
+    hipError_t e = hipFuncSetAttribute((const void *)gemm_bf16_dma_kernel<BM_, BN_, WR, WC, EPI>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return e;
     configured = true;
   }
-  hipExtLaunchKernelGGL((gemm_bf16_dma_kernel<BM_, BN_, WR, WC>), dim3(grid), dim3(WR * WC * 64), smem,
+  hipExtLaunchKernelGGL((gemm_bf16_dma_kernel<BM_, BN_, WR, WC, EPI>), dim3(grid), dim3(WR * WC * 64), smem,
                         lc.stream, lc.ev_start, lc.ev_stop, 0, g);
   return hipGetLastError();
 }
@@ -507,7 +546,7 @@ static hipError_t launch_gemm_dma(const LaunchCtx &lc, const GemmDesc &g, uint32
 // C = sum over splits of workspace[split] (float4 per thread; sizes are multiples of 4 or the
 // tail is handled scalar)
 __global__ void __launch_bounds__(256) splitk_reduce_kernel(const float *ws, float *c, uint64_t n,
-                                                            uint32_t splits) {
+                                                            uint32_t splits, const float *cadd) {
   const uint64_t n4 = n / 4;
   for (uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x; i < n4;
        i += (uint64_t)gridDim.x * 256) {
@@ -516,13 +555,17 @@ __global__ void __launch_bounds__(256) splitk_reduce_kernel(const float *ws, flo
       const float4 v = ((const float4 *)(ws + (uint64_t)k * n))[i];
       s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
     }
+    if (cadd) {
+      const float4 v = ((const float4 *)cadd)[i];
+      s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+    }
     ((float4 *)c)[i] = s;
   }
   if (blockIdx.x == 0 && threadIdx.x < (n & 3)) {
     const uint64_t i = n4 * 4 + threadIdx.x;
     float s = ws[i];
     for (uint32_t k = 1; k < splits; ++k) s += ws[(uint64_t)k * n + i];
-    c[i] = s;
+    c[i] = s + (cadd ? cadd[i] : 0.f);
   }
 }
 
@@ -1181,6 +1224,13 @@ static bool gemm_fast_path(const GemmDesc &g, int av, int bv) {
          (g.sbk == 1 || g.sbn == 1) && g.K % 8 == 0 && (g.sbk == 1 || g.N % 8 == 0) && av && bv;
 }
 
+bool gemm_epilogue_ok(const GemmDesc &g) {
+  const int asz = g.a_stype == ST_BF16 ? 2 : 4, bsz = g.b_stype == ST_BF16 ? 2 : 4;
+  const int av = vec_ok(g.a, asz, g.sak == 1 ? g.sam : g.sak, g.sa_b0, g.sa_b1);
+  const int bv = vec_ok(g.b, bsz, g.sbk == 1 ? g.sbn : g.sbk, g.sb_b0, g.sb_b1);
+  return gemm_fast_path(g, av, bv) && gemm_dma_ok(g) && g.splits <= 1 && !g.b_index && !g.c_add && g.N % 4 == 0;
+}
+
 // Split-K factor for a problem too small to fill the CUs with 128x128 tiles (0/1 = none).
 // The caller provides g.workspace of splits * batch * M * N floats and sets g.splits/k_per_split.
 uint32_t gemm_split_k(const LaunchCtx &lc, const GemmDesc &g) {
@@ -1203,9 +1253,11 @@ hipError_t launch_matmul(const LaunchCtx &lc, const GemmDesc &g, const char **ke
   const bool b_unit_n = g.sbn == 1 || g.N == 1;
   const int av = vec_ok(g.a, asz, a_unit_k ? g.sam : g.sak, g.sa_b0, g.sa_b1);
   const int bv = vec_ok(g.b, bsz, b_unit_k ? g.sbn : g.sbk, g.b_index ? g.sb_index : g.sb_b0, g.sb_b1);
-  // only the one-row kernels follow b_index and c_add
-  if ((g.b_index || g.c_add) && !(g.M <= 8 && g.a_stype == ST_F32 && g.K > 0 && (b_unit_k || b_unit_n)))
-    return hipErrorInvalidValue;
+  // only the one-row kernels follow b_index and c_add (and the k-slice sum of a split GEMM adds c_add)
+  const bool one_row = g.M <= 8 && g.a_stype == ST_F32 && g.K > 0 && (b_unit_k || b_unit_n);
+  if (g.b_index && !one_row) return hipErrorInvalidValue;
+  if (g.c_add && !one_row && !(gemm_fast_path(g, av, bv) && g.splits > 1)) return hipErrorInvalidValue;
+  if ((g.glu_gate || g.c16) && !gemm_epilogue_ok(g)) return hipErrorInvalidValue;
 
   if (g.M <= 8 && g.a_stype == ST_F32 && g.K > 0) {
     if (b_unit_k) {
@@ -1248,7 +1300,10 @@ hipError_t launch_matmul(const LaunchCtx &lc, const GemmDesc &g, const char **ke
     if (gemm_dma_ok(g)) {
       const uint64_t t256 = (uint64_t)((g.M + 255) / 256) * ((g.N + 255) / 256) * batch * splits;
       hipError_t e;
-      if (t256 >= (uint64_t)lc.n_cus) {
+      if (g.glu_gate || g.c16) {  // the epilogue variant stages a 128 x 128 tile
+        const uint64_t t128 = (uint64_t)((g.M + 127) / 128) * ((g.N + 127) / 128) * batch * splits;
+        e = launch_gemm_dma<128, 128, 2, 2, true>(lc, gg, (uint32_t)t128);
+      } else if (t256 >= (uint64_t)lc.n_cus) {
         e = launch_gemm_dma<256, 256, 2, 4>(lc, gg, (uint32_t)t256);
       } else {
         const uint64_t t128 = (uint64_t)((g.M + 127) / 128) * ((g.N + 127) / 128) * batch * splits;
@@ -1273,7 +1328,7 @@ hipError_t launch_matmul(const LaunchCtx &lc, const GemmDesc &g, const char **ke
       const uint64_t n = (uint64_t)batch * g.M * g.N;
       uint64_t blocks = (n / 4 + 255) / 256, cap = (uint64_t)lc.n_cus * 16;
       CG_LAUNCH(untimed, (splitk_reduce_kernel), (unsigned)(blocks < cap ? (blocks ? blocks : 1) : cap), 256,
-                (const float *)g.workspace, g.c, n, splits);
+                (const float *)g.workspace, g.c, n, splits, g.c_add);
     }
     return hipGetLastError();
   }

@@ -165,12 +165,13 @@ hipError_t launch_attn_decode(const LaunchCtx &lc, const AttnDecodeDesc &d);
 // q, v: f32 with unit stride along d (v through the kv-head strides as in AttnDecodeDesc; only read for
 // rows whose every key is masked); k16: the keys as bf16 through the same kind of strides; vt16: the
 // values as bf16, transposed, contiguous [b, kv heads, d, t]; t % 8 == 0;
-// mask: additive f32 through its strides (0 = broadcast) or a constant; out contiguous [b, heads, s, d].
+// mask: additive f32 through its strides (0 = broadcast) or a constant; out [b, heads, s, d] through its strides.
 struct AttnPrefillDesc {
   const float *q, *v, *mask;
   const uint16_t *k16, *vt16;
   float *out;
-  uint16_t *out16;                     // optional bf16 copy of out
+  uint16_t *out16;                     // optional bf16 copy of out, same indexing
+  int64_t o_sb, o_sh, o_ss;            // out[b, h, s, :] strides (unit stride along d)
   int64_t q_sb, q_sh, q_ss;
   int64_t k_sb, k_skv, k_srep, k_st;
   int64_t v_sb, v_skv, v_srep, v_st;
@@ -204,9 +205,19 @@ struct GemmDesc {
   int64_t b_index_stride, sb_index;
   uint32_t b_index_limit;
   uint32_t *err;
+  // optional epilogue of the direct-to-LDS bf16 GEMM without split-K (gemm_epilogue_ok):
+  // C = act(glu_gate) * (A . B), glu_gate laid out like C (glu_kind 0 = silu, 1 = gelu), i.e. the
+  // gated activation of an MLP applied where up_proj's product is still in registers;
+  // c16: a bf16 copy of C, same indexing
+  const float *glu_gate;
+  int32_t glu_kind;
+  uint16_t *c16;
 };
 // split factor launch_matmul should be given for this problem (1 = none)
 uint32_t gemm_split_k(const LaunchCtx &lc, const GemmDesc &g);
+// whether launch_matmul would run this problem (splits as given) on the kernel that honours
+// glu_gate / c16
+bool gemm_epilogue_ok(const GemmDesc &g);
 hipError_t launch_matmul(const LaunchCtx &lc, const GemmDesc &g, const char **kernel_name);
 // contiguous f32 -> bf16 (RNE); n % 8 == 0, 16-byte aligned
 hipError_t launch_cast_bf16(const LaunchCtx &lc, const float *in, void *out, uint64_t n);

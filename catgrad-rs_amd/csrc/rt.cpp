@@ -1278,12 +1278,48 @@ bool match_glu(cg_tensor *root, cg_tensor **gate, cg_tensor **up, int *gelu) {
   return true;
 }
 
+// What a GEMM may apply to its product before storing it: act(gate) * product (the gated activation
+// of an MLP in up_proj's epilogue).  `applied` tells the caller whether the kernel that ran could.
+struct MatmulEpilogue {
+  const float *gate = nullptr;  // laid out like the product
+  int gelu = 0;
+  bool applied = false;
+};
+int realize_matmul(cg_backend *be, cg_tensor *n, cg_tensor *addend, bool *added, MatmulEpilogue *ep);
+
 int try_glu(cg_backend *be, cg_tensor *root, bool *done) {
   cg_tensor *gate = nullptr, *up = nullptr;
   int gelu = 0;
   if (!match_glu(root, &gate, &up, &gelu)) return CG_OK;
   cg_tensor *gc = nullptr, *uc = nullptr;
   TRY(contiguous(be, gate, &gc));
+  // bf16 mode, many rows: up_proj's GEMM applies act(gate) to its product before storing it.  A
+  // reshape between the product and the multiply (batch folded into the rows for the linear and
+  // unfolded again) changes nothing in memory.
+  cg_tensor *mm = up;
+  if (mm->op == N_RESHAPE && refs(mm) == 1) mm = mm->in[0];
+  if ((be->flags & CG_FLAG_BF16) && mm->op == N_MATMUL && refs(mm) == 1 && refs(up) == 1 && mm->dtype == CG_F32 &&
+      !mm->gemv_candidate && gc->stype == ST_F32 && is_contiguous(gc)) {
+    MatmulEpilogue ep;
+    ep.gate = (const float *)data_ptr(gc);
+    ep.gelu = gelu;
+    int mst = realize_matmul(be, mm, nullptr, nullptr, &ep);
+    if (mst) {
+      node_release(gc);
+      return mst;
+    }
+    if (ep.applied) {  // mm holds the gated activations and nobody else can see it: root takes its storage
+      root->st = mm->st;
+      root->st->rc.fetch_add(1);
+      root->stype = mm->stype;
+      root->offset = mm->offset;
+      contiguous_strides(root->rank, root->shape, root->strides);  // mm is dense: same order, root's shape
+      node_release(gc);
+      finish_fused(root);
+      *done = true;
+      return CG_OK;
+    }
+  }
   int st = contiguous(be, up, &uc);
   if (!st) st = alloc_result(be, root, ST_F32);
   if (!st) {
@@ -1302,8 +1338,7 @@ int try_glu(cg_backend *be, cg_tensor *root, bool *done) {
   return CG_OK;
 }
 
-// a single f32 add/sub/mul/div of two tensors that are (or will be) in memory anyway
-int realize_matmul(cg_backend *be, cg_tensor *n, cg_tensor *addend, bool *added);
+int realize_matmul(cg_backend *be, cg_tensor *n, cg_tensor *addend, bool *added, MatmulEpilogue *ep);
 
 // residual + linear(x) on a decode step (models/llama.rs:166-186: `res + attention`, `res + mlp`):
 // the add rides in the epilogue of the one-row matmul kernel instead of a launch of its own.
@@ -1311,12 +1346,14 @@ int try_gemv_add(cg_backend *be, cg_tensor *root, bool *done) {
   if (root->dtype != CG_F32 || !is_bin(root, E_ADD_F)) return CG_OK;
   for (int side = 0; side < 2; ++side) {
     cg_tensor *mm = root->in[side], *other = root->in[1 - side];
-    if (mm->op != N_MATMUL || refs(mm) != 1 || !mm->gemv_candidate || mm->dtype != CG_F32) continue;
+    // one-row products add in their epilogue; in bf16 mode so does the k-slice sum of a split GEMM
+    if (mm->op != N_MATMUL || refs(mm) != 1 || mm->dtype != CG_F32) continue;
+    if (!mm->gemv_candidate && !(be->flags & CG_FLAG_BF16)) continue;
     if (other->op == N_CONST || ((other->op == N_BIN || other->op == N_UN) && refs(other) == 1)) continue;
     TRY(realize(be, other));
     if (other->stype != ST_F32 || !is_contiguous(other)) return CG_OK;
     bool added = false;
-    TRY(realize_matmul(be, mm, other, &added));
+    TRY(realize_matmul(be, mm, other, &added, nullptr));
     if (!added) return CG_OK;  // the product is realised; the generic add takes it from here
     // mm now holds the sum and nobody else can see it: root takes over its storage
     root->st = mm->st;
@@ -1762,11 +1799,20 @@ int try_attn_prefill(cg_backend *be, cg_tensor *n, bool *done) {
   // the bf16 keys are read eight at a time
   if (Kop.t->offset % 8 || Kop.strides[0] % 8 || Kop.strides[1] % 8 || Kop.strides[2] % 8 || Kop.strides[4] % 8) return CG_OK;
   TRY(alloc_result(be, n, ST_F32));
+  // The models merge the heads next (`transpose(1, 2)` + `reshape [b, s, heads * d]`, llama.rs:107-109):
+  // the result is laid out [b, s, heads, d] in memory and handed back as the [b, heads, s, d] view of
+  // it, so that merge is a view and the bf16 twin is already the o_proj operand.
+  n->strides[0] = Sq * heads * d;
+  n->strides[1] = d;
+  n->strides[2] = heads * d;
+  n->strides[3] = 1;
   AttnPrefillDesc a;
   std::memset(&a, 0, sizeof(a));
   a.q = (const float *)data_ptr(q);
   a.v = (const float *)data_ptr(Vop.t);
   a.out = (float *)n->st->ptr;
+  a.o_sb = n->strides[0]; a.o_sh = n->strides[1]; a.o_ss = n->strides[2];
+  TRY(twin_for_result(be, n, &a.out16));
   a.q_sb = q->strides[0]; a.q_sh = q->strides[1]; a.q_ss = q->strides[2];
   a.k_sb = Kop.strides[0]; a.k_skv = Kop.strides[1]; a.k_srep = Kop.strides[2]; a.k_st = Kop.strides[4];
   a.v_sb = Vop.strides[0]; a.v_skv = Vop.strides[1]; a.v_srep = Vop.strides[2]; a.v_st = Vop.strides[3];
@@ -2401,7 +2447,7 @@ int try_moe_gemv(cg_backend *be, cg_tensor *n, bool *done) {
 
 // `addend` (optional; realised, f32, contiguous, shaped like n) is added in the epilogue when a
 // one-row kernel runs the product; *added tells the caller whether that happened.
-int realize_matmul(cg_backend *be, cg_tensor *n, cg_tensor *addend = nullptr, bool *added = nullptr) {
+int realize_matmul(cg_backend *be, cg_tensor *n, cg_tensor *addend, bool *added, MatmulEpilogue *ep) {
   if (!addend && n->dtype == CG_F32 && n->rank == 4 && n->shape[2] == 1 && !(be->flags & CG_FLAG_NO_PATTERNS)) {
     bool done = false;
     TRY(try_attn_decode(be, n, &done));
@@ -2654,6 +2700,16 @@ int realize_matmul(cg_backend *be, cg_tensor *n, cg_tensor *addend = nullptr, bo
       g.workspace = (float *)ws->ptr;
       g.splits = splits;
       g.k_per_split = ((K + splits - 1) / splits + 63) / 64 * 64;
+      if (addend && !g.c_add && !g.b_index) {  // the pass that sums the k-slices adds the residual too
+        g.c_add = (const float *)data_ptr(addend);
+        *added = true;
+      }
+    }
+    if (ep && !g.c_add && gemm_epilogue_ok(g)) {
+      g.glu_gate = ep->gate;
+      g.glu_kind = ep->gelu;
+      (void)twin_for_result(be, n, &g.c16);  // the gated activations are down_proj's operand
+      ep->applied = true;
     }
     const char *kname = "gemm";
     hipError_t e;
@@ -2818,7 +2874,7 @@ int realize(cg_backend *be, cg_tensor *n) {
     case N_BROADCAST:
     case N_RESHAPE:
     case N_SLICE: return realize_view(be, n);
-    case N_MATMUL: return realize_matmul(be, n);
+    case N_MATMUL: return realize_matmul(be, n, nullptr, nullptr, nullptr);
     case N_REDUCE: return realize_reduce(be, n);
     case N_CONCAT: return realize_concat(be, n);
     case N_INDEX: return realize_index(be, n);

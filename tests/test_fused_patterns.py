@@ -166,6 +166,53 @@ def test_residual_add_in_gemv_epilogue(oracle, hip, hip_nopat, shape, order):
     assert np.allclose(gen, ref, rtol=1e-4, atol=1e-5)
 
 
+@pytest.mark.parametrize("act", ["silu", "gelu"])
+@pytest.mark.parametrize("shape", [(256, 512, 1024), (200, 256, 384), (100, 192, 160)])  # rows, K, N
+def test_gated_activation_in_the_gemm_epilogue(oracle, hip_bf16, shape, act):
+    """bf16 mode, many rows: act(gate_proj(x)) * up_proj(x) with the activation applied by up_proj's GEMM
+    (no launch of its own), followed by down_proj reading the bf16 copy that GEMM wrote."""
+    *rows, K, N = shape
+    g = np.random.default_rng(K + N)
+    x = vectors.bf16_round(g.standard_normal((*rows, K) if len(rows) > 1 else (1, *rows, K)).astype(np.float32))
+    p = {"g.weight": vectors.bf16_round((g.standard_normal((N, K)) * 0.05).astype(np.float32)),
+         "u.weight": vectors.bf16_round((g.standard_normal((N, K)) * 0.05).astype(np.float32)),
+         "d.weight": vectors.bf16_round((g.standard_normal((K, N)) * 0.05).astype(np.float32))}
+
+    def f(b, xv):
+        xv = xv + xv - xv
+        gt = nn.linear_no_bias(b, K, N, lang.path(["g"]), xv)
+        up = nn.linear_no_bias(b, K, N, lang.path(["u"]), xv)
+        h = (nn.silu(b, gt) if act == "silu" else nn.gelu(b, gt)) * up
+        return nn.linear_no_bias(b, N, K, lang.path(["d"]), h), h
+    ref = vectors.run(oracle, f, 2, x, params=p)
+    got, names = run_traced(hip_bf16, f, 2, x, params=p)
+    assert "swiglu_fused" not in names and "geglu_fused" not in names, sorted(names)
+    for r, d in zip(ref, got):
+        assert np.max(np.abs(d - r)) <= 2e-2 * np.abs(r).max()
+
+
+@pytest.mark.parametrize("shape", [(256, 2048, 512), (512, 8192, 2048), (130, 1024, 192), (2048, 2048, 2048)])  # M, K, N
+def test_residual_add_with_a_split_gemm(oracle, hip_bf16, shape):
+    """bf16 mode, many rows: when the product is split along k, the pass that sums the slices adds the
+    residual; otherwise the generic add runs.  Same values either way."""
+    M, K, N = shape
+    g = np.random.default_rng(M + K + N)
+    x = vectors.bf16_round(g.standard_normal((1, M, K)).astype(np.float32))
+    w = vectors.bf16_round((g.standard_normal((N, K)) * 0.05).astype(np.float32))
+    res = g.standard_normal((1, M, N)).astype(np.float32)
+
+    def f(b, xv, rv):
+        xv = xv + xv - xv
+        return rv + nn.linear_no_bias(b, K, N, lang.path(["l"]), xv)
+    p = {"l.weight": w}
+    (ref,) = vectors.run(oracle, f, 1, x, res, params=p)
+    got, names = run_traced(hip_bf16, f, 1, x, res, params=p)
+    assert "gemm_mfma_bf16" in names
+    if shape in ((256, 2048, 512), (512, 8192, 2048)):        # few tiles, deep k: split
+        assert "binary_f32" not in names, sorted(names)
+    assert np.max(np.abs(got[0] - ref)) <= 2e-2 * np.abs(ref).max()
+
+
 @pytest.mark.parametrize("cfg", [(1, 32, 8, 513, 64), (1, 4, 4, 7, 16), (2, 8, 2, 100, 128), (1, 4, 1, 33, 256),
                                  (1, 16, 16, 1, 64), (1, 2, 1, 9000, 64), (1, 32, 8, 2049, 128),
                                  (3, 4, 2, 700, 256)])  # b, heads, kv heads, T, d
