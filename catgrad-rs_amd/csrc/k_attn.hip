@@ -2,7 +2,7 @@
 //
 // The op sequence of catgrad-llm/src/models/llama.rs:95-107 (also gemma3.rs:153-186):
 //   scores = matmul(q, transpose(k));  scores / sqrt(d);  + mask;  softmax;  matmul(., v)
-// materialises [b, h, S, T] twice on the generic path.  Here a workgroup takes 128 query rows of one
+// materialises [b, h, S, T] twice on the generic path.  Here a workgroup takes 128 (or 64) query rows of one
 // (batch, head) and walks the keys 64 at a time with the running maximum / sum of the row
 // (online softmax); scores and probabilities only ever exist in registers.
 //
@@ -37,20 +37,22 @@ __device__ __forceinline__ a_bf16x8 pack8(const float *v) {
 
 // BN keys per step; the K / V rows and the mask values of step i+1 are fetched into registers while
 // step i is being computed, so global latency is paid once per workgroup, not once per step.
-template <int D, int BN>
-__global__ void __launch_bounds__(256) attn_prefill_kernel(AttnPrefillDesc a) {
+// NW waves of 32 queries each per workgroup (4, or 2 when that is what it takes to occupy the CUs).
+template <int D, int BN, int NW>
+__global__ void __launch_bounds__(NW * 64) attn_prefill_kernel(AttnPrefillDesc a) {
+  constexpr int NT = NW * 64;
   constexpr int KP = D + 8;              // K tile row pitch (bf16 elements)
   constexpr int VP = BN + 8;             // V^T tile row pitch
   constexpr int DT = D / 32;             // 32-row tiles of O^T
   constexpr int KT = BN / 32;            // 32-key tiles of S^T
-  constexpr int KCH = BN * D / 8 / 256;  // 16-byte chunks of the K tile / of the V^T tile per thread
+  constexpr int KCH = BN * D / 8 / NT;   // 16-byte chunks of the K tile / of the V^T tile per thread
   __shared__ __attribute__((aligned(16))) uint16_t Ks[BN * KP];
   __shared__ __attribute__((aligned(16))) uint16_t Vt[D * VP];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int col = lane & 31, half = lane >> 5;
   const uint32_t h = blockIdx.y, b = blockIdx.z;
   const uint32_t kvh = h / a.rep, rp = h % a.rep;
-  const uint32_t query = blockIdx.x * 128 + wave * 32 + col;
+  const uint32_t query = blockIdx.x * (NW * 32) + wave * 32 + col;
   const bool q_ok = query < a.s;
   const uint32_t qc = q_ok ? query : a.s - 1;  // loads of lanes past the end go to a valid row
   const float *Q = a.q + (int64_t)b * a.q_sb + (int64_t)h * a.q_sh + (int64_t)qc * a.q_ss;
@@ -91,12 +93,12 @@ __global__ void __launch_bounds__(256) attn_prefill_kernel(AttnPrefillDesc a) {
   auto fetch = [&](uint32_t t0) {
 #pragma unroll
     for (int c = 0; c < KCH; ++c) {
-      const int ch = tid + c * 256, key = ch / (D / 8), d8 = (ch % (D / 8)) * 8;
+      const int ch = tid + c * NT, key = ch / (D / 8), d8 = (ch % (D / 8)) * 8;
       kreg[c] = *(const uint4 *)(K + (int64_t)min(t0 + key, a.t - 1) * a.k_st + d8);
     }
 #pragma unroll
     for (int c = 0; c < KCH; ++c) {
-      const int ch = tid + c * 256, dim = ch / (BN / 8), k8 = (ch % (BN / 8)) * 8;
+      const int ch = tid + c * NT, dim = ch / (BN / 8), k8 = (ch % (BN / 8)) * 8;
       vreg[c] = *(const uint4 *)(VT + (int64_t)dim * a.t + min(t0 + k8, a.t - 8));
     }
     if (M) {  // mask rows allow 16-byte loads and T % 8 == 0 (checked by the host)
@@ -131,12 +133,12 @@ __global__ void __launch_bounds__(256) attn_prefill_kernel(AttnPrefillDesc a) {
       // ---- registers -> LDS: K [BN, D] and V^T [D, BN]
 #pragma unroll
       for (int c = 0; c < KCH; ++c) {
-        const int ch = tid + c * 256, key = ch / (D / 8), d8 = (ch % (D / 8)) * 8;
+        const int ch = tid + c * NT, key = ch / (D / 8), d8 = (ch % (D / 8)) * 8;
         *(uint4 *)(&Ks[key * KP + d8]) = (t0 + key < a.t) ? kreg[c] : make_uint4(0u, 0u, 0u, 0u);
       }
 #pragma unroll
       for (int c = 0; c < KCH; ++c) {
-        const int ch = tid + c * 256, dim = ch / (BN / 8), k8 = (ch % (BN / 8)) * 8;
+        const int ch = tid + c * NT, dim = ch / (BN / 8), k8 = (ch % (BN / 8)) * 8;
         *(uint4 *)(&Vt[dim * VP + k8]) = (t0 + k8 < a.t) ? vreg[c] : make_uint4(0u, 0u, 0u, 0u);
       }
     }
@@ -258,10 +260,20 @@ __global__ void __launch_bounds__(256) attn_prefill_kernel(AttnPrefillDesc a) {
 hipError_t launch_attn_prefill(const LaunchCtx &lc, const AttnPrefillDesc &d) {
   if (!d.b || !d.heads || !d.s) return hipSuccess;
   dim3 grid((d.s + 127) / 128, d.heads, d.b);
+  if ((uint64_t)grid.x * grid.y * grid.z < (uint64_t)lc.n_cus) {  // too few workgroups of 128 queries: 64 each
+    grid.x = (d.s + 63) / 64;
+    switch (d.d) {
+      case 64: CG_LAUNCH(lc, (attn_prefill_kernel<64, 64, 2>), grid, 128, d); break;
+      case 128: CG_LAUNCH(lc, (attn_prefill_kernel<128, 64, 2>), grid, 128, d); break;
+      case 256: CG_LAUNCH(lc, (attn_prefill_kernel<256, 32, 2>), grid, 128, d); break;
+      default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+  }
   switch (d.d) {
-    case 64: CG_LAUNCH(lc, (attn_prefill_kernel<64, 64>), grid, 256, d); break;
-    case 128: CG_LAUNCH(lc, (attn_prefill_kernel<128, 64>), grid, 256, d); break;
-    case 256: CG_LAUNCH(lc, (attn_prefill_kernel<256, 32>), grid, 256, d); break;
+    case 64: CG_LAUNCH(lc, (attn_prefill_kernel<64, 64, 4>), grid, 256, d); break;
+    case 128: CG_LAUNCH(lc, (attn_prefill_kernel<128, 64, 4>), grid, 256, d); break;
+    case 256: CG_LAUNCH(lc, (attn_prefill_kernel<256, 32, 4>), grid, 256, d); break;
     default: return hipErrorInvalidValue;
   }
   return hipGetLastError();

@@ -1251,8 +1251,10 @@ hipError_t launch_matmul(const LaunchCtx &lc, const GemmDesc &g, const char **ke
   const int asz = g.a_stype == ST_BF16 ? 2 : 4, bsz = g.b_stype == ST_BF16 ? 2 : 4;
   const bool a_unit_k = g.sak == 1 || g.K == 1, b_unit_k = g.sbk == 1 || g.K == 1;
   const bool b_unit_n = g.sbn == 1 || g.N == 1;
-  const int av = vec_ok(g.a, asz, a_unit_k ? g.sam : g.sak, g.sa_b0, g.sa_b1);
-  const int bv = vec_ok(g.b, bsz, b_unit_k ? g.sbn : g.sbk, g.b_index ? g.sb_index : g.sb_b0, g.sb_b1);
+  // the stride of an axis of length 1 is never used: it must not spoil the alignment test
+  const int av = vec_ok(g.a, asz, a_unit_k ? (g.M == 1 ? 0 : g.sam) : (g.K == 1 ? 0 : g.sak), g.sa_b0, g.sa_b1);
+  const int bv = vec_ok(g.b, bsz, b_unit_k ? (g.N == 1 ? 0 : g.sbn) : (g.K == 1 ? 0 : g.sbk),
+                        g.b_index ? g.sb_index : g.sb_b0, g.sb_b1);
   // only the one-row kernels follow b_index and c_add (and the k-slice sum of a split GEMM adds c_add)
   const bool one_row = g.M <= 8 && g.a_stype == ST_F32 && g.K > 0 && (b_unit_k || b_unit_n);
   if (g.b_index && !one_row) return hipErrorInvalidValue;

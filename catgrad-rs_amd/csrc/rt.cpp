@@ -147,6 +147,8 @@ void forget_gemv_candidate(cg_tensor *n) {
 
 enum { PREFETCH_BYTES = 4096 };  // pinned buffer of a prefetched tensor: data + 8 bytes of error words
 
+void forget_shared(cg_tensor *n);
+
 void node_release(cg_tensor *t) {
   if (!t || t->rc.fetch_sub(1) != 1) return;  // the common case takes no allocation
   std::vector<cg_tensor *> stack{t};
@@ -155,6 +157,7 @@ void node_release(cg_tensor *t) {
     stack.pop_back();
     if (n != t && n->rc.fetch_sub(1) != 1) continue;
     if (n->gemv_candidate) forget_gemv_candidate(n);
+    forget_shared(n);
     if (n->in[0]) stack.push_back(n->in[0]);
     if (n->in[1]) stack.push_back(n->in[1]);
     storage_release(n->st);
@@ -173,6 +176,15 @@ void node_release(cg_tensor *t) {
 cg_tensor *retain(cg_tensor *t) {
   t->rc.fetch_add(1);
   return t;
+}
+
+// a deleted node leaves the table of shared nodes
+void forget_shared(cg_tensor *n) {
+  if (!n->cse_key) return;
+  auto it = n->be->shared_nodes.find(*n->cse_key);
+  if (it != n->be->shared_nodes.end() && it->second == n) n->be->shared_nodes.erase(it);
+  delete n->cse_key;
+  n->cse_key = nullptr;
 }
 
 void drop_inputs(cg_tensor *n) {
@@ -2895,7 +2907,48 @@ int sync_and_check(cg_backend *be) {
   return CG_OK;
 }
 
+// Structural sharing of values built from constants and aranges only (masks).  Such a node carries
+// a key that spells out how it is computed - the op with its parameters and shape, constants by
+// value, other inputs by their own keys - so the key stays true after the node is realised and
+// after its inputs are gone.  A second request for the same computation gets the same node.
+bool share_node(cg_backend *be, cg_tensor *n, cg_tensor **out) {
+  if (n->cse_key) return false;
+  switch (n->op) {
+    case N_BIN: case N_UN: case N_TRANSPOSE: case N_BROADCAST: case N_RESHAPE: case N_SLICE: break;
+    default: return false;
+  }
+  std::string key;
+  auto put = [&key](const void *p, size_t len) { key.append((const char *)p, len); };
+  put(&n->op, 1); put(&n->ew, 1); put(&n->dtype, sizeof n->dtype); put(&n->rank, sizeof n->rank);
+  put(n->shape, sizeof(int64_t) * n->rank); put(&n->p0, 8); put(&n->p1, 8); put(&n->cbits, 4);
+  for (cg_tensor *in : n->in) {
+    if (!in) { key += 'n'; continue; }
+    if (in->op == N_CONST) {
+      key += 'c';
+      put(&in->dtype, sizeof in->dtype); put(&in->cbits, 4); put(&in->rank, sizeof in->rank);
+      put(in->shape, sizeof(int64_t) * in->rank);
+    } else if (in->cse_key && in->cse_key->size() < 2048) {
+      key += '(';
+      key += *in->cse_key;
+      key += ')';
+    } else {
+      return false;
+    }
+  }
+  auto it = be->shared_nodes.find(key);
+  if (it != be->shared_nodes.end()) {
+    *out = retain(it->second);
+    node_release(n);
+    return true;
+  }
+  n->const_like = true;
+  n->cse_key = new std::string(key);
+  if (be->shared_nodes.size() < 4096) be->shared_nodes.emplace(std::move(key), n);
+  return false;
+}
+
 int finish(cg_backend *be, cg_tensor *n, cg_tensor **out) {
+  if (!(be->flags & CG_FLAG_EAGER) && share_node(be, n, out)) return CG_OK;
   if (be->flags & CG_FLAG_EAGER) {
     int st = realize(be, n);
     if (st) {
@@ -3432,6 +3485,7 @@ int cg_broadcast(cg_backend *be, cg_tensor *x, const size_t *dims, int rank, cg_
   cg_tensor *n = new_node(be, x->dtype, rank, shape);
   n->op = N_BROADCAST;
   n->in[0] = retain(x);
+  if (!(be->flags & CG_FLAG_EAGER) && share_node(be, n, out)) return CG_OK;
   if (x->op == N_REAL) TRY(realize_view(be, n));
   return finish(be, n, out);
 }
@@ -3449,6 +3503,7 @@ int cg_reshape(cg_backend *be, cg_tensor *x, const size_t *dims, int rank, cg_te
   cg_tensor *n = new_node(be, x->dtype, rank, shape);
   n->op = N_RESHAPE;
   n->in[0] = retain(x);
+  if (!(be->flags & CG_FLAG_EAGER) && share_node(be, n, out)) return CG_OK;
   // a reshape that is a pure view of realised data costs nothing: do it now
   int64_t tmp[CG_MAX_RANK];
   if (x->op == N_REAL && (sz == 0 || try_reshape_view(x->rank, x->shape, x->strides, rank, shape, tmp)))
@@ -3469,6 +3524,7 @@ int cg_transpose(cg_backend *be, cg_tensor *x, size_t d0, size_t d1, cg_tensor *
   n->p0 = (int64_t)d0;
   n->p1 = (int64_t)d1;
   n->in[0] = retain(x);
+  if (!(be->flags & CG_FLAG_EAGER) && share_node(be, n, out)) return CG_OK;
   if (x->op == N_REAL) TRY(realize_view(be, n));
   return finish(be, n, out);
 }
@@ -3606,6 +3662,7 @@ int cg_slice(cg_backend *be, cg_tensor *x, size_t dim, size_t start, size_t len,
   n->p0 = (int64_t)dim;
   n->p1 = (int64_t)start;
   n->in[0] = retain(x);
+  if (!(be->flags & CG_FLAG_EAGER) && share_node(be, n, out)) return CG_OK;
   if (x->op == N_REAL) TRY(realize_view(be, n));
   return finish(be, n, out);
 }
@@ -3624,6 +3681,8 @@ int cg_arange(cg_backend *be, size_t end, cg_tensor **out) {
     if (be->arange_cache.size() < 32) {
       cg_tensor *n = new_node(be, CG_U32, 1, shape);
       n->op = N_ARANGE;
+      n->const_like = true;
+      n->cse_key = new std::string("arange" + std::to_string(end));
       be->arange_cache[(int64_t)end] = retain(n);
       return finish(be, n, out);
     }

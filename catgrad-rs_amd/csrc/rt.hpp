@@ -12,6 +12,7 @@
 #include <atomic>
 #include <cstdint>
 #include <map>
+#include <unordered_map>
 #include <string>
 #include <vector>
 
@@ -80,6 +81,10 @@ struct cg_tensor {
   int64_t p0 = 0, p1 = 0;
   uint32_t cbits = 0;
   bool gemv_candidate = false;  // listed in cg_backend::gemv_candidates (a weak reference)
+  // a value that depends on nothing but constants and aranges (a causal mask, say); such nodes are
+  // shared: cse_key is this node's entry in cg_backend::shared_nodes while it is still deferred
+  bool const_like = false;
+  std::string *cse_key = nullptr;
   // cg_tensor_prefetch: a pinned host copy in flight (data, then the backend's error words) and the
   // event recorded behind the copy
   void *host_copy = nullptr;
@@ -117,6 +122,10 @@ struct cg_backend {
   // arange(n) is immutable and models ask for the same few n over and over (masks, RoPE tables of
   // every layer): one node per n, realised once
   std::map<int64_t, cg_tensor *> arange_cache;
+  // deferred nodes built from constants and aranges only, by structure: every layer of a model asks
+  // for the same causal mask, and gets the same node (weak references; an entry goes when its node is
+  // realised or deleted)
+  std::unordered_map<std::string, cg_tensor *> shared_nodes;
   // recycled pinned buffers (PREFETCH_BYTES each) and events of cg_tensor_prefetch
   std::vector<void *> pinned_pool;
   std::vector<hipEvent_t> event_pool;
