@@ -387,9 +387,12 @@ template <int N> __device__ __forceinline__ void wait_vmcnt() {
 
 // EPI: the product goes through LDS on its way out, so that the optional gate (C = act(gate) * product)
 // is read, and C and its bf16 copy are written, 16 bytes per lane along rows.
-template <int BM_, int BN_, int WR, int WC, bool EPI>
+// NS stages of operand tiles in LDS: two when several workgroups share a CU (large problems, bound by
+// the L2 -> LDS rate), four when a CU holds one workgroup and every k-step would otherwise wait out a
+// full trip to HBM (few tiles, cold weights: the prefill-sized products).
+template <int BM_, int BN_, int WR, int WC, bool EPI, int NS>
 __global__ void __launch_bounds__(WR *WC * 64) gemm_bf16_dma_kernel(GemmDesc g) {
-  constexpr int NW = WR * WC, BK = 64, S = 2;
+  constexpr int NW = WR * WC, BK = 64;
   constexpr int WM = BM_ / WR, WN = BN_ / WC, TM = WM / 32, TN = WN / 32;
   constexpr int LPW = (BM_ + BN_) / 8 / NW;   // 1 KB loads per wave per stage
   constexpr int STAGE = (BM_ + BN_) * BK * 2;  // bytes
@@ -411,11 +414,23 @@ __global__ void __launch_bounds__(WR *WC * 64) gemm_bf16_dma_kernel(GemmDesc g) 
   constexpr uint32_t GM = 4;
   const uint32_t first_m = t / (GM * tiles_n) * GM, gsz = min(tiles_m - first_m, GM);
   const uint32_t tg = t % (GM * tiles_n);
-  const uint32_t m0 = (first_m + tg % gsz) * BM_, n0 = tg / gsz * BN_;
+  const uint32_t m0 = (first_m + tg % gsz) * BM_, n0_all = tg / gsz * BN_;
   const uint16_t *A = (const uint16_t *)g.a + b0 * g.sa_b0 + b1 * g.sa_b1;
   const uint16_t *B = (const uint16_t *)g.b + b0 * g.sb_b0 + b1 * g.sb_b1;
   float *C = (g.splits > 1 ? g.workspace + (uint64_t)split * batch * g.M * g.N : g.c) +
              (uint64_t)bz * g.M * g.N;
+  // grouped products: this tile's columns belong to one of them (tiles never straddle two)
+  uint32_t n0 = n0_all, Nl = g.N;
+  if (g.n_group) {
+    uint32_t p = 0;
+    while (p + 1 < g.n_group && n0 >= g.grp_n[p]) {
+      n0 -= g.grp_n[p];
+      ++p;
+    }
+    B = (const uint16_t *)g.grp_b[p];
+    C = g.grp_c[p];
+    Nl = g.grp_n[p];
+  }
   const float *Gate = g.glu_gate ? g.glu_gate + (uint64_t)bz * g.M * g.N : nullptr;  // only without split-K
   uint16_t *C16 = g.c16 ? g.c16 + (uint64_t)bz * g.M * g.N : nullptr;
   const uint32_t k_begin = split * g.k_per_split;
@@ -437,7 +452,7 @@ __global__ void __launch_bounds__(WR *WC * 64) gemm_bf16_dma_kernel(GemmDesc g) 
     const int R = q * 8 + (lane >> 3);
     const int c = (lane & 7) ^ ((R >> 1) & 7);
     if (q * 8 < BM_) gp[i] = A + (int64_t)min(m0 + R, g.M - 1) * g.sam + k_begin + c * 8;
-    else gp[i] = B + (int64_t)min(n0 + (R - BM_), g.N - 1) * g.sbn + k_begin + c * 8;
+    else gp[i] = B + (int64_t)min(n0 + (R - BM_), Nl - 1) * g.sbn + k_begin + c * 8;
   }
   auto issue = [&](int buf) {
 #pragma unroll
@@ -473,12 +488,17 @@ __global__ void __launch_bounds__(WR *WC * 64) gemm_bf16_dma_kernel(GemmDesc g) 
     }
   };
   const int n_steps = k_end > k_begin ? (int)((k_end - k_begin) / BK) : 0;
-  if (n_steps > 0) issue(0);
+#pragma unroll
+  for (int s0 = 0; s0 < NS - 1; ++s0)
+    if (s0 < n_steps) issue(s0);
   for (int step = 0; step < n_steps; ++step) {
-    wait_vmcnt<0>();   // stage `step` has landed (this wave's part) ...
-    __syncthreads();   // ... and everyone's; all waves are done reading the other buffer
-    if (step + 1 < n_steps) issue((step + 1) & 1);
-    compute(step & 1);
+    // stage `step` has landed (this wave's part): at most the NS - 2 younger stages are still in
+    // flight; in the tail, where fewer were issued, wait for everything
+    if (step + NS - 1 <= n_steps) wait_vmcnt<(NS - 2) * LPW>();
+    else wait_vmcnt<0>();
+    __syncthreads();   // ... and everyone's; all waves are done reading the buffer refilled next
+    if (step + NS - 1 < n_steps) issue((step + NS - 1) % NS);
+    compute(step % NS);
   }
   if constexpr (EPI) {
     constexpr int TP = BN_ + 4;  // row pitch of the staged tile (floats)
@@ -496,8 +516,8 @@ __global__ void __launch_bounds__(WR *WC * 64) gemm_bf16_dma_kernel(GemmDesc g) 
     for (int idx = tid; idx < BM_ * BN_ / 4; idx += NW * 64) {
       const int r = idx / (BN_ / 4), c4 = (idx % (BN_ / 4)) * 4;
       const uint32_t row = m0 + r, col = n0 + c4;
-      if (row < g.M && col < g.N) {  // N % 4 == 0: a group of four columns is inside or outside
-        const uint64_t at = (uint64_t)row * g.N + col;
+      if (row < g.M && col < Nl) {  // N % 4 == 0: a group of four columns is inside or outside
+        const uint64_t at = (uint64_t)row * Nl + col;
         float4 v = *(const float4 *)(&T[r * TP + c4]);
         if (Gate) {
           const float4 gt = *(const float4 *)(Gate + at);
@@ -522,23 +542,23 @@ __global__ void __launch_bounds__(WR *WC * 64) gemm_bf16_dma_kernel(GemmDesc g) 
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
         const uint32_t row = m0 + wm * WM + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
-        if (row < g.M && col < g.N) C[(uint64_t)row * g.N + col] = acc[i][j][e];
+        if (row < g.M && col < Nl) C[(uint64_t)row * Nl + col] = acc[i][j][e];
       }
     }
 }
 
-template <int BM_, int BN_, int WR, int WC, bool EPI = false>
+template <int BM_, int BN_, int WR, int WC, bool EPI = false, int NS = 2>
 static hipError_t launch_gemm_dma(const LaunchCtx &lc, const GemmDesc &g, uint32_t grid) {
-  constexpr int stages = 2 * (BM_ + BN_) * 64 * 2, staged_tile = EPI ? BM_ * (BN_ + 4) * 4 : 0;
+  constexpr int stages = NS * (BM_ + BN_) * 64 * 2, staged_tile = EPI ? BM_ * (BN_ + 4) * 4 : 0;
   constexpr int smem = stages > staged_tile ? stages : staged_tile;
   static bool configured = false;  // one attribute call per kernel and process
   if (!configured) {
-    hipError_t e = hipFuncSetAttribute((const void *)gemm_bf16_dma_kernel<BM_, BN_, WR, WC, EPI>,
+    hipError_t e = hipFuncSetAttribute((const void *)gemm_bf16_dma_kernel<BM_, BN_, WR, WC, EPI, NS>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return e;
     configured = true;
   }
-  hipExtLaunchKernelGGL((gemm_bf16_dma_kernel<BM_, BN_, WR, WC, EPI>), dim3(grid), dim3(WR * WC * 64), smem,
+  hipExtLaunchKernelGGL((gemm_bf16_dma_kernel<BM_, BN_, WR, WC, EPI, NS>), dim3(grid), dim3(WR * WC * 64), smem,
                         lc.stream, lc.ev_start, lc.ev_stop, 0, g);
   return hipGetLastError();
 }
@@ -1259,7 +1279,7 @@ hipError_t launch_matmul(const LaunchCtx &lc, const GemmDesc &g, const char **ke
   const bool one_row = g.M <= 8 && g.a_stype == ST_F32 && g.K > 0 && (b_unit_k || b_unit_n);
   if (g.b_index && !one_row) return hipErrorInvalidValue;
   if (g.c_add && !one_row && !(gemm_fast_path(g, av, bv) && g.splits > 1)) return hipErrorInvalidValue;
-  if ((g.glu_gate || g.c16) && !gemm_epilogue_ok(g)) return hipErrorInvalidValue;
+  if ((g.glu_gate || g.c16 || g.n_group) && !gemm_epilogue_ok(g)) return hipErrorInvalidValue;
 
   if (g.M <= 8 && g.a_stype == ST_F32 && g.K > 0) {
     if (b_unit_k) {
@@ -1302,17 +1322,27 @@ hipError_t launch_matmul(const LaunchCtx &lc, const GemmDesc &g, const char **ke
     if (gemm_dma_ok(g)) {
       const uint64_t t256 = (uint64_t)((g.M + 255) / 256) * ((g.N + 255) / 256) * batch * splits;
       hipError_t e;
+      bool grp256 = true;  // 256-column tiles must not straddle two grouped products
+      for (uint32_t p = 0; p < g.n_group; ++p) grp256 = grp256 && g.grp_n[p] % 256 == 0;
+      if (g.n_group && (batch != 1 || splits != 1 || g.glu_gate || g.c16)) return hipErrorInvalidValue;
+      const uint64_t t128 = (uint64_t)((g.M + 127) / 128) * ((g.N + 127) / 128) * batch * splits;
+      const bool deep = t128 < 2 * (uint64_t)lc.n_cus;  // at most one workgroup per CU at a time: four stages
       if (g.glu_gate || g.c16) {  // the epilogue variant stages a 128 x 128 tile
-        const uint64_t t128 = (uint64_t)((g.M + 127) / 128) * ((g.N + 127) / 128) * batch * splits;
-        e = launch_gemm_dma<128, 128, 2, 2, true>(lc, gg, (uint32_t)t128);
-      } else if (t256 >= (uint64_t)lc.n_cus) {
+        if (deep) e = launch_gemm_dma<128, 128, 2, 2, true, 4>(lc, gg, (uint32_t)t128);
+        else e = launch_gemm_dma<128, 128, 2, 2, true, 2>(lc, gg, (uint32_t)t128);
+      } else if (t256 >= (uint64_t)lc.n_cus && grp256) {
         e = launch_gemm_dma<256, 256, 2, 4>(lc, gg, (uint32_t)t256);
+      } else if (splits == 1 && t128 * 2 <= (uint64_t)lc.n_cus && g.N >= 128) {
+        // too few 128 x 128 tiles for the CUs and no split-K to multiply them: halve the tile
+        e = launch_gemm_dma<128, 64, 2, 2, false, 4>(lc, gg, (uint32_t)((uint64_t)((g.M + 127) / 128) * ((g.N + 63) / 64) * batch));
+      } else if (deep) {
+        e = launch_gemm_dma<128, 128, 2, 2, false, 4>(lc, gg, (uint32_t)t128);
       } else {
-        const uint64_t t128 = (uint64_t)((g.M + 127) / 128) * ((g.N + 127) / 128) * batch * splits;
         e = launch_gemm_dma<128, 128, 2, 2>(lc, gg, (uint32_t)t128);
       }
       if (e != hipSuccess) return e;
     } else {
+    if (g.n_group) return hipErrorInvalidValue;
     const uint64_t big_tiles = (uint64_t)((g.M + 127) / 128) * ((g.N + 127) / 128) * batch * splits;
     if (big_tiles * 2 >= (uint64_t)lc.n_cus && g.N > 64) {
       dim3 gr((g.N + 127) / 128, (g.M + 127) / 128, batch * splits);

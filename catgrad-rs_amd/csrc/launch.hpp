@@ -212,6 +212,13 @@ struct GemmDesc {
   const float *glu_gate;
   int32_t glu_kind;
   uint16_t *c16;
+  // optional (same kernel, one batch, no split-K): n_group products that share A, K and the strides of
+  // B (q/k/v of a prefill) as one launch.  N is the sum of grp_n; columns [0, grp_n[0]) belong to the
+  // first product, and so on; every grp_n is a multiple of 128; b and c are ignored.
+  uint32_t n_group;
+  const void *grp_b[3];
+  float *grp_c[3];
+  uint32_t grp_n[3];
 };
 // split factor launch_matmul should be given for this problem (1 = none)
 uint32_t gemm_split_k(const LaunchCtx &lc, const GemmDesc &g);

@@ -145,6 +145,17 @@ void forget_gemv_candidate(cg_tensor *n) {
   n->gemv_candidate = false;
 }
 
+void forget_gemm_candidate(cg_tensor *n) {
+  auto &v = n->be->gemm_candidates;
+  for (size_t i = 0; i < v.size(); ++i)
+    if (v[i] == n) {
+      v[i] = v.back();
+      v.pop_back();
+      break;
+    }
+  n->gemm_candidate = false;
+}
+
 enum { PREFETCH_BYTES = 4096 };  // pinned buffer of a prefetched tensor: data + 8 bytes of error words
 
 void forget_shared(cg_tensor *n);
@@ -157,6 +168,7 @@ void node_release(cg_tensor *t) {
     stack.pop_back();
     if (n != t && n->rc.fetch_sub(1) != 1) continue;
     if (n->gemv_candidate) forget_gemv_candidate(n);
+    if (n->gemm_candidate) forget_gemm_candidate(n);
     forget_shared(n);
     if (n->in[0]) stack.push_back(n->in[0]);
     if (n->in[1]) stack.push_back(n->in[1]);
@@ -2705,8 +2717,37 @@ int realize_matmul(cg_backend *be, cg_tensor *n, cg_tensor *addend, bool *added,
         return CG_OK;
       }
     }
+    // q/k/v of a prefill: the other deferred many-row products on the same left operand join this
+    // launch as further column ranges (their own weights, their own outputs)
+    std::vector<cg_tensor *> group;
+    if (n->gemm_candidate && !addend && !ep && !ex.w && batch == 1 && g.bf16_math && g.a_stype == ST_BF16 &&
+        g.b_stype == ST_BF16 && g.sbk == 1 && N % 128 == 0 && gemm_epilogue_ok(g)) {
+      for (cg_tensor *c : std::vector<cg_tensor *>(be->gemm_candidates)) {
+        if (c == n || group.size() >= 2 || c->op != N_MATMUL || c->in[0] != n->in[0] || c->rank != n->rank) continue;
+        cg_tensor *w = c->in[1];
+        if (w->op != N_REAL || w->rank != 3 || w->stype != ST_BF16 || w->shape[0] != 1) continue;
+        if (w->shape[1] != (int64_t)K || w->strides[1] != 1 || w->strides[2] != g.sbn) continue;
+        if (w->shape[2] % 128 || (uintptr_t)data_ptr(w) % 16) continue;
+        group.push_back(c);
+      }
+      if (group.size() < 2) group.clear();  // pairs (gate / up) keep their own launches and epilogues
+    }
+    if (!group.empty()) {
+      g.n_group = 1;
+      g.grp_b[0] = g.b;
+      g.grp_c[0] = g.c;
+      g.grp_n[0] = N;
+      for (cg_tensor *c : group) {
+        TRY(alloc_result(be, c, ST_F32));
+        g.grp_b[g.n_group] = data_ptr(c->in[1]);
+        g.grp_c[g.n_group] = (float *)c->st->ptr;
+        g.grp_n[g.n_group] = (uint32_t)c->in[1]->shape[2];
+        g.N += g.grp_n[g.n_group];
+        ++g.n_group;
+      }
+    }
     Storage *ws = nullptr;
-    const uint32_t splits = gemm_split_k(be->lc(), g);
+    const uint32_t splits = group.empty() ? gemm_split_k(be->lc(), g) : 1;
     if (splits > 1) {
       TRY(dev_alloc(be, (size_t)splits * n->size() * 4, &ws));
       g.workspace = (float *)ws->ptr;
@@ -2726,21 +2767,30 @@ int realize_matmul(cg_backend *be, cg_tensor *n, cg_tensor *addend, bool *added,
     const char *kname = "gemm";
     hipError_t e;
     {
-      KernelScope ks(be, kname, uniq(A, sao) + uniq(B, sbo) * (ex.w ? (double)batch : 1.0) + (double)n->size() * 4,
-                     2.0 * batch * M * N * K);
+      // grouped: g.N counts every member's columns; B and C bytes scale with it
+      KernelScope ks(be, kname,
+                     uniq(A, sao) + (uniq(B, sbo) * (ex.w ? (double)batch : 1.0) + (double)n->size() * 4) * ((double)g.N / N),
+                     2.0 * batch * M * g.N * K);
       e = launch_matmul(be->lc(), g, &kname);
       ks.rename(kname);
       if (be->trace_shapes) {  // per-shape records: gemm_mfma_bf16[b32,512x512x64,s1]
         char buf[96];
-        snprintf(buf, sizeof buf, "%s[b%lld,%ux%ux%u,s%u]", kname, (long long)batch, M, N, K, splits);
+        snprintf(buf, sizeof buf, "%s[b%lld,%ux%ux%u,s%u%s]", kname, (long long)batch, M, g.N, K, splits,
+                 group.empty() ? "" : ",grouped");
         ks.rename(buf);
       }
+    }
+    for (cg_tensor *c : group) {
+      forget_gemm_candidate(c);
+      c->op = N_REAL;
+      drop_inputs(c);
     }
     storage_release(ws);
     storage_release(bt);
     HIPCHK(be, e);
   }
   if (n->gemv_candidate) forget_gemv_candidate(n);
+  if (n->gemm_candidate) forget_gemm_candidate(n);
   n->op = N_REAL;
   drop_inputs(n);
   return CG_OK;
@@ -3438,6 +3488,12 @@ int cg_matmul(cg_backend *be, cg_tensor *a, cg_tensor *b, cg_tensor **out) {
     if (be->gemv_candidates.size() >= 4096) forget_gemv_candidate(be->gemv_candidates.front());
     be->gemv_candidates.push_back(n);
     n->gemv_candidate = true;
+  }
+  if (a->dtype == CG_F32 && a->rank == 3 && shape[0] == 1 && shape[1] >= 64 && (be->flags & CG_FLAG_BF16) &&
+      !(be->flags & (CG_FLAG_EAGER | CG_FLAG_NO_PATTERNS))) {
+    if (be->gemm_candidates.size() >= 1024) forget_gemm_candidate(be->gemm_candidates.front());
+    be->gemm_candidates.push_back(n);
+    n->gemm_candidate = true;
   }
   return finish(be, n, out);
 }

@@ -81,6 +81,7 @@ struct cg_tensor {
   int64_t p0 = 0, p1 = 0;
   uint32_t cbits = 0;
   bool gemv_candidate = false;  // listed in cg_backend::gemv_candidates (a weak reference)
+  bool gemm_candidate = false;  // listed in cg_backend::gemm_candidates (a weak reference)
   // a value that depends on nothing but constants and aranges (a causal mask, say); such nodes are
   // shared: cse_key is this node's entry in cg_backend::shared_nodes while it is still deferred
   bool const_like = false;
@@ -118,6 +119,8 @@ struct cg_backend {
   // deferred small-M matmuls, so that those sharing their left operand (q/k/v, gate/up) can be
   // issued as one launch; weak references, removed when a node is realised or deleted
   std::vector<cg_tensor *> gemv_candidates;
+  // the same for many-row products in bf16 mode (q/k/v of a prefill as one grouped GEMM)
+  std::vector<cg_tensor *> gemm_candidates;
   hipEvent_t cur_start = nullptr, cur_stop = nullptr;  // set while a traced launch is issued
   // arange(n) is immutable and models ask for the same few n over and over (masks, RoPE tables of
   // every layer): one node per n, realised once

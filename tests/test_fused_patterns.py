@@ -166,6 +166,30 @@ def test_residual_add_in_gemv_epilogue(oracle, hip, hip_nopat, shape, order):
     assert np.allclose(gen, ref, rtol=1e-4, atol=1e-5)
 
 
+@pytest.mark.parametrize("shape", [(512, 2048, (2048, 512, 512)), (130, 256, (256, 128, 384)), (64, 64, (128, 128, 128))])
+def test_sibling_products_as_one_grouped_gemm(oracle, hip_bf16, shape):
+    """bf16 mode, many rows: q_proj, k_proj, v_proj of one input go out as one launch; each product
+    lands in its own tensor."""
+    M, K, Ns = shape
+    g = np.random.default_rng(M + K)
+    x = vectors.bf16_round(g.standard_normal((1, M, K)).astype(np.float32))
+    p = {f"w{i}.weight": vectors.bf16_round((g.standard_normal((n, K)) * 0.05).astype(np.float32)) for i, n in enumerate(Ns)}
+
+    def f(b, xv):
+        xv = xv + xv - xv
+        return tuple(nn.linear_no_bias(b, K, n, lang.path([f"w{i}"]), xv) for i, n in enumerate(Ns))
+    ref = vectors.run(oracle, f, 3, x, params=p)
+    hip_bf16.trace(2)
+    hip_bf16.trace_reset()
+    got = vectors.run(hip_bf16, f, 3, x, params=p)
+    rep = hip_bf16.trace_report()
+    hip_bf16.trace(False)
+    gemms = {k: v["launches"] for k, v in rep.items() if k.startswith("gemm_mfma_bf16")}
+    assert sum(gemms.values()) == 1 and "grouped" in next(iter(gemms)), gemms
+    for r, d in zip(ref, got):
+        assert d.shape == r.shape and np.max(np.abs(d - r)) <= 2e-2 * np.abs(r).max()
+
+
 @pytest.mark.parametrize("act", ["silu", "gelu"])
 @pytest.mark.parametrize("shape", [(256, 512, 1024), (200, 256, 384), (100, 192, 160)])  # rows, K, N
 def test_gated_activation_in_the_gemm_epilogue(oracle, hip_bf16, shape, act):
