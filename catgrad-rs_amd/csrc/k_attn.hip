@@ -25,13 +25,17 @@ namespace cgk {
 typedef __attribute__((ext_vector_type(8))) __bf16 a_bf16x8;
 typedef __attribute__((ext_vector_type(16))) float a_f32x16;
 
+typedef __attribute__((ext_vector_type(2))) __bf16 a_bf16x2;
+typedef __attribute__((ext_vector_type(2))) float a_f32x2;
+
+// eight floats -> eight bf16 (round to nearest even: v_cvt_pk_bf16_f32, one instruction per pair)
 __device__ __forceinline__ a_bf16x8 pack8(const float *v) {
   union {
-    uint32_t u[4];
+    a_bf16x2 h2[4];
     a_bf16x8 h;
   } r;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) r.u[i] = bf16_bits(v[2 * i]) | (bf16_bits(v[2 * i + 1]) << 16);
+  for (int i = 0; i < 4; ++i) r.h2[i] = __builtin_convertvector((a_f32x2){v[2 * i], v[2 * i + 1]}, a_bf16x2);
   return r.h;
 }
 
@@ -113,20 +117,27 @@ __global__ void __launch_bounds__(NW * 64) attn_prefill_kernel(AttnPrefillDesc a
   for (uint32_t t0 = 0; t0 < a.t; t0 += BN) {
     // ---- is any (query, key) pair of this step unmasked?  A causal or sliding-window mask kills
     // most steps; a dead step only adds terms that the first live step rescales to zero.
+    const bool tail = t0 + BN > a.t;  // the only step with keys past the end (uniform)
     bool live_pair = !M;
     float4 mcur[KT][4];
     if (M) {
+      float mmax = -3.40282347e+38f;
 #pragma unroll
       for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           mcur[kt][j] = mreg[kt][j];
-          const uint32_t key = t0 + kt * 32 + j * 8 + half * 4;
-          const float4 mk = mcur[kt][j];
-          if (q_ok && ((key < a.t && mk.x > -3.0e38f) || (key + 1 < a.t && mk.y > -3.0e38f) ||
-                       (key + 2 < a.t && mk.z > -3.0e38f) || (key + 3 < a.t && mk.w > -3.0e38f)))
-            live_pair = true;
+          float4 mk = mcur[kt][j];
+          if (tail) {
+            const uint32_t key = t0 + kt * 32 + j * 8 + half * 4;
+            if (key >= a.t) mk.x = -3.40282347e+38f;
+            if (key + 1 >= a.t) mk.y = -3.40282347e+38f;
+            if (key + 2 >= a.t) mk.z = -3.40282347e+38f;
+            if (key + 3 >= a.t) mk.w = -3.40282347e+38f;
+          }
+          mmax = fmaxf(mmax, fmaxf(fmaxf(mk.x, mk.y), fmaxf(mk.z, mk.w)));
         }
+      live_pair = q_ok && mmax > -3.0e38f;
     }
     const bool live = __syncthreads_or(live_pair);  // also: the previous step's fragments have been read
     if (live) {
@@ -172,7 +183,7 @@ __global__ void __launch_bounds__(NW * 64) attn_prefill_kernel(AttnPrefillDesc a
           if (a.has_scale) s = s * inv_scale;
           if (M) s = s + mv[i];
           else if (a.has_mask_const) s = s + a.mask_const;
-          if (key + i >= a.t) s = -3.40282347e+38f;  // past the end: contributes exp(..) = 0
+          if (tail && key + i >= a.t) s = -3.40282347e+38f;  // past the end: contributes exp(..) = 0
           st[kt][j * 4 + i] = s;
           tmax = fmaxf(tmax, s);
         }
@@ -190,7 +201,8 @@ __global__ void __launch_bounds__(NW * 64) attn_prefill_kernel(AttnPrefillDesc a
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
           const uint32_t key = t0 + kt * 32 + (blk * 2 + (i >> 2)) * 8 + half * 4 + (i & 3);
-          p[i] = key < a.t ? __expf(st[kt][blk * 8 + i] - m_new) : 0.f;
+          p[i] = __expf(st[kt][blk * 8 + i] - m_new);
+          if (tail && key >= a.t) p[i] = 0.f;
           psum += p[i];
         }
         pf[kt * 2 + blk] = pack8(p);
