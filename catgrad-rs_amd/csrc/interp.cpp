@@ -128,7 +128,6 @@ struct Ctx {
   const cg_env *env;
   const cg_params *params;
   uint32_t err_id = 0;
-  int depth = 0;  // nesting of eval_term (definitions)
 };
 
 int eval_term(Ctx &cx, cg_term *term, std::vector<Value> &args, std::vector<Value> &results);
@@ -460,43 +459,11 @@ int eval_term(Ctx &cx, cg_term *term, std::vector<Value> &args, std::vector<Valu
     args[i].kind = -1;
   }
 
-  // Issue work while the term is still being walked.  A backend that defers its ops would otherwise
-  // start the device only when the caller asks for a result, after the whole walk (a millisecond for
-  // a prefill).  A large tensor that has been waiting for its consumer for FLUSH_AGE ops (the
-  // residual stream across a block, the keys and values a layer returns) is the end of whatever is
-  // computed into it: asking the backend to realise it starts the device on everything before it,
-  // and cannot split a fused pattern, whose interior values are consumed within a few ops.
-  // One-row values (decode steps) are left alone.
-  enum { FLUSH_AGE = 96, FLUSH_EVERY = 32, FLUSH_ROWS = 64 };
-  struct Waiting {
-    uint32_t node, born;
-  };
-  std::vector<Waiting> waiting;
-  uint32_t clock = 0;
-  const bool top = cx.depth == 0;
-  ++cx.depth;
-  struct DepthGuard {
-    int &d;
-    ~DepthGuard() { --d; }
-  } depth_guard{cx.depth};
-
   std::vector<Value> a, out;
   for (uint32_t e : term->order) {
     const Op &op = term->ops[e];
     a.clear();
     out.clear();
-    if (top && ++clock % FLUSH_EVERY == 0 && !waiting.empty()) {
-      size_t keep = 0;
-      for (const Waiting &w : waiting) {
-        if (state[w.node].kind != CG_VAL_TENSOR) continue;  // consumed
-        if (clock - w.born < FLUSH_AGE) {
-          waiting[keep++] = w;
-          continue;
-        }
-        (void)cg_tensor_realize(cx.be, state[w.node].tensor);  // a failure resurfaces when the value is used
-      }
-      waiting.resize(keep);
-    }
     for (uint32_t n : op.src) {
       if (state[n].kind == -1) {
         cx.err_id = n;
@@ -527,12 +494,6 @@ int eval_term(Ctx &cx, cg_term *term, std::vector<Value> &args, std::vector<Valu
         return ierr(CG_ERR_MULTIPLE_WRITE, "MultipleWrite(NodeId(" + std::to_string(n) + "))");
       }
       state[n] = out[i];
-      if (top && out[i].kind == CG_VAL_TENSOR && op.op != CG_OP_LOAD) {
-        const int r = cg_tensor_rank(out[i].tensor);
-        size_t dims[CG_MAX_RANK];
-        if (r >= 2 && cg_tensor_shape(out[i].tensor, dims) == CG_OK && dims[r - 2] >= FLUSH_ROWS)
-          waiting.push_back(Waiting{n, clock});
-      }
     }
   }
 
