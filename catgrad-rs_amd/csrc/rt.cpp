@@ -2993,7 +2993,15 @@ bool share_node(cg_backend *be, cg_tensor *n, cg_tensor **out) {
   }
   n->const_like = true;
   n->cse_key = new std::string(key);
-  if (be->shared_nodes.size() < 4096) be->shared_nodes.emplace(std::move(key), n);
+  if (be->shared_nodes.size() < 4096) {
+    be->shared_nodes.emplace(std::move(key), n);
+    be->shared_keep.push_back(retain(n));
+    if (be->shared_keep.size() > 256) {
+      cg_tensor *old = be->shared_keep.front();
+      be->shared_keep.pop_front();
+      node_release(old);
+    }
+  }
   return false;
 }
 
@@ -3010,10 +3018,24 @@ int finish(cg_backend *be, cg_tensor *n, cg_tensor **out) {
   return CG_OK;
 }
 
+// the block-closing value noted by the previous call (see `binary`), if any, is realised now
+int run_pending_flush(cg_backend *be) {
+  cg_tensor *f = be->flush_node;
+  if (!f) return CG_OK;
+  be->flush_node = nullptr;
+  int st = CG_OK;
+  if (f->rc.load() > 1 && f->op != N_REAL) {  // somebody still wants it
+    hipError_t e = hipSetDevice(be->device);
+    st = e == hipSuccess ? realize(be, f) : fail(be, CG_ERR_DEVICE, hipGetErrorString(e));
+  }
+  node_release(f);
+  return st;
+}
+
 int check_args(cg_backend *be, cg_tensor *a, cg_tensor *b, void *out) {
   if (!be || !a || !out || (b && b->be != be) || a->be != be)
     return fail(be, CG_ERR_ARG, "null or foreign argument");
-  return CG_OK;
+  return run_pending_flush(be);
 }
 
 int to_shape(cg_backend *be, const size_t *dims, int rank, int64_t *shape) {
@@ -3076,7 +3098,26 @@ int binary(cg_backend *be, cg_tensor *a, cg_tensor *b, cg_tensor **out, EwOp f_o
   n->ew = a->dtype == CG_F32 ? f_op : u_op;
   n->in[0] = retain(a);
   n->in[1] = retain(b);
-  return finish(be, n, out);
+  // `residual + linear(...)` over many rows (models/llama.rs:166-186 at prefill sizes) closes a block:
+  // everything the block computes has been recorded, nothing fuses across this add, and the next block
+  // takes a millisecond to record.  Realising it now starts the device on this block while the
+  // caller records the next one.  One-row steps (decode) stay deferred: there the caller overlaps
+  // whole steps.  A broadcast operand (a bias) is not a residual.
+  bool block_end = false;
+  if (n->ew == E_ADD_F && n->rank == 3 && n->shape[1] >= 64 && !(be->flags & (CG_FLAG_EAGER | CG_FLAG_NO_PATTERNS))) {
+    for (int side = 0; side < 2 && !block_end; ++side) {
+      const cg_tensor *mm = n->in[side], *other = n->in[1 - side];
+      if (mm->op == N_RESHAPE) mm = mm->in[0];  // batch folded into the rows for the linear and unfolded again
+      if (mm->op != N_MATMUL || other->op == N_CONST || other->op == N_BROADCAST) continue;
+      bool dense = true;
+      if (other->op == N_REAL)
+        for (int i = 0; i < other->rank; ++i) dense = dense && (other->shape[i] == 1 || other->strides[i] != 0);
+      block_end = dense;
+    }
+  }
+  TRY(finish(be, n, out));
+  if (block_end && *out == n && !be->flush_node) be->flush_node = retain(n);
+  return CG_OK;
 }
 
 int unary(cg_backend *be, cg_tensor *x, cg_tensor **out, EwOp op, cg_dtype out_dtype) {
@@ -3222,6 +3263,14 @@ void cg_backend_destroy(cg_backend *be) {
   std::map<int64_t, cg_tensor *> cache;
   cache.swap(be->arange_cache);
   for (auto &kv : cache) node_release(kv.second);
+  std::deque<cg_tensor *> keep;
+  keep.swap(be->shared_keep);
+  for (cg_tensor *t : keep) node_release(t);
+  if (be->flush_node) {
+    cg_tensor *f = be->flush_node;
+    be->flush_node = nullptr;
+    node_release(f);
+  }
   backend_release(be);
 }
 const char *cg_last_error(const cg_backend *be) { return be ? be->err.c_str() : ""; }

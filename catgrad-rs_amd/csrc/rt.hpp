@@ -11,6 +11,7 @@
 
 #include <atomic>
 #include <cstdint>
+#include <deque>
 #include <map>
 #include <unordered_map>
 #include <string>
@@ -129,6 +130,12 @@ struct cg_backend {
   // for the same causal mask, and gets the same node (weak references; an entry goes when its node is
   // realised or deleted)
   std::unordered_map<std::string, cg_tensor *> shared_nodes;
+  // the most recent of them are kept alive (a realised mask survives from one block to the next, and
+  // from one run to the next), oldest first
+  std::deque<cg_tensor *> shared_keep;
+  // a block-closing value (residual + linear over many rows) to realise at the next call, when its
+  // creator has let go of the operands
+  cg_tensor *flush_node = nullptr;
   // recycled pinned buffers (PREFETCH_BYTES each) and events of cg_tensor_prefetch
   std::vector<void *> pinned_pool;
   std::vector<hipEvent_t> event_pool;
