@@ -3102,16 +3102,17 @@ int binary(cg_backend *be, cg_tensor *a, cg_tensor *b, cg_tensor **out, EwOp f_o
   // everything the block computes has been recorded, nothing fuses across this add, and the next block
   // takes a millisecond to record.  Realising it now starts the device on this block while the
   // caller records the next one.  One-row steps (decode) stay deferred: there the caller overlaps
-  // whole steps.  A broadcast operand (a bias) is not a residual.
+  // whole steps.  A broadcast operand (a bias) is not a residual, nor is a value that is still deferred.
   bool block_end = false;
   if (n->ew == E_ADD_F && n->rank == 3 && n->shape[1] >= 64 && !(be->flags & (CG_FLAG_EAGER | CG_FLAG_NO_PATTERNS))) {
     for (int side = 0; side < 2 && !block_end; ++side) {
       const cg_tensor *mm = n->in[side], *other = n->in[1 - side];
       if (mm->op == N_RESHAPE) mm = mm->in[0];  // batch folded into the rows for the linear and unfolded again
-      if (mm->op != N_MATMUL || other->op == N_CONST || other->op == N_BROADCAST) continue;
+      // the residual stream is a value in memory (the previous block end); anything still deferred
+      // on the other side may be part of a pattern around the product (gelu's x + c x^3)
+      if (mm->op != N_MATMUL || other->op != N_REAL) continue;
       bool dense = true;
-      if (other->op == N_REAL)
-        for (int i = 0; i < other->rank; ++i) dense = dense && (other->shape[i] == 1 || other->strides[i] != 0);
+      for (int i = 0; i < other->rank; ++i) dense = dense && (other->shape[i] == 1 || other->strides[i] != 0);
       block_end = dense;
     }
   }

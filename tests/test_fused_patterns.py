@@ -209,8 +209,16 @@ def test_gated_activation_in_the_gemm_epilogue(oracle, hip_bf16, shape, act):
         h = (nn.silu(b, gt) if act == "silu" else nn.gelu(b, gt)) * up
         return nn.linear_no_bias(b, N, K, lang.path(["d"]), h), h
     ref = vectors.run(oracle, f, 2, x, params=p)
-    got, names = run_traced(hip_bf16, f, 2, x, params=p)
-    assert "swiglu_fused" not in names and "geglu_fused" not in names, sorted(names)
+    hip_bf16.trace(True)
+    hip_bf16.trace_reset()
+    got = vectors.run(hip_bf16, f, 2, x, params=p)
+    rep = hip_bf16.trace_report()
+    hip_bf16.trace(False)
+    launches = {k: v["launches"] for k, v in rep.items()}
+    # x + x - x, three GEMMs, nothing else: no activation kernel, no generic program, no narrowing pass for h
+    assert launches.get("gemm_mfma_bf16") == 3 and launches.get("ew_fused") == 1, launches
+    # (ew_to_bf16: the uploads of x and the three weights)
+    assert set(launches) <= {"gemm_mfma_bf16", "ew_fused", "cast_bf16", "ew_to_bf16"} and launches.get("cast_bf16", 0) <= 1, launches
     for r, d in zip(ref, got):
         assert np.max(np.abs(d - r)) <= 2e-2 * np.abs(r).max()
 

@@ -5,6 +5,7 @@ import numpy as np
 import pytest
 
 import llama_util as U
+import vectors
 
 
 def greedy_reference_style(be, cfg, arrays, prompt, steps):
@@ -106,6 +107,36 @@ def test_llama_bf16_logits(oracle, hip_bf16):
     _, gl = g.step(tok)
     rl, gl = oracle.to_vec(rl), hip_bf16.to_vec(gl)
     assert np.max(np.abs(rl - gl)) <= 2e-2 * np.abs(rl).max()
+
+
+@pytest.mark.gpu
+def test_llama_prefill_of_many_rows(oracle, hip, hip_bf16):
+    """A 256-token prompt: the sizes at which products are grouped, split along k with the residual
+    added by the summing pass, gated activations applied by up_proj's GEMM, and blocks issued while
+    the next is recorded.  f32 at 1e-4, bf16 at 2e-2, and the bf16 launch mix."""
+    cfg = U.tiny_config(hidden_size=256, intermediate_size=512, num_hidden_layers=3, num_attention_heads=4,
+                        num_key_value_heads=2, vocab_size=300)
+    arrays = U.param_arrays(cfg, seed=11, std=0.05)
+    rounded = {k: (vectors.bf16_round(a) if a.ndim >= 2 else a) for k, a in arrays.items()}
+    prompt = list(np.random.default_rng(9).integers(0, cfg.vocab_size, 256))
+    _, rl = U.CachedRunner(oracle, cfg, arrays, 300).prefill(prompt)
+    _, gl = U.CachedRunner(hip, cfg, arrays, 300).prefill(prompt)
+    rl, gl = oracle.to_vec(rl), hip.to_vec(gl)
+    assert np.max(np.abs(rl - gl)) <= 1e-4 * np.abs(rl).max()
+    _, rl = U.CachedRunner(oracle, cfg, rounded, 300).prefill(prompt)
+    g = U.CachedRunner(hip_bf16, cfg, arrays, 300)
+    hip_bf16.trace(True)
+    hip_bf16.trace_reset()
+    _, gl = g.prefill(prompt)
+    rl, gl = oracle.to_vec(rl), hip_bf16.to_vec(gl)
+    rep = hip_bf16.trace_report()
+    hip_bf16.trace(False)
+    assert np.max(np.abs(rl - gl)) <= 2e-2 * np.abs(rl).max()
+    launches = {k: v["launches"] for k, v in rep.items()}
+    # per layer: q/k/v grouped, o_proj, gate_proj, up_proj (with the activation), down_proj, and the two
+    # products of an attention this short (the one-pass kernel starts at 512 keys) = 7 GEMMs
+    assert launches.get("gemm_mfma_bf16") == 7 * cfg.num_hidden_layers, launches
+    assert "swiglu_fused" not in launches, launches
 
 
 @pytest.mark.gpu
