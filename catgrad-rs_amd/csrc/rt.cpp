@@ -2996,7 +2996,7 @@ bool share_node(cg_backend *be, cg_tensor *n, cg_tensor **out) {
   if (be->shared_nodes.size() < 4096) {
     be->shared_nodes.emplace(std::move(key), n);
     be->shared_keep.push_back(retain(n));
-    if (be->shared_keep.size() > 256) {
+    if (be->shared_keep.size() > 64) {  // a handful of masks: each may hold S x S floats once realised
       cg_tensor *old = be->shared_keep.front();
       be->shared_keep.pop_front();
       node_release(old);
