@@ -275,6 +275,10 @@ struct GemvProDesc {
   uint32_t *err;
 };
 hipError_t launch_gemv_pro(const LaunchCtx &lc, const GemvProDesc &g);
+// The batched, expert-indexed form for many tokens (a MoE prefill): same descriptor (bf16 weights,
+// PRO_NONE / PRO_SWIGLU / PRO_GEGLU, no c_add), each expert's matrix read once per 128 columns
+// instead of once per token; inputs are rounded to bf16 like every many-row product in bf16 mode.
+hipError_t launch_moe_gemm(const LaunchCtx &lc, const GemvProDesc &g);
 // wrapping u32 matmul (ndarray's generic dot); all operands contiguous
 hipError_t launch_matmul_u32(const LaunchCtx &lc, const uint32_t *a, const uint32_t *b, uint32_t *c,
                              uint32_t batch, uint32_t M, uint32_t N, uint32_t K);

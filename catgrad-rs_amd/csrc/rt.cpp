@@ -2451,7 +2451,16 @@ int try_moe_gemv(cg_backend *be, cg_tensor *n, bool *done) {
     bytes += (double)S * pr.N * K * esize(w->stype) + (double)S * pr.N * 4;
     flops += 2.0 * S * pr.N * K;
   }
-  if (!st) {
+  // many tokens (a prefill): expert-major, each expert's matrix read once per column tile instead of
+  // once per token
+  const bool many = S >= 64 && b_stype == ST_BF16 && (be->flags & CG_FLAG_BF16);
+  if (!st && many) {
+    double wbytes = 0;
+    for (int i = 0; i < d.m.n_prob; ++i) wbytes += (double)d.b_index_limit * d.m.p[i].N * K * 2 + (double)S * d.m.p[i].N * 4;
+    KernelScope ks(be, "gemm_experts_bf16", (double)S * K * 4 * (pro == PRO_NONE ? 1 : 2) + wbytes, flops);
+    hipError_t e = launch_moe_gemm(be->lc(), d);
+    if (e != hipSuccess) st = fail(be, CG_ERR_DEVICE, hipGetErrorString(e));
+  } else if (!st) {
     const char *base = b_stype == ST_BF16 ? "gemv_experts_bf16" : "gemv_experts_f32";
     KernelScope ks(be, base, bytes, flops);
     hipError_t e = launch_gemv_pro(be->lc(), d);

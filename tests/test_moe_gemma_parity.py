@@ -125,7 +125,9 @@ def U_round(a):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("dev_name", ["hip", "hip_bf16"])
-@pytest.mark.parametrize("shape", [(5, 8, 24, 64), (1, 4, 96, 1024), (33, 6, 40, 72)])  # S, E, N, K
+@pytest.mark.parametrize("shape", [(5, 8, 24, 64), (1, 4, 96, 1024), (33, 6, 40, 72),
+                                   (200, 5, 160, 128), (1100, 3, 136, 72)])  # S, E, N, K; from 64 tokens on, bf16
+                                                                              # mode multiplies expert by expert
 def test_expert_indirect_matmul(request, oracle, hip_nopat, dev_name, shape):
     """matmul(x[S,1,K], transpose(1,2, index(0, idx, W[E,N,K]))) reads the expert matrices in place
     (no gather launch), with the same result as the oracle and as the gathering path."""
@@ -176,6 +178,40 @@ def test_expert_index_out_of_bounds_is_reported(hip):
     # the flag is cleared: the next evaluation is clean
     (ok,) = vectors.run(hip, f, 1, x, np.array([1, 2], np.uint32), w)
     assert np.array_equal(ok, np.full((2, 1, 8), 16.0, np.float32))
+
+
+@pytest.mark.gpu
+def test_expert_mlp_over_many_tokens(oracle, hip_bf16):
+    """One expert slot of the MoE block (models/qwen3.rs:104-123) over 300 tokens in bf16 mode: gate and
+    up as expert-major products, SwiGLU computed on the way into down_proj's product; and an index
+    past the last expert is reported there too."""
+    import vectors
+    lang, nn = vectors.lang, vectors.nn
+    S, E, F, H = 300, 7, 96, 128
+    g = np.random.default_rng(5)
+    x = g.standard_normal((S, 1, H)).astype(np.float32)
+    wg, wu = (U_round((g.standard_normal((E, F, H)) * 0.1).astype(np.float32)) for _ in range(2))
+    wd = U_round((g.standard_normal((E, H, F)) * 0.1).astype(np.float32))
+    idx = g.integers(0, E, (S, 1)).astype(np.uint32)
+
+    def f(b, xv, iv, g_all, u_all, d_all):
+        xv = xv + xv - xv
+        sel = lambda w: lang.transpose(b, 1, 2, lang.index(b, 0, iv, w))
+        gate = lang.matmul(b, xv, sel(g_all))
+        up = lang.matmul(b, xv, sel(u_all))
+        return lang.matmul(b, nn.silu(b, gate) * up, sel(d_all))
+    (ref,) = vectors.run(oracle, f, 1, x, idx, wg, wu, wd)
+    hip_bf16.trace(True)
+    hip_bf16.trace_reset()
+    (got,) = vectors.run(hip_bf16, f, 1, x, idx, wg, wu, wd)
+    rep = hip_bf16.trace_report()
+    hip_bf16.trace(False)
+    assert rep["gemm_experts_bf16"]["launches"] == 2 and "gather" not in rep and "swiglu_fused" not in rep, sorted(rep)
+    assert np.max(np.abs(got - ref)) <= 2e-2 * np.abs(ref).max()
+    bad = idx.copy()
+    bad[17, 0] = E
+    with pytest.raises(cg.abi.BackendPanic, match="index out of bounds"):
+        vectors.run(hip_bf16, f, 1, x, bad, wg, wu, wd)
 
 
 def moe_cached_generate(be, cfg, arrays, prompts, steps):
