@@ -414,6 +414,28 @@ def test_bf16_mode_matmul(cg, oracle, hip_bf16):
     assert_bits(got, rne[idx])
 
 
+@pytest.mark.gpu
+def test_bf16_mode_matmul_shape_sweep(oracle, hip_bf16):
+    """Many-row products in bf16 mode across the shapes that select different GEMM variants (tile
+    sizes, two or four LDS stages, split-K, tails in every dimension, batches), against the oracle on
+    operands already rounded to bf16."""
+    import vectors
+    g = rng(61)
+    shapes = [(1, 64, 64, 64), (1, 64, 128, 128), (1, 100, 192, 200), (1, 512, 320, 512), (1, 130, 1024, 192),
+              (1, 256, 2048, 256), (1, 1024, 64, 1024), (1, 2048, 256, 2048), (3, 200, 128, 136), (2, 64, 4096, 64),
+              (1, 72, 72, 72), (1, 512, 8192, 128)]       # batch, M, K, N
+    for (b, m, k, n) in shapes:
+        x = vectors.bf16_round(g.standard_normal((b, m, k)).astype(np.float32))
+        w = vectors.bf16_round((g.standard_normal((b, n, k)) * 0.05).astype(np.float32))
+
+        def f(be, x, w):
+            x = be.add(x, be.sub(x, x))                      # a computed f32 value
+            return be.matmul(x, be.transpose(w, 1, 2))
+        r, d = both(oracle, hip_bf16, f, x, w)
+        scale = np.matmul(np.abs(x), np.abs(np.swapaxes(w, 1, 2)))
+        assert_close(r[0], d[0], RTOL_BF16, scale=scale)
+
+
 def test_row_fusion_layernorm_and_softmax_views(oracle, hip, hip_eager):
     """Row programs (reduction stages + final segment in one kernel) on strided inputs: softmax of
     a transposed view, layernorm with gamma/beta broadcasts, and a row value read twice."""
