@@ -1105,113 +1105,172 @@ hipError_t launch_gemv_pro(const LaunchCtx &lc, const GemvProDesc &g) {
 }
 
 // ---- routed experts over many tokens (a MoE prefill) ----------------------------------------------------
-// The same batched product as above (batch z = token z, its expert b_index[z]) when there are enough
-// tokens for an expert's matrix to be worth reading once instead of once per token: a workgroup
-// owns (128 output columns, one expert, one problem).  It walks the index vector in segments of
-// 1024 tokens, collects the tokens routed to its expert in LDS, and multiplies them 32 at a time
-// against its weight tile with v_mfma_f32_32x32x16_bf16 (token rows gathered, narrowed to bf16 and -
-// for down_proj - computed from gate and up on the way into LDS); rows are scattered back to their
-// tokens.  Every token belongs to exactly one expert, so every output row is written once.  An index
+// The batched, expert-indexed product above once there are enough tokens for an expert's matrix to
+// be worth reading once instead of once per token: a workgroup owns (128 output columns, one
+// expert, one problem).  It walks the (slot, token) pairs in segments of 4096, collects those
+// routed to its expert in LDS, and multiplies them 128 at a time against its weight tile with
+// v_mfma_f32_32x32x16_bf16 (token rows gathered, narrowed to bf16 and - for down_proj - computed
+// from gate and up on the way into LDS); rows are scattered back to their slot's output.  Every
+// (slot, token) pair belongs to exactly one expert, so every output row is written once.  An index
 // past the last expert is flagged and served by the last expert, like the one-row kernel's clamp.
-__global__ void __launch_bounds__(256) moe_gemm_kernel(GemvProDesc g) {
-  constexpr int BM_ = 32, BN_ = 128, BK = 64, LD = BK + 8, SEG = 1024;
+// NP weight tiles per workgroup: 1, or 2 for the fused gate / up form (fuse_glu).
+template <int NP>
+__global__ void __launch_bounds__(256) moe_gemm_kernel(MoeGemmDesc g) {
+  constexpr int BM_ = 128, BN_ = 128, BK = 64, LD = BK + 8, SEG = 4096, MT = BM_ / 32;
   __shared__ __attribute__((aligned(16))) uint16_t As[BM_ * LD];
-  __shared__ __attribute__((aligned(16))) uint16_t Bs[BN_ * LD];
-  __shared__ uint32_t list[SEG];
+  __shared__ __attribute__((aligned(16))) uint16_t Bs[NP][BN_ * LD];
+  __shared__ uint32_t list[SEG];  // slot << 16 | token
   __shared__ uint32_t count;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const uint32_t e = blockIdx.y, n0 = blockIdx.x * BN_, prob = blockIdx.z;
-  const uint32_t K = g.m.K, N = g.m.p[prob].N, S = g.batch;
-  const int64_t sbn = g.m.p[prob].sbn;
-  const uint16_t *W = (const uint16_t *)g.m.p[prob].b + (int64_t)e * g.sb_index;
-  float *C = g.m.p[prob].c;
-  const bool last = e + 1 == g.b_index_limit;
-  // staging roles: A chunk (row, 8 k) per thread; B chunks (col, 8 k) four per thread
-  const int a_row = tid >> 3, a_k8 = (tid & 7) * 8;
-  for (uint32_t s0 = 0; s0 < S; s0 += SEG) {
+  const uint32_t e = blockIdx.y, n0 = blockIdx.x * BN_, prob = NP == 2 ? 0 : blockIdx.z;
+  const uint32_t K = g.K, N = g.prob[prob].N, S = g.S;
+  if (n0 >= N) return;  // the other problem is wider
+  const uint16_t *W[NP];
+  int64_t sbn[NP];
+#pragma unroll
+  for (int p = 0; p < NP; ++p) {
+    W[p] = (const uint16_t *)g.prob[prob + p].w + (int64_t)e * g.sb_index;
+    sbn[p] = g.prob[prob + p].sbn;
+  }
+  const bool last = e + 1 == g.n_expert;
+  const uint32_t pairs = S * g.n_slot;
+  const int a_k8 = (tid & 7) * 8;  // this thread's 8 k of the staged rows tid >> 3, + 32, + 64, + 96
+  for (uint32_t s0 = 0; s0 < pairs; s0 += SEG) {
     if (tid == 0) count = 0;
     __syncthreads();
-    for (uint32_t t = s0 + tid; t < min(S, s0 + SEG); t += 256) {
-      const uint32_t ix = g.b_index[(int64_t)t * g.b_index_stride];
-      if (ix >= g.b_index_limit) atomicOr(g.err, ERRF_INDEX_OOB);
-      if (ix == e || (last && ix >= g.b_index_limit)) list[atomicAdd(&count, 1u)] = t;
+    for (uint32_t p = s0 + tid; p < min(pairs, s0 + SEG); p += 256) {
+      const uint32_t sl = p / S, t = p - sl * S;
+      const uint32_t ix = g.slot[sl].idx[(int64_t)t * g.slot[sl].idx_stride];
+      if (ix >= g.n_expert) atomicOr(g.err, ERRF_INDEX_OOB);
+      if (ix == e || (last && ix >= g.n_expert)) list[atomicAdd(&count, 1u)] = sl << 16 | t;
     }
     __syncthreads();
     const uint32_t cnt = count;
     for (uint32_t m0 = 0; m0 < cnt; m0 += BM_) {
-      f32x16 acc;
+      const int live_tiles = (int)min((uint32_t)MT, (cnt - m0 + 31) / 32);  // 32-row tiles with any row (uniform)
+      f32x16 acc[NP][MT];
 #pragma unroll
-      for (int i = 0; i < 16; ++i) acc[i] = 0.f;
-      const bool a_live = m0 + a_row < cnt;
-      const uint32_t tok = a_live ? list[m0 + a_row] : 0u;
-      const float *arow = g.a + (int64_t)tok * g.a_bstride, *xrow = g.aux ? g.aux + (int64_t)tok * g.aux_bstride : nullptr;
-      for (uint32_t k0 = 0; k0 < K; k0 += BK) {
-        // ---- token rows -> LDS (bf16)
-        float v[8];
-        if (a_live && k0 + a_k8 < K) {
-          const float4 x0 = *(const float4 *)(arow + k0 + a_k8), x1 = *(const float4 *)(arow + k0 + a_k8 + 4);
-          v[0] = x0.x; v[1] = x0.y; v[2] = x0.z; v[3] = x0.w; v[4] = x1.x; v[5] = x1.y; v[6] = x1.z; v[7] = x1.w;
-          if (g.pro == PRO_SWIGLU || g.pro == PRO_GEGLU) {
-            const float4 u0 = *(const float4 *)(xrow + k0 + a_k8), u1 = *(const float4 *)(xrow + k0 + a_k8 + 4);
-            const float u[8] = {u0.x, u0.y, u0.z, u0.w, u1.x, u1.y, u1.z, u1.w};
+      for (int p = 0; p < NP; ++p)
 #pragma unroll
-            for (int i = 0; i < 8; ++i) v[i] = (g.pro == PRO_GEGLU ? gelu_ref(v[i]) : v[i] * sigmoid_ref(v[i])) * u[i];
+        for (int h = 0; h < MT; ++h)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) acc[p][h][i] = 0.f;
+      const float *arow[MT], *xrow[MT];
+      const uint16_t *hrow[MT];
+      bool a_live[MT];
+#pragma unroll
+      for (int h = 0; h < MT; ++h) {
+        const uint32_t r = m0 + (tid >> 3) + h * 32;
+        a_live[h] = r < cnt;
+        const uint32_t ent = a_live[h] ? list[r] : 0u, sl = ent >> 16, tok = ent & 0xFFFFu;
+        arow[h] = g.slot[sl].a ? g.slot[sl].a + (int64_t)tok * g.slot[sl].a_bs : nullptr;
+        xrow[h] = g.slot[sl].aux ? g.slot[sl].aux + (int64_t)tok * g.slot[sl].aux_bs : nullptr;
+        hrow[h] = g.slot[sl].a16 ? g.slot[sl].a16 + (int64_t)tok * g.slot[sl].a_bs : nullptr;
+      }
+      // registers of the k-step in flight: token rows (as bf16) and the weight tiles
+      uint4 q[MT];
+      u32x4n wq[NP][4];
+      auto fetch = [&](uint32_t k0) {
+#pragma unroll
+        for (int h = 0; h < MT; ++h) {
+          if (!a_live[h] || k0 + a_k8 >= K) {
+            q[h] = make_uint4(0u, 0u, 0u, 0u);
+          } else if (hrow[h]) {
+            q[h] = *(const uint4 *)(hrow[h] + k0 + a_k8);
+          } else {
+            const float4 x0 = *(const float4 *)(arow[h] + k0 + a_k8), x1 = *(const float4 *)(arow[h] + k0 + a_k8 + 4);
+            float v[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
+            if (g.pro == PRO_SWIGLU || g.pro == PRO_GEGLU) {
+              const float4 u0 = *(const float4 *)(xrow[h] + k0 + a_k8), u1 = *(const float4 *)(xrow[h] + k0 + a_k8 + 4);
+              const float u[8] = {u0.x, u0.y, u0.z, u0.w, u1.x, u1.y, u1.z, u1.w};
+#pragma unroll
+              for (int i = 0; i < 8; ++i) v[i] = (g.pro == PRO_GEGLU ? gelu_ref(v[i]) : v[i] * sigmoid_ref(v[i])) * u[i];
+            }
+            const uint2 lo = bf16_pack4(make_float4(v[0], v[1], v[2], v[3])), hi = bf16_pack4(make_float4(v[4], v[5], v[6], v[7]));
+            q[h] = make_uint4(lo.x, lo.y, hi.x, hi.y);
           }
-        } else {
-#pragma unroll
-          for (int i = 0; i < 8; ++i) v[i] = 0.f;
         }
-        uint4 q;
-        q.x = bf16_bits(v[0]) | (bf16_bits(v[1]) << 16); q.y = bf16_bits(v[2]) | (bf16_bits(v[3]) << 16);
-        q.z = bf16_bits(v[4]) | (bf16_bits(v[5]) << 16); q.w = bf16_bits(v[6]) | (bf16_bits(v[7]) << 16);
-        // ---- weight tile -> LDS
-        u32x4n wq[4];
 #pragma unroll
-        for (int c = 0; c < 4; ++c) {
-          const int ch = tid + c * 256, col = ch >> 3, k8 = (ch & 7) * 8;
-          wq[c] = (k0 + k8 < K) ? __builtin_nontemporal_load((const u32x4n *)(W + (int64_t)min(n0 + col, N - 1) * sbn + k0 + k8))
-                                : (u32x4n){0u, 0u, 0u, 0u};
-        }
+        for (int p = 0; p < NP; ++p)
+#pragma unroll
+          for (int c = 0; c < 4; ++c) {
+            const int ch = tid + c * 256, col = ch >> 3, k8 = (ch & 7) * 8;
+            wq[p][c] = (k0 + k8 < K)
+                           ? __builtin_nontemporal_load((const u32x4n *)(W[p] + (int64_t)min(n0 + col, N - 1) * sbn[p] + k0 + k8))
+                           : (u32x4n){0u, 0u, 0u, 0u};
+          }
+      };
+      fetch(0);
+      for (uint32_t k0 = 0; k0 < K; k0 += BK) {
         __syncthreads();  // the previous step's fragments have been read
-        *(uint4 *)(&As[a_row * LD + a_k8]) = q;
 #pragma unroll
-        for (int c = 0; c < 4; ++c) {
-          const int ch = tid + c * 256, col = ch >> 3, k8 = (ch & 7) * 8;
-          *(u32x4n *)(&Bs[col * LD + k8]) = wq[c];
-        }
+        for (int h = 0; h < MT; ++h) *(uint4 *)(&As[((tid >> 3) + h * 32) * LD + a_k8]) = q[h];
+#pragma unroll
+        for (int p = 0; p < NP; ++p)
+#pragma unroll
+          for (int c = 0; c < 4; ++c) {
+            const int ch = tid + c * 256, col = ch >> 3, k8 = (ch & 7) * 8;
+            *(u32x4n *)(&Bs[p][col * LD + k8]) = wq[p][c];
+          }
         __syncthreads();
+        if (k0 + BK < K) fetch(k0 + BK);  // in flight during the products below
 #pragma unroll
         for (int ks = 0; ks < BK / 16; ++ks) {
-          const bf16x8 af = *(const bf16x8 *)(&As[(lane & 31) * LD + ks * 16 + (lane >> 5) * 8]);
-          const bf16x8 bf = *(const bf16x8 *)(&Bs[(wave * 32 + (lane & 31)) * LD + ks * 16 + (lane >> 5) * 8]);
-          acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af, bf, acc, 0, 0, 0);
+          bf16x8 bf[NP];
+#pragma unroll
+          for (int p = 0; p < NP; ++p)
+            bf[p] = *(const bf16x8 *)(&Bs[p][(wave * 32 + (lane & 31)) * LD + ks * 16 + (lane >> 5) * 8]);
+#pragma unroll
+          for (int h = 0; h < MT; ++h) {
+            if (h < live_tiles) {
+              const bf16x8 af = *(const bf16x8 *)(&As[(h * 32 + (lane & 31)) * LD + ks * 16 + (lane >> 5) * 8]);
+#pragma unroll
+              for (int p = 0; p < NP; ++p) acc[p][h] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af, bf[p], acc[p][h], 0, 0, 0);
+            }
+          }
         }
       }
-      // ---- rows back to their tokens: register i is row (i >> 2) * 8 + (lane >> 5) * 4 + (i & 3), column lane & 31
+      // ---- rows back to their slot and token: register i of tile h is row
+      // h * 32 + (i >> 2) * 8 + (lane >> 5) * 4 + (i & 3), column lane & 31
       const uint32_t col = n0 + wave * 32 + (lane & 31);
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const uint32_t r = m0 + (i >> 2) * 8 + (lane >> 5) * 4 + (i & 3);
-        if (r < cnt && col < N) C[(uint64_t)list[r] * N + col] = acc[i];
-      }
+      for (int h = 0; h < MT; ++h)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const uint32_t r = m0 + h * 32 + (i >> 2) * 8 + (lane >> 5) * 4 + (i & 3);
+          if (r < cnt && col < N) {
+            const uint32_t ent = list[r];
+            const uint64_t at = (uint64_t)(ent & 0xFFFFu) * N + col;
+            if (NP == 2) {
+              const float gt = acc[0][h][i];
+              const float hv = (g.fuse_glu == PRO_GEGLU ? gelu_ref(gt) : gt * sigmoid_ref(gt)) * acc[NP - 1][h][i];
+              g.slot[ent >> 16].h16[at] = (uint16_t)bf16_bits(hv);
+            } else {
+              g.slot[ent >> 16].c[prob][at] = acc[0][h][i];
+            }
+          }
+        }
       __syncthreads();  // As / Bs and the list are reused
     }
     __syncthreads();
   }
 }
 
-hipError_t launch_moe_gemm(const LaunchCtx &lc, const GemvProDesc &g) {
-  if (!g.batch || !g.m.n_prob || !g.b_index || !g.b_index_limit) return hipSuccess;
-  if (g.m.b_stype != ST_BF16 || g.m.K % 8 || g.pro == PRO_RMSNORM || g.glu_epilogue || g.b_index_limit > 65535)
+hipError_t launch_moe_gemm(const LaunchCtx &lc, const MoeGemmDesc &g) {
+  if (!g.S || !g.n_prob || !g.n_slot || !g.n_expert) return hipSuccess;
+  if (g.S > 65535 || g.n_slot > 8 || g.n_prob > 2 || g.n_expert > 65535 || g.K % 8 || g.pro == PRO_RMSNORM)
     return hipErrorInvalidValue;
   uint32_t max_n = 0;
-  for (int i = 0; i < g.m.n_prob; ++i) {
-    if (g.m.p[i].c_add) return hipErrorInvalidValue;
-    max_n = g.m.p[i].N > max_n ? g.m.p[i].N : max_n;
-  }
+  for (uint32_t i = 0; i < g.n_prob; ++i) max_n = g.prob[i].N > max_n ? g.prob[i].N : max_n;
   if (!max_n) return hipSuccess;
-  dim3 grid((max_n + 127) / 128, g.b_index_limit, g.m.n_prob);
-  CG_LAUNCH(lc, moe_gemm_kernel, grid, 256, g);
+  if (g.fuse_glu) {
+    if (g.n_prob != 2 || g.prob[0].N != g.prob[1].N || g.pro != PRO_NONE) return hipErrorInvalidValue;
+    dim3 grid((max_n + 127) / 128, g.n_expert, 1);
+    CG_LAUNCH(lc, moe_gemm_kernel<2>, grid, 256, g);
+  } else {
+    dim3 grid((max_n + 127) / 128, g.n_expert, g.n_prob);
+    CG_LAUNCH(lc, moe_gemm_kernel<1>, grid, 256, g);
+  }
   return hipGetLastError();
 }
 

@@ -275,10 +275,37 @@ struct GemvProDesc {
   uint32_t *err;
 };
 hipError_t launch_gemv_pro(const LaunchCtx &lc, const GemvProDesc &g);
-// The batched, expert-indexed form for many tokens (a MoE prefill): same descriptor (bf16 weights,
-// PRO_NONE / PRO_SWIGLU / PRO_GEGLU, no c_add), each expert's matrix read once per 128 columns
-// instead of once per token; inputs are rounded to bf16 like every many-row product in bf16 mode.
-hipError_t launch_moe_gemm(const LaunchCtx &lc, const GemvProDesc &g);
+// The routed experts of a MoE layer over many tokens (a prefill; models/qwen3.rs:104-123), expert by
+// expert.  A slot is one of the k choices of every token: its index vector, its input rows and its
+// outputs.  A problem is one stacked weight tensor [E, N, K] (bf16): gate_proj and up_proj share
+// input rows and indices, so they go out together (n_prob = 2); down_proj (n_prob = 1) computes its
+// rows from gate and up (pro = PRO_SWIGLU / PRO_GEGLU, aux = up).  All slots of a layer go out in one
+// launch, so an expert's matrix is read once per 128 columns for every token that chose it in any
+// slot.  Inputs are rounded to bf16 like every many-row product in bf16 mode.
+struct MoeGemmDesc {
+  uint32_t S, K, n_slot, n_prob, n_expert;  // S <= 65535 tokens, n_slot <= 8, n_prob <= 2
+  int32_t pro;                              // PRO_NONE, PRO_SWIGLU or PRO_GEGLU (f32 input rows only)
+  // 0, or PRO_SWIGLU / PRO_GEGLU with n_prob == 2 problems of equal N (gate, up): a workgroup computes
+  // both products of its tokens and stores act(first) * second as bf16 into slot[].h16; c is unused
+  int32_t fuse_glu;
+  int64_t sb_index;                         // elements between two experts' matrices
+  struct {
+    const uint32_t *idx;                    // idx[t * idx_stride] = expert of token t in this slot
+    int64_t idx_stride;
+    const float *a, *aux;                   // f32 input rows: a + t * a_bs (aux + t * aux_bs), unit stride along k
+    const uint16_t *a16;                    // or bf16 input rows (a16 + t * a_bs), taken as they are
+    int64_t a_bs, aux_bs;
+    float *c[2];                            // outputs per problem, contiguous [S, N]
+    uint16_t *h16;                          // fuse_glu: gated activations, contiguous bf16 [S, N]
+  } slot[8];
+  struct {
+    const void *w;                          // [E, N, K], unit stride along k, row stride sbn
+    int64_t sbn;
+    uint32_t N;
+  } prob[2];
+  uint32_t *err;                            // ERRF_INDEX_OOB for an index >= n_expert (served by the last expert)
+};
+hipError_t launch_moe_gemm(const LaunchCtx &lc, const MoeGemmDesc &g);
 // wrapping u32 matmul (ndarray's generic dot); all operands contiguous
 hipError_t launch_matmul_u32(const LaunchCtx &lc, const uint32_t *a, const uint32_t *b, uint32_t *c,
                              uint32_t batch, uint32_t M, uint32_t N, uint32_t K);

@@ -2355,8 +2355,292 @@ bool match_expert_operand(const cg_tensor *t, int64_t S, ExpertOperand *o) {
   return true;
 }
 
+// The same products over many tokens (a prefill, bf16 mode): expert by expert instead of token by
+// token, and all k slots of the layer in one launch - every deferred expert product on the same
+// stacked weights joins, with its own indices, input rows and output (launch_moe_gemm).
+int try_moe_gemm(cg_backend *be, cg_tensor *n, bool *done) {
+  const int64_t S = n->shape[0];
+  if (S < 64 || S > 65535 || !(be->flags & CG_FLAG_BF16)) return CG_OK;
+  ExpertOperand eo;
+  if (!match_expert_operand(n->in[1], S, &eo)) return CG_OK;
+  const int64_t K = n->in[0]->shape[2];
+  if (n->in[0]->rank != 3 || K % 8 || K < 8) return CG_OK;
+  cg_tensor *gate = nullptr, *up = nullptr;
+  int gelu = 0;
+  const bool glu = n->in[0]->op != N_REAL && refs(n->in[0]) == 1 && match_glu(n->in[0], &gate, &up, &gelu);
+  struct Member {
+    cg_tensor *c, *w, *idx;
+    int slot, prob;
+  };
+  std::vector<Member> members;
+  std::vector<cg_tensor *> slot_idx, prob_w, slot_a;
+  auto find_or_add = [](std::vector<cg_tensor *> &v, cg_tensor *t) {
+    for (size_t i = 0; i < v.size(); ++i)
+      if (v[i] == t) return (int)i;
+    v.push_back(t);
+    return (int)v.size() - 1;
+  };
+  // n first, then every other deferred expert product that fits: same rows and any of the same
+  // weight tensors (gate / up), or - for down_proj - the same weights and its own gated rows
+  std::vector<cg_tensor *> cands{n};
+  for (cg_tensor *c : be->gemv_candidates)
+    if (c != n) cands.push_back(c);
+  for (cg_tensor *c : cands) {
+    if (c->op != N_MATMUL || c->rank != 3 || c->shape[0] != S || c->shape[1] != 1 || c->in[0]->rank != 3 || c->in[0]->shape[2] != K)
+      continue;
+    ExpertOperand co;
+    if (!match_expert_operand(c->in[1], S, &co)) continue;
+    if (glu) {
+      cg_tensor *g2 = nullptr, *u2 = nullptr;
+      int ge2 = 0;
+      if (co.w != eo.w || c->in[0]->op == N_REAL || refs(c->in[0]) != 1 || !match_glu(c->in[0], &g2, &u2, &ge2) || ge2 != gelu)
+        continue;
+      if (slot_idx.size() >= 8 && c != n) continue;
+      members.push_back(Member{c, co.w, co.idx, (int)slot_idx.size(), 0});
+      slot_idx.push_back(co.idx);
+      slot_a.push_back(c->in[0]);
+      if (prob_w.empty()) prob_w.push_back(co.w);
+    } else {
+      if (c->in[0] != n->in[0]) continue;
+      // a third weight tensor or a ninth slot stays outside
+      bool known_w = false, known_i = false;
+      for (cg_tensor *w : prob_w) known_w = known_w || w == co.w;
+      for (cg_tensor *i : slot_idx) known_i = known_i || i == co.idx;
+      if ((!known_w && prob_w.size() >= 2) || (!known_i && slot_idx.size() >= 8)) continue;
+      members.push_back(Member{c, co.w, co.idx, find_or_add(slot_idx, co.idx), find_or_add(prob_w, co.w)});
+    }
+  }
+  // every (slot, problem) pair exactly once, or only n's own slot
+  auto complete = [&]() {
+    if (members.size() != slot_idx.size() * prob_w.size()) return false;
+    std::vector<int> seen(slot_idx.size() * prob_w.size(), 0);
+    for (const Member &m : members)
+      if (seen[m.slot * prob_w.size() + m.prob]++) return false;
+    return true;
+  };
+  if (!complete()) {
+    std::vector<Member> own;
+    for (const Member &m : members)
+      if (m.idx == eo.idx && (glu ? m.c == n : true)) own.push_back(m);
+    members.swap(own);
+    slot_idx.assign(1, eo.idx);
+    if (glu) slot_a.assign(1, n->in[0]);
+    prob_w.clear();
+    for (Member &m : members) {
+      m.slot = 0;
+      m.prob = find_or_add(prob_w, m.w);
+    }
+    if (!complete()) return CG_OK;
+  }
+  MoeGemmDesc d;
+  std::memset(&d, 0, sizeof(d));
+  d.S = (uint32_t)S;
+  d.K = (uint32_t)K;
+  d.n_slot = (uint32_t)slot_idx.size();
+  d.n_prob = (uint32_t)prob_w.size();
+  d.pro = glu ? (gelu ? PRO_GEGLU : PRO_SWIGLU) : PRO_NONE;
+  d.err = be->d_words;
+  // weights: bf16, unit stride along k, one expert stride for every problem
+  for (size_t p = 0; p < prob_w.size(); ++p) {
+    cg_tensor *w = prob_w[p];
+    TRY(realize(be, w));
+    if (w->rank != 3 || w->stype != ST_BF16 || w->shape[2] != K || w->strides[2] != 1 || w->shape[0] != prob_w[0]->shape[0] ||
+        w->strides[0] != prob_w[0]->strides[0] || (uintptr_t)data_ptr(w) % 16 || w->strides[1] % 8 || w->strides[0] % 8)
+      return CG_OK;
+    d.prob[p].w = data_ptr(w);
+    d.prob[p].sbn = w->strides[1];
+    d.prob[p].N = (uint32_t)w->shape[1];
+  }
+  d.n_expert = (uint32_t)prob_w[0]->shape[0];
+  d.sb_index = prob_w[0]->strides[0];
+  if (d.n_expert > 65535) return CG_OK;
+  // indices: u32, one stride between consecutive tokens
+  for (size_t sl = 0; sl < slot_idx.size(); ++sl) {
+    cg_tensor *idx = slot_idx[sl];
+    TRY(realize(be, idx));
+    if (idx->dtype != CG_U32) return CG_OK;
+    int64_t istride = 1, expect = -1;
+    for (int i = idx->rank - 1; i >= 0; --i) {
+      if (idx->shape[i] == 1) continue;
+      if (expect < 0) istride = idx->strides[i];
+      else if (idx->strides[i] != expect) return CG_OK;
+      expect = idx->strides[i] * idx->shape[i];
+    }
+    d.slot[sl].idx = (const uint32_t *)data_ptr(idx);
+    d.slot[sl].idx_stride = istride;
+  }
+  // The whole expert MLP of every slot in two launches: when the gated rows of down_proj come from
+  // expert products of one input x that nobody else reads, gate and up are never stored - one
+  // workgroup computes both for its tokens and keeps act(gate) * up as bf16 rows, which the second
+  // launch multiplies with down_proj's matrices.
+  if (glu) {
+    bool fits = true;
+    cg_tensor *x = nullptr, *wg = nullptr, *wu = nullptr;
+    for (size_t sl = 0; sl < slot_a.size() && fits; ++sl) {
+      cg_tensor *g2 = nullptr, *u2 = nullptr;
+      int ge2 = 0;
+      ExpertOperand og, ou;
+      fits = match_glu(slot_a[sl], &g2, &u2, &ge2) && g2->op == N_MATMUL && u2->op == N_MATMUL && refs(g2) == 1 &&
+             refs(u2) == 1 && g2->rank == 3 && u2->rank == 3 && g2->in[0] == u2->in[0] &&
+             match_expert_operand(g2->in[1], S, &og) && match_expert_operand(u2->in[1], S, &ou) && og.idx == slot_idx[sl] &&
+             ou.idx == slot_idx[sl];
+      if (!fits) break;
+      if (!x) {
+        x = g2->in[0];
+        wg = og.w;
+        wu = ou.w;
+      }
+      fits = g2->in[0] == x && og.w == wg && ou.w == wu;
+    }
+    if (fits && x && x->rank == 3 && x->shape[0] == S && x->shape[1] == 1) {
+      const int64_t H = x->shape[2], F = K;
+      TRY(realize(be, x));
+      TRY(realize(be, wg));
+      TRY(realize(be, wu));
+      auto w_ok = [&](const cg_tensor *w, int64_t n_rows, int64_t k) {
+        return w->rank == 3 && w->stype == ST_BF16 && w->shape[0] == d.n_expert && w->shape[1] == n_rows && w->shape[2] == k &&
+               w->strides[2] == 1 && (uintptr_t)data_ptr(w) % 16 == 0 && w->strides[1] % 8 == 0 && w->strides[0] % 8 == 0;
+      };
+      if (H % 8 == 0 && x->stype == ST_F32 && x->strides[2] == 1 && x->strides[0] % 8 == 0 && x->offset % 8 == 0 &&
+          x->st->bytes % 32 == 0 && x->st->grow_dim < 0 && w_ok(wg, F, H) && w_ok(wu, F, H) && wg->strides[0] == wu->strides[0]) {
+        Storage *xsh = nullptr;
+        TRY(bf16_shadow(be, x->st, &xsh));
+        std::vector<Storage *> hbuf(slot_a.size(), nullptr);
+        auto drop_h = [&]() {
+          for (Storage *h : hbuf) storage_release(h);
+        };
+        int st = CG_OK;
+        for (size_t sl = 0; sl < hbuf.size() && !st; ++sl) st = dev_alloc(be, (size_t)S * F * 2, &hbuf[sl]);
+        for (const Member &m : members)
+          if (!st) st = alloc_result(be, m.c, ST_F32);
+        if (st) {
+          drop_h();
+          return st;
+        }
+        MoeGemmDesc f = d;  // same slots' indices and experts; products gate and up over x
+        f.K = (uint32_t)H;
+        f.n_prob = 2;
+        f.pro = PRO_NONE;
+        f.fuse_glu = gelu ? PRO_GEGLU : PRO_SWIGLU;
+        f.sb_index = wg->strides[0];
+        f.prob[0].w = data_ptr(wg); f.prob[0].sbn = wg->strides[1]; f.prob[0].N = (uint32_t)F;
+        f.prob[1].w = data_ptr(wu); f.prob[1].sbn = wu->strides[1]; f.prob[1].N = (uint32_t)F;
+        for (size_t sl = 0; sl < hbuf.size(); ++sl) {
+          f.slot[sl].a16 = (const uint16_t *)xsh->ptr + x->offset;
+          f.slot[sl].a_bs = x->strides[0];
+          f.slot[sl].h16 = (uint16_t *)hbuf[sl]->ptr;
+          d.slot[sl].a16 = (const uint16_t *)hbuf[sl]->ptr;
+          d.slot[sl].a_bs = F;
+        }
+        d.pro = PRO_NONE;
+        for (const Member &m : members) d.slot[m.slot].c[0] = (float *)m.c->st->ptr;
+        hipError_t e;
+        {
+          KernelScope ks(be, "gemm_experts_bf16", 2.0 * d.n_expert * F * H * 2 + (double)S * H * 2 + (double)d.n_slot * S * F * 2,
+                         4.0 * d.n_slot * S * F * H);
+          e = launch_moe_gemm(be->lc(), f);
+        }
+        if (e == hipSuccess) {
+          KernelScope ks(be, "gemm_experts_bf16",
+                         (double)d.n_expert * d.prob[0].N * F * 2 + (double)d.n_slot * S * (F * 2 + d.prob[0].N * 4),
+                         2.0 * d.n_slot * S * d.prob[0].N * F);
+          e = launch_moe_gemm(be->lc(), d);
+        }
+        drop_h();
+        if (e != hipSuccess) return fail(be, CG_ERR_DEVICE, hipGetErrorString(e));
+        for (const Member &m : members) {
+          forget_gemv_candidate(m.c);
+          m.c->op = N_REAL;
+          drop_inputs(m.c);  // the gate and up products under it were never needed as tensors
+        }
+        *done = true;
+        return CG_OK;
+      }
+    }
+  }
+  // input rows
+  std::vector<cg_tensor *> held;
+  auto drop_held = [&]() {
+    for (cg_tensor *t : held) node_release(t);
+  };
+  if (!glu) {
+    cg_tensor *A = n->in[0];
+    TRY(realize(be, A));
+    if (A->stype != ST_F32 || A->strides[2] != 1 || A->strides[0] % 4 || (uintptr_t)data_ptr(A) % 16) return CG_OK;
+    for (size_t sl = 0; sl < slot_idx.size(); ++sl) {
+      d.slot[sl].a = (const float *)data_ptr(A);
+      d.slot[sl].a_bs = A->strides[0];
+    }
+  } else {
+    for (size_t sl = 0; sl < slot_a.size(); ++sl) {
+      cg_tensor *g2 = nullptr, *u2 = nullptr, *gc = nullptr, *uc = nullptr;
+      int ge2 = 0;
+      if (!match_glu(slot_a[sl], &g2, &u2, &ge2)) {
+        drop_held();
+        return CG_OK;
+      }
+      int st = contiguous(be, g2, &gc);
+      if (!st) {
+        held.push_back(gc);
+        st = contiguous(be, u2, &uc);
+      }
+      if (st) {
+        drop_held();
+        return st;
+      }
+      held.push_back(uc);
+      if (gc->stype != ST_F32 || uc->stype != ST_F32 || (uintptr_t)data_ptr(gc) % 16 || (uintptr_t)data_ptr(uc) % 16 || K % 4) {
+        drop_held();
+        return CG_OK;
+      }
+      d.slot[sl].a = (const float *)data_ptr(gc);
+      d.slot[sl].aux = (const float *)data_ptr(uc);
+      d.slot[sl].a_bs = d.slot[sl].aux_bs = K;
+    }
+    // realising gate and up may have run this very function for them; n itself is still deferred
+    if (n->op != N_MATMUL) {
+      drop_held();
+      *done = true;
+      return CG_OK;
+    }
+  }
+  double bytes = 0, flops = 0;
+  int st = CG_OK;
+  for (const Member &m : members) {
+    if (m.c->op != N_MATMUL) {  // realised on the way (cannot happen for a complete set; be safe)
+      drop_held();
+      return CG_OK;
+    }
+  }
+  for (const Member &m : members) {
+    st = alloc_result(be, m.c, ST_F32);
+    if (st) break;
+    d.slot[m.slot].c[m.prob] = (float *)m.c->st->ptr;
+    bytes += (double)S * d.prob[m.prob].N * 4;
+    flops += 2.0 * S * d.prob[m.prob].N * K;
+  }
+  if (!st) {
+    for (uint32_t p = 0; p < d.n_prob; ++p) bytes += (double)d.n_expert * d.prob[p].N * K * 2;
+    bytes += (double)S * K * 4 * (glu ? 2.0 * d.n_slot : 1.0);
+    KernelScope ks(be, "gemm_experts_bf16", bytes, flops);
+    hipError_t e = launch_moe_gemm(be->lc(), d);
+    if (e != hipSuccess) st = fail(be, CG_ERR_DEVICE, hipGetErrorString(e));
+  }
+  drop_held();
+  if (st) return st;
+  for (const Member &m : members) {
+    forget_gemv_candidate(m.c);
+    m.c->op = N_REAL;
+    drop_inputs(m.c);
+  }
+  *done = true;
+  return CG_OK;
+}
+
 int try_moe_gemv(cg_backend *be, cg_tensor *n, bool *done) {
   if (n->rank != 3 || n->shape[1] != 1 || !n->gemv_candidate || n->size() == 0) return CG_OK;
+  TRY(try_moe_gemm(be, n, done));
+  if (*done) return CG_OK;
   const int64_t S = n->shape[0];
   ExpertOperand eo;
   if (!match_expert_operand(n->in[1], S, &eo)) return CG_OK;
@@ -2451,16 +2735,7 @@ int try_moe_gemv(cg_backend *be, cg_tensor *n, bool *done) {
     bytes += (double)S * pr.N * K * esize(w->stype) + (double)S * pr.N * 4;
     flops += 2.0 * S * pr.N * K;
   }
-  // many tokens (a prefill): expert-major, each expert's matrix read once per column tile instead of
-  // once per token
-  const bool many = S >= 64 && b_stype == ST_BF16 && (be->flags & CG_FLAG_BF16);
-  if (!st && many) {
-    double wbytes = 0;
-    for (int i = 0; i < d.m.n_prob; ++i) wbytes += (double)d.b_index_limit * d.m.p[i].N * K * 2 + (double)S * d.m.p[i].N * 4;
-    KernelScope ks(be, "gemm_experts_bf16", (double)S * K * 4 * (pro == PRO_NONE ? 1 : 2) + wbytes, flops);
-    hipError_t e = launch_moe_gemm(be->lc(), d);
-    if (e != hipSuccess) st = fail(be, CG_ERR_DEVICE, hipGetErrorString(e));
-  } else if (!st) {
+  if (!st) {
     const char *base = b_stype == ST_BF16 ? "gemv_experts_bf16" : "gemv_experts_f32";
     KernelScope ks(be, base, bytes, flops);
     hipError_t e = launch_gemv_pro(be->lc(), d);

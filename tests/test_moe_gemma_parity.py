@@ -101,6 +101,29 @@ def test_qwen_moe_hip_vs_oracle(oracle, hip, hip_nopat, hip_bf16, mode):
 
 
 @pytest.mark.gpu
+def test_qwen_moe_prefill_of_many_tokens(oracle, hip_bf16):
+    """2 x 48 tokens in bf16 mode: the routed experts of a layer run expert by expert, all slots in one
+    launch for gate and up and one for down_proj; same logits as the oracle on the rounded parameters."""
+    cfg = MU.qwen_moe_config()
+    P = MU.qwen_moe_params(cfg, seed=9, std=0.15)
+    ids = np.random.default_rng(10).integers(0, cfg.vocab_size, (2, 48))
+    model = llm.qwen_moe.QwenMoeModel(cfg, 48)
+    P_ref = {k: (U_round(v) if v.ndim >= 2 else v) for k, v in P.items()}
+    rt, rl = run_model(oracle, model, P_ref, ids)
+    hip_bf16.trace(True)
+    hip_bf16.trace_reset()
+    gt, gl = run_model(hip_bf16, model, P, ids)
+    rep = hip_bf16.trace_report()
+    hip_bf16.trace(False)
+    # a router probability within bf16 rounding of its neighbour may pick another expert for a token
+    # (a discontinuity of top-k, not an error of the products): bound the bulk, not the worst token
+    err = np.abs(rl - gl).max(axis=-1).reshape(-1)
+    assert np.quantile(err, 0.9) <= 4e-2 * np.abs(rl).max(), np.sort(err)[-10:]
+    assert rep["gemm_experts_bf16"]["launches"] == 2 * cfg.num_hidden_layers, {k: v["launches"] for k, v in rep.items()}
+    assert "gemv_experts_bf16" not in rep
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("mode", ["f32", "nopat", "bf16"])
 def test_gemma3_hip_vs_oracle(oracle, hip, hip_nopat, hip_bf16, mode):
     cfg = MU.gemma_config()
@@ -178,6 +201,44 @@ def test_expert_index_out_of_bounds_is_reported(hip):
     # the flag is cleared: the next evaluation is clean
     (ok,) = vectors.run(hip, f, 1, x, np.array([1, 2], np.uint32), w)
     assert np.array_equal(ok, np.full((2, 1, 8), 16.0, np.float32))
+
+
+@pytest.mark.gpu
+def test_expert_slots_over_many_tokens(oracle, hip_bf16):
+    """The routed half of the MoE block as the model emits it (models/qwen3.rs:104-123) with the indices
+    given: three slots, each gate / up / SwiGLU / down over 150 tokens, weighted and summed.  All slots
+    share two launches; values against the oracle."""
+    import vectors
+    lang, nn = vectors.lang, vectors.nn
+    S, E, F, H, k = 150, 6, 64, 128, 3
+    g = np.random.default_rng(6)
+    x = g.standard_normal((S, 1, H)).astype(np.float32)
+    wg, wu = (U_round((g.standard_normal((E, F, H)) * 0.1).astype(np.float32)) for _ in range(2))
+    wd = U_round((g.standard_normal((E, H, F)) * 0.1).astype(np.float32))
+    idx = g.integers(0, E, (S, k)).astype(np.uint32)
+    val = g.random((S, k)).astype(np.float32)
+
+    def f(b, xv, iv, vv, g_all, u_all, d_all):
+        xv = xv + xv - xv
+        total = None
+        for i in range(k):
+            slot = lang.get(b, 1, i, iv)
+            sel = lambda w: lang.transpose(b, 1, 2, lang.index(b, 0, slot, w))
+            gate = lang.matmul(b, xv, sel(g_all))
+            up = lang.matmul(b, xv, sel(u_all))
+            y = lang.matmul(b, nn.silu(b, gate) * up, sel(d_all))
+            wgt = lang.reshape(b, lang.shape(b, lang.get(b, 2, 0, y)), lang.get(b, 1, i, vv))
+            y = y * lang.broadcast(b, wgt, lang.shape(b, y))
+            total = y if total is None else total + y
+        return total
+    (ref,) = vectors.run(oracle, f, 1, x, idx, val, wg, wu, wd)
+    hip_bf16.trace(True)
+    hip_bf16.trace_reset()
+    (got,) = vectors.run(hip_bf16, f, 1, x, idx, val, wg, wu, wd)
+    rep = hip_bf16.trace_report()
+    hip_bf16.trace(False)
+    assert rep["gemm_experts_bf16"]["launches"] == 2, {n: v["launches"] for n, v in rep.items()}
+    assert np.max(np.abs(got - ref)) <= 2e-2 * np.abs(ref).max()
 
 
 @pytest.mark.gpu
