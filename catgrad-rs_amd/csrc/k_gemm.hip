@@ -115,10 +115,14 @@ __global__ void __launch_bounds__(256) gemm_kernel(GemmDesc g, int a_vec, int b_
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
   const uint32_t m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
-  const uint32_t bz = blockIdx.z, b0 = bz / g.nb1, b1 = bz - b0 * g.nb1;
+  // split-K: slice `split` of k goes to workspace[split] and a second pass sums the slices
+  const uint32_t batch = g.nb0 * g.nb1, split = blockIdx.z / batch, bz = blockIdx.z - split * batch;
+  const uint32_t b0 = bz / g.nb1, b1 = bz - b0 * g.nb1;
   const TA *A = (const TA *)g.a + b0 * g.sa_b0 + b1 * g.sa_b1;
   const TB *B = (const TB *)g.b + b0 * g.sb_b0 + b1 * g.sb_b1;
-  float *C = g.c + (uint64_t)bz * g.M * g.N;
+  float *C = (g.splits > 1 ? g.workspace + (uint64_t)split * batch * g.M * g.N : g.c) + (uint64_t)bz * g.M * g.N;
+  const uint32_t k_begin = g.splits > 1 ? min(g.K, split * g.k_per_split) : 0;
+  const uint32_t k_end = g.splits > 1 ? min(g.K, k_begin + g.k_per_split) : g.K;
 
   f32x16 acc[2][2];
 #pragma unroll
@@ -136,17 +140,17 @@ __global__ void __launch_bounds__(256) gemm_kernel(GemmDesc g, int a_vec, int b_
       const int chunk = tid + c * 256;
       if (A_KC) {
         const int row = chunk / (BK / 8), kc = (chunk % (BK / 8)) * 8;
-        load8<TA, true>(A, g.sam, g.sak, m0 + row, k0 + kc, g.M, g.K, a_vec, ra[c]);
+        load8<TA, true>(A, g.sam, g.sak, m0 + row, k0 + kc, g.M, k_end, a_vec, ra[c]);
       } else {
         const int kk = chunk / (BM / 8), rc = (chunk % (BM / 8)) * 8;
-        load8<TA, false>(A, g.sam, g.sak, m0 + rc, k0 + kk, g.M, g.K, a_vec, ra[c]);
+        load8<TA, false>(A, g.sam, g.sak, m0 + rc, k0 + kk, g.M, k_end, a_vec, ra[c]);
       }
       if (B_KC) {
         const int row = chunk / (BK / 8), kc = (chunk % (BK / 8)) * 8;
-        load8<TB, true>(B, g.sbn, g.sbk, n0 + row, k0 + kc, g.N, g.K, b_vec, rb[c]);
+        load8<TB, true>(B, g.sbn, g.sbk, n0 + row, k0 + kc, g.N, k_end, b_vec, rb[c]);
       } else {
         const int kk = chunk / (BN / 8), rc = (chunk % (BN / 8)) * 8;
-        load8<TB, false>(B, g.sbn, g.sbk, n0 + rc, k0 + kk, g.N, g.K, b_vec, rb[c]);
+        load8<TB, false>(B, g.sbn, g.sbk, n0 + rc, k0 + kk, g.N, k_end, b_vec, rb[c]);
       }
     }
   };
@@ -184,13 +188,13 @@ __global__ void __launch_bounds__(256) gemm_kernel(GemmDesc g, int a_vec, int b_
     }
   };
 
-  const uint32_t n_steps = (g.K + BK - 1) / BK;
-  if (n_steps) fetch(0);
+  const uint32_t n_steps = (k_end - k_begin + BK - 1) / BK;
+  if (n_steps) fetch(k_begin);
   for (uint32_t s = 0; s < n_steps; ++s) {
     __syncthreads();  // previous step's MFMA reads are done
     stash();
     __syncthreads();
-    if (s + 1 < n_steps) fetch((s + 1) * BK);
+    if (s + 1 < n_steps) fetch(k_begin + (s + 1) * BK);
     if (BF16) {
 #pragma unroll
       for (int kk = 0; kk < BK; kk += 16) {
@@ -1428,9 +1432,15 @@ uint32_t gemm_split_k(const LaunchCtx &lc, const GemmDesc &g) {
   const int asz = g.a_stype == ST_BF16 ? 2 : 4, bsz = g.b_stype == ST_BF16 ? 2 : 4;
   const int av = vec_ok(g.a, asz, g.sak == 1 ? g.sam : g.sak, g.sa_b0, g.sa_b1);
   const int bv = vec_ok(g.b, bsz, g.sbk == 1 ? g.sbn : g.sbk, g.sb_b0, g.sb_b1);
-  if (!gemm_fast_path(g, av, bv) || g.N <= 64) return 1;
   const uint64_t tiles = (uint64_t)((g.M + 127) / 128) * ((g.N + 127) / 128) * batch;
   uint32_t splits = 1;
+  if (!gemm_fast_path(g, av, bv)) {
+    // the generic kernel (f32 products): same idea, shorter k-steps, so thinner slices still pay
+    if (g.M <= 8 || g.b_index || !g.K) return 1;
+    while (tiles * splits * 2 <= (uint64_t)lc.n_cus && g.K / (splits * 2) >= 256 && splits < 16) splits *= 2;
+    return splits;
+  }
+  if (g.N <= 64) return 1;
   while (tiles * splits * 2 <= (uint64_t)lc.n_cus && g.K / (splits * 2) >= 512 && splits < 8) splits *= 2;
   return splits;
 }
@@ -1448,7 +1458,7 @@ hipError_t launch_matmul(const LaunchCtx &lc, const GemmDesc &g, const char **ke
   // only the one-row kernels follow b_index and c_add (and the k-slice sum of a split GEMM adds c_add)
   const bool one_row = g.M <= 8 && g.a_stype == ST_F32 && g.K > 0 && (b_unit_k || b_unit_n);
   if (g.b_index && !one_row) return hipErrorInvalidValue;
-  if (g.c_add && !one_row && !(gemm_fast_path(g, av, bv) && g.splits > 1)) return hipErrorInvalidValue;
+  if (g.c_add && !one_row && g.splits <= 1) return hipErrorInvalidValue;
   if ((g.glu_gate || g.c16 || g.n_group) && !gemm_epilogue_ok(g)) return hipErrorInvalidValue;
 
   if (g.M <= 8 && g.a_stype == ST_F32 && g.K > 0) {
@@ -1534,7 +1544,18 @@ hipError_t launch_matmul(const LaunchCtx &lc, const GemmDesc &g, const char **ke
     }
     return hipGetLastError();
   }
-  dim3 grid((g.N + BN - 1) / BN, (g.M + BM - 1) / BM, batch);
+  const uint32_t gsplits = g.splits > 1 ? g.splits : 1;
+  dim3 grid((g.N + BN - 1) / BN, (g.M + BM - 1) / BM, batch * gsplits);
+  auto sum_slices = [&]() {
+    if (gsplits > 1) {
+      LaunchCtx untimed = lc;
+      untimed.ev_start = untimed.ev_stop = nullptr;
+      const uint64_t n = (uint64_t)batch * g.M * g.N;
+      uint64_t blocks = (n / 4 + 255) / 256, cap = (uint64_t)lc.n_cus * 16;
+      CG_LAUNCH(untimed, (splitk_reduce_kernel), (unsigned)(blocks < cap ? (blocks ? blocks : 1) : cap), 256,
+                (const float *)g.workspace, g.c, n, gsplits, g.c_add);
+    }
+  };
   if (g.bf16_math) {
     if (kernel_name) *kernel_name = "gemm_mfma_bf16";
     if (g.a_stype == ST_F32 && g.b_stype == ST_BF16) launch_gemm_layout<float, uint16_t, true>(lc, g, grid, av, bv);
@@ -1546,6 +1567,7 @@ hipError_t launch_matmul(const LaunchCtx &lc, const GemmDesc &g, const char **ke
     if (g.a_stype != ST_F32 || g.b_stype != ST_F32) return hipErrorInvalidValue;
     launch_gemm_layout<float, float, false>(lc, g, grid, av, bv);
   }
+  sum_slices();
   return hipGetLastError();
 }
 

@@ -1370,9 +1370,9 @@ int try_gemv_add(cg_backend *be, cg_tensor *root, bool *done) {
   if (root->dtype != CG_F32 || !is_bin(root, E_ADD_F)) return CG_OK;
   for (int side = 0; side < 2; ++side) {
     cg_tensor *mm = root->in[side], *other = root->in[1 - side];
-    // one-row products add in their epilogue; in bf16 mode so does the k-slice sum of a split GEMM
+    // one-row products add in their epilogue; so does the pass that sums the k-slices of a split GEMM
     if (mm->op != N_MATMUL || refs(mm) != 1 || mm->dtype != CG_F32) continue;
-    if (!mm->gemv_candidate && !(be->flags & CG_FLAG_BF16)) continue;
+    if (!mm->gemv_candidate && mm->rank > 3) continue;  // attention products have fusions of their own
     if (other->op == N_CONST || ((other->op == N_BIN || other->op == N_UN) && refs(other) == 1)) continue;
     TRY(realize(be, other));
     if (other->stype != ST_F32 || !is_contiguous(other)) return CG_OK;
