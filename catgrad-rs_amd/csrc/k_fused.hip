@@ -135,6 +135,7 @@ __global__ void __launch_bounds__(BLOCK) softmax_vec_kernel(SoftmaxDesc d) {
   __shared__ float lds[BLOCK / 64];
   const uint32_t row = blockIdx.x, tid = threadIdx.x;
   const float *x = d.x + (int64_t)row * d.x_row_stride;
+  const uint16_t *x16 = (const uint16_t *)d.x + (int64_t)row * d.x_row_stride;  // when the rows are stored as bf16
   float *y = d.y + (int64_t)row * d.n;
   const float *mk = nullptr;
   if (d.mask) {
@@ -146,7 +147,15 @@ __global__ void __launch_bounds__(BLOCK) softmax_vec_kernel(SoftmaxDesc d) {
 #pragma unroll
   for (int e = 0; e < CH; ++e) {
     const uint32_t c = (tid + e * BLOCK) * 4;
-    if (c < d.n) v[e] = *(const float4 *)(x + c);
+    if (c < d.n) {
+      if (d.x_bf16) {
+        const uint2 h = *(const uint2 *)(x16 + c);
+        v[e] = make_float4(__uint_as_float(h.x << 16), __uint_as_float(h.x & 0xFFFF0000u), __uint_as_float(h.y << 16),
+                           __uint_as_float(h.y & 0xFFFF0000u));
+      } else {
+        v[e] = *(const float4 *)(x + c);
+      }
+    }
   }
 #pragma unroll
   for (int e = 0; e < CH; ++e) {
@@ -196,6 +205,7 @@ hipError_t launch_softmax(const LaunchCtx &lc, const SoftmaxDesc &d) {
                    (uintptr_t)d.y % 16 == 0 &&
                    (!d.mask || (d.mask_col_stride == 1 && (uintptr_t)d.mask % 16 == 0 && d.mask_row_stride % 4 == 0 &&
                                 d.mask_group_stride % 4 == 0));
+  if (d.x_bf16 && !vec) return hipErrorInvalidValue;
   if (vec) {
     if (d.n <= 512) CG_LAUNCH(lc, (softmax_vec_kernel<64, 2>), d.rows, 64, d);
     else if (d.n <= 1024) CG_LAUNCH(lc, (softmax_vec_kernel<256, 1>), d.rows, 256, d);
@@ -603,12 +613,20 @@ hipError_t launch_glu(const LaunchCtx &lc, int gelu, const float *gate, const fl
 }
 
 // ---- one f32 binary op, a contiguous, b contiguous or a row vector repeated over rows ---------------
-template <int OP>
+// A16: a is stored as bf16 (an uploaded matrix used directly in an elementwise op)
+template <int OP, bool A16>
 __global__ void __launch_bounds__(256) binary_kernel(const float *a, const float *b, float *out,
                                                      uint64_t n4, uint32_t b_period4) {
   for (uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x; i < n4;
        i += (uint64_t)gridDim.x * 256) {
-    const float4 x = ((const float4 *)a)[i];
+    float4 x;
+    if (A16) {
+      const uint2 h = ((const uint2 *)a)[i];
+      x = make_float4(__uint_as_float(h.x << 16), __uint_as_float(h.x & 0xFFFF0000u), __uint_as_float(h.y << 16),
+                      __uint_as_float(h.y & 0xFFFF0000u));
+    } else {
+      x = ((const float4 *)a)[i];
+    }
     const float4 y = ((const float4 *)b)[b_period4 ? i % b_period4 : i];
     float4 o;
     if (OP == 0) { o.x = x.x + y.x; o.y = x.y + y.y; o.z = x.z + y.z; o.w = x.w + y.w; }
@@ -620,17 +638,26 @@ __global__ void __launch_bounds__(256) binary_kernel(const float *a, const float
 }
 
 hipError_t launch_binary_f32(const LaunchCtx &lc, int op, const float *a, const float *b, float *out,
-                             uint64_t n, uint32_t b_period) {
+                             uint64_t n, uint32_t b_period, bool a_bf16) {
   if (!n) return hipSuccess;
   const uint64_t n4 = n / 4;
   uint64_t blocks = (n4 + 255) / 256, cap = (uint64_t)lc.n_cus * 16;
   const unsigned grid = (unsigned)(blocks < cap ? blocks : cap);
   const uint32_t p4 = b_period / 4;
+  if (a_bf16) {
+    switch (op) {
+      case 0: CG_LAUNCH(lc, (binary_kernel<0, true>), grid, 256, a, b, out, n4, p4); break;
+      case 1: CG_LAUNCH(lc, (binary_kernel<1, true>), grid, 256, a, b, out, n4, p4); break;
+      case 2: CG_LAUNCH(lc, (binary_kernel<2, true>), grid, 256, a, b, out, n4, p4); break;
+      default: CG_LAUNCH(lc, (binary_kernel<3, true>), grid, 256, a, b, out, n4, p4); break;
+    }
+    return hipGetLastError();
+  }
   switch (op) {
-    case 0: CG_LAUNCH(lc, (binary_kernel<0>), grid, 256, a, b, out, n4, p4); break;
-    case 1: CG_LAUNCH(lc, (binary_kernel<1>), grid, 256, a, b, out, n4, p4); break;
-    case 2: CG_LAUNCH(lc, (binary_kernel<2>), grid, 256, a, b, out, n4, p4); break;
-    default: CG_LAUNCH(lc, (binary_kernel<3>), grid, 256, a, b, out, n4, p4); break;
+    case 0: CG_LAUNCH(lc, (binary_kernel<0, false>), grid, 256, a, b, out, n4, p4); break;
+    case 1: CG_LAUNCH(lc, (binary_kernel<1, false>), grid, 256, a, b, out, n4, p4); break;
+    case 2: CG_LAUNCH(lc, (binary_kernel<2, false>), grid, 256, a, b, out, n4, p4); break;
+    default: CG_LAUNCH(lc, (binary_kernel<3, false>), grid, 256, a, b, out, n4, p4); break;
   }
   return hipGetLastError();
 }

@@ -104,6 +104,7 @@ struct SoftmaxDesc {
   uint32_t rows, n, mask_rows;
   int32_t has_scale, has_mask_const;
   float scale, mask_const;
+  int32_t x_bf16;        // x points at bf16 rows (vector kernels only: n % 4 == 0, n >= 256, 8-byte aligned rows)
 };
 hipError_t launch_softmax(const LaunchCtx &lc, const SoftmaxDesc &d);
 
@@ -122,7 +123,7 @@ hipError_t launch_glu(const LaunchCtx &lc, int gelu, const float *gate, const fl
 // op: 0 add, 1 sub, 2 mul, 3 div; b is contiguous (b_period = 0) or a vector of b_period floats
 // repeated; n % 4 == 0, b_period % 4 == 0
 hipError_t launch_binary_f32(const LaunchCtx &lc, int op, const float *a, const float *b, float *out,
-                             uint64_t n, uint32_t b_period);
+                             uint64_t n, uint32_t b_period, bool a_bf16 = false);  // a_bf16: a points at bf16 values
 
 // One-query attention (a decode step): out[b, h, :] = softmax(q[b, h, :] . K[b, h, t, :] / scale + mask_const) . V
 // K and V rows are read in place from the (growable) cache through strides; head h of a

@@ -946,7 +946,15 @@ int try_softmax(cg_backend *be, cg_tensor *root, bool *done) {
   d.mask_const = sm_.mask_const;
   cg_tensor *xs = nullptr, *ms = nullptr;
   int64_t row_stride = 0;
-  TRY(as_rows(be, src, &xs, &row_stride));
+  // rows stored as bf16 (an uploaded matrix) are read as they are by the 16-byte kernel
+  TRY(realize(be, src));
+  if (src->stype == ST_BF16 && !mask && is_contiguous(src) && n % 4 == 0 && n >= 256 && (uintptr_t)data_ptr(src) % 16 == 0) {
+    xs = retain(src);
+    row_stride = n;
+    d.x_bf16 = 1;
+  } else {
+    TRY(as_rows(be, src, &xs, &row_stride));
+  }
   int st = CG_OK;
   if (mask) {
     st = realize(be, mask);
@@ -996,7 +1004,7 @@ int try_softmax(cg_backend *be, cg_tensor *root, bool *done) {
     d.x_row_stride = row_stride;
     d.rows = (uint32_t)(root->size() / n);
     d.n = (uint32_t)n;
-    KernelScope ks(be, "softmax_fused", (double)root->size() * (d.y16 ? 10 : 8), 0);
+    KernelScope ks(be, "softmax_fused", (double)root->size() * ((d.y16 ? 6 : 4) + (d.x_bf16 ? 2 : 4)), 0);
     hipError_t e = launch_softmax(be->lc(), d);
     if (e != hipSuccess) st = fail(be, CG_ERR_DEVICE, hipGetErrorString(e));
   }
@@ -1409,7 +1417,8 @@ int try_binary(cg_backend *be, cg_tensor *root, bool *done) {
   if (!leaf(a) || !leaf(b)) return CG_OK;
   TRY(realize(be, a));
   TRY(realize(be, b));
-  if (a->stype != ST_F32 || b->stype != ST_F32 || !is_contiguous(a) || (uintptr_t)data_ptr(a) % 16 ||
+  const bool a16 = a->stype == ST_BF16;  // an uploaded matrix used as it is stored
+  if ((a->stype != ST_F32 && !a16) || b->stype != ST_F32 || !is_contiguous(a) || (uintptr_t)data_ptr(a) % 16 ||
       (uintptr_t)data_ptr(b) % 16)
     return CG_OK;
   uint32_t period = 0;
@@ -1428,9 +1437,9 @@ int try_binary(cg_backend *be, cg_tensor *root, bool *done) {
   }
   TRY(alloc_result(be, root, ST_F32));
   {
-    KernelScope ks(be, "binary_f32", (double)root->size() * (period ? 8 : 12) + period * 4.0, 0);
+    KernelScope ks(be, "binary_f32", (double)root->size() * ((period ? 4 : 8) + (a16 ? 2 : 4)) + period * 4.0, 0);
     HIPCHK(be, launch_binary_f32(be->lc(), op, (const float *)data_ptr(a), (const float *)data_ptr(b),
-                                 (float *)root->st->ptr, (uint64_t)root->size(), period));
+                                 (float *)root->st->ptr, (uint64_t)root->size(), period, a16));
   }
   finish_fused(root);
   *done = true;

@@ -235,8 +235,11 @@ def test_residual_add_with_a_split_gemm(oracle, hip_bf16, shape):
 
     def f(b, xv, rv):
         xv = xv + xv - xv
-        return rv + nn.linear_no_bias(b, K, N, lang.path(["l"]), xv)
+        y = nn.linear_no_bias(b, K, N, lang.path(["l"]), xv)
+        rv = lang.reshape(b, lang.shape(b, y), rv)      # the residual stream: an f32 value in memory
+        return rv + y
     p = {"l.weight": w}
+    res = res.reshape(-1)                               # rank 1: stays f32 in bf16 mode
     (ref,) = vectors.run(oracle, f, 1, x, res, params=p)
     got, names = run_traced(hip_bf16, f, 1, x, res, params=p)
     assert "gemm_mfma_bf16" in names
