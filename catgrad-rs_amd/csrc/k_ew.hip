@@ -100,13 +100,21 @@ __device__ __forceinline__ uint32_t apply_un(uint8_t op, uint32_t a) {
   }
 }
 
+// A program staged in LDS (ST) is read with vector instructions; the values that steer control
+// flow are the same in every lane and go back to scalar registers so that branches stay uniform.
+template <bool ST>
+__device__ __forceinline__ uint32_t uni(uint32_t v) {
+  return ST ? (uint32_t)__builtin_amdgcn_readfirstlane((int)v) : v;
+}
+
 // Load VEC consecutive elements (along the innermost dim) of one operand at element offset off.
-template <int VEC>
+template <int VEC, bool ST = false>
 __device__ __forceinline__ void load_vec(const Operand &in, int64_t off, int64_t inner,
                                          uint32_t *v) {
-  if (in.stype == ST_BF16) {
+  const uint32_t stype = uni<ST>((uint32_t)in.stype), vec = uni<ST>((uint32_t)in.vec);
+  if (stype == ST_BF16) {
     const uint16_t *p = (const uint16_t *)in.ptr + off;
-    if (VEC == 4 && in.vec) {
+    if (VEC == 4 && vec) {
       uint2 q = *(const uint2 *)p;
       v[0] = q.x << 16; v[1 % VEC] = q.x & 0xFFFF0000u;
       v[2 % VEC] = q.y << 16; v[3 % VEC] = q.y & 0xFFFF0000u;
@@ -116,10 +124,10 @@ __device__ __forceinline__ void load_vec(const Operand &in, int64_t off, int64_t
     }
   } else {
     const uint32_t *p = (const uint32_t *)in.ptr + off;
-    if (VEC == 4 && in.vec) {
+    if (VEC == 4 && vec) {
       uint4 q = *(const uint4 *)p;
       v[0] = q.x; v[1 % VEC] = q.y; v[2 % VEC] = q.z; v[3 % VEC] = q.w;
-    } else if (inner == 0) {
+    } else if (uni<ST>((uint32_t)(inner == 0))) {
       uint32_t s = p[0];
 #pragma unroll
       for (int j = 0; j < VEC; ++j) v[j] = s;
@@ -139,21 +147,22 @@ __device__ __forceinline__ void load_vec(const Operand &in, int64_t off, int64_t
 // ignored); chunk k is skipped when bit k of `valid` is clear.  Running one instruction over
 // K * VEC elements amortises the (wave-uniform) instruction decode.
 // All K chunks of one operand for this thread.
-template <int VEC, int K>
+template <int VEC, int K, bool ST = false>
 __device__ __forceinline__ void load_chunks(const Program &p, int slot,
                                             const uint32_t (&idx)[MAX_DIMS], uint32_t c0,
                                             uint32_t cstride, uint32_t valid,
                                             uint32_t (&t)[K * VEC]) {
   const Operand &in = p.in[slot];
+  const int n_dims = (int)uni<ST>((uint32_t)p.n_dims);
   int64_t off = 0;
 #pragma unroll
   for (int d = 0; d < MAX_DIMS - 1; ++d)
-    if (d < p.n_dims - 1) off += (int64_t)idx[d] * in.stride[d];
-  const int64_t inner = in.stride[p.n_dims - 1];
+    if (d < n_dims - 1) off += (int64_t)idx[d] * in.stride[d];
+  const int64_t inner = in.stride[n_dims - 1];
 #pragma unroll
   for (int k = 0; k < K; ++k) {
     if (valid & (1u << k)) {
-      load_vec<VEC>(in, off + (int64_t)(c0 + k * cstride) * inner, inner, &t[k * VEC]);
+      load_vec<VEC, ST>(in, off + (int64_t)(c0 + k * cstride) * inner, inner, &t[k * VEC]);
     } else {
 #pragma unroll
       for (int j = 0; j < VEC; ++j) t[k * VEC + j] = 0u;
@@ -161,7 +170,7 @@ __device__ __forceinline__ void load_chunks(const Program &p, int slot,
   }
 }
 
-template <int VEC, int K>
+template <int VEC, int K, bool ST = false>
 __device__ __forceinline__ void eval_program(const Program &p, int pc0, int pc1,
                                              const uint32_t (&idx)[MAX_DIMS], uint32_t c0,
                                              uint32_t cstride, uint32_t valid, uint32_t row0,
@@ -170,18 +179,26 @@ __device__ __forceinline__ void eval_program(const Program &p, int pc0, int pc1,
   constexpr int E = K * VEC;
   uint32_t r[MAX_STACK][E];
   for (int pc = pc0; pc < pc1; ++pc) {
-    const Instr ins = p.code[pc];
+    Instr ins;
+    if (ST) {
+      const uint32_t w = uni<ST>(*(const uint32_t *)&p.code[pc]);
+      ins.op = (uint8_t)(w & 0xFFu);
+      ins.depth = (uint8_t)((w >> 8) & 0xFFu);
+      ins.arg = (uint16_t)(w >> 16);
+    } else {
+      ins = p.code[pc];
+    }
     if (ins.op <= E_ROW1) {
       uint32_t t[E];
       if (ins.op == E_LOAD) {
-        load_chunks<VEC, K>(p, ins.arg, idx, c0, cstride, valid, t);
+        load_chunks<VEC, K, ST>(p, ins.arg, idx, c0, cstride, valid, t);
       } else if (ins.op == E_IOTA) {
 #pragma unroll
         for (int k = 0; k < K; ++k)
 #pragma unroll
           for (int j = 0; j < VEC; ++j) t[k * VEC + j] = c0 + k * cstride + j;
       } else {
-        uint32_t c = ins.op == E_CONST ? p.imm[ins.arg] : (ins.op == E_ROW0 ? row0 : row1);
+        uint32_t c = ins.op == E_CONST ? uni<ST>(p.imm[ins.arg]) : (ins.op == E_ROW0 ? row0 : row1);
 #pragma unroll
         for (int j = 0; j < E; ++j) t[j] = c;
       }
@@ -241,13 +258,15 @@ __device__ __forceinline__ void eval_program(const Program &p, int pc0, int pc1,
   for (int j = 0; j < E; ++j) res[j] = r[0][j];
 }
 
+template <bool ST = false>
 __device__ __forceinline__ void decompose(const Program &p, uint64_t lin,
                                           uint32_t (&idx)[MAX_DIMS]) {
   // all programs stay below 2^32 elements (checked on the host)
   uint32_t rem = (uint32_t)lin;
+  const int n_dims = (int)uni<ST>((uint32_t)p.n_dims);
 #pragma unroll
   for (int d = MAX_DIMS - 1; d >= 0; --d) {
-    if (d < p.n_dims) {
+    if (d < n_dims) {
       if (d == 0) {
         idx[d] = rem;
       } else {
@@ -261,26 +280,40 @@ __device__ __forceinline__ void decompose(const Program &p, uint64_t lin,
   }
 }
 
-template <int VEC>
-__global__ void __launch_bounds__(256) ew_kernel(const Program p, OutDesc o, uint64_t n_groups,
+// ST: the launch is small (every thread runs the program once).  Walking the program through the
+// kernel-argument segment costs one scalar-cache miss per operand descriptor and code line, one
+// after the other, in memory the host has just written - most of such a launch's duration.  All
+// threads copy the program into LDS in one round trip instead and the walk reads it from there.
+template <int VEC, bool ST>
+__global__ void __launch_bounds__(256) ew_kernel(const Program pk, OutDesc o, uint64_t n_groups,
                                                  uint32_t *err) {
+  __shared__ __attribute__((aligned(16))) uint32_t staged[ST ? sizeof(Program) / 4 : 4];
+  if (ST) {
+    static_assert(sizeof(Program) % 16 == 0, "program copied in 16-byte pieces");
+    const uint4 *src = (const uint4 *)&pk;
+    for (uint32_t i = threadIdx.x; i < sizeof(Program) / 16; i += 256) ((uint4 *)staged)[i] = src[i];
+    __syncthreads();
+  }
+  const Program &p = ST ? *(const Program *)staged : pk;
+  const int n_dims = (int)uni<ST>((uint32_t)p.n_dims);
+  const int n_instr = (int)uni<ST>((uint32_t)p.n_instr);
   for (uint64_t g = (uint64_t)blockIdx.x * 256 + threadIdx.x; g < n_groups;
        g += (uint64_t)gridDim.x * 256) {
     uint32_t idx[MAX_DIMS];
     const uint64_t lin = g * VEC;
-    decompose(p, lin, idx);
+    decompose<ST>(p, lin, idx);
     uint32_t v[VEC];
     uint32_t c0 = 0;
 #pragma unroll
     for (int d = 0; d < MAX_DIMS; ++d)
-      if (d == p.n_dims - 1) c0 = idx[d];
+      if (d == n_dims - 1) c0 = idx[d];
     // rank-1 programs (the only ones with E_IOTA) have c0 == lin
-    eval_program<VEC, 1>(p, 0, p.n_instr, idx, c0, 0u, 1u, 0u, 0u, err, v);
+    eval_program<VEC, 1, ST>(p, 0, n_instr, idx, c0, 0u, 1u, 0u, 0u, err, v);
     int64_t off = 0;
 #pragma unroll
     for (int d = 0; d < MAX_DIMS; ++d)
-      if (d < p.n_dims) off += (int64_t)idx[d] * o.stride[d];
-    const int64_t inner = o.stride[p.n_dims - 1];
+      if (d < n_dims) off += (int64_t)idx[d] * o.stride[d];
+    const int64_t inner = o.stride[n_dims - 1];
     if (o.stype == ST_BF16) {
       uint16_t *q = (uint16_t *)o.ptr + off;
 #pragma unroll
@@ -727,12 +760,19 @@ static inline unsigned grid_for(uint64_t blocks_needed, const LaunchCtx &lc) {
 hipError_t launch_ew(const LaunchCtx &lc, const Program &p, const OutDesc &o, uint64_t n_elems,
                      bool vec4) {
   if (n_elems == 0) return hipSuccess;
+  // up to one group per thread of the grid: the staged walk (see ew_kernel)
+  const uint64_t one_pass = (uint64_t)lc.n_cus * 8 * 256;
   if (vec4) {
     uint64_t groups = n_elems / 4;
-    CG_LAUNCH(lc, (ew_kernel<4>), grid_for((groups + 255) / 256, lc), 256, p, o, groups, lc.err_flag);
+    if (groups <= one_pass)
+      CG_LAUNCH(lc, (ew_kernel<4, true>), grid_for((groups + 255) / 256, lc), 256, p, o, groups, lc.err_flag);
+    else
+      CG_LAUNCH(lc, (ew_kernel<4, false>), grid_for((groups + 255) / 256, lc), 256, p, o, groups, lc.err_flag);
   } else {
-    CG_LAUNCH(lc, (ew_kernel<1>), grid_for((n_elems + 255) / 256, lc), 256, p, o, n_elems,
-                                                                             lc.err_flag);
+    if (n_elems <= one_pass)
+      CG_LAUNCH(lc, (ew_kernel<1, true>), grid_for((n_elems + 255) / 256, lc), 256, p, o, n_elems, lc.err_flag);
+    else
+      CG_LAUNCH(lc, (ew_kernel<1, false>), grid_for((n_elems + 255) / 256, lc), 256, p, o, n_elems, lc.err_flag);
   }
   return hipGetLastError();
 }

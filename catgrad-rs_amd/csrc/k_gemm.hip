@@ -243,6 +243,94 @@ __global__ void __launch_bounds__(256) gemm_kernel(GemmDesc g, int a_vec, int b_
     }
 }
 
+// ---- small f32 products ----------------------------------------------------------------------------
+// A product with a handful of 128 x 128 tiles (the 64 x 256 and 64 x 10 layers of a small MLP) leaves
+// the kernel above with one or two workgroups walking K sixteen columns at a time, every step a full
+// memory round trip.  Here a workgroup owns a 32 x 32 tile of C and its four wavefronts each take a
+// quarter of K: every lane fetches its own MFMA operands straight from memory, 32 values of k per
+// round trip and the next round trip already in flight, and the four partial tiles meet in LDS.
+// Lane (r, h) = (lane % 32, lane / 32) supplies A[m0 + r][k] and B[k][n0 + r] for
+// k = chunk * 32 + q * 8 + h * 4 + j; MFMA (q, j) pairs element j of both.
+template <bool KC>
+__device__ __forceinline__ float4 load4(const float *base, int64_t s_k, uint32_t k, uint32_t K, bool ok, int vec) {
+  float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (!ok) return v;
+  if (KC && vec && k + 4 <= K) return *(const float4 *)(base + k);
+  const float *p = base + (int64_t)k * s_k;
+  if (k < K) v.x = p[0];
+  if (k + 1 < K) v.y = p[s_k];
+  if (k + 2 < K) v.z = p[2 * s_k];
+  if (k + 3 < K) v.w = p[3 * s_k];
+  return v;
+}
+
+template <bool A_KC, bool B_KC>
+__global__ void __launch_bounds__(256) gemm_small_f32_kernel(GemmDesc g, int a_vec, int b_vec) {
+  __shared__ float part[4][16 * 64];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, h = lane >> 5;
+  const uint32_t m0 = blockIdx.y * 32, n0 = blockIdx.x * 32;
+  // split-K as in gemm_kernel: slice `split` of k goes to workspace[split], summed by a second pass
+  const uint32_t batch = g.nb0 * g.nb1, split = blockIdx.z / batch, bz = blockIdx.z - split * batch;
+  const uint32_t b0 = bz / g.nb1, b1 = bz - b0 * g.nb1;
+  const float *A = (const float *)g.a + b0 * g.sa_b0 + b1 * g.sa_b1;
+  const float *B = (const float *)g.b + b0 * g.sb_b0 + b1 * g.sb_b1;
+  float *C = (g.splits > 1 ? g.workspace + (uint64_t)split * batch * g.M * g.N : g.c) + (uint64_t)bz * g.M * g.N;
+  const uint32_t k_begin = g.splits > 1 ? min(g.K, split * g.k_per_split) : 0;  // a multiple of 32
+  const uint32_t k_end = g.splits > 1 ? min(g.K, k_begin + g.k_per_split) : g.K;
+  const uint32_t chunks = (k_end - k_begin + 31) / 32, per = (chunks + 3) / 4;
+  const uint32_t c_begin = min(chunks, wave * per), c_end = min(chunks, c_begin + per);
+  const bool row_ok = m0 + r < g.M, col_ok = n0 + r < g.N;
+  const float *Ar = A + (int64_t)(m0 + r) * g.sam, *Bc = B + (int64_t)(n0 + r) * g.sbn;
+  const int64_t sak = A_KC ? 1 : g.sak, sbk = B_KC ? 1 : g.sbk;
+  f32x16 acc;
+#pragma unroll
+  for (int e = 0; e < 16; ++e) acc[e] = 0.f;
+  float4 ra[2][4], rb[2][4];
+  auto fetch = [&](int buf, uint32_t c) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const uint32_t k = k_begin + c * 32 + q * 8 + h * 4;
+      ra[buf][q] = load4<A_KC>(Ar, sak, k, k_end, row_ok, a_vec);
+      rb[buf][q] = load4<B_KC>(Bc, sbk, k, k_end, col_ok, b_vec);
+    }
+  };
+  auto multiply = [&](int buf) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ra[buf][q].x, rb[buf][q].x, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ra[buf][q].y, rb[buf][q].y, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ra[buf][q].z, rb[buf][q].z, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ra[buf][q].w, rb[buf][q].w, acc, 0, 0, 0);
+    }
+  };
+  if (c_begin < c_end) fetch(0, c_begin);
+  for (uint32_t c = c_begin; c < c_end; c += 2) {
+    if (c + 1 < c_end) fetch(1, c + 1);
+    multiply(0);
+    if (c + 1 < c_end) {
+      if (c + 2 < c_end) fetch(0, c + 2);
+      multiply(1);
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < 16; ++e) part[wave][e * 64 + lane] = acc[e];
+  __syncthreads();
+  // element e of lane l: row (e / 4) * 8 + (l / 32) * 4 + e % 4, column l % 32
+  for (int i = tid; i < 1024; i += 256) {
+    const int e = i >> 6, l = i & 63;
+    const uint32_t row = m0 + (e >> 2) * 8 + (l >> 5) * 4 + (e & 3), col = n0 + (l & 31);
+    if (row < g.M && col < g.N)
+      C[(uint64_t)row * g.N + col] = (part[0][i] + part[1][i]) + (part[2][i] + part[3][i]);
+  }
+}
+
+// few enough 32 x 32 tiles that the kernel above has the machine to itself
+static bool gemm_small_ok(const LaunchCtx &lc, const GemmDesc &g) {
+  if (g.bf16_math || g.a_stype != ST_F32 || g.b_stype != ST_F32 || g.M <= 8 || g.b_index || !g.K) return false;
+  const uint64_t t32 = (uint64_t)((g.M + 31) / 32) * ((g.N + 31) / 32) * g.nb0 * g.nb1;
+  return t32 <= 2 * (uint64_t)lc.n_cus;
+}
+
 // ---- bf16 x bf16 "NT" GEMM: the prefill fast path --------------------------------------------------
 // A[M, K] and B[N, K] both bf16 with unit stride along k (activations are narrowed once by
 // cast_bf16_kernel and the copy is shared by every GEMM that reads them; weights are stored
@@ -1434,6 +1522,12 @@ uint32_t gemm_split_k(const LaunchCtx &lc, const GemmDesc &g) {
   const int bv = vec_ok(g.b, bsz, g.sbk == 1 ? g.sbn : g.sbk, g.sb_b0, g.sb_b1);
   const uint64_t tiles = (uint64_t)((g.M + 127) / 128) * ((g.N + 127) / 128) * batch;
   uint32_t splits = 1;
+  if (gemm_small_ok(lc, g)) {
+    // deep and tiny: more workgroups along k while each wavefront keeps two 32-wide chunks
+    const uint64_t t32 = (uint64_t)((g.M + 31) / 32) * ((g.N + 31) / 32) * batch;
+    while (t32 * splits * 2 <= (uint64_t)lc.n_cus && g.K / (splits * 2) >= 256 && splits < 64) splits *= 2;
+    return splits;
+  }
   if (!gemm_fast_path(g, av, bv)) {
     // the generic kernel (f32 products): same idea, shorter k-steps, so thinner slices still pay
     if (g.M <= 8 || g.b_index || !g.K) return 1;
@@ -1545,7 +1639,6 @@ hipError_t launch_matmul(const LaunchCtx &lc, const GemmDesc &g, const char **ke
     return hipGetLastError();
   }
   const uint32_t gsplits = g.splits > 1 ? g.splits : 1;
-  dim3 grid((g.N + BN - 1) / BN, (g.M + BM - 1) / BM, batch * gsplits);
   auto sum_slices = [&]() {
     if (gsplits > 1) {
       LaunchCtx untimed = lc;
@@ -1556,6 +1649,18 @@ hipError_t launch_matmul(const LaunchCtx &lc, const GemmDesc &g, const char **ke
                 (const float *)g.workspace, g.c, n, gsplits, g.c_add);
     }
   };
+  if (gemm_small_ok(lc, g)) {
+    if (kernel_name) *kernel_name = "gemm_mfma_f32";
+    dim3 gr((g.N + 31) / 32, (g.M + 31) / 32, batch * gsplits);
+    const bool akc = a_unit_k, bkc = b_unit_k;
+    if (akc && bkc) CG_LAUNCH(lc, (gemm_small_f32_kernel<true, true>), gr, 256, g, av, bv);
+    else if (akc) CG_LAUNCH(lc, (gemm_small_f32_kernel<true, false>), gr, 256, g, av, 0);
+    else if (bkc) CG_LAUNCH(lc, (gemm_small_f32_kernel<false, true>), gr, 256, g, 0, bv);
+    else CG_LAUNCH(lc, (gemm_small_f32_kernel<false, false>), gr, 256, g, 0, 0);
+    sum_slices();
+    return hipGetLastError();
+  }
+  dim3 grid((g.N + BN - 1) / BN, (g.M + BM - 1) / BM, batch * gsplits);
   if (g.bf16_math) {
     if (kernel_name) *kernel_name = "gemm_mfma_bf16";
     if (g.a_stype == ST_F32 && g.b_stype == ST_BF16) launch_gemm_layout<float, uint16_t, true>(lc, g, grid, av, bv);

@@ -436,6 +436,46 @@ def test_bf16_mode_matmul_shape_sweep(oracle, hip_bf16):
         assert_close(r[0], d[0], RTOL_BF16, scale=scale)
 
 
+@pytest.mark.gpu
+def test_small_f32_matmul_layouts_and_tails(oracle, hip):
+    """Products of a few 32 x 32 tiles in f32 (the layers of a small MLP): either operand with unit
+    stride along k or along its other axis, sizes that leave tails in M, N and K (K below and across
+    the 32-wide chunks, not a multiple of 4, deep enough to be split over workgroups), batches, a broadcast right
+    operand and a sliced left one."""
+    g = rng(62)
+    shapes = [(1, 9, 1, 1), (1, 33, 5, 31), (1, 64, 256, 10), (1, 64, 128, 256), (1, 70, 300, 70), (1, 17, 37, 130),
+              (3, 40, 129, 50), (2, 100, 1000, 12), (1, 32, 4096, 32), (1, 12, 3, 300), (1, 11, 2048, 9),
+              (2, 64, 8200, 64)]       # batch, M, K, N; the deep ones are split along k
+    for (b, m, k, n) in shapes:
+        x = g.standard_normal((b, m, k)).astype(np.float32)
+        w = g.standard_normal((b, k, n)).astype(np.float32)
+        xt = np.ascontiguousarray(np.swapaxes(x, 1, 2))
+        wt = np.ascontiguousarray(np.swapaxes(w, 1, 2))
+        xpad = g.standard_normal((b, m, k + 3)).astype(np.float32)
+
+        def f(be, x, w, xt, wt, xpad):
+            y0 = be.matmul(x, w)                                             # A along k, B along n
+            y1 = be.matmul(x, be.transpose(wt, 1, 2))                        # both along k
+            y2 = be.matmul(be.transpose(xt, 1, 2), w)                        # neither
+            y3 = be.matmul(be.transpose(xt, 1, 2), be.transpose(wt, 1, 2))   # A along m, B along k
+            y4 = be.matmul(be.slice(xpad, 2, 1, k), w)                       # rows that start off 16-byte alignment
+            w0 = be.broadcast(be.slice(w, 0, 0, 1), (b, k, n))               # one matrix for every batch
+            return y0, y1, y2, y3, y4, be.matmul(x, w0)
+        r, d = both(oracle, hip, f, x, w, xt, wt, xpad)
+        truth = np.matmul(x.astype(np.float64), w.astype(np.float64))
+        scale = np.matmul(np.abs(x).astype(np.float64), np.abs(w).astype(np.float64))
+        for i in range(4):
+            assert_close(truth.astype(np.float32), d[i], RTOL_F32, scale=scale)
+        xs = xpad[:, :, 1:1 + k].astype(np.float64)
+        assert_close(np.matmul(xs, w.astype(np.float64)).astype(np.float32), d[4], RTOL_F32,
+                     scale=np.matmul(np.abs(xs), np.abs(w).astype(np.float64)))
+        w0 = np.broadcast_to(w[:1], w.shape).astype(np.float64)
+        assert_close(np.matmul(x.astype(np.float64), w0).astype(np.float32), d[5], RTOL_F32,
+                     scale=np.matmul(np.abs(x).astype(np.float64), np.abs(w0)))
+        for i in range(6):
+            assert_close(r[i], d[i], 2 * RTOL_F32, scale=scale if i != 4 else np.matmul(np.abs(xs), np.abs(w).astype(np.float64)))
+
+
 def test_row_fusion_layernorm_and_softmax_views(oracle, hip, hip_eager):
     """Row programs (reduction stages + final segment in one kernel) on strided inputs: softmax of
     a transposed view, layernorm with gamma/beta broadcasts, and a row value read twice."""
