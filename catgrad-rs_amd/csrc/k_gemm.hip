@@ -1348,6 +1348,222 @@ __global__ void __launch_bounds__(256) moe_gemm_kernel(MoeGemmDesc g) {
   }
 }
 
+// ---- the same with the routing done once and the operands streamed like the dense GEMM ------------------
+// One workgroup of 1024 threads sorts the (slot, token) pairs by expert: a histogram in LDS, a scan,
+// and a scatter through per-expert cursors.  The order of an expert's pairs depends on the order
+// the atomics land in, which only decides the tile row a token occupies, never its result.
+__global__ void __launch_bounds__(1024) moe_route_kernel(MoeGemmDesc g, uint32_t *count, uint32_t *offset, uint32_t *list) {
+  __shared__ uint32_t hist[MOE_ROUTE_MAX_EXPERTS], cursor[MOE_ROUTE_MAX_EXPERTS], scan[1024];
+  const uint32_t tid = threadIdx.x, E = g.n_expert, S = g.S, pairs = S * g.n_slot;
+  for (uint32_t i = tid; i < E; i += 1024) hist[i] = 0;
+  __syncthreads();
+  for (uint32_t p = tid; p < pairs; p += 1024) {
+    const uint32_t sl = p / S, t = p - sl * S;
+    uint32_t ix = g.slot[sl].idx[(int64_t)t * g.slot[sl].idx_stride];
+    if (ix >= E) {
+      atomicOr(g.err, ERRF_INDEX_OOB);
+      ix = E - 1;
+    }
+    atomicAdd(&hist[ix], 1u);
+  }
+  __syncthreads();
+  const uint32_t per = (E + 1023) / 1024, first = tid * per;
+  uint32_t local = 0;
+  for (uint32_t i = first; i < min(E, first + per); ++i) local += hist[i];
+  scan[tid] = local;
+  __syncthreads();
+  for (uint32_t d = 1; d < 1024; d <<= 1) {
+    const uint32_t v = tid >= d ? scan[tid - d] : 0u;
+    __syncthreads();
+    scan[tid] += v;
+    __syncthreads();
+  }
+  uint32_t at = scan[tid] - local;
+  for (uint32_t i = first; i < min(E, first + per); ++i) {
+    count[i] = hist[i];
+    offset[i] = at;
+    cursor[i] = at;
+    at += hist[i];
+  }
+  __syncthreads();
+  for (uint32_t p = tid; p < pairs; p += 1024) {
+    const uint32_t sl = p / S, t = p - sl * S;
+    const uint32_t ix = min(g.slot[sl].idx[(int64_t)t * g.slot[sl].idx_stride], E - 1);
+    list[atomicAdd(&cursor[ix], 1u)] = sl << 16 | t;
+  }
+}
+
+hipError_t launch_moe_route(const LaunchCtx &lc, const MoeGemmDesc &g, uint32_t *count, uint32_t *offset, uint32_t *list) {
+  if (!g.S || !g.n_slot || !g.n_expert) return hipSuccess;
+  if (g.n_expert > MOE_ROUTE_MAX_EXPERTS || g.S > 65535 || g.n_slot > 8) return hipErrorInvalidValue;
+  CG_LAUNCH(lc, moe_route_kernel, 1, 1024, g, count, offset, list);
+  return hipGetLastError();
+}
+
+// A workgroup owns (128 output columns of NP problems, one expert) and walks that expert's pairs 128
+// at a time.  Token rows (gathered through the sorted list, bf16) and weight rows travel to LDS with
+// global_load_lds_dwordx4 exactly as in gemm_bf16_dma_kernel - same 1 KB wave loads, same XOR
+// swizzle, NS stages in flight - so a k-step no longer waits out a trip to memory.  Wavefront w
+// computes columns [32 w, 32 w + 32) of every 32-row tile that has a live row.
+template <int NP, int NS>
+__global__ void __launch_bounds__(256) moe_gemm_dma_kernel(MoeGemmDesc g) {
+  constexpr int BM_ = 128, BN_ = 128, BK = 64, MT = BM_ / 32;
+  constexpr int ROWS = BM_ + NP * BN_;    // the stacked [A; B0; B1] tile of a stage
+  constexpr int LPW = ROWS / 8 / 4;       // 1 KB loads per wave per stage
+  constexpr int STAGE = ROWS * BK * 2;    // bytes
+  extern __shared__ __attribute__((aligned(16))) uint16_t dma_smem[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const uint32_t prob = NP == 2 ? 0 : blockIdx.y;
+  const uint32_t K = g.K, N = g.prob[prob].N;
+  const uint32_t tiles_n = (N + BN_ - 1) / BN_;
+  // workgroups are dealt round-robin to the 8 XCDs: keep the column tiles of an expert (which share
+  // its token rows) on one of them
+  uint32_t id = blockIdx.x;
+  if (gridDim.x % 8 == 0) id = (id % 8) * (gridDim.x / 8) + id / 8;
+  const uint32_t e = id / tiles_n, n0 = (id - e * tiles_n) * BN_;
+  if (e >= g.n_expert) return;  // the grid is sized for the wider problem
+  const uint32_t cnt = g.route_count[e];
+  const uint32_t *list = g.route_list + g.route_offset[e];
+  const uint16_t *W[NP];
+  int64_t sbn[NP];
+#pragma unroll
+  for (int p = 0; p < NP; ++p) {
+    W[p] = (const uint16_t *)g.prob[prob + p].w + (int64_t)e * g.sb_index;
+    sbn[p] = g.prob[prob + p].sbn;
+  }
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint16_t *)dma_smem;
+  const int sw = (lane >> 1) & 7, half = lane >> 5;
+  const int n_steps = (int)(K / BK);
+  for (uint32_t m0 = 0; m0 < cnt; m0 += BM_) {
+    const int live_tiles = (int)min((uint32_t)MT, (cnt - m0 + 31) / 32);  // wave-uniform
+    f32x16 acc[NP][MT];
+#pragma unroll
+    for (int p = 0; p < NP; ++p)
+#pragma unroll
+      for (int h = 0; h < MT; ++h)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[p][h][i] = 0.f;
+    const uint16_t *gp[LPW];  // per-lane source of each of this wave's loads; advances by BK per stage
+#pragma unroll
+    for (int i = 0; i < LPW; ++i) {
+      const int q = wave * LPW + i;  // 8-row block of the stacked tile
+      const int R = q * 8 + (lane >> 3);
+      const int c = (lane & 7) ^ ((R >> 1) & 7);
+      if (q * 8 < BM_) {
+        // rows past the expert's last pair repeat it: loaded, multiplied, never stored
+        const uint32_t ent = list[min(m0 + (uint32_t)R, cnt - 1)], sl = ent >> 16, tok = ent & 0xFFFFu;
+        const uint16_t *rows = g.slot[0].a16;
+        int64_t bs = g.slot[0].a_bs;
+#pragma unroll
+        for (int s = 1; s < 8; ++s)
+          if (sl == (uint32_t)s) {
+            rows = g.slot[s].a16;
+            bs = g.slot[s].a_bs;
+          }
+        gp[i] = rows + (int64_t)tok * bs + c * 8;
+      } else {
+        const int rb = R - BM_, p = rb / BN_, col = rb - p * BN_;
+        gp[i] = W[p < NP ? p : 0] + (int64_t)min(n0 + (uint32_t)col, N - 1) * sbn[p < NP ? p : 0] + c * 8;
+      }
+    }
+    auto issue = [&](int buf) {
+#pragma unroll
+      for (int i = 0; i < LPW; ++i) {
+        lds_dma16(gp[i], lds0 + buf * STAGE + (wave * LPW + i) * 1024);
+        gp[i] += BK;
+      }
+    };
+    auto compute = [&](int buf) {
+      const uint16_t *As = dma_smem + buf * (STAGE / 2), *Bs = As + BM_ * BK;
+      bf16x8 af[2][MT], bfr[2][NP];
+      auto frags = [&](int ks, int set) {
+        const int o = ((ks * 2 + half) ^ sw) * 8;
+#pragma unroll
+        for (int h = 0; h < MT; ++h)
+          if (h < live_tiles) af[set][h] = *(const bf16x8 *)(&As[(h * 32 + (lane & 31)) * BK + o]);
+#pragma unroll
+        for (int p = 0; p < NP; ++p) bfr[set][p] = *(const bf16x8 *)(&Bs[(p * BN_ + wave * 32 + (lane & 31)) * BK + o]);
+      };
+      frags(0, 0);
+#pragma unroll
+      for (int ks = 0; ks < BK / 16; ++ks) {
+        if (ks + 1 < BK / 16) frags(ks + 1, (ks + 1) & 1);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int h = 0; h < MT; ++h)
+          if (h < live_tiles)
+#pragma unroll
+            for (int p = 0; p < NP; ++p)
+              acc[p][h] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[ks & 1][h], bfr[ks & 1][p], acc[p][h], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    };
+#pragma unroll
+    for (int s0 = 0; s0 < NS - 1; ++s0)
+      if (s0 < n_steps) issue(s0);
+    for (int step = 0; step < n_steps; ++step) {
+      if (step + NS - 1 <= n_steps) wait_vmcnt<(NS - 2) * LPW>();
+      else wait_vmcnt<0>();
+      __syncthreads();
+      if (step + NS - 1 < n_steps) issue((step + NS - 1) % NS);
+      compute(step % NS);
+    }
+    // ---- rows back to their slot and token: register i of tile h is row
+    // h * 32 + (i >> 2) * 8 + (lane >> 5) * 4 + (i & 3), column lane & 31
+    const uint32_t col = n0 + wave * 32 + (lane & 31);
+#pragma unroll
+    for (int h = 0; h < MT; ++h)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const uint32_t r = m0 + h * 32 + (i >> 2) * 8 + (lane >> 5) * 4 + (i & 3);
+        if (r < cnt && col < N) {
+          const uint32_t ent = list[r], sl = ent >> 16;
+          const uint64_t at = (uint64_t)(ent & 0xFFFFu) * N + col;
+          if (NP == 2) {
+            const float gt = acc[0][h][i];
+            const float hv = (g.fuse_glu == PRO_GEGLU ? gelu_ref(gt) : gt * sigmoid_ref(gt)) * acc[NP - 1][h][i];
+            uint16_t *out = g.slot[0].h16;
+#pragma unroll
+            for (int s = 1; s < 8; ++s)
+              if (sl == (uint32_t)s) out = g.slot[s].h16;
+            out[at] = (uint16_t)bf16_bits(hv);
+          } else {
+            float *out = g.slot[0].c[prob];
+#pragma unroll
+            for (int s = 1; s < 8; ++s)
+              if (sl == (uint32_t)s) out = g.slot[s].c[prob];
+            out[at] = acc[0][h][i];
+          }
+        }
+      }
+    wait_vmcnt<0>();
+    __syncthreads();  // the stages are refilled for the next 128 pairs
+  }
+}
+
+bool moe_gemm_pipelined_ok(const MoeGemmDesc &g) {
+  if (!g.route_count || !g.route_offset || !g.route_list || g.K % 64 || g.K < 64 || g.pro != PRO_NONE) return false;
+  for (uint32_t s = 0; s < g.n_slot; ++s)
+    if (!g.slot[s].a16 || (uintptr_t)g.slot[s].a16 % 16 || g.slot[s].a_bs % 8) return false;
+  for (uint32_t p = 0; p < g.n_prob; ++p)
+    if ((uintptr_t)g.prob[p].w % 16 || g.prob[p].sbn % 8 || g.sb_index % 8) return false;
+  return true;
+}
+
+template <int NP, int NS>
+static hipError_t launch_moe_gemm_dma(const LaunchCtx &lc, const MoeGemmDesc &g, dim3 grid) {
+  constexpr int smem = NS * (128 + NP * 128) * 64 * 2;
+  static bool configured = false;  // one attribute call per kernel and process
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute((const void *)moe_gemm_dma_kernel<NP, NS>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    if (e != hipSuccess) return e;
+    configured = true;
+  }
+  hipExtLaunchKernelGGL((moe_gemm_dma_kernel<NP, NS>), grid, dim3(256), smem, lc.stream, lc.ev_start, lc.ev_stop, 0, g);
+  return hipGetLastError();
+}
+
 hipError_t launch_moe_gemm(const LaunchCtx &lc, const MoeGemmDesc &g) {
   if (!g.S || !g.n_prob || !g.n_slot || !g.n_expert) return hipSuccess;
   if (g.S > 65535 || g.n_slot > 8 || g.n_prob > 2 || g.n_expert > 65535 || g.K % 8 || g.pro == PRO_RMSNORM)
@@ -1357,8 +1573,11 @@ hipError_t launch_moe_gemm(const LaunchCtx &lc, const MoeGemmDesc &g) {
   if (!max_n) return hipSuccess;
   if (g.fuse_glu) {
     if (g.n_prob != 2 || g.prob[0].N != g.prob[1].N || g.pro != PRO_NONE) return hipErrorInvalidValue;
+    if (moe_gemm_pipelined_ok(g)) return launch_moe_gemm_dma<2, 3>(lc, g, dim3((max_n + 127) / 128 * g.n_expert, 1, 1));
     dim3 grid((max_n + 127) / 128, g.n_expert, 1);
     CG_LAUNCH(lc, moe_gemm_kernel<2>, grid, 256, g);
+  } else if (moe_gemm_pipelined_ok(g)) {
+    return launch_moe_gemm_dma<1, 4>(lc, g, dim3((max_n + 127) / 128 * g.n_expert, g.n_prob, 1));
   } else {
     dim3 grid((max_n + 127) / 128, g.n_expert, g.n_prob);
     CG_LAUNCH(lc, moe_gemm_kernel<1>, grid, 256, g);

@@ -305,8 +305,18 @@ struct MoeGemmDesc {
     uint32_t N;
   } prob[2];
   uint32_t *err;                            // ERRF_INDEX_OOB for an index >= n_expert (served by the last expert)
+  // optional: the (slot, token) pairs already sorted by expert (launch_moe_route): pairs
+  // route_list[route_offset[e] .. + route_count[e]) = slot << 16 | token chose expert e
+  const uint32_t *route_count, *route_offset, *route_list;
 };
 hipError_t launch_moe_gemm(const LaunchCtx &lc, const MoeGemmDesc &g);
+// Sorts the S * n_slot (slot, token) pairs of g by expert into count / offset (n_expert words each) and
+// list (S * n_slot words); n_expert <= MOE_ROUTE_MAX_EXPERTS.  With these in g.route_*, bf16 input rows
+// (slot[].a16 for every slot) and K % 64 == 0, launch_moe_gemm streams the weights through a
+// multi-stage direct-to-LDS pipeline.
+enum { MOE_ROUTE_MAX_EXPERTS = 4096 };
+hipError_t launch_moe_route(const LaunchCtx &lc, const MoeGemmDesc &g, uint32_t *count, uint32_t *offset, uint32_t *list);
+bool moe_gemm_pipelined_ok(const MoeGemmDesc &g);
 // wrapping u32 matmul (ndarray's generic dot); all operands contiguous
 hipError_t launch_matmul_u32(const LaunchCtx &lc, const uint32_t *a, const uint32_t *b, uint32_t *c,
                              uint32_t batch, uint32_t M, uint32_t N, uint32_t K);

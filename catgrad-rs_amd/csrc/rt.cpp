@@ -2489,7 +2489,7 @@ int try_moe_gemm(cg_backend *be, cg_tensor *n, bool *done) {
       cg_tensor *g2 = nullptr, *u2 = nullptr;
       int ge2 = 0;
       ExpertOperand og, ou;
-      fits = match_glu(slot_a[sl], &g2, &u2, &ge2) && g2->op == N_MATMUL && u2->op == N_MATMUL && refs(g2) == 1 &&
+      fits = match_glu(slot_a[sl], &g2, &u2, &ge2) && g2->op == N_MATMUL && u2->op == N_MATMUL && refs(g2) == (ge2 ? 3 : 2) &&
              refs(u2) == 1 && g2->rank == 3 && u2->rank == 3 && g2->in[0] == u2->in[0] &&
              match_expert_operand(g2->in[1], S, &og) && match_expert_operand(u2->in[1], S, &ou) && og.idx == slot_idx[sl] &&
              ou.idx == slot_idx[sl];
@@ -2543,19 +2543,40 @@ int try_moe_gemm(cg_backend *be, cg_tensor *n, bool *done) {
         }
         d.pro = PRO_NONE;
         for (const Member &m : members) d.slot[m.slot].c[0] = (float *)m.c->st->ptr;
-        hipError_t e;
-        {
+        hipError_t e = hipSuccess;
+        // the pairs sorted by expert once, for both launches: count, offset (one word per expert), list
+        Storage *route = nullptr;
+        if (d.n_expert <= MOE_ROUTE_MAX_EXPERTS && H % 64 == 0 && F % 64 == 0) {
+          const size_t words = 2 * (size_t)d.n_expert + (size_t)S * d.n_slot;
+          st = dev_alloc(be, words * 4, &route);
+          if (st) {
+            drop_h();
+            return st;
+          }
+          uint32_t *rc = (uint32_t *)route->ptr, *ro = rc + d.n_expert, *rl = ro + d.n_expert;
+          {
+            KernelScope ks(be, "experts_route", (double)S * d.n_slot * 8, 0);
+            e = launch_moe_route(be->lc(), d, rc, ro, rl);
+          }
+          f.route_count = d.route_count = rc;
+          f.route_offset = d.route_offset = ro;
+          f.route_list = d.route_list = rl;
+        }
+        if (e == hipSuccess) {
           KernelScope ks(be, "gemm_experts_bf16", 2.0 * d.n_expert * F * H * 2 + (double)S * H * 2 + (double)d.n_slot * S * F * 2,
                          4.0 * d.n_slot * S * F * H);
+          if (be->trace_shapes) ks.rename("gemm_experts_bf16[gate*up]");
           e = launch_moe_gemm(be->lc(), f);
         }
         if (e == hipSuccess) {
           KernelScope ks(be, "gemm_experts_bf16",
                          (double)d.n_expert * d.prob[0].N * F * 2 + (double)d.n_slot * S * (F * 2 + d.prob[0].N * 4),
                          2.0 * d.n_slot * S * d.prob[0].N * F);
+          if (be->trace_shapes) ks.rename("gemm_experts_bf16[down]");
           e = launch_moe_gemm(be->lc(), d);
         }
         drop_h();
+        storage_release(route);
         if (e != hipSuccess) return fail(be, CG_ERR_DEVICE, hipGetErrorString(e));
         for (const Member &m : members) {
           forget_gemv_candidate(m.c);

@@ -242,6 +242,54 @@ def test_expert_slots_over_many_tokens(oracle, hip_bf16):
 
 
 @pytest.mark.gpu
+def test_expert_slots_sorted_by_expert(oracle, hip_bf16):
+    """The same block where both products have k a multiple of 64: the (slot, token) pairs are sorted by
+    expert once and both launches stream their operands through LDS stages.  A skewed routing: one
+    expert takes most pairs (several 128-row passes over its matrices, the last one partly filled), one
+    takes none, the others a few rows.  An index past the last expert is reported from there as well."""
+    import vectors
+    lang, nn = vectors.lang, vectors.nn
+    S, E, F, H, k = 600, 9, 192, 256, 2
+    g = np.random.default_rng(8)
+    x = g.standard_normal((S, 1, H)).astype(np.float32)
+    wg, wu = (U_round((g.standard_normal((E, F, H)) * 0.1).astype(np.float32)) for _ in range(2))
+    wd = U_round((g.standard_normal((E, H, F)) * 0.1).astype(np.float32))
+    idx = g.choice(np.array([0, 1, 2, 3, 4, 6, 7, 8]), size=(S, k), p=[.04, .04, .7, .04, .04, .04, .05, .05]).astype(np.uint32)
+    assert (idx == 2).sum() > 3 * 128 and not (idx == 5).any()
+    val = g.random((S, k)).astype(np.float32)
+
+    def f(b, xv, iv, vv, g_all, u_all, d_all):
+        xv = xv + xv - xv
+        total = None
+        for i in range(k):
+            slot = lang.get(b, 1, i, iv)
+            sel = lambda w: lang.transpose(b, 1, 2, lang.index(b, 0, slot, w))
+            gate = lang.matmul(b, xv, sel(g_all))
+            up = lang.matmul(b, xv, sel(u_all))
+            y = lang.matmul(b, nn.silu(b, gate) * up, sel(d_all))
+            wgt = lang.reshape(b, lang.shape(b, lang.get(b, 2, 0, y)), lang.get(b, 1, i, vv))
+            y = y * lang.broadcast(b, wgt, lang.shape(b, y))
+            total = y if total is None else total + y
+        return total
+    (ref,) = vectors.run(oracle, f, 1, x, idx, val, wg, wu, wd)
+    hip_bf16.trace(True)
+    hip_bf16.trace_reset()
+    (got,) = vectors.run(hip_bf16, f, 1, x, idx, val, wg, wu, wd)
+    rep = hip_bf16.trace_report()
+    hip_bf16.trace(False)
+    launches = {n: v["launches"] for n, v in rep.items()}
+    assert launches.get("gemm_experts_bf16") == 2 and launches.get("experts_route") == 1, launches
+    assert np.max(np.abs(got - ref)) <= 2e-2 * np.abs(ref).max()
+    # every row on its own: a token routed to the crowded expert and one routed to a quiet one
+    err = np.abs(got - ref).reshape(S, -1).max(axis=1)
+    assert err.max() <= 2e-2 * np.abs(ref).max()
+    bad = idx.copy()
+    bad[S - 1, 1] = E + 3
+    with pytest.raises(cg.abi.BackendPanic, match="index out of bounds"):
+        vectors.run(hip_bf16, f, 1, x, bad, val, wg, wu, wd)
+
+
+@pytest.mark.gpu
 def test_expert_mlp_over_many_tokens(oracle, hip_bf16):
     """One expert slot of the MoE block (models/qwen3.rs:104-123) over 300 tokens in bf16 mode: gate and
     up as expert-major products, SwiGLU computed on the way into down_proj's product; and an index
