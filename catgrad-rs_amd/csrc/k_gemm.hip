@@ -473,6 +473,11 @@ __device__ __forceinline__ void lds_dma16(const void *gptr, uint32_t lds_byte_of
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_byte_off), "v"(gptr)
                : "memory", "m0");
 }
+// the same for data read once (an expert's weight rows): streamed past the L2 lines worth keeping
+__device__ __forceinline__ void lds_dma16_stream(const void *gptr, uint32_t lds_byte_off) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off nt" ::"s"(lds_byte_off), "v"(gptr)
+               : "memory", "m0");
+}
 template <int N> __device__ __forceinline__ void wait_vmcnt() {
   __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
 }
@@ -1417,10 +1422,9 @@ __global__ void __launch_bounds__(256) moe_gemm_dma_kernel(MoeGemmDesc g) {
   const uint32_t prob = NP == 2 ? 0 : blockIdx.y;
   const uint32_t K = g.K, N = g.prob[prob].N;
   const uint32_t tiles_n = (N + BN_ - 1) / BN_;
-  // workgroups are dealt round-robin to the 8 XCDs: keep the column tiles of an expert (which share
-  // its token rows) on one of them
-  uint32_t id = blockIdx.x;
-  if (gridDim.x % 8 == 0) id = (id % 8) * (gridDim.x / 8) + id / 8;
+  // consecutive workgroups (dealt round-robin to the 8 XCDs) take the column tiles of one expert: giving an
+  // XCD a contiguous range of experts instead measured 10 % slower
+  const uint32_t id = blockIdx.x;
   const uint32_t e = id / tiles_n, n0 = (id - e * tiles_n) * BN_;
   if (e >= g.n_expert) return;  // the grid is sized for the wider problem
   const uint32_t cnt = g.route_count[e];
@@ -1470,7 +1474,8 @@ __global__ void __launch_bounds__(256) moe_gemm_dma_kernel(MoeGemmDesc g) {
     auto issue = [&](int buf) {
 #pragma unroll
       for (int i = 0; i < LPW; ++i) {
-        lds_dma16(gp[i], lds0 + buf * STAGE + (wave * LPW + i) * 1024);
+        if ((wave * LPW + i) * 8 < BM_) lds_dma16(gp[i], lds0 + buf * STAGE + (wave * LPW + i) * 1024);
+        else lds_dma16_stream(gp[i], lds0 + buf * STAGE + (wave * LPW + i) * 1024);
         gp[i] += BK;
       }
     };
@@ -1509,34 +1514,57 @@ __global__ void __launch_bounds__(256) moe_gemm_dma_kernel(MoeGemmDesc g) {
       if (step + NS - 1 < n_steps) issue((step + NS - 1) % NS);
       compute(step % NS);
     }
-    // ---- rows back to their slot and token: register i of tile h is row
-    // h * 32 + (i >> 2) * 8 + (lane >> 5) * 4 + (i & 3), column lane & 31
-    const uint32_t col = n0 + wave * 32 + (lane & 31);
+    // ---- rows back to their slot and token.  Register i of tile h is row
+    // h * 32 + (i >> 2) * 8 + (lane >> 5) * 4 + (i & 3), column lane & 31.  The tile is staged in LDS
+    // (the operand stages are free now) so that a row leaves as 16-byte pieces: f32 for a plain
+    // product, bf16 act(gate) * up for the fused pair.
+    __syncthreads();  // every wave is done reading the last stage
+    constexpr int TP = NP == 2 ? BN_ + 8 : BN_ + 4;  // row pitch in elements (keeps 16-byte alignment)
+    if (NP == 2) {
+      uint16_t *T = dma_smem;
 #pragma unroll
-    for (int h = 0; h < MT; ++h)
+      for (int h = 0; h < MT; ++h)
+        if (h < live_tiles)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const uint32_t r = m0 + h * 32 + (i >> 2) * 8 + (lane >> 5) * 4 + (i & 3);
-        if (r < cnt && col < N) {
-          const uint32_t ent = list[r], sl = ent >> 16;
-          const uint64_t at = (uint64_t)(ent & 0xFFFFu) * N + col;
-          if (NP == 2) {
+          for (int i = 0; i < 16; ++i) {
             const float gt = acc[0][h][i];
             const float hv = (g.fuse_glu == PRO_GEGLU ? gelu_ref(gt) : gt * sigmoid_ref(gt)) * acc[NP - 1][h][i];
-            uint16_t *out = g.slot[0].h16;
-#pragma unroll
-            for (int s = 1; s < 8; ++s)
-              if (sl == (uint32_t)s) out = g.slot[s].h16;
-            out[at] = (uint16_t)bf16_bits(hv);
-          } else {
-            float *out = g.slot[0].c[prob];
-#pragma unroll
-            for (int s = 1; s < 8; ++s)
-              if (sl == (uint32_t)s) out = g.slot[s].c[prob];
-            out[at] = acc[0][h][i];
+            T[(h * 32 + (i >> 2) * 8 + (lane >> 5) * 4 + (i & 3)) * TP + wave * 32 + (lane & 31)] = (uint16_t)bf16_bits(hv);
           }
+    } else {
+      float *T = (float *)dma_smem;
+#pragma unroll
+      for (int h = 0; h < MT; ++h)
+        if (h < live_tiles)
+#pragma unroll
+          for (int i = 0; i < 16; ++i)
+            T[(h * 32 + (i >> 2) * 8 + (lane >> 5) * 4 + (i & 3)) * TP + wave * 32 + (lane & 31)] = acc[0][h][i];
+    }
+    __syncthreads();
+    {
+      constexpr int EPV = NP == 2 ? 8 : 4;        // elements per 16-byte piece
+      constexpr int PPR = BN_ / EPV;              // pieces per row
+      const uint32_t rows_here = min((uint32_t)BM_, cnt - m0);
+      for (uint32_t idx = tid; idx < rows_here * PPR; idx += 256) {
+        const uint32_t r = idx / PPR, c = (idx - r * PPR) * EPV;
+        if (n0 + c >= N) continue;  // N % 8 == 0: a piece is inside or outside
+        const uint32_t ent = list[m0 + r], sl = ent >> 16;
+        const uint64_t at = (uint64_t)(ent & 0xFFFFu) * N + n0 + c;
+        if (NP == 2) {
+          uint16_t *out = g.slot[0].h16;
+#pragma unroll
+          for (int s2 = 1; s2 < 8; ++s2)
+            if (sl == (uint32_t)s2) out = g.slot[s2].h16;
+          *(uint4 *)(out + at) = *(const uint4 *)(dma_smem + r * TP + c);
+        } else {
+          float *out = g.slot[0].c[prob];
+#pragma unroll
+          for (int s2 = 1; s2 < 8; ++s2)
+            if (sl == (uint32_t)s2) out = g.slot[s2].c[prob];
+          *(float4 *)(out + at) = *(const float4 *)((const float *)dma_smem + r * TP + c);
         }
       }
+    }
     wait_vmcnt<0>();
     __syncthreads();  // the stages are refilled for the next 128 pairs
   }
@@ -1547,13 +1575,18 @@ bool moe_gemm_pipelined_ok(const MoeGemmDesc &g) {
   for (uint32_t s = 0; s < g.n_slot; ++s)
     if (!g.slot[s].a16 || (uintptr_t)g.slot[s].a16 % 16 || g.slot[s].a_bs % 8) return false;
   for (uint32_t p = 0; p < g.n_prob; ++p)
-    if ((uintptr_t)g.prob[p].w % 16 || g.prob[p].sbn % 8 || g.sb_index % 8) return false;
+    if ((uintptr_t)g.prob[p].w % 16 || g.prob[p].sbn % 8 || g.sb_index % 8 || g.prob[p].N % 8) return false;
+  for (uint32_t s = 0; s < g.n_slot; ++s)  // rows leave as 16-byte pieces
+    if (g.fuse_glu ? (uintptr_t)g.slot[s].h16 % 16 != 0 : ((uintptr_t)g.slot[s].c[0] % 16 != 0 || (g.n_prob > 1 && (uintptr_t)g.slot[s].c[1] % 16 != 0)))
+      return false;
   return true;
 }
 
 template <int NP, int NS>
 static hipError_t launch_moe_gemm_dma(const LaunchCtx &lc, const MoeGemmDesc &g, dim3 grid) {
-  constexpr int smem = NS * (128 + NP * 128) * 64 * 2;
+  // the operand stages, or the staged output tile (f32 rows of 128 + 4, or bf16 rows of 128 + 8) if that is larger
+  constexpr int stages = NS * (128 + NP * 128) * 64 * 2, tile = NP == 2 ? 128 * (128 + 8) * 2 : 128 * (128 + 4) * 4;
+  constexpr int smem = stages > tile ? stages : tile;
   static bool configured = false;  // one attribute call per kernel and process
   if (!configured) {
     hipError_t e = hipFuncSetAttribute((const void *)moe_gemm_dma_kernel<NP, NS>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
@@ -1577,7 +1610,7 @@ hipError_t launch_moe_gemm(const LaunchCtx &lc, const MoeGemmDesc &g) {
     dim3 grid((max_n + 127) / 128, g.n_expert, 1);
     CG_LAUNCH(lc, moe_gemm_kernel<2>, grid, 256, g);
   } else if (moe_gemm_pipelined_ok(g)) {
-    return launch_moe_gemm_dma<1, 4>(lc, g, dim3((max_n + 127) / 128 * g.n_expert, g.n_prob, 1));
+    return launch_moe_gemm_dma<1, 2>(lc, g, dim3((max_n + 127) / 128 * g.n_expert, g.n_prob, 1));
   } else {
     dim3 grid((max_n + 127) / 128, g.n_expert, g.n_prob);
     CG_LAUNCH(lc, moe_gemm_kernel<1>, grid, 256, g);
