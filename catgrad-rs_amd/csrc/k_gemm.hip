@@ -487,17 +487,24 @@ template <int N> __device__ __forceinline__ void wait_vmcnt() {
 // NS stages of operand tiles in LDS: two when several workgroups share a CU (large problems, bound by
 // the L2 -> LDS rate), four when a CU holds one workgroup and every k-step would otherwise wait out a
 // full trip to HBM (few tiles, cold weights: the prefill-sized products).
-template <int BM_, int BN_, int WR, int WC, bool EPI, int NS>
+// DUAL (with EPI): the B tile stacks 128 rows of g.b (gate_proj) on 128 rows of g.dual_b (up_proj), a
+// wavefront holds the same columns of both products, and the tile that leaves is act(gate) * up,
+// 128 columns wide (BN_ = 256 counts the stacked rows): the gated MLP's two products and its
+// activation in one pass over the activations, neither product ever stored.
+template <int BM_, int BN_, int WR, int WC, bool EPI, int NS, bool DUAL = false>
 __global__ void __launch_bounds__(WR *WC * 64) gemm_bf16_dma_kernel(GemmDesc g) {
   constexpr int NW = WR * WC, BK = 64;
   constexpr int WM = BM_ / WR, WN = BN_ / WC, TM = WM / 32, TN = WN / 32;
+  constexpr int BNO = DUAL ? BN_ / 2 : BN_;    // output columns of a tile
+  constexpr int OC = BNO / WC, TNH = OC / 32;  // DUAL: output columns per wave, fragments per product
+  static_assert(!DUAL || (EPI && BN_ == 256 && TN == 2 * TNH), "stacked gate / up tile");
   constexpr int LPW = (BM_ + BN_) / 8 / NW;   // 1 KB loads per wave per stage
   constexpr int STAGE = (BM_ + BN_) * BK * 2;  // bytes
   extern __shared__ __attribute__((aligned(16))) uint16_t dma_smem[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / WC, wn = wave % WC;
-  const uint32_t tiles_m = (g.M + BM_ - 1) / BM_, tiles_n = (g.N + BN_ - 1) / BN_;
+  const uint32_t tiles_m = (g.M + BM_ - 1) / BM_, tiles_n = (g.N + BNO - 1) / BNO;
   const uint32_t per_batch = tiles_m * tiles_n, batch = g.nb0 * g.nb1;
   // Workgroups are dealt round-robin to the 8 XCDs (one L2 each): give every XCD a contiguous
   // range of logical tiles, and walk tiles in groups of 4 tile rows so that the ~32 tiles an
@@ -511,9 +518,10 @@ __global__ void __launch_bounds__(WR *WC * 64) gemm_bf16_dma_kernel(GemmDesc g) 
   constexpr uint32_t GM = 4;
   const uint32_t first_m = t / (GM * tiles_n) * GM, gsz = min(tiles_m - first_m, GM);
   const uint32_t tg = t % (GM * tiles_n);
-  const uint32_t m0 = (first_m + tg % gsz) * BM_, n0_all = tg / gsz * BN_;
+  const uint32_t m0 = (first_m + tg % gsz) * BM_, n0_all = tg / gsz * BNO;
   const uint16_t *A = (const uint16_t *)g.a + b0 * g.sa_b0 + b1 * g.sa_b1;
   const uint16_t *B = (const uint16_t *)g.b + b0 * g.sb_b0 + b1 * g.sb_b1;
+  const uint16_t *B2 = DUAL ? (const uint16_t *)g.dual_b + b0 * g.sb_b0 + b1 * g.sb_b1 : nullptr;
   float *C = (g.splits > 1 ? g.workspace + (uint64_t)split * batch * g.M * g.N : g.c) +
              (uint64_t)bz * g.M * g.N;
   // grouped products: this tile's columns belong to one of them (tiles never straddle two)
@@ -549,6 +557,7 @@ __global__ void __launch_bounds__(WR *WC * 64) gemm_bf16_dma_kernel(GemmDesc g) 
     const int R = q * 8 + (lane >> 3);
     const int c = (lane & 7) ^ ((R >> 1) & 7);
     if (q * 8 < BM_) gp[i] = A + (int64_t)min(m0 + R, g.M - 1) * g.sam + k_begin + c * 8;
+    else if (DUAL) gp[i] = (R - BM_ < BNO ? B : B2) + (int64_t)min(n0 + (uint32_t)((R - BM_) % BNO), Nl - 1) * g.sbn + k_begin + c * 8;
     else gp[i] = B + (int64_t)min(n0 + (R - BM_), Nl - 1) * g.sbn + k_begin + c * 8;
   }
   auto issue = [&](int buf) {
@@ -568,8 +577,11 @@ __global__ void __launch_bounds__(WR *WC * 64) gemm_bf16_dma_kernel(GemmDesc g) 
       for (int i = 0; i < TM; ++i)
         af[set][i] = *(const bf16x8 *)(&As[(wm * WM + i * 32 + (lane & 31)) * BK + p]);
 #pragma unroll
-      for (int j = 0; j < TN; ++j)
-        bfr[set][j] = *(const bf16x8 *)(&Bs[(wn * WN + j * 32 + (lane & 31)) * BK + p]);
+      for (int j = 0; j < TN; ++j) {
+        // DUAL: fragments [0, TNH) are this wave's gate columns, [TNH, TN) the same columns of up
+        const int brow = DUAL ? (j / TNH) * BNO + wn * OC + (j % TNH) * 32 : wn * WN + j * 32;
+        bfr[set][j] = *(const bf16x8 *)(&Bs[(brow + (lane & 31)) * BK + p]);
+      }
     };
     frags(0, 0);
 #pragma unroll
@@ -598,35 +610,62 @@ __global__ void __launch_bounds__(WR *WC * 64) gemm_bf16_dma_kernel(GemmDesc g) 
     compute(step % NS);
   }
   if constexpr (EPI) {
-    constexpr int TP = BN_ + 4;  // row pitch of the staged tile (floats)
+    constexpr int TP = BNO + 4;  // row pitch of the staged tile (floats)
     float *T = (float *)dma_smem;
     __syncthreads();  // every wave is done with the operand stages
+    if constexpr (DUAL) {
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
+      for (int i = 0; i < TM; ++i)
 #pragma unroll
-      for (int j = 0; j < TN; ++j)
+        for (int j = 0; j < TNH; ++j)
 #pragma unroll
-        for (int e = 0; e < 16; ++e)
-          T[(wm * WM + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3)) * TP + wn * WN + j * 32 + (lane & 31)] =
-              acc[i][j][e];
+          for (int e = 0; e < 16; ++e) {
+            const float gt = acc[i][j][e];
+            T[(wm * WM + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3)) * TP + wn * OC + j * 32 + (lane & 31)] =
+                (g.glu_kind ? gelu_ref(gt) : gt * sigmoid_ref(gt)) * acc[i][TNH + j][e];
+          }
+    } else {
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+          for (int e = 0; e < 16; ++e)
+            T[(wm * WM + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3)) * TP + wn * WN + j * 32 + (lane & 31)] =
+                acc[i][j][e];
+    }
     __syncthreads();
-    for (int idx = tid; idx < BM_ * BN_ / 4; idx += NW * 64) {
-      const int r = idx / (BN_ / 4), c4 = (idx % (BN_ / 4)) * 4;
-      const uint32_t row = m0 + r, col = n0 + c4;
-      if (row < g.M && col < Nl) {  // N % 4 == 0: a group of four columns is inside or outside
-        const uint64_t at = (uint64_t)row * Nl + col;
+    // four 16-byte pieces per thread and round: the gate values of a round are requested together, so a
+    // round waits for memory once (a store to C could alias Gate as far as the compiler knows, which
+    // would otherwise order every load behind the previous piece's stores)
+    constexpr int PIECES = BM_ * BNO / 4, ROUND = NW * 64 * 4;
+    for (int base = 0; base < PIECES; base += ROUND) {
+      float4 gt[4];
+      uint64_t at[4];
+      bool live[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int idx = base + u * NW * 64 + tid, r = idx / (BNO / 4), c4 = (idx % (BNO / 4)) * 4;
+        const uint32_t row = m0 + r, col = n0 + c4;
+        live[u] = idx < PIECES && row < g.M && col < Nl;  // N % 4 == 0: a group of four columns is inside or outside
+        at[u] = (uint64_t)row * Nl + col;
+        if (!DUAL && Gate && live[u]) gt[u] = *(const float4 *)(Gate + at[u]);
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        if (!live[u]) continue;
+        const int idx = base + u * NW * 64 + tid, r = idx / (BNO / 4), c4 = (idx % (BNO / 4)) * 4;
         float4 v = *(const float4 *)(&T[r * TP + c4]);
-        if (Gate) {
-          const float4 gt = *(const float4 *)(Gate + at);
+        if (!DUAL && Gate) {
           if (g.glu_kind) {
-            v.x *= gelu_ref(gt.x); v.y *= gelu_ref(gt.y); v.z *= gelu_ref(gt.z); v.w *= gelu_ref(gt.w);
+            v.x *= gelu_ref(gt[u].x); v.y *= gelu_ref(gt[u].y); v.z *= gelu_ref(gt[u].z); v.w *= gelu_ref(gt[u].w);
           } else {
-            v.x *= gt.x * sigmoid_ref(gt.x); v.y *= gt.y * sigmoid_ref(gt.y);
-            v.z *= gt.z * sigmoid_ref(gt.z); v.w *= gt.w * sigmoid_ref(gt.w);
+            v.x *= gt[u].x * sigmoid_ref(gt[u].x); v.y *= gt[u].y * sigmoid_ref(gt[u].y);
+            v.z *= gt[u].z * sigmoid_ref(gt[u].z); v.w *= gt[u].w * sigmoid_ref(gt[u].w);
           }
         }
-        *(float4 *)(C + at) = v;
-        if (C16) *(uint2 *)(C16 + at) = bf16_pack4(v);
+        *(float4 *)(C + at[u]) = v;
+        if (C16) *(uint2 *)(C16 + at[u]) = bf16_pack4(v);
       }
     }
     return;
@@ -644,18 +683,18 @@ __global__ void __launch_bounds__(WR *WC * 64) gemm_bf16_dma_kernel(GemmDesc g) 
     }
 }
 
-template <int BM_, int BN_, int WR, int WC, bool EPI = false, int NS = 2>
+template <int BM_, int BN_, int WR, int WC, bool EPI = false, int NS = 2, bool DUAL = false>
 static hipError_t launch_gemm_dma(const LaunchCtx &lc, const GemmDesc &g, uint32_t grid) {
-  constexpr int stages = NS * (BM_ + BN_) * 64 * 2, staged_tile = EPI ? BM_ * (BN_ + 4) * 4 : 0;
+  constexpr int stages = NS * (BM_ + BN_) * 64 * 2, staged_tile = EPI ? BM_ * ((DUAL ? BN_ / 2 : BN_) + 4) * 4 : 0;
   constexpr int smem = stages > staged_tile ? stages : staged_tile;
   static bool configured = false;  // one attribute call per kernel and process
   if (!configured) {
-    hipError_t e = hipFuncSetAttribute((const void *)gemm_bf16_dma_kernel<BM_, BN_, WR, WC, EPI, NS>,
+    hipError_t e = hipFuncSetAttribute((const void *)gemm_bf16_dma_kernel<BM_, BN_, WR, WC, EPI, NS, DUAL>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return e;
     configured = true;
   }
-  hipExtLaunchKernelGGL((gemm_bf16_dma_kernel<BM_, BN_, WR, WC, EPI, NS>), dim3(grid), dim3(WR * WC * 64), smem,
+  hipExtLaunchKernelGGL((gemm_bf16_dma_kernel<BM_, BN_, WR, WC, EPI, NS, DUAL>), dim3(grid), dim3(WR * WC * 64), smem,
                         lc.stream, lc.ev_start, lc.ev_stop, 0, g);
   return hipGetLastError();
 }
@@ -1805,7 +1844,7 @@ hipError_t launch_matmul(const LaunchCtx &lc, const GemmDesc &g, const char **ke
   const bool one_row = g.M <= 8 && g.a_stype == ST_F32 && g.K > 0 && (b_unit_k || b_unit_n);
   if (g.b_index && !one_row) return hipErrorInvalidValue;
   if (g.c_add && !one_row && g.splits <= 1) return hipErrorInvalidValue;
-  if ((g.glu_gate || g.c16 || g.n_group) && !gemm_epilogue_ok(g)) return hipErrorInvalidValue;
+  if ((g.glu_gate || g.c16 || g.n_group || g.dual_b) && !gemm_epilogue_ok(g)) return hipErrorInvalidValue;
 
   if (g.M <= 8 && g.a_stype == ST_F32 && g.K > 0) {
     if (b_unit_k) {
@@ -1853,7 +1892,13 @@ hipError_t launch_matmul(const LaunchCtx &lc, const GemmDesc &g, const char **ke
       if (g.n_group && (batch != 1 || splits != 1 || g.glu_gate || g.c16)) return hipErrorInvalidValue;
       const uint64_t t128 = (uint64_t)((g.M + 127) / 128) * ((g.N + 127) / 128) * batch * splits;
       const bool deep = t128 < 2 * (uint64_t)lc.n_cus;  // at most one workgroup per CU at a time: four stages
-      if (g.glu_gate || g.c16) {  // the epilogue variant stages a 128 x 128 tile
+      if (g.dual_b) {  // gate and up stacked: 128 output columns per tile, 256 rows when that still fills the CUs
+        if (g.n_group || g.glu_gate || splits != 1) return hipErrorInvalidValue;
+        const uint64_t d256 = (uint64_t)((g.M + 255) / 256) * ((g.N + 127) / 128) * batch;
+        const uint64_t d128 = (uint64_t)((g.M + 127) / 128) * ((g.N + 127) / 128) * batch;
+        if (d256 >= (uint64_t)lc.n_cus) e = launch_gemm_dma<256, 256, 2, 4, true, 2, true>(lc, gg, (uint32_t)d256);
+        else e = launch_gemm_dma<128, 256, 2, 2, true, 3, true>(lc, gg, (uint32_t)d128);
+      } else if (g.glu_gate || g.c16) {  // the epilogue variant stages a 128 x 128 tile
         if (deep) e = launch_gemm_dma<128, 128, 2, 2, true, 4>(lc, gg, (uint32_t)t128);
         else e = launch_gemm_dma<128, 128, 2, 2, true, 2>(lc, gg, (uint32_t)t128);
       } else if (t256 >= (uint64_t)lc.n_cus && grp256) {

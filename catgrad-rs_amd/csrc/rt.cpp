@@ -1314,16 +1314,61 @@ bool match_glu(cg_tensor *root, cg_tensor **gate, cg_tensor **up, int *gelu) {
 // of an MLP in up_proj's epilogue).  `applied` tells the caller whether the kernel that ran could.
 struct MatmulEpilogue {
   const float *gate = nullptr;  // laid out like the product
+  // or: the right operand of the gate product itself (realised, laid out like this product's); the
+  // kernel then computes both products and stores act(A . dual_w) * (A . B)
+  cg_tensor *dual_w = nullptr;
   int gelu = 0;
   bool applied = false;
 };
 int realize_matmul(cg_backend *be, cg_tensor *n, cg_tensor *addend, bool *added, MatmulEpilogue *ep);
+
+// the same tensor, or two reshapes of one tensor to one shape (each linear folds the batch into its rows itself)
+static bool same_rows(const cg_tensor *a, const cg_tensor *b) {
+  if (a == b) return true;
+  return a->op == N_RESHAPE && b->op == N_RESHAPE && a->in[0] == b->in[0] && a->rank == b->rank &&
+         std::equal(a->shape, a->shape + a->rank, b->shape);
+}
 
 int try_glu(cg_backend *be, cg_tensor *root, bool *done) {
   cg_tensor *gate = nullptr, *up = nullptr;
   int gelu = 0;
   if (!match_glu(root, &gate, &up, &gelu)) return CG_OK;
   cg_tensor *gc = nullptr, *uc = nullptr;
+  // bf16 mode, many rows, gate and up both still deferred products of the same rows: one GEMM over the
+  // two weight matrices stacked tile by tile, the activation applied where both products sit in
+  // registers; the gate product never exists as a tensor.
+  if ((be->flags & CG_FLAG_BF16) && root->dtype == CG_F32) {
+    cg_tensor *gm = gate, *um = up;
+    if (gm->op == N_RESHAPE && refs(gm->in[0]) == 1) gm = gm->in[0];
+    if (um->op == N_RESHAPE && refs(um) == 1) um = um->in[0];
+    const int r = um->rank;
+    if (gm->op == N_MATMUL && um->op == N_MATMUL && gm != um && refs(gate) == (gelu ? 3 : 2) && refs(up) == 1 && refs(um) == 1 &&
+        same_rows(gm->in[0], um->in[0]) && !gm->gemv_candidate && !um->gemv_candidate && gm->rank == r && r >= 2 &&
+        std::equal(gm->shape, gm->shape + r, um->shape) && um->size() == um->shape[r - 2] * um->shape[r - 1] &&
+        um->shape[r - 2] >= 64 && um->shape[r - 1] >= 64 && um->shape[r - 1] % 8 == 0 && um->in[0]->shape[r - 1] % 64 == 0) {
+      cg_tensor *wg = gm->in[1], *wu = um->in[1];
+      TRY(realize(be, wg));
+      TRY(realize(be, wu));
+      if (wg->stype == ST_BF16 && wu->stype == ST_BF16 && wg->rank == wu->rank && std::equal(wg->shape, wg->shape + wg->rank, wu->shape) &&
+          std::equal(wg->strides, wg->strides + wg->rank, wu->strides) && wu->strides[wu->rank - 2] == 1 &&
+          (uintptr_t)data_ptr(wg) % 16 == 0 && (uintptr_t)data_ptr(wu) % 16 == 0) {
+        MatmulEpilogue ep;
+        ep.dual_w = wg;
+        ep.gelu = gelu;
+        TRY(realize_matmul(be, um, nullptr, nullptr, &ep));
+        if (ep.applied) {  // um holds the gated activations and nobody else can see it: root takes its storage
+          root->st = um->st;
+          root->st->rc.fetch_add(1);
+          root->stype = um->stype;
+          root->offset = um->offset;
+          contiguous_strides(root->rank, root->shape, root->strides);
+          finish_fused(root);  // releases the activation chain and with it the gate product
+          *done = true;
+          return CG_OK;
+        }
+      }
+    }
+  }
   TRY(contiguous(be, gate, &gc));
   // bf16 mode, many rows: up_proj's GEMM applies act(gate) to its product before storing it.  A
   // reshape between the product and the multiply (batch folded into the rows for the linear and
@@ -3061,7 +3106,8 @@ int realize_matmul(cg_backend *be, cg_tensor *n, cg_tensor *addend, bool *added,
       }
     }
     Storage *ws = nullptr;
-    const uint32_t splits = group.empty() ? gemm_split_k(be->lc(), g) : 1;
+    const bool dual = ep && ep->dual_w;  // twice the work per tile: no k-slices on top
+    const uint32_t splits = group.empty() && !dual ? gemm_split_k(be->lc(), g) : 1;
     if (splits > 1) {
       TRY(dev_alloc(be, (size_t)splits * n->size() * 4, &ws));
       g.workspace = (float *)ws->ptr;
@@ -3072,7 +3118,15 @@ int realize_matmul(cg_backend *be, cg_tensor *n, cg_tensor *addend, bool *added,
         *added = true;
       }
     }
-    if (ep && !g.c_add && gemm_epilogue_ok(g)) {
+    if (dual) {
+      if (!g.c_add && batch == 1 && !ex.w && g.sbk == 1 && g.b_stype == ST_BF16 && gemm_epilogue_ok(g)) {
+        g.dual_b = g.b;  // this product is up_proj's; the activation goes on the other one
+        g.b = data_ptr(ep->dual_w);
+        g.glu_kind = ep->gelu;
+        (void)twin_for_result(be, n, &g.c16);  // the gated activations are down_proj's operand
+        ep->applied = true;
+      }
+    } else if (ep && !g.c_add && gemm_epilogue_ok(g)) {
       g.glu_gate = ep->gate;
       g.glu_kind = ep->gelu;
       (void)twin_for_result(be, n, &g.c16);  // the gated activations are down_proj's operand
@@ -3082,15 +3136,17 @@ int realize_matmul(cg_backend *be, cg_tensor *n, cg_tensor *addend, bool *added,
     hipError_t e;
     {
       // grouped: g.N counts every member's columns; B and C bytes scale with it
+      // stacked gate / up: two weight matrices read, two products computed
+      const double nb = g.dual_b ? 2.0 : 1.0;
       KernelScope ks(be, kname,
-                     uniq(A, sao) + (uniq(B, sbo) * (ex.w ? (double)batch : 1.0) + (double)n->size() * 4) * ((double)g.N / N),
-                     2.0 * batch * M * g.N * K);
+                     uniq(A, sao) + (uniq(B, sbo) * nb * (ex.w ? (double)batch : 1.0) + (double)n->size() * 4) * ((double)g.N / N),
+                     2.0 * nb * batch * M * g.N * K);
       e = launch_matmul(be->lc(), g, &kname);
       ks.rename(kname);
       if (be->trace_shapes) {  // per-shape records: gemm_mfma_bf16[b32,512x512x64,s1]
         char buf[96];
         snprintf(buf, sizeof buf, "%s[b%lld,%ux%ux%u,s%u%s]", kname, (long long)batch, M, g.N, K, splits,
-                 group.empty() ? "" : ",grouped");
+                 g.dual_b ? ",gate*up" : group.empty() ? "" : ",grouped");
         ks.rename(buf);
       }
     }
