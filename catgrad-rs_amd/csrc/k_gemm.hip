@@ -664,7 +664,7 @@ __global__ void __launch_bounds__(WR *WC * 64) gemm_bf16_dma_kernel(GemmDesc g) 
             v.z *= gt[u].z * sigmoid_ref(gt[u].z); v.w *= gt[u].w * sigmoid_ref(gt[u].w);
           }
         }
-        *(float4 *)(C + at[u]) = v;
+        if (!DUAL || g.c) *(float4 *)(C + at[u]) = v;
         if (C16) *(uint2 *)(C16 + at[u]) = bf16_pack4(v);
       }
     }

@@ -215,7 +215,7 @@ struct GemmDesc {
   uint16_t *c16;
   // optional (same conditions): a second B matrix laid out like b (same strides, same N).  The kernel computes
   // both products and stores C = act(A . b) * (A . dual_b) - gate_proj, up_proj and the gated activation of an
-  // MLP in one launch
+  // MLP in one launch; c may be null when only the bf16 copy c16 is wanted
   const void *dual_b;
   // optional (same kernel, one batch, no split-K): n_group products that share A, K and the strides of
   // B (q/k/v of a prefill) as one launch.  N is the sum of grp_n; columns [0, grp_n[0]) belong to the

@@ -3123,7 +3123,13 @@ int realize_matmul(cg_backend *be, cg_tensor *n, cg_tensor *addend, bool *added,
         g.dual_b = g.b;  // this product is up_proj's; the activation goes on the other one
         g.b = data_ptr(ep->dual_w);
         g.glu_kind = ep->gelu;
-        (void)twin_for_result(be, n, &g.c16);  // the gated activations are down_proj's operand
+        // The gated activations are down_proj's operand, which reads them as bf16: store them as bf16
+        // only (a later reader of another kind widens them, like a matrix uploaded in this mode).
+        storage_release(n->st);
+        n->st = nullptr;
+        TRY(alloc_result(be, n, ST_BF16));
+        g.c = nullptr;
+        g.c16 = (uint16_t *)n->st->ptr;
         ep->applied = true;
       }
     } else if (ep && !g.c_add && gemm_epilogue_ok(g)) {
