@@ -1902,7 +1902,13 @@ hipError_t launch_matmul(const LaunchCtx &lc, const GemmDesc &g, const char **ke
         if (deep) e = launch_gemm_dma<128, 128, 2, 2, true, 4>(lc, gg, (uint32_t)t128);
         else e = launch_gemm_dma<128, 128, 2, 2, true, 2>(lc, gg, (uint32_t)t128);
       } else if (t256 >= (uint64_t)lc.n_cus && grp256) {
-        e = launch_gemm_dma<256, 256, 2, 4>(lc, gg, (uint32_t)t256);
+        // 256 x 256 tiles run one to a CU, 128 x 128 two to a CU: when the big tiles leave the last round of
+        // workgroups mostly empty (320 tiles on 256 CUs), the small ones fill the machine better
+        auto fill = [&](uint64_t tiles, uint64_t slots) { return (double)tiles / (double)((tiles + slots - 1) / slots * slots); };
+        if (!g.n_group && fill(t128, 2 * (uint64_t)lc.n_cus) > 1.15 * fill(t256, (uint64_t)lc.n_cus))
+          e = launch_gemm_dma<128, 128, 2, 2>(lc, gg, (uint32_t)t128);
+        else
+          e = launch_gemm_dma<256, 256, 2, 4>(lc, gg, (uint32_t)t256);
       } else if (splits == 1 && t128 * 2 <= (uint64_t)lc.n_cus && g.N >= 128) {
         // too few 128 x 128 tiles for the CUs and no split-K to multiply them: halve the tile
         e = launch_gemm_dma<128, 64, 2, 2, false, 4>(lc, gg, (uint32_t)((uint64_t)((g.M + 127) / 128) * ((g.N + 63) / 64) * batch));
