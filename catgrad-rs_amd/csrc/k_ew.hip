@@ -280,6 +280,79 @@ __device__ __forceinline__ void decompose(const Program &p, uint64_t lin,
   }
 }
 
+// The evaluator of a small launch.  Such a launch spends its time fetching instructions, not data: it
+// starts with a cold instruction cache, and the register-file evaluator above is a few hundred
+// cache lines of unrolled moves (one copy per stack depth) that a short program hops across.  Here
+// the stack lives in LDS, indexed by the depth the instruction carries, so the code is one compact
+// loop: a load path and one case per opcode, each written once for the VEC elements of a thread.
+template <int VEC>
+__device__ __forceinline__ void bin_vec(uint32_t op, const uint32_t *a, const uint32_t *b, uint32_t *r, uint32_t *err) {
+#define CG_BIN(EXPR) _Pragma("unroll") for (int j = 0; j < VEC; ++j) { const uint32_t x = a[j * 256], y = b[j * 256]; r[j * 256] = (EXPR); } break;
+  switch (op) {
+    case E_ADD_F: CG_BIN(as_u(as_f(x) + as_f(y)))
+    case E_SUB_F: CG_BIN(as_u(as_f(x) - as_f(y)))
+    case E_MUL_F: CG_BIN(as_u(as_f(x) * as_f(y)))
+    case E_DIV_F: CG_BIN(as_u(as_f(x) / as_f(y)))
+    case E_POW_F: CG_BIN(as_u(nf_pow(as_f(x), as_f(y))))
+    case E_LT_F: CG_BIN(as_u(as_f(x) < as_f(y) ? 1.f : 0.f))
+    case E_EQ_F: CG_BIN(as_u(as_f(x) == as_f(y) ? 1.f : 0.f))
+    case E_ADD_U: CG_BIN(x + y)
+    case E_SUB_U: CG_BIN(x - y)
+    case E_MUL_U: CG_BIN(x * y)
+    case E_POW_U: CG_BIN(upow(x, y))
+    case E_LT_U: CG_BIN(x < y ? 1u : 0u)
+    case E_EQ_U: CG_BIN(x == y ? 1u : 0u)
+    default: CG_BIN(apply_bin((uint8_t)op, x, y, err))  // E_DIV_U: flags a zero divisor
+  }
+#undef CG_BIN
+}
+
+template <int VEC>
+__device__ __forceinline__ void un_vec(uint32_t op, uint32_t *a) {
+#define CG_UN(EXPR) _Pragma("unroll") for (int j = 0; j < VEC; ++j) { const uint32_t x = a[j * 256]; a[j * 256] = (EXPR); } break;
+  switch (op) {
+    case E_NEG_F: CG_UN(x ^ 0x80000000u)
+    case E_EXP_F: CG_UN(as_u(expf(as_f(x))))
+    case E_RCP_F: CG_UN(as_u(1.0f / as_f(x)))
+    case E_SQRT_F: CG_UN(as_u(sqrt_like_pow(as_f(x))))
+    case E_CUBE_F: CG_UN(as_u(as_f(x) * as_f(x) * as_f(x)))
+    default: CG_UN(apply_un((uint8_t)op, x))
+  }
+#undef CG_UN
+}
+
+// `stk` points at this thread's column of the LDS stack: element j of depth d is stk[(d * VEC + j) * 256]
+template <int VEC>
+__device__ __forceinline__ void eval_program_small(const Program &p, int n_instr, const uint32_t (&idx)[MAX_DIMS],
+                                                   uint32_t c0, uint32_t *err, uint32_t *stk, uint32_t (&res)[VEC]) {
+  for (int pc = 0; pc < n_instr; ++pc) {
+    const uint32_t w = uni<true>(*(const uint32_t *)&p.code[pc]);
+    const uint32_t op = w & 0xFFu, depth = (w >> 8) & 0xFFu, arg = w >> 16;
+    uint32_t *top = stk + depth * VEC * 256;  // where a push lands
+    if (op <= E_ROW1) {
+      uint32_t t[VEC];
+      if (op == E_LOAD) {
+        load_chunks<VEC, 1, true>(p, (int)arg, idx, c0, 0u, 1u, t);
+      } else if (op == E_IOTA) {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) t[j] = c0 + j;
+      } else {  // plain programs have no reduction stages: E_CONST
+        const uint32_t c = uni<true>(p.imm[arg]);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) t[j] = c;
+      }
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) top[j * 256] = t[j];
+    } else if (op <= E_EQ_U) {
+      bin_vec<VEC>(op, top - 2 * VEC * 256, top - VEC * 256, top - 2 * VEC * 256, err);
+    } else {
+      un_vec<VEC>(op, top - VEC * 256);
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) res[j] = stk[j * 256];
+}
+
 // ST: the launch is small (every thread runs the program once).  Walking the program through the
 // kernel-argument segment costs one scalar-cache miss per operand descriptor and code line, one
 // after the other, in memory the host has just written - most of such a launch's duration.  All
@@ -288,6 +361,7 @@ template <int VEC, bool ST>
 __global__ void __launch_bounds__(256) ew_kernel(const Program pk, OutDesc o, uint64_t n_groups,
                                                  uint32_t *err) {
   __shared__ __attribute__((aligned(16))) uint32_t staged[ST ? sizeof(Program) / 4 : 4];
+  __shared__ uint32_t stack[ST ? MAX_STACK * VEC * 256 : 1];
   if (ST) {
     static_assert(sizeof(Program) % 16 == 0, "program copied in 16-byte pieces");
     const uint4 *src = (const uint4 *)&pk;
@@ -308,7 +382,8 @@ __global__ void __launch_bounds__(256) ew_kernel(const Program pk, OutDesc o, ui
     for (int d = 0; d < MAX_DIMS; ++d)
       if (d == n_dims - 1) c0 = idx[d];
     // rank-1 programs (the only ones with E_IOTA) have c0 == lin
-    eval_program<VEC, 1, ST>(p, 0, n_instr, idx, c0, 0u, 1u, 0u, 0u, err, v);
+    if (ST) eval_program_small<VEC>(p, n_instr, idx, c0, err, stack + threadIdx.x, v);
+    else eval_program<VEC, 1, false>(p, 0, n_instr, idx, c0, 0u, 1u, 0u, 0u, err, v);
     int64_t off = 0;
 #pragma unroll
     for (int d = 0; d < MAX_DIMS; ++d)
