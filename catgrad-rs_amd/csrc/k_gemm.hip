@@ -1052,15 +1052,19 @@ hipError_t launch_gemv_multi(const LaunchCtx &lc, const GemvMultiDesc &g) {
 // pair and take a quarter of k each (deep, narrow matrices).
 // GLUEPI (two problems of equal N, no k-split): a wave computes column n of both and stores
 // act(first) * second, i.e. gate_proj, up_proj and the SwiGLU / GeGLU between them in one pass.
-template <typename TB, bool KSPLIT, bool GLUEPI>
+// MR: input rows that share the weights (a decode step of a small batch): MR rows of K floats are
+// staged (rows * K <= GEMV_PRO_MAX_K), every weight vector fetched is used for each of them, and the
+// outputs are the rows of a contiguous [rows, N] matrix.
+template <typename TB, bool KSPLIT, bool GLUEPI, int MR>
 __global__ void __launch_bounds__(256) gemv_pro_kernel(GemvProDesc g) {
   typedef typename WVec<TB>::type VT;
   constexpr int EPL = WVec<TB>::EPL, UNROLL = 4, R = 2;
   __shared__ __attribute__((aligned(16))) float xs[GEMV_PRO_MAX_K];
-  __shared__ float lds[4];
-  __shared__ float part[4][R];
+  __shared__ float lds[4 * MR];
+  __shared__ float part[4][R][MR];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const uint32_t K = g.m.K, bz = blockIdx.z;
+  const uint32_t rows = MR == 1 ? 1u : g.rows;
   const float *ga = g.a + (int64_t)bz * g.a_bstride;
   const float *gaux = g.aux ? g.aux + (int64_t)bz * g.aux_bstride : nullptr;
   // ---- which rows of which matrix
@@ -1108,48 +1112,88 @@ __global__ void __launch_bounds__(256) gemv_pro_kernel(GemvProDesc g) {
   };
   bool requested = slot * CPS < N;
   if (requested) request(slot * CPS, k_begin + lane * EPL);
-  // ---- prologue: the input row
+  // ---- prologue: the input rows
+  float ssq[MR];  // RMSNorm: the rows' sums of squares, reduced together (one exchange through LDS)
   if (g.pro == PRO_RMSNORM) {
-    float ss = 0.f;
-    for (uint32_t k = tid * 4; k < K; k += 1024) {
-      const float4 v = *(const float4 *)(ga + k);
-      ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+#pragma unroll
+    for (int m = 0; m < MR; ++m) {
+      float ss = 0.f;
+      if (MR == 1 || (uint32_t)m < rows)
+        for (uint32_t k = tid * 4; k < K; k += 1024) {
+          const float4 v = *(const float4 *)(ga + (int64_t)m * g.a_rstride + k);
+          ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+        }
+      ssq[m] = wave_sum(ss);
     }
-    ss = block_reduce<256, false>(ss, lds);
-    const float rms = sqrtf(ss / g.n_as_float + g.eps);
-    for (uint32_t k = tid * 4; k < K; k += 1024) {
-      const float4 v = *(const float4 *)(ga + k);
-      float4 o;
-      o.x = v.x / rms; o.y = v.y / rms; o.z = v.z / rms; o.w = v.w / rms;
-      if (gaux) {
-        const float4 gm = *(const float4 *)(gaux + k);
-        o.x *= g.gamma_offset + gm.x; o.y *= g.gamma_offset + gm.y;
-        o.z *= g.gamma_offset + gm.z; o.w *= g.gamma_offset + gm.w;
+    if (lane == 0)
+#pragma unroll
+      for (int m = 0; m < MR; ++m) lds[wave * MR + m] = ssq[m];
+    __syncthreads();
+#pragma unroll
+    for (int m = 0; m < MR; ++m) ssq[m] = (lds[m] + lds[MR + m]) + (lds[2 * MR + m] + lds[3 * MR + m]);
+  }
+#pragma unroll
+  for (int m = 0; m < MR; ++m) {
+    if (MR > 1 && (uint32_t)m >= rows) break;
+    const float *gam = ga + (int64_t)m * g.a_rstride;
+    float *xm = xs + (size_t)m * K;
+    if (g.pro == PRO_RMSNORM) {
+      const float rms = sqrtf(ssq[m] / g.n_as_float + g.eps);
+      for (uint32_t k = tid * 4; k < K; k += 1024) {
+        const float4 v = *(const float4 *)(gam + k);
+        float4 o;
+        o.x = v.x / rms; o.y = v.y / rms; o.z = v.z / rms; o.w = v.w / rms;
+        if (gaux) {  // gamma: one vector for every row
+          const float4 gm = *(const float4 *)(gaux + k);
+          o.x *= g.gamma_offset + gm.x; o.y *= g.gamma_offset + gm.y;
+          o.z *= g.gamma_offset + gm.z; o.w *= g.gamma_offset + gm.w;
+        }
+        *(float4 *)(xm + k) = o;
       }
-      *(float4 *)(xs + k) = o;
-    }
-  } else if (g.pro == PRO_NONE) {
-    for (uint32_t k = tid * 4; k < K; k += 1024) *(float4 *)(xs + k) = *(const float4 *)(ga + k);
-  } else {
-    for (uint32_t k = tid * 4; k < K; k += 1024) {
-      const float4 a = *(const float4 *)(ga + k), u = *(const float4 *)(gaux + k);
-      float4 o;
-      if (g.pro == PRO_GEGLU) {
-        o.x = gelu_ref(a.x) * u.x; o.y = gelu_ref(a.y) * u.y;
-        o.z = gelu_ref(a.z) * u.z; o.w = gelu_ref(a.w) * u.w;
-      } else {
-        o.x = a.x * sigmoid_ref(a.x) * u.x; o.y = a.y * sigmoid_ref(a.y) * u.y;
-        o.z = a.z * sigmoid_ref(a.z) * u.z; o.w = a.w * sigmoid_ref(a.w) * u.w;
+    } else if (g.pro == PRO_NONE) {
+      for (uint32_t k = tid * 4; k < K; k += 1024) *(float4 *)(xm + k) = *(const float4 *)(gam + k);
+    } else {
+      const float *gum = gaux + (int64_t)m * g.aux_rstride;
+      for (uint32_t k = tid * 4; k < K; k += 1024) {
+        const float4 a = *(const float4 *)(gam + k), u = *(const float4 *)(gum + k);
+        float4 o;
+        if (g.pro == PRO_GEGLU) {
+          o.x = gelu_ref(a.x) * u.x; o.y = gelu_ref(a.y) * u.y;
+          o.z = gelu_ref(a.z) * u.z; o.w = gelu_ref(a.w) * u.w;
+        } else {
+          o.x = a.x * sigmoid_ref(a.x) * u.x; o.y = a.y * sigmoid_ref(a.y) * u.y;
+          o.z = a.z * sigmoid_ref(a.z) * u.z; o.w = a.w * sigmoid_ref(a.w) * u.w;
+        }
+        *(float4 *)(xm + k) = o;
       }
-      *(float4 *)(xs + k) = o;
     }
   }
   __syncthreads();
+  // Several rows: a lane meets the same k positions in every column (K <= 64 * EPL * UNROLL, one pass
+  // over k), so its share of the staged rows moves to registers once and the column loop reads no LDS.
+  float xr[MR > 1 ? MR : 1][UNROLL][EPL];
+  if (MR > 1) {
+#pragma unroll
+    for (int m = 0; m < MR; ++m)
+#pragma unroll
+      for (int u = 0; u < UNROLL; ++u) {
+        const uint32_t k = lane * EPL + u * 64 * EPL;
+#pragma unroll
+        for (int j4 = 0; j4 < EPL; j4 += 4) {
+          float4 t = make_float4(0.f, 0.f, 0.f, 0.f);
+          if ((uint32_t)m < rows && k < K) t = *(const float4 *)(xs + (size_t)m * K + k + j4);
+          xr[MR > 1 ? m : 0][u][j4] = t.x; xr[MR > 1 ? m : 0][u][j4 + 1] = t.y;
+          xr[MR > 1 ? m : 0][u][j4 + 2] = t.z; xr[MR > 1 ? m : 0][u][j4 + 3] = t.w;
+        }
+      }
+  }
   // ---- the products
   for (uint32_t nb = slot * CPS; nb < N; nb += n_slots * CPS) {  // uniform per workgroup when KSPLIT
-    float acc[R];
+    float acc[R][MR];
 #pragma unroll
-    for (int r = 0; r < R; ++r) acc[r] = 0.f;
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+      for (int m = 0; m < MR; ++m) acc[r][m] = 0.f;
     for (uint32_t k0 = k_begin + lane * EPL; k0 < k_end; k0 += 64 * EPL * UNROLL) {
       if (!requested) request(nb, k0);
       requested = false;
@@ -1158,10 +1202,12 @@ __global__ void __launch_bounds__(256) gemv_pro_kernel(GemvProDesc g) {
         const uint32_t k = k0 + u * 64 * EPL;
         if (k < k_end) {
           float xv[EPL];
+          if (MR == 1) {
 #pragma unroll
-          for (int j4 = 0; j4 < EPL; j4 += 4) {
-            const float4 t = *(const float4 *)(xs + k + j4);
-            xv[j4] = t.x; xv[j4 + 1] = t.y; xv[j4 + 2] = t.z; xv[j4 + 3] = t.w;
+            for (int j4 = 0; j4 < EPL; j4 += 4) {
+              const float4 t = *(const float4 *)(xs + k + j4);
+              xv[j4] = t.x; xv[j4 + 1] = t.y; xv[j4 + 2] = t.z; xv[j4 + 3] = t.w;
+            }
           }
 #pragma unroll
           for (int r = 0; r < R; ++r) {
@@ -1169,73 +1215,103 @@ __global__ void __launch_bounds__(256) gemv_pro_kernel(GemvProDesc g) {
               float w[EPL];
               WVec<TB>::widen(q[r][u], w);
 #pragma unroll
-              for (int j = 0; j < EPL; ++j) acc[r] += w[j] * xv[j];
+              for (int m = 0; m < MR; ++m)
+#pragma unroll
+                for (int j = 0; j < EPL; ++j) acc[r][m] += w[j] * (MR == 1 ? xv[j] : xr[MR > 1 ? m : 0][u][j]);
             }
           }
         }
       }
     }
 #pragma unroll
-    for (int r = 0; r < R; ++r) acc[r] = wave_sum(acc[r]);
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+      for (int m = 0; m < MR; ++m) acc[r][m] = wave_sum(acc[r][m]);
     if (GLUEPI) {
       if (lane == 0)
-        C[nb] = (g.glu_epilogue == PRO_GEGLU ? gelu_ref(acc[0]) : acc[0] * sigmoid_ref(acc[0])) * acc[1];
+#pragma unroll
+        for (int m = 0; m < MR; ++m)
+          if ((uint32_t)m < rows)
+            C[(uint64_t)m * N + nb] =
+                (g.glu_epilogue == PRO_GEGLU ? gelu_ref(acc[0][m]) : acc[0][m] * sigmoid_ref(acc[0][m])) * acc[1][m];
     } else if (KSPLIT) {
       __syncthreads();
       if (lane == 0)
 #pragma unroll
-        for (int r = 0; r < R; ++r) part[wave][r] = acc[r];
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+          for (int m = 0; m < MR; ++m) part[wave][r][m] = acc[r][m];
       __syncthreads();
-      if (tid < R && nb + tid < N)
-        C[nb + tid] = ((part[0][tid] + part[1][tid]) + (part[2][tid] + part[3][tid])) + (Cadd ? Cadd[nb + tid] : 0.f);
+      if (tid < R * MR) {
+        const int r = tid % R, m = tid / R;
+        if ((uint32_t)m < rows && nb + r < N) {
+          const uint64_t at = (uint64_t)m * N + nb + r;
+          C[at] = ((part[0][r][m] + part[1][r][m]) + (part[2][r][m] + part[3][r][m])) + (Cadd ? Cadd[at] : 0.f);
+        }
+      }
     } else if (lane == 0) {
 #pragma unroll
       for (int r = 0; r < R; ++r)
-        if (nb + r < N) C[nb + r] = acc[r] + (Cadd ? Cadd[nb + r] : 0.f);
+#pragma unroll
+        for (int m = 0; m < MR; ++m)
+          if ((uint32_t)m < rows && nb + r < N) {
+            const uint64_t at = (uint64_t)m * N + nb + r;
+            C[at] = acc[r][m] + (Cadd ? Cadd[at] : 0.f);
+          }
     }
   }
 }
 
-template <typename TB, bool KSPLIT>
+template <typename TB, bool KSPLIT, int MR>
 static void launch_gemv_pro_block(const LaunchCtx &lc, const GemvProDesc &g, uint32_t slots) {
   // `slots` = column pairs per problem; 256-thread workgroups (wider ones stream worse).  Long input
   // rows cost more to recompute, so fewer workgroups each take several column pairs.
   const uint32_t per_wg = KSPLIT ? 1 : 4;
   uint32_t blocks = (slots + per_wg - 1) / per_wg;
   const uint32_t batch = g.batch ? g.batch : 1;
-  const uint32_t cap = (uint32_t)lc.n_cus * (g.m.K >= 4096 ? 2 : 4) / (g.m.n_prob * batch);
+  // (several rows: two workgroups fit a CU and staging the rows costs as much as a pass of columns - one round)
+  const uint32_t cap = (uint32_t)lc.n_cus * (MR > 1 || g.m.K >= 4096 ? 2 : 4) / (g.m.n_prob * batch);
   if (blocks > cap) blocks = cap ? cap : 1;
   dim3 grid(blocks, g.m.n_prob, batch);
-  CG_LAUNCH(lc, (gemv_pro_kernel<TB, KSPLIT, false>), grid, 256, g);
+  CG_LAUNCH(lc, (gemv_pro_kernel<TB, KSPLIT, false, MR>), grid, 256, g);
 }
 
-template <typename TB>
+template <typename TB, int MR>
 static void launch_gemv_pro_glu(const LaunchCtx &lc, const GemvProDesc &g) {
   const uint32_t slots = g.m.p[0].N;  // one (gate, up) column pair per wave pass
   uint32_t blocks = (slots + 3) / 4;
-  const uint32_t cap = (uint32_t)lc.n_cus * 4;
+  const uint32_t cap = (uint32_t)lc.n_cus * (MR > 1 ? 2 : 4);
   if (blocks > cap) blocks = cap;
-  CG_LAUNCH(lc, (gemv_pro_kernel<TB, false, true>), dim3(blocks, 1, 1), 256, g);
+  CG_LAUNCH(lc, (gemv_pro_kernel<TB, false, true, MR>), dim3(blocks, 1, 1), 256, g);
 }
+
+uint32_t gemv_pro_multi_row_max_k(int b_stype) { return 64u * (b_stype == ST_BF16 ? 8u : 4u) * 4u; }
 
 hipError_t launch_gemv_pro(const LaunchCtx &lc, const GemvProDesc &g) {
   uint32_t max_n = 0;
   for (int i = 0; i < g.m.n_prob; ++i) max_n = g.m.p[i].N > max_n ? g.m.p[i].N : max_n;
   if (!max_n || !g.m.n_prob) return hipSuccess;
+  const bool multi = g.rows > 1;  // several input rows share the weights
+  // several rows: one pass over k per column (K <= 64 lanes x 16 bytes x 4 loads)
+  if (multi && (g.rows > 4 || (uint64_t)g.rows * g.m.K > GEMV_PRO_MAX_K || g.batch > 1 || g.b_index ||
+                g.m.K > gemv_pro_multi_row_max_k(g.m.b_stype)))
+    return hipErrorInvalidValue;
   if (g.glu_epilogue) {
     if (g.m.n_prob != 2 || g.m.p[0].N != g.m.p[1].N || g.batch > 1 || g.b_index) return hipErrorInvalidValue;
-    if (g.m.b_stype == ST_BF16) launch_gemv_pro_glu<uint16_t>(lc, g);
-    else launch_gemv_pro_glu<float>(lc, g);
+    if (g.m.b_stype == ST_BF16) multi ? launch_gemv_pro_glu<uint16_t, 4>(lc, g) : launch_gemv_pro_glu<uint16_t, 1>(lc, g);
+    else multi ? launch_gemv_pro_glu<float, 4>(lc, g) : launch_gemv_pro_glu<float, 1>(lc, g);
     return hipGetLastError();
   }
   const uint32_t slots = (max_n + 1) / 2;
   const bool ksplit = g.m.K >= 4096 && slots * (uint32_t)g.m.n_prob <= (uint32_t)lc.n_cus * 8;
   if (g.m.b_stype == ST_BF16) {
-    if (ksplit) launch_gemv_pro_block<uint16_t, true>(lc, g, slots);
-    else launch_gemv_pro_block<uint16_t, false>(lc, g, slots);
+    if (multi) launch_gemv_pro_block<uint16_t, false, 4>(lc, g, slots);  // rows * K <= 8192: K < 4096
+    else if (ksplit) launch_gemv_pro_block<uint16_t, true, 1>(lc, g, slots);
+    else launch_gemv_pro_block<uint16_t, false, 1>(lc, g, slots);
   } else {
-    if (ksplit) launch_gemv_pro_block<float, true>(lc, g, slots);
-    else launch_gemv_pro_block<float, false>(lc, g, slots);
+    if (multi) launch_gemv_pro_block<float, false, 4>(lc, g, slots);
+    else if (ksplit) launch_gemv_pro_block<float, true, 1>(lc, g, slots);
+    else launch_gemv_pro_block<float, false, 1>(lc, g, slots);
   }
   return hipGetLastError();
 }

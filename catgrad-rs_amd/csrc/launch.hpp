@@ -274,12 +274,19 @@ struct GemvProDesc {
   int32_t glu_epilogue;
   uint32_t batch;   // 0 or 1: a single row
   int64_t a_bstride, aux_bstride;
+  // 0 / 1, or up to 4 input rows that share the weights (rows * K <= GEMV_PRO_MAX_K, no batch, no b_index):
+  // row r of the input is a + r * a_rstride (aux + r * aux_rstride; gamma is one vector for all rows) and
+  // the outputs (and c_add) are the rows of contiguous [rows, N] matrices
+  uint32_t rows;
+  int64_t a_rstride, aux_rstride;
   const uint32_t *b_index;
   int64_t b_index_stride, sb_index;
   uint32_t b_index_limit;
   uint32_t *err;
 };
 hipError_t launch_gemv_pro(const LaunchCtx &lc, const GemvProDesc &g);
+// largest K the several-row form takes for weights of this storage type
+uint32_t gemv_pro_multi_row_max_k(int b_stype);
 // The routed experts of a MoE layer over many tokens (a prefill; models/qwen3.rs:104-123), expert by
 // expert.  A slot is one of the k choices of every token: its index vector, its input rows and its
 // outputs.  A problem is one stacked weight tensor [E, N, K] (bf16): gate_proj and up_proj share

@@ -1329,11 +1329,17 @@ static bool same_rows(const cg_tensor *a, const cg_tensor *b) {
          std::equal(a->shape, a->shape + a->rank, b->shape);
 }
 
+int try_gate_up_glu(cg_backend *be, cg_tensor *glu, cg_tensor *g, cg_tensor *u, int gelu, bool *done);
+
 int try_glu(cg_backend *be, cg_tensor *root, bool *done) {
   cg_tensor *gate = nullptr, *up = nullptr;
   int gelu = 0;
   if (!match_glu(root, &gate, &up, &gelu)) return CG_OK;
   cg_tensor *gc = nullptr, *uc = nullptr;
+  if (!(be->flags & CG_FLAG_NO_PATTERNS)) {  // a few rows: both products and the activation in one launch
+    TRY(try_gate_up_glu(be, root, gate, up, gelu, done));
+    if (*done) return CG_OK;
+  }
   // bf16 mode, many rows, gate and up both still deferred products of the same rows: one GEMM over the
   // two weight matrices stacked tile by tile, the activation applied where both products sit in
   // registers; the gate product never exists as a tensor.
@@ -1423,6 +1429,9 @@ int try_gemv_add(cg_backend *be, cg_tensor *root, bool *done) {
   if (root->dtype != CG_F32 || !is_bin(root, E_ADD_F)) return CG_OK;
   for (int side = 0; side < 2; ++side) {
     cg_tensor *mm = root->in[side], *other = root->in[1 - side];
+    // a batch-folding linear hands its product back through a reshape: the same rows in the same order
+    const bool folded = mm->op == N_RESHAPE && refs(mm) == 1 && mm->in[0]->op == N_MATMUL && mm->in[0]->size() == mm->size();
+    if (folded) mm = mm->in[0];
     // one-row products add in their epilogue; so does the pass that sums the k-slices of a split GEMM
     if (mm->op != N_MATMUL || refs(mm) != 1 || mm->dtype != CG_F32) continue;
     if (!mm->gemv_candidate && mm->rank > 3) continue;  // attention products have fusions of their own
@@ -1437,7 +1446,8 @@ int try_gemv_add(cg_backend *be, cg_tensor *root, bool *done) {
     root->st->rc.fetch_add(1);
     root->stype = mm->stype;
     root->offset = mm->offset;
-    std::copy(mm->strides, mm->strides + mm->rank, root->strides);
+    if (folded) contiguous_strides(root->rank, root->shape, root->strides);  // products are dense
+    else std::copy(mm->strides, mm->strides + mm->rank, root->strides);
     finish_fused(root);
     *done = true;
     return CG_OK;
@@ -2196,22 +2206,41 @@ int try_attn_decode(cg_backend *be, cg_tensor *n, bool *done) {
   return CG_OK;
 }
 
+// A batch-folding linear reshapes its input ([B, 1, K] -> [1, B, K]) and its product back; such a
+// reshape only regroups rows.  The node under a reshape that nobody else holds and that keeps the
+// last axis, else the node itself.
+static cg_tensor *rows_base(cg_tensor *t) {
+  if (t->op == N_RESHAPE && refs(t) == 1 && t->rank >= 1 && t->in[0]->rank >= 1 &&
+      t->in[0]->shape[t->in[0]->rank - 1] == t->shape[t->rank - 1])
+    return t->in[0];
+  return t;
+}
+
 // h = act(gate_proj(x)) * up_proj(x) with one input row (models/llama.rs:11-35): both products and the
 // activation in one launch, a wave computing column n of gate and of up (and x itself from its
 // RMSNorm when nothing else reads the normed row).  `glu` is the deferred act(g) * u node; on
 // success it becomes a realised tensor and g, u are never materialised.
 int try_gate_up_glu(cg_backend *be, cg_tensor *glu, cg_tensor *g, cg_tensor *u, int gelu, bool *done) {
+  // the activation reads the gate two (three) times, the product once; either may sit under a reshape
+  if (refs(g) != (gelu ? 3 : 2) || refs(u) != 1) return CG_OK;
+  if (g->op == N_RESHAPE && refs(g->in[0]) == 1 && g->in[0]->size() == g->size()) g = g->in[0];
+  u = rows_base(u);
   if (g->op != N_MATMUL || u->op != N_MATMUL || !g->gemv_candidate || !u->gemv_candidate) return CG_OK;
-  if (refs(g) != (gelu ? 3 : 2) || refs(u) != 1 || g->in[0] != u->in[0] || g->size() != u->size()) return CG_OK;
-  cg_tensor *X = g->in[0];
+  if (refs(u) != 1 || rows_base(g->in[0]) != rows_base(u->in[0]) || g->size() != u->size()) return CG_OK;
+  cg_tensor *X = rows_base(g->in[0]);
   const int64_t K = X->shape[X->rank - 1], N = g->shape[g->rank - 1];
-  if (X->size() != K || g->size() != N || K % 8 || K < 256 || K > GEMV_PRO_MAX_K || glu->size() != N) return CG_OK;
+  // one row, or the few rows of a small batch: [B, 1, K] against weights repeated over the batch
+  const int64_t rows = K > 0 ? X->size() / K : 0;
+  if (rows < 1 || rows > 4 || X->size() != rows * K || rows * K > GEMV_PRO_MAX_K || g->size() != rows * N || K % 8 || K < 256 ||
+      glu->size() != rows * N)
+    return CG_OK;
   cg_tensor *ws[2] = {g->in[1], u->in[1]};
   for (cg_tensor *w : ws) {
     TRY(realize(be, w));
+    if (rows > 1 && K > (int64_t)gemv_pro_multi_row_max_k(w->stype)) return CG_OK;
     if (w->rank < 2 || w->shape[w->rank - 2] != K || w->strides[w->rank - 2] != 1) return CG_OK;
     for (int i = 0; i + 2 < w->rank; ++i)
-      if (w->shape[i] != 1) return CG_OK;
+      if (w->shape[i] != 1 && w->strides[i] != 0) return CG_OK;
     if ((w->stype != ST_F32 && w->stype != ST_BF16) || w->stype != ws[0]->stype) return CG_OK;
     if ((uintptr_t)data_ptr(w) % 16 || w->strides[w->rank - 1] % (16 / esize(w->stype))) return CG_OK;
   }
@@ -2245,6 +2274,8 @@ int try_gate_up_glu(cg_backend *be, cg_tensor *glu, cg_tensor *g, cg_tensor *u, 
     d.a = (const float *)data_ptr(a0);
     d.aux = a1 ? (const float *)data_ptr(a1) : nullptr;
     d.glu_epilogue = gelu ? PRO_GEGLU : PRO_SWIGLU;
+    d.rows = (uint32_t)rows;
+    d.a_rstride = d.aux_rstride = K;
     d.m.K = (uint32_t)K;
     d.m.b_stype = ws[0]->stype;
     d.m.n_prob = 2;
@@ -2255,11 +2286,11 @@ int try_gate_up_glu(cg_backend *be, cg_tensor *glu, cg_tensor *g, cg_tensor *u, 
       d.m.p[i].N = (uint32_t)N;
     }
     const char *base = ws[0]->stype == ST_BF16 ? "gemv_rowdot_bf16" : "gemv_rowdot_f32";
-    KernelScope ks(be, base, 2.0 * N * K * esize(ws[0]->stype) + (double)K * 8 + (double)N * 4, 4.0 * N * K);
+    KernelScope ks(be, base, 2.0 * N * K * esize(ws[0]->stype) + (double)rows * (K * 8 + N * 4), 4.0 * rows * N * K);
     if (be->trace_shapes) {
       char buf[96];
-      snprintf(buf, sizeof buf, "%s[%sgate*up,K%lld,N%lld]", base, d.pro == PRO_RMSNORM ? "rmsnorm+" : "", (long long)K,
-               (long long)(2 * N));
+      snprintf(buf, sizeof buf, "%s[%sgate*up,M%lld,K%lld,N%lld]", base, d.pro == PRO_RMSNORM ? "rmsnorm+" : "", (long long)rows,
+               (long long)K, (long long)(2 * N));
       ks.rename(buf);
     }
     hipError_t e = launch_gemv_pro(be->lc(), d);
@@ -2277,10 +2308,11 @@ int try_gate_up_glu(cg_backend *be, cg_tensor *glu, cg_tensor *g, cg_tensor *u, 
 // or a SwiGLU/GeGLU of earlier values.  When every consumer of that row is such a product, the
 // row is computed inside the product kernel (launch_gemv_pro) and its node is never realised.
 int try_gemv_prologue(cg_backend *be, cg_tensor *n, cg_tensor *addend, bool *added, bool *done) {
-  cg_tensor *A = n->in[0];
+  cg_tensor *A = rows_base(n->in[0]);
   if (A->op == N_REAL || A->dtype != CG_F32 || !n->gemv_candidate || A->rank < 1) return CG_OK;
   const int64_t K = A->shape[A->rank - 1];
-  if (A->size() != K || K % 8 || K < 256 || K > GEMV_PRO_MAX_K) return CG_OK;
+  const int64_t rows = K > 0 ? A->size() / K : 0;  // one row, or the few rows of a small batch
+  if (rows < 1 || rows > 4 || A->size() != rows * K || K % 8 || K < 256 || rows * K > GEMV_PRO_MAX_K) return CG_OK;
   RmsNormMatch rm;
   cg_tensor *gate = nullptr, *up = nullptr;
   int gelu = 0, pro = 0;
@@ -2297,20 +2329,21 @@ int try_gemv_prologue(cg_backend *be, cg_tensor *n, cg_tensor *addend, bool *add
   // the group: every deferred one-row product reading A (n first)
   std::vector<cg_tensor *> members{n};
   for (cg_tensor *c : be->gemv_candidates)
-    if (c != n && c->op == N_MATMUL && c->in[0] == A) members.push_back(c);
+    if (c != n && c->op == N_MATMUL && rows_base(c->in[0]) == A) members.push_back(c);
   if ((int)members.size() != refs(A) || members.size() > 4) return CG_OK;
   GemvProDesc d;
   std::memset(&d, 0, sizeof(d));
   int b_stype = -1;
   for (cg_tensor *c : members) {
     cg_tensor *w = c->in[1];
-    if (c->rank != A->rank || c->size() != c->shape[c->rank - 1]) return CG_OK;
+    if (c->size() != rows * c->shape[c->rank - 1]) return CG_OK;
     TRY(realize(be, w));
     if (w->rank < 2 || w->shape[w->rank - 2] != K || w->strides[w->rank - 2] != 1) return CG_OK;
     for (int i = 0; i + 2 < w->rank; ++i)
-      if (w->shape[i] != 1) return CG_OK;
+      if (w->shape[i] != 1 && w->strides[i] != 0) return CG_OK;
     if (w->stype != ST_F32 && w->stype != ST_BF16) return CG_OK;
     if (b_stype >= 0 && w->stype != b_stype) return CG_OK;
+    if (rows > 1 && K > (int64_t)gemv_pro_multi_row_max_k(w->stype)) return CG_OK;
     b_stype = w->stype;
     if ((uintptr_t)data_ptr(w) % 16 || w->strides[w->rank - 1] % (16 / esize(w->stype))) return CG_OK;
   }
@@ -2345,9 +2378,11 @@ int try_gemv_prologue(cg_backend *be, cg_tensor *n, cg_tensor *addend, bool *add
   d.n_as_float = rm.n_as_float;
   d.eps = rm.eps;
   d.gamma_offset = rm.gamma_offset;
+  d.rows = (uint32_t)rows;
+  d.a_rstride = d.aux_rstride = K;
   d.m.K = (uint32_t)K;
   d.m.b_stype = b_stype;
-  double bytes = (double)K * 8, flops = 0;
+  double bytes = (double)rows * K * 8, flops = 0;
   int st = CG_OK;
   for (cg_tensor *c : members) {
     cg_tensor *w = c->in[1];
@@ -2359,16 +2394,16 @@ int try_gemv_prologue(cg_backend *be, cg_tensor *n, cg_tensor *addend, bool *add
     pr.c_add = (c == n && addend) ? (const float *)data_ptr(addend) : nullptr;
     pr.sbn = w->strides[w->rank - 1];
     pr.N = (uint32_t)w->shape[w->rank - 1];
-    bytes += (double)pr.N * K * esize(w->stype) + (double)pr.N * 4;
-    flops += 2.0 * pr.N * K;
+    bytes += (double)pr.N * K * esize(w->stype) + (double)rows * pr.N * 4;
+    flops += 2.0 * rows * pr.N * K;
   }
   if (!st) {
     const char *base = b_stype == ST_BF16 ? "gemv_rowdot_bf16" : "gemv_rowdot_f32";
     KernelScope ks(be, base, bytes, flops);
     if (be->trace_shapes) {
       char buf[96];
-      snprintf(buf, sizeof buf, "%s[%s%d,K%lld,N%.0f]", base, pro == PRO_RMSNORM ? "rmsnorm+multi" : "glu+multi",
-               d.m.n_prob, (long long)K, flops / (2.0 * K));
+      snprintf(buf, sizeof buf, "%s[%s%d,M%lld,K%lld,N%.0f]", base, pro == PRO_RMSNORM ? "rmsnorm+multi" : "glu+multi",
+               d.m.n_prob, (long long)rows, (long long)K, flops / (2.0 * rows * K));
       ks.rename(buf);
     }
     hipError_t e = launch_gemv_pro(be->lc(), d);
@@ -3910,7 +3945,9 @@ int cg_matmul(cg_backend *be, cg_tensor *a, cg_tensor *b, cg_tensor **out) {
   n->op = N_MATMUL;
   n->in[0] = retain(a);
   n->in[1] = retain(b);
-  if (a->dtype == CG_F32 && shape[a->rank - 2] == 1 && !(be->flags & CG_FLAG_EAGER)) {
+  // one input row per batch, or the rows of a small batch folded into one matrix ([1, B, K])
+  const bool few_rows = shape[a->rank - 2] == 1 || (a->rank == 3 && shape[0] == 1 && shape[1] <= 4);
+  if (a->dtype == CG_F32 && few_rows && !(be->flags & CG_FLAG_EAGER)) {
     if (be->gemv_candidates.size() >= 4096) forget_gemv_candidate(be->gemv_candidates.front());
     be->gemv_candidates.push_back(n);
     n->gemv_candidate = true;
