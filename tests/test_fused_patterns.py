@@ -351,6 +351,59 @@ def test_glu_in_projection_prologue(oracle, hip, hip_nopat, K, N, act):
     assert np.allclose(gen, ref, rtol=1e-4, atol=1e-5)
 
 
+def _folded_linear(b, i, o, name, x):
+    """A linear over [B, 1, K] the way a batch-correct model writes it: the batch folded into the rows
+    of one matrix for the product and unfolded again (catgrad-llm/src/legacy/nn/layers.rs:435-456)."""
+    bb, ss, hh = lang.unpack(b, 3, lang.shape(b, x))
+    y = nn.linear_no_bias(b, i, o, lang.path([name]), lang.reshape(b, lang.make_shape(b, 1, bb * ss, hh), x))
+    return lang.reshape(b, lang.make_shape(b, bb, ss, o), y)
+
+
+@pytest.mark.parametrize("rows", [2, 3, 4])
+@pytest.mark.parametrize("act", ["silu", "gelu"])
+def test_decoder_block_of_a_small_batch(oracle, hip, hip_bf16, hip_nopat, rows, act):
+    """One decode step of `rows` sequences through the projections of a decoder layer, each linear
+    folding the batch itself: RMSNorm inside the grouped q/k/v launch, the residual in o_proj's
+    epilogue, gate_proj, up_proj and the activation as one launch - five launches where the rows taken
+    one product at a time need eleven - and the same values as the oracle."""
+    K, F = 512, 1024
+    g = np.random.default_rng(rows * 10 + len(act))
+    x = (g.standard_normal((rows, 1, K)) * 2).astype(np.float32)
+    p = {"n1.weight": g.standard_normal(K).astype(np.float32), "n2.weight": g.standard_normal(K).astype(np.float32)}
+    for name, (o, i) in {"q": (K, K), "k": (128, K), "v": (128, K), "o": (K, K), "g": (F, K), "u": (F, K), "d": (K, F)}.items():
+        p[name + ".weight"] = (g.standard_normal((o, i)) * 0.05).astype(np.float32)
+
+    def f(b, xv):
+        xv = xv + xv - xv
+        h = helpers.rmsnorm(b, 1e-5, lang.path(["n1"]), xv)
+        q, k, v = (_folded_linear(b, K, o, nm, h) for nm, o in (("q", K), ("k", 128), ("v", 128)))
+        xv = xv + _folded_linear(b, K, K, "o", q)        # (attention itself is not part of this test)
+        h = helpers.rmsnorm(b, 1e-5, lang.path(["n2"]), xv)
+        gt, up = _folded_linear(b, K, F, "g", h), _folded_linear(b, K, F, "u", h)
+        m = (nn.silu(b, gt) if act == "silu" else nn.gelu(b, gt)) * up
+        return xv + _folded_linear(b, F, K, "d", m), k, v
+    ref = vectors.run(oracle, f, 3, x, params=p)
+    got, names = run_traced(hip, f, 3, x, params=p)
+    gen = vectors.run(hip_nopat, f, 3, x, params=p)
+    assert not ({"rmsnorm_fused", "swiglu_fused", "geglu_fused", "binary_f32"} & names), sorted(names)
+    hip.trace(True)
+    hip.trace_reset()
+    vectors.run(hip, f, 3, x, params=p)
+    rep = hip.trace_report()
+    hip.trace(False)
+    # x + x - x, then q/k/v, o_proj, gate/up, down_proj
+    assert rep["gemv_rowdot_f32"]["launches"] == 4 and sum(v["launches"] for v in rep.values()) == 5, {k: v["launches"] for k, v in rep.items()}
+    for r, a, c in zip(ref, got, gen):
+        assert a.shape == r.shape and np.allclose(a, r, rtol=1e-4, atol=1e-4), np.abs(a - r).max()
+        assert np.allclose(c, r, rtol=1e-4, atol=1e-4)
+    p16 = {k: (vectors.bf16_round(v) if v.ndim >= 2 else v) for k, v in p.items()}
+    ref16 = vectors.run(oracle, f, 3, x, params=p16)
+    got16, names16 = run_traced(hip_bf16, f, 3, x, params=p)
+    assert not ({"rmsnorm_fused", "swiglu_fused", "geglu_fused", "binary_f32"} & names16), sorted(names16)
+    for r, a in zip(ref16, got16):
+        assert np.max(np.abs(a - r)) <= 2e-2 * np.abs(r).max()
+
+
 @pytest.mark.parametrize("order", ["res_first", "norm_first"])
 @pytest.mark.parametrize("shape", [(2, 33, 1152), (1, 7, 64)])
 def test_rmsnorm_plus_residual(oracle, hip, hip_nopat, shape, order):
