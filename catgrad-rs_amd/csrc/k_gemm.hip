@@ -1065,15 +1065,19 @@ __global__ void __launch_bounds__(256) gemv_pro_kernel(GemvProDesc g) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const uint32_t K = g.m.K, bz = blockIdx.z;
   const uint32_t rows = MR == 1 ? 1u : g.rows;
-  const float *ga = g.a + (int64_t)bz * g.a_bstride;
-  const float *gaux = g.aux ? g.aux + (int64_t)bz * g.aux_bstride : nullptr;
+  // batch entry -> (slot, token) when several MoE slots share the launch
+  const uint32_t tz = g.slot_tokens ? bz % g.slot_tokens : bz, sz = g.slot_tokens ? bz / g.slot_tokens : 0u;
+  const uint32_t az = g.a_by_token ? tz : bz;
+  const float *ga = g.a + (int64_t)az * g.a_bstride;
+  const float *gaux = g.aux ? g.aux + (int64_t)az * g.aux_bstride : nullptr;
   // ---- which rows of which matrix
   const uint32_t N = g.m.p[blockIdx.y].N;
   const TB *B = (const TB *)g.m.p[blockIdx.y].b;
   const TB *B2 = GLUEPI ? (const TB *)g.m.p[1].b : nullptr;
   const int64_t sbn2 = GLUEPI ? g.m.p[1].sbn : 0;
-  if (g.b_index) {
-    uint32_t ix = g.b_index[(int64_t)bz * g.b_index_stride];
+  if (g.b_index || g.slot_tokens) {
+    const uint32_t *bi = g.slot_tokens ? g.b_index_slot[sz] : g.b_index;
+    uint32_t ix = bi[(int64_t)tz * g.b_index_stride];
     if (ix >= g.b_index_limit) {  // the reference's select() panics; flag it and stay in bounds
       atomicOr(g.err, ERRF_INDEX_OOB);
       ix = g.b_index_limit - 1;
@@ -1293,11 +1297,11 @@ hipError_t launch_gemv_pro(const LaunchCtx &lc, const GemvProDesc &g) {
   if (!max_n || !g.m.n_prob) return hipSuccess;
   const bool multi = g.rows > 1;  // several input rows share the weights
   // several rows: one pass over k per column (K <= 64 lanes x 16 bytes x 4 loads)
-  if (multi && (g.rows > 4 || (uint64_t)g.rows * g.m.K > GEMV_PRO_MAX_K || g.batch > 1 || g.b_index ||
+  if (multi && (g.rows > 4 || (uint64_t)g.rows * g.m.K > GEMV_PRO_MAX_K || g.batch > 1 || g.b_index || g.slot_tokens ||
                 g.m.K > gemv_pro_multi_row_max_k(g.m.b_stype)))
     return hipErrorInvalidValue;
   if (g.glu_epilogue) {
-    if (g.m.n_prob != 2 || g.m.p[0].N != g.m.p[1].N || g.batch > 1 || g.b_index) return hipErrorInvalidValue;
+    if (g.m.n_prob != 2 || g.m.p[0].N != g.m.p[1].N || g.batch > 1 || g.b_index || g.slot_tokens) return hipErrorInvalidValue;
     if (g.m.b_stype == ST_BF16) multi ? launch_gemv_pro_glu<uint16_t, 4>(lc, g) : launch_gemv_pro_glu<uint16_t, 1>(lc, g);
     else multi ? launch_gemv_pro_glu<float, 4>(lc, g) : launch_gemv_pro_glu<float, 1>(lc, g);
     return hipGetLastError();

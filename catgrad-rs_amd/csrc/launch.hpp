@@ -283,6 +283,13 @@ struct GemvProDesc {
   int64_t b_index_stride, sb_index;
   uint32_t b_index_limit;
   uint32_t *err;
+  // Several slots of a MoE layer in one batched launch (slot_tokens > 0): batch z is token z % slot_tokens
+  // of slot z / slot_tokens and reads expert b_index_slot[slot][token * b_index_stride] (b_index is unused);
+  // outputs and - unless a_by_token - inputs are laid out [slot][token]; with a_by_token every slot reads
+  // the same input rows a + token * a_bstride
+  uint32_t slot_tokens;
+  int32_t a_by_token;
+  const uint32_t *b_index_slot[8];
 };
 hipError_t launch_gemv_pro(const LaunchCtx &lc, const GemvProDesc &g);
 // largest K the several-row form takes for weights of this storage type

@@ -2747,9 +2747,185 @@ int try_moe_gemm(cg_backend *be, cg_tensor *n, bool *done) {
   return CG_OK;
 }
 
+// A decode step's routed experts, all k slots of the layer in one batched launch per stage instead of
+// one per slot: gate_proj and up_proj of every (slot, token) pair, then down_proj of every pair with
+// the gated activation in its prologue.  The products of a stage share one storage laid out
+// [slot][token][N] (each product tensor is a view of its slot's part), which is what lets the second
+// stage address its inputs by pair.  Anything that does not fit leaves the slot-by-slot path below.
+int try_moe_gemv_slots(cg_backend *be, cg_tensor *n, bool *done) {
+  const int64_t S = n->shape[0];
+  ExpertOperand eo;
+  if (!match_expert_operand(n->in[1], S, &eo)) return CG_OK;
+  cg_tensor *A = n->in[0];
+  const int64_t K = A->shape[2];
+  if (A->rank != 3 || A->shape[0] != S || A->shape[1] != 1 || K % 8 || K < 64 || K > GEMV_PRO_MAX_K || S > 4096) return CG_OK;
+  cg_tensor *gate = nullptr, *up = nullptr;
+  int gelu = 0;
+  const bool glu = A->op != N_REAL && refs(A) == 1 && match_glu(A, &gate, &up, &gelu);
+  if (glu) {  // the first stage (this function again, for gate's product) puts every slot's rows in place
+    TRY(realize(be, gate));
+    TRY(realize(be, up));
+    if (n->op != N_MATMUL) return CG_OK;
+  }
+  struct Member {
+    cg_tensor *c, *idx;
+    int slot, prob;
+  };
+  std::vector<Member> members;
+  std::vector<cg_tensor *> slot_idx, prob_w;
+  auto find_or_add = [](std::vector<cg_tensor *> &v, cg_tensor *t) {
+    for (size_t i = 0; i < v.size(); ++i)
+      if (v[i] == t) return (int)i;
+    v.push_back(t);
+    return (int)v.size() - 1;
+  };
+  std::vector<cg_tensor *> cands{n};
+  for (cg_tensor *c : be->gemv_candidates)
+    if (c != n) cands.push_back(c);
+  Storage *gs = nullptr, *us = nullptr;  // second stage: the storages every slot's gate / up rows live in
+  for (cg_tensor *c : cands) {
+    if (c->op != N_MATMUL || c->rank != 3 || c->shape[0] != S || c->shape[1] != 1 || c->in[0]->rank != 3 || c->in[0]->shape[2] != K)
+      continue;
+    ExpertOperand co;
+    if (!match_expert_operand(c->in[1], S, &co)) continue;
+    if (!glu) {
+      if (c->in[0] != A) continue;
+      bool known_w = false, known_i = false;
+      for (cg_tensor *w : prob_w) known_w = known_w || w == co.w;
+      for (cg_tensor *i : slot_idx) known_i = known_i || i == co.idx;
+      if ((!known_w && prob_w.size() >= 2) || (!known_i && slot_idx.size() >= 8)) continue;
+      members.push_back(Member{c, co.idx, find_or_add(slot_idx, co.idx), find_or_add(prob_w, co.w)});
+    } else {
+      cg_tensor *g2 = nullptr, *u2 = nullptr;
+      int ge2 = 0;
+      if (co.w != eo.w || c->in[0]->op == N_REAL || refs(c->in[0]) != 1 || !match_glu(c->in[0], &g2, &u2, &ge2) || ge2 != gelu) continue;
+      // rows written by the first stage: dense views of two shared storages, the same slot in both
+      if (g2->op != N_REAL || u2->op != N_REAL || g2->stype != ST_F32 || u2->stype != ST_F32 || !is_contiguous(g2) ||
+          !is_contiguous(u2) || g2->offset != u2->offset || g2->offset % (S * K))
+        continue;
+      if (!gs) gs = g2->st, us = u2->st;
+      if (g2->st != gs || u2->st != us || gs == us) continue;
+      const int slot = (int)(g2->offset / (S * K));
+      if (slot >= 8 || members.size() >= 8) continue;
+      members.push_back(Member{c, co.idx, slot, 0});
+      if (prob_w.empty()) prob_w.push_back(co.w);
+    }
+  }
+  const size_t n_slot = glu ? members.size() : slot_idx.size();
+  if (n_slot < 2 || members.size() != n_slot * prob_w.size()) return CG_OK;
+  {
+    std::vector<int> seen(n_slot * prob_w.size(), 0);
+    for (const Member &m : members)
+      if (m.slot >= (int)n_slot || seen[m.slot * prob_w.size() + m.prob]++) return CG_OK;
+  }
+  if (glu && ((size_t)gs->bytes < n_slot * S * K * 4 || (size_t)us->bytes < n_slot * S * K * 4)) return CG_OK;
+  bool has_n = false;
+  for (const Member &m : members) has_n = has_n || m.c == n;
+  if (!has_n) return CG_OK;
+  GemvProDesc d;
+  std::memset(&d, 0, sizeof(d));
+  // indices: u32, one stride between consecutive tokens, the same stride in every slot
+  int64_t istride0 = -1;
+  for (const Member &m : members) {
+    cg_tensor *idx = m.idx;
+    TRY(realize(be, idx));
+    if (idx->dtype != CG_U32) return CG_OK;
+    int64_t istride = 1, expect = -1;
+    for (int i = idx->rank - 1; i >= 0; --i) {
+      if (idx->shape[i] == 1) continue;
+      if (expect < 0) istride = idx->strides[i];
+      else if (idx->strides[i] != expect) return CG_OK;
+      expect = idx->strides[i] * idx->shape[i];
+    }
+    if (istride0 >= 0 && istride != istride0) return CG_OK;
+    istride0 = istride;
+    d.b_index_slot[m.slot] = (const uint32_t *)data_ptr(idx);
+  }
+  int b_stype = -1;
+  for (cg_tensor *w : prob_w) {
+    TRY(realize(be, w));
+    if (w->rank != 3 || w->shape[2] != K || w->strides[2] != 1 || (w->stype != ST_F32 && w->stype != ST_BF16)) return CG_OK;
+    if (b_stype >= 0 && (w->stype != b_stype || w->shape[0] != prob_w[0]->shape[0] || w->strides[0] != prob_w[0]->strides[0]))
+      return CG_OK;
+    b_stype = w->stype;
+    const int q = 16 / esize(w->stype);
+    if ((uintptr_t)data_ptr(w) % 16 || w->strides[1] % q || w->strides[0] % q) return CG_OK;
+  }
+  if (!glu) {
+    TRY(realize(be, A));
+    if (A->stype != ST_F32 || A->strides[2] != 1 || A->strides[0] % 4 || (uintptr_t)data_ptr(A) % 16) return CG_OK;
+    d.pro = PRO_NONE;
+    d.a = (const float *)data_ptr(A);
+    d.a_bstride = A->strides[0];
+    d.a_by_token = 1;
+  } else {
+    if ((uintptr_t)gs->ptr % 16 || (uintptr_t)us->ptr % 16) return CG_OK;
+    d.pro = gelu ? PRO_GEGLU : PRO_SWIGLU;
+    d.a = (const float *)gs->ptr;
+    d.aux = (const float *)us->ptr;
+    d.a_bstride = d.aux_bstride = K;
+  }
+  d.batch = (uint32_t)(n_slot * S);
+  d.slot_tokens = (uint32_t)S;
+  d.b_index_stride = istride0;
+  d.sb_index = prob_w[0]->strides[0];
+  d.b_index_limit = (uint32_t)prob_w[0]->shape[0];
+  d.err = be->d_words;
+  d.m.K = (uint32_t)K;
+  d.m.b_stype = b_stype;
+  // one storage per problem, [slot][token][N]
+  std::vector<Storage *> outs(prob_w.size(), nullptr);
+  auto drop_outs = [&]() {
+    for (Storage *o : outs) storage_release(o);
+  };
+  double bytes = (double)(glu ? 2 * n_slot : 1) * S * K * 4, flops = 0;
+  for (size_t p2 = 0; p2 < prob_w.size(); ++p2) {
+    cg_tensor *w = prob_w[p2];
+    const int64_t N = w->shape[1];
+    int st = dev_alloc(be, (size_t)n_slot * S * N * 4, &outs[p2]);
+    if (st) {
+      drop_outs();
+      return st;
+    }
+    auto &pr = d.m.p[d.m.n_prob++];
+    pr.b = data_ptr(w);
+    pr.c = (float *)outs[p2]->ptr;
+    pr.sbn = w->strides[1];
+    pr.N = (uint32_t)N;
+    bytes += (double)n_slot * S * N * (K * esize(w->stype) + 4);
+    flops += 2.0 * n_slot * S * N * K;
+  }
+  hipError_t e;
+  {
+    KernelScope ks(be, b_stype == ST_BF16 ? "gemv_experts_bf16" : "gemv_experts_f32", bytes, flops);
+    e = launch_gemv_pro(be->lc(), d);
+  }
+  if (e != hipSuccess) {
+    drop_outs();
+    return fail(be, CG_ERR_DEVICE, hipGetErrorString(e));
+  }
+  for (const Member &m : members) {
+    cg_tensor *c = m.c;
+    const int64_t N = prob_w[m.prob]->shape[1];
+    c->st = outs[m.prob];
+    c->st->rc.fetch_add(1);
+    c->stype = ST_F32;
+    c->offset = (int64_t)m.slot * S * N;
+    contiguous_strides(c->rank, c->shape, c->strides);
+    forget_gemv_candidate(c);
+    c->op = N_REAL;
+    drop_inputs(c);
+  }
+  drop_outs();
+  *done = true;
+  return CG_OK;
+}
+
 int try_moe_gemv(cg_backend *be, cg_tensor *n, bool *done) {
   if (n->rank != 3 || n->shape[1] != 1 || !n->gemv_candidate || n->size() == 0) return CG_OK;
   TRY(try_moe_gemm(be, n, done));
+  if (*done) return CG_OK;
+  TRY(try_moe_gemv_slots(be, n, done));
   if (*done) return CG_OK;
   const int64_t S = n->shape[0];
   ExpertOperand eo;

@@ -242,6 +242,56 @@ def test_expert_slots_over_many_tokens(oracle, hip_bf16):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("dev_name", ["hip", "hip_bf16"])
+@pytest.mark.parametrize("S,k", [(4, 4), (1, 2), (7, 3)])
+def test_expert_slots_of_a_decode_step(request, oracle, dev_name, S, k):
+    """The routed half of the MoE block for the few tokens of a decode step: all k slots share one
+    batched launch for gate and up and one for down_proj (with the SwiGLU in its prologue), every
+    (slot, token) pair reading its expert's rows in place; an index past the last expert is reported."""
+    import vectors
+    lang, nn = vectors.lang, vectors.nn
+    dev = request.getfixturevalue(dev_name)
+    E, F, H = 6, 96, 128
+    g = np.random.default_rng(S * 10 + k)
+    x = g.standard_normal((S, 1, H)).astype(np.float32)
+    wg, wu = ((g.standard_normal((E, F, H)) * 0.1).astype(np.float32) for _ in range(2))
+    wd = (g.standard_normal((E, H, F)) * 0.1).astype(np.float32)
+    if dev_name == "hip_bf16":
+        wg, wu, wd = U_round(wg), U_round(wu), U_round(wd)
+    idx = g.integers(0, E, (S, k)).astype(np.uint32)
+    val = g.random((S, k)).astype(np.float32)
+
+    def f(b, xv, iv, vv, g_all, u_all, d_all):
+        xv = xv + xv - xv
+        total = None
+        for i in range(k):
+            slot = lang.get(b, 1, i, iv)
+            sel = lambda w: lang.transpose(b, 1, 2, lang.index(b, 0, slot, w))
+            gate = lang.matmul(b, xv, sel(g_all))
+            up = lang.matmul(b, xv, sel(u_all))
+            y = lang.matmul(b, nn.silu(b, gate) * up, sel(d_all))
+            wgt = lang.reshape(b, lang.shape(b, lang.get(b, 2, 0, y)), lang.get(b, 1, i, vv))
+            y = y * lang.broadcast(b, wgt, lang.shape(b, y))
+            total = y if total is None else total + y
+        return total
+    (ref,) = vectors.run(oracle, f, 1, x, idx, val, wg, wu, wd)
+    dev.trace(True)
+    dev.trace_reset()
+    (got,) = vectors.run(dev, f, 1, x, idx, val, wg, wu, wd)
+    rep = dev.trace_report()
+    dev.trace(False)
+    name = "gemv_experts_bf16" if dev_name == "hip_bf16" else "gemv_experts_f32"
+    launches = {n: v["launches"] for n, v in rep.items()}
+    assert launches.get(name) == 2 and "gather" not in launches and "swiglu_fused" not in launches, launches
+    tol = 2e-2 if dev_name == "hip_bf16" else 1e-4
+    assert np.max(np.abs(got - ref)) <= tol * np.abs(ref).max()
+    bad = idx.copy()
+    bad[S - 1, k - 1] = E
+    with pytest.raises(cg.abi.BackendPanic, match="index out of bounds"):
+        vectors.run(dev, f, 1, x, bad, val, wg, wu, wd)
+
+
+@pytest.mark.gpu
 def test_expert_slots_sorted_by_expert(oracle, hip_bf16):
     """The same block where both products have k a multiple of 64: the (slot, token) pairs are sorted by
     expert once and both launches stream their operands through LDS stages.  A skewed routing: one
