@@ -694,8 +694,7 @@ static hipError_t launch_gemm_dma(const LaunchCtx &lc, const GemmDesc &g, uint32
     if (e != hipSuccess) return e;
     configured = true;
   }
-  hipExtLaunchKernelGGL((gemm_bf16_dma_kernel<BM_, BN_, WR, WC, EPI, NS, DUAL>), dim3(grid), dim3(WR * WC * 64), smem,
-                        lc.stream, lc.ev_start, lc.ev_stop, 0, g);
+  cg_launch(lc, gemm_bf16_dma_kernel<BM_, BN_, WR, WC, EPI, NS, DUAL>, dim3(grid), dim3(WR * WC * 64), smem, g);
   return hipGetLastError();
 }
 
@@ -1712,7 +1711,7 @@ static hipError_t launch_moe_gemm_dma(const LaunchCtx &lc, const MoeGemmDesc &g,
     if (e != hipSuccess) return e;
     configured = true;
   }
-  hipExtLaunchKernelGGL((moe_gemm_dma_kernel<NP, NS>), grid, dim3(256), smem, lc.stream, lc.ev_start, lc.ev_stop, 0, g);
+  cg_launch(lc, moe_gemm_dma_kernel<NP, NS>, grid, dim3(256), smem, g);
   return hipGetLastError();
 }
 

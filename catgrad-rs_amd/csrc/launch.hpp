@@ -5,6 +5,7 @@
 #include <hip/hip_ext.h>
 #include <stdint.h>
 #include "program.hpp"
+#include "launch_queue.hpp"
 
 namespace cgk {
 
@@ -17,13 +18,23 @@ struct LaunchCtx {
   uint32_t *err_flag;  // device word
   // when tracing: events that receive the kernel's own begin / end timestamps
   hipEvent_t ev_start, ev_stop;
+  // when set, launches are handed to this queue's thread instead of being made by the caller
+  LaunchQueue *queue;
 };
 
-// Every kernel is launched through this: with null events it is an ordinary launch; with events
-// the runtime stamps them at the kernel's start and end (what a profiler reports as duration).
-#define CG_LAUNCH(lc, kernel, grid, block, ...)                                            \
-  hipExtLaunchKernelGGL(kernel, dim3(grid), dim3(block), 0, (lc).stream, (lc).ev_start, \
-                        (lc).ev_stop, 0, __VA_ARGS__)
+// Every kernel is launched through this: with null events it is an ordinary launch (made by the
+// queue's thread when there is one); with events the runtime stamps them at the kernel's start and
+// end (what a profiler reports as duration), and the launch is made here, after the queue drained.
+template <typename... KArgs, typename... Args>
+inline void cg_launch(const LaunchCtx &lc, void (*kernel)(KArgs...), dim3 grid, dim3 block, size_t smem, Args &&...args) {
+  if (lc.queue && !lc.ev_start && !lc.ev_stop) {
+    lc.queue->launch(kernel, grid, block, smem, lc.stream, std::forward<Args>(args)...);
+    return;
+  }
+  if (lc.queue) lc.queue->drain();
+  hipExtLaunchKernelGGL(kernel, grid, block, smem, lc.stream, lc.ev_start, lc.ev_stop, 0, static_cast<KArgs>(args)...);
+}
+#define CG_LAUNCH(lc, kernel, grid, block, ...) cgk::cg_launch((lc), kernel, dim3(grid), dim3(block), 0, __VA_ARGS__)
 
 // ---- k_ew.hip
 hipError_t launch_ew(const LaunchCtx &lc, const Program &p, const OutDesc &o, uint64_t n_elems,

@@ -53,6 +53,7 @@ size_t size_class(size_t bytes) {
 }
 
 void trim_pool(cg_backend *be) {
+  if (be->queue) be->queue->drain();  // a launch still in the queue may read what is about to be freed
   for (auto &kv : be->pool)
     for (void *p : kv.second) {
       (void)hipFree(p);
@@ -106,7 +107,7 @@ void storage_release(Storage *s) {
 void backend_release(cg_backend *be) {
   if (!be || be->rc.fetch_sub(1) != 1) return;
   (void)hipSetDevice(be->device);
-  (void)hipStreamSynchronize(be->stream);
+  (void)hipStreamSynchronize(be->ordered_stream());
   for (auto &pe : be->trace_pending) {
     (void)hipEventDestroy(pe.start);
     (void)hipEventDestroy(pe.stop);
@@ -118,6 +119,8 @@ void backend_release(cg_backend *be) {
   if (be->attn_part) (void)hipFree(be->attn_part);
   if (be->attn_count) (void)hipFree(be->attn_count);
   if (be->h_words) (void)hipHostFree(be->h_words);
+  delete be->queue;  // drains and joins its thread
+  be->queue = nullptr;
   if (be->stream) (void)hipStreamDestroy(be->stream);
   delete be;
 }
@@ -288,7 +291,7 @@ struct KernelScope {
 
 void trace_collect(cg_backend *be) {
   if (be->trace_pending.empty()) return;
-  (void)hipStreamSynchronize(be->stream);
+  (void)hipStreamSynchronize(be->ordered_stream());
   for (auto &pe : be->trace_pending) {
     float ms = 0.f;
     if (hipEventElapsedTime(&ms, pe.start, pe.stop) == hipSuccess) {  // fails if nothing was launched
@@ -1964,7 +1967,7 @@ int attn_decode_scratch(cg_backend *be, size_t part_floats, size_t count_words) 
   if (part_floats > be->attn_part_floats) {
     size_t want = 1 << 16;
     while (want < part_floats) want <<= 1;
-    HIPCHK(be, hipStreamSynchronize(be->stream));
+    HIPCHK(be, hipStreamSynchronize(be->ordered_stream()));
     if (be->attn_part) (void)hipFree(be->attn_part);
     be->attn_part = nullptr;
     be->attn_part_floats = 0;
@@ -1974,12 +1977,12 @@ int attn_decode_scratch(cg_backend *be, size_t part_floats, size_t count_words) 
   if (count_words > be->attn_count_words) {
     size_t want = 1 << 10;
     while (want < count_words) want <<= 1;
-    HIPCHK(be, hipStreamSynchronize(be->stream));
+    HIPCHK(be, hipStreamSynchronize(be->ordered_stream()));
     if (be->attn_count) (void)hipFree(be->attn_count);
     be->attn_count = nullptr;
     be->attn_count_words = 0;
     HIPCHK(be, hipMalloc((void **)&be->attn_count, want * sizeof(uint32_t)));
-    HIPCHK(be, hipMemsetAsync(be->attn_count, 0, want * sizeof(uint32_t), be->stream));
+    HIPCHK(be, hipMemsetAsync(be->attn_count, 0, want * sizeof(uint32_t), be->ordered_stream()));
     be->attn_count_words = want;
   }
   return CG_OK;
@@ -3533,8 +3536,9 @@ int realize(cg_backend *be, cg_tensor *n) {
 
 // wait for the stream and surface device-side error flags
 int sync_and_check(cg_backend *be) {
-  HIPCHK(be, hipMemcpyAsync(be->h_words, be->d_words, 8, hipMemcpyDeviceToHost, be->stream));
-  HIPCHK(be, hipStreamSynchronize(be->stream));
+  HIPCHK(be, hipMemcpyAsync(be->h_words, be->d_words, 8, hipMemcpyDeviceToHost, be->ordered_stream()));
+  if (be->queue) HIPCHK(be, be->queue->take_error());  // a launch the queue's thread could not make
+  HIPCHK(be, hipStreamSynchronize(be->ordered_stream()));
   const uint32_t e = be->h_words[0];
   if (e) {
     HIPCHK(be, launch_fill_u32(be->lc(), be->d_words, 0u, 1));
@@ -3690,8 +3694,10 @@ int binary(cg_backend *be, cg_tensor *a, cg_tensor *b, cg_tensor **out, EwOp f_o
   // takes a millisecond to record.  Realising it now starts the device on this block while the
   // caller records the next one.  One-row steps (decode) stay deferred: there the caller overlaps
   // whole steps.  A broadcast operand (a bias) is not a residual, nor is a value that is still deferred.
+  // With a launch thread the same holds for the few rows of a decode step: the block's kernels are
+  // handed over now and reach the runtime while this thread records the next block.
   bool block_end = false;
-  if (n->ew == E_ADD_F && n->rank == 3 && n->shape[1] >= 64 && !(be->flags & (CG_FLAG_EAGER | CG_FLAG_NO_PATTERNS))) {
+  if (n->ew == E_ADD_F && n->rank == 3 && (n->shape[1] >= 64 || be->queue) && !(be->flags & (CG_FLAG_EAGER | CG_FLAG_NO_PATTERNS))) {
     for (int side = 0; side < 2 && !block_end; ++side) {
       const cg_tensor *mm = n->in[side], *other = n->in[1 - side];
       if (mm->op == N_RESHAPE) mm = mm->in[0];  // batch folded into the rows for the linear and unfolded again
@@ -3745,8 +3751,8 @@ int upload(cg_backend *be, const void *data, size_t n, const int64_t *shape, int
   }
   hipError_t e = hipSuccess;
   if (!narrow) {
-    e = hipMemcpyAsync(t->st->ptr, data, n * 4, hipMemcpyHostToDevice, be->stream);
-    if (e == hipSuccess) e = hipStreamSynchronize(be->stream);
+    e = hipMemcpyAsync(t->st->ptr, data, n * 4, hipMemcpyHostToDevice, be->ordered_stream());
+    if (e == hipSuccess) e = hipStreamSynchronize(be->ordered_stream());
   } else {
     // stage through a bounded f32 buffer, narrow with the copy program (RNE)
     const size_t chunk = (size_t)16 << 20;  // elements
@@ -3758,7 +3764,7 @@ int upload(cg_backend *be, const void *data, size_t n, const int64_t *shape, int
     }
     for (size_t o = 0; o < n && e == hipSuccess; o += chunk) {
       const size_t c = std::min(chunk, n - o);
-      e = hipMemcpyAsync(stage->ptr, (const char *)data + o * 4, c * 4, hipMemcpyHostToDevice, be->stream);
+      e = hipMemcpyAsync(stage->ptr, (const char *)data + o * 4, c * 4, hipMemcpyHostToDevice, be->ordered_stream());
       if (e != hipSuccess) break;
       Program p;
       std::memset(&p, 0, sizeof(p));
@@ -3779,7 +3785,7 @@ int upload(cg_backend *be, const void *data, size_t n, const int64_t *shape, int
       od.stride[0] = 1;
       KernelScope ks(be, "ew_to_bf16", (double)c * 6, 0);
       e = launch_ew(be->lc(), p, od, c, c % 4 == 0);
-      if (e == hipSuccess) e = hipStreamSynchronize(be->stream);
+      if (e == hipSuccess) e = hipStreamSynchronize(be->ordered_stream());
     }
     storage_release(stage);
   }
@@ -3809,7 +3815,7 @@ int download(cg_backend *be, cg_tensor *x, void *dst, size_t n, cg_dtype want) {
   TRY(contiguous(be, x, &c));
   int st = CG_OK;
   if (n) {
-    hipError_t e = hipMemcpyAsync(dst, data_ptr(c), n * 4, hipMemcpyDeviceToHost, be->stream);
+    hipError_t e = hipMemcpyAsync(dst, data_ptr(c), n * 4, hipMemcpyDeviceToHost, be->ordered_stream());
     if (e != hipSuccess) st = fail(be, CG_ERR_DEVICE, hipGetErrorString(e));
   }
   if (!st) st = sync_and_check(be);
@@ -3836,11 +3842,13 @@ int cg_backend_create(int device, uint32_t flags, cg_backend **out) {
   if (hipGetDeviceProperties(&prop, device) == hipSuccess) be->n_cus = prop.multiProcessorCount;
   if (hipStreamCreate(&be->stream) != hipSuccess || hipMalloc((void **)&be->d_words, 256) != hipSuccess ||
       hipHostMalloc((void **)&be->h_words, 256, hipHostMallocDefault) != hipSuccess ||
-      hipMemsetAsync(be->d_words, 0, 256, be->stream) != hipSuccess ||
-      hipStreamSynchronize(be->stream) != hipSuccess) {
+      hipMemsetAsync(be->d_words, 0, 256, be->ordered_stream()) != hipSuccess ||
+      hipStreamSynchronize(be->ordered_stream()) != hipSuccess) {
     delete be;
     return CG_ERR_DEVICE;
   }
+  // deferred evaluation issues kernels in bursts: a second thread makes the runtime calls
+  if (!(flags & CG_FLAG_EAGER)) be->queue = new cgk::LaunchQueue(device);
   *out = be;
   return CG_OK;
 }
@@ -3892,10 +3900,10 @@ int cg_tensor_prefetch(cg_backend *be, cg_tensor *t) {
     be->pinned_pool.push_back(buf);
     return fail(be, CG_ERR_DEVICE, "hipEventCreate failed");
   }
-  hipError_t e = hipMemcpyAsync(buf, data_ptr(t), bytes, hipMemcpyDeviceToHost, be->stream);
+  hipError_t e = hipMemcpyAsync(buf, data_ptr(t), bytes, hipMemcpyDeviceToHost, be->ordered_stream());
   if (e == hipSuccess)
-    e = hipMemcpyAsync((char *)buf + PREFETCH_BYTES - 8, be->d_words, 8, hipMemcpyDeviceToHost, be->stream);
-  if (e == hipSuccess) e = hipEventRecord(ev, be->stream);
+    e = hipMemcpyAsync((char *)buf + PREFETCH_BYTES - 8, be->d_words, 8, hipMemcpyDeviceToHost, be->ordered_stream());
+  if (e == hipSuccess) e = hipEventRecord(ev, be->ordered_stream());
   if (e != hipSuccess) {
     be->pinned_pool.push_back(buf);
     be->event_pool.push_back(ev);
@@ -3976,8 +3984,8 @@ int cg_from_bf16(cg_backend *be, const uint16_t *bits, size_t n, const size_t *d
   hipError_t e = hipSuccess;
   if (n == 0) {
   } else if (keep) {
-    e = hipMemcpyAsync(t->st->ptr, bits, n * 2, hipMemcpyHostToDevice, be->stream);
-    if (e == hipSuccess) e = hipStreamSynchronize(be->stream);
+    e = hipMemcpyAsync(t->st->ptr, bits, n * 2, hipMemcpyHostToDevice, be->ordered_stream());
+    if (e == hipSuccess) e = hipStreamSynchronize(be->ordered_stream());
   } else {
     const size_t chunk = (size_t)16 << 20;  // elements per staged piece
     Storage *stage = nullptr;
@@ -3988,7 +3996,7 @@ int cg_from_bf16(cg_backend *be, const uint16_t *bits, size_t n, const size_t *d
     }
     for (size_t o = 0; o < n && e == hipSuccess; o += chunk) {
       const size_t c = std::min(chunk, n - o);
-      e = hipMemcpyAsync(stage->ptr, bits + o, c * 2, hipMemcpyHostToDevice, be->stream);
+      e = hipMemcpyAsync(stage->ptr, bits + o, c * 2, hipMemcpyHostToDevice, be->ordered_stream());
       if (e != hipSuccess) break;
       Program p;
       std::memset(&p, 0, sizeof(p));
@@ -4009,7 +4017,7 @@ int cg_from_bf16(cg_backend *be, const uint16_t *bits, size_t n, const size_t *d
       od.stride[0] = 1;
       KernelScope ks(be, "ew_from_bf16", (double)c * 6, 0);
       e = launch_ew(be->lc(), p, od, c, c % 4 == 0);
-      if (e == hipSuccess) e = hipStreamSynchronize(be->stream);
+      if (e == hipSuccess) e = hipStreamSynchronize(be->ordered_stream());
     }
     storage_release(stage);
   }
@@ -4070,7 +4078,7 @@ int cg_stack(cg_backend *be, cg_tensor *const *parts, size_t n, cg_tensor **out)
   const size_t each = (size_t)parts[0]->size() * esize(dense[0]->stype);
   hipError_t e = hipSuccess;
   for (size_t i = 0; i < n && e == hipSuccess && each; ++i)
-    e = hipMemcpyAsync((char *)t->st->ptr + i * each, data_ptr(dense[i]), each, hipMemcpyDeviceToDevice, be->stream);
+    e = hipMemcpyAsync((char *)t->st->ptr + i * each, data_ptr(dense[i]), each, hipMemcpyDeviceToDevice, be->ordered_stream());
   drop();
   if (e != hipSuccess) {
     node_release(t);
@@ -4410,10 +4418,10 @@ int cg_peak_copy_gbs(cg_backend *be, size_t bytes, int iters, double *gbs) {
   lc.ev_start = lc.ev_stop = nullptr;
   if (e == hipSuccess) e = launch_fill_u32(lc, (uint32_t *)a->ptr, 0x3F800000u, bytes / 4);
   if (e == hipSuccess) e = launch_peak_copy(lc, a->ptr, b->ptr, bytes);  // warm-up
-  if (e == hipSuccess) e = hipEventRecord(e0, be->stream);
+  if (e == hipSuccess) e = hipEventRecord(e0, be->ordered_stream());
   for (int i = 0; i < iters && e == hipSuccess; ++i) e = launch_peak_copy(lc, a->ptr, b->ptr, bytes);
-  if (e == hipSuccess) e = hipEventRecord(e1, be->stream);
-  if (e == hipSuccess) e = hipStreamSynchronize(be->stream);
+  if (e == hipSuccess) e = hipEventRecord(e1, be->ordered_stream());
+  if (e == hipSuccess) e = hipStreamSynchronize(be->ordered_stream());
   float ms = 0.f;
   if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
   if (e0) (void)hipEventDestroy(e0);
@@ -4438,10 +4446,10 @@ int cg_peak_mfma_tflops(cg_backend *be, cg_dtype operand, int iters, double *tfl
   LaunchCtx lc = be->lc();
   lc.ev_start = lc.ev_stop = nullptr;
   if (e == hipSuccess) e = launch_peak_mfma(lc, bf16, (float *)o->ptr, grid, 64);
-  if (e == hipSuccess) e = hipEventRecord(e0, be->stream);
+  if (e == hipSuccess) e = hipEventRecord(e0, be->ordered_stream());
   if (e == hipSuccess) e = launch_peak_mfma(lc, bf16, (float *)o->ptr, grid, iters);
-  if (e == hipSuccess) e = hipEventRecord(e1, be->stream);
-  if (e == hipSuccess) e = hipStreamSynchronize(be->stream);
+  if (e == hipSuccess) e = hipEventRecord(e1, be->ordered_stream());
+  if (e == hipSuccess) e = hipStreamSynchronize(be->ordered_stream());
   float ms = 0.f;
   if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
   if (e0) (void)hipEventDestroy(e0);

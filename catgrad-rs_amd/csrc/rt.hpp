@@ -145,5 +145,13 @@ struct cg_backend {
   uint32_t *attn_count = nullptr;
   size_t attn_part_floats = 0, attn_count_words = 0;
 
-  cgk::LaunchCtx lc() const { return cgk::LaunchCtx{stream, n_cus, d_words, cur_start, cur_stop}; }
+  // kernel launches go through this thread's queue; null when the backend launches inline (CG_FLAG_EAGER)
+  cgk::LaunchQueue *queue = nullptr;
+  cgk::LaunchCtx lc() const { return cgk::LaunchCtx{stream, n_cus, d_words, cur_start, cur_stop, queue}; }
+  // the stream, once every launch handed to the queue has reached it: what anything but a kernel launch
+  // (copies, events, synchronisation, frees) must use to keep program order
+  hipStream_t ordered_stream() const {
+    if (queue) queue->drain();
+    return stream;
+  }
 };
