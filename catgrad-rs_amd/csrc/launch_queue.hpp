@@ -14,6 +14,7 @@
 #include <hip/hip_ext.h>
 #include <stdint.h>
 #include <atomic>
+#include <chrono>
 #include <condition_variable>
 #include <mutex>
 #include <new>
@@ -63,8 +64,10 @@ class LaunchQueue {
           [q](auto &...a) { hipExtLaunchKernelGGL(q->kernel, q->grid, q->block, q->smem, q->stream, nullptr, nullptr, 0, a...); },
           q->a);
     };
-    head_.store(h + 1, std::memory_order_release);
-    if (sleeping_.load(std::memory_order_acquire)) wake();
+    // sequentially consistent on both sides: either this thread sees the worker asleep, or the worker's
+    // last look at the ring before it sleeps sees this slot
+    head_.store(h + 1);
+    if (sleeping_.load()) wake();
   }
 
   // Returns once every launch handed over so far has been given to the runtime.
@@ -104,11 +107,9 @@ class LaunchQueue {
           continue;
         }
         std::unique_lock<std::mutex> lk(m_);
-        sleeping_.store(true, std::memory_order_release);
-        cv_.wait_for(lk, std::chrono::milliseconds(50), [this, t] {
-          return head_.load(std::memory_order_acquire) != t || stop_.load(std::memory_order_acquire);
-        });
-        sleeping_.store(false, std::memory_order_release);
+        sleeping_.store(true);
+        cv_.wait_for(lk, std::chrono::milliseconds(50), [this, t] { return head_.load() != t || stop_.load(); });
+        sleeping_.store(false);
         idle = 0;
         continue;
       }
