@@ -94,6 +94,15 @@ __global__ void __launch_bounds__(NW * 64) attn_prefill_kernel(AttnPrefillDesc a
   float4 mreg[KT][4];
   // All loads are unconditional (indices clamped into range) so that they are issued back to back;
   // chunks past the end are zeroed when the registers are consumed.
+  // With a class table, dead key tiles are never visited and all-zero ones need no mask values.
+  const uint8_t *cls = a.tile_class ? a.tile_class + (size_t)blockIdx.x * a.tile_cols : nullptr;
+  auto next_step = [&](uint32_t t0) {  // the first step at or after t0 that is not dead (>= a.t: none)
+    if (!cls) return t0;
+    uint32_t i = t0 / BN;
+    while (i < a.tile_cols && cls[i] == 0) ++i;
+    return i * (uint32_t)BN;
+  };
+  auto step_mask = [&](uint32_t t0) { return M && !(cls && t0 < a.t && cls[t0 / BN] == 2); };
   auto fetch = [&](uint32_t t0) {
 #pragma unroll
     for (int c = 0; c < KCH; ++c) {
@@ -105,7 +114,7 @@ __global__ void __launch_bounds__(NW * 64) attn_prefill_kernel(AttnPrefillDesc a
       const int ch = tid + c * NT, dim = ch / (BN / 8), k8 = (ch % (BN / 8)) * 8;
       vreg[c] = *(const uint4 *)(VT + (int64_t)dim * a.t + min(t0 + k8, a.t - 8));
     }
-    if (M) {  // mask rows allow 16-byte loads and T % 8 == 0 (checked by the host)
+    if (step_mask(t0)) {  // mask rows allow 16-byte loads and T % 8 == 0 (checked by the host)
 #pragma unroll
       for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
@@ -113,14 +122,17 @@ __global__ void __launch_bounds__(NW * 64) attn_prefill_kernel(AttnPrefillDesc a
           mreg[kt][j] = *(const float4 *)(M + min(t0 + kt * 32 + j * 8 + half * 4, a.t - 4));
     }
   };
-  fetch(0);
-  for (uint32_t t0 = 0; t0 < a.t; t0 += BN) {
+  uint32_t t0 = next_step(0);
+  if (t0 < a.t) fetch(t0);
+  for (; t0 < a.t;) {
+    const uint32_t t_next = next_step(t0 + BN);
+    const bool use_mask = step_mask(t0);  // uniform
     // ---- is any (query, key) pair of this step unmasked?  A causal or sliding-window mask kills
     // most steps; a dead step only adds terms that the first live step rescales to zero.
     const bool tail = t0 + BN > a.t;  // the only step with keys past the end (uniform)
-    bool live_pair = !M;
+    bool live_pair = !use_mask;
     float4 mcur[KT][4];
-    if (M) {
+    if (use_mask) {
       float mmax = -3.40282347e+38f;
 #pragma unroll
       for (int kt = 0; kt < KT; ++kt)
@@ -154,7 +166,9 @@ __global__ void __launch_bounds__(NW * 64) attn_prefill_kernel(AttnPrefillDesc a
       }
     }
     __syncthreads();
-    if (t0 + BN < a.t) fetch(t0 + BN);  // in flight during the arithmetic below
+    if (t_next < a.t) fetch(t_next);  // in flight during the arithmetic below
+    const uint32_t t_cur = t0;
+    t0 = t_next;
     if (!live) continue;
     // ---- S^T = K . Q^T
     a_f32x16 st[KT];
@@ -174,15 +188,15 @@ __global__ void __launch_bounds__(NW * 64) attn_prefill_kernel(AttnPrefillDesc a
     for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const uint32_t key = t0 + kt * 32 + j * 8 + half * 4;
+        const uint32_t key = t_cur + kt * 32 + j * 8 + half * 4;
         float mv[4] = {0.f, 0.f, 0.f, 0.f};
-        if (M) { mv[0] = mcur[kt][j].x; mv[1] = mcur[kt][j].y; mv[2] = mcur[kt][j].z; mv[3] = mcur[kt][j].w; }
+        if (use_mask) { mv[0] = mcur[kt][j].x; mv[1] = mcur[kt][j].y; mv[2] = mcur[kt][j].z; mv[3] = mcur[kt][j].w; }
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           float s = st[kt][j * 4 + i];
           if (a.has_scale) s = s * inv_scale;
-          if (M) s = s + mv[i];
-          else if (a.has_mask_const) s = s + a.mask_const;
+          if (use_mask) s = s + mv[i];
+          else if (!M && a.has_mask_const) s = s + a.mask_const;
           if (tail && key + i >= a.t) s = -3.40282347e+38f;  // past the end: contributes exp(..) = 0
           st[kt][j * 4 + i] = s;
           tmax = fmaxf(tmax, s);
@@ -200,7 +214,7 @@ __global__ void __launch_bounds__(NW * 64) attn_prefill_kernel(AttnPrefillDesc a
         float p[8];
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-          const uint32_t key = t0 + kt * 32 + (blk * 2 + (i >> 2)) * 8 + half * 4 + (i & 3);
+          const uint32_t key = t_cur + kt * 32 + (blk * 2 + (i >> 2)) * 8 + half * 4 + (i & 3);
           p[i] = __expf(st[kt][blk * 8 + i] - m_new);
           if (tail && key >= a.t) p[i] = 0.f;
           psum += p[i];
@@ -269,10 +283,47 @@ __global__ void __launch_bounds__(NW * 64) attn_prefill_kernel(AttnPrefillDesc a
   }
 }
 
+static bool attn_prefill_small_tiles(const LaunchCtx &lc, const AttnPrefillDesc &d) {
+  return (uint64_t)((d.s + 127) / 128) * d.heads * d.b < (uint64_t)lc.n_cus;  // too few workgroups of 128 queries: 64 each
+}
+
+void attn_prefill_tiling(const LaunchCtx &lc, const AttnPrefillDesc &d, uint32_t *q_rows, uint32_t *keys) {
+  *q_rows = attn_prefill_small_tiles(lc, d) ? 64 : 128;
+  *keys = d.d == 256 ? 32 : 64;
+}
+
+// one workgroup per (key tile, query tile): any value above the masked level, any value that is not zero
+__global__ void __launch_bounds__(256) mask_tiles_kernel(const float *mask, int64_t m_ss, uint32_t s, uint32_t t, uint32_t q_rows,
+                                                         uint32_t keys, uint8_t *out) {
+  __shared__ uint32_t flags;
+  if (threadIdx.x == 0) flags = 0;
+  __syncthreads();
+  const uint32_t q0 = blockIdx.y * q_rows, k0 = blockIdx.x * keys;
+  uint32_t f = 0;  // bit 0: some pair is not masked, bit 1: some value is not zero
+  for (uint32_t i = threadIdx.x; i < q_rows * keys; i += 256) {
+    const uint32_t q = q0 + i / keys, k = k0 + i % keys;
+    if (q < s && k < t) {
+      const float v = mask[(int64_t)q * m_ss + k];
+      if (v > -3.0e38f) f |= 1u;
+      if (v != 0.f) f |= 2u;
+    }
+  }
+  if (f) atomicOr(&flags, f);
+  __syncthreads();
+  if (threadIdx.x == 0) out[(size_t)blockIdx.y * gridDim.x + blockIdx.x] = !(flags & 1u) ? 0 : (flags & 2u) ? 1 : 2;
+}
+
+hipError_t launch_mask_tiles(const LaunchCtx &lc, const float *mask, int64_t m_ss, uint32_t s, uint32_t t, uint32_t q_rows,
+                             uint32_t keys, uint8_t *out) {
+  if (!s || !t) return hipSuccess;
+  CG_LAUNCH(lc, mask_tiles_kernel, dim3((t + keys - 1) / keys, (s + q_rows - 1) / q_rows), 256, mask, m_ss, s, t, q_rows, keys, out);
+  return hipGetLastError();
+}
+
 hipError_t launch_attn_prefill(const LaunchCtx &lc, const AttnPrefillDesc &d) {
   if (!d.b || !d.heads || !d.s) return hipSuccess;
   dim3 grid((d.s + 127) / 128, d.heads, d.b);
-  if ((uint64_t)grid.x * grid.y * grid.z < (uint64_t)lc.n_cus) {  // too few workgroups of 128 queries: 64 each
+  if (attn_prefill_small_tiles(lc, d)) {
     grid.x = (d.s + 63) / 64;
     switch (d.d) {
       case 64: CG_LAUNCH(lc, (attn_prefill_kernel<64, 64, 2>), grid, 128, d); break;

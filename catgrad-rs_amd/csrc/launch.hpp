@@ -191,8 +191,20 @@ struct AttnPrefillDesc {
   uint32_t b, heads, rep, s, t, d;
   int32_t has_scale, has_mask_const, m_vec;  // m_vec: mask rows allow 16-byte loads
   float scale, mask_const;
+  // optional, for a mask shared by every batch and head (m_sb == m_sh == 0): the class of every
+  // (query tile, key tile) pair from launch_mask_tiles with the tiling of attn_prefill_tiling - 0 = every
+  // pair masked (the tile is skipped without being fetched), 2 = every value zero (the tile is computed
+  // without reading the mask), 1 = anything else; row q of the table has tile_cols entries
+  const uint8_t *tile_class;
+  uint32_t tile_cols;
 };
 hipError_t launch_attn_prefill(const LaunchCtx &lc, const AttnPrefillDesc &d);
+// query rows and keys per tile that launch_attn_prefill uses for this problem
+void attn_prefill_tiling(const LaunchCtx &lc, const AttnPrefillDesc &d, uint32_t *q_rows, uint32_t *keys);
+// out[qt * ceil(t / keys) + kt] = class of mask[qt * q_rows .., kt * keys ..] (values <= -3e38 count as masked);
+// mask is [s, t] with unit stride along t and row stride m_ss
+hipError_t launch_mask_tiles(const LaunchCtx &lc, const float *mask, int64_t m_ss, uint32_t s, uint32_t t, uint32_t q_rows,
+                             uint32_t keys, uint8_t *out);
 
 // ---- k_gemm.hip
 struct GemmDesc {

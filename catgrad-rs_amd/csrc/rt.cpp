@@ -97,6 +97,7 @@ void backend_release(cg_backend *be);
 void storage_release(Storage *s) {
   if (!s || s->rc.fetch_sub(1) != 1) return;
   storage_release(s->shadow);
+  storage_release(s->tiles);
   cg_backend *be = s->be;
   // Safe to recycle at once: every consumer was enqueued on the backend's only stream.
   be->pool[s->bytes].push_back(s->ptr);
@@ -1948,6 +1949,34 @@ int try_attn_prefill(cg_backend *be, cg_tensor *n, bool *done) {
   a.scale = m.scale;
   a.has_mask_const = m.has_mask_const;
   a.mask_const = m.mask_const;
+  // One mask for every batch and head (the causal or sliding-window mask of a model): classify its
+  // tiles once - the table stays with the mask's storage, so every layer of the run finds it - and let
+  // the kernel skip the key tiles no query of a tile can see.
+  if (mask && a.m_sb == 0 && a.m_sh == 0 && a.m_ss > 0 && mask->st->grow_dim < 0) {
+    uint32_t q_rows = 0, keys = 0;
+    attn_prefill_tiling(be->lc(), a, &q_rows, &keys);
+    Storage *ms = mask->st;
+    const int64_t key[5] = {mask->offset, Sq, T, q_rows, keys};
+    const size_t rows = (size_t)(Sq + q_rows - 1) / q_rows, cols = (size_t)(T + keys - 1) / keys;
+    if (!ms->tiles || !std::equal(key, key + 5, ms->tiles_key)) {
+      storage_release(ms->tiles);
+      ms->tiles = nullptr;
+      int st = dev_alloc(be, rows * cols, &ms->tiles);
+      if (st) {
+        storage_release(vt);
+        return st;
+      }
+      std::copy(key, key + 5, ms->tiles_key);
+      KernelScope ks(be, "attn_mask_tiles", (double)Sq * T * 4, 0);
+      hipError_t me = launch_mask_tiles(be->lc(), a.mask, a.m_ss, (uint32_t)Sq, (uint32_t)T, q_rows, keys, (uint8_t *)ms->tiles->ptr);
+      if (me != hipSuccess) {
+        storage_release(vt);
+        return fail(be, CG_ERR_DEVICE, hipGetErrorString(me));
+      }
+    }
+    a.tile_class = (const uint8_t *)ms->tiles->ptr;
+    a.tile_cols = (uint32_t)cols;
+  }
   {
     const double qo = 2.0 * nb * heads * Sq * d * 4, kvb = 2.0 * nb * Kop.shape[1] * T * d * 4;
     KernelScope ks(be, "attn_prefill", qo + kvb + (mask ? (double)Sq * T * 4 : 0.0), 4.0 * nb * heads * Sq * T * d);

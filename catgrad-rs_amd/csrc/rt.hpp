@@ -33,6 +33,10 @@ struct Storage {
   // bf16 copy of this (f32) storage, element for element, made on demand for the MFMA GEMM and
   // shared by every matmul that reads a view of it (q/k/v, gate/up read the same activations)
   Storage *shadow = nullptr;
+  // an attention mask's table of tile classes (launch_mask_tiles), made on demand and shared by every
+  // layer that reads the mask; tiles_key = {element offset of the mask, rows, keys, query rows per tile, keys per tile}
+  Storage *tiles = nullptr;
+  int64_t tiles_key[5] = {-1, 0, 0, 0, 0};
 };
 
 enum NodeOp : uint8_t {

@@ -431,6 +431,43 @@ def hip_bf16_flash():
     return cg.Backend(cg.load_library(), flags=cg.abi.FLAG_BF16 | cg.abi.FLAG_ATTN_ONE_PASS)
 
 
+def test_attention_prefill_with_an_arbitrary_shared_mask(oracle, hip_bf16_flash):
+    """One [S, T] mask for every batch and head, given as data: its key tiles are classified once
+    (all masked: skipped unfetched; all zero: computed without reading the mask; mixed) and the kernel
+    must give the oracle's values for each kind - including rows that see no key at all, which the
+    reference turns into the mean of V."""
+    nb, H, KV, S, d = 2, 4, 2, 384, 64
+    g = np.random.default_rng(77)
+    q = g.standard_normal((nb, H, S, d)).astype(np.float32)
+    k = g.standard_normal((nb, KV, S, d)).astype(np.float32)
+    v = g.standard_normal((nb, KV, S, d)).astype(np.float32)
+    lo = np.finfo(np.float32).min
+    mask = np.where(g.random((S, S)) < 0.5, lo, 0.0).astype(np.float32)      # mixed everywhere ...
+    mask[:128, 128:] = lo                                                    # ... except dead tiles,
+    mask[128:256, :192] = 0.0                                                # all-zero tiles,
+    mask[300:303, :] = lo                                                    # rows that see nothing,
+    mask[256:, 64:128] = lo                                                  # and a dead column of tiles in the middle
+    mask = mask.reshape(-1)      # uploaded as rank 1 (a value, kept f32 in bf16 mode) and shaped in the graph
+
+    def f(b, qv, kv, vv, mv):
+        qv, kv, vv = qv + qv - qv, kv + kv - kv, vv + vv - vv
+        mv = lang.reshape(b, lang.make_shape(b, 1, 1, S, S), mv)
+        kr = helpers.repeat_kv(b, H // KV, kv)
+        vr = helpers.repeat_kv(b, H // KV, vv)
+        attn = lang.matmul(b, qv, lang.transpose(b, 2, 3, kr))
+        sh = lang.shape(b, attn)
+        attn = attn / lang.constant(b, float(np.sqrt(np.float32(d))), sh)
+        attn = attn + lang.broadcast(b, mv, sh)
+        return lang.matmul(b, nn.softmax(b, attn), vr)
+    (ref,) = vectors.run(oracle, f, 1, q, k, v, mask)
+    got, names = run_traced(hip_bf16_flash, f, 1, q, k, v, mask)
+    assert "attn_prefill" in names and "attn_mask_tiles" in names and "softmax_fused" not in names, sorted(names)
+    scale = np.abs(ref).max()
+    assert np.max(np.abs(got[0] - ref)) <= 2e-2 * scale, np.max(np.abs(got[0] - ref)) / scale
+    # the rows that see nothing: the mean of V, for every head
+    assert np.max(np.abs(got[0][:, :, 300:303] - np.repeat(v, H // KV, axis=1).mean(axis=2, keepdims=True))) <= 2e-2 * scale
+
+
 @pytest.mark.parametrize("cfg", [(1, 32, 8, 512, 64), (2, 4, 2, 100, 128), (2, 4, 2, 104, 128), (1, 4, 1, 200, 256),
                                  (1, 8, 8, 33, 64), (1, 2, 1, 1024, 64)])
 @pytest.mark.parametrize("mask_kind", ["causal", "window"])
