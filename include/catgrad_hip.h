@@ -62,7 +62,9 @@ enum {
 /* cg_backend_create flags */
 enum {
   /* F32 tensors of rank >= 2 handed over with cg_from_f32 are stored as bf16 and every
-   * matmul rounds its operands to bf16 (f32 accumulation).  Everything else stays f32. */
+   * matmul rounds its operands to bf16 (f32 accumulation).  Everything else stays f32, except a
+   * value computed only to be such an operand (the gated activation of an MLP over many rows),
+   * which may be kept in the rounded form the matmul would read anyway. */
   CG_FLAG_BF16 = 1u,
   /* run every op when it is issued instead of deferring and fusing */
   CG_FLAG_EAGER = 2u,
