@@ -1086,6 +1086,7 @@ __global__ void __launch_bounds__(256) gemv_pro_kernel(GemvProDesc g) {
   const int64_t sbn = g.m.p[blockIdx.y].sbn;
   float *C = g.m.p[blockIdx.y].c + (uint64_t)bz * N;
   const float *Cadd = g.m.p[blockIdx.y].c_add ? g.m.p[blockIdx.y].c_add + (uint64_t)bz * N : nullptr;
+  const uint32_t cadd_rs = g.m.p[blockIdx.y].c_add_is_row ? 0u : N;  // a bias vector or a [rows, N] residual
   const uint32_t slot = KSPLIT ? blockIdx.x : blockIdx.x * 4 + wave;
   const uint32_t n_slots = KSPLIT ? gridDim.x : gridDim.x * 4;
   uint32_t k_begin = 0, k_end = K;
@@ -1249,7 +1250,8 @@ __global__ void __launch_bounds__(256) gemv_pro_kernel(GemvProDesc g) {
         const int r = tid % R, m = tid / R;
         if ((uint32_t)m < rows && nb + r < N) {
           const uint64_t at = (uint64_t)m * N + nb + r;
-          C[at] = ((part[0][r][m] + part[1][r][m]) + (part[2][r][m] + part[3][r][m])) + (Cadd ? Cadd[at] : 0.f);
+          C[at] = ((part[0][r][m] + part[1][r][m]) + (part[2][r][m] + part[3][r][m])) +
+                  (Cadd ? Cadd[(uint64_t)m * cadd_rs + nb + r] : 0.f);
         }
       }
     } else if (lane == 0) {
@@ -1259,7 +1261,7 @@ __global__ void __launch_bounds__(256) gemv_pro_kernel(GemvProDesc g) {
         for (int m = 0; m < MR; ++m)
           if ((uint32_t)m < rows && nb + r < N) {
             const uint64_t at = (uint64_t)m * N + nb + r;
-            C[at] = acc[r][m] + (Cadd ? Cadd[at] : 0.f);
+            C[at] = acc[r][m] + (Cadd ? Cadd[(uint64_t)m * cadd_rs + nb + r] : 0.f);
           }
     }
   }

@@ -273,6 +273,9 @@ struct GemvMultiDesc {
     const float *c_add;  // optional: c = x . b^T + c_add
     int64_t sbn;
     uint32_t N;
+    // several input rows (GemvProDesc::rows): c_add is a vector added to every row (a bias) instead of
+    // a [rows, N] matrix (a residual)
+    int32_t c_add_is_row;
   } p[4];
 };
 hipError_t launch_gemv_multi(const LaunchCtx &lc, const GemvMultiDesc &g);

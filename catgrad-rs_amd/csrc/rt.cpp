@@ -174,6 +174,7 @@ void node_release(cg_tensor *t) {
     if (n->gemv_candidate) forget_gemv_candidate(n);
     if (n->gemm_candidate) forget_gemm_candidate(n);
     forget_shared(n);
+    if (n->bias_of && n->bias_of->bias_user == n) n->bias_of->bias_user = nullptr;  // its inputs are still alive here
     if (n->in[0]) stack.push_back(n->in[0]);
     if (n->in[1]) stack.push_back(n->in[1]);
     storage_release(n->st);
@@ -204,6 +205,10 @@ void forget_shared(cg_tensor *n) {
 }
 
 void drop_inputs(cg_tensor *n) {
+  if (n->bias_of) {
+    if (n->bias_of->bias_user == n) n->bias_of->bias_user = nullptr;
+    n->bias_of = nullptr;
+  }
   cg_tensor *a = n->in[0], *b = n->in[1];
   n->in[0] = n->in[1] = nullptr;
   node_release(a);
@@ -1334,6 +1339,8 @@ static bool same_rows(const cg_tensor *a, const cg_tensor *b) {
 }
 
 int try_gate_up_glu(cg_backend *be, cg_tensor *glu, cg_tensor *g, cg_tensor *u, int gelu, bool *done);
+cg_tensor *bias_vector_of(cg_tensor *other, const cg_tensor *like);
+bool bias_vector_ready(const cg_tensor *v);
 
 int try_glu(cg_backend *be, cg_tensor *root, bool *done) {
   cg_tensor *gate = nullptr, *up = nullptr;
@@ -1440,10 +1447,22 @@ int try_gemv_add(cg_backend *be, cg_tensor *root, bool *done) {
     if (mm->op != N_MATMUL || refs(mm) != 1 || mm->dtype != CG_F32) continue;
     if (!mm->gemv_candidate && mm->rank > 3) continue;  // attention products have fusions of their own
     if (other->op == N_CONST || ((other->op == N_BIN || other->op == N_UN) && refs(other) == 1)) continue;
-    TRY(realize(be, other));
-    if (other->stype != ST_F32 || !is_contiguous(other)) return CG_OK;
     bool added = false;
-    TRY(realize_matmul(be, mm, other, &added, nullptr));
+    // (a single row in memory goes the residual's way below: every one-row kernel can add that)
+    const bool plain_row = other->op == N_REAL && other->stype == ST_F32 && is_contiguous(other);
+    if (cg_tensor *bv = (!folded && !plain_row && mm->gemv_candidate) ? bias_vector_of(other, root) : nullptr) {
+      // linear(x) + bias on a few rows: the grouped product launch adds the vector to every row
+      TRY(realize(be, bv));
+      if (!bias_vector_ready(bv)) return CG_OK;
+      be->addend_is_row = true;
+      int st = realize_matmul(be, mm, bv, &added, nullptr);
+      be->addend_is_row = false;
+      if (st) return st;
+    } else {
+      TRY(realize(be, other));
+      if (other->stype != ST_F32 || !is_contiguous(other)) return CG_OK;
+      TRY(realize_matmul(be, mm, other, &added, nullptr));
+    }
     if (!added) return CG_OK;  // the product is realised; the generic add takes it from here
     // mm now holds the sum and nobody else can see it: root takes over its storage
     root->st = mm->st;
@@ -2416,14 +2435,31 @@ int try_gemv_prologue(cg_backend *be, cg_tensor *n, cg_tensor *addend, bool *add
   d.m.b_stype = b_stype;
   double bytes = (double)rows * K * 8, flops = 0;
   int st = CG_OK;
-  for (cg_tensor *c : members) {
+  // A sibling whose only reader adds a bias vector to it: the launch stores the sum, as that add's value
+  // (the root's own bias arrives as `addend`).
+  std::vector<cg_tensor *> bias_add(members.size(), nullptr), bias_vec(members.size(), nullptr);
+  for (size_t i = 0; i < members.size(); ++i) {
+    cg_tensor *c = members[i], *add = c->bias_user;
+    if (c == n || !add || refs(c) != 1 || add->op != N_BIN || add->bias_of != c || add->size() != c->size()) continue;
+    cg_tensor *bv = bias_vector_of(add->in[add->in[0] == c ? 1 : 0], add);
+    if (!bv) continue;
+    st = realize(be, bv);
+    if (st) break;
+    if (!bias_vector_ready(bv)) continue;
+    bias_add[i] = add;
+    bias_vec[i] = bv;
+  }
+  for (size_t i = 0; i < members.size() && !st; ++i) {
+    cg_tensor *c = members[i];
     cg_tensor *w = c->in[1];
-    st = alloc_result(be, c, ST_F32);
+    cg_tensor *dest = bias_add[i] ? bias_add[i] : c;
+    st = alloc_result(be, dest, ST_F32);
     if (st) break;
     auto &pr = d.m.p[d.m.n_prob++];
     pr.b = data_ptr(w);
-    pr.c = (float *)c->st->ptr;
-    pr.c_add = (c == n && addend) ? (const float *)data_ptr(addend) : nullptr;
+    pr.c = (float *)dest->st->ptr;
+    pr.c_add = (c == n && addend) ? (const float *)data_ptr(addend) : bias_vec[i] ? (const float *)data_ptr(bias_vec[i]) : nullptr;
+    pr.c_add_is_row = (c == n && addend) ? (be->addend_is_row ? 1 : 0) : bias_vec[i] ? 1 : 0;
     pr.sbn = w->strides[w->rank - 1];
     pr.N = (uint32_t)w->shape[w->rank - 1];
     bytes += (double)pr.N * K * esize(w->stype) + (double)rows * pr.N * 4;
@@ -2445,7 +2481,12 @@ int try_gemv_prologue(cg_backend *be, cg_tensor *n, cg_tensor *addend, bool *add
   node_release(a1);
   if (st) return st;
   if (addend) *added = true;
-  for (cg_tensor *c : members) {
+  for (size_t i = 0; i < members.size(); ++i) {
+    if (bias_add[i]) {  // the add holds the value; letting go of its inputs deletes the product node
+      finish_fused(bias_add[i]);
+      continue;
+    }
+    cg_tensor *c = members[i];
     forget_gemv_candidate(c);
     c->op = N_REAL;
     drop_inputs(c);
@@ -3233,7 +3274,7 @@ int realize_matmul(cg_backend *be, cg_tensor *n, cg_tensor *addend, bool *added,
       g.sb_b1 = g.sb_b1 ? (int64_t)N * K : 0;
       g.sb_b0 = g.sb_b0 ? (int64_t)tb1 * N * K : 0;
     }
-    if (addend && M <= 8 && g.a_stype == ST_F32 && K > 0 && (g.sbk == 1 || g.sbn == 1 || K == 1 || N == 1)) {
+    if (addend && !be->addend_is_row && M <= 8 && g.a_stype == ST_F32 && K > 0 && (g.sbk == 1 || g.sbn == 1 || K == 1 || N == 1)) {
       g.c_add = (const float *)data_ptr(addend);
       *added = true;
     }
@@ -3356,7 +3397,7 @@ int realize_matmul(cg_backend *be, cg_tensor *n, cg_tensor *addend, bool *added,
       g.workspace = (float *)ws->ptr;
       g.splits = splits;
       g.k_per_split = ((K + splits - 1) / splits + 63) / 64 * 64;
-      if (addend && !g.c_add && !g.b_index) {  // the pass that sums the k-slices adds the residual too
+      if (addend && !be->addend_is_row && !g.c_add && !g.b_index) {  // the pass that sums the k-slices adds the residual too
         g.c_add = (const float *)data_ptr(addend);
         *added = true;
       }
@@ -3702,6 +3743,33 @@ bool fold_binary(EwOp op, uint32_t a, uint32_t b, uint32_t *out) {
 
 cg_tensor *const_node(cg_backend *be, cg_dtype dt, int rank, const int64_t *shape, uint32_t bits);
 
+static cg_tensor *rows_base(cg_tensor *t);
+
+// `other` adds one f32 row vector to every row of `like`'s shape: a deferred broadcast of a rank-1
+// tensor (the vector is returned), or - what a broadcast of a value already in memory is - a view
+// whose every stride but the last is zero (the view itself is returned: its first row is the
+// vector).  Null otherwise.
+cg_tensor *bias_vector_of(cg_tensor *other, const cg_tensor *like) {
+  if (other->dtype != CG_F32 || other->rank != like->rank || like->rank < 1 ||
+      !std::equal(other->shape, other->shape + other->rank, like->shape))
+    return nullptr;
+  const int r = other->rank;
+  if (other->op == N_BROADCAST) {
+    cg_tensor *v = other->in[0];
+    return v && v->rank == 1 && v->shape[0] == like->shape[r - 1] ? v : nullptr;
+  }
+  if (other->op != N_REAL || other->stype != ST_F32 || (other->shape[r - 1] != 1 && other->strides[r - 1] != 1)) return nullptr;
+  for (int i = 0; i + 1 < r; ++i)
+    if (other->shape[i] != 1 && other->strides[i] != 0) return nullptr;
+  return other;  // (with a single row, a bias and a residual are the same thing)
+}
+
+// the vector bias_vector_of returned, once realised: N contiguous f32 values at data_ptr
+bool bias_vector_ready(const cg_tensor *v) {
+  if (v->op != N_REAL || v->stype != ST_F32) return false;
+  return v->rank == 1 ? is_contiguous(v) : true;  // the view form was checked when it was recognised
+}
+
 int binary(cg_backend *be, cg_tensor *a, cg_tensor *b, cg_tensor **out, EwOp f_op, EwOp u_op) {
   TRY(check_args(be, a, b, out));
   if (!b) return fail(be, CG_ERR_ARG, "null argument");
@@ -3735,11 +3803,28 @@ int binary(cg_backend *be, cg_tensor *a, cg_tensor *b, cg_tensor **out, EwOp f_o
       if (mm->op != N_MATMUL || other->op != N_REAL) continue;
       bool dense = true;
       for (int i = 0; i < other->rank; ++i) dense = dense && (other->shape[i] == 1 || other->strides[i] != 0);
+      // a few-row product with siblings on the same rows (q/k/v, each about to get its bias) is the
+      // middle of a block: the siblings' adds are not recorded yet
+      if (dense && mm->gemv_candidate)
+        for (const cg_tensor *c : be->gemv_candidates)
+          if (c != mm && c->op == N_MATMUL && rows_base(c->in[0]) == rows_base(mm->in[0])) dense = false;
       block_end = dense;
     }
   }
+  // `linear(x) + bias` on a few rows: the product's launch can add the bias itself (try_gemv_prologue)
+  if (n->ew == E_ADD_F && !(be->flags & (CG_FLAG_EAGER | CG_FLAG_NO_PATTERNS))) {
+    for (int side = 0; side < 2; ++side) {
+      cg_tensor *mm = n->in[side], *other = n->in[1 - side];
+      if (mm->op == N_MATMUL && mm->gemv_candidate && !mm->bias_user && bias_vector_of(other, n) != nullptr) {
+        mm->bias_user = n;
+        n->bias_of = mm;
+        break;
+      }
+    }
+  }
   TRY(finish(be, n, out));
-  if (block_end && *out == n && !be->flush_node) be->flush_node = retain(n);
+  if (*out != n) return CG_OK;  // folded or shared: n is gone
+  if (block_end && !be->flush_node) be->flush_node = retain(n);
   return CG_OK;
 }
 

@@ -87,6 +87,9 @@ struct cg_tensor {
   uint32_t cbits = 0;
   bool gemv_candidate = false;  // listed in cg_backend::gemv_candidates (a weak reference)
   bool gemm_candidate = false;  // listed in cg_backend::gemm_candidates (a weak reference)
+  // `linear(x) + bias`: on a deferred few-row product, the add that reads it next to a broadcast bias
+  // vector (a weak reference, cleared when that add lets go of its inputs); on the add, the product
+  cg_tensor *bias_user = nullptr, *bias_of = nullptr;
   // a value that depends on nothing but constants and aranges (a causal mask, say); such nodes are
   // shared: cse_key is this node's entry in cg_backend::shared_nodes while it is still deferred
   bool const_like = false;
@@ -140,6 +143,9 @@ struct cg_backend {
   // a block-closing value (residual + linear over many rows) to realise at the next call, when its
   // creator has let go of the operands
   cg_tensor *flush_node = nullptr;
+  // set by try_gemv_add around realize_matmul when the addend it passes is a bias vector (one row added
+  // to every row of the product) instead of a tensor shaped like the product
+  bool addend_is_row = false;
   // recycled pinned buffers (PREFETCH_BYTES each) and events of cg_tensor_prefetch
   std::vector<void *> pinned_pool;
   std::vector<hipEvent_t> event_pool;

@@ -359,6 +359,48 @@ def _folded_linear(b, i, o, name, x):
     return lang.reshape(b, lang.make_shape(b, bb, ss, o), y)
 
 
+@pytest.mark.parametrize("rows", [1, 3])
+def test_biased_projections_of_a_decode_step(oracle, hip, hip_bf16, hip_nopat, rows):
+    """q/k/v linears with a bias (Qwen-style attention) on the normed rows of a decode step: one launch
+    that computes the norm, the three products and adds each bias vector to every row of its product."""
+    K = 512
+    g = np.random.default_rng(rows)
+    x = (g.standard_normal((rows, 1, K)) * 2).astype(np.float32)
+    p = {"n.weight": g.standard_normal(K).astype(np.float32)}
+    outs = {"q": K, "k": 128, "v": 192}
+    for name, o in outs.items():
+        p[name + ".weight"] = (g.standard_normal((o, K)) * 0.05).astype(np.float32)
+        p[name + ".bias"] = g.standard_normal(o).astype(np.float32)
+
+    def lin(b, o, name, h):
+        bb, ss, hh = lang.unpack(b, 3, lang.shape(b, h))
+        y = nn.linear(b, K, o, lang.path([name]), lang.reshape(b, lang.make_shape(b, 1, bb * ss, hh), h))
+        return lang.reshape(b, lang.make_shape(b, bb, ss, o), y)
+
+    def f(b, xv):
+        xv = xv + xv - xv
+        h = helpers.rmsnorm(b, 1e-5, lang.path(["n"]), xv)
+        return [lin(b, o, name, h) for name, o in outs.items()]
+    ref = vectors.run(oracle, f, 3, x, params=p)
+    hip.trace(True)
+    hip.trace_reset()
+    got = vectors.run(hip, f, 3, x, params=p)
+    rep = hip.trace_report()
+    hip.trace(False)
+    launches = {k: v["launches"] for k, v in rep.items()}
+    assert launches == {"ew_fused": 1, "gemv_rowdot_f32": 1}, launches      # x + x - x, then everything else
+    gen = vectors.run(hip_nopat, f, 3, x, params=p)
+    for r, a, c in zip(ref, got, gen):
+        assert a.shape == r.shape and np.allclose(a, r, rtol=1e-4, atol=1e-4), np.abs(a - r).max()
+        assert np.allclose(c, r, rtol=1e-4, atol=1e-4)
+    p16 = {k: (vectors.bf16_round(v) if v.ndim >= 2 else v) for k, v in p.items()}
+    ref16 = vectors.run(oracle, f, 3, x, params=p16)
+    got16, names16 = run_traced(hip_bf16, f, 3, x, params=p)
+    assert "binary_f32" not in names16 and "rmsnorm_fused" not in names16, sorted(names16)
+    for r, a in zip(ref16, got16):
+        assert np.max(np.abs(a - r)) <= 2e-2 * np.abs(r).max()
+
+
 @pytest.mark.parametrize("rows", [2, 3, 4])
 @pytest.mark.parametrize("act", ["silu", "gelu"])
 def test_decoder_block_of_a_small_batch(oracle, hip, hip_bf16, hip_nopat, rows, act):
