@@ -6,6 +6,7 @@
 // All HBM- or latency-bound; index moves 16 bytes per lane along the innermost axis.
 #include <hip/hip_runtime.h>
 #include "launch.hpp"
+#include "dev_common.hpp"
 
 namespace cgk {
 
@@ -123,6 +124,87 @@ __global__ void __launch_bounds__(256) topk_kernel(const float *x, float *values
       indices[(uint64_t)row * k + t] = bi;
     }
   }
+}
+
+// The router of a MoE layer (models/qwen3.rs:64-80): topk(softmax(x)) over rows of at most 256
+// logits.  One wavefront per row keeps the row in registers: the probabilities are computed exactly
+// as softmax_kernel<64, EPT> computes them (same folds, same order), then the selection rounds of
+// topk_kernel run on the registers - no launch and no [rows, n] tensor in between.
+template <int EPT>
+__global__ void __launch_bounds__(256) softmax_topk_kernel(const float *x, int64_t x_row_stride, float *values, uint32_t *indices,
+                                                           uint32_t rows, uint32_t n, uint32_t k) {
+  const uint32_t lane = threadIdx.x, row = blockIdx.x * 4 + threadIdx.y;
+  if (row >= rows) return;  // the whole wave exits together
+  const float *xr = x + (int64_t)row * x_row_stride;
+  float v[EPT];
+  float mx = -3.40282347e+38f;  // max folds from f32::MIN (ndarray.rs:455-460)
+#pragma unroll
+  for (int e = 0; e < EPT; ++e) {
+    const uint32_t c = lane + e * 64;
+    if (c < n) {
+      v[e] = xr[c];
+      mx = fmaxf(mx, v[e]);
+    }
+  }
+  mx = wave_max(mx);
+  float sum = 0.f;
+#pragma unroll
+  for (int e = 0; e < EPT; ++e) {
+    const uint32_t c = lane + e * 64;
+    if (c < n) {
+      v[e] = expf(v[e] - mx);
+      sum += v[e];
+    }
+  }
+  sum = wave_sum(sum);
+#pragma unroll
+  for (int e = 0; e < EPT; ++e) v[e] = v[e] / sum;
+  int32_t prev_key = 0;
+  uint32_t prev_idx = 0;
+  for (uint32_t t = 0; t < k; ++t) {
+    int32_t bk = 0;
+    uint32_t bi = 0xFFFFFFFFu;  // none
+    float bv = 0.f;
+#pragma unroll
+    for (int e = 0; e < EPT; ++e) {
+      const uint32_t c = lane + e * 64;
+      if (c < n) {
+        const int32_t key = total_key_f(v[e]);
+        const bool eligible = t == 0 || key < prev_key || (key == prev_key && c > prev_idx);
+        if (eligible && (bi == 0xFFFFFFFFu || key > bk || (key == bk && c < bi))) {
+          bk = key;
+          bi = c;
+          bv = v[e];
+        }
+      }
+    }
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) {
+      const int32_t ok = __shfl_xor(bk, m, 64);
+      const uint32_t oi = (uint32_t)__shfl_xor((int)bi, m, 64);
+      const float ov = __shfl_xor(bv, m, 64);
+      if (oi != 0xFFFFFFFFu && (bi == 0xFFFFFFFFu || ok > bk || (ok == bk && oi < bi))) {
+        bk = ok;
+        bi = oi;
+        bv = ov;
+      }
+    }
+    prev_key = bk;
+    prev_idx = bi;
+    if (lane == 0) {
+      values[(uint64_t)row * k + t] = bv;
+      indices[(uint64_t)row * k + t] = bi;
+    }
+  }
+}
+
+hipError_t launch_softmax_topk(const LaunchCtx &lc, const float *x, int64_t x_row_stride, float *values, uint32_t *indices,
+                               uint32_t rows, uint32_t n, uint32_t k) {
+  if (!rows || !k) return hipSuccess;
+  if (n > 256 || k > n) return hipErrorInvalidValue;
+  if (n <= 64) CG_LAUNCH(lc, (softmax_topk_kernel<1>), (rows + 3) / 4, dim3(64, 4), x, x_row_stride, values, indices, rows, n, k);
+  else CG_LAUNCH(lc, (softmax_topk_kernel<4>), (rows + 3) / 4, dim3(64, 4), x, x_row_stride, values, indices, rows, n, k);
+  return hipGetLastError();
 }
 
 hipError_t launch_topk(const LaunchCtx &lc, const float *x, float *values, uint32_t *indices,

@@ -68,6 +68,10 @@ struct GatherDesc {
 };
 hipError_t launch_gather(const LaunchCtx &lc, const GatherDesc &g, uint64_t n_out);
 // stable descending top-k per row of a contiguous [rows, n] f32 tensor
+// topk(softmax(x)) of rows of at most 256 values (row r at x + r * x_row_stride), probabilities as the softmax
+// kernel for such rows computes them
+hipError_t launch_softmax_topk(const LaunchCtx &lc, const float *x, int64_t x_row_stride, float *values, uint32_t *indices,
+                               uint32_t rows, uint32_t n, uint32_t k);
 hipError_t launch_topk(const LaunchCtx &lc, const float *x, float *values, uint32_t *indices,
                        uint32_t rows, uint32_t n, uint32_t k);
 // *flag |= 1 if any element differs (u32: bit compare, f32: IEEE ==, so NaN differs)

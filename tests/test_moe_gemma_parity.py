@@ -242,6 +242,38 @@ def test_expert_slots_over_many_tokens(oracle, hip_bf16):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("rows,n,k", [(4, 60, 4), (7, 128, 8), (1, 256, 2), (3, 64, 64), (130, 40, 5), (2, 300, 4)])
+def test_router_softmax_and_topk_in_one_launch(oracle, hip, hip_nopat, rows, n, k):
+    """topk(softmax(logits)) as a MoE router emits it (models/qwen3.rs:64-80): rows of at most 256 logits
+    take one launch that never stores the probabilities; same values as the two-launch path bit for bit,
+    the oracle's indices, and ties (equal logits) resolved towards the lower index."""
+    import vectors
+    lang, nn = vectors.lang, vectors.nn
+    g = np.random.default_rng(rows * n + k)
+    x = (g.standard_normal((rows, 1, n)) * 3).astype(np.float32)
+    x[0, 0, 5] = x[0, 0, 2] = x[0, 0].max() + 1.0          # an exact tie at the top of the first row
+
+    def f(b, xv):
+        xv = xv + xv - xv
+        return lang.topk(b, k, nn.softmax(b, xv))
+    rv, ri = vectors.run(oracle, f, 2, x)
+    hip.trace(True)
+    hip.trace_reset()
+    gv, gi = vectors.run(hip, f, 2, x)
+    rep = hip.trace_report()
+    hip.trace(False)
+    nv, ni = vectors.run(hip_nopat, f, 2, x)
+    if n <= 256:
+        assert "softmax_topk" in rep and "softmax_fused" not in rep and "topk" not in rep, sorted(rep)
+        assert np.array_equal(gv.view(np.uint32), nv.view(np.uint32)) or np.allclose(gv, nv, rtol=1e-6, atol=0)
+    else:
+        assert "softmax_topk" not in rep
+    assert np.array_equal(gi, ri) and np.array_equal(ni, ri)
+    assert gi[0, 0, 0] == 2 and gi[0, 0, 1] == 5
+    assert np.allclose(gv, rv, rtol=1e-4, atol=1e-7)
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("dev_name", ["hip", "hip_bf16"])
 @pytest.mark.parametrize("S,k", [(4, 4), (1, 2), (7, 3)])
 def test_expert_slots_of_a_decode_step(request, oracle, dev_name, S, k):
