@@ -3365,8 +3365,23 @@ int realize_matmul(cg_backend *be, cg_tensor *n, cg_tensor *addend, bool *added,
     std::vector<cg_tensor *> group;
     if (n->gemm_candidate && !addend && !ep && !ex.w && batch == 1 && g.bf16_math && g.a_stype == ST_BF16 &&
         g.b_stype == ST_BF16 && g.sbk == 1 && N % 128 == 0 && gemm_epilogue_ok(g)) {
+      // the same rows: one node, or - each linear folding the batch itself - dense reshapes of one value
+      auto dense_view = [](const cg_tensor *t, const Storage **st, int64_t *off) {
+        const cg_tensor *base = t->op == N_RESHAPE && t->in[0] ? t->in[0] : t;
+        if (base->op != N_REAL || !is_contiguous(base) || (t != base && t->size() != base->size())) return false;
+        *st = base->st;
+        *off = base->offset;
+        return true;
+      };
+      auto same_matrix = [&](const cg_tensor *a, const cg_tensor *b) {
+        if (a == b) return true;
+        const Storage *sa = nullptr, *sb = nullptr;
+        int64_t oa = 0, ob = 0;
+        return a->rank == b->rank && std::equal(a->shape, a->shape + a->rank, b->shape) && dense_view(a, &sa, &oa) &&
+               dense_view(b, &sb, &ob) && sa == sb && oa == ob;
+      };
       for (cg_tensor *c : std::vector<cg_tensor *>(be->gemm_candidates)) {
-        if (c == n || group.size() >= 2 || c->op != N_MATMUL || c->in[0] != n->in[0] || c->rank != n->rank) continue;
+        if (c == n || group.size() >= 2 || c->op != N_MATMUL || !same_matrix(c->in[0], n->in[0]) || c->rank != n->rank) continue;
         cg_tensor *w = c->in[1];
         if (w->op != N_REAL || w->rank != 3 || w->stype != ST_BF16 || w->shape[0] != 1) continue;
         if (w->shape[1] != (int64_t)K || w->strides[1] != 1 || w->strides[2] != g.sbn) continue;
@@ -3626,6 +3641,7 @@ bool share_node(cg_backend *be, cg_tensor *n, cg_tensor **out) {
   if (n->cse_key) return false;
   switch (n->op) {
     case N_BIN: case N_UN: case N_TRANSPOSE: case N_BROADCAST: case N_RESHAPE: case N_SLICE: break;
+    case N_CONCAT: break;  // the two halves of a RoPE table
     default: return false;
   }
   std::string key;

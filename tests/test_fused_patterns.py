@@ -190,6 +190,30 @@ def test_sibling_products_as_one_grouped_gemm(oracle, hip_bf16, shape):
         assert d.shape == r.shape and np.max(np.abs(d - r)) <= 2e-2 * np.abs(r).max()
 
 
+def test_sibling_products_of_a_batch_folded_per_linear(oracle, hip_bf16):
+    """bf16 mode, a batch of prompts: every linear folds the batch into the rows with a reshape of its
+    own, so q_proj, k_proj, v_proj read three nodes that are one matrix in memory; they still go out
+    as one launch."""
+    B, S, K, Ns = 4, 96, 256, (256, 128, 128)
+    g = np.random.default_rng(B * S)
+    x = vectors.bf16_round(g.standard_normal((B, S, K)).astype(np.float32))
+    p = {f"w{i}.weight": vectors.bf16_round((g.standard_normal((n, K)) * 0.05).astype(np.float32)) for i, n in enumerate(Ns)}
+
+    def f(b, xv):
+        xv = xv + xv - xv
+        return tuple(_folded_linear(b, K, n, f"w{i}", xv) for i, n in enumerate(Ns))
+    ref = vectors.run(oracle, f, 3, x, params=p)
+    hip_bf16.trace(2)
+    hip_bf16.trace_reset()
+    got = vectors.run(hip_bf16, f, 3, x, params=p)
+    rep = hip_bf16.trace_report()
+    hip_bf16.trace(False)
+    gemms = {k: v["launches"] for k, v in rep.items() if k.startswith("gemm_mfma_bf16")}
+    assert sum(gemms.values()) == 1 and "grouped" in next(iter(gemms)), gemms
+    for r, d in zip(ref, got):
+        assert d.shape == r.shape and np.max(np.abs(d - r)) <= 2e-2 * np.abs(r).max()
+
+
 @pytest.mark.parametrize("act", ["silu", "gelu"])
 @pytest.mark.parametrize("shape", [(256, 512, 1024), (200, 256, 384), (100, 192, 160), (2100, 128, 3080)])  # rows, K, N
 def test_gated_activation_in_the_gemm_epilogue(oracle, hip_bf16, shape, act):
