@@ -27,8 +27,15 @@ template <int BLOCK, int EPT>  // EPT = float4 chunks per thread
 __global__ void __launch_bounds__(BLOCK) rmsnorm_kernel(RmsNormDesc d) {
   __shared__ float lds[BLOCK / 64];
   const uint32_t row = blockIdx.x;
-  const float *x = d.x + (int64_t)row * d.x_row_stride;
-  float *y = d.y + (int64_t)row * d.n;
+  int64_t xoff;
+  if (d.x_d1 <= 1 && d.x_d2 <= 1) {
+    xoff = (int64_t)row * d.x_row_stride;
+  } else {
+    const uint32_t d2 = d.x_d2 ? d.x_d2 : 1, d1 = d.x_d1 ? d.x_d1 : 1, q = row / d2;
+    xoff = (int64_t)(q / d1) * d.x_row_stride + (int64_t)(q % d1) * d.x_s1 + (int64_t)(row % d2) * d.x_s2;
+  }
+  const float *x = d.x + xoff;
+  float *y = d.y ? d.y + (int64_t)row * d.n : nullptr;
   float4 v[EPT];
   float ss = 0.f;
 #pragma unroll
@@ -57,7 +64,7 @@ __global__ void __launch_bounds__(BLOCK) rmsnorm_kernel(RmsNormDesc d) {
         const float4 r = *(const float4 *)(d.residual + (int64_t)row * d.n + c);
         o.x += r.x; o.y += r.y; o.z += r.z; o.w += r.w;
       }
-      *(float4 *)(y + c) = o;
+      if (y) *(float4 *)(y + c) = o;
       if (d.y16) *(uint2 *)(d.y16 + (int64_t)row * d.n + c) = bf16_pack4(o);
     }
   }

@@ -99,12 +99,15 @@ hipError_t launch_peak_mfma(const LaunchCtx &lc, int bf16, float *out, unsigned 
 
 // ---- k_fused.hip
 struct RmsNormDesc {
-  const float *x;        // rows of n contiguous floats, row r at x + r * x_row_stride
+  const float *x;        // rows of n contiguous floats, row r at x + r * x_row_stride; with x_d1 or x_d2 above 1
+                         // the row index splits as ((i0 * x_d1) + i1) * x_d2 + i2 and the row sits at
+                         // x + i0 * x_row_stride + i1 * x_s1 + i2 * x_s2 (a transposed view, read in place)
   const float *gamma;    // n floats or null
   const float *residual; // contiguous [rows, n] added to the result, or null
-  uint16_t *y16;         // optional bf16 copy of y (the operand of the GEMMs that follow), or null
-  float *y;              // contiguous [rows, n]
-  int64_t x_row_stride;
+  uint16_t *y16;         // bf16 copy of y (the operand of the GEMMs that follow), or null
+  float *y;              // contiguous [rows, n]; null when only the bf16 form is wanted
+  int64_t x_row_stride, x_s1, x_s2;
+  uint32_t x_d1, x_d2;   // 0 counts as 1
   uint32_t rows, n;
   float n_as_float, eps, gamma_offset;  // gamma_offset: 0 (llama) or 1 (gemma's 1 + gamma)
 };

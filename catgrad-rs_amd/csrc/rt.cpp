@@ -861,6 +861,79 @@ bool rows_view(const cg_tensor *t, int64_t *row_stride) {
   return true;
 }
 
+// Rows of a realised f32 tensor reached through up to three (extent, stride) pairs over the row
+// index, outermost first (d0 is implied): [B, H, S, D] seen through a transpose of [B, S, H, D].
+struct RowMap {
+  uint32_t d1 = 1, d2 = 1;
+  int64_t s0 = 0, s1 = 0, s2 = 0;
+};
+bool rows_map(const cg_tensor *t, RowMap *m) {
+  if (t->op != N_REAL || t->stype != ST_F32 || t->rank == 0) return false;
+  const int r = t->rank;
+  if (t->shape[r - 1] != 1 && t->strides[r - 1] != 1) return false;
+  int64_t ext[3], str[3];
+  int g = 0;  // groups of dims that one stride walks, innermost first
+  for (int i = r - 2; i >= 0; --i) {
+    if (t->shape[i] == 1) continue;
+    if (g && t->strides[i] == str[g - 1] * ext[g - 1]) {
+      ext[g - 1] *= t->shape[i];
+      continue;
+    }
+    if (g == 3) return false;
+    ext[g] = t->shape[i];
+    str[g] = t->strides[i];
+    ++g;
+  }
+  for (int i = 0; i < g; ++i)
+    if (str[i] % 4 || ext[i] > UINT32_MAX) return false;
+  *m = RowMap();
+  if (g == 0) return true;
+  m->s0 = str[g - 1];
+  if (g == 2) {
+    m->d2 = (uint32_t)ext[0];
+    m->s2 = str[0];
+  } else if (g == 3) {
+    m->d2 = (uint32_t)ext[0];
+    m->s2 = str[0];
+    m->d1 = (uint32_t)ext[1];
+    m->s1 = str[1];
+  }
+  return true;
+}
+
+// Products still waiting that read n as their left operand, directly or through a reshape that only
+// products hold.  all: every holder of n is one of them - n is needed in its bf16 form only.
+int gemm_readers(cg_backend *be, const cg_tensor *n, bool *all) {
+  int direct = 0, via = 0;
+  const cg_tensor *seen[8];
+  int readers[8], n_seen = 0;
+  for (const cg_tensor *c : be->gemm_candidates) {
+    if (c->op != N_MATMUL || !c->in[0]) continue;
+    const cg_tensor *a = c->in[0];
+    if (a == n) {
+      ++direct;
+    } else if (a->op == N_RESHAPE && a->in[0] == n) {
+      int k = 0;
+      while (k < n_seen && seen[k] != a) ++k;
+      if (k == n_seen) {
+        if (n_seen == 8) continue;
+        seen[n_seen] = a;
+        readers[n_seen++] = 0;
+      }
+      ++readers[k];
+      ++via;
+    }
+  }
+  int holders = direct;
+  bool whole = true;
+  for (int k = 0; k < n_seen; ++k) {
+    ++holders;
+    if (readers[k] != refs(seen[k])) whole = false;
+  }
+  *all = whole && holders > 0 && holders == refs(n);
+  return direct + via;
+}
+
 // a realised f32 tensor usable as contiguous rows: itself or a contiguous copy
 int as_rows(cg_backend *be, cg_tensor *t, cg_tensor **out, int64_t *row_stride) {
   TRY(realize(be, t));
@@ -1121,18 +1194,51 @@ int try_rmsnorm(cg_backend *be, cg_tensor *root, bool *done) {
   }
   cg_tensor *xs = nullptr;
   int64_t row_stride = 0;
-  TRY(as_rows(be, x, &xs, &row_stride));
-  int st = alloc_result(be, root, ST_F32);
+  RowMap rmap;
+  // gemma3.rs:99-117 norms q and k after the head transpose, folded to [b * heads * s, head_dim]: a
+  // reshape that strides cannot express.  The rows are read where they lie instead of from a copy.
+  cg_tensor *view = x;
+  while (view->op == N_RESHAPE && view->in[0] && view->in[0]->rank >= 1 && view->in[0]->shape[view->in[0]->rank - 1] == n)
+    view = view->in[0];
+  TRY(realize(be, view));
+  if (rows_map(view, &rmap) && (rmap.d1 > 1 || rmap.d2 > 1) && (uintptr_t)data_ptr(view) % 16 == 0 &&
+      root->size() / n <= UINT32_MAX) {
+    xs = retain(view);
+    row_stride = rmap.s0;
+  } else {
+    rmap = RowMap();
+    TRY(as_rows(be, x, &xs, &row_stride));
+  }
+  // In bf16 mode with many rows: the GEMMs that wait for this value read it as bf16.  If nothing
+  // else holds it, it is written in that form only; if something else does, in both.
+  bool to_gemms = false, only_gemms = false;
+  if (!residual && (be->flags & CG_FLAG_BF16) && root->rank >= 2 && n % 8 == 0 && root->size() / n >= 32)
+    to_gemms = gemm_readers(be, root, &only_gemms) > 0;
+  int st = alloc_result(be, root, only_gemms ? ST_BF16 : ST_F32);
   if (!st) {
     d.x = (const float *)data_ptr(xs);
     d.gamma = gs ? (const float *)data_ptr(gs) : nullptr;
-    d.y = (float *)root->st->ptr;
     d.x_row_stride = row_stride;
+    d.x_d1 = rmap.d1;
+    d.x_d2 = rmap.d2;
+    d.x_s1 = rmap.s1;
+    d.x_s2 = rmap.s2;
     d.rows = (uint32_t)(root->size() / n);
     d.n = (uint32_t)n;
     d.residual = rs ? (const float *)data_ptr(rs) : nullptr;
-    if (!residual) st = twin_for_result(be, root, &d.y16);  // a residual stream feeds no GEMM directly
-    KernelScope ks(be, "rmsnorm_fused", (double)root->size() * (rs ? 12 : 8) + (d.y16 ? 2.0 * root->size() : 0.0) + n * 4, 0);
+    if (only_gemms) {
+      d.y16 = (uint16_t *)root->st->ptr;
+    } else {
+      d.y = (float *)root->st->ptr;
+      if (to_gemms) st = twin_for_result(be, root, &d.y16);
+    }
+    KernelScope ks(be, "rmsnorm_fused", (double)root->size() * ((rs ? 8 : 4) + (d.y ? 4 : 0) + (d.y16 ? 2 : 0)) + n * 4, 0);
+    if (be->trace_shapes) {  // per-shape records: rmsnorm_fused[16384x1152,+res,f32+bf16]
+      char buf[96];
+      snprintf(buf, sizeof buf, "rmsnorm_fused[%ux%u%s%s,%s]", d.rows, d.n, rs ? ",+res" : "", rmap.d1 > 1 || rmap.d2 > 1 ? ",strided" : "",
+               !d.y ? "bf16" : d.y16 ? "f32+bf16" : "f32");
+      ks.rename(buf);
+    }
     hipError_t e = launch_rmsnorm(be->lc(), d);
     if (e != hipSuccess) st = fail(be, CG_ERR_DEVICE, hipGetErrorString(e));
   }

@@ -62,6 +62,66 @@ def test_rmsnorm_of_strided_rows(oracle, hip, hip_nopat):
     check(oracle, hip, hip_nopat, f, 1, [x], "rmsnorm_fused")
 
 
+@pytest.mark.parametrize("dims", [(2, 40, 4, 64), (3, 5, 2, 256), (1, 7, 3, 32), (2, 9, 1, 64)])
+def test_rmsnorm_of_rows_behind_a_head_transpose(oracle, hip, hip_nopat, dims):
+    """gemma3.rs:99-117 norms q and k after the head transpose, folded to [b * heads * s, head_dim] - a
+    reshape that strides cannot express.  The kernel reads the rows where the projection left them;
+    nothing is copied into row-major order first."""
+    B, S, H, D = dims
+    g = np.random.default_rng(B * S + H)
+    x = (g.standard_normal((B, S, H * D)) * 2).astype(np.float32)
+    p = {"n.weight": (g.standard_normal(D) * 0.3).astype(np.float32)}
+
+    def f(b, v):
+        v = v + v - v
+        q = lang.transpose(b, 1, 2, lang.reshape(b, lang.make_shape(b, B, S, H, D), v))
+        q = lang.reshape(b, lang.make_shape(b, B * H * S, D), q)
+        gm = lang.param(b, lang.path(["n", "weight"]))
+        lr = helpers.rmsnorm_raw(b, 1e-6, lang.reshape(b, lang.make_shape(b, 1, B * H * S, D), q))
+        gm = lang.broadcast(b, gm, lang.shape(b, lr))
+        q = lr * (lang.constant(b, 1.0, lang.shape(b, gm)) + gm)
+        return lang.reshape(b, lang.make_shape(b, B, H, S, D), q)
+    check(oracle, hip, hip_nopat, f, 1, [x], "rmsnorm_fused", params=p, rtol=1e-4, atol=1e-5)
+    _, names = run_traced(hip, f, 1, x, params=p)
+    assert "ew_copy" not in names, sorted(names)
+    (ref,) = vectors.run(oracle, f, 1, x, params=p)
+    xr = x.reshape(B, S, H, D).transpose(0, 2, 1, 3).astype(np.float64)
+    want = xr / np.sqrt((xr * xr).mean(-1, keepdims=True) + 1e-6) * (1 + p["n.weight"].astype(np.float64))
+    assert np.allclose(ref, want, rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("extra_reader", [False, True])
+def test_rmsnorm_written_for_the_gemms_that_wait_for_it(oracle, hip_bf16, extra_reader):
+    """bf16 mode, many rows: a norm whose only readers are products is written as bf16 alone (the form
+    the GEMMs read); with any other reader it is written as f32 with a bf16 copy beside it."""
+    M, K, N = 192, 256, 128
+    g = np.random.default_rng(M + extra_reader)
+    x = vectors.bf16_round((g.standard_normal((1, M, K)) * 2).astype(np.float32))  # (matrices are uploaded as bf16)
+    p = {"n.weight": g.standard_normal(K).astype(np.float32)}
+    for nm in ("q", "k"):
+        p[nm + ".weight"] = vectors.bf16_round((g.standard_normal((N, K)) * 0.05).astype(np.float32))
+
+    def f(b, v):
+        v = v + v - v
+        h = helpers.rmsnorm(b, 1e-5, lang.path(["n"]), v)
+        q, k = (nn.linear_no_bias(b, K, N, lang.path([nm]), h) for nm in ("q", "k"))
+        return (q, k, h * h) if extra_reader else (q, k)
+    n_out = 3 if extra_reader else 2
+    ref = vectors.run(oracle, f, n_out, x, params=p)
+    hip_bf16.trace(2)
+    hip_bf16.trace_reset()
+    got = vectors.run(hip_bf16, f, n_out, x, params=p)
+    rep = hip_bf16.trace_report()
+    hip_bf16.trace(False)
+    norms = [k for k in rep if k.startswith("rmsnorm_fused")]
+    assert norms == [f"rmsnorm_fused[{M}x{K},{'f32+bf16' if extra_reader else 'bf16'}]"], sorted(rep)
+    assert not any(k.startswith("cast") or "narrow" in k for k in rep), sorted(rep)
+    for r, d in zip(ref[:2], got[:2]):
+        assert d.shape == r.shape and np.max(np.abs(d - r)) <= 2e-2 * np.abs(r).max()
+    if extra_reader:  # the other reader sees the f32 values
+        assert np.allclose(got[2], ref[2], rtol=1e-4, atol=1e-5)
+
+
 @pytest.mark.parametrize("shape", [(1, 32, 1, 530), (1, 4, 19, 19), (2, 3, 64, 512), (1, 2, 5, 1500),
                                    (1, 1, 3, 5000), (3, 60)])
 def test_softmax(oracle, hip, hip_nopat, shape):
