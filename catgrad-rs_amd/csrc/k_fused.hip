@@ -23,10 +23,17 @@ namespace cgk {
 // ---- rmsnorm ----------------------------------------------------------------------------------
 // y = x / sqrt(sum(x*x) / n + eps) * (gamma_offset + gamma), rows contiguous along the last axis.
 // One workgroup per row; the row lives in registers between the two phases.
-template <int BLOCK, int EPT>  // EPT = float4 chunks per thread
-__global__ void __launch_bounds__(BLOCK) rmsnorm_kernel(RmsNormDesc d) {
+// PAIR (gemma3.rs:198-240, sandwich norms): the row with its residual added is the stream the next
+// norm reads; it is written to y_mid and normed a second time (gamma2) from the registers it sits in.
+// RPW rows per workgroup: with many short rows (a prefill) a wave takes a whole row (BLOCK = 64) - no
+// barrier, no LDS - and four such waves share a workgroup.
+template <int BLOCK, int EPT, bool PAIR, int RPW = 1>  // BLOCK = threads per row, EPT = float4 chunks per thread
+__global__ void __launch_bounds__(BLOCK * RPW) rmsnorm_kernel(RmsNormDesc d) {
+  static_assert(RPW == 1 || BLOCK == 64, "several rows per workgroup: one wave each");
   __shared__ float lds[BLOCK / 64];
-  const uint32_t row = blockIdx.x;
+  const uint32_t row = blockIdx.x * RPW + (RPW > 1 ? threadIdx.x / BLOCK : 0);
+  const uint32_t tid = RPW > 1 ? threadIdx.x % BLOCK : threadIdx.x;
+  if (RPW > 1 && row >= d.rows) return;  // whole waves leave; the one-wave-per-row form has no barrier
   int64_t xoff;
   if (d.x_d1 <= 1 && d.x_d2 <= 1) {
     xoff = (int64_t)row * d.x_row_stride;
@@ -40,7 +47,7 @@ __global__ void __launch_bounds__(BLOCK) rmsnorm_kernel(RmsNormDesc d) {
   float ss = 0.f;
 #pragma unroll
   for (int e = 0; e < EPT; ++e) {
-    const uint32_t c = (threadIdx.x + e * BLOCK) * 4;
+    const uint32_t c = (tid + e * BLOCK) * 4;
     if (c < d.n) {
       v[e] = *(const float4 *)(x + c);
       ss += v[e].x * v[e].x + v[e].y * v[e].y + v[e].z * v[e].z + v[e].w * v[e].w;
@@ -49,9 +56,10 @@ __global__ void __launch_bounds__(BLOCK) rmsnorm_kernel(RmsNormDesc d) {
   ss = block_reduce<BLOCK, false>(ss, lds);
   // the reference divides by sqrt (pow(.., 0.5)); keep a true division for the 1e-4 bar
   const float rms = sqrtf(ss / d.n_as_float + d.eps);
+  float ss2 = 0.f;
 #pragma unroll
   for (int e = 0; e < EPT; ++e) {
-    const uint32_t c = (threadIdx.x + e * BLOCK) * 4;
+    const uint32_t c = (tid + e * BLOCK) * 4;
     if (c < d.n) {
       float4 o;
       o.x = v[e].x / rms; o.y = v[e].y / rms; o.z = v[e].z / rms; o.w = v[e].w / rms;
@@ -64,20 +72,56 @@ __global__ void __launch_bounds__(BLOCK) rmsnorm_kernel(RmsNormDesc d) {
         const float4 r = *(const float4 *)(d.residual + (int64_t)row * d.n + c);
         o.x += r.x; o.y += r.y; o.z += r.z; o.w += r.w;
       }
+      if (PAIR) {
+        *(float4 *)(d.y_mid + (int64_t)row * d.n + c) = o;
+        v[e] = o;
+        ss2 += o.x * o.x + o.y * o.y + o.z * o.z + o.w * o.w;
+      } else {
+        if (y) *(float4 *)(y + c) = o;
+        if (d.y16) *(uint2 *)(d.y16 + (int64_t)row * d.n + c) = bf16_pack4(o);
+      }
+    }
+  }
+  if (!PAIR) return;
+  ss2 = block_reduce<BLOCK, false>(ss2, lds);
+  const float rms2 = sqrtf(ss2 / d.n_as_float + d.eps2);
+#pragma unroll
+  for (int e = 0; e < EPT; ++e) {
+    const uint32_t c = (tid + e * BLOCK) * 4;
+    if (c < d.n) {
+      const float4 g = *(const float4 *)(d.gamma2 + c);
+      float4 o;
+      o.x = v[e].x / rms2 * (d.gamma2_offset + g.x); o.y = v[e].y / rms2 * (d.gamma2_offset + g.y);
+      o.z = v[e].z / rms2 * (d.gamma2_offset + g.z); o.w = v[e].w / rms2 * (d.gamma2_offset + g.w);
       if (y) *(float4 *)(y + c) = o;
       if (d.y16) *(uint2 *)(d.y16 + (int64_t)row * d.n + c) = bf16_pack4(o);
     }
   }
 }
 
+template <bool PAIR>
+static void launch_rmsnorm_as(const LaunchCtx &lc, const RmsNormDesc &d) {
+  // n % 4 == 0 and n <= 16384 are checked by the caller
+  if (d.rows >= 2048 && d.n <= 2048) {  // a wave per row, four rows per workgroup
+    const uint32_t wgs = (d.rows + 3) / 4;
+    if (d.n <= 256) CG_LAUNCH(lc, (rmsnorm_kernel<64, 1, PAIR, 4>), wgs, 256, d);
+    else if (d.n <= 512) CG_LAUNCH(lc, (rmsnorm_kernel<64, 2, PAIR, 4>), wgs, 256, d);
+    else if (d.n <= 1024) CG_LAUNCH(lc, (rmsnorm_kernel<64, 4, PAIR, 4>), wgs, 256, d);
+    else if (d.n <= 1280) CG_LAUNCH(lc, (rmsnorm_kernel<64, 5, PAIR, 4>), wgs, 256, d);
+    else CG_LAUNCH(lc, (rmsnorm_kernel<64, 8, PAIR, 4>), wgs, 256, d);
+    return;
+  }
+  if (d.n <= 256) CG_LAUNCH(lc, (rmsnorm_kernel<64, 1, PAIR>), d.rows, 64, d);
+  else if (d.n <= 1024) CG_LAUNCH(lc, (rmsnorm_kernel<256, 1, PAIR>), d.rows, 256, d);
+  else if (d.n <= 2048) CG_LAUNCH(lc, (rmsnorm_kernel<256, 2, PAIR>), d.rows, 256, d);
+  else if (d.n <= 4096) CG_LAUNCH(lc, (rmsnorm_kernel<256, 4, PAIR>), d.rows, 256, d);
+  else CG_LAUNCH(lc, (rmsnorm_kernel<1024, 4, PAIR>), d.rows, 1024, d);
+}
+
 hipError_t launch_rmsnorm(const LaunchCtx &lc, const RmsNormDesc &d) {
   if (!d.rows || !d.n) return hipSuccess;
-  // n % 4 == 0 and n <= 16384 are checked by the caller
-  if (d.n <= 256) CG_LAUNCH(lc, (rmsnorm_kernel<64, 1>), d.rows, 64, d);
-  else if (d.n <= 1024) CG_LAUNCH(lc, (rmsnorm_kernel<256, 1>), d.rows, 256, d);
-  else if (d.n <= 2048) CG_LAUNCH(lc, (rmsnorm_kernel<256, 2>), d.rows, 256, d);
-  else if (d.n <= 4096) CG_LAUNCH(lc, (rmsnorm_kernel<256, 4>), d.rows, 256, d);
-  else CG_LAUNCH(lc, (rmsnorm_kernel<1024, 4>), d.rows, 1024, d);
+  if (d.y_mid) launch_rmsnorm_as<true>(lc, d);
+  else launch_rmsnorm_as<false>(lc, d);
   return hipGetLastError();
 }
 

@@ -110,6 +110,11 @@ struct RmsNormDesc {
   uint32_t x_d1, x_d2;   // 0 counts as 1
   uint32_t rows, n;
   float n_as_float, eps, gamma_offset;  // gamma_offset: 0 (llama) or 1 (gemma's 1 + gamma)
+  // Two norms in a row (non-null y_mid): the first result (with its residual) goes to y_mid, contiguous
+  // [rows, n], and is normed again with gamma2 (n floats, not null) into y / y16.
+  float *y_mid;
+  const float *gamma2;
+  float eps2, gamma2_offset;
 };
 hipError_t launch_rmsnorm(const LaunchCtx &lc, const RmsNormDesc &d);
 

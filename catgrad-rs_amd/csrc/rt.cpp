@@ -1151,6 +1151,80 @@ int gamma_row_vector(cg_backend *be, cg_tensor *gb, bool *ok) {
   return CG_OK;
 }
 
+// gemma3.rs:198-240, many rows: `mid = res + rmsnorm(y)` followed by `rmsnorm(mid)` - the post-attention
+// norm and the pre-feedforward one, the post-feedforward norm and the next layer's input norm.  One
+// kernel writes mid (the residual stream, which later adds read) and norms it again from registers.
+int try_rmsnorm_pair(cg_backend *be, cg_tensor *root, const RmsNormMatch &outer, bool *done) {
+  cg_tensor *mid = outer.x;
+  const int64_t n = root->shape[root->rank - 1];
+  if (!mid || mid->op == N_REAL || mid->dtype != CG_F32 || !is_bin(mid, E_ADD_F) || !outer.gamma || mid->size() != root->size() ||
+      root->size() / n < 32 || root->size() / n > UINT32_MAX)
+    return CG_OK;
+  RmsNormMatch inner;
+  int side = -1;
+  for (int i = 0; i < 2 && side < 0; ++i)
+    if (mid->in[i]->op != N_REAL && refs(mid->in[i]) == 1 && match_rmsnorm(mid->in[i], &inner)) side = i;
+  if (side < 0 || !inner.gamma || inner.n_as_float != outer.n_as_float) return CG_OK;
+  cg_tensor *residual = mid->in[1 - side];
+  if (residual->op == N_CONST || ((residual->op == N_BIN || residual->op == N_UN) && refs(residual) == 1)) return CG_OK;
+  bool v1 = false, v2 = false;
+  TRY(gamma_row_vector(be, inner.gamma, &v1));
+  TRY(gamma_row_vector(be, outer.gamma, &v2));
+  if (!v1 || !v2) return CG_OK;
+  cg_tensor *rs = nullptr, *xs = nullptr;
+  struct Rel {
+    cg_tensor *&t;
+    ~Rel() { node_release(t); }
+  } rel_rs{rs}, rel_xs{xs};
+  // the normed value first: what it is computed from (a layer's feed-forward) reads the norm of the
+  // residual stream, and that norm pairs up with the one that produces the stream only while the
+  // stream is still unwritten
+  int64_t row_stride = 0;
+  TRY(as_rows(be, inner.x, &xs, &row_stride));
+  if (mid->op == N_REAL || root->op == N_REAL) return CG_OK;
+  TRY(contiguous(be, residual, &rs));
+  if ((uintptr_t)data_ptr(rs) % 16) return CG_OK;
+  bool to_gemms = false, only_gemms = false;
+  if ((be->flags & CG_FLAG_BF16) && root->rank >= 2 && n % 8 == 0) to_gemms = gemm_readers(be, root, &only_gemms) > 0;
+  TRY(alloc_result(be, mid, ST_F32));
+  TRY(alloc_result(be, root, only_gemms ? ST_BF16 : ST_F32));
+  RmsNormDesc d;
+  std::memset(&d, 0, sizeof(d));
+  d.x = (const float *)data_ptr(xs);
+  d.x_row_stride = row_stride;
+  d.gamma = (const float *)data_ptr(inner.gamma);
+  d.eps = inner.eps;
+  d.gamma_offset = inner.gamma_offset;
+  d.n_as_float = inner.n_as_float;
+  d.residual = (const float *)data_ptr(rs);
+  d.y_mid = (float *)mid->st->ptr;
+  d.gamma2 = (const float *)data_ptr(outer.gamma);
+  d.eps2 = outer.eps;
+  d.gamma2_offset = outer.gamma_offset;
+  d.rows = (uint32_t)(root->size() / n);
+  d.n = (uint32_t)n;
+  if (only_gemms) {
+    d.y16 = (uint16_t *)root->st->ptr;
+  } else {
+    d.y = (float *)root->st->ptr;
+    if (to_gemms) TRY(twin_for_result(be, root, &d.y16));
+  }
+  {
+    KernelScope ks(be, "rmsnorm_fused", (double)root->size() * (12 + (d.y ? 4 : 0) + (d.y16 ? 2 : 0)) + n * 8, 0);
+    if (be->trace_shapes) {  // rmsnorm_fused[16384x1152,+res,+norm,bf16]
+      char buf[96];
+      snprintf(buf, sizeof buf, "rmsnorm_fused[%ux%u,+res,+norm,%s]", d.rows, d.n, !d.y ? "bf16" : d.y16 ? "f32+bf16" : "f32");
+      ks.rename(buf);
+    }
+    hipError_t e = launch_rmsnorm(be->lc(), d);
+    if (e != hipSuccess) return fail(be, CG_ERR_DEVICE, hipGetErrorString(e));
+  }
+  finish_fused(mid);
+  finish_fused(root);
+  *done = true;
+  return CG_OK;
+}
+
 // also `res + rmsnorm(..)` / `rmsnorm(..) + res` (gemma3.rs:198-240 adds the residual right after the
 // post-attention and post-feedforward norms): the addend rides along in the same kernel
 int try_rmsnorm(cg_backend *be, cg_tensor *root, bool *done) {
@@ -1165,6 +1239,10 @@ int try_rmsnorm(cg_backend *be, cg_tensor *root, bool *done) {
     residual = root->in[1 - side];
     if (residual->op == N_CONST || ((residual->op == N_BIN || residual->op == N_UN) && refs(residual) == 1))
       return CG_OK;  // the addend is itself an unrealised expression: leave it to the generic fusion
+  }
+  if (!residual) {
+    TRY(try_rmsnorm_pair(be, root, rm, done));
+    if (*done) return CG_OK;
   }
   cg_tensor *x = rm.x, *gb = rm.gamma;
   const int64_t n = root->shape[root->rank - 1];

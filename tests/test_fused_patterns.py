@@ -30,7 +30,10 @@ def check(oracle, hip, hip_nopat, fn, n_out, arrays, kernel, params=None, rtol=1
         assert np.allclose(h, r, rtol=rtol, atol=atol), np.abs(h - r).max()
 
 
-@pytest.mark.parametrize("shape", [(1, 1, 2048), (1, 7, 64), (2, 33, 1152), (1, 3, 8192), (5, 16)])
+@pytest.mark.parametrize("shape", [(1, 1, 2048), (1, 7, 64), (2, 33, 1152), (1, 3, 8192), (5, 16),
+                                   # thousands of rows: a wave per row, several rows per workgroup
+                                   (1, 2050, 1152), (2, 1025, 256), (1, 2049, 2048), (1, 2051, 512), (1, 2048, 1024),
+                                   (1, 2053, 64), (1, 2049, 2052)])
 def test_rmsnorm(oracle, hip, hip_nopat, shape):
     g = np.random.default_rng(sum(shape))
     x = (g.standard_normal(shape) * 3).astype(np.float32)
@@ -62,7 +65,7 @@ def test_rmsnorm_of_strided_rows(oracle, hip, hip_nopat):
     check(oracle, hip, hip_nopat, f, 1, [x], "rmsnorm_fused")
 
 
-@pytest.mark.parametrize("dims", [(2, 40, 4, 64), (3, 5, 2, 256), (1, 7, 3, 32), (2, 9, 1, 64)])
+@pytest.mark.parametrize("dims", [(2, 40, 4, 64), (3, 5, 2, 256), (1, 7, 3, 32), (2, 9, 1, 64), (2, 301, 4, 64)])
 def test_rmsnorm_of_rows_behind_a_head_transpose(oracle, hip, hip_nopat, dims):
     """gemma3.rs:99-117 norms q and k after the head transpose, folded to [b * heads * s, head_dim] - a
     reshape that strides cannot express.  The kernel reads the rows where the projection left them;
@@ -547,6 +550,47 @@ def test_rmsnorm_plus_residual(oracle, hip, hip_nopat, shape, order):
         h = raw * (lang.constant(b, 1.0, lang.shape(b, gm)) + gm)
         return rv + h if order == "res_first" else h + rv
     check(oracle, hip, hip_nopat, f, 1, [x, res], "rmsnorm_fused", params=p, rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize("shape", [(2, 33, 1152), (1, 40, 64), (4, 64, 256), (1, 7, 64), (1, 2050, 1152), (2, 1027, 640)])
+def test_two_norms_around_a_residual_add(oracle, hip, hip_bf16, hip_nopat, shape):
+    """gemma3.rs:198-240: `mid = res + norm(y)` and right after it `norm(mid)` (post-attention and
+    pre-feedforward norms; post-feedforward and the next layer's input norm).  With many rows one
+    launch writes mid and norms it again; a later reader of mid (the next residual add) finds it in
+    memory."""
+    g = np.random.default_rng(shape[1] + shape[2])
+    y = (g.standard_normal(shape) * 2).astype(np.float32)
+    res = g.standard_normal(shape).astype(np.float32)
+    p = {"a.weight": (g.standard_normal(shape[-1]) * 0.1).astype(np.float32),
+         "b.weight": (g.standard_normal(shape[-1]) * 0.1).astype(np.float32)}
+
+    def gemma_norm(b, name, v):
+        gm = lang.param(b, lang.path([name, "weight"]))
+        raw = helpers.rmsnorm_raw(b, 1e-6, v)
+        gm = lang.broadcast(b, gm, lang.shape(b, raw))
+        return raw * (lang.constant(b, 1.0, lang.shape(b, gm)) + gm)
+
+    def f(b, yv, rv):
+        yv = yv + yv - yv
+        mid = rv + gemma_norm(b, "a", yv)
+        h = gemma_norm(b, "b", mid)
+        return h, mid + h
+    ref = vectors.run(oracle, f, 2, y, res, params=p)
+    hip.trace(True)
+    hip.trace_reset()
+    got = vectors.run(hip, f, 2, y, res, params=p)
+    rep = hip.trace_report()
+    hip.trace(False)
+    gen = vectors.run(hip_nopat, f, 2, y, res, params=p)
+    many = shape[0] * shape[1] >= 32
+    assert rep["rmsnorm_fused"]["launches"] == (1 if many else 2), {k: v["launches"] for k, v in rep.items()}
+    for r, a, c in zip(ref, got, gen):
+        assert np.allclose(a, r, rtol=1e-4, atol=1e-5), np.abs(a - r).max()
+        assert np.allclose(c, r, rtol=1e-4, atol=1e-5)
+    got16 = vectors.run(hip_bf16, f, 2, vectors.bf16_round(y), vectors.bf16_round(res), params=p)
+    ref16 = vectors.run(oracle, f, 2, vectors.bf16_round(y), vectors.bf16_round(res), params=p)
+    for r, a in zip(ref16, got16):
+        assert np.max(np.abs(a - r)) <= 2e-2 * np.abs(r).max()
 
 
 @pytest.fixture(scope="module")
