@@ -712,6 +712,11 @@ int launch_compiled(cg_backend *be, EwCompiler &c, cg_tensor *root, void *dst,
     return CG_OK;
   }
   KernelScope ks(be, name, bytes_in + (double)n * esize(dst_stype), 0);
+  if (be->trace_shapes) {  // per-shape records: ew_fused[n8192,i7,in3]
+    char buf[96];
+    snprintf(buf, sizeof buf, "%s[n%lld,i%d,in%d]", name, (long long)n, (int)c.p.n_instr, (int)c.p.n_in);
+    ks.rename(buf);
+  }
   HIPCHK(be, launch_ew(be->lc(), c.p, o, (uint64_t)n, vec4));
   return CG_OK;
 }
