@@ -468,7 +468,7 @@ __global__ void __launch_bounds__(256) gemm_bf16_nt_kernel(GemmDesc g) {
 // s and complete under its MFMAs; the compiler does not know the asm writes LDS, so the waits
 // are explicit (s_waitcnt vmcnt + barrier before the stage is read).  Rows past M / N are
 // clamped on the load side and masked at the store.  Fragment reads of k-slice ks+1 are issued
-// before the MFMAs of slice ks (sched_barrier keeps the order).
+// among the MFMAs of slice ks, one read behind each of the first MFMAs (sched_group_barrier).
 __device__ __forceinline__ void lds_dma16(const void *gptr, uint32_t lds_byte_off) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_byte_off), "v"(gptr)
                : "memory", "m0");
@@ -587,12 +587,23 @@ __global__ void __launch_bounds__(WR *WC * 64) gemm_bf16_dma_kernel(GemmDesc g) 
 #pragma unroll
     for (int ks = 0; ks < BK / 16; ++ks) {
       if (ks + 1 < BK / 16) frags(ks + 1, (ks + 1) & 1);
-      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[ks & 1][i], bfr[ks & 1][j], acc[i][j], 0, 0, 0);
+      // Issue order within the slice: one LDS read behind each of the first MFMAs, so that the reads of
+      // the next slice go out while the matrix pipe is busy instead of in a block during which it drains
+      // (measured on 4096^3: 0.93 -> 1.06 PFLOP/s).
+      if (ks + 1 < BK / 16) {
+        constexpr int READS = TM + TN < TM * TN ? TM + TN : TM * TN;
+#pragma unroll
+        for (int q = 0; q < READS; ++q) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one LDS read
+        }
+        if (TM * TN > READS) __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - READS, 0);
+      }
       __builtin_amdgcn_sched_barrier(0);
     }
   };
