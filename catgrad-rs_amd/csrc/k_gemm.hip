@@ -584,6 +584,8 @@ __global__ void __launch_bounds__(WR *WC * 64) gemm_bf16_dma_kernel(GemmDesc g) 
       }
     };
     frags(0, 0);
+    // the wave that is in its MFMA phase goes first when both waves of a SIMD have something to issue
+    __builtin_amdgcn_s_setprio(1);
 #pragma unroll
     for (int ks = 0; ks < BK / 16; ++ks) {
       if (ks + 1 < BK / 16) frags(ks + 1, (ks + 1) & 1);
@@ -606,6 +608,7 @@ __global__ void __launch_bounds__(WR *WC * 64) gemm_bf16_dma_kernel(GemmDesc g) 
       }
       __builtin_amdgcn_sched_barrier(0);
     }
+    __builtin_amdgcn_s_setprio(0);
   };
   const int n_steps = k_end > k_begin ? (int)((k_end - k_begin) / BK) : 0;
 #pragma unroll
