@@ -167,7 +167,8 @@ int cg_to_u32(cg_backend *be, cg_tensor *x, uint32_t *dst, size_t n);
 /* ---- tracing (no counterpart in the reference) -------------------------------------
  * When enabled every kernel launch is bracketed by two events on the backend's stream.
  * cg_trace_report writes one line per kernel name: "name launches total_ms bytes flops".
- * on = 2 additionally keys matmul records by problem shape ("gemm_mfma_bf16[b1,512x2048x2048,s4]").
+ * on = 2 additionally keys the records of matmuls, RMSNorms and elementwise programs by problem shape
+ * ("gemm_mfma_bf16[b1,512x2048x2048,s4]", "rmsnorm_fused[16384x1152,+res,+norm,bf16]", "ew_fused[n8192,i5,in3]").
  */
 int cg_trace_enable(cg_backend *be, int on);
 /* Peak probes (no counterpart in the reference): what this device gives a plain 16-byte grid-stride
