@@ -1186,7 +1186,11 @@ int try_rmsnorm_pair(cg_backend *be, cg_tensor *root, const RmsNormMatch &outer,
   // stream is still unwritten
   int64_t row_stride = 0;
   TRY(as_rows(be, inner.x, &xs, &row_stride));
-  if (mid->op == N_REAL || root->op == N_REAL) return CG_OK;
+  if (root->op == N_REAL) {  // (realised on the way: nothing left to do)
+    *done = true;
+    return CG_OK;
+  }
+  if (mid->op == N_REAL) return CG_OK;
   TRY(contiguous(be, residual, &rs));
   if ((uintptr_t)data_ptr(rs) % 16) return CG_OK;
   bool to_gemms = false, only_gemms = false;
