@@ -80,6 +80,7 @@ _SIGNATURES = {
     "cg_broadcast": (C.c_int, [_P, _P, _SZP, C.c_int, _PP]),
     "cg_reshape": (C.c_int, [_P, _P, _SZP, C.c_int, _PP]),
     "cg_transpose": (C.c_int, [_P, _P, _SZ, _SZ, _PP]),
+    "cg_argmax_into": (C.c_int, [_P, _P, _P]),
     "cg_topk": (C.c_int, [_P, _P, _SZ, _PP, _PP]),
     "cg_compare": (C.c_int, [_P, _P, _P, C.POINTER(C.c_int)]),
     "cg_concat": (C.c_int, [_P, _P, _P, _SZ, _PP]),
@@ -285,6 +286,11 @@ class Backend:
 
     def transpose(self, x, dim0, dim1):
         return self._out(self.lib.cg_transpose, x.ptr, dim0, dim1)
+
+    def argmax_into(self, x, out):
+        """argmax of `x` into the tensor `out` (both already in memory); allocates nothing."""
+        self._check(self.lib.cg_argmax_into(self.ptr, x.ptr, out.ptr))
+        return out
 
     def topk(self, x, k):
         v, i = C.c_void_p(), C.c_void_p()

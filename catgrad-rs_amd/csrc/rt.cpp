@@ -4148,6 +4148,38 @@ int download(cg_backend *be, cg_tensor *x, void *dst, size_t n, cg_dtype want) {
 
 }  // namespace
 
+namespace cgrt {
+
+// The generic (program-prologue) path of realize_reduce on memory the caller brings: `x` and `out` are
+// realised tensors, `scratch` receives the per-chunk accumulators when the rows are split over several
+// workgroups (3 words per chunk).  Calls no allocator; traced launches are not recorded.
+int reduce_into(cg_backend *be, int kind, cg_tensor *x, cg_tensor *out, uint32_t *scratch, size_t scratch_bytes) {
+  Region reg;
+  EwCompiler c(be, &reg);
+  TRY(c.load(c.final_code, x, 0));
+  c.flatten();
+  std::vector<int64_t> ostr;
+  TRY(finish_program(be, c, x->rank, x->shape, nullptr, true, ostr, nullptr));
+  const int64_t cols = x->shape[x->rank - 1];
+  const int64_t rows = x->size() / cols;
+  const uint32_t chunks = reduce_split_chunks(be->lc(), (uint32_t)rows, (uint32_t)cols);
+  if (chunks > 1 && (size_t)rows * chunks * 3 * 4 > scratch_bytes)
+    return fail(be, CG_ERR_ARG, "reduction of " + std::to_string(rows) + " rows in " + std::to_string(chunks) +
+                                    " chunks needs " + std::to_string((size_t)rows * chunks * 12) +
+                                    " bytes of scratch, above the fixed " + std::to_string(scratch_bytes));
+  be->launches++;
+  LaunchCtx lc = be->lc();
+  lc.ev_start = lc.ev_stop = nullptr;
+  HIPCHK(be, launch_reduce(lc, kind, c.p, data_ptr(out), (uint32_t)rows, (uint32_t)cols, cols % 4 == 0 && cols >= 4,
+                           chunks > 1 ? scratch : nullptr, chunks));
+  return CG_OK;
+}
+
+int fail_with(cg_backend *be, int code, const std::string &msg) { return fail(be, code, msg); }
+bool tensor_is_contiguous(const cg_tensor *t) { return is_contiguous(t); }
+
+}  // namespace cgrt
+
 extern "C" {
 
 int cg_backend_create(int device, uint32_t flags, cg_backend **out) {
@@ -4158,6 +4190,7 @@ int cg_backend_create(int device, uint32_t flags, cg_backend **out) {
     return CG_ERR_DEVICE;
   }
   if (hipSetDevice(device) != hipSuccess) return CG_ERR_DEVICE;
+  if (cgrt::noalloc_init_device(device) != CG_OK) return CG_ERR_DEVICE;
   cg_backend *be = new cg_backend();
   be->device = device;
   be->flags = flags;

@@ -66,6 +66,14 @@ struct PendingEvent {
   double bytes, flops;
 };
 
+// ---- shared with noalloc.cpp -------------------------------------------------------------------
+// Resolves, once per device and with that device current, the address of the library's fixed scratch
+// array; cg_backend_create calls it.
+int noalloc_init_device(int device);
+int reduce_into(cg_backend *be, int kind, cg_tensor *x, cg_tensor *out, uint32_t *scratch, size_t scratch_bytes);
+int fail_with(cg_backend *be, int code, const std::string &msg);
+bool tensor_is_contiguous(const cg_tensor *t);
+
 }  // namespace cgrt
 
 struct cg_tensor {

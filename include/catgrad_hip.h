@@ -150,6 +150,16 @@ int cg_transpose(cg_backend *be, cg_tensor *x, size_t dim0, size_t dim1, cg_tens
 int cg_max(cg_backend *be, cg_tensor *x, cg_tensor **out);
 int cg_sum(cg_backend *be, cg_tensor *x, cg_tensor **out);
 int cg_argmax(cg_backend *be, cg_tensor *x, cg_tensor **out);
+/* cg_argmax into memory the caller brings.  No counterpart in the reference: it is for callers that
+ * cannot allocate device memory (code under HIP graph capture, serving loops with a fixed footprint,
+ * harnesses that forbid hipMalloc).  `x` must already be in memory (an uploaded tensor, or one passed
+ * through cg_tensor_realize) and `out` a contiguous U32 tensor in memory shaped like x with a last
+ * axis of 1; both stay the caller's.  The call makes no hipMalloc / hipFree and creates no handle: the
+ * per-chunk accumulators of long rows that are split over workgroups go to a fixed 16 KiB array in the
+ * library's device image (12 bytes per row and chunk; a shape needing more is refused with
+ * CG_ERR_ARG).  Each GPU has one such array, shared by every backend on it and holding the last
+ * call's contents: calls that overlap on one GPU race. */
+int cg_argmax_into(cg_backend *be, cg_tensor *x, cg_tensor *out);
 /* topk (mod.rs:58, ndarray.rs:248-257, 495-520): f32 only; values f32, indices u32 */
 int cg_topk(cg_backend *be, cg_tensor *x, size_t k, cg_tensor **values, cg_tensor **indices);
 /* compare (mod.rs:59, ndarray.rs:337-343): *equal = 1 iff same shape and all elements == */

@@ -541,6 +541,19 @@ int cg_argmax(cg_backend *be, cg_tensor *x, cg_tensor **out) {
   return CG_OK;
 }
 
+// cg_argmax into a tensor the caller brings (the product's entry point for callers that cannot allocate);
+// here only so that both libraries export one ABI
+int cg_argmax_into(cg_backend *be, cg_tensor *x, cg_tensor *out) {
+  if (!x || !out) return fail(be, CG_ERR_ARG, "null argument");
+  cg_tensor *t = nullptr;
+  if (int e = cg_argmax(be, x, &t)) return e;
+  int st = CG_OK;
+  if (out->dtype != CG_U32 || out->shape != t->shape) st = fail(be, CG_ERR_SHAPE, "cg_argmax_into: out must be U32 and shaped like x with a last axis of 1");
+  else out->bits = t->bits;
+  cg_tensor_release(t);
+  return st;
+}
+
 // ndarray.rs:495-520: stable sort of the indices by descending total_cmp, take k
 int cg_topk(cg_backend *be, cg_tensor *x, size_t k, cg_tensor **values, cg_tensor **indices) {
   if (x->dtype != CG_F32) return fail(be, CG_ERR_DTYPE, "Unsupported type for topk");
