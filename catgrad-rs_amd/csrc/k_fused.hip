@@ -518,22 +518,31 @@ __global__ void __launch_bounds__(256) attn_decode_split_kernel(AttnDecodeDesc a
       a.out[((uint64_t)b * a.heads + h) * a.d + tid] = o / L;
       return;
     }
-    // agent-scope stores go through to where every compute unit sees them; no cache write-back
-    // or invalidation is needed around the counter below
+    // The hand-over to the merging workgroup (another compute unit, usually another XCD).  A release
+    // fence at agent scope would do it by the book, but it also writes back every dirty line of this
+    // XCD's L2 (5 us per launch, measured); the partials need less.  They are agent-scope atomic
+    // stores, which go through to the level every compute unit reads from, and a wave's vmcnt only
+    // counts such a store down once it has been acknowledged from there.  So: every wave waits for its
+    // own stores, then the barrier, and only then does thread 0 move the counter - no workgroup can
+    // find the counter at splits - 1 before all the partials of the other splits have landed.
     __hip_atomic_store(mine + 2 + tid, o, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     if (tid == 0) {
       __hip_atomic_store(mine, M, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       __hip_atomic_store(mine + 1, L, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   }
   if (a.splits == 1) return;
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // the stores above have completed ...
-  __syncthreads();                                        // ... in every wave before the counter moves
+  __syncthreads();
   uint32_t *counter = a.count + (uint64_t)b * a.heads + h;
   if (tid == 0)
     last_flag = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == a.splits - 1 ? 1u : 0u;
   __syncthreads();
   if (!last_flag) return;
+  // The merging side: its loads of the partials are issued after the counter's value came back (the
+  // branch above depends on it, and the compiler may not move atomic loads above the barrier), and
+  // they are agent-scope atomic loads, which are served from the level the stores went through to,
+  // never from this compute unit's own caches.
   const float *base = a.part + ((uint64_t)b * a.heads + h) * a.splits * pw;
   if ((uint32_t)tid < a.splits) {
     cm[tid] = __hip_atomic_load(base + tid * pw, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

@@ -63,6 +63,24 @@ void trim_pool(cg_backend *be) {
   be->pool_bytes = 0;
 }
 
+// Called at synchronisation points (the stream is idle): a long run over changing sizes would otherwise
+// keep every block it ever freed.  Above POOL_CAP of cached blocks the largest size classes go back to
+// the driver until the pool is under half the cap; the working set of a steady loop (the same sizes
+// every step) stays far below it and is never touched.
+void cap_pool(cg_backend *be) {
+  const uint64_t POOL_CAP = (uint64_t)32 << 30;
+  if (be->pool_bytes <= POOL_CAP) return;
+  for (auto it = be->pool.rbegin(); it != be->pool.rend() && be->pool_bytes > POOL_CAP / 2; ++it) {
+    std::vector<void *> &blocks = it->second;
+    while (!blocks.empty() && be->pool_bytes > POOL_CAP / 2) {
+      (void)hipFree(blocks.back());
+      blocks.pop_back();
+      be->pool_bytes -= it->first;
+      be->device_bytes -= it->first;
+    }
+  }
+}
+
 int dev_alloc(cg_backend *be, size_t bytes, Storage **out) {
   const size_t cls = size_class(bytes);
   void *p = nullptr;
@@ -2231,6 +2249,12 @@ int attn_decode_scratch(cg_backend *be, size_t part_floats, size_t count_words) 
 
 // The cache update of a decode step, `concat(2, cached, new)` (legacy/models/utils.rs:222-223), seen
 // from the attention that reads it: the node under the repeat_kv chain of a K or V operand.
+// `x` (realised) walks its storage exactly as the tensor the storage's spare room was laid out for
+bool has_grow_layout(const cg_tensor *x) {
+  const Storage *s = x->st;
+  return s && x->rank == s->grow_rank && std::equal(x->strides, x->strides + x->rank, s->grow_strides);
+}
+
 cg_tensor *kv_concat_under(cg_tensor *t) {
   if (t->op == N_TRANSPOSE && refs(t) == 1 && t->rank == 4 &&
       ((t->p0 == 2 && t->p1 == 3) || (t->p0 == 3 && t->p1 == 2)))
@@ -2267,7 +2291,7 @@ int row_append_candidate(cg_backend *be, cg_tensor *c, bool allow_rope, RowAppen
   TRY(realize(be, x));
   const int64_t xd = x->shape[2];
   if (!(refs(x) == 1 && x->st->rc.load() == 1 && x->st->grow_dim == 2 && xd + 1 <= x->st->grow_cap &&
-        x->offset == 0 && x->stype == ST_F32))
+        x->offset == 0 && x->stype == ST_F32 && has_grow_layout(x)))
     return CG_OK;
   if (x->strides[3] != 1 || x->strides[0] % 4 || x->strides[1] % 4 || x->strides[2] % 4 ||
       (uintptr_t)data_ptr(x) % 16)
@@ -2310,6 +2334,35 @@ void commit_row_append(cg_tensor *c) {
   drop_inputs(c);
 }
 
+// The rows of a committed append written by kernels of their own: what is left to do when the attention
+// kernel that was to store them cannot be launched after all.
+int write_row_append(cg_backend *be, const RowAppend &ra) {
+  cg_tensor *c = ra.concat, *src = ra.src;
+  float *dst = (float *)c->st->ptr + (c->shape[2] - 1) * c->strides[2];
+  if (!ra.cos) return run_ew(be, src, true, dst, c->strides, ST_F32, "kv_append");
+  RopeDesc d;
+  std::memset(&d, 0, sizeof(d));
+  d.x = (const float *)data_ptr(src);
+  d.cos = ra.cos;
+  d.sin = ra.sin;
+  d.out = dst;
+  d.x_sb = src->strides[0];
+  d.x_sh = src->strides[1];
+  d.x_ss = src->strides[2];
+  d.o_sb = c->strides[0];
+  d.o_sh = c->strides[1];
+  d.o_ss = c->strides[2];
+  d.cs_ss = 0;  // one position
+  d.b = (uint32_t)c->shape[0];
+  d.h = (uint32_t)c->shape[1];
+  d.s = 1;
+  d.dim = (uint32_t)c->shape[3];
+  d.half = d.dim / 2;
+  KernelScope ks(be, "rope_kv_append", (double)d.b * d.h * d.dim * 8, 0);
+  HIPCHK(be, launch_rope(be->lc(), d));
+  return CG_OK;
+}
+
 int try_attn_decode(cg_backend *be, cg_tensor *n, bool *done) {
   cg_tensor *P = n->in[0];
   if (P->op == N_REAL || refs(P) != 1 || P->rank != 4) return CG_OK;
@@ -2337,11 +2390,16 @@ int try_attn_decode(cg_backend *be, cg_tensor *n, bool *done) {
       }
     }
   }
-  // from here on a fused append must end in the launch: its rows exist nowhere else
-#define ATTN_BAIL()                                                                            \
-  do {                                                                                         \
-    if (fused_append) return fail(be, CG_ERR_INTERNAL, "attention: cache rows left unwritten"); \
-    return CG_OK;                                                                              \
+  // From here on the caches claim their new rows (the views above them must see realised values), and
+  // the launch below is what stores them.  When a later check finds the kernel cannot take this graph,
+  // the rows are written by kernels of their own and the unfused path goes on from two ordinary caches.
+#define ATTN_BAIL()                               \
+  do {                                            \
+    if (fused_append) {                           \
+      TRY(write_row_append(be, ka));              \
+      TRY(write_row_append(be, va));              \
+    }                                             \
+    return CG_OK;                                 \
   } while (0)
   MatOperand Kop, Vop;
   bool pk = false, pv = false;
@@ -3675,7 +3733,7 @@ int realize_concat(cg_backend *be, cg_tensor *n) {
   const int64_t xd = x->shape[dim], yd = y->shape[dim];
   const int plain = n->dtype == CG_F32 ? ST_F32 : ST_U32;
   const bool in_place = xd > 0 && yd > 0 && refs(x) == 1 && x->st->rc.load() == 1 && x->st->grow_dim == dim &&
-                        xd + yd <= x->st->grow_cap && x->offset == 0 && x->stype == plain;
+                        xd + yd <= x->st->grow_cap && x->offset == 0 && x->stype == plain && has_grow_layout(x);
   // the new key rows arrive through apply_rope_embedding: rotate them straight into the cache slot
   RopeMatch rope;
   const bool rope_y = in_place && !(be->flags & CG_FLAG_NO_PATTERNS) && y->op != N_REAL && refs(y) == 1 &&
@@ -3692,11 +3750,17 @@ int realize_concat(cg_backend *be, cg_tensor *n) {
     std::memcpy(n->strides, x->strides, sizeof(n->strides));
     char *dst = (char *)n->st->ptr + xd * n->strides[dim] * 4;
     bool roped = false;
+    int st = CG_OK;
     if (rope_y) {
-      TRY(rope_into(be, y, rope, (float *)dst, n->strides, "rope_kv_append", &roped));
-      if (!roped) TRY(realize(be, y));
+      st = rope_into(be, y, rope, (float *)dst, n->strides, "rope_kv_append", &roped);
+      if (!st && !roped) st = realize(be, y);
     }
-    if (!roped) TRY(run_ew(be, y, true, dst, n->strides, plain, "kv_append"));
+    if (!st && !roped) st = run_ew(be, y, true, dst, n->strides, plain, "kv_append");
+    if (st) {  // still a deferred concat: give the storage reference back
+      storage_release(n->st);
+      n->st = nullptr;
+      return st;
+    }
     n->op = N_REAL;
     drop_inputs(n);
     return CG_OK;
@@ -3719,6 +3783,8 @@ int realize_concat(cg_backend *be, cg_tensor *n) {
     n->stype = plain;
     n->offset = 0;
     contiguous_strides(n->rank, cshape, n->strides);
+    s->grow_rank = n->rank;
+    std::copy(n->strides, n->strides + n->rank, s->grow_strides);
     TRY(run_ew(be, x, true, s->ptr, n->strides, plain, "ew_concat"));
     char *dst = (char *)s->ptr + xd * n->strides[dim] * 4;
     TRY(run_ew(be, y, true, dst, n->strides, plain, "ew_concat"));
@@ -3817,6 +3883,7 @@ int sync_and_check(cg_backend *be) {
   HIPCHK(be, hipMemcpyAsync(be->h_words, be->d_words, 8, hipMemcpyDeviceToHost, be->ordered_stream()));
   if (be->queue) HIPCHK(be, be->queue->take_error());  // a launch the queue's thread could not make
   HIPCHK(be, hipStreamSynchronize(be->ordered_stream()));
+  cap_pool(be);
   const uint32_t e = be->h_words[0];
   if (e) {
     HIPCHK(be, launch_fill_u32(be->lc(), be->d_words, 0u, 1));
@@ -3899,6 +3966,13 @@ int run_pending_flush(cg_backend *be) {
     st = e == hipSuccess ? realize(be, f) : fail(be, CG_ERR_DEVICE, hipGetErrorString(e));
   }
   node_release(f);
+  return st;
+}
+
+// realize_view for a node its creator has not handed out yet: on failure the node goes
+int realize_view_or_release(cg_backend *be, cg_tensor *n) {
+  const int st = realize_view(be, n);
+  if (st) node_release(n);
   return st;
 }
 
@@ -4545,7 +4619,7 @@ int cg_broadcast(cg_backend *be, cg_tensor *x, const size_t *dims, int rank, cg_
   n->op = N_BROADCAST;
   n->in[0] = retain(x);
   if (!(be->flags & CG_FLAG_EAGER) && share_node(be, n, out)) return CG_OK;
-  if (x->op == N_REAL) TRY(realize_view(be, n));
+  if (x->op == N_REAL) TRY(realize_view_or_release(be, n));
   return finish(be, n, out);
 }
 
@@ -4566,7 +4640,7 @@ int cg_reshape(cg_backend *be, cg_tensor *x, const size_t *dims, int rank, cg_te
   // a reshape that is a pure view of realised data costs nothing: do it now
   int64_t tmp[CG_MAX_RANK];
   if (x->op == N_REAL && (sz == 0 || try_reshape_view(x->rank, x->shape, x->strides, rank, shape, tmp)))
-    TRY(realize_view(be, n));
+    TRY(realize_view_or_release(be, n));
   return finish(be, n, out);
 }
 
@@ -4584,7 +4658,7 @@ int cg_transpose(cg_backend *be, cg_tensor *x, size_t d0, size_t d1, cg_tensor *
   n->p1 = (int64_t)d1;
   n->in[0] = retain(x);
   if (!(be->flags & CG_FLAG_EAGER) && share_node(be, n, out)) return CG_OK;
-  if (x->op == N_REAL) TRY(realize_view(be, n));
+  if (x->op == N_REAL) TRY(realize_view_or_release(be, n));
   return finish(be, n, out);
 }
 
@@ -4737,7 +4811,7 @@ int cg_slice(cg_backend *be, cg_tensor *x, size_t dim, size_t start, size_t len,
   n->p1 = (int64_t)start;
   n->in[0] = retain(x);
   if (!(be->flags & CG_FLAG_EAGER) && share_node(be, n, out)) return CG_OK;
-  if (x->op == N_REAL) TRY(realize_view(be, n));
+  if (x->op == N_REAL) TRY(realize_view_or_release(be, n));
   return finish(be, n, out);
 }
 

@@ -30,6 +30,11 @@ struct Storage {
   // set by concat when the buffer was laid out with spare room along one axis (KV cache)
   int grow_dim = -1;
   int64_t grow_cap = 0;
+  // the layout the spare room belongs to: rank and element strides of the tensor it was allocated for.
+  // Only a view with exactly these strides may be appended to in place (a transposed or regrouped
+  // view of the same storage would write its new rows over live elements).
+  int grow_rank = 0;
+  int64_t grow_strides[CG_MAX_RANK] = {};
   // bf16 copy of this (f32) storage, element for element, made on demand for the MFMA GEMM and
   // shared by every matmul that reads a view of it (q/k/v, gate/up read the same activations)
   Storage *shadow = nullptr;

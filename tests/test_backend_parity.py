@@ -525,6 +525,35 @@ def test_concat_append_in_place_keeps_values(dev):
     assert np.allclose(out, np.matmul(cur, w), rtol=1e-5, atol=1e-5)
 
 
+@pytest.mark.parametrize("view", ["transposed", "regrouped", "sliced"])
+def test_concat_onto_another_view_of_a_cache_copies(oracle, dev, view):
+    """A sole-owner view of a cache's storage that does not walk it like the cache (a transpose, a
+    reshape that merges rows and columns) must not be appended to in place: its "next row" lies on
+    live elements, or past the room of a head."""
+    g = rng(("view", view))
+    base = g.standard_normal((1, 2, 8, 4)).astype(np.float32)
+    first = g.standard_normal((1, 2, 1, 4)).astype(np.float32)
+    cache_np = np.concatenate([base, first], axis=2)                   # [1, 2, 9, 4], storage with spare rows
+    outs = []
+    for be in (oracle, dev):
+        t = be.concat(be.tensor(base), be.tensor(first), 2)
+        be.to_vec(t)                                                   # in memory now
+        if view == "transposed":
+            v, v_np = be.transpose(t, 2, 3), cache_np.transpose(0, 1, 3, 2)            # [1, 2, 4, 9]
+        elif view == "regrouped":
+            v, v_np = be.reshape(t, (1, 2, 3, 12)), cache_np.reshape(1, 2, 3, 12)
+        else:
+            v, v_np = be.slice(t, 3, 0, 2), cache_np[..., :2]                          # walks it like the cache
+        be.to_vec(v)
+        del t                                                          # the view is the only owner left
+        y = g.standard_normal(v_np.shape[:2] + (1,) + v_np.shape[3:]).astype(np.float32) if be is oracle else y
+        r = be.concat(v, be.tensor(y), 2)
+        del v
+        outs.append(be.numpy(r))
+        assert_bits(outs[-1], np.concatenate([v_np, y], axis=2))
+    assert_bits(outs[0], outs[1])
+
+
 def test_repeat_kv_matmul(oracle, dev):
     """q @ repeat_kv(k)^T and p @ repeat_kv(v) (helpers.rs:147-161, models/llama.rs:95-108)."""
     import vectors

@@ -371,6 +371,54 @@ def test_attention_decode(oracle, hip, hip_nopat, cfg):
     assert np.allclose(gen[0], ref, rtol=1e-4, atol=1e-5)
 
 
+def test_attention_decode_that_cannot_be_fused_still_appends_its_rows(oracle, hip_bf16, cg):
+    """A decode step whose caches qualify for the append inside the attention kernel, but whose query
+    does not (an uploaded rank-4 tensor is bf16 storage in bf16 mode): the new key and value rows must
+    end up in the caches all the same, and the step must give the unfused path's result."""
+    H, KV, T0, d = 4, 2, 12, 16
+    g = np.random.default_rng(77)
+    bf = vectors.bf16_round
+    k0, v0 = (bf(g.standard_normal((1, KV, T0, d)).astype(np.float32)) for _ in range(2))
+    k1, v1, kn, vn = (bf(g.standard_normal((1, KV, 1, d)).astype(np.float32)) for _ in range(4))
+    q = bf(g.standard_normal((1, H, 1, d)).astype(np.float32))
+
+    def grow(b, a, c):                                   # a computed f32 cache with spare rows
+        return lang.concat(b, 2, a + a - a, c + c - c)
+
+    def step(b, qv, kc, vc, kx, vx):
+        k = lang.concat(b, 2, kc, kx + kx - kx)
+        v = lang.concat(b, 2, vc, vx + vx - vx)
+        kr, vr = helpers.repeat_kv(b, H // KV, k), helpers.repeat_kv(b, H // KV, v)
+        attn = lang.matmul(b, qv, lang.transpose(b, 2, 3, kr))
+        sh = lang.shape(b, attn)
+        attn = attn / lang.constant(b, float(np.sqrt(np.float32(d))), sh)
+        attn = attn + lang.broadcast(b, helpers.causal_mask(b, lang.to_nat(b, 1)), sh)
+        return lang.matmul(b, nn.softmax(b, attn), vr), k, v
+
+    res = []
+    for be in (oracle, hip_bf16):
+        it = cg.Interpreter(be, cg.stdlib())
+        gt = vectors.Fn("grow", 2, 1, grow).term()
+        (kc,) = it.run(gt, [be.tensor(k0), be.tensor(k1)])
+        (vc,) = it.run(gt, [be.tensor(v0), be.tensor(v1)])
+        be.realize(kc), be.realize(vc)
+        st = vectors.Fn("step", 5, 3, step).term()
+        if be is hip_bf16:
+            be.trace(True)
+            be.trace_reset()
+        out, k, v = it.run(st, [be.tensor(q), kc, vc, be.tensor(kn), be.tensor(vn)], moved=(1, 2))
+        res.append([be.numpy(out), be.numpy(k), be.numpy(v)])
+        if be is hip_bf16:
+            names = set(be.trace_report())
+            be.trace(False)
+            # the rows went in through their own launches, into the caches' own storage
+            assert "kv_append" in names and "attn_decode" not in names, sorted(names)
+    (ro, rk, rv), (go, gk, gv) = res
+    assert np.array_equal(rk, np.concatenate([k0, k1, kn], axis=2)) and np.array_equal(gk, rk)
+    assert np.array_equal(gv, rv) and np.array_equal(rv, np.concatenate([v0, v1, vn], axis=2))
+    assert np.max(np.abs(go - ro)) <= 2e-2 * np.abs(ro).max()
+
+
 @pytest.mark.parametrize("K", [2048, 256, 1152])
 @pytest.mark.parametrize("variant", ["llama", "gemma", "extra_consumer"])
 def test_rmsnorm_in_projection_prologue(oracle, hip, hip_bf16, hip_nopat, K, variant):
