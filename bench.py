@@ -18,21 +18,26 @@ import numpy as np
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
-sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per launch of the decode GEMV kernels at the default workload (bf16, 16 layers), from two
-# rocprofv3 --pmc runs of this file (FETCH_SIZE, WRITE_SIZE), each scaled by what the same counter
-# read for the 1 GiB peak_copy_kernel in the same run (x2.000 and x1.000); a profiler cannot run
-# inside this process, so the figure is carried here and reported only for that workload
-PMC_TRAFFIC_BYTES_PER_LAUNCH = {("bf16", 16, "gemv_rowdot_bf16"): 38325390.0}
 MFMA_PEAK_TFLOPS = {"bf16": 2500.0, "f32": 157.3}
+# HBM bytes per launch of the decode GEMV kernels at the default workload come from two rocprofv3 --pmc
+# runs of this file (FETCH_SIZE, WRITE_SIZE; a profiler cannot run inside this process).  Their
+# summary, with the commands, is this file; its "traffic_bytes_per_launch" line is read, so the figure
+# reported is the one the committed counters show, for the workload they were taken on only.
+PMC_SUMMARY = os.path.join(ROOT, "profiles", "gemv_rowdot_bf16_llama1b_decode_pmc.txt")
 
 
-def llama_1b_config(llm, layers):
-    return llm.Config(hidden_size=2048, intermediate_size=8192, num_hidden_layers=layers,
-                      num_attention_heads=32, num_key_value_heads=8, vocab_size=128256,
-                      rms_norm_eps=1e-5, rope_theta=500000.0, tie_word_embeddings=True)
+def pmc_traffic_bytes_per_launch(dtype, layers, kernel):
+    """The `traffic_bytes_per_launch[dtype,layers,kernel] = N` line of the PMC summary, or None."""
+    key = f"traffic_bytes_per_launch[{dtype},{layers},{kernel}]"
+    try:
+        for line in open(PMC_SUMMARY):
+            if key in line:
+                return float(line.split("=")[1].split()[0])
+    except OSError:
+        pass
+    return None
 
 
 def matmul_params(cfg):
@@ -40,6 +45,41 @@ def matmul_params(cfg):
     kv = h // (cfg.num_attention_heads // cfg.num_key_value_heads)
     per_layer = 2 * h * h + 2 * kv * h + 3 * f * h
     return cfg.num_hidden_layers * per_layer + v * h
+
+
+def other_configs(lib, args):
+    """The other BASELINE configurations, after the timed region: configs[1] op by op (f32 and bf16
+    storage, each with its roofline fraction), configs[0] (the 64x128x256x10 MLP, microseconds per run),
+    configs[3] (Qwen-MoE layout) and configs[4] (Gemma-3 shape) at full size."""
+    opbench = importlib.import_module("benchmarks.opbench")
+    mb = importlib.import_module("benchmarks.modelbench")
+    res = {}
+    recs = opbench.run_all(lib, iters=20)
+    for dtype in ("f32", "bf16"):
+        table = {}
+        for r in recs:
+            if r["dtype"] != dtype or r["bound"] == "latency":
+                continue
+            table[r["op"]] = {"bound": r["bound"], "achieved": r["tflops"] if r["bound"] == "mfma" else r["gbs"],
+                              "unit": "TFLOP/s" if r["bound"] == "mfma" else "GB/s", "frac": r["frac"],
+                              "kernel_us": r["kernel_us"], "wall_us": r["wall_us"]}
+        res["ops_" + dtype] = table
+    mlp = [r for r in recs if r["bound"] == "latency"]
+    if mlp:
+        res["mlp_us"] = {"wall_us_per_run": mlp[0]["wall_us"], "kernel_us_per_run": mlp[0]["kernel_us"],
+                         "launches": sum(mlp[0]["kernels"].values())}
+    q = mb.run_qwen_moe(lib, steps=16, warmup=2)
+    res["qwen_moe"] = {"ms_per_step": q["ms_per_step"], "decode_tokens_per_s": q["decode_tokens_per_s"],
+                       "prefill_ms": q["prefill_ms"], "prefill_tokens_per_s": q["prefill_tokens_per_s"],
+                       "kernel_launches_per_step": q["kernel_launches_per_step"],
+                       "roofline_frac_hbm_upper_bound_bytes": q["decode_hbm_fraction_at_upper_bound"],
+                       "workload": q["workload"]}
+    g = mb.run_gemma3(lib)
+    res["gemma3"] = {"prefill_ms": g["prefill_ms"], "prefill_tokens_per_s": g["prefill_tokens_per_s"],
+                     "tflops_end_to_end": g["matmul_tflops_end_to_end"],
+                     "roofline_frac_mfma_end_to_end": g["matmul_tflops_end_to_end"] / MFMA_PEAK_TFLOPS["bf16"],
+                     "gemm_tflops": g["gemm_tflops"], "workload": g["workload"]}
+    return res
 
 
 def main():
@@ -58,7 +98,9 @@ def main():
     ap.add_argument("--sync-each-step", action="store_true",
                     help="read every token on the host before starting the next step")
     ap.add_argument("--profile-only", action="store_true",
-                    help="skip the CPU baseline and the traced pass (for rocprofv3 runs)")
+                    help="skip the CPU baseline, the traced pass and the other configurations (for rocprofv3 runs)")
+    ap.add_argument("--no-extras", action="store_true",
+                    help="skip the other BASELINE configurations (ops, MLP, Qwen-MoE, Gemma-3) after the timed region")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (no collectives, no sharding); "
@@ -67,11 +109,10 @@ def main():
 
     cg = importlib.import_module("catgrad-rs_amd")
     llm = importlib.import_module("catgrad-rs_amd.llm")
-    import llama_util as U
 
     lib = cg.load_library()
     if args.workload in ("qwen_moe", "gemma3"):
-        mb = importlib.import_module("catgrad-rs_amd.modelbench")
+        mb = importlib.import_module("benchmarks.modelbench")
         if args.workload == "qwen_moe":
             rec = mb.run_qwen_moe(lib, layers=args.layers or 24, steps=args.steps, warmup=args.warmup)
         else:
@@ -79,9 +120,9 @@ def main():
         print(json.dumps({"metric": rec.pop("workload"), "n_gpus": 1, "dtype": "bf16", "data": "synthetic", **rec}))
         return
     args.layers = args.layers or 16
-    cfg = llama_1b_config(llm, args.layers)
+    cfg = llm.random_init.llama_1b_config(llm.Config, args.layers)
     if args.workload == "ops":
-        opbench = importlib.import_module("catgrad-rs_amd.opbench")
+        opbench = importlib.import_module("benchmarks.opbench")
         recs = opbench.run_all(lib, iters=max(args.steps, 10))
         print(json.dumps({"metric": "single-op microbenchmarks through the evaluator (BASELINE configs[0], [1])",
                           "n_gpus": 1, "data": "synthetic", "hbm_peak_gbs": HBM_PEAK_GBS,
@@ -89,8 +130,8 @@ def main():
         return
     be = cg.Backend(lib, flags=cg.FLAG_BF16 if args.dtype == "bf16" else 0)
     t0 = time.time()
-    arrays = U.param_arrays(cfg, seed=0, std=0.02)
-    runner = U.CachedRunner(be, cfg, arrays, args.prompt + args.warmup + args.steps + 16)
+    arrays = llm.random_init.llama_params(cfg, seed=0, std=0.02)
+    runner = llm.CachedRunner(be, cfg, arrays, args.prompt + args.warmup + args.steps + 16)
     be.sync()
     setup_s = time.time() - t0
     prompt = np.random.default_rng(1).integers(0, cfg.vocab_size, args.prompt).astype(np.uint32)
@@ -189,7 +230,7 @@ def main():
             achieved = r["bytes"] / (r["ms"] * 1e-3) / 1e9
             out["roofline"] = {"bound": "hbm", "kernel": gemv, "achieved": achieved, "peak": HBM_PEAK_GBS,
                                "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-                               "traffic": PMC_TRAFFIC_BYTES_PER_LAUNCH.get((args.dtype, args.layers, gemv)),
+                               "traffic": pmc_traffic_bytes_per_launch(args.dtype, args.layers, gemv),
                                "launches_per_step": r["launches"] / n_tr,
                                "avg_us": r["ms"] * 1e3 / r["launches"],
                                "algorithmic_bytes_per_launch": r["bytes"] / r["launches"]}
@@ -223,19 +264,46 @@ def main():
         # decode step at any cache length here).
         olib = cg.load_library(os.path.join(ROOT, "oracle", "liboracle.so"))
         obe = cg.Backend(olib)
-        cr = U.CachedRunner(obe, cfg, arrays, 64)
-        tk, _ = cr.prefill(prompt[:16])
+        cr = llm.CachedRunner(obe, cfg, arrays, 64)
+        tk, lg = cr.prefill(prompt[:16])
         tkn = int(obe.to_vec(tk)[0])
+        o_toks, o_logits = [tkn], [obe.to_vec(lg)]
         t = time.perf_counter()
         for _ in range(args.cpu_steps):
-            tk, _ = cr.step(tkn)
+            tk, lg = cr.step(tkn)
             tkn = int(obe.to_vec(tk)[0])
+            o_toks.append(tkn)
+            o_logits.append(obe.to_vec(lg))
         cpu_s = time.perf_counter() - t
         out["cpu_baseline"] = {
             "value": args.cpu_steps / cpu_s, "unit": "tokens/s", "cores": 1, "kind": "port",
             "host_cores": os.cpu_count(),
             "sample": f"{args.cpu_steps} KV-cached decode steps at cache length 16.. after a 16-token "
                       "prefill, f32, restated ndarray backend (Rust toolchain unavailable), 1 thread"}
+        del cr
+        # ---- the same sample on the device in f32, compared with what the oracle just computed
+        # (outside every timed region): identical tokens and logits within rel 1e-4, per element
+        # against max(|logit|, rms of the row)
+        del runner
+        fbe = cg.Backend(lib)
+        gr = llm.CachedRunner(fbe, cfg, arrays, 64)
+        g_toks, g_logits = gr.generate(prompt[:16], args.cpu_steps + 1)
+        worst, margin = 0.0, None
+        for a, b_ in zip(o_logits, g_logits):
+            a64 = a.astype(np.float64)
+            floor = np.sqrt(np.mean(a64 * a64))
+            worst = max(worst, float(np.max(np.abs(a64 - b_) / np.maximum(np.abs(a64), floor))))
+            top = np.sort(a64)[-2:]
+            m = float((top[1] - top[0]) / floor)
+            margin = m if margin is None else min(margin, m)
+        out["parity_checked"] = bool(worst <= 1e-4 and g_toks == o_toks)
+        out["parity"] = {"against": "the oracle's logits and tokens on the CPU-baseline sample (full shape, f32)",
+                         "positions": len(o_logits), "max_rel_err": worst, "tolerance": 1e-4,
+                         "tokens_identical": g_toks == o_toks, "min_top1_top2_margin_over_rms": margin}
+        del gr, fbe
+
+    if not args.profile_only and not args.no_extras:
+        out.update(other_configs(lib, args))
 
     print(json.dumps(out))
 

@@ -9,9 +9,13 @@ import time
 
 import numpy as np
 
-from . import abi
-from .interpreter import Interpreter, Parameters, stdlib
-from .llm import Config, gemma3, llama, qwen_moe
+import importlib
+
+cg = importlib.import_module("catgrad-rs_amd")
+_llm = importlib.import_module("catgrad-rs_amd.llm")
+abi = cg.abi
+Interpreter, Parameters, stdlib = cg.Interpreter, cg.Parameters, cg.stdlib
+Config, gemma3, llama, qwen_moe = _llm.Config, _llm.gemma3, _llm.llama, _llm.qwen_moe
 
 
 def _normal(g, shape, std, pool):
@@ -64,37 +68,6 @@ def qwen_moe_parameters(be, cfg, seed=0, std=0.02):
     return P
 
 
-class _Runner:
-    """KV-cached greedy decoding for [B, S] prompts (prefill term per prompt length, one decode term)."""
-
-    def __init__(self, be, cfg, P, max_positions, prefill_cls, decode_cls):
-        self.be, self.cfg = be, cfg
-        self.it = Interpreter(be, stdlib(), P)
-        self.cos, self.sin = self.it.run(llama.RopeTables(cfg).term(), [max_positions])
-        self.prefill_cls = prefill_cls
-        self.decode_term = decode_cls(cfg).term()
-        self.terms = {}
-
-    def prefill(self, ids):
-        ids = np.asarray(ids, np.uint32)
-        self.batch, n = ids.shape
-        if n not in self.terms:
-            self.terms[n] = self.prefill_cls(self.cfg, n).term()
-        out = self.it.run(self.terms[n], [self.be.tensor(ids), self.cos, self.sin])
-        self.kv, self.pos = out[2:], n
-        return out[0], out[1]
-
-    def step(self, tok):
-        ids = self.be.reshape(tok, [self.batch, 1])
-        # the cache tensors are given away (Interpreter::run takes its values by value): the step may
-        # then append to them in place
-        out = self.it.run(self.decode_term, [ids, self.pos, self.cos, self.sin] + self.kv,
-                          moved=range(4, 4 + len(self.kv)))
-        self.kv = out[2:]
-        self.pos += 1
-        return out[0], out[1]
-
-
 def run_qwen_moe(lib, layers=24, batch=4, prompt=256, steps=64, warmup=2):
     be = abi.Backend(lib, flags=abi.FLAG_BF16)
     cfg = qwen_moe_config(layers)
@@ -102,7 +75,7 @@ def run_qwen_moe(lib, layers=24, batch=4, prompt=256, steps=64, warmup=2):
     P = qwen_moe_parameters(be, cfg)
     be.sync()
     setup_s = time.time() - t0
-    r = _Runner(be, cfg, P, prompt + steps + warmup + 8, qwen_moe.QwenMoePrefill, qwen_moe.QwenMoeDecode)
+    r = _llm.CachedRunner(be, cfg, P, prompt + steps + warmup + 8, qwen_moe.QwenMoePrefill, qwen_moe.QwenMoeDecode)
     ids = np.random.default_rng(1).integers(0, cfg.vocab_size, (batch, prompt)).astype(np.uint32)
     # batch rows are independent: row 0 alone gives row 0 of the batch
     tok1, lg1 = r.prefill(ids[:1])

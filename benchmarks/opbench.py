@@ -11,8 +11,11 @@ import time
 
 import numpy as np
 
-from . import abi, lang, nn
-from .interpreter import Interpreter, Parameters, stdlib
+import importlib
+
+cg = importlib.import_module("catgrad-rs_amd")
+abi, lang, nn = cg.abi, cg.lang, cg.nn
+Interpreter, Parameters, stdlib = cg.Interpreter, cg.Parameters, cg.stdlib
 
 HBM_PEAK_GBS = 8000.0
 MFMA_PEAK_TFLOPS = {"bf16": 2500.0, "f32": 157.3}

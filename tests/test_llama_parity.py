@@ -5,6 +5,7 @@ import numpy as np
 import pytest
 
 import llama_util as U
+import parity
 import vectors
 
 
@@ -46,10 +47,6 @@ def test_op_counts_of_emitters(oracle):
     assert 100 <= per_layer <= 160, per_layer      # ~130 Backend calls per Llama layer
 
 
-def margins(logits):
-    s = np.sort(logits)
-    return float(s[-1] - s[-2])
-
 
 @pytest.mark.gpu
 def test_llama_f32_logits_and_tokens(oracle, hip):
@@ -61,11 +58,11 @@ def test_llama_f32_logits_and_tokens(oracle, hip):
     rt, rl = U.CachedRunner(oracle, cfg, arrays, 64).generate(prompt, steps)
     gt, gl = U.CachedRunner(hip, cfg, arrays, 64).generate(prompt, steps)
     for i in range(steps):
-        scale = np.abs(rl[i]).max()
-        assert np.max(np.abs(rl[i] - gl[i])) <= 1e-4 * scale, f"step {i}"
+        parity.assert_f32(rl[i], gl[i], f"step {i}")
         if rt[i] != gt[i]:
             # only acceptable when the oracle's own top-2 margin is inside the f32 error bound
-            assert margins(rl[i]) <= 2e-4 * scale, f"step {i}: tokens differ, margin {margins(rl[i])}"
+            gap = parity.top2_gap_over_max(rl[i])[0]
+            assert gap <= 2 * parity.RTOL_F32, f"step {i}: tokens differ, top-2 gap {gap}"
             break
     else:
         assert rt == gt
@@ -101,12 +98,12 @@ def test_llama_bf16_logits(oracle, hip_bf16):
     _, rl = r.prefill(prompt)
     _, gl = g.prefill(prompt)
     rl, gl = oracle.to_vec(rl), hip_bf16.to_vec(gl)
-    assert np.max(np.abs(rl - gl)) <= 2e-2 * np.abs(rl).max()
+    parity.assert_bf16(rl, gl, "prefill")
     tok = int(np.argmax(rl))
     _, rl = r.step(tok)
     _, gl = g.step(tok)
     rl, gl = oracle.to_vec(rl), hip_bf16.to_vec(gl)
-    assert np.max(np.abs(rl - gl)) <= 2e-2 * np.abs(rl).max()
+    parity.assert_bf16(rl, gl, "decode step")
 
 
 @pytest.mark.gpu
@@ -122,7 +119,7 @@ def test_llama_prefill_of_many_rows(oracle, hip, hip_bf16):
     _, rl = U.CachedRunner(oracle, cfg, arrays, 300).prefill(prompt)
     _, gl = U.CachedRunner(hip, cfg, arrays, 300).prefill(prompt)
     rl, gl = oracle.to_vec(rl), hip.to_vec(gl)
-    assert np.max(np.abs(rl - gl)) <= 1e-4 * np.abs(rl).max()
+    parity.assert_f32(rl, gl, "prefill of 256 rows")
     _, rl = U.CachedRunner(oracle, cfg, rounded, 300).prefill(prompt)
     g = U.CachedRunner(hip_bf16, cfg, arrays, 300)
     hip_bf16.trace(True)
@@ -131,7 +128,7 @@ def test_llama_prefill_of_many_rows(oracle, hip, hip_bf16):
     rl, gl = oracle.to_vec(rl), hip_bf16.to_vec(gl)
     rep = hip_bf16.trace_report()
     hip_bf16.trace(False)
-    assert np.max(np.abs(rl - gl)) <= 2e-2 * np.abs(rl).max()
+    parity.assert_bf16(rl, gl, "prefill of 256 rows")
     launches = {k: v["launches"] for k, v in rep.items()}
     # per layer: q/k/v grouped, o_proj, gate_proj with up_proj (and the activation), down_proj, and the two
     # products of an attention this short (the one-pass kernel starts at 512 keys) = 6 GEMMs
@@ -160,3 +157,27 @@ def test_pipelined_decode_gives_the_same_tokens(hip, hip_bf16):
     big = hip.add(hip.tensor(np.ones(5000, np.float32)), hip.tensor(np.ones(5000, np.float32)))
     hip.prefetch(big)                           # too large for the pinned slot: falls back to the plain read
     assert np.array_equal(hip.to_vec(big), np.full(5000, 2.0, np.float32))
+
+
+@pytest.mark.gpu
+def test_llama_1b_full_shape_f32(oracle, hip):
+    """The north-star model at its real shape (16 layers, hidden 2048, 32/8 heads of 64, FFN 8192,
+    vocabulary 128256, tied lm_head), f32: a 16-token prompt and 3 KV-cached decode steps, HIP against
+    the oracle.  Logits rel 1e-4, identical tokens; the oracle's top-1/top-2 gap is recorded so that a
+    token flip on a near tie would be told apart from an error.  (About half a minute of oracle time.)"""
+    llm = U.llm
+    cfg = llm.random_init.llama_1b_config(llm.Config, 16)
+    arrays = llm.random_init.llama_params(cfg, seed=0, std=0.02)
+    prompt = list(np.random.default_rng(1).integers(0, cfg.vocab_size, 16))
+    steps = 4                                         # the prefill's token + 3 decode steps
+    rt, rl = U.CachedRunner(oracle, cfg, arrays, 32).generate(prompt, steps)
+    gt, gl = U.CachedRunner(hip, cfg, arrays, 32).generate(prompt, steps)
+    gaps = [float(parity.top2_gap_over_max(a)[0]) for a in rl]
+    for i in range(steps):
+        parity.assert_f32(rl[i], gl[i], f"position {i} (top-2 gap {gaps[i]:.2e})")
+    for i in range(steps):
+        assert rt[i] == gt[i] or gaps[i] <= 2 * parity.RTOL_F32, (i, rt, gt, gaps)
+        if rt[i] != gt[i]:
+            break
+    # and bf16 mode at the same shape against the oracle's logits on rounded parameters would need a
+    # second oracle pass; the bf16 bar is held at reduced shapes above and kernel by kernel elsewhere

@@ -6,6 +6,7 @@ import pytest
 
 import llama_util as U
 import model_util as MU
+import parity
 
 cg, llm = U.cg, U.llm
 
@@ -94,10 +95,29 @@ def test_qwen_moe_hip_vs_oracle(oracle, hip, hip_nopat, hip_bf16, mode):
         P_ref = P
     rt, rl = run_model(oracle, model, P_ref, ids)
     gt, gl = run_model(dev, model, P, ids)
-    tol = 4e-2 if mode == "bf16" else 2e-4
-    assert np.max(np.abs(rl - gl)) <= tol * np.abs(rl).max()
+    parity.assert_logits(rl, gl, mode, "Qwen-MoE layout")
     if mode != "bf16":
         assert np.array_equal(rt, gt)
+
+
+class _QwenMoeWithRouterLogits(llm.qwen_moe.QwenMoeModel):
+    """The model, with every layer's router logits ([1, B*S, E]) as extra results."""
+
+    def sort(self):
+        i, o = super().sort()
+        return i, o + [o[0]] * self.config.num_hidden_layers
+
+    def moe(self, builder, p, x):
+        from importlib import import_module
+        nn = import_module("catgrad-rs_amd.nn")
+        c = self.config
+        self._router.append(nn.linear_no_bias(builder, c.hidden_size, c.num_experts, p.extend(["gate"]), x))
+        return super().moe(builder, p, x)
+
+    def def_(self, builder, args):
+        self._router = []
+        out = super().def_(builder, args)
+        return out + self._router
 
 
 @pytest.mark.gpu
@@ -115,10 +135,24 @@ def test_qwen_moe_prefill_of_many_tokens(oracle, hip_bf16):
     gt, gl = run_model(hip_bf16, model, P, ids)
     rep = hip_bf16.trace_report()
     hip_bf16.trace(False)
-    # a router probability within bf16 rounding of its neighbour may pick another expert for a token
-    # (a discontinuity of top-k, not an error of the products): bound the bulk, not the worst token
-    err = np.abs(rl - gl).max(axis=-1).reshape(-1)
-    assert np.quantile(err, 0.9) <= 4e-2 * np.abs(rl).max(), np.sort(err)[-10:]
+    # Every token is held to the bf16 bar, except where top-k itself is discontinuous: a token whose
+    # router logits - in some layer, for itself or for an earlier token of its sequence (attention
+    # carries a changed token forward) - have their k-th and (k+1)-th largest closer than the bf16 bar
+    # on those logits may be routed to another expert on the device than in the oracle.
+    err = parity.per_row_bf16(rl, gl).reshape(ids.shape)
+    outs = U.interpreter(oracle, P_ref).run(_QwenMoeWithRouterLogits(cfg, 48).term(),
+                                            [oracle.tensor(np.asarray(ids, np.uint32))])
+    k = cfg.num_experts_per_tok
+    near_tie = np.zeros(ids.shape, bool)
+    for layer in outs[2:]:
+        lg = oracle.numpy(layer).reshape(ids.shape + (cfg.num_experts,)).astype(np.float64)
+        srt = np.sort(lg, axis=-1)
+        gap = srt[..., -k] - srt[..., -k - 1]
+        near_tie |= gap <= parity.RTOL_BF16 * np.abs(lg).max(axis=-1)
+    exposed = np.maximum.accumulate(near_tie, axis=1)         # the token itself or an earlier one
+    over = err > parity.RTOL_BF16
+    assert not (over & ~exposed).any(), (np.argwhere(over & ~exposed)[:5], err[over & ~exposed][:5])
+    assert (~over).mean() >= 0.5, "most tokens must meet the bar outright"
     assert rep["gemm_experts_bf16"]["launches"] == 2 * cfg.num_hidden_layers, {k: v["launches"] for k, v in rep.items()}
     assert "gemv_experts_bf16" not in rep
 
@@ -135,8 +169,7 @@ def test_gemma3_hip_vs_oracle(oracle, hip, hip_nopat, hip_bf16, mode):
     rt, rl = run_model(oracle, model, P_ref, ids)
     gt, gl = run_model(dev, model, P, ids)
     assert rl.shape == (2, 1, cfg.vocab_size)
-    tol = 4e-2 if mode == "bf16" else 2e-4
-    assert np.max(np.abs(rl - gl)) <= tol * np.abs(rl).max()
+    parity.assert_logits(rl, gl, mode, "Gemma-3")
     if mode != "bf16":
         assert np.array_equal(rt, gt)
 
@@ -443,10 +476,18 @@ def test_moe_cached_decode_hip_vs_oracle(oracle, hip, hip_bf16, mode):
     P_ref = {k: (U_round(v) if v.ndim >= 2 else v) for k, v in P.items()} if mode == "bf16" else P
     rt, rl = moe_cached_generate(oracle, cfg, P_ref, prompts, 6)
     gt, gl = moe_cached_generate(dev, cfg, P, prompts, 6)
-    tol = 4e-2 if mode == "bf16" else 2e-4
+    compared = 0
     for i in range(6):
+        parity.assert_logits(rl[i], gl[i], mode, f"step {i}")   # same history up to here
+        compared += 1
         if not np.array_equal(rt[i], gt[i]):
-            break   # sequences diverged on a near tie: later steps are not comparable
-        assert np.max(np.abs(rl[i] - gl[i])) <= tol * np.abs(rl[i]).max(), i
+            # the sequences part here; only on a near tie of the oracle's own top two logits may they
+            # (bf16 mode), and later steps have different histories and are not comparable
+            assert mode == "bf16"
+            rows = np.flatnonzero(np.asarray(rt[i]).reshape(-1) != np.asarray(gt[i]).reshape(-1))
+            gap = parity.top2_gap_over_max(rl[i])[rows]     # each of the two may move by the bar
+            assert np.all(gap <= 2 * parity.RTOL_BF16), (i, rows, gap)
+            break
+    assert compared >= 1
     if mode == "f32":
         assert np.array_equal(rt, gt)

@@ -8,7 +8,7 @@ import pytest
 
 import vectors
 
-opbench = importlib.import_module("catgrad-rs_amd.opbench")
+opbench = importlib.import_module("benchmarks.opbench")
 EXACT = {"transpose", "gather", "argmax"}
 
 
