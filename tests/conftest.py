@@ -8,7 +8,8 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
-ORACLE_LIB = os.path.join(ROOT, "oracle", "liboracle.so")
+# CATGRAD_ORACLE_LIB: another build of the oracle (the sanitizer build of `make -C oracle SAN=1 san-test`)
+ORACLE_LIB = os.environ.get("CATGRAD_ORACLE_LIB") or os.path.join(ROOT, "oracle", "liboracle.so")
 
 
 def pytest_configure(config):
