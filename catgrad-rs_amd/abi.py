@@ -92,6 +92,7 @@ _SIGNATURES = {
     "cg_trace_enable": (C.c_int, [_P, C.c_int]),
     "cg_trace_reset": (C.c_int, [_P]),
     "cg_trace_report": (_SZ, [_P, C.c_char_p, _SZ]),
+    "cg_launch_counts": (_SZ, [_P, C.c_int, C.c_char_p, _SZ]),
     "cg_stats": (C.c_int, [_P, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]),
     "cg_term_create": (C.c_int, [_PP]),
     "cg_term_destroy": (None, [_P]),
@@ -355,6 +356,20 @@ class Backend:
                 rep[f[0]] = {"launches": int(f[1]), "ms": float(f[2]), "bytes": float(f[3]),
                              "flops": float(f[4])}
         return rep
+
+    def launch_counts(self, reset=False):
+        """{kernel family: launches} since creation or the last reset (no tracing needed)."""
+        n = self.lib.cg_launch_counts(self.ptr, 0, None, 0)
+        buf = C.create_string_buffer(n + 1)
+        self.lib.cg_launch_counts(self.ptr, int(reset), buf, n + 1)
+        out = {}
+        for line in buf.value.decode().splitlines():
+            name, cnt = line.rsplit(" ", 1)
+            if int(cnt):
+                out[name] = int(cnt)
+        return out
+
+    GENERIC_PROGRAMS = ("ew_fused", "row_fused")
 
     def stats(self):
         a, b, c = C.c_uint64(), C.c_uint64(), C.c_uint64()

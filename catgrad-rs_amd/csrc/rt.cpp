@@ -294,6 +294,7 @@ struct KernelScope {
   bool on;
   KernelScope(cg_backend *b, const char *name, double bytes, double flops) : be(b), on(b->trace) {
     be->launches++;
+    count(name);
     if (!on) return;
     pe.name = name;
     pe.bytes = bytes;
@@ -302,6 +303,18 @@ struct KernelScope {
     (void)hipEventCreate(&pe.stop);
     be->cur_start = pe.start;
     be->cur_stop = pe.stop;
+  }
+  // one cached slot per name pointer: the names are string literals
+  void count(const char *name) {
+    static thread_local const char *last_name = nullptr;
+    static thread_local uint64_t last_be = 0;
+    static thread_local uint64_t *last_slot = nullptr;
+    if (name != last_name || be->uid != last_be) {
+      last_slot = &be->launch_counts[name];
+      last_name = name;
+      last_be = be->uid;
+    }
+    ++*last_slot;
   }
   void rename(const std::string &name) {
     if (on && !name.empty()) pe.name = name;
@@ -4266,6 +4279,8 @@ int cg_backend_create(int device, uint32_t flags, cg_backend **out) {
   if (hipSetDevice(device) != hipSuccess) return CG_ERR_DEVICE;
   if (cgrt::noalloc_init_device(device) != CG_OK) return CG_ERR_DEVICE;
   cg_backend *be = new cg_backend();
+  static std::atomic<uint64_t> next_uid{1};
+  be->uid = next_uid.fetch_add(1);
   be->device = device;
   be->flags = flags;
   hipDeviceProp_t prop;
@@ -4936,6 +4951,22 @@ size_t cg_trace_report(cg_backend *be, char *buf, size_t cap) {
   }
   return s.size() + 1;
 }
+size_t cg_launch_counts(cg_backend *be, int reset, char *buf, size_t cap) {
+  if (!be) return 0;
+  std::string out;
+  for (auto &kv : be->launch_counts) out += kv.first + " " + std::to_string(kv.second) + "\n";
+  if (buf && cap) {
+    const size_t n = std::min(cap - 1, out.size());
+    std::memcpy(buf, out.data(), n);
+    buf[n] = 0;
+  }
+  if (reset) {
+    // the slots stay (KernelScope caches a pointer to the last one): zero them
+    for (auto &kv : be->launch_counts) kv.second = 0;
+  }
+  return out.size() + 1;
+}
+
 int cg_stats(cg_backend *be, uint64_t *l, uint64_t *d, uint64_t *p) {
   if (!be) return CG_ERR_ARG;
   if (l) *l = be->launches;

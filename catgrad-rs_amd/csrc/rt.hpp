@@ -131,6 +131,10 @@ struct cg_backend {
   // caching allocator
   std::map<size_t, std::vector<void *>> pool;
   uint64_t pool_bytes = 0, device_bytes = 0, launches = 0;
+  // launches by kernel family (the names of the trace records), counted always: which hand-written
+  // pattern kernels ran and how many launches fell to the generic programs ("ew_fused", "row_fused", ...)
+  std::map<std::string, uint64_t> launch_counts;
+  uint64_t uid = 0;  // distinct for every backend ever created in the process
   // tracing
   bool trace = false;
   bool trace_shapes = false;  // cg_trace_enable(be, 2): matmul records carry their shape

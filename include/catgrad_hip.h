@@ -190,6 +190,14 @@ int cg_peak_mfma_tflops(cg_backend *be, cg_dtype operand, int iters, double *tfl
 int cg_trace_reset(cg_backend *be);
 /* returns the number of bytes needed (including the NUL); writes at most cap bytes */
 size_t cg_trace_report(cg_backend *be, char *buf, size_t cap);
+/* Launches by kernel family since the backend was created (or since the last call with reset != 0),
+ * one line per name, "name count"; counted whether or not tracing is on.  The hand-written pattern
+ * kernels have names of their own ("softmax_fused", "rmsnorm_fused", "rope_fused", "swiglu_fused",
+ * "attn_decode", "gemv_rowdot_bf16", ...); what no pattern took runs as a generic program ("ew_fused",
+ * "row_fused", "reduce_sum" / "reduce_max" / "reduce_argmax").  A caller that expects a model's hot ops
+ * to be pattern kernels can assert that here.  Returns the bytes needed (including the NUL); writes at
+ * most cap bytes.  Zero-count names are listed after a reset. */
+size_t cg_launch_counts(cg_backend *be, int reset, char *buf, size_t cap);
 /* counters: launches issued, bytes allocated from the device, bytes held in the pool */
 int cg_stats(cg_backend *be, uint64_t *launches, uint64_t *device_bytes, uint64_t *pool_bytes);
 

@@ -181,3 +181,38 @@ def test_llama_1b_full_shape_f32(oracle, hip):
             break
     # and bf16 mode at the same shape against the oracle's logits on rounded parameters would need a
     # second oracle pass; the bf16 bar is held at reduced shapes above and kernel by kernel elsewhere
+
+
+@pytest.mark.gpu
+def test_llama_steps_run_on_pattern_kernels(hip, hip_bf16):
+    """No launch of a Llama prefill or decode step falls to the generic elementwise / row programs:
+    every hot op is taken by a hand-written kernel (counted by kernel family, no tracing involved).
+    A reordered emitter that made a matcher miss would show up here as "ew_fused" / "row_fused"."""
+    cfg = U.tiny_config(hidden_size=256, intermediate_size=512, num_hidden_layers=2, num_attention_heads=4,
+                        num_key_value_heads=2, vocab_size=512)
+    arrays = U.param_arrays(cfg, seed=21, std=0.05)
+    prompt = list(np.random.default_rng(22).integers(0, cfg.vocab_size, 48))
+    layers = cfg.num_hidden_layers
+    for be in (hip, hip_bf16):
+        r = U.CachedRunner(be, cfg, arrays, 128)
+        tok, _ = r.prefill(prompt)
+        be.to_vec(tok)
+        be.launch_counts(reset=True)
+        tok, _ = r.prefill(prompt)
+        be.to_vec(tok)
+        pre = be.launch_counts(reset=True)
+        assert not set(pre) & set(be.GENERIC_PROGRAMS), pre
+        assert pre.get("rmsnorm_fused") == 2 * layers + 1 and pre.get("rope_fused") == 2 * layers, pre
+        tok, _ = r.step(int(be.to_vec(tok)[0]))
+        be.to_vec(tok)
+        be.launch_counts(reset=True)
+        tok, _ = r.step(int(be.to_vec(tok)[0]))
+        be.to_vec(tok)
+        dec = be.launch_counts(reset=True)
+        assert not set(dec) & set(be.GENERIC_PROGRAMS), dec
+        gemv = "gemv_rowdot_bf16" if be is hip_bf16 else "gemv_rowdot_f32"
+        # q/k/v, o_proj, gate + up, down_proj per layer and the lm_head; norms, RoPE, the gated activation,
+        # residual adds and the cache append ride inside them and inside the attention launch
+        products = dec.pop(gemv, 0) + dec.pop("gemm", 0)      # narrow products of this small shape take the tile kernel
+        assert products == 4 * layers + 1, (products, dec)
+        assert dec == {"attn_decode": layers, "gather": 1, "reduce_argmax": 1, "fill": 1}, dec

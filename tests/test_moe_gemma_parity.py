@@ -491,3 +491,37 @@ def test_moe_cached_decode_hip_vs_oracle(oracle, hip, hip_bf16, mode):
     assert compared >= 1
     if mode == "f32":
         assert np.array_equal(rt, gt)
+
+
+@pytest.mark.gpu
+def test_generic_program_launches_of_the_other_decoders(hip_bf16):
+    """Which launches of a Gemma-3 prefill and of a Qwen-MoE-layout decode step are generic programs:
+    the embedding scale (one per Gemma run) and the weighted expert sum around the routed experts (three
+    per MoE layer); everything else is a pattern kernel."""
+    be = hip_bf16
+    gcfg = MU.gemma_config()
+    P = MU.gemma_params(gcfg, seed=9, std=0.2)
+    ids = np.random.default_rng(10).integers(0, gcfg.vocab_size, (2, 11)).astype(np.uint32)
+    it = U.interpreter(be, P)
+    term = llm.gemma3.Gemma3Model(gcfg, 11, last_position_only=True).term()
+    be.to_vec(it.run(term, [be.tensor(ids)])[0])
+    be.launch_counts(reset=True)
+    be.to_vec(it.run(term, [be.tensor(ids)])[0])
+    counts = be.launch_counts(reset=True)
+    assert sum(counts.get(k, 0) for k in be.GENERIC_PROGRAMS) == 1, counts
+    assert counts.get("rmsnorm_fused") == 6 * gcfg.num_hidden_layers + 1 and counts.get("geglu_fused", 0) + \
+        counts.get("gemm_mfma_bf16", 0) >= gcfg.num_hidden_layers, counts
+    qcfg = MU.qwen_moe_config()
+    P = MU.qwen_moe_params(qcfg, seed=13, std=0.15)
+    prompts = np.random.default_rng(14).integers(0, qcfg.vocab_size, (3, 9))
+    r = U.CachedRunner(be, qcfg, P, 32, prefill_cls=llm.qwen_moe.QwenMoePrefill, decode_cls=llm.qwen_moe.QwenMoeDecode)
+    tok, _ = r.prefill(prompts)
+    t = be.to_vec(tok).reshape(-1)
+    tok, _ = r.step(t)
+    t = be.to_vec(tok).reshape(-1)
+    be.launch_counts(reset=True)
+    tok, _ = r.step(t)
+    be.to_vec(tok)
+    counts = be.launch_counts(reset=True)
+    assert sum(counts.get(k, 0) for k in be.GENERIC_PROGRAMS) == 3 * qcfg.num_hidden_layers, counts
+    assert counts.get("softmax_topk") == qcfg.num_hidden_layers and counts.get("attn_decode") == qcfg.num_hidden_layers
