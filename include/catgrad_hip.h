@@ -30,6 +30,10 @@
 #ifdef __cplusplus
 extern "C" {
 #endif
+/* the functions declared here are the library's exported symbols (it is built with hidden visibility) */
+#if defined(__GNUC__)
+#pragma GCC visibility push(default)
+#endif
 
 typedef struct cg_backend cg_backend;
 typedef struct cg_tensor cg_tensor;
@@ -331,6 +335,9 @@ int cg_params_stack_experts(cg_backend *be, cg_params *params, const char *prefi
  * this thread */
 const char *cg_weights_last_error(void);
 
+#if defined(__GNUC__)
+#pragma GCC visibility pop
+#endif
 #ifdef __cplusplus
 }
 #endif
