@@ -607,11 +607,10 @@ hipError_t launch_attn_decode(const LaunchCtx &lc, const AttnDecodeDesc &d) {
 // out[b,h,s,j] = cos[s,j] * x[b,h,s,j] + sin[s,j] * rot, rot = j < half ? -x[..,j+half] : x[..,j-half]
 // x is read through (b, h, s) strides with a unit stride along j, so the transposed view of the
 // q/k projection is consumed in place; out is contiguous.  One thread per 4 consecutive j.
-__global__ void __launch_bounds__(256) rope_kernel(RopeDesc d) {
+__device__ __forceinline__ void rope_rows(const RopeDesc &d, uint32_t block, uint32_t n_blocks) {
   const uint32_t q4 = d.dim / 4;
   const uint64_t total = (uint64_t)d.b * d.h * d.s * q4;
-  for (uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x; i < total;
-       i += (uint64_t)gridDim.x * 256) {
+  for (uint64_t i = (uint64_t)block * 256 + threadIdx.x; i < total; i += (uint64_t)n_blocks * 256) {
     const uint32_t j = (uint32_t)(i % q4) * 4;
     uint64_t r = i / q4;
     const uint32_t s = (uint32_t)(r % d.s);
@@ -633,11 +632,32 @@ __global__ void __launch_bounds__(256) rope_kernel(RopeDesc d) {
   }
 }
 
-hipError_t launch_rope(const LaunchCtx &lc, const RopeDesc &d) {
+__global__ void __launch_bounds__(256) rope_kernel(RopeDesc d) { rope_rows(d, blockIdx.x, gridDim.x); }
+
+// queries and keys of one attention in one launch: the first blocks0 workgroups rotate d0, the rest d1
+__global__ void __launch_bounds__(256) rope_pair_kernel(RopeDesc d0, RopeDesc d1, uint32_t blocks0) {
+  if (blockIdx.x < blocks0) rope_rows(d0, blockIdx.x, blocks0);
+  else rope_rows(d1, blockIdx.x - blocks0, gridDim.x - blocks0);
+}
+
+static unsigned rope_blocks(const LaunchCtx &lc, const RopeDesc &d) {
   const uint64_t total = (uint64_t)d.b * d.h * d.s * (d.dim / 4);
-  if (!total) return hipSuccess;
-  uint64_t blocks = (total + 255) / 256, cap = (uint64_t)lc.n_cus * 8;
-  CG_LAUNCH(lc, (rope_kernel), (unsigned)(blocks < cap ? blocks : cap), 256, d);
+  const uint64_t blocks = (total + 255) / 256, cap = (uint64_t)lc.n_cus * 8;
+  return (unsigned)(blocks < cap ? blocks : cap);
+}
+
+hipError_t launch_rope(const LaunchCtx &lc, const RopeDesc &d) {
+  const unsigned blocks = rope_blocks(lc, d);
+  if (!blocks) return hipSuccess;
+  CG_LAUNCH(lc, (rope_kernel), blocks, 256, d);
+  return hipGetLastError();
+}
+
+hipError_t launch_rope_pair(const LaunchCtx &lc, const RopeDesc &d0, const RopeDesc &d1) {
+  const unsigned b0 = rope_blocks(lc, d0), b1 = rope_blocks(lc, d1);
+  if (!b0) return launch_rope(lc, d1);
+  if (!b1) return launch_rope(lc, d0);
+  CG_LAUNCH(lc, (rope_pair_kernel), b0 + b1, 256, d0, d1, (uint32_t)b0);
   return hipGetLastError();
 }
 

@@ -140,6 +140,8 @@ struct RopeDesc {
   uint32_t b, h, s, dim, half;
 };
 hipError_t launch_rope(const LaunchCtx &lc, const RopeDesc &d);
+// two rotations (the queries and the keys of an attention) as one launch
+hipError_t launch_rope_pair(const LaunchCtx &lc, const RopeDesc &d0, const RopeDesc &d1);
 // out = silu(gate) * up (gelu = 0) or gelu(gate) * up (gelu = 1); contiguous, n % 4 == 0
 hipError_t launch_glu(const LaunchCtx &lc, int gelu, const float *gate, const float *up, float *out,
                       uint64_t n, uint16_t *out16 = nullptr);  // out16: optional bf16 copy of out

@@ -27,12 +27,17 @@ int try_attn_prefill(cg_backend *be, cg_tensor *n, bool *done) {
   // above it the scores of one layer run to hundreds of MB.  CG_FLAG_ATTN_ONE_PASS lifts the threshold.
   if (T < 512 && !(be->flags & CG_FLAG_ATTN_ONE_PASS)) return CG_OK;
   if (nb > 65535 || heads > 65535) return CG_OK;
+  cg_tensor *q = S->in[0];
+  // queries and keys both still to be rotated: one launch for the two (each alone otherwise, below)
+  if (cg_tensor *kr = node_under_repeat_kv(S->in[1])) {
+    bool paired = false;
+    TRY(try_rope_pair(be, q, kr, &paired));
+  }
   MatOperand Kop, Vop;
   bool pk = false, pv = false;
   TRY(peel_repeat_kv(be, S->in[1], &Kop, &pk));
   TRY(peel_repeat_kv(be, n->in[1], &Vop, &pv));
   if (!pk || !pv) return CG_OK;  // operands get realised by the generic path below
-  cg_tensor *q = S->in[0];
   TRY(realize(be, q));
   cg_tensor *mask = m.mask;
   if (mask) TRY(realize(be, mask));
@@ -187,6 +192,20 @@ bool has_grow_layout(const cg_tensor *x) {
   return s && x->rank == s->grow_rank && std::equal(x->strides, x->strides + x->rank, s->grow_strides);
 }
 
+
+// The tensor that repeat_kv (helpers.rs:147-161: reshape, broadcast, reshape) and an optional transpose of the
+// last two axes were applied to, when nobody else reads the views in between; null otherwise.
+cg_tensor *node_under_repeat_kv(cg_tensor *t) {
+  if (t->op == N_TRANSPOSE && refs(t) == 1 && t->rank == 4 &&
+      ((t->p0 == 2 && t->p1 == 3) || (t->p0 == 3 && t->p1 == 2)))
+    t = t->in[0];
+  if (t->op != N_RESHAPE || refs(t) != 1 || t->rank != 4) return nullptr;
+  cg_tensor *u = t->in[0];
+  if (u->op != N_BROADCAST || refs(u) != 1 || u->rank != 5) return nullptr;
+  cg_tensor *r5 = u->in[0];
+  if (r5->op != N_RESHAPE || refs(r5) != 1 || r5->rank != 5 || r5->shape[2] != 1) return nullptr;
+  return r5->in[0];
+}
 
 cg_tensor *kv_concat_under(cg_tensor *t) {
   if (t->op == N_TRANSPOSE && refs(t) == 1 && t->rank == 4 &&

@@ -118,6 +118,10 @@ int rope_operands(cg_backend *be, const RopeMatch &m, bool *ok);
 int rope_into(cg_backend *be, cg_tensor *root, const RopeMatch &m, float *out, const int64_t *o_strides,
               const char *name, bool *done, uint16_t *out16 = nullptr);
 int try_rope(cg_backend *be, cg_tensor *root, bool *done);
+int rope_describe(cg_backend *be, cg_tensor *root, const RopeMatch &m, float *out, const int64_t *o_strides,
+                  uint16_t *out16, RopeDesc *dsc, cg_tensor **xs_out, bool *ok);
+int try_rope_pair(cg_backend *be, cg_tensor *rq, cg_tensor *rk, bool *done);
+cg_tensor *node_under_repeat_kv(cg_tensor *t);
 bool is_sigmoid_of(const cg_tensor *s, const cg_tensor **arg);
 bool is_gelu_of(const cg_tensor *g, const cg_tensor **arg);
 bool match_glu(cg_tensor *root, cg_tensor **gate, cg_tensor **up, int *gelu);

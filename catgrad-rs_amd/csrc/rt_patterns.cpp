@@ -551,25 +551,28 @@ int rope_operands(cg_backend *be, const RopeMatch &m, bool *ok) {
 }
 
 
-// Launches the rope kernel for `root` (matched as m) into `out` with the given element strides.
-// *done = false: layout requirements not met, nothing was launched.
-int rope_into(cg_backend *be, cg_tensor *root, const RopeMatch &m, float *out, const int64_t *o_strides,
-              const char *name, bool *done, uint16_t *out16) {
+// Fills the rope kernel's descriptor for `root` (matched as m) writing to `out` with the given element
+// strides.  *xs receives a retained tensor the descriptor reads from (release it after the launch);
+// *ok = false: layout requirements not met, nothing to launch.
+int rope_describe(cg_backend *be, cg_tensor *root, const RopeMatch &m, float *out, const int64_t *o_strides,
+                  uint16_t *out16, RopeDesc *dsc, cg_tensor **xs_out, bool *ok) {
+  *ok = false;
+  *xs_out = nullptr;
   bool tables = false;
   TRY(rope_operands(be, m, &tables));
   if (!tables) return CG_OK;
   cg_tensor *x = m.x, *cb = m.cb, *sb = m.sb;
   cg_tensor *xs = retain(x);
-  bool ok = x->stype == ST_F32 && x->strides[3] == 1 && (uintptr_t)data_ptr(x) % 16 == 0;
+  bool fits = x->stype == ST_F32 && x->strides[3] == 1 && (uintptr_t)data_ptr(x) % 16 == 0;
   for (int i = 0; i < 3; ++i)
-    if (x->strides[i] % 4) ok = false;
-  if (!ok) {
+    if (x->strides[i] % 4) fits = false;
+  if (!fits) {
     node_release(xs);
     xs = nullptr;
     TRY(materialize(be, x, &xs));
   }
   const int64_t dim = root->shape[3];
-  RopeDesc d;
+  RopeDesc &d = *dsc;
   std::memset(&d, 0, sizeof(d));
   d.x = (const float *)data_ptr(xs);
   d.cos = (const float *)data_ptr(cb);
@@ -588,6 +591,20 @@ int rope_into(cg_backend *be, cg_tensor *root, const RopeMatch &m, float *out, c
   d.s = (uint32_t)root->shape[2];
   d.dim = (uint32_t)dim;
   d.half = (uint32_t)(dim / 2);
+  *xs_out = xs;
+  *ok = true;
+  return CG_OK;
+}
+
+// Launches the rope kernel for `root` (matched as m) into `out` with the given element strides.
+// *done = false: layout requirements not met, nothing was launched.
+int rope_into(cg_backend *be, cg_tensor *root, const RopeMatch &m, float *out, const int64_t *o_strides,
+              const char *name, bool *done, uint16_t *out16) {
+  RopeDesc d;
+  cg_tensor *xs = nullptr;
+  bool ok = false;
+  TRY(rope_describe(be, root, m, out, o_strides, out16, &d, &xs, &ok));
+  if (!ok) return CG_OK;
   int st = CG_OK;
   {
     KernelScope ks(be, name, (double)root->size() * 8, 0);
@@ -600,6 +617,48 @@ int rope_into(cg_backend *be, cg_tensor *root, const RopeMatch &m, float *out, c
   return CG_OK;
 }
 
+// The queries and the keys of an attention, both straight from apply_rope_embedding and both still
+// deferred: one launch rotates both.  *done = false: nothing was changed (each is then realised alone).
+int try_rope_pair(cg_backend *be, cg_tensor *rq, cg_tensor *rk, bool *done) {
+  *done = false;
+  if (be->flags & CG_FLAG_NO_PATTERNS) return CG_OK;
+  if (rq == rk || rq->op == N_REAL || rk->op == N_REAL) return CG_OK;
+  RopeMatch mq, mk;
+  if (!match_rope(rq, &mq) || !match_rope(rk, &mk)) return CG_OK;
+  bool tq = false, tk = false;
+  TRY(rope_operands(be, mq, &tq));
+  TRY(rope_operands(be, mk, &tk));
+  if (!tq || !tk) return CG_OK;
+  cg_tensor *roots[2] = {rq, rk};
+  const RopeMatch *ms[2] = {&mq, &mk};
+  RopeDesc d[2];
+  cg_tensor *xs[2] = {nullptr, nullptr};
+  int st = CG_OK;
+  bool ok = true;
+  for (int i = 0; i < 2 && !st && ok; ++i) {
+    st = alloc_result(be, roots[i], ST_F32);
+    uint16_t *y16 = nullptr;
+    if (!st) st = twin_for_result(be, roots[i], &y16);
+    if (!st) st = rope_describe(be, roots[i], *ms[i], (float *)roots[i]->st->ptr, roots[i]->strides, y16, &d[i], &xs[i], &ok);
+  }
+  if (!st && ok) {
+    KernelScope ks(be, "rope_fused", (double)(rq->size() + rk->size()) * 8, 0);
+    hipError_t e = launch_rope_pair(be->lc(), d[0], d[1]);
+    if (e != hipSuccess) st = fail(be, CG_ERR_DEVICE, hipGetErrorString(e));
+  }
+  for (int i = 0; i < 2; ++i) node_release(xs[i]);
+  if (st || !ok) {  // nothing was launched: both stay deferred
+    for (int i = 0; i < 2; ++i) {
+      storage_release(roots[i]->st);
+      roots[i]->st = nullptr;
+    }
+    return st;
+  }
+  finish_fused(rq);
+  finish_fused(rk);
+  *done = true;
+  return CG_OK;
+}
 
 // apply_rope_embedding (catgrad-llm/src/helpers.rs:195-221): cos * x + sin * rotate_half(x)
 int try_rope(cg_backend *be, cg_tensor *root, bool *done) {

@@ -724,3 +724,36 @@ def test_attention_prefill_bf16(oracle, hip_bf16_flash, hip_bf16, hip_nopat, cfg
     scale = np.abs(ref).max()
     assert np.max(np.abs(got[0] - ref)) <= 2e-2 * scale, np.max(np.abs(got[0] - ref)) / scale
     assert np.max(np.abs(gen - ref)) <= 1e-4 * scale
+
+
+def test_queries_and_keys_rotated_by_one_launch(oracle, hip_bf16_flash, cg):
+    """A prefill attention whose queries and keys both come straight from apply_rope_embedding: one
+    launch rotates both (and the rotated keys, a result of the term, are the oracle's)."""
+    nb, H, KV, S, d = 1, 4, 2, 96, 64
+    g = np.random.default_rng(123)
+    # values bf16 storage keeps exactly: the oracle then rotates the same numbers
+    q = vectors.bf16_round(g.standard_normal((nb, H, S, d)).astype(np.float32))
+    k = vectors.bf16_round(g.standard_normal((nb, KV, S, d)).astype(np.float32))
+    v = vectors.bf16_round(g.standard_normal((nb, KV, S, d)).astype(np.float32))
+    llm = __import__("importlib").import_module("catgrad-rs_amd.llm")
+    cfg = llm.Config(hidden_size=H * d, num_attention_heads=H, num_key_value_heads=KV, rope_theta=10000.0)
+
+    def f(b, qv, kv, vv):
+        qv, kv, vv = qv + qv - qv, kv + kv - kv, vv + vv - vv
+        cache = helpers.Cache.init(b, cfg, S)
+        qr = helpers.apply_rope_embedding(b, 0, d, cache.cos, cache.sin, qv)
+        kr = helpers.apply_rope_embedding(b, 0, d, cache.cos, cache.sin, kv)
+        kk = helpers.repeat_kv(b, H // KV, kr)
+        vr = helpers.repeat_kv(b, H // KV, vv)
+        attn = lang.matmul(b, qr, lang.transpose(b, 2, 3, kk))
+        sh = lang.shape(b, attn)
+        attn = attn / lang.constant(b, float(np.sqrt(np.float32(d))), sh)
+        attn = attn + lang.broadcast(b, helpers.causal_mask(b, lang.to_nat(b, S)), sh)
+        return lang.matmul(b, nn.softmax(b, attn), vr), kr
+    ref = vectors.run(oracle, f, 2, q, k, v)
+    hip_bf16_flash.launch_counts(reset=True)
+    got = vectors.run(hip_bf16_flash, f, 2, q, k, v)
+    counts = hip_bf16_flash.launch_counts(reset=True)
+    assert counts.get("rope_fused") == 1 and counts.get("attn_prefill") == 1, counts
+    assert np.allclose(got[1], ref[1], rtol=1e-4, atol=1e-5)                 # the rotated keys
+    assert np.max(np.abs(got[0] - ref[0])) <= 2e-2 * np.abs(ref[0]).max()
