@@ -1992,9 +1992,9 @@ hipError_t launch_matmul(const LaunchCtx &lc, const GemmDesc &g, const char **ke
         const uint64_t d256 = (uint64_t)((g.M + 255) / 256) * ((g.N + 127) / 128) * batch;
         const uint64_t d128 = (uint64_t)((g.M + 127) / 128) * ((g.N + 127) / 128) * batch;
         if (d256 >= (uint64_t)lc.n_cus) e = launch_gemm_dma<256, 256, 2, 4, true, 2, true>(lc, gg, (uint32_t)d256);
-        else e = launch_gemm_dma<128, 256, 2, 2, true, 3, true>(lc, gg, (uint32_t)d128);
+        else e = launch_gemm_dma<128, 256, 2, 4, true, 3, true>(lc, gg, (uint32_t)d128);
       } else if (g.glu_gate || g.c16) {  // the epilogue variant stages a 128 x 128 tile
-        if (deep) e = launch_gemm_dma<128, 128, 2, 2, true, 4>(lc, gg, (uint32_t)t128);
+        if (deep) e = launch_gemm_dma<128, 128, 2, 4, true, 4>(lc, gg, (uint32_t)t128);
         else e = launch_gemm_dma<128, 128, 2, 2, true, 2>(lc, gg, (uint32_t)t128);
       } else if (t256 >= (uint64_t)lc.n_cus && grp256) {
         // 256 x 256 tiles run one to a CU, 128 x 128 two to a CU: when the big tiles leave the last round of
@@ -2006,9 +2006,9 @@ hipError_t launch_matmul(const LaunchCtx &lc, const GemmDesc &g, const char **ke
           e = launch_gemm_dma<256, 256, 2, 4>(lc, gg, (uint32_t)t256);
       } else if (splits == 1 && t128 * 2 <= (uint64_t)lc.n_cus && g.N >= 128) {
         // too few 128 x 128 tiles for the CUs and no split-K to multiply them: halve the tile
-        e = launch_gemm_dma<128, 64, 2, 2, false, 4>(lc, gg, (uint32_t)((uint64_t)((g.M + 127) / 128) * ((g.N + 63) / 64) * batch));
+        e = launch_gemm_dma<128, 64, 4, 2, false, 4>(lc, gg, (uint32_t)((uint64_t)((g.M + 127) / 128) * ((g.N + 63) / 64) * batch));
       } else if (deep) {
-        e = launch_gemm_dma<128, 128, 2, 2, false, 4>(lc, gg, (uint32_t)t128);
+        e = launch_gemm_dma<128, 128, 2, 4, false, 4>(lc, gg, (uint32_t)t128);
       } else {
         e = launch_gemm_dma<128, 128, 2, 2>(lc, gg, (uint32_t)t128);
       }
