@@ -50,7 +50,8 @@ def matmul_params(cfg):
 def other_configs(lib, args):
     """The other BASELINE configurations, after the timed region: configs[1] op by op (f32 and bf16
     storage, each with its roofline fraction), configs[0] (the 64x128x256x10 MLP, microseconds per run),
-    configs[3] (Qwen-MoE layout) and configs[4] (Gemma-3 shape) at full size."""
+    configs[3] (Qwen-MoE layout) and configs[4] (Gemma-3 shape) at full size; and the bf16 GEMM alone over
+    the cubes and the models' product shapes."""
     opbench = importlib.import_module("benchmarks.opbench")
     mb = importlib.import_module("benchmarks.modelbench")
     res = {}
@@ -68,6 +69,9 @@ def other_configs(lib, args):
     if mlp:
         res["mlp_us"] = {"wall_us_per_run": mlp[0]["wall_us"], "kernel_us_per_run": mlp[0]["kernel_us"],
                          "launches": sum(mlp[0]["kernels"].values())}
+    sweep = importlib.import_module("benchmarks.gemm_sweep")
+    res["gemm_bf16_sweep"] = {r["shape"]: {"achieved": r["tflops"], "unit": "TFLOP/s", "frac": r["frac"], "us": r["us"]}
+                              for r in sweep.run(lib, iters=5)}
     q = mb.run_qwen_moe(lib, steps=16, warmup=2)
     res["qwen_moe"] = {"ms_per_step": q["ms_per_step"], "decode_tokens_per_s": q["decode_tokens_per_s"],
                        "prefill_ms": q["prefill_ms"], "prefill_tokens_per_s": q["prefill_tokens_per_s"],

@@ -1925,9 +1925,16 @@ uint32_t gemm_split_k(const LaunchCtx &lc, const GemmDesc &g) {
   return splits;
 }
 
-hipError_t launch_matmul(const LaunchCtx &lc, const GemmDesc &g, const char **kernel_name) {
+hipError_t launch_matmul(const LaunchCtx &lc_in, const GemmDesc &g, const char **kernel_name) {
   const uint32_t batch = g.nb0 * g.nb1;
   if (!batch || !g.M || !g.N) return hipSuccess;
+  // A product split along k is two launches (the slices, then their sum): when the launch is timed, the
+  // start event goes with the first and the stop event with the second, so the record covers both.
+  LaunchCtx lc = lc_in, tail = lc_in;
+  if (g.splits > 1) {
+    lc.ev_stop = nullptr;
+    tail.ev_start = nullptr;
+  }
   const int asz = g.a_stype == ST_BF16 ? 2 : 4, bsz = g.b_stype == ST_BF16 ? 2 : 4;
   const bool a_unit_k = g.sak == 1 || g.K == 1, b_unit_k = g.sbk == 1 || g.K == 1;
   const bool b_unit_n = g.sbn == 1 || g.N == 1;
@@ -2027,11 +2034,9 @@ hipError_t launch_matmul(const LaunchCtx &lc, const GemmDesc &g, const char **ke
     }
     }
     if (splits > 1) {
-      LaunchCtx untimed = lc;
-      untimed.ev_start = untimed.ev_stop = nullptr;
       const uint64_t n = (uint64_t)batch * g.M * g.N;
       uint64_t blocks = (n / 4 + 255) / 256, cap = (uint64_t)lc.n_cus * 16;
-      CG_LAUNCH(untimed, (splitk_reduce_kernel), (unsigned)(blocks < cap ? (blocks ? blocks : 1) : cap), 256,
+      CG_LAUNCH(tail, (splitk_reduce_kernel), (unsigned)(blocks < cap ? (blocks ? blocks : 1) : cap), 256,
                 (const float *)g.workspace, g.c, n, splits, g.c_add);
     }
     return hipGetLastError();
@@ -2039,11 +2044,9 @@ hipError_t launch_matmul(const LaunchCtx &lc, const GemmDesc &g, const char **ke
   const uint32_t gsplits = g.splits > 1 ? g.splits : 1;
   auto sum_slices = [&]() {
     if (gsplits > 1) {
-      LaunchCtx untimed = lc;
-      untimed.ev_start = untimed.ev_stop = nullptr;
       const uint64_t n = (uint64_t)batch * g.M * g.N;
       uint64_t blocks = (n / 4 + 255) / 256, cap = (uint64_t)lc.n_cus * 16;
-      CG_LAUNCH(untimed, (splitk_reduce_kernel), (unsigned)(blocks < cap ? (blocks ? blocks : 1) : cap), 256,
+      CG_LAUNCH(tail, (splitk_reduce_kernel), (unsigned)(blocks < cap ? (blocks ? blocks : 1) : cap), 256,
                 (const float *)g.workspace, g.c, n, gsplits, g.c_add);
     }
   };
