@@ -1,4 +1,5 @@
-// k_attn.hip — attention over many query rows (prefill) in one pass, bf16 MFMA, f32 accumulation.
+// k_attn.hip — attention over many query rows (prefill) in one pass: bf16 MFMA with f32 accumulation,
+// and an all-f32 variant for a backend without the bf16 flag.
 //
 // The op sequence of catgrad-llm/src/models/llama.rs:95-107 (also gemma3.rs:153-186):
 //   scores = matmul(q, transpose(k));  scores / sqrt(d);  + mask;  softmax;  matmul(., v)
@@ -283,13 +284,269 @@ __global__ void __launch_bounds__(NW * 64) attn_prefill_kernel(AttnPrefillDesc a
   }
 }
 
+// The same pass with every product in f32 (v_mfma_f32_32x32x2_f32), for a backend without the bf16 flag:
+// the results stay within the f32 bar of the reference's three-step sequence, and the [b, h, S, T]
+// scores are still never written.  One MFMA consumes two values of the reduction axis, one per lane
+// half, so
+//   S^T: A = K[key kt*32 + col][dim 2 ks + half] (LDS, row pitch D + 2: 64 lanes, 64 banks),
+//        B = the lane's query, dim 2 ks + half (registers);
+//   O^T: B = register i of the lane's probabilities, which is key (i>>2)*8 + half*4 + (i&3) of the tile,
+//        A = V[that key][dim t*32 + col] (LDS, rows as they lie in memory: no transpose).
+// K and V take turns in one LDS tile: the V rows of a step are fetched while its scores are computed,
+// the K rows of the next step while the V product runs.
+// QLDS: the queries of the workgroup stay in LDS instead of registers (a 256-wide head would need 128
+// registers per lane for them, on top of 128 for O^T).
+template <bool QLDS, int D, int BN, int NW>
+__global__ void __launch_bounds__(NW * 64) attn_prefill_f32_kernel(AttnPrefillDesc a) {
+  constexpr int NT = NW * 64;
+  constexpr int KP = D + 2;              // K tile row pitch (floats)
+  constexpr int VP = D + 8;              // V tile row pitch
+  constexpr int DT = D / 32;
+  constexpr int KT = BN / 32;
+  constexpr int CH = BN * D / 4 / NT;    // 16-byte chunks of a tile per thread
+  constexpr bool AHEAD = !QLDS;          // fetch the next tile during the arithmetic (costs CH x 4 registers throughout)
+  __shared__ __attribute__((aligned(16))) float tile[BN * VP];
+  __shared__ __attribute__((aligned(16))) float qs[QLDS ? NW * 32 * KP : 2];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int col = lane & 31, half = lane >> 5;
+  const uint32_t h = blockIdx.y, b = blockIdx.z;
+  const uint32_t kvh = h / a.rep, rp = h % a.rep;
+  const uint32_t query = blockIdx.x * (NW * 32) + wave * 32 + col;
+  const bool q_ok = query < a.s;
+  const uint32_t qc = q_ok ? query : a.s - 1;
+  const float *Q = a.q + (int64_t)b * a.q_sb + (int64_t)h * a.q_sh + (int64_t)qc * a.q_ss;
+  const float *K = a.k + (int64_t)b * a.k_sb + (int64_t)kvh * a.k_skv + (int64_t)rp * a.k_srep;
+  const float *V = a.v + (int64_t)b * a.v_sb + (int64_t)kvh * a.v_skv + (int64_t)rp * a.v_srep;
+  const float *M = a.mask ? a.mask + (int64_t)b * a.m_sb + (int64_t)h * a.m_sh + (int64_t)qc * a.m_ss : nullptr;
+
+  float qf[QLDS ? 1 : D / 2];
+  if constexpr (QLDS) {  // the workgroup's rows, zero past the end; first read after the loop's first barrier
+    const float *Q0 = a.q + (int64_t)b * a.q_sb + (int64_t)h * a.q_sh;
+#pragma unroll
+    for (int c = 0; c < NW * 32 * D / 4 / NT; ++c) {
+      const int ch = tid + c * NT, r = ch / (D / 4), d4 = (ch % (D / 4)) * 4;
+      const uint32_t row = blockIdx.x * (NW * 32) + r;
+      float4 x = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (row < a.s) x = *(const float4 *)(Q0 + (int64_t)row * a.q_ss + d4);
+      *(float2 *)(&qs[r * KP + d4]) = make_float2(x.x, x.y);
+      *(float2 *)(&qs[r * KP + d4 + 2]) = make_float2(x.z, x.w);
+    }
+  } else {
+#pragma unroll
+    for (int c = 0; c < D / 4; ++c) {  // dims 4c .. 4c+3: k-steps 2c (x, y) and 2c+1 (z, w)
+      float4 x = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (q_ok) x = *(const float4 *)(Q + c * 4);
+      qf[2 * c] = half ? x.y : x.x;
+      qf[2 * c + 1] = half ? x.w : x.z;
+    }
+  }
+  a_f32x16 o[DT];
+#pragma unroll
+  for (int t = 0; t < DT; ++t)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) o[t][e] = 0.f;
+  float m_run = -3.40282347e+38f, l_run = 0.f;
+
+  float4 treg[CH];
+  float4 mreg[KT][4];
+  const uint8_t *cls = a.tile_class ? a.tile_class + (size_t)blockIdx.x * a.tile_cols : nullptr;
+  auto next_step = [&](uint32_t t0) {
+    if (!cls) return t0;
+    uint32_t i = t0 / BN;
+    while (i < a.tile_cols && cls[i] == 0) ++i;
+    return i * (uint32_t)BN;
+  };
+  auto step_mask = [&](uint32_t t0) { return M && !(cls && t0 < a.t && cls[t0 / BN] == 2); };
+  // rows of K (or V) of the step at t0 into registers; rows past the end repeat the last one and are
+  // zeroed when they are written to LDS
+  auto fetch_rows = [&](const float *base, int64_t row_stride, uint32_t t0) {
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+      const int ch = tid + c * NT, key = ch / (D / 4), d4 = (ch % (D / 4)) * 4;
+      treg[c] = *(const float4 *)(base + (int64_t)min(t0 + key, a.t - 1) * row_stride + d4);
+    }
+  };
+  auto fetch_mask = [&](uint32_t t0) {
+    if (step_mask(t0)) {
+#pragma unroll
+      for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          mreg[kt][j] = *(const float4 *)(M + min(t0 + kt * 32 + j * 8 + half * 4, a.t - 4));
+    }
+  };
+  uint32_t t0 = next_step(0);
+  if (t0 < a.t) {
+    if (AHEAD) fetch_rows(K, a.k_st, t0);
+    fetch_mask(t0);
+  }
+  for (; t0 < a.t;) {
+    const uint32_t t_next = next_step(t0 + BN);
+    const bool use_mask = step_mask(t0);
+    const bool tail = t0 + BN > a.t;
+    bool live_pair = !use_mask;
+    float4 mcur[KT][4];
+    if (use_mask) {
+      float mmax = -3.40282347e+38f;
+#pragma unroll
+      for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          mcur[kt][j] = mreg[kt][j];
+          float4 mk = mcur[kt][j];
+          if (tail) {
+            const uint32_t key = t0 + kt * 32 + j * 8 + half * 4;
+            if (key >= a.t) mk.x = -3.40282347e+38f;
+            if (key + 1 >= a.t) mk.y = -3.40282347e+38f;
+            if (key + 2 >= a.t) mk.z = -3.40282347e+38f;
+            if (key + 3 >= a.t) mk.w = -3.40282347e+38f;
+          }
+          mmax = fmaxf(mmax, fmaxf(fmaxf(mk.x, mk.y), fmaxf(mk.z, mk.w)));
+        }
+      live_pair = q_ok && mmax > -3.0e38f;
+    }
+    const bool live = __syncthreads_or(live_pair);  // also: the V rows of the previous step have been read
+    const uint32_t t_cur = t0;
+    t0 = t_next;
+    if (!live) {  // uniform
+      if (t_next < a.t) {
+        if (AHEAD) fetch_rows(K, a.k_st, t_next);
+        fetch_mask(t_next);
+      }
+      continue;
+    }
+    if (!AHEAD) fetch_rows(K, a.k_st, t_cur);
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+      const int ch = tid + c * NT, key = ch / (D / 4), d4 = (ch % (D / 4)) * 4;
+      const float4 x = (t_cur + key < a.t) ? treg[c] : make_float4(0.f, 0.f, 0.f, 0.f);
+      *(float2 *)(&tile[key * KP + d4]) = make_float2(x.x, x.y);
+      *(float2 *)(&tile[key * KP + d4 + 2]) = make_float2(x.z, x.w);
+    }
+    __syncthreads();
+    if (AHEAD) fetch_rows(V, a.v_st, t_cur);  // in flight during the score product
+    // ---- S^T = K . Q^T
+    a_f32x16 st[KT];
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt) {
+#pragma unroll
+      for (int e = 0; e < 16; ++e) st[kt][e] = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < D / 2; ++ks) {
+        float qv;
+        if constexpr (QLDS) qv = qs[(wave * 32 + col) * KP + 2 * ks + half];
+        else qv = qf[ks];
+        st[kt] = __builtin_amdgcn_mfma_f32_32x32x2f32(tile[(kt * 32 + col) * KP + 2 * ks + half], qv, st[kt], 0, 0, 0);
+        // keep the scheduler from hoisting a whole tile's LDS reads above the MFMAs (registers)
+        if (ks % 16 == 15) __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    // ---- scale, mask, running maximum.  Register e of tile kt is key t_cur + kt*32 + (e>>2)*8 + half*4 + (e&3)
+    float tmax = -3.40282347e+38f;
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const uint32_t key = t_cur + kt * 32 + j * 8 + half * 4;
+        float mv[4] = {0.f, 0.f, 0.f, 0.f};
+        if (use_mask) { mv[0] = mcur[kt][j].x; mv[1] = mcur[kt][j].y; mv[2] = mcur[kt][j].z; mv[3] = mcur[kt][j].w; }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          float s = st[kt][j * 4 + i];
+          if (a.has_scale) s = s / a.scale;  // the reference's quotient
+          if (use_mask) s = s + mv[i];
+          else if (!M && a.has_mask_const) s = s + a.mask_const;
+          if (tail && key + i >= a.t) s = -3.40282347e+38f;
+          st[kt][j * 4 + i] = s;
+          tmax = fmaxf(tmax, s);
+        }
+      }
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+    const float m_new = fmaxf(m_run, tmax);
+    const float alpha = expf(m_run - m_new);
+    float psum = 0.f;
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const uint32_t key = t_cur + kt * 32 + (e >> 2) * 8 + half * 4 + (e & 3);
+        float p = expf(st[kt][e] - m_new);
+        if (tail && key >= a.t) p = 0.f;
+        st[kt][e] = p;
+        psum += p;
+      }
+    psum += __shfl_xor(psum, 32, 64);
+    l_run = l_run * alpha + psum;
+    m_run = m_new;
+    if (__any(alpha != 1.0f)) {
+#pragma unroll
+      for (int t = 0; t < DT; ++t) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) o[t][e] *= alpha;
+        __builtin_amdgcn_sched_barrier(0);  // one tile of O^T at a time through the VALU registers
+      }
+    }
+    if (!AHEAD) fetch_rows(V, a.v_st, t_cur);
+    __syncthreads();  // every wave has read its K fragments
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+      const int ch = tid + c * NT, key = ch / (D / 4), d4 = (ch % (D / 4)) * 4;
+      *(float4 *)(&tile[key * VP + d4]) = (t_cur + key < a.t) ? treg[c] : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    __syncthreads();
+    if (t_next < a.t) {  // in flight during the value product
+      if (AHEAD) fetch_rows(K, a.k_st, t_next);
+      fetch_mask(t_next);
+    }
+    // ---- O^T += V^T . P^T
+#pragma unroll
+    for (int t = 0; t < DT; ++t)
+#pragma unroll
+      for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int key = kt * 32 + (i >> 2) * 8 + half * 4 + (i & 3);
+          o[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(tile[key * VP + t * 32 + col], st[kt][i], o[t], 0, 0, 0);
+          if (i == 15) __builtin_amdgcn_sched_barrier(0);
+        }
+  }
+  if (M && q_ok && m_run <= -3.0e38f) {  // every key masked: uniform weights, as on the reference path
+    l_run = (float)a.t;
+#pragma unroll
+    for (int t = 0; t < DT; ++t)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) o[t][e] = 0.f;
+    for (uint32_t key = 0; key < a.t; ++key)
+#pragma unroll
+      for (int t = 0; t < DT; ++t)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float4 vv = *(const float4 *)(V + (int64_t)key * a.v_st + t * 32 + j * 8 + half * 4);
+          o[t][j * 4 + 0] += vv.x; o[t][j * 4 + 1] += vv.y; o[t][j * 4 + 2] += vv.z; o[t][j * 4 + 3] += vv.w;
+        }
+  }
+  if (q_ok) {
+    float *out = a.out + (int64_t)b * a.o_sb + (int64_t)h * a.o_sh + (int64_t)query * a.o_ss;
+#pragma unroll
+    for (int t = 0; t < DT; ++t)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        float4 r;
+        r.x = o[t][j * 4 + 0] / l_run; r.y = o[t][j * 4 + 1] / l_run;
+        r.z = o[t][j * 4 + 2] / l_run; r.w = o[t][j * 4 + 3] / l_run;
+        *(float4 *)(out + t * 32 + j * 8 + half * 4) = r;
+      }
+  }
+}
+
 static bool attn_prefill_small_tiles(const LaunchCtx &lc, const AttnPrefillDesc &d) {
+  if (d.f32 && d.d == 256) return true;  // its queries live in LDS: 64 of them fit beside the K / V tile
   return (uint64_t)((d.s + 127) / 128) * d.heads * d.b < (uint64_t)lc.n_cus;  // too few workgroups of 128 queries: 64 each
 }
 
 void attn_prefill_tiling(const LaunchCtx &lc, const AttnPrefillDesc &d, uint32_t *q_rows, uint32_t *keys) {
   *q_rows = attn_prefill_small_tiles(lc, d) ? 64 : 128;
-  *keys = d.d == 256 ? 32 : 64;
+  *keys = (d.d == 256 || (d.f32 && d.d == 128)) ? 32 : 64;
 }
 
 // one workgroup per (key tile, query tile): any value above the masked level, any value that is not zero
@@ -322,23 +579,31 @@ hipError_t launch_mask_tiles(const LaunchCtx &lc, const float *mask, int64_t m_s
 
 hipError_t launch_attn_prefill(const LaunchCtx &lc, const AttnPrefillDesc &d) {
   if (!d.b || !d.heads || !d.s) return hipSuccess;
+  if (d.f32 ? !d.k : (!d.k16 || !d.vt16)) return hipErrorInvalidValue;
   dim3 grid((d.s + 127) / 128, d.heads, d.b);
-  if (attn_prefill_small_tiles(lc, d)) {
-    grid.x = (d.s + 63) / 64;
+  const bool small = attn_prefill_small_tiles(lc, d);
+  if (small) grid.x = (d.s + 63) / 64;
+#define CG_ATTN_CASE(DD, ...)                                               \
+  case DD:                                                                  \
+    if (small) CG_LAUNCH(lc, (__VA_ARGS__, 2>), grid, 128, d);              \
+    else CG_LAUNCH(lc, (__VA_ARGS__, 4>), grid, 256, d);                    \
+    break;
+  if (d.f32) {
     switch (d.d) {
-      case 64: CG_LAUNCH(lc, (attn_prefill_kernel<64, 64, 2>), grid, 128, d); break;
-      case 128: CG_LAUNCH(lc, (attn_prefill_kernel<128, 64, 2>), grid, 128, d); break;
-      case 256: CG_LAUNCH(lc, (attn_prefill_kernel<256, 32, 2>), grid, 128, d); break;
+      CG_ATTN_CASE(64, attn_prefill_f32_kernel<false, 64, 64)
+      CG_ATTN_CASE(128, attn_prefill_f32_kernel<false, 128, 32)
+      case 256: CG_LAUNCH(lc, (attn_prefill_f32_kernel<true, 256, 32, 2>), grid, 128, d); break;
       default: return hipErrorInvalidValue;
     }
-    return hipGetLastError();
+  } else {
+    switch (d.d) {
+      CG_ATTN_CASE(64, attn_prefill_kernel<64, 64)
+      CG_ATTN_CASE(128, attn_prefill_kernel<128, 64)
+      CG_ATTN_CASE(256, attn_prefill_kernel<256, 32)
+      default: return hipErrorInvalidValue;
+    }
   }
-  switch (d.d) {
-    case 64: CG_LAUNCH(lc, (attn_prefill_kernel<64, 64, 4>), grid, 256, d); break;
-    case 128: CG_LAUNCH(lc, (attn_prefill_kernel<128, 64, 4>), grid, 256, d); break;
-    case 256: CG_LAUNCH(lc, (attn_prefill_kernel<256, 32, 4>), grid, 256, d); break;
-    default: return hipErrorInvalidValue;
-  }
+#undef CG_ATTN_CASE
   return hipGetLastError();
 }
 

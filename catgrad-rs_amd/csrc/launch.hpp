@@ -194,7 +194,9 @@ hipError_t launch_attn_decode(const LaunchCtx &lc, const AttnDecodeDesc &d);
 // mask: additive f32 through its strides (0 = broadcast) or a constant; out [b, heads, s, d] through its strides.
 struct AttnPrefillDesc {
   const float *q, *v, *mask;
-  const uint16_t *k16, *vt16;
+  const uint16_t *k16, *vt16;          // bf16 products: keys as bf16 rows, values as bf16 V^T [b, kv, d, T]
+  const float *k;                      // f32 products (f32 != 0): keys as f32 rows; k16 / vt16 unused
+  int32_t f32;
   float *out;
   uint16_t *out16;                     // optional bf16 copy of out, same indexing
   int64_t o_sb, o_sh, o_ss;            // out[b, h, s, :] strides (unit stride along d)

@@ -8,12 +8,13 @@ namespace cgrt {
 //   matmul(softmax(matmul(q, K^T) / sqrt(d) + mask), V)
 // in one launch that reads K and V rows in place from the cache; the [b, h, 1, T] scores and
 // probabilities never exist in HBM.
-// Attention over many query rows (prefill; models/llama.rs:95-107, gemma3.rs:153-186) in bf16 mode:
+// Attention over many query rows (prefill; models/llama.rs:95-107, gemma3.rs:153-186):
 //   matmul(softmax(matmul(q, K^T) / sqrt(d) + mask), V)
 // as one pass with online softmax (k_attn.hip); the [b, h, S, T] scores and probabilities are
-// never written.  f32 mode keeps the generic path (the 1e-4 bar wants f32 products).
+// never written.  With the bf16 flag the products run on bf16 MFMA (keys from their bf16 twin, values
+// from a bf16 V^T made once per call); without it every product is f32 and K / V are read as they lie.
 int try_attn_prefill(cg_backend *be, cg_tensor *n, bool *done) {
-  if (!(be->flags & CG_FLAG_BF16)) return CG_OK;
+  const bool f32 = !(be->flags & CG_FLAG_BF16);
   cg_tensor *P = n->in[0];
   if (P->op == N_REAL || refs(P) != 1 || P->rank != 4) return CG_OK;
   SoftmaxMatch m;
@@ -54,7 +55,7 @@ int try_attn_prefill(cg_backend *be, cg_tensor *n, bool *done) {
       !ok4(data_ptr(Vop.t), Vop.strides[4], {Vop.strides[0], Vop.strides[1], Vop.strides[2], Vop.strides[3]}))
     return CG_OK;
   // the bf16 keys are read eight at a time
-  if (Kop.t->offset % 8 || Kop.strides[0] % 8 || Kop.strides[1] % 8 || Kop.strides[2] % 8 || Kop.strides[4] % 8) return CG_OK;
+  if (!f32 && (Kop.t->offset % 8 || Kop.strides[0] % 8 || Kop.strides[1] % 8 || Kop.strides[2] % 8 || Kop.strides[4] % 8)) return CG_OK;
   TRY(alloc_result(be, n, ST_F32));
   // The models merge the heads next (`transpose(1, 2)` + `reshape [b, s, heads * d]`, llama.rs:107-109):
   // the result is laid out [b, s, heads, d] in memory and handed back as the [b, heads, s, d] view of
@@ -81,20 +82,25 @@ int try_attn_prefill(cg_backend *be, cg_tensor *n, bool *done) {
     a.m_st = mask->shape[3] == 1 ? 0 : mask->strides[3];
     a.m_vec = a.m_st == 1 && (uintptr_t)a.mask % 16 == 0 && a.m_sb % 4 == 0 && a.m_sh % 4 == 0 && a.m_ss % 4 == 0;
   }
-  // the kernel reads mask rows and value columns 16 bytes at a time, and the keys from their bf16 twin
+  // the kernel reads mask rows and value columns 16 bytes at a time, and (bf16) the keys from their bf16 twin
   Storage *ksh = nullptr;
-  const bool twin_ok = Kop.t->st->grow_dim < 0 && Kop.t->st->bytes % 32 == 0;
+  const bool twin_ok = f32 || (Kop.t->st->grow_dim < 0 && Kop.t->st->bytes % 32 == 0);
   if ((mask && !a.m_vec) || T % 8 || !twin_ok) {
     storage_release(n->st);
     n->st = nullptr;
     return CG_OK;
   }
-  TRY(bf16_shadow(be, Kop.t->st, &ksh));
-  a.k16 = (const uint16_t *)ksh->ptr + Kop.t->offset;
   Storage *vt = nullptr;
   const int64_t kvh = Kop.shape[1];
-  TRY(dev_alloc(be, (size_t)nb * kvh * d * T * 2, &vt));
-  {
+  if (f32) {
+    a.f32 = 1;
+    a.k = (const float *)data_ptr(Kop.t);
+  } else {
+    TRY(bf16_shadow(be, Kop.t->st, &ksh));
+    a.k16 = (const uint16_t *)ksh->ptr + Kop.t->offset;
+    TRY(dev_alloc(be, (size_t)nb * kvh * d * T * 2, &vt));
+  }
+  if (!f32) {
     KernelScope ks(be, "transpose_cast_bf16", (double)nb * kvh * d * T * 6, 0);
     hipError_t te = launch_transpose_cast_bf16(be->lc(), data_ptr(Vop.t), ST_F32, vt->ptr, (uint32_t)T, (uint32_t)d,
                                                Vop.strides[3], (uint32_t)nb, (uint32_t)kvh, Vop.strides[0], Vop.strides[1]);
@@ -103,7 +109,7 @@ int try_attn_prefill(cg_backend *be, cg_tensor *n, bool *done) {
       return fail(be, CG_ERR_DEVICE, hipGetErrorString(te));
     }
   }
-  a.vt16 = (const uint16_t *)vt->ptr;
+  if (vt) a.vt16 = (const uint16_t *)vt->ptr;
   a.b = (uint32_t)nb;
   a.heads = (uint32_t)heads;
   a.rep = (uint32_t)Kop.shape[2];

@@ -649,7 +649,16 @@ def hip_bf16_flash():
     return cg.Backend(cg.load_library(), flags=cg.abi.FLAG_BF16 | cg.abi.FLAG_ATTN_ONE_PASS)
 
 
-def test_attention_prefill_with_an_arbitrary_shared_mask(oracle, hip_bf16_flash):
+@pytest.fixture(scope="module")
+def hip_f32_flash():
+    """f32 mode with the one-pass attention kernel enabled for every length."""
+    import importlib
+    cg = importlib.import_module("catgrad-rs_amd")
+    return cg.Backend(cg.load_library(), flags=cg.abi.FLAG_ATTN_ONE_PASS)
+
+
+@pytest.mark.parametrize("mode", ["bf16", "f32"])
+def test_attention_prefill_with_an_arbitrary_shared_mask(oracle, hip_bf16_flash, hip_f32_flash, mode):
     """One [S, T] mask for every batch and head, given as data: its key tiles are classified once
     (all masked: skipped unfetched; all zero: computed without reading the mask; mixed) and the kernel
     must give the oracle's values for each kind - including rows that see no key at all, which the
@@ -678,12 +687,13 @@ def test_attention_prefill_with_an_arbitrary_shared_mask(oracle, hip_bf16_flash)
         attn = attn + lang.broadcast(b, mv, sh)
         return lang.matmul(b, nn.softmax(b, attn), vr)
     (ref,) = vectors.run(oracle, f, 1, q, k, v, mask)
-    got, names = run_traced(hip_bf16_flash, f, 1, q, k, v, mask)
+    be, bar = (hip_bf16_flash, 2e-2) if mode == "bf16" else (hip_f32_flash, 1e-4)
+    got, names = run_traced(be, f, 1, q, k, v, mask)
     assert "attn_prefill" in names and "attn_mask_tiles" in names and "softmax_fused" not in names, sorted(names)
     scale = np.abs(ref).max()
-    assert np.max(np.abs(got[0] - ref)) <= 2e-2 * scale, np.max(np.abs(got[0] - ref)) / scale
+    assert np.max(np.abs(got[0] - ref)) <= bar * scale, np.max(np.abs(got[0] - ref)) / scale
     # the rows that see nothing: the mean of V, for every head
-    assert np.max(np.abs(got[0][:, :, 300:303] - np.repeat(v, H // KV, axis=1).mean(axis=2, keepdims=True))) <= 2e-2 * scale
+    assert np.max(np.abs(got[0][:, :, 300:303] - np.repeat(v, H // KV, axis=1).mean(axis=2, keepdims=True))) <= bar * scale
 
 
 @pytest.mark.parametrize("cfg", [(1, 32, 8, 512, 64), (2, 4, 2, 100, 128), (2, 4, 2, 104, 128), (1, 4, 1, 200, 256),
@@ -724,6 +734,45 @@ def test_attention_prefill_bf16(oracle, hip_bf16_flash, hip_bf16, hip_nopat, cfg
     scale = np.abs(ref).max()
     assert np.max(np.abs(got[0] - ref)) <= 2e-2 * scale, np.max(np.abs(got[0] - ref)) / scale
     assert np.max(np.abs(gen - ref)) <= 1e-4 * scale
+
+
+@pytest.mark.parametrize("cfg", [(1, 32, 8, 512, 64), (2, 4, 2, 100, 128), (2, 4, 2, 104, 128), (1, 4, 1, 200, 256),
+                                 (1, 8, 8, 40, 64), (1, 2, 1, 1024, 64), (1, 8, 2, 320, 128), (2, 2, 2, 72, 256)])
+@pytest.mark.parametrize("mask_kind", ["causal", "window", "none"])
+def test_attention_prefill_f32(oracle, hip_f32_flash, hip, cfg, mask_kind):
+    """Attention over many query rows without the bf16 flag: the same single launch with every product
+    in f32, against the oracle at the f32 bar (values relative to the largest of the result)."""
+    import importlib
+    gemma3 = importlib.import_module("catgrad-rs_amd.llm.gemma3")
+    nb, H, KV, S, d = cfg
+    g = np.random.default_rng(S + d + 1)
+    q = g.standard_normal((nb, H, S, d)).astype(np.float32)
+    k = g.standard_normal((nb, KV, S, d)).astype(np.float32)
+    v = g.standard_normal((nb, KV, S, d)).astype(np.float32)
+    model = gemma3.Gemma3Model(importlib.import_module("catgrad-rs_amd.llm").Config(), S)
+
+    def f(b, qv, kv, vv):
+        qv, kv, vv = qv + qv - qv, kv + kv - kv, vv + vv - vv
+        kr = helpers.repeat_kv(b, H // KV, kv)
+        vr = helpers.repeat_kv(b, H // KV, vv)
+        attn = lang.matmul(b, qv, lang.transpose(b, 2, 3, kr))
+        sh = lang.shape(b, attn)
+        attn = attn / lang.constant(b, float(np.sqrt(np.float32(d))), sh)
+        if mask_kind != "none":
+            n = lang.to_nat(b, S)
+            mask = helpers.causal_mask(b, n) if mask_kind == "causal" else model.window_mask(b, n, 17)
+            attn = attn + lang.broadcast(b, mask, sh)
+        return lang.matmul(b, nn.softmax(b, attn), vr)
+    (ref,) = vectors.run(oracle, f, 1, q, k, v)
+    got, names = run_traced(hip_f32_flash, f, 1, q, k, v)
+    _, default_names = run_traced(hip, f, 1, q, k, v)
+    assert ("attn_prefill" in default_names) == (S >= 512)
+    if S % 8 == 0:
+        assert "attn_prefill" in names and "softmax_fused" not in names, sorted(names)
+    else:       # mask rows are read 16 bytes at a time: other lengths take the three-launch path
+        assert "attn_prefill" not in names
+    scale = np.abs(ref).max()
+    assert np.max(np.abs(got[0] - ref)) <= 1e-4 * scale, np.max(np.abs(got[0] - ref)) / scale
 
 
 def test_queries_and_keys_rotated_by_one_launch(oracle, hip_bf16_flash, cg):
