@@ -17,6 +17,26 @@ __device__ __forceinline__ float wave_max(float v) {
   return v;
 }
 
+// Sum over aligned groups of LANES lanes (a power of two, 2 .. 64); every lane of a group gets the sum.
+// Inside a row of 16 lanes the exchanges are DPP operands of the adds - no trip through the LDS
+// crossbar: quad permutes for distances 1 and 2, then the mirrors of 8 and of 16 lanes, which pair a
+// lane with one of the other half (whose lanes all hold that half's sum by then).  The lanes of a
+// group must be active together.
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float v) {
+  return v + __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
+}
+template <int LANES>
+__device__ __forceinline__ float group_sum(float v) {
+  if (LANES >= 2) v = dpp_add<0xB1>(v);    // quad_perm [1, 0, 3, 2]
+  if (LANES >= 4) v = dpp_add<0x4E>(v);    // quad_perm [2, 3, 0, 1]
+  if (LANES >= 8) v = dpp_add<0x141>(v);   // row_half_mirror
+  if (LANES >= 16) v = dpp_add<0x140>(v);  // row_mirror
+  if (LANES >= 32) v += __shfl_xor(v, 16, 64);
+  if (LANES >= 64) v += __shfl_xor(v, 32, 64);
+  return v;
+}
+
 // Reduce across the workgroup (BLOCK threads, a multiple of 64); every thread gets the result.
 template <int BLOCK, bool IS_MAX>
 __device__ __forceinline__ float block_reduce(float v, float *lds) {

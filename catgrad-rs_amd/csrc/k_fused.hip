@@ -349,8 +349,7 @@ __global__ void __launch_bounds__(BLOCK) attn_decode_kernel(AttnDecodeDesc a) {
     for (int u = 0; u < U; ++u) {
       const uint32_t t = t0 + u * STRIDE;
       float s = qv.x * kr[u].x + qv.y * kr[u].y + qv.z * kr[u].z + qv.w * kr[u].w;
-#pragma unroll
-      for (int m = LPK / 2; m >= 1; m >>= 1) s += __shfl_xor(s, m, 64);
+      s = group_sum<LPK>(s);
       if (a.has_scale) s = s / a.scale;
       if (a.has_mask_const) s = s + a.mask_const;
       if (t < a.t) {
@@ -411,7 +410,6 @@ __global__ void __launch_bounds__(256) attn_decode_split_kernel(AttnDecodeDesc a
   constexpr float FMIN = -3.40282347e+38f;
   __shared__ float red[STRIDE][LPK * 4];
   __shared__ float red_m[STRIDE], red_l[STRIDE];
-  __shared__ float cm[64], cl[64];  // partial maxima and sums while merging (splits <= 64)
   __shared__ uint32_t last_flag;
   const uint32_t h = blockIdx.x, b = blockIdx.y, c = blockIdx.z;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -422,6 +420,18 @@ __global__ void __launch_bounds__(256) attn_decode_split_kernel(AttnDecodeDesc a
   const float *V = a.v + (int64_t)b * a.v_sb + (int64_t)kv * a.v_skv + (int64_t)rp * a.v_srep;
   const bool live = (uint32_t)sub * 4 < a.d;
   const uint32_t t_begin = c * a.chunk, t_end = min(a.t, t_begin + a.chunk);
+  // The cache rows of the first pass are asked for before anything else: the query, its rotation and
+  // this step's own rows come back during the same trip to memory.
+  float4 kn[U], vn[U];
+  auto fetch_rows = [&](uint32_t t0) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const uint32_t tc = min(t0 + u * STRIDE, t_end - 1);
+      kn[u] = *(const float4 *)(K + (int64_t)tc * a.k_st + (live ? sub * 4 : 0));
+      vn[u] = *(const float4 *)(V + (int64_t)tc * a.v_st + (live ? sub * 4 : 0));
+    }
+  };
+  if (t_begin + grp < t_end) fetch_rows(t_begin + grp);
   float4 qv = make_float4(0.f, 0.f, 0.f, 0.f);
   if (live) {
     qv = *(const float4 *)(q + sub * 4);
@@ -453,11 +463,11 @@ __global__ void __launch_bounds__(256) attn_decode_split_kernel(AttnDecodeDesc a
       knew.z = cs.z * knew.z + sn.z * pv.z; knew.w = cs.w * knew.w + sn.w * pv.w;
     }
     vnew = *(const float4 *)(a.v_new + (int64_t)b * a.vn_sb + (int64_t)kv * a.vn_skv + j);
-    if (rp == 0 && grp == 0) {  // one writer per (batch, kv head)
-      *(float4 *)(const_cast<float *>(K) + (int64_t)t_new * a.k_st + j) = knew;
-      *(float4 *)(const_cast<float *>(V) + (int64_t)t_new * a.v_st + j) = vnew;
-    }
   }
+  // A decode step is a chain of short dependent phases, so the arithmetic between two memory trips is
+  // kept short: one reciprocal instead of a quotient per score, and the hardware exponential (2 ulp,
+  // far inside the f32 bar for scores of this size).
+  const float inv_scale = a.has_scale ? 1.0f / a.scale : 1.0f;
   float m_run = FMIN, l_run = 0.f;
   float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
   for (uint32_t t0 = t_begin + grp; t0 < t_end; t0 += STRIDE * U) {
@@ -466,36 +476,43 @@ __global__ void __launch_bounds__(256) attn_decode_split_kernel(AttnDecodeDesc a
     for (int u = 0; u < U; ++u) {
       const uint32_t t = t0 + u * STRIDE;
       const bool in = live && t < t_end && t != t_new;
-      const uint32_t tc = min(t, t_end - 1);
-      kr[u] = *(const float4 *)(K + (int64_t)tc * a.k_st + (live ? sub * 4 : 0));
-      vr[u] = *(const float4 *)(V + (int64_t)tc * a.v_st + (live ? sub * 4 : 0));
+      kr[u] = kn[u];
+      vr[u] = vn[u];
       if (t == t_new) { kr[u] = knew; vr[u] = vnew; }
       else if (!in) { kr[u] = make_float4(0.f, 0.f, 0.f, 0.f); vr[u] = kr[u]; }
     }
+    if (t0 + STRIDE * U < t_end) fetch_rows(t0 + STRIDE * U);  // the next pass, in flight during this one
     float sv[U], mx = FMIN;
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       float s = qv.x * kr[u].x + qv.y * kr[u].y + qv.z * kr[u].z + qv.w * kr[u].w;
-#pragma unroll
-      for (int m = LPK / 2; m >= 1; m >>= 1) s += __shfl_xor(s, m, 64);
-      if (a.has_scale) s = s / a.scale;
+      s = group_sum<LPK>(s);
+      if (a.has_scale) s = s * inv_scale;
       if (a.has_mask_const) s = s + a.mask_const;
       sv[u] = s;
       if (t0 + u * STRIDE < t_end) mx = fmaxf(mx, s);
     }
     const float m_new = fmaxf(m_run, mx);
-    const float alpha = expf(m_run - m_new);
+    const float alpha = __expf(m_run - m_new);
     l_run *= alpha;
     acc.x *= alpha; acc.y *= alpha; acc.z *= alpha; acc.w *= alpha;
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       if (t0 + u * STRIDE < t_end) {
-        const float p = expf(sv[u] - m_new);
+        const float p = __expf(sv[u] - m_new);
         l_run += p;
         acc.x += p * vr[u].x; acc.y += p * vr[u].y; acc.z += p * vr[u].z; acc.w += p * vr[u].w;
       }
     }
     m_run = m_new;
+  }
+  // The new row goes into the cache here, not where it was loaded: a store waits for its data, and
+  // every cache row above was asked for without waiting for the projections' row first.  (The loop
+  // never uses what memory holds at t_new.)
+  if (has_new && live && rp == 0 && grp == 0) {  // one writer per (batch, kv head)
+    const uint32_t j = sub * 4;
+    *(float4 *)(const_cast<float *>(K) + (int64_t)t_new * a.k_st + j) = knew;
+    *(float4 *)(const_cast<float *>(V) + (int64_t)t_new * a.v_st + j) = vnew;
   }
   // merge the lane groups of this workgroup
   *(float4 *)(&red[grp][sub * 4]) = acc;
@@ -510,7 +527,7 @@ __global__ void __launch_bounds__(256) attn_decode_split_kernel(AttnDecodeDesc a
     float L = 0.f, o = 0.f;
 #pragma unroll
     for (int g = 0; g < STRIDE; ++g) {
-      const float w = expf(red_m[g] - M);
+      const float w = __expf(red_m[g] - M);
       L += w * red_l[g];
       o += w * red[g][tid];
     }
@@ -543,33 +560,36 @@ __global__ void __launch_bounds__(256) attn_decode_split_kernel(AttnDecodeDesc a
   // branch above depends on it, and the compiler may not move atomic loads above the barrier), and
   // they are agent-scope atomic loads, which are served from the level the stores went through to,
   // never from this compute unit's own caches.
+  // Every thread asks for all it needs at once - the maxima and sums of all partials (the same
+  // addresses in every lane: one request) and its own column of values - so the merge costs one trip
+  // to memory, not one for the statistics and another for the values.
   const float *base = a.part + ((uint64_t)b * a.heads + h) * a.splits * pw;
-  if ((uint32_t)tid < a.splits) {
-    cm[tid] = __hip_atomic_load(base + tid * pw, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    cl[tid] = __hip_atomic_load(base + tid * pw + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  }
-  __syncthreads();
   if ((uint32_t)tid < a.d) {
-    float M = FMIN;
-    for (uint32_t s = 0; s < a.splits; ++s) M = fmaxf(M, cm[s]);
-    float L = 0.f, o = 0.f;
-    uint32_t s = 0;
-    for (; s + 8 <= a.splits; s += 8) {
-      float pv[8];
-#pragma unroll
-      for (int u = 0; u < 8; ++u)
-        pv[u] = __hip_atomic_load(base + (s + u) * pw + 2 + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    float M = FMIN, L = 0.f, o = 0.f;
+    for (uint32_t s0 = 0; s0 < a.splits; s0 += 8) {
+      float pm[8], pl[8], pv[8];
 #pragma unroll
       for (int u = 0; u < 8; ++u) {
-        const float w = expf(cm[s + u] - M);
-        L += w * cl[s + u];
-        o += w * pv[u];
+        const uint32_t s = min(s0 + u, a.splits - 1);
+        pm[u] = __hip_atomic_load(base + s * pw, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        pl[u] = __hip_atomic_load(base + s * pw + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        pv[u] = __hip_atomic_load(base + s * pw + 2 + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
-    }
-    for (; s < a.splits; ++s) {
-      const float w = expf(cm[s] - M);
-      L += w * cl[s];
-      o += w * __hip_atomic_load(base + s * pw + 2 + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      float mx = M;
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        if (s0 + u < a.splits) mx = fmaxf(mx, pm[u]);
+      const float keep = __expf(M - mx);  // rescale what the earlier groups of eight added up
+      L *= keep;
+      o *= keep;
+      M = mx;
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        if (s0 + u < a.splits) {
+          const float w = __expf(pm[u] - M);
+          L += w * pl[u];
+          o += w * pv[u];
+        }
     }
     a.out[((uint64_t)b * a.heads + h) * a.d + tid] = o / L;
   }
