@@ -6,10 +6,23 @@
 
 namespace cgk {
 
+// Sum over the 64 lanes of a wavefront (all active); every lane gets it.  The exchanges are DPP operands
+// of the adds, not trips through the LDS crossbar: inside each row of 16 lanes quad permutes (distances
+// 1 and 2) and the mirrors of 8 and 16 lanes - after which every lane of a row holds the row's sum -
+// then lane 15 of rows 0 and 2 is added into rows 1 and 3 (row_bcast15), lane 31 into rows 2 and 3
+// (row_bcast31), and lane 63 holds the total.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_add(float v) {
+  return v + __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, ROW_MASK, 0xF, ROW_MASK == 0xF));
+}
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, 64);
-  return v;
+  v = dpp_add<0xB1, 0xF>(v);   // quad_perm [1, 0, 3, 2]
+  v = dpp_add<0x4E, 0xF>(v);   // quad_perm [2, 3, 0, 1]
+  v = dpp_add<0x141, 0xF>(v);  // row_half_mirror
+  v = dpp_add<0x140, 0xF>(v);  // row_mirror
+  v = dpp_add<0x142, 0xA>(v);  // row_bcast15 into rows 1 and 3
+  v = dpp_add<0x143, 0xC>(v);  // row_bcast31 into rows 2 and 3
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
 }
 __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll
@@ -18,22 +31,15 @@ __device__ __forceinline__ float wave_max(float v) {
 }
 
 // Sum over aligned groups of LANES lanes (a power of two, 2 .. 64); every lane of a group gets the sum.
-// Inside a row of 16 lanes the exchanges are DPP operands of the adds - no trip through the LDS
-// crossbar: quad permutes for distances 1 and 2, then the mirrors of 8 and of 16 lanes, which pair a
-// lane with one of the other half (whose lanes all hold that half's sum by then).  The lanes of a
-// group must be active together.
-template <int CTRL>
-__device__ __forceinline__ float dpp_add(float v) {
-  return v + __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
-}
+// The lanes of a group must be active together.
 template <int LANES>
 __device__ __forceinline__ float group_sum(float v) {
-  if (LANES >= 2) v = dpp_add<0xB1>(v);    // quad_perm [1, 0, 3, 2]
-  if (LANES >= 4) v = dpp_add<0x4E>(v);    // quad_perm [2, 3, 0, 1]
-  if (LANES >= 8) v = dpp_add<0x141>(v);   // row_half_mirror
-  if (LANES >= 16) v = dpp_add<0x140>(v);  // row_mirror
+  if (LANES >= 64) return wave_sum(v);
+  if (LANES >= 2) v = dpp_add<0xB1, 0xF>(v);
+  if (LANES >= 4) v = dpp_add<0x4E, 0xF>(v);
+  if (LANES >= 8) v = dpp_add<0x141, 0xF>(v);
+  if (LANES >= 16) v = dpp_add<0x140, 0xF>(v);
   if (LANES >= 32) v += __shfl_xor(v, 16, 64);
-  if (LANES >= 64) v += __shfl_xor(v, 32, 64);
   return v;
 }
 

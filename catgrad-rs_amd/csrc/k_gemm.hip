@@ -950,8 +950,7 @@ __global__ void __launch_bounds__(256) gemv_rowdot_kernel(GemmDesc g, int b_vec,
     for (int r = 0; r < R; ++r)
 #pragma unroll
       for (int m = 0; m < MROWS; ++m)
-#pragma unroll
-        for (int s = LPR / 2; s >= 1; s >>= 1) acc[r][m] += __shfl_xor(acc[r][m], s, 64);
+        acc[r][m] = group_sum<LPR>(acc[r][m]);
     if (KSPLIT > 1) {
       __syncthreads();
       if (sub == 0)
@@ -1036,8 +1035,7 @@ __global__ void __launch_bounds__(256) gemv_multi_kernel(GemvMultiDesc g) {
     }
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-#pragma unroll
-      for (int s = 32; s >= 1; s >>= 1) acc[r] += __shfl_xor(acc[r], s, 64);
+      acc[r] = wave_sum(acc[r]);
       if (lane == 0 && nb + r < N) C[nb + r] = acc[r] + (Cadd ? Cadd[nb + r] : 0.f);
     }
   }
