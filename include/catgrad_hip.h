@@ -75,8 +75,9 @@ enum {
   /* keep deferring, but never dispatch to the hand-written pattern kernels (softmax, RMSNorm,
    * RoPE, gated activations): everything goes through the generic fused-program kernels */
   CG_FLAG_NO_PATTERNS = 4u,
-  /* bf16 mode: use the one-pass attention kernel for every sequence length (by default only from
-   * 512 keys on, where the score tensor it avoids is large) */
+  /* use the one-pass attention kernels over many query rows for every sequence length (by default
+   * only from 512 keys on, where the score tensor they avoid is large); bf16 or f32 products, as
+   * CG_FLAG_BF16 says */
   CG_FLAG_ATTN_ONE_PASS = 8u
 };
 
