@@ -6,6 +6,39 @@
 
 namespace cgk {
 
+// A kernel whose argument is a large descriptor reads it field by field as its control flow reaches
+// each use: a chain of dependent scalar loads, each a trip of ~0.17 us to the argument segment in
+// device memory when its 64-byte line is not in the scalar cache yet (eight of them, 1.2 us, stood in
+// front of the first weight request of a one-row product in a stand-alone harness).  Touching every
+// line of the descriptor at the top, all at once, turns the chain into cache hits: one trip, then the
+// fields as they are needed.  Used by the one-row product kernels, where it measured faster inside a
+// decode step as well (0.1 - 0.7 us per launch); kernels with short chains lose the up-front wait.
+// (Reads only; the wait inside the statement means the scratch registers are dead when it ends.)
+template <int OFF, int LINES>
+__device__ __forceinline__ void warm_kernel_argument_lines() {
+  const auto ka = __builtin_amdgcn_kernarg_segment_ptr();
+  uint32_t t0, t1, t2, t3, t4, t5, t6, t7;
+  constexpr int LAST = OFF + (LINES - 1) * 64;  // fewer than eight lines: the last one is touched again
+#define CG_KA_LINE(i) (OFF + (i) * 64 < LAST ? OFF + (i) * 64 : LAST)
+  asm volatile("s_load_dword %0, %8, %9\n\ts_load_dword %1, %8, %10\n\ts_load_dword %2, %8, %11\n\t"
+               "s_load_dword %3, %8, %12\n\ts_load_dword %4, %8, %13\n\ts_load_dword %5, %8, %14\n\t"
+               "s_load_dword %6, %8, %15\n\ts_load_dword %7, %8, %16\n\ts_waitcnt lgkmcnt(0)"
+               : "=&s"(t0), "=&s"(t1), "=&s"(t2), "=&s"(t3), "=&s"(t4), "=&s"(t5), "=&s"(t6), "=&s"(t7)
+               : "s"(ka), "i"(CG_KA_LINE(0)), "i"(CG_KA_LINE(1)), "i"(CG_KA_LINE(2)), "i"(CG_KA_LINE(3)),
+                 "i"(CG_KA_LINE(4)), "i"(CG_KA_LINE(5)), "i"(CG_KA_LINE(6)), "i"(CG_KA_LINE(7))
+               : "memory");
+#undef CG_KA_LINE
+}
+// BYTES: size of the kernel's arguments (they start at offset 0 of the segment)
+template <int BYTES>
+__device__ __forceinline__ void warm_kernel_arguments() {
+  constexpr int LINES = (BYTES + 63) / 64;
+  static_assert(LINES >= 1 && LINES <= 24, "descriptor size");
+  warm_kernel_argument_lines<0, (LINES < 8 ? LINES : 8)>();
+  if constexpr (LINES > 8) warm_kernel_argument_lines<512, (LINES - 8 < 8 ? LINES - 8 : 8)>();
+  if constexpr (LINES > 16) warm_kernel_argument_lines<1024, LINES - 16>();
+}
+
 // Sum over the 64 lanes of a wavefront (all active); every lane gets it.  The exchanges are DPP operands
 // of the adds, not trips through the LDS crossbar: inside each row of 16 lanes quad permutes (distances
 // 1 and 2) and the mirrors of 8 and 16 lanes - after which every lane of a row holds the row's sum -

@@ -652,7 +652,9 @@ __device__ __forceinline__ void rope_rows(const RopeDesc &d, uint32_t block, uin
   }
 }
 
-__global__ void __launch_bounds__(256) rope_kernel(RopeDesc d) { rope_rows(d, blockIdx.x, gridDim.x); }
+__global__ void __launch_bounds__(256) rope_kernel(RopeDesc d) {
+  rope_rows(d, blockIdx.x, gridDim.x);
+}
 
 // queries and keys of one attention in one launch: the first blocks0 workgroups rotate d0, the rest d1
 __global__ void __launch_bounds__(256) rope_pair_kernel(RopeDesc d0, RopeDesc d1, uint32_t blocks0) {

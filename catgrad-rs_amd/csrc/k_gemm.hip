@@ -861,6 +861,7 @@ template <> struct WVec<uint16_t> {
 // column group, each taking a contiguous 1/KSPLIT of k (for deep, narrow matrices).
 template <typename TB, int LPR, int MROWS, int R, int KSPLIT>
 __global__ void __launch_bounds__(256) gemv_rowdot_kernel(GemmDesc g, int b_vec, int a_vec) {
+  warm_kernel_arguments<sizeof(GemmDesc)>();
   typedef typename WVec<TB>::type VT;
   constexpr int EPL = WVec<TB>::EPL;  // elements per 16-byte load
   constexpr int UNROLL = 4;
@@ -988,6 +989,7 @@ __global__ void __launch_bounds__(256) gemv_rowdot_kernel(GemmDesc g, int b_vec,
 // Same streaming scheme as gemv_rowdot_kernel<.., 64, 1, 2, 1>; blockIdx.y selects the problem.
 template <typename TB>
 __global__ void __launch_bounds__(256) gemv_multi_kernel(GemvMultiDesc g) {
+  warm_kernel_arguments<sizeof(GemvMultiDesc)>();
   typedef typename WVec<TB>::type VT;
   constexpr int EPL = WVec<TB>::EPL, UNROLL = 4, R = 2;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -1073,6 +1075,7 @@ __global__ void __launch_bounds__(256) gemv_pro_kernel(GemvProDesc g) {
   __shared__ __attribute__((aligned(16))) float xs[GEMV_PRO_MAX_K];
   __shared__ float lds[4 * MR];
   __shared__ float part[4][R][MR];
+  warm_kernel_arguments<sizeof(GemvProDesc)>();
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const uint32_t K = g.m.K, bz = blockIdx.z;
   const uint32_t rows = MR == 1 ? 1u : g.rows;
@@ -1754,6 +1757,7 @@ hipError_t launch_moe_gemm(const LaunchCtx &lc, const MoeGemmDesc &g) {
 // 16 column groups of 4 columns x KS k-slices per workgroup; slices meet in LDS.
 template <typename TB, int MROWS, int KS>
 __global__ void __launch_bounds__(16 * KS) gemv_col_kernel(GemmDesc g, int b_vec) {
+  warm_kernel_arguments<sizeof(GemmDesc)>();
   __shared__ float part[KS][MROWS][64 + 4];
   const int cg = threadIdx.x & 15, ks = threadIdx.x >> 4;
   const uint32_t bz = blockIdx.y, b0 = bz / g.nb1, b1 = bz - b0 * g.nb1;
