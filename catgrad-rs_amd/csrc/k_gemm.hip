@@ -1068,7 +1068,8 @@ hipError_t launch_gemv_multi(const LaunchCtx &lc, const GemvMultiDesc &g) {
 // MR: input rows that share the weights (a decode step of a small batch): MR rows of K floats are
 // staged (rows * K <= GEMV_PRO_MAX_K), every weight vector fetched is used for each of them, and the
 // outputs are the rows of a contiguous [rows, N] matrix.
-template <typename TB, bool KSPLIT, bool GLUEPI, int MR>
+// XV: 16-byte pieces of the input rows per thread (rows * K <= XV * 1024 floats).
+template <typename TB, bool KSPLIT, bool GLUEPI, int MR, int XV>
 __global__ void __launch_bounds__(256) gemv_pro_kernel(GemvProDesc g) {
   typedef typename WVec<TB>::type VT;
   constexpr int EPL = WVec<TB>::EPL, UNROLL = 4, R = 2;
@@ -1113,79 +1114,94 @@ __global__ void __launch_bounds__(256) gemv_pro_kernel(GemvProDesc g) {
   constexpr int CPS = GLUEPI ? 1 : R;  // output columns per slot
   // The weight rows of the first pass do not depend on the input row: request them before the
   // prologue so that their latency overlaps it.
+  // Every request is R * UNROLL loads, no fewer (positions past the end repeat the last valid piece
+  // and are not used): the prologue below waits for its own, older loads by count.
   VT q[R][UNROLL];
   auto request = [&](uint32_t nb, uint32_t k0) {
 #pragma unroll
     for (int r = 0; r < R; ++r)
 #pragma unroll
       for (int u = 0; u < UNROLL; ++u) {
-        const uint32_t k = k0 + u * 64 * EPL;
-        if (GLUEPI) {
-          if (k < k_end)
-            q[r][u] = __builtin_nontemporal_load(
-                (const VT *)((r == 0 ? B + (int64_t)nb * sbn : B2 + (int64_t)nb * sbn2) + k));
-        } else if (k < k_end && nb + r < N) {
-          q[r][u] = __builtin_nontemporal_load((const VT *)(B + (int64_t)(nb + r) * sbn + k));
-        }
+        const uint32_t k = min(k0 + u * 64 * EPL, k_end - EPL);
+        if (GLUEPI) q[r][u] = __builtin_nontemporal_load((const VT *)((r == 0 ? B + (int64_t)nb * sbn : B2 + (int64_t)nb * sbn2) + k));
+        else q[r][u] = __builtin_nontemporal_load((const VT *)(B + (int64_t)min(nb + r, N - 1) * sbn + k));
       }
   };
-  bool requested = slot * CPS < N;
-  if (requested) request(slot * CPS, k_begin + lane * EPL);
-  // ---- prologue: the input rows
-  float ssq[MR];  // RMSNorm: the rows' sums of squares, reduced together (one exchange through LDS)
-  if (g.pro == PRO_RMSNORM) {
+  // A workgroup with no column to compute (the narrower problems of a grouped launch) has nothing to stage.
+  if ((KSPLIT ? blockIdx.x : blockIdx.x * 4) * CPS >= N) return;
+  // The input rows first: rows * K floats are at most XV 16-byte pieces per thread (K % 8 == 0: a piece
+  // lies in one row), requested together with what the prologue combines them with (RMSNorm: gamma, one
+  // vector for every row; GLU: the up rows).  They are older than the weight requests that follow, so
+  // they come back first, and - every load here being unconditional, positions past the end repeating
+  // the last piece - the compiler's wait for them is a count that leaves the weight loads in flight: the
+  // prologue's arithmetic runs while the weights are still on their way.
+  const uint32_t pieces = rows * K / 4;
+  const bool has_aux = g.pro == PRO_RMSNORM ? gaux != nullptr : g.pro != PRO_NONE;
+  const float *aux_base = has_aux ? gaux : ga;  // no aux: the loads below repeat the row's own pieces
+  const int64_t aux_rs = !has_aux ? g.a_rstride : g.pro == PRO_RMSNORM ? 0 : g.aux_rstride;
+  float4 xv[XV], gv[XV];
+  uint32_t pm[XV], pk[XV];
 #pragma unroll
-    for (int m = 0; m < MR; ++m) {
-      float ss = 0.f;
-      if (MR == 1 || (uint32_t)m < rows)
-        for (uint32_t k = tid * 4; k < K; k += 1024) {
-          const float4 v = *(const float4 *)(ga + (int64_t)m * g.a_rstride + k);
-          ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
-        }
-      ssq[m] = wave_sum(ss);
-    }
+  for (int j = 0; j < XV; ++j) {
+    const uint32_t e = min((uint32_t)tid + j * 256u, pieces - 1) * 4;
+    pm[j] = MR == 1 ? 0u : e / K;
+    pk[j] = MR == 1 ? e : e % K;
+    xv[j] = *(const float4 *)(ga + (int64_t)pm[j] * g.a_rstride + pk[j]);
+  }
+#pragma unroll
+  for (int j = 0; j < XV; ++j) gv[j] = *(const float4 *)(aux_base + (int64_t)pm[j] * aux_rs + pk[j]);
+  bool requested = true;
+  request(min(slot * CPS, N - 1), k_begin + lane * EPL);
+  // ---- prologue: the input rows, from the registers loaded above into LDS
+  if (g.pro == PRO_RMSNORM) {
+    float ssq[MR];
+#pragma unroll
+    for (int m = 0; m < MR; ++m) ssq[m] = 0.f;
+#pragma unroll
+    for (int j = 0; j < XV; ++j)
+      if (tid + j * 256 < pieces) {
+        const float s = xv[j].x * xv[j].x + xv[j].y * xv[j].y + xv[j].z * xv[j].z + xv[j].w * xv[j].w;
+#pragma unroll
+        for (int m = 0; m < MR; ++m) ssq[m] += (MR == 1 || pm[j] == (uint32_t)m) ? s : 0.f;
+      }
+#pragma unroll
+    for (int m = 0; m < MR; ++m) ssq[m] = wave_sum(ssq[m]);
     if (lane == 0)
 #pragma unroll
       for (int m = 0; m < MR; ++m) lds[wave * MR + m] = ssq[m];
     __syncthreads();
+    float rms[MR];
 #pragma unroll
-    for (int m = 0; m < MR; ++m) ssq[m] = (lds[m] + lds[MR + m]) + (lds[2 * MR + m] + lds[3 * MR + m]);
-  }
+    for (int m = 0; m < MR; ++m)
+      rms[m] = sqrtf(((lds[m] + lds[MR + m]) + (lds[2 * MR + m] + lds[3 * MR + m])) / g.n_as_float + g.eps);
 #pragma unroll
-  for (int m = 0; m < MR; ++m) {
-    if (MR > 1 && (uint32_t)m >= rows) break;
-    const float *gam = ga + (int64_t)m * g.a_rstride;
-    float *xm = xs + (size_t)m * K;
-    if (g.pro == PRO_RMSNORM) {
-      const float rms = sqrtf(ssq[m] / g.n_as_float + g.eps);
-      for (uint32_t k = tid * 4; k < K; k += 1024) {
-        const float4 v = *(const float4 *)(gam + k);
+    for (int j = 0; j < XV; ++j)
+      if (tid + j * 256 < pieces) {
+        float r = rms[0];
+#pragma unroll
+        for (int m = 1; m < MR; ++m) r = pm[j] == (uint32_t)m ? rms[m] : r;
         float4 o;
-        o.x = v.x / rms; o.y = v.y / rms; o.z = v.z / rms; o.w = v.w / rms;
-        if (gaux) {  // gamma: one vector for every row
-          const float4 gm = *(const float4 *)(gaux + k);
-          o.x *= g.gamma_offset + gm.x; o.y *= g.gamma_offset + gm.y;
-          o.z *= g.gamma_offset + gm.z; o.w *= g.gamma_offset + gm.w;
+        o.x = xv[j].x / r; o.y = xv[j].y / r; o.z = xv[j].z / r; o.w = xv[j].w / r;
+        if (has_aux) {
+          o.x *= g.gamma_offset + gv[j].x; o.y *= g.gamma_offset + gv[j].y;
+          o.z *= g.gamma_offset + gv[j].z; o.w *= g.gamma_offset + gv[j].w;
         }
-        *(float4 *)(xm + k) = o;
+        *(float4 *)(xs + (size_t)pm[j] * K + pk[j]) = o;
       }
-    } else if (g.pro == PRO_NONE) {
-      for (uint32_t k = tid * 4; k < K; k += 1024) *(float4 *)(xm + k) = *(const float4 *)(gam + k);
-    } else {
-      const float *gum = gaux + (int64_t)m * g.aux_rstride;
-      for (uint32_t k = tid * 4; k < K; k += 1024) {
-        const float4 a = *(const float4 *)(gam + k), u = *(const float4 *)(gum + k);
-        float4 o;
+  } else {
+#pragma unroll
+    for (int j = 0; j < XV; ++j)
+      if (tid + j * 256 < pieces) {
+        float4 o = xv[j];
         if (g.pro == PRO_GEGLU) {
-          o.x = gelu_ref(a.x) * u.x; o.y = gelu_ref(a.y) * u.y;
-          o.z = gelu_ref(a.z) * u.z; o.w = gelu_ref(a.w) * u.w;
-        } else {
-          o.x = a.x * sigmoid_ref(a.x) * u.x; o.y = a.y * sigmoid_ref(a.y) * u.y;
-          o.z = a.z * sigmoid_ref(a.z) * u.z; o.w = a.w * sigmoid_ref(a.w) * u.w;
+          o.x = gelu_ref(o.x) * gv[j].x; o.y = gelu_ref(o.y) * gv[j].y;
+          o.z = gelu_ref(o.z) * gv[j].z; o.w = gelu_ref(o.w) * gv[j].w;
+        } else if (g.pro == PRO_SWIGLU) {
+          o.x = o.x * sigmoid_ref(o.x) * gv[j].x; o.y = o.y * sigmoid_ref(o.y) * gv[j].y;
+          o.z = o.z * sigmoid_ref(o.z) * gv[j].z; o.w = o.w * sigmoid_ref(o.w) * gv[j].w;
         }
-        *(float4 *)(xm + k) = o;
+        *(float4 *)(xs + (size_t)pm[j] * K + pk[j]) = o;
       }
-    }
   }
   __syncthreads();
   // Several rows: a lane meets the same k positions in every column (K <= 64 * EPL * UNROLL, one pass
@@ -1293,7 +1309,10 @@ static void launch_gemv_pro_block(const LaunchCtx &lc, const GemvProDesc &g, uin
   const uint32_t cap = (uint32_t)lc.n_cus * (MR > 1 || g.m.K >= 4096 ? 2 : 4) / (g.m.n_prob * batch);
   if (blocks > cap) blocks = cap ? cap : 1;
   dim3 grid(blocks, g.m.n_prob, batch);
-  CG_LAUNCH(lc, (gemv_pro_kernel<TB, KSPLIT, false, MR>), grid, 256, g);
+  const uint32_t xv = ((MR > 1 ? g.rows : 1u) * g.m.K / 4 + 255) / 256;  // 16-byte pieces of the input rows per thread
+  if (xv <= 2) CG_LAUNCH(lc, (gemv_pro_kernel<TB, KSPLIT, false, MR, 2>), grid, 256, g);
+  else if (xv <= 4) CG_LAUNCH(lc, (gemv_pro_kernel<TB, KSPLIT, false, MR, 4>), grid, 256, g);
+  else CG_LAUNCH(lc, (gemv_pro_kernel<TB, KSPLIT, false, MR, 8>), grid, 256, g);
 }
 
 template <typename TB, int MR>
@@ -1302,7 +1321,10 @@ static void launch_gemv_pro_glu(const LaunchCtx &lc, const GemvProDesc &g) {
   uint32_t blocks = (slots + 3) / 4;
   const uint32_t cap = (uint32_t)lc.n_cus * (MR > 1 ? 2 : 4);
   if (blocks > cap) blocks = cap;
-  CG_LAUNCH(lc, (gemv_pro_kernel<TB, false, true, MR>), dim3(blocks, 1, 1), 256, g);
+  const uint32_t xv = ((MR > 1 ? g.rows : 1u) * g.m.K / 4 + 255) / 256;
+  if (xv <= 2) CG_LAUNCH(lc, (gemv_pro_kernel<TB, false, true, MR, 2>), dim3(blocks, 1, 1), 256, g);
+  else if (xv <= 4) CG_LAUNCH(lc, (gemv_pro_kernel<TB, false, true, MR, 4>), dim3(blocks, 1, 1), 256, g);
+  else CG_LAUNCH(lc, (gemv_pro_kernel<TB, false, true, MR, 8>), dim3(blocks, 1, 1), 256, g);
 }
 
 uint32_t gemv_pro_multi_row_max_k(int b_stype) { return 64u * (b_stype == ST_BF16 ? 8u : 4u) * 4u; }
