@@ -501,6 +501,7 @@ __global__ void __launch_bounds__(WR *WC * 64) gemm_bf16_dma_kernel(GemmDesc g) 
   constexpr int LPW = (BM_ + BN_) / 8 / NW;   // 1 KB loads per wave per stage
   constexpr int STAGE = (BM_ + BN_) * BK * 2;  // bytes
   extern __shared__ __attribute__((aligned(16))) uint16_t dma_smem[];
+  warm_kernel_arguments<sizeof(GemmDesc)>();
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / WC, wn = wave % WC;
