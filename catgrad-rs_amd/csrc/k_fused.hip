@@ -535,6 +535,15 @@ __global__ void __launch_bounds__(256) attn_decode_split_kernel(AttnDecodeDesc a
       a.out[((uint64_t)b * a.heads + h) * a.d + tid] = o / L;
       return;
     }
+    if (a.merge_later) {  // the reader of the result merges: plain stores, the kernel boundary orders them
+      float *rec = a.part + (((uint64_t)b * a.heads + h) * a.splits + c) * (a.d + 4);
+      rec[tid] = o;
+      if (tid == 0) {
+        rec[a.d] = M;
+        rec[a.d + 1] = L;
+      }
+      return;
+    }
     // The hand-over to the merging workgroup (another compute unit, usually another XCD).  A release
     // fence at agent scope would do it by the book, but it also writes back every dirty line of this
     // XCD's L2 (5 us per launch, measured); the partials need less.  They are agent-scope atomic
@@ -549,7 +558,7 @@ __global__ void __launch_bounds__(256) attn_decode_split_kernel(AttnDecodeDesc a
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   }
-  if (a.splits == 1) return;
+  if (a.splits == 1 || a.merge_later) return;
   __syncthreads();
   uint32_t *counter = a.count + (uint64_t)b * a.heads + h;
   if (tid == 0)

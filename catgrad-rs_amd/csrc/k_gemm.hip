@@ -1071,13 +1071,21 @@ hipError_t launch_gemv_multi(const LaunchCtx &lc, const GemvMultiDesc &g) {
 // staged (rows * K <= GEMV_PRO_MAX_K), every weight vector fetched is used for each of them, and the
 // outputs are the rows of a contiguous [rows, N] matrix.
 // XV: 16-byte pieces of the input rows per thread (rows * K <= XV * 1024 floats).
-template <typename TB, bool KSPLIT, bool GLUEPI, int MR, int XV>
+// MERGE (PRO_ATTN_MERGE): the input row is the result of a split decode attention that stopped at its
+// partials; every workgroup merges them on its way in - the maxima and sums of all (head, split) records,
+// one per thread, meet in LDS, and a thread combines the value pieces of its positions with the weights
+// exp(max_s - max) / sum.  All of it is requested with the first loads, so the attention launch needs no
+// hand-over between its workgroups (acknowledged stores, a counter, a second pass over the partials:
+// 2.8 us of a 6.7 us kernel) and the merge costs this launch one LDS exchange.
+template <typename TB, bool KSPLIT, bool GLUEPI, int MR, int XV, bool MERGE = false>
 __global__ void __launch_bounds__(256) gemv_pro_kernel(GemvProDesc g) {
   typedef typename WVec<TB>::type VT;
   constexpr int EPL = WVec<TB>::EPL, UNROLL = 4, R = 2;
   __shared__ __attribute__((aligned(16))) float xs[GEMV_PRO_MAX_K];
   __shared__ float lds[4 * MR];
   __shared__ float part[4][R][MR];
+  __shared__ float2 merge_ml[MERGE ? 256 : 1];
+  static_assert(!MERGE || (MR == 1 && !GLUEPI && !KSPLIT), "the attention merge feeds one row to a plain product");
   warm_kernel_arguments<sizeof(GemvProDesc)>();
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const uint32_t K = g.m.K, bz = blockIdx.z;
@@ -1143,19 +1151,59 @@ __global__ void __launch_bounds__(256) gemv_pro_kernel(GemvProDesc g) {
   const int64_t aux_rs = !has_aux ? g.a_rstride : g.pro == PRO_RMSNORM ? 0 : g.aux_rstride;
   float4 xv[XV], gv[XV];
   uint32_t pm[XV], pk[XV];
+  constexpr int MS = MERGE ? ATTN_MERGE_MAX_SPLITS : 1;
+  float4 mv[XV][MS];  // MERGE: the value pieces of every split
+  float2 my_ml = make_float2(0.f, 0.f);
+  if constexpr (MERGE) {
+    const uint32_t pw = g.merge_d + 4, records = g.merge_heads * g.merge_splits;
+    my_ml = *(const float2 *)(g.merge_part + (uint64_t)min((uint32_t)tid, records - 1) * pw + g.merge_d);
 #pragma unroll
-  for (int j = 0; j < XV; ++j) {
-    const uint32_t e = min((uint32_t)tid + j * 256u, pieces - 1) * 4;
-    pm[j] = MR == 1 ? 0u : e / K;
-    pk[j] = MR == 1 ? e : e % K;
-    xv[j] = *(const float4 *)(ga + (int64_t)pm[j] * g.a_rstride + pk[j]);
+    for (int j = 0; j < XV; ++j) {
+      const uint32_t e = min((uint32_t)tid + j * 256u, pieces - 1) * 4;
+      pm[j] = 0u;
+      pk[j] = e;
+      const uint32_t h = e / g.merge_d, t = e % g.merge_d;
+#pragma unroll
+      for (int sp = 0; sp < MS; ++sp)
+        mv[j][sp] = *(const float4 *)(g.merge_part + (uint64_t)(h * g.merge_splits + min((uint32_t)sp, g.merge_splits - 1)) * pw + t);
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < XV; ++j) {
+      const uint32_t e = min((uint32_t)tid + j * 256u, pieces - 1) * 4;
+      pm[j] = MR == 1 ? 0u : e / K;
+      pk[j] = MR == 1 ? e : e % K;
+      xv[j] = *(const float4 *)(ga + (int64_t)pm[j] * g.a_rstride + pk[j]);
+    }
+#pragma unroll
+    for (int j = 0; j < XV; ++j) gv[j] = *(const float4 *)(aux_base + (int64_t)pm[j] * aux_rs + pk[j]);
   }
-#pragma unroll
-  for (int j = 0; j < XV; ++j) gv[j] = *(const float4 *)(aux_base + (int64_t)pm[j] * aux_rs + pk[j]);
   bool requested = true;
   request(min(slot * CPS, N - 1), k_begin + lane * EPL);
   // ---- prologue: the input rows, from the registers loaded above into LDS
-  if (g.pro == PRO_RMSNORM) {
+  if constexpr (MERGE) {
+    merge_ml[tid] = my_ml;  // record (head, split) = tid: (maximum, sum)
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < XV; ++j)
+      if (tid + j * 256 < pieces) {
+        const uint32_t h = pk[j] / g.merge_d;
+        const float2 *ml = merge_ml + h * g.merge_splits;
+        float mx = -3.40282347e+38f;
+        for (uint32_t sp = 0; sp < g.merge_splits; ++sp) mx = fmaxf(mx, ml[sp].x);
+        float l = 0.f;
+        float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+        for (int sp = 0; sp < MS; ++sp)
+          if ((uint32_t)sp < g.merge_splits) {
+            const float w = __expf(ml[sp].x - mx);
+            l += w * ml[sp].y;
+            o.x += w * mv[j][sp].x; o.y += w * mv[j][sp].y; o.z += w * mv[j][sp].z; o.w += w * mv[j][sp].w;
+          }
+        o.x /= l; o.y /= l; o.z /= l; o.w /= l;
+        *(float4 *)(xs + pk[j]) = o;
+      }
+  } else if (g.pro == PRO_RMSNORM) {
     float ssq[MR];
 #pragma unroll
     for (int m = 0; m < MR; ++m) ssq[m] = 0.f;
@@ -1335,6 +1383,20 @@ hipError_t launch_gemv_pro(const LaunchCtx &lc, const GemvProDesc &g) {
   uint32_t max_n = 0;
   for (int i = 0; i < g.m.n_prob; ++i) max_n = g.m.p[i].N > max_n ? g.m.p[i].N : max_n;
   if (!max_n || !g.m.n_prob) return hipSuccess;
+  if (g.pro == PRO_ATTN_MERGE) {
+    if (!g.merge_part || g.merge_splits < 1 || g.merge_splits > ATTN_MERGE_MAX_SPLITS || g.merge_d % 4 || !g.merge_d ||
+        g.merge_heads * g.merge_splits > 256 || g.m.K != g.merge_heads * g.merge_d || g.m.K > 2048 || g.m.K % 8 ||
+        g.rows > 1 || g.batch > 1 || g.b_index || g.slot_tokens || g.glu_epilogue)
+      return hipErrorInvalidValue;
+    const uint32_t slots = (max_n + 1) / 2;
+    uint32_t blocks = (slots + 3) / 4;
+    const uint32_t cap = (uint32_t)lc.n_cus * 4 / g.m.n_prob;
+    if (blocks > cap) blocks = cap ? cap : 1;
+    dim3 grid(blocks, g.m.n_prob, 1);
+    if (g.m.b_stype == ST_BF16) CG_LAUNCH(lc, (gemv_pro_kernel<uint16_t, false, false, 1, 2, true>), grid, 256, g);
+    else CG_LAUNCH(lc, (gemv_pro_kernel<float, false, false, 1, 2, true>), grid, 256, g);
+    return hipGetLastError();
+  }
   const bool multi = g.rows > 1;  // several input rows share the weights
   // several rows: one pass over k per column (K <= 64 lanes x 16 bytes x 4 loads)
   if (multi && (g.rows > 4 || (uint64_t)g.rows * g.m.K > GEMV_PRO_MAX_K || g.batch > 1 || g.b_index || g.slot_tokens ||

@@ -179,6 +179,11 @@ struct AttnDecodeDesc {
   uint32_t splits, chunk;
   float *part;
   uint32_t *count;
+  // splits >= 2 only: stop after the partials and leave their merge to the kernel that reads the result
+  // (GemvProDesc::pro == PRO_ATTN_MERGE).  part then holds, per (batch, head, split), d values, the
+  // maximum, the sum and two unused floats (stride d + 4: every record 16-byte aligned); out and count
+  // are not touched.
+  int32_t merge_later;
 };
 enum { ATTN_DECODE_MAX_T = 8192, ATTN_DECODE_MAX_D = 256 };
 // keys one workgroup of the split form visits per pass over its chunk
@@ -305,7 +310,10 @@ hipError_t launch_gemv_multi(const LaunchCtx &lc, const GemvMultiDesc &g);
 // input row (a + z * a_bstride, aux + z * aux_bstride), its own output rows (c + z * N) and reads
 // the weight matrices of expert b_index[z * b_index_stride] (b + index * sb_index); an index >=
 // b_index_limit raises ERRF_INDEX_OOB in *err and is clamped.
-enum { PRO_NONE = 0, PRO_RMSNORM = 1, PRO_SWIGLU = 2, PRO_GEGLU = 3, GEMV_PRO_MAX_K = 8192 };
+//   PRO_ATTN_MERGE: x = the output row of a split decode attention launched with merge_later, merged here
+//     from its partials (one row, K = heads * d <= 2048, at most 8 splits, heads * splits <= 256); a is unused
+enum { PRO_NONE = 0, PRO_RMSNORM = 1, PRO_SWIGLU = 2, PRO_GEGLU = 3, PRO_ATTN_MERGE = 4, GEMV_PRO_MAX_K = 8192 };
+enum { ATTN_MERGE_MAX_SPLITS = 8 };
 struct GemvProDesc {
   GemvMultiDesc m;  // m.x is ignored
   int32_t pro;
@@ -332,6 +340,9 @@ struct GemvProDesc {
   uint32_t slot_tokens;
   int32_t a_by_token;
   const uint32_t *b_index_slot[8];
+  // PRO_ATTN_MERGE: the attention's partials (AttnDecodeDesc::part with merge_later) and their geometry
+  const float *merge_part;
+  uint32_t merge_splits, merge_heads, merge_d;
 };
 hipError_t launch_gemv_pro(const LaunchCtx &lc, const GemvProDesc &g);
 // largest K the several-row form takes for weights of this storage type

@@ -312,7 +312,7 @@ int write_row_append(cg_backend *be, const RowAppend &ra) {
 }
 
 
-int try_attn_decode(cg_backend *be, cg_tensor *n, bool *done) {
+int try_attn_decode(cg_backend *be, cg_tensor *n, bool *done, AttnMergeLater *later) {
   cg_tensor *P = n->in[0];
   if (P->op == N_REAL || refs(P) != 1 || P->rank != 4) return CG_OK;
   SoftmaxMatch m;
@@ -442,9 +442,20 @@ int try_attn_decode(cg_backend *be, cg_tensor *n, bool *done) {
       const int64_t chunk = (T + ns - 1) / ns;
       a.chunk = (uint32_t)chunk;
       a.splits = (uint32_t)((T + chunk - 1) / chunk);
-      TRY(attn_decode_scratch(be, (size_t)bh * a.splits * (d + 2), (size_t)bh));
+      // the reader of the result merges the partials when it can (one row, few splits)
+      if (later && nb == 1 && a.splits >= 2 && a.splits <= ATTN_MERGE_MAX_SPLITS && heads * a.splits <= 256 &&
+          heads * d <= 2048 && d % 4 == 0)
+        a.merge_later = 1;
+      TRY(attn_decode_scratch(be, (size_t)bh * a.splits * (d + 4), (size_t)bh));
       a.part = be->attn_part;
       a.count = be->attn_count;
+      if (a.merge_later) {
+        later->part = a.part;
+        later->splits = a.splits;
+        later->heads = (uint32_t)heads;
+        later->d = (uint32_t)d;
+        later->deferred = true;
+      }
     }
     const double kv_bytes = 2.0 * nb * Kop.shape[1] * T * d * 4;
     KernelScope ks(be, "attn_decode", kv_bytes + 2.0 * nb * heads * d * 4, 4.0 * nb * heads * T * d);

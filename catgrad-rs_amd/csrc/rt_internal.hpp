@@ -148,7 +148,16 @@ cg_tensor *kv_concat_under(cg_tensor *t);
 int row_append_candidate(cg_backend *be, cg_tensor *c, bool allow_rope, RowAppend *out, bool *ok);
 void commit_row_append(cg_tensor *c);
 int write_row_append(cg_backend *be, const RowAppend &ra);
-int try_attn_decode(cg_backend *be, cg_tensor *n, bool *done);
+// later (optional): when the launch divides the keys over workgroups and the caller can merge the
+// partials itself (launch_gemv_pro with PRO_ATTN_MERGE), the attention stops at its partials, *later
+// describes them and n's own storage is left unwritten.
+struct AttnMergeLater {
+  const float *part = nullptr;
+  uint32_t splits = 0, heads = 0, d = 0;
+  bool deferred = false;
+};
+int try_attn_decode(cg_backend *be, cg_tensor *n, bool *done, AttnMergeLater *later = nullptr);
+int try_gemv_attn_merge(cg_backend *be, cg_tensor *n, cg_tensor *addend, bool *added, bool *done);
 cg_tensor *rows_base(cg_tensor *t);
 int try_gate_up_glu(cg_backend *be, cg_tensor *glu, cg_tensor *g, cg_tensor *u, int gelu, bool *done);
 int try_gemv_prologue(cg_backend *be, cg_tensor *n, cg_tensor *addend, bool *added, bool *done);

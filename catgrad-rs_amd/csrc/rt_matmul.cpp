@@ -380,6 +380,71 @@ int try_gemv_prologue(cg_backend *be, cg_tensor *n, cg_tensor *addend, bool *add
 }
 
 
+// o_proj of a decode step: a one-row product whose input row is the attention of this step, seen through
+// the head merge (`transpose(1, 2)` + `reshape [b, 1, heads * d]`, models/llama.rs:107-110; one batch row, so
+// both are views of the same memory order) and read by nobody else.  The attention is launched here and
+// stops at the partial results of its key ranges; this product's kernel merges them on its way in, so
+// the attention needs no hand-over between its workgroups and its value is never stored.
+int try_gemv_attn_merge(cg_backend *be, cg_tensor *n, cg_tensor *addend, bool *added, bool *done) {
+  if (!n->gemv_candidate) return CG_OK;
+  cg_tensor *att = n->in[0];
+  while ((att->op == N_RESHAPE || att->op == N_TRANSPOSE) && refs(att) == 1) att = att->in[0];
+  if (att == n->in[0] || att->op != N_MATMUL || att->dtype != CG_F32 || att->rank != 4 || refs(att) != 1) return CG_OK;
+  if (att->shape[0] != 1 || att->shape[2] != 1) return CG_OK;
+  const int64_t K = att->shape[1] * att->shape[3];
+  cg_tensor *w = n->in[1];
+  if (n->in[0]->size() != K || K % 8 || K < 256 || K > 2048 || n->size() != n->shape[n->rank - 1]) return CG_OK;
+  TRY(realize(be, w));
+  if (w->rank < 2 || w->shape[w->rank - 2] != K || w->strides[w->rank - 2] != 1) return CG_OK;
+  for (int i = 0; i + 2 < w->rank; ++i)
+    if (w->shape[i] != 1 && w->strides[i] != 0) return CG_OK;
+  if (w->stype != ST_F32 && w->stype != ST_BF16) return CG_OK;
+  if ((uintptr_t)data_ptr(w) % 16 || w->strides[w->rank - 1] % (16 / esize(w->stype))) return CG_OK;
+  if (addend && (addend->stype != ST_F32 || be->addend_is_row)) return CG_OK;
+  AttnMergeLater later;
+  bool att_done = false;
+  TRY(try_attn_decode(be, att, &att_done, &later));
+  if (!att_done || !later.deferred) return CG_OK;  // not an attention, or one that wrote its result: the usual path
+  int st = alloc_result(be, n, ST_F32);
+  if (st) return st;
+  GemvProDesc d;
+  std::memset(&d, 0, sizeof(d));
+  d.pro = PRO_ATTN_MERGE;
+  d.merge_part = later.part;
+  d.merge_splits = later.splits;
+  d.merge_heads = later.heads;
+  d.merge_d = later.d;
+  d.m.K = (uint32_t)K;
+  d.m.n_prob = 1;
+  d.m.b_stype = w->stype;
+  d.m.p[0].b = data_ptr(w);
+  d.m.p[0].c = (float *)n->st->ptr;
+  d.m.p[0].c_add = addend ? (const float *)data_ptr(addend) : nullptr;
+  d.m.p[0].sbn = w->strides[w->rank - 1];
+  d.m.p[0].N = (uint32_t)w->shape[w->rank - 1];
+  d.err = be->d_words;
+  d.b_index_limit = 1;
+  {
+    const double N = (double)d.m.p[0].N;
+    const char *base = w->stype == ST_BF16 ? "gemv_rowdot_bf16" : "gemv_rowdot_f32";
+    KernelScope ks(be, base, N * K * esize(w->stype) + K * 4 + N * 4, 2.0 * N * K);
+    if (be->trace_shapes) {
+      char buf[96];
+      snprintf(buf, sizeof buf, "%s[attn-merge,M1,K%lld,N%.0f]", base, (long long)K, N);
+      ks.rename(buf);
+    }
+    hipError_t e = launch_gemv_pro(be->lc(), d);
+    if (e != hipSuccess) return fail(be, CG_ERR_DEVICE, hipGetErrorString(e));
+  }
+  if (addend) *added = true;
+  forget_gemv_candidate(n);
+  n->op = N_REAL;
+  drop_inputs(n);  // lets go of the head-merge views and, with them, of the attention node
+  *done = true;
+  return CG_OK;
+}
+
+
 // `addend` (optional; realised, f32, contiguous, shaped like n) is added in the epilogue when a
 // one-row kernel runs the product; *added tells the caller whether that happened.
 int realize_matmul(cg_backend *be, cg_tensor *n, cg_tensor *addend, bool *added, MatmulEpilogue *ep) {
@@ -398,6 +463,8 @@ int realize_matmul(cg_backend *be, cg_tensor *n, cg_tensor *addend, bool *added,
     if (!addend) TRY(try_moe_gemv(be, n, &done));
     if (done) return CG_OK;
     TRY(try_gemv_prologue(be, n, addend, added, &done));
+    if (done) return CG_OK;
+    TRY(try_gemv_attn_merge(be, n, addend, added, &done));
     if (done) return CG_OK;
   }
   MatOperand A, B;
