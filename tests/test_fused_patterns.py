@@ -371,6 +371,51 @@ def test_attention_decode(oracle, hip, hip_nopat, cfg):
     assert np.allclose(gen[0], ref, rtol=1e-4, atol=1e-5)
 
 
+@pytest.mark.parametrize("T", [20, 40, 300, 540, 1000, 1500])
+@pytest.mark.parametrize("mode", ["f32", "bf16"])
+def test_attention_decode_merged_by_the_output_projection(oracle, hip, hip_bf16, cg, T, mode):
+    """llama.rs:107-112 for one query row: the attention, the head merge (transpose + reshape) and
+    `residual + o_proj(.)`.  When the keys are divided over 2 .. 8 workgroups per head the attention launch
+    stops at its partial results and the projection's kernel merges them on its way in (a launch named
+    ...[attn-merge...]); shorter and longer caches take the attention kernel's own merge.  Either way the
+    result is the oracle's."""
+    H, KV, d, N = 32, 8, 64, 384
+    g = np.random.default_rng(T)
+    bf = vectors.bf16_round if mode == "bf16" else (lambda a: a)
+    q = g.standard_normal((1, H, 1, d)).astype(np.float32)
+    k = g.standard_normal((1, KV, T, d)).astype(np.float32)
+    v = g.standard_normal((1, KV, T, d)).astype(np.float32)
+    res = g.standard_normal((1, 1, N)).astype(np.float32)
+    w = bf((g.standard_normal((N, H * d)) * 0.05).astype(np.float32))
+    p = {"o.weight": w}
+
+    def f(b, qv, kv, vv, rv):
+        qv, kv, vv, rv = qv + qv - qv, kv + kv - kv, vv + vv - vv, rv + rv - rv
+        kr = helpers.repeat_kv(b, H // KV, kv)
+        vr = helpers.repeat_kv(b, H // KV, vv)
+        attn = lang.matmul(b, qv, lang.transpose(b, 2, 3, kr))
+        sh = lang.shape(b, attn)
+        attn = attn / lang.constant(b, float(np.sqrt(np.float32(d))), sh)
+        attn = attn + lang.broadcast(b, helpers.causal_mask(b, lang.to_nat(b, 1)), sh)
+        out = lang.matmul(b, nn.softmax(b, attn), vr)
+        out = lang.reshape(b, lang.make_shape(b, 1, 1, H * d), lang.transpose(b, 1, 2, out))
+        return rv + nn.linear_no_bias(b, H * d, N, lang.path(["o"]), out)
+    (ref,) = vectors.run(oracle, f, 1, q, k, v, res, params=p)
+    be = hip_bf16 if mode == "bf16" else hip
+    be.trace(2)
+    be.trace_reset()
+    (got,) = vectors.run(be, f, 1, q, k, v, res, params=p)
+    names = set(be.trace_report())
+    be.trace(False)
+    assert any(nm.startswith("attn_decode") for nm in names), sorted(names)
+    merged = any("attn-merge" in nm for nm in names)
+    ns = max(-(-T // 128), min(8, -(-T // 32)))              # the runtime's rule for 32 heads on 256 CUs
+    splits = -(-T // -(-T // ns)) if ns >= 2 else 1
+    assert merged == (2 <= splits <= 8), (splits, sorted(names))
+    tol = 2e-2 if mode == "bf16" else 1e-4
+    assert np.max(np.abs(got - ref)) <= tol * np.abs(ref).max(), np.max(np.abs(got - ref)) / np.abs(ref).max()
+
+
 def test_attention_decode_that_cannot_be_fused_still_appends_its_rows(oracle, hip_bf16, cg):
     """A decode step whose caches qualify for the append inside the attention kernel, but whose query
     does not (an uploaded rank-4 tensor is bf16 storage in bf16 mode): the new key and value rows must
