@@ -438,6 +438,11 @@ int try_attn_decode(cg_backend *be, cg_tensor *n, bool *done, AttnMergeLater *la
     const int64_t bh = nb * heads, rpp = attn_decode_rows_per_pass((uint32_t)d);
     int64_t ns = std::max((T + rpp - 1) / rpp, std::min((be->n_cus + bh - 1) / bh, (T + 31) / 32));
     ns = std::min<int64_t>(ns, 64);
+    // When the reader merges the partials (every one of its workgroups reads all of them), fewer and
+    // longer key ranges pay: about one pass of a workgroup each, three ranges at least.  Swept on the
+    // whole decode loop: T ~ 540: 4 ranges 1367, 5 1392, 6 1382, 8 1372 tokens/s; T ~ 200: 2 1415, 3 1421,
+    // 4 1421, 8 1397.
+    if (later && nb == 1 && ns <= ATTN_MERGE_MAX_SPLITS) ns = std::max<int64_t>((T + 109) / 110, std::min<int64_t>(3, (T + 31) / 32));
     if (ns >= 2 || T > ATTN_DECODE_MAX_T) {
       const int64_t chunk = (T + ns - 1) / ns;
       a.chunk = (uint32_t)chunk;
