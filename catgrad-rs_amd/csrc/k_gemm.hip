@@ -1369,7 +1369,9 @@ template <typename TB, int MR>
 static void launch_gemv_pro_glu(const LaunchCtx &lc, const GemvProDesc &g) {
   const uint32_t slots = g.m.p[0].N;  // one (gate, up) column pair per wave pass
   uint32_t blocks = (slots + 3) / 4;
-  const uint32_t cap = (uint32_t)lc.n_cus * (MR > 1 ? 2 : 4);
+  // two workgroups per CU, each wave walking several column pairs: swept on the whole decode loop (workgroups
+  // per CU: 1 -> 1344, 2 -> 1400-1407, 3 -> 1401, 4 -> 1383 tokens/s; more than four, with LDS sized per launch, 1323)
+  const uint32_t cap = (uint32_t)lc.n_cus * 2;
   if (blocks > cap) blocks = cap;
   const uint32_t xv = ((MR > 1 ? g.rows : 1u) * g.m.K / 4 + 255) / 256;
   if (xv <= 2) CG_LAUNCH(lc, (gemv_pro_kernel<TB, false, true, MR, 2>), dim3(blocks, 1, 1), 256, g);
