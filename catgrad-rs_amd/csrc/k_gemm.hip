@@ -1381,6 +1381,237 @@ static void launch_gemv_pro_glu(const LaunchCtx &lc, const GemvProDesc &g) {
 
 uint32_t gemv_pro_multi_row_max_k(int b_stype) { return 64u * (b_stype == ST_BF16 ? 8u : 4u) * 4u; }
 
+// ---- a few input rows against shared bf16 weights, on the matrix cores ---------------------------------
+// A decode step of a small batch multiplies 2 to 16 rows by every weight matrix.  The kernel above does
+// that with one multiply-add per lane, weight and row, and at four rows its arithmetic, not the stream of
+// weights, sets the pace (17 us for 25 MB).  Here a weight vector goes from memory straight into the A
+// operand of v_mfma_f32_16x16x32_bf16 - lane (n = lane & 15, kb = lane >> 4) holds k = kb * 8 .. + 7 of
+// column n, 16 bytes of that column's row.  Loaded by that lane itself, neighbouring lanes would read
+// from 16 different rows and the address unit, not memory, would set the pace (3.5 us for 64 KB per
+// workgroup); so lane l loads piece l & 3 of column l >> 2 - four neighbours share 64 bytes - and
+// ds_bpermute hands every piece to the lane that multiplies it.  The input rows, narrowed to bf16 in
+// LDS by the prologue (RMSNorm, SwiGLU / GeGLU or none, as above), are the B operand: lane (m, kb)
+// reads row m, or zeros past the last row.  A workgroup owns groups of 16 output columns; its four waves
+// take a quarter of k each (K % 128 == 0) and meet in LDS, where thread (m, n) adds the four quarters,
+// applies the epilogue and stores.  D[n][m] sits in lane m + 16 * (n / 4), register n % 4.
+// The inputs are rounded to bf16 like those of every many-row product in bf16 mode.
+// XV: 16-byte pieces of the input rows per lane in the RMSNorm prologue, where a wave owns whole rows
+// (rows wave, wave + 4, ...) so that a row's sum of squares never leaves the wave.
+enum { GEMV_ROWS_MAX = 16, GEMV_ROWS_LDS = 24576 };
+template <bool GLUEPI, int XV>
+__global__ void __launch_bounds__(256) gemv_rows_mfma_kernel(GemvProDesc g) {
+  typedef WVec<uint16_t>::type VT;
+  constexpr int UN = GLUEPI ? 8 : 16, NM = GLUEPI ? 2 : 1;  // k-steps of 32 in flight per wave; weight matrices
+  __shared__ __attribute__((aligned(16))) uint16_t xs[GEMV_ROWS_LDS];  // [rows][K + 8] bf16
+  __shared__ float red[NM][4][16][17];
+  warm_kernel_arguments<sizeof(GemvProDesc)>();
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r = lane & 15, kb = lane >> 4;
+  const uint32_t K = g.m.K, rows = g.rows, pitch = K + 8;
+  const uint32_t N = g.m.p[blockIdx.y].N, groups = (N + 15) / 16;
+  if (blockIdx.x >= groups) return;  // the narrower problems of a grouped launch
+  const uint16_t *B = (const uint16_t *)g.m.p[blockIdx.y].b;
+  const uint16_t *B2 = GLUEPI ? (const uint16_t *)g.m.p[1].b : nullptr;
+  const int64_t sbn = g.m.p[blockIdx.y].sbn, sbn2 = GLUEPI ? g.m.p[1].sbn : 0;
+  float *C = g.m.p[blockIdx.y].c;
+  const float *Cadd = g.m.p[blockIdx.y].c_add;
+  const uint32_t cadd_rs = g.m.p[blockIdx.y].c_add_is_row ? 0u : N;
+  const uint32_t spw = K / 128;              // k-steps of this wave
+  const uint32_t k_begin = wave * spw * 32;  // and where they start
+  // Every request is NM * UN loads, no fewer (steps past the wave's last repeat it and are not used), so
+  // the prologue's wait for its own, older loads is a count that leaves these in flight.
+  VT q[NM][UN];
+  auto request = [&](uint32_t group, uint32_t s0) {
+    const uint32_t n = min(group * 16 + (lane >> 2), N - 1);
+    const uint16_t *p0 = B + (int64_t)n * sbn + k_begin + (lane & 3) * 8;
+    const uint16_t *p1 = GLUEPI ? B2 + (int64_t)n * sbn2 + k_begin + (lane & 3) * 8 : nullptr;
+#pragma unroll
+    for (int u = 0; u < UN; ++u) {
+      const uint32_t s = min(s0 + u, spw - 1);
+      q[0][u] = __builtin_nontemporal_load((const VT *)(p0 + s * 32));
+      if (GLUEPI) q[NM - 1][u] = __builtin_nontemporal_load((const VT *)(p1 + s * 32));
+    }
+  };
+  auto narrow = [](const float4 &o) {
+    union { bf16x2_t h[2]; uint2 u; } pk;
+    pk.h[0] = __builtin_convertvector((f32x2_t){o.x, o.y}, bf16x2_t);
+    pk.h[1] = __builtin_convertvector((f32x2_t){o.z, o.w}, bf16x2_t);
+    return pk.u;
+  };
+  // ---- the input rows, to LDS as bf16
+  if (g.pro == PRO_RMSNORM) {
+    const uint32_t ppr = (K + 255) / 256;  // pieces of a row per lane; slot j = (row slot j / ppr, piece j % ppr)
+    float4 xv[XV], gv[XV];
+    {
+      uint32_t rs = 0, i = 0;
+#pragma unroll
+      for (int j = 0; j < XV; ++j) {
+        const uint32_t row = min(wave + 4 * rs, rows - 1), k = min((lane + 64 * i) * 4, K - 4);
+        xv[j] = *(const float4 *)(g.a + (int64_t)row * g.a_rstride + k);
+        gv[j] = *(const float4 *)((g.aux ? g.aux : g.a) + k);  // gamma: one vector for every row
+        if (++i == ppr) { i = 0; ++rs; }
+      }
+    }
+    request(blockIdx.x, 0);
+    float ssq[4] = {0.f, 0.f, 0.f, 0.f};
+    {
+      uint32_t rs = 0, i = 0;
+#pragma unroll
+      for (int j = 0; j < XV; ++j) {
+        const bool valid = wave + 4 * rs < rows && (lane + 64 * i) * 4 < K;
+        const float s = valid ? xv[j].x * xv[j].x + xv[j].y * xv[j].y + xv[j].z * xv[j].z + xv[j].w * xv[j].w : 0.f;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) ssq[t] += rs == (uint32_t)t ? s : 0.f;
+        if (++i == ppr) { i = 0; ++rs; }
+      }
+    }
+    float rms[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) rms[t] = sqrtf(wave_sum(ssq[t]) / g.n_as_float + g.eps);
+    {
+      uint32_t rs = 0, i = 0;
+#pragma unroll
+      for (int j = 0; j < XV; ++j) {
+        const uint32_t row = wave + 4 * rs, k = (lane + 64 * i) * 4;
+        if (row < rows && k < K) {
+          float d = rms[0];
+#pragma unroll
+          for (int t = 1; t < 4; ++t) d = rs == (uint32_t)t ? rms[t] : d;
+          float4 o;
+          o.x = xv[j].x / d; o.y = xv[j].y / d; o.z = xv[j].z / d; o.w = xv[j].w / d;
+          if (g.aux) {
+            o.x *= g.gamma_offset + gv[j].x; o.y *= g.gamma_offset + gv[j].y;
+            o.z *= g.gamma_offset + gv[j].z; o.w *= g.gamma_offset + gv[j].w;
+          }
+          *(uint2 *)(xs + (size_t)row * pitch + k) = narrow(o);
+        }
+        if (++i == ppr) { i = 0; ++rs; }
+      }
+    }
+  } else {
+    // elementwise prologues: the pieces of all rows, 8 per thread and pass
+    const uint32_t kp = K / 4, pieces = rows * kp;
+    const bool glu = g.pro != PRO_NONE;
+    float4 xv[8], gv[8];
+    auto load_pass = [&](uint32_t p0) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const uint32_t p = min(p0 + tid + j * 256u, pieces - 1), m = p / kp, k = (p - m * kp) * 4;
+        xv[j] = *(const float4 *)(g.a + (int64_t)m * g.a_rstride + k);
+        gv[j] = *(const float4 *)(glu ? g.aux + (int64_t)m * g.aux_rstride + k : g.a + (int64_t)m * g.a_rstride + k);
+      }
+    };
+    auto store_pass = [&](uint32_t p0) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const uint32_t p = p0 + tid + j * 256u;
+        if (p < pieces) {
+          const uint32_t m = p / kp, k = (p - m * kp) * 4;
+          float4 o = xv[j];
+          if (g.pro == PRO_GEGLU) {
+            o.x = gelu_ref(o.x) * gv[j].x; o.y = gelu_ref(o.y) * gv[j].y;
+            o.z = gelu_ref(o.z) * gv[j].z; o.w = gelu_ref(o.w) * gv[j].w;
+          } else if (g.pro == PRO_SWIGLU) {
+            o.x = o.x * sigmoid_ref(o.x) * gv[j].x; o.y = o.y * sigmoid_ref(o.y) * gv[j].y;
+            o.z = o.z * sigmoid_ref(o.z) * gv[j].z; o.w = o.w * sigmoid_ref(o.w) * gv[j].w;
+          }
+          *(uint2 *)(xs + (size_t)m * pitch + k) = narrow(o);
+        }
+      }
+    };
+    load_pass(0);
+    request(blockIdx.x, 0);
+    store_pass(0);
+    for (uint32_t p0 = 2048; p0 < pieces; p0 += 2048) {
+      load_pass(p0);
+      store_pass(p0);
+    }
+  }
+  __syncthreads();
+  // ---- the products
+  const bool live = (uint32_t)r < rows;
+  const uint16_t *xrow = xs + (size_t)min((uint32_t)r, rows - 1) * pitch + k_begin + kb * 8;
+  const int from = (4 * r + kb) * 4;  // ds_bpermute: the lane that loaded piece kb of column r
+  for (uint32_t group = blockIdx.x; group < groups; group += gridDim.x) {
+    f32x4n acc[NM];
+#pragma unroll
+    for (int e = 0; e < NM; ++e) acc[e] = (f32x4n){0.f, 0.f, 0.f, 0.f};
+    for (uint32_t s0 = 0; s0 < spw; s0 += UN) {
+      VT cur[NM][UN];
+#pragma unroll
+      for (int e = 0; e < NM; ++e)
+#pragma unroll
+        for (int u = 0; u < UN; ++u) cur[e][u] = q[e][u];
+      // the next vectors - of this group, or the first of the workgroup's next group - while these multiply
+      if (s0 + UN < spw) request(group, s0 + UN);
+      else if (group + gridDim.x < groups) request(group + gridDim.x, 0);
+#pragma unroll
+      for (int u = 0; u < UN; ++u)
+        if (s0 + u < spw) {
+          union { uint4 u4; bf16x8 h; } xb;
+          xb.u4 = *(const uint4 *)(xrow + (s0 + u) * 32);
+          if (!live) xb.u4 = make_uint4(0u, 0u, 0u, 0u);
+#pragma unroll
+          for (int e = 0; e < NM; ++e) {
+            union { VT v; bf16x8 h; } w;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) w.v[c] = __builtin_amdgcn_ds_bpermute(from, cur[e][u][c]);
+            acc[e] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w.h, xb.h, acc[e], 0, 0, 0);
+          }
+        }
+    }
+    __syncthreads();  // the previous group's sums have been read
+#pragma unroll
+    for (int e = 0; e < NM; ++e)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) red[e][wave][kb * 4 + v][r] = acc[e][v];
+    __syncthreads();
+    const uint32_t m = tid >> 4, n = tid & 15, col = group * 16 + n;
+    if (m < rows && col < N) {
+      float v0 = (red[0][0][n][m] + red[0][1][n][m]) + (red[0][2][n][m] + red[0][3][n][m]);
+      if (GLUEPI) {
+        const float v1 = (red[NM - 1][0][n][m] + red[NM - 1][1][n][m]) + (red[NM - 1][2][n][m] + red[NM - 1][3][n][m]);
+        v0 = (g.glu_epilogue == PRO_GEGLU ? gelu_ref(v0) : v0 * sigmoid_ref(v0)) * v1;
+      } else if (Cadd) {
+        v0 += Cadd[(uint64_t)m * cadd_rs + col];
+      }
+      C[(uint64_t)m * N + col] = v0;
+    }
+  }
+}
+
+// Whether the kernel above takes `rows` input rows of K values with prologue `pro`.
+bool gemv_rows_mfma_ok(int b_stype, uint32_t rows, uint32_t K, int pro) {
+  if (b_stype != ST_BF16 || rows < 2 || rows > GEMV_ROWS_MAX || K < 128 || K % 128) return false;
+  if ((uint64_t)rows * (K + 8) > GEMV_ROWS_LDS) return false;
+  if (pro == PRO_RMSNORM && ((rows + 3) / 4) * ((K + 255) / 256) > 16) return false;
+  return pro == PRO_NONE || pro == PRO_RMSNORM || pro == PRO_SWIGLU || pro == PRO_GEGLU;
+}
+
+bool gemv_pro_rows_ok(int b_stype, uint32_t rows, uint32_t K, int pro) {
+  if (rows <= 1) return rows == 1 && K <= GEMV_PRO_MAX_K;
+  if (gemv_rows_mfma_ok(b_stype, rows, K, pro)) return true;
+  return rows <= 4 && (uint64_t)rows * K <= GEMV_PRO_MAX_K && K <= gemv_pro_multi_row_max_k(b_stype);
+}
+
+static hipError_t launch_gemv_rows_mfma(const LaunchCtx &lc, const GemvProDesc &g, uint32_t max_n) {
+  const uint32_t groups = (max_n + 15) / 16;
+  // two workgroups (56 KB of LDS each) per CU; a workgroup stages the rows once and walks its groups
+  uint32_t cap = (uint32_t)lc.n_cus * 2 / (g.glu_epilogue ? 1 : g.m.n_prob);
+  if (!cap) cap = 1;
+  const uint32_t blocks = groups < cap ? groups : cap;
+  const uint32_t xv = ((g.rows + 3) / 4) * ((g.m.K + 255) / 256);
+  if (g.glu_epilogue) {
+    if (g.pro == PRO_RMSNORM && xv > 8) CG_LAUNCH(lc, (gemv_rows_mfma_kernel<true, 16>), dim3(blocks, 1, 1), 256, g);
+    else CG_LAUNCH(lc, (gemv_rows_mfma_kernel<true, 8>), dim3(blocks, 1, 1), 256, g);
+  } else {
+    if (g.pro == PRO_RMSNORM && xv > 8) CG_LAUNCH(lc, (gemv_rows_mfma_kernel<false, 16>), dim3(blocks, g.m.n_prob, 1), 256, g);
+    else CG_LAUNCH(lc, (gemv_rows_mfma_kernel<false, 8>), dim3(blocks, g.m.n_prob, 1), 256, g);
+  }
+  return hipGetLastError();
+}
+
+
 hipError_t launch_gemv_pro(const LaunchCtx &lc, const GemvProDesc &g) {
   uint32_t max_n = 0;
   for (int i = 0; i < g.m.n_prob; ++i) max_n = g.m.p[i].N > max_n ? g.m.p[i].N : max_n;
@@ -1400,6 +1631,13 @@ hipError_t launch_gemv_pro(const LaunchCtx &lc, const GemvProDesc &g) {
     return hipGetLastError();
   }
   const bool multi = g.rows > 1;  // several input rows share the weights
+  if (multi && g.batch <= 1 && !g.b_index && !g.slot_tokens && gemv_rows_mfma_ok(g.m.b_stype, g.rows, g.m.K, g.pro)) {
+    if (g.glu_epilogue && (g.m.n_prob != 2 || g.m.p[0].N != g.m.p[1].N)) return hipErrorInvalidValue;
+    if ((uintptr_t)g.a % 16 || g.a_rstride % 4 || (g.aux && ((uintptr_t)g.aux % 16 || g.aux_rstride % 4))) return hipErrorInvalidValue;
+    for (int i = 0; i < g.m.n_prob; ++i)
+      if ((uintptr_t)g.m.p[i].b % 16 || g.m.p[i].sbn % 8) return hipErrorInvalidValue;
+    return launch_gemv_rows_mfma(lc, g, max_n);
+  }
   // several rows: one pass over k per column (K <= 64 lanes x 16 bytes x 4 loads)
   if (multi && (g.rows > 4 || (uint64_t)g.rows * g.m.K > GEMV_PRO_MAX_K || g.batch > 1 || g.b_index || g.slot_tokens ||
                 g.m.K > gemv_pro_multi_row_max_k(g.m.b_stype)))
@@ -1989,6 +2227,18 @@ bool gemm_epilogue_ok(const GemmDesc &g) {
   return gemm_fast_path(g, av, bv) && gemm_dma_ok(g) && g.splits <= 1 && !g.b_index && !g.c_add && g.N % 4 == 0;
 }
 
+// A plain product of 2 to 16 rows with bf16 weights [N][K] that gemv_rows_mfma_kernel takes.
+bool gemv_rows_plain_ok(const LaunchCtx &lc, const GemmDesc &g) {
+  // deep and narrow (down_proj of a wide MLP, 4 x 5632 x 2048): fewer 16-column groups than half the CUs, each
+  // a chain of several trips to memory - the vector kernel splits k further and is faster there (12.6 against 16.7 us)
+  if (g.K >= 4096 && (g.N + 15) / 16 * 2 <= (uint32_t)lc.n_cus && g.M <= 8) return false;
+  if (g.M < 2 || g.M > GEMV_ROWS_MAX || g.nb0 * g.nb1 != 1 || g.b_index || g.splits > 1) return false;
+  if (g.a_stype != ST_F32 || g.b_stype != ST_BF16 || !g.bf16_math || g.sak != 1 || g.sbk != 1 || g.N < 64) return false;
+  if (g.glu_gate || g.c16 || g.n_group || g.dual_b || (g.c_add && g.M > 8)) return false;
+  if ((uintptr_t)g.a % 16 || g.sam % 4 || (uintptr_t)g.b % 16 || g.sbn % 8) return false;
+  return gemv_rows_mfma_ok(ST_BF16, g.M, g.K, PRO_NONE);
+}
+
 // Split-K factor for a problem too small to fill the CUs with 128x128 tiles (0/1 = none).
 // The caller provides g.workspace of splits * batch * M * N floats and sets g.splits/k_per_split.
 uint32_t gemm_split_k(const LaunchCtx &lc, const GemmDesc &g) {
@@ -1998,6 +2248,7 @@ uint32_t gemm_split_k(const LaunchCtx &lc, const GemmDesc &g) {
   const int bv = vec_ok(g.b, bsz, g.sbk == 1 ? g.sbn : g.sbk, g.sb_b0, g.sb_b1);
   const uint64_t tiles = (uint64_t)((g.M + 127) / 128) * ((g.N + 127) / 128) * batch;
   uint32_t splits = 1;
+  if (gemv_rows_plain_ok(lc, g)) return 1;
   if (gemm_small_ok(lc, g)) {
     // deep and tiny: more workgroups along k while each wavefront keeps two 32-wide chunks
     const uint64_t t32 = (uint64_t)((g.M + 31) / 32) * ((g.N + 31) / 32) * batch;
@@ -2038,6 +2289,25 @@ hipError_t launch_matmul(const LaunchCtx &lc_in, const GemmDesc &g, const char *
   if (g.c_add && !one_row && g.splits <= 1) return hipErrorInvalidValue;
   if ((g.glu_gate || g.c16 || g.n_group || g.dual_b) && !gemm_epilogue_ok(g)) return hipErrorInvalidValue;
 
+  if (gemv_rows_plain_ok(lc_in, g)) {
+    // a few rows against bf16 weights: the matrix-core kernel, without a prologue
+    if (kernel_name) *kernel_name = "gemv_rows_bf16";
+    GemvProDesc p;
+    std::memset(&p, 0, sizeof(p));
+    p.m.K = g.K;
+    p.m.n_prob = 1;
+    p.m.b_stype = g.b_stype;
+    p.m.p[0].b = g.b;
+    p.m.p[0].c = g.c;
+    p.m.p[0].c_add = g.c_add;
+    p.m.p[0].sbn = g.sbn;
+    p.m.p[0].N = g.N;
+    p.pro = PRO_NONE;
+    p.a = (const float *)g.a;
+    p.rows = g.M;
+    p.a_rstride = g.sam;
+    return launch_gemv_pro(lc, p);
+  }
   if (g.M <= 8 && g.a_stype == ST_F32 && g.K > 0) {
     if (b_unit_k) {
       if (kernel_name) *kernel_name = g.b_stype == ST_BF16 ? "gemv_rowdot_bf16" : "gemv_rowdot_f32";

@@ -324,7 +324,7 @@ struct GemvProDesc {
   int32_t glu_epilogue;
   uint32_t batch;   // 0 or 1: a single row
   int64_t a_bstride, aux_bstride;
-  // 0 / 1, or up to 4 input rows that share the weights (rows * K <= GEMV_PRO_MAX_K, no batch, no b_index):
+  // 0 / 1, or several input rows that share the weights (gemv_pro_rows_ok; no batch, no b_index):
   // row r of the input is a + r * a_rstride (aux + r * aux_rstride; gamma is one vector for all rows) and
   // the outputs (and c_add) are the rows of contiguous [rows, N] matrices
   uint32_t rows;
@@ -345,8 +345,15 @@ struct GemvProDesc {
   uint32_t merge_splits, merge_heads, merge_d;
 };
 hipError_t launch_gemv_pro(const LaunchCtx &lc, const GemvProDesc &g);
-// largest K the several-row form takes for weights of this storage type
+// largest K the several-row form on the vector ALUs takes for weights of this storage type
 uint32_t gemv_pro_multi_row_max_k(int b_stype);
+// most input rows any several-row form takes
+enum { GEMV_PRO_MAX_ROWS = 16 };
+// whether launch_gemv_pro takes `rows` input rows of K values with prologue `pro` against weights of this
+// storage type: one row; up to 4 on the vector ALUs; up to 16 against bf16 weights on the matrix cores
+// (K % 128 == 0, rows * (K + 8) <= 24576, inputs rounded to bf16)
+bool gemv_pro_rows_ok(int b_stype, uint32_t rows, uint32_t K, int pro);
+bool gemv_rows_mfma_ok(int b_stype, uint32_t rows, uint32_t K, int pro);
 // The routed experts of a MoE layer over many tokens (a prefill; models/qwen3.rs:104-123), expert by
 // expert.  A slot is one of the k choices of every token: its index vector, its input rows and its
 // outputs.  A problem is one stacked weight tensor [E, N, K] (bf16): gate_proj and up_proj share

@@ -347,7 +347,9 @@ int cg_matmul(cg_backend *be, cg_tensor *a, cg_tensor *b, cg_tensor **out) {
   n->in[0] = retain(a);
   n->in[1] = retain(b);
   // one input row per batch, or the rows of a small batch folded into one matrix ([1, B, K])
-  const bool few_rows = shape[a->rank - 2] == 1 || (a->rank == 3 && shape[0] == 1 && shape[1] <= 4);
+  // (up to 4 rows on the vector ALUs, up to 16 against bf16 weights on the matrix cores)
+  const bool few_rows = shape[a->rank - 2] == 1 ||
+                        (a->rank == 3 && shape[0] == 1 && shape[1] <= ((be->flags & CG_FLAG_BF16) ? GEMV_PRO_MAX_ROWS : 4));
   if (a->dtype == CG_F32 && few_rows && !(be->flags & CG_FLAG_EAGER)) {
     if (be->gemv_candidates.size() >= 4096) forget_gemv_candidate(be->gemv_candidates.front());
     be->gemv_candidates.push_back(n);

@@ -165,13 +165,13 @@ int try_gate_up_glu(cg_backend *be, cg_tensor *glu, cg_tensor *g, cg_tensor *u, 
   const int64_t K = X->shape[X->rank - 1], N = g->shape[g->rank - 1];
   // one row, or the few rows of a small batch: [B, 1, K] against weights repeated over the batch
   const int64_t rows = K > 0 ? X->size() / K : 0;
-  if (rows < 1 || rows > 4 || X->size() != rows * K || rows * K > GEMV_PRO_MAX_K || g->size() != rows * N || K % 8 || K < 256 ||
+  if (rows < 1 || rows > GEMV_PRO_MAX_ROWS || X->size() != rows * K || g->size() != rows * N || K % 8 || K < 256 ||
       glu->size() != rows * N)
     return CG_OK;
   cg_tensor *ws[2] = {g->in[1], u->in[1]};
   for (cg_tensor *w : ws) {
     TRY(realize(be, w));
-    if (rows > 1 && K > (int64_t)gemv_pro_multi_row_max_k(w->stype)) return CG_OK;
+    if (!gemv_pro_rows_ok(w->stype, (uint32_t)rows, (uint32_t)K, PRO_NONE)) return CG_OK;
     if (w->rank < 2 || w->shape[w->rank - 2] != K || w->strides[w->rank - 2] != 1) return CG_OK;
     for (int i = 0; i + 2 < w->rank; ++i)
       if (w->shape[i] != 1 && w->strides[i] != 0) return CG_OK;
@@ -182,7 +182,8 @@ int try_gate_up_glu(cg_backend *be, cg_tensor *glu, cg_tensor *g, cg_tensor *u, 
   std::memset(&d, 0, sizeof(d));
   RmsNormMatch rm;
   cg_tensor *a0 = nullptr, *a1 = nullptr;
-  if (X->op != N_REAL && refs(X) == 2 && match_rmsnorm(X, &rm)) {
+  if (X->op != N_REAL && refs(X) == 2 && gemv_pro_rows_ok(ws[0]->stype, (uint32_t)rows, (uint32_t)K, PRO_RMSNORM) &&
+      match_rmsnorm(X, &rm)) {
     bool vec = true;
     if (rm.gamma) TRY(gamma_row_vector(be, rm.gamma, &vec));
     TRY(realize(be, rm.x));
@@ -219,7 +220,9 @@ int try_gate_up_glu(cg_backend *be, cg_tensor *glu, cg_tensor *g, cg_tensor *u, 
       d.m.p[i].sbn = ws[i]->strides[ws[i]->rank - 1];
       d.m.p[i].N = (uint32_t)N;
     }
-    const char *base = ws[0]->stype == ST_BF16 ? "gemv_rowdot_bf16" : "gemv_rowdot_f32";
+    const char *base = rows > 1 && gemv_rows_mfma_ok(ws[0]->stype, (uint32_t)rows, (uint32_t)K, d.pro) ? "gemv_rows_bf16"
+                       : ws[0]->stype == ST_BF16                                                          ? "gemv_rowdot_bf16"
+                                                                                                          : "gemv_rowdot_f32";
     KernelScope ks(be, base, 2.0 * N * K * esize(ws[0]->stype) + (double)rows * (K * 8 + N * 4), 4.0 * rows * N * K);
     if (be->trace_shapes) {
       char buf[96];
@@ -247,7 +250,7 @@ int try_gemv_prologue(cg_backend *be, cg_tensor *n, cg_tensor *addend, bool *add
   if (A->op == N_REAL || A->dtype != CG_F32 || !n->gemv_candidate || A->rank < 1) return CG_OK;
   const int64_t K = A->shape[A->rank - 1];
   const int64_t rows = K > 0 ? A->size() / K : 0;  // one row, or the few rows of a small batch
-  if (rows < 1 || rows > 4 || A->size() != rows * K || K % 8 || K < 256 || rows * K > GEMV_PRO_MAX_K) return CG_OK;
+  if (rows < 1 || rows > GEMV_PRO_MAX_ROWS || A->size() != rows * K || K % 8 || K < 256) return CG_OK;
   RmsNormMatch rm;
   cg_tensor *gate = nullptr, *up = nullptr;
   int gelu = 0, pro = 0;
@@ -278,7 +281,7 @@ int try_gemv_prologue(cg_backend *be, cg_tensor *n, cg_tensor *addend, bool *add
       if (w->shape[i] != 1 && w->strides[i] != 0) return CG_OK;
     if (w->stype != ST_F32 && w->stype != ST_BF16) return CG_OK;
     if (b_stype >= 0 && w->stype != b_stype) return CG_OK;
-    if (rows > 1 && K > (int64_t)gemv_pro_multi_row_max_k(w->stype)) return CG_OK;
+    if (!gemv_pro_rows_ok(w->stype, (uint32_t)rows, (uint32_t)K, pro)) return CG_OK;
     b_stype = w->stype;
     if ((uintptr_t)data_ptr(w) % 16 || w->strides[w->rank - 1] % (16 / esize(w->stype))) return CG_OK;
   }
@@ -350,7 +353,9 @@ int try_gemv_prologue(cg_backend *be, cg_tensor *n, cg_tensor *addend, bool *add
     flops += 2.0 * rows * pr.N * K;
   }
   if (!st) {
-    const char *base = b_stype == ST_BF16 ? "gemv_rowdot_bf16" : "gemv_rowdot_f32";
+    const char *base = rows > 1 && gemv_rows_mfma_ok(b_stype, (uint32_t)rows, (uint32_t)K, pro) ? "gemv_rows_bf16"
+                       : b_stype == ST_BF16                                                      ? "gemv_rowdot_bf16"
+                                                                                                 : "gemv_rowdot_f32";
     KernelScope ks(be, base, bytes, flops);
     if (be->trace_shapes) {
       char buf[96];

@@ -583,14 +583,84 @@ def test_biased_projections_of_a_decode_step(oracle, hip, hip_bf16, hip_nopat, r
         assert np.max(np.abs(a - r)) <= 2e-2 * np.abs(r).max()
 
 
-@pytest.mark.parametrize("rows", [2, 3, 4])
+@pytest.mark.parametrize("rows,K,N", [(2, 128, 64), (5, 256, 200), (8, 1152, 1000), (16, 1024, 72), (3, 5632, 2100),
+                                      (4, 2048, 2050), (16, 1408, 64), (7, 384, 83), (13, 640, 4099)])
+def test_few_rows_on_the_matrix_cores(hip_bf16, rows, K, N):
+    """2 to 16 rows against a bf16 weight matrix: the weights go from memory into the MFMA operand and the
+    rows are rounded to bf16 on their way into LDS, so the result is the product of the rounded operands,
+    accumulated in f32 - checked against exactly that in float64, with and without a residual."""
+    g = np.random.default_rng(rows * 100 + K)
+    x = g.standard_normal((rows, 1, K)).astype(np.float32)
+    res = g.standard_normal((rows, 1, N)).astype(np.float32)
+    p = {"w.weight": (g.standard_normal((N, K)) * 0.05).astype(np.float32)}
+    want = vectors.bf16_round(x.reshape(rows, K)).astype(np.float64) @ vectors.bf16_round(p["w.weight"]).astype(np.float64).T
+    scale = np.abs(want).max()
+
+    def plain(b, xv):
+        return _folded_linear(b, K, N, "w", xv + xv - xv)
+
+    def with_residual(b, xv, rv):
+        rv = rv + rv - rv   # (arrays of two or more axes are loaded as bf16 in this mode: an f32 value with two readers)
+        return rv + _folded_linear(b, K, N, "w", xv + xv - xv), rv
+    (got,), names = run_traced(hip_bf16, plain, 1, x, params=p)
+    assert "gemv_rows_bf16" in names, sorted(names)
+    assert got.shape == (rows, 1, N) and np.max(np.abs(got.reshape(rows, N) - want)) <= 1e-5 * scale
+    (got, r16), names = run_traced(hip_bf16, with_residual, 2, x, res, params=p)
+    assert "gemv_rows_bf16" in names and (rows > 8 or "binary_f32" not in names), sorted(names)
+    assert np.array_equal(r16, vectors.bf16_round(res))
+    assert np.max(np.abs(got.reshape(rows, N) - (want + r16.reshape(rows, N)))) <= 1e-5 * (scale + np.abs(res).max())
+
+
+@pytest.mark.parametrize("rows,K,N", [(3, 1152, 520), (16, 1408, 96), (4, 5632, 130)])
 @pytest.mark.parametrize("act", ["silu", "gelu"])
-def test_decoder_block_of_a_small_batch(oracle, hip, hip_bf16, hip_nopat, rows, act):
+def test_glu_of_a_few_rows_in_the_prologue_of_the_matrix_core_kernel(oracle, hip_bf16, rows, K, N, act):
+    """down_proj over the rows of a small batch when gate and up arrive as tensors: the activation and the
+    product are computed on the way into LDS."""
+    g = np.random.default_rng(rows + K + len(act))
+    gate, up = (g.standard_normal((rows, 1, K)).astype(np.float32) for _ in range(2))
+    res = g.standard_normal((rows, 1, N)).astype(np.float32)
+    p = {"d.weight": (g.standard_normal((N, K)) * 0.05).astype(np.float32)}
+
+    def f(b, gv, uv, rv):
+        gv, uv = gv + gv - gv, uv + uv - uv
+        h = (nn.silu(b, gv) if act == "silu" else nn.gelu(b, gv)) * uv
+        return _folded_linear(b, K, N, "d", h) + rv
+    p16 = {k: vectors.bf16_round(v) for k, v in p.items()}
+    (ref,) = vectors.run(oracle, f, 1, gate, up, res, params=p16)
+    (got,), names = run_traced(hip_bf16, f, 1, gate, up, res, params=p)
+    assert "gemv_rows_bf16" in names and not ({"swiglu_fused", "geglu_fused"} & names), sorted(names)
+    assert np.max(np.abs(got - ref)) <= 1e-2 * np.abs(ref).max()
+
+
+@pytest.mark.parametrize("rows,K", [(17, 256), (16, 2048), (4, 320), (4, 5632)])
+def test_rows_the_matrix_core_kernel_does_not_take(oracle, hip_bf16, rows, K):
+    """More than 16 rows, rows that do not fit its LDS, K that its four waves cannot split evenly, or a
+    deep matrix with too few columns to occupy the CUs: another kernel computes the product, to the
+    tolerance of bf16 mode."""
+    N = 96
+    g = np.random.default_rng(rows + K)
+    x = g.standard_normal((rows, 1, K)).astype(np.float32)
+    p = {"w.weight": (g.standard_normal((N, K)) * 0.05).astype(np.float32)}
+
+    def f(b, xv):
+        return _folded_linear(b, K, N, "w", xv + xv - xv)
+    p16 = {k: vectors.bf16_round(v) for k, v in p.items()}
+    (ref,) = vectors.run(oracle, f, 1, x, params=p16)
+    (got,), names = run_traced(hip_bf16, f, 1, x, params=p)
+    assert "gemv_rows_bf16" not in names, sorted(names)
+    assert np.max(np.abs(got - ref)) <= 2e-2 * np.abs(ref).max()
+
+
+@pytest.mark.parametrize("rows,dims", [(2, (512, 1024)), (3, (512, 1024)), (4, (512, 1024)), (4, (640, 1152)), (8, (512, 1024)),
+                                       (13, (640, 1152)), (16, (512, 1024)), (16, (640, 1152))])
+@pytest.mark.parametrize("act", ["silu", "gelu"])
+def test_decoder_block_of_a_small_batch(oracle, hip, hip_bf16, hip_nopat, rows, dims, act):
     """One decode step of `rows` sequences through the projections of a decoder layer, each linear
     folding the batch itself: RMSNorm inside the grouped q/k/v launch, the residual in o_proj's
     epilogue, gate_proj, up_proj and the activation as one launch - five launches where the rows taken
-    one product at a time need eleven - and the same values as the oracle."""
-    K, F = 512, 1024
+    one product at a time need eleven - and the same values as the oracle.  f32 weights take up to 4 rows
+    this way; bf16 weights up to 16, on the matrix cores."""
+    K, F = dims
     g = np.random.default_rng(rows * 10 + len(act))
     x = (g.standard_normal((rows, 1, K)) * 2).astype(np.float32)
     p = {"n1.weight": g.standard_normal(K).astype(np.float32), "n2.weight": g.standard_normal(K).astype(np.float32)}
@@ -609,21 +679,30 @@ def test_decoder_block_of_a_small_batch(oracle, hip, hip_bf16, hip_nopat, rows, 
     ref = vectors.run(oracle, f, 3, x, params=p)
     got, names = run_traced(hip, f, 3, x, params=p)
     gen = vectors.run(hip_nopat, f, 3, x, params=p)
-    assert not ({"rmsnorm_fused", "swiglu_fused", "geglu_fused", "binary_f32"} & names), sorted(names)
+    if rows <= 4:
+        assert not ({"rmsnorm_fused", "swiglu_fused", "geglu_fused", "binary_f32"} & names), sorted(names)
     hip.trace(True)
     hip.trace_reset()
     vectors.run(hip, f, 3, x, params=p)
     rep = hip.trace_report()
     hip.trace(False)
     # x + x - x, then q/k/v, o_proj, gate/up, down_proj
-    assert rep["gemv_rowdot_f32"]["launches"] == 4 and sum(v["launches"] for v in rep.values()) == 5, {k: v["launches"] for k, v in rep.items()}
+    if rows <= 4:
+        assert rep["gemv_rowdot_f32"]["launches"] == 4 and sum(v["launches"] for v in rep.values()) == 5, {k: v["launches"] for k, v in rep.items()}
     for r, a, c in zip(ref, got, gen):
         assert a.shape == r.shape and np.allclose(a, r, rtol=1e-4, atol=1e-4), np.abs(a - r).max()
         assert np.allclose(c, r, rtol=1e-4, atol=1e-4)
     p16 = {k: (vectors.bf16_round(v) if v.ndim >= 2 else v) for k, v in p.items()}
     ref16 = vectors.run(oracle, f, 3, x, params=p16)
     got16, names16 = run_traced(hip_bf16, f, 3, x, params=p)
-    assert not ({"rmsnorm_fused", "swiglu_fused", "geglu_fused", "binary_f32"} & names16), sorted(names16)
+    if rows <= 8:   # (a residual rides in the epilogue for up to 8 rows)
+        assert not ({"rmsnorm_fused", "swiglu_fused", "geglu_fused", "binary_f32"} & names16), sorted(names16)
+    hip_bf16.trace(True)
+    hip_bf16.trace_reset()
+    vectors.run(hip_bf16, f, 3, x, params=p)
+    rep = hip_bf16.trace_report()
+    hip_bf16.trace(False)
+    assert rep["gemv_rows_bf16"]["launches"] == 4, {k: v["launches"] for k, v in rep.items()}
     for r, a in zip(ref16, got16):
         assert np.max(np.abs(a - r)) <= 2e-2 * np.abs(r).max()
 
