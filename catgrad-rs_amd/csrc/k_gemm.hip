@@ -1384,31 +1384,38 @@ uint32_t gemv_pro_multi_row_max_k(int b_stype) { return 64u * (b_stype == ST_BF1
 // ---- a few input rows against shared bf16 weights, on the matrix cores ---------------------------------
 // A decode step of a small batch multiplies 2 to 16 rows by every weight matrix.  The kernel above does
 // that with one multiply-add per lane, weight and row, and at four rows its arithmetic, not the stream of
-// weights, sets the pace (17 us for 25 MB).  Here a weight vector goes from memory straight into the A
-// operand of v_mfma_f32_16x16x32_bf16 - lane (n = lane & 15, kb = lane >> 4) holds k = kb * 8 .. + 7 of
-// column n, 16 bytes of that column's row.  Loaded by that lane itself, neighbouring lanes would read
-// from 16 different rows and the address unit, not memory, would set the pace (3.5 us for 64 KB per
-// workgroup); so lane l loads piece l & 3 of column l >> 2 - four neighbours share 64 bytes - and
-// ds_bpermute hands every piece to the lane that multiplies it.  The input rows, narrowed to bf16 in
-// LDS by the prologue (RMSNorm, SwiGLU / GeGLU or none, as above), are the B operand: lane (m, kb)
-// reads row m, or zeros past the last row.  A workgroup owns groups of 16 output columns; its four waves
-// take a quarter of k each (K % 128 == 0) and meet in LDS, where thread (m, n) adds the four quarters,
-// applies the epilogue and stores.  D[n][m] sits in lane m + 16 * (n / 4), register n % 4.
+// weights, sets the pace (17 us for 25 MB).  Here v_mfma_f32_16x16x32_bf16 does the arithmetic: its A
+// operand is 16 weight columns - lane (n = lane & 15, kb = lane >> 4) holds k = kb * 8 .. + 7 of column n -
+// and its B operand the input rows, narrowed to bf16 in LDS by the prologue (RMSNorm, SwiGLU / GeGLU or
+// none, as above): lane (m, kb) reads row m, or zeros past the last row.  D[n][m] sits in lane
+// m + 16 * (n / 4), register n % 4.
+// Memory wants long runs: a load instruction whose lanes follow the operand layout touches 16 weight rows,
+// 64 bytes of each, and streams at 5 TB/s; one that reads 512 contiguous bytes of two rows reaches 6.5.  So
+// a lane loads piece lane & 31 (8 values) of row 2u + (lane >> 5) of a window of 256 k, 8 instructions a
+// window, and the wave turns the window around in 8 KB of LDS of its own (rows 528 bytes apart, free of
+// bank conflicts both ways) before it reads the operands.  Two windows are in flight per lane.
+// A workgroup owns groups of 16 output columns; its four waves take a quarter of k each (K % 128 == 0) and
+// meet in LDS, where thread (m, n) adds the four quarters, applies the epilogue and stores.  GLUEPI: a
+// group is 8 columns of gate_proj and the same 8 of up_proj, rows 0-7 and 8-15 of one operand, and thread
+// (m, n < 8) stores act(gate) * up.
 // The inputs are rounded to bf16 like those of every many-row product in bf16 mode.
-// XV: 16-byte pieces of the input rows per lane in the RMSNorm prologue, where a wave owns whole rows
-// (rows wave, wave + 4, ...) so that a row's sum of squares never leaves the wave.
-enum { GEMV_ROWS_MAX = 16, GEMV_ROWS_LDS = 24576 };
-template <bool GLUEPI, int XV>
+// RS, PP: the prologue keeps the rows of a wave - rows wave, wave + 4, ... (RS of them), so that a row's sum
+// of squares never leaves the wave - as PP 16-byte pieces per lane and row in registers; RMSNorm needs the
+// whole row at once (K <= 256 * PP), the elementwise prologues take K in several passes.
+enum { GEMV_ROWS_MAX = 16, GEMV_ROWS_LDS = 20480, GEMV_ROWS_TP = 264 };
+template <bool GLUEPI, int RS, int PP>
 __global__ void __launch_bounds__(256) gemv_rows_mfma_kernel(GemvProDesc g) {
   typedef WVec<uint16_t>::type VT;
-  constexpr int UN = GLUEPI ? 8 : 16, NM = GLUEPI ? 2 : 1;  // k-steps of 32 in flight per wave; weight matrices
+  constexpr int UN = 16;               // 16-byte loads in flight per lane: two windows of 8
+  constexpr int CG = GLUEPI ? 8 : 16;  // output columns per group
   __shared__ __attribute__((aligned(16))) uint16_t xs[GEMV_ROWS_LDS];  // [rows][K + 8] bf16
-  __shared__ float red[NM][4][16][17];
+  __shared__ __attribute__((aligned(16))) uint16_t turn[4][16 * GEMV_ROWS_TP];
+  __shared__ float red[4][16][17];
   warm_kernel_arguments<sizeof(GemvProDesc)>();
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 15, kb = lane >> 4;
   const uint32_t K = g.m.K, rows = g.rows, pitch = K + 8;
-  const uint32_t N = g.m.p[blockIdx.y].N, groups = (N + 15) / 16;
+  const uint32_t N = g.m.p[blockIdx.y].N, groups = (N + CG - 1) / CG;
   if (blockIdx.x >= groups) return;  // the narrower problems of a grouped launch
   const uint16_t *B = (const uint16_t *)g.m.p[blockIdx.y].b;
   const uint16_t *B2 = GLUEPI ? (const uint16_t *)g.m.p[1].b : nullptr;
@@ -1416,22 +1423,32 @@ __global__ void __launch_bounds__(256) gemv_rows_mfma_kernel(GemvProDesc g) {
   float *C = g.m.p[blockIdx.y].c;
   const float *Cadd = g.m.p[blockIdx.y].c_add;
   const uint32_t cadd_rs = g.m.p[blockIdx.y].c_add_is_row ? 0u : N;
-  const uint32_t spw = K / 128;              // k-steps of this wave
-  const uint32_t k_begin = wave * spw * 32;  // and where they start
-  // Every request is NM * UN loads, no fewer (steps past the wave's last repeat it and are not used), so
-  // the prologue's wait for its own, older loads is a count that leaves these in flight.
-  VT q[NM][UN];
-  auto request = [&](uint32_t group, uint32_t s0) {
-    const uint32_t n = min(group * 16 + (lane >> 2), N - 1);
-    const uint16_t *p0 = B + (int64_t)n * sbn + k_begin + (lane & 3) * 8;
-    const uint16_t *p1 = GLUEPI ? B2 + (int64_t)n * sbn2 + k_begin + (lane & 3) * 8 : nullptr;
+  const uint32_t kw = K / 4, k_begin = wave * kw;  // this wave's share of k
+  const uint32_t nbatch = (kw + 511) / 512;        // requests (two windows of 256) per group
+  const uint32_t lrow = lane >> 5, lk = (lane & 31) * 8;
+  // Every request is UN loads, no fewer (pieces past the end of the wave's share repeat its last and are not
+  // used), so the prologue's wait for its own, older loads is a count that leaves these in flight.
+  VT q[UN];
+  auto request = [&](uint32_t group, uint32_t batch) {
 #pragma unroll
-    for (int u = 0; u < UN; ++u) {
-      const uint32_t s = min(s0 + u, spw - 1);
-      q[0][u] = __builtin_nontemporal_load((const VT *)(p0 + s * 32));
-      if (GLUEPI) q[NM - 1][u] = __builtin_nontemporal_load((const VT *)(p1 + s * 32));
+    for (int u = 0; u < 8; ++u) {
+      const uint32_t v = 2 * u + lrow;  // row of the operand
+      const uint16_t *row;
+      if (GLUEPI) row = u < 4 ? B + (int64_t)min(group * 8 + v, N - 1) * sbn : B2 + (int64_t)min(group * 8 + v - 8, N - 1) * sbn2;
+      else row = B + (int64_t)min(group * 16 + v, N - 1) * sbn;
+#pragma unroll
+      for (int w2 = 0; w2 < 2; ++w2) {
+        const uint32_t kl = min((batch * 2 + w2) * 256 + lk, kw - 8);
+        q[w2 * 8 + u] = __builtin_nontemporal_load((const VT *)(row + k_begin + kl));
+      }
     }
   };
+  // Everything the prologue loads is used in straight-line code, down to the LDS store (pieces past the end of
+  // a row or of the rows go to a spare location): a load whose only use sits inside a branch - gamma under
+  // `if (aux)`, or the whole piece under `if (k < K)` - is moved there by the compiler, behind the request for
+  // the weights, where it waits for them to arrive.
+  auto early_load = [](const float *p) { return *(const float4 *)p; };
+  uint16_t *spare = turn[wave] + lane * 4;  // (the wave's window buffer is not in use yet)
   auto narrow = [](const float4 &o) {
     union { bf16x2_t h[2]; uint2 u; } pk;
     pk.h[0] = __builtin_convertvector((f32x2_t){o.x, o.y}, bf16x2_t);
@@ -1440,137 +1457,127 @@ __global__ void __launch_bounds__(256) gemv_rows_mfma_kernel(GemvProDesc g) {
   };
   // ---- the input rows, to LDS as bf16
   if (g.pro == PRO_RMSNORM) {
-    const uint32_t ppr = (K + 255) / 256;  // pieces of a row per lane; slot j = (row slot j / ppr, piece j % ppr)
-    float4 xv[XV], gv[XV];
-    {
-      uint32_t rs = 0, i = 0;
+    float4 xv[RS][PP], gv[PP];
 #pragma unroll
-      for (int j = 0; j < XV; ++j) {
-        const uint32_t row = min(wave + 4 * rs, rows - 1), k = min((lane + 64 * i) * 4, K - 4);
-        xv[j] = *(const float4 *)(g.a + (int64_t)row * g.a_rstride + k);
-        gv[j] = *(const float4 *)((g.aux ? g.aux : g.a) + k);  // gamma: one vector for every row
-        if (++i == ppr) { i = 0; ++rs; }
-      }
+    for (int i = 0; i < PP; ++i) {
+      const uint32_t k = min((lane + 64 * i) * 4u, K - 4);
+      gv[i] = early_load((g.aux ? g.aux : g.a) + k);  // gamma: one vector for every row
+#pragma unroll
+      for (int rs = 0; rs < RS; ++rs) xv[rs][i] = early_load(g.a + (int64_t)min(wave + 4u * rs, rows - 1) * g.a_rstride + k);
     }
     request(blockIdx.x, 0);
-    float ssq[4] = {0.f, 0.f, 0.f, 0.f};
-    {
-      uint32_t rs = 0, i = 0;
+    const float has_gamma = g.aux ? 1.f : 0.f, no_gamma = 1.f - has_gamma;
 #pragma unroll
-      for (int j = 0; j < XV; ++j) {
-        const bool valid = wave + 4 * rs < rows && (lane + 64 * i) * 4 < K;
-        const float s = valid ? xv[j].x * xv[j].x + xv[j].y * xv[j].y + xv[j].z * xv[j].z + xv[j].w * xv[j].w : 0.f;
+    for (int rs = 0; rs < RS; ++rs) {
+      float ssq = 0.f;
 #pragma unroll
-        for (int t = 0; t < 4; ++t) ssq[t] += rs == (uint32_t)t ? s : 0.f;
-        if (++i == ppr) { i = 0; ++rs; }
-      }
-    }
-    float rms[4];
+      for (int i = 0; i < PP; ++i)
+        if ((lane + 64 * i) * 4u < K) ssq += xv[rs][i].x * xv[rs][i].x + xv[rs][i].y * xv[rs][i].y + xv[rs][i].z * xv[rs][i].z + xv[rs][i].w * xv[rs][i].w;
+      const float inv = 1.0f / sqrtf(wave_sum(ssq) / g.n_as_float + g.eps);
+      const uint32_t row = wave + 4u * rs;
 #pragma unroll
-    for (int t = 0; t < 4; ++t) rms[t] = sqrtf(wave_sum(ssq[t]) / g.n_as_float + g.eps);
-    {
-      uint32_t rs = 0, i = 0;
-#pragma unroll
-      for (int j = 0; j < XV; ++j) {
-        const uint32_t row = wave + 4 * rs, k = (lane + 64 * i) * 4;
-        if (row < rows && k < K) {
-          float d = rms[0];
-#pragma unroll
-          for (int t = 1; t < 4; ++t) d = rs == (uint32_t)t ? rms[t] : d;
-          float4 o;
-          o.x = xv[j].x / d; o.y = xv[j].y / d; o.z = xv[j].z / d; o.w = xv[j].w / d;
-          if (g.aux) {
-            o.x *= g.gamma_offset + gv[j].x; o.y *= g.gamma_offset + gv[j].y;
-            o.z *= g.gamma_offset + gv[j].z; o.w *= g.gamma_offset + gv[j].w;
-          }
-          *(uint2 *)(xs + (size_t)row * pitch + k) = narrow(o);
-        }
-        if (++i == ppr) { i = 0; ++rs; }
+      for (int i = 0; i < PP; ++i) {
+        const uint32_t k = (lane + 64 * i) * 4u;
+        float4 o;  // x / rms * (offset + gamma), or x / rms without a gamma (has_gamma = 0: the factor is 1)
+        o.x = xv[rs][i].x * inv * (has_gamma * (g.gamma_offset + gv[i].x) + no_gamma);
+        o.y = xv[rs][i].y * inv * (has_gamma * (g.gamma_offset + gv[i].y) + no_gamma);
+        o.z = xv[rs][i].z * inv * (has_gamma * (g.gamma_offset + gv[i].z) + no_gamma);
+        o.w = xv[rs][i].w * inv * (has_gamma * (g.gamma_offset + gv[i].w) + no_gamma);
+        *(uint2 *)(row < rows && k < K ? xs + (size_t)row * pitch + k : spare) = narrow(o);
       }
     }
   } else {
-    // elementwise prologues: the pieces of all rows, 8 per thread and pass
-    const uint32_t kp = K / 4, pieces = rows * kp;
+    // elementwise prologues: PP pieces per lane and row at a time
     const bool glu = g.pro != PRO_NONE;
-    float4 xv[8], gv[8];
-    auto load_pass = [&](uint32_t p0) {
+    const float is_glu = glu ? 1.f : 0.f, not_glu = 1.f - is_glu;
+    const uint32_t ppr = (K + 255) / 256;
+    float4 xv[RS][PP], gv[RS][PP];
+    auto load_pass = [&](uint32_t i0) {
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const uint32_t p = min(p0 + tid + j * 256u, pieces - 1), m = p / kp, k = (p - m * kp) * 4;
-        xv[j] = *(const float4 *)(g.a + (int64_t)m * g.a_rstride + k);
-        gv[j] = *(const float4 *)(glu ? g.aux + (int64_t)m * g.aux_rstride + k : g.a + (int64_t)m * g.a_rstride + k);
+      for (int rs = 0; rs < RS; ++rs) {
+        const uint32_t row = min(wave + 4u * rs, rows - 1);
+        const float *xa = g.a + (int64_t)row * g.a_rstride;
+        const float *xb = glu ? g.aux + (int64_t)row * g.aux_rstride : xa;  // no second operand: the row's own pieces again
+#pragma unroll
+        for (int i = 0; i < PP; ++i) {
+          const uint32_t k = min((lane + 64 * (i0 + i)) * 4u, K - 4);
+          xv[rs][i] = early_load(xa + k);
+          gv[rs][i] = early_load(xb + k);
+        }
       }
     };
-    auto store_pass = [&](uint32_t p0) {
+    auto store_pass = [&](uint32_t i0) {
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const uint32_t p = p0 + tid + j * 256u;
-        if (p < pieces) {
-          const uint32_t m = p / kp, k = (p - m * kp) * 4;
-          float4 o = xv[j];
+      for (int rs = 0; rs < RS; ++rs) {
+        const uint32_t row = wave + 4u * rs;
+#pragma unroll
+        for (int i = 0; i < PP; ++i) {
+          const uint32_t k = (lane + 64 * (i0 + i)) * 4u;
+          float4 o = xv[rs][i];
           if (g.pro == PRO_GEGLU) {
-            o.x = gelu_ref(o.x) * gv[j].x; o.y = gelu_ref(o.y) * gv[j].y;
-            o.z = gelu_ref(o.z) * gv[j].z; o.w = gelu_ref(o.w) * gv[j].w;
+            o.x = gelu_ref(o.x); o.y = gelu_ref(o.y); o.z = gelu_ref(o.z); o.w = gelu_ref(o.w);
           } else if (g.pro == PRO_SWIGLU) {
-            o.x = o.x * sigmoid_ref(o.x) * gv[j].x; o.y = o.y * sigmoid_ref(o.y) * gv[j].y;
-            o.z = o.z * sigmoid_ref(o.z) * gv[j].z; o.w = o.w * sigmoid_ref(o.w) * gv[j].w;
+            o.x *= sigmoid_ref(o.x); o.y *= sigmoid_ref(o.y); o.z *= sigmoid_ref(o.z); o.w *= sigmoid_ref(o.w);
           }
-          *(uint2 *)(xs + (size_t)m * pitch + k) = narrow(o);
+          // times the second operand, or times 1 without one (is_glu = 0)
+          o.x *= is_glu * gv[rs][i].x + not_glu; o.y *= is_glu * gv[rs][i].y + not_glu;
+          o.z *= is_glu * gv[rs][i].z + not_glu; o.w *= is_glu * gv[rs][i].w + not_glu;
+          *(uint2 *)(row < rows && k < K ? xs + (size_t)row * pitch + k : spare) = narrow(o);
         }
       }
     };
     load_pass(0);
     request(blockIdx.x, 0);
     store_pass(0);
-    for (uint32_t p0 = 2048; p0 < pieces; p0 += 2048) {
-      load_pass(p0);
-      store_pass(p0);
+    for (uint32_t i0 = PP; i0 < ppr; i0 += PP) {
+      load_pass(i0);
+      store_pass(i0);
     }
   }
   __syncthreads();
   // ---- the products
   const bool live = (uint32_t)r < rows;
   const uint16_t *xrow = xs + (size_t)min((uint32_t)r, rows - 1) * pitch + k_begin + kb * 8;
-  const int from = (4 * r + kb) * 4;  // ds_bpermute: the lane that loaded piece kb of column r
+  uint16_t *mine = turn[wave];
   for (uint32_t group = blockIdx.x; group < groups; group += gridDim.x) {
-    f32x4n acc[NM];
+    f32x4n acc = {0.f, 0.f, 0.f, 0.f};
+    for (uint32_t batch = 0; batch < nbatch; ++batch) {
+      VT cur[UN];
 #pragma unroll
-    for (int e = 0; e < NM; ++e) acc[e] = (f32x4n){0.f, 0.f, 0.f, 0.f};
-    for (uint32_t s0 = 0; s0 < spw; s0 += UN) {
-      VT cur[NM][UN];
-#pragma unroll
-      for (int e = 0; e < NM; ++e)
-#pragma unroll
-        for (int u = 0; u < UN; ++u) cur[e][u] = q[e][u];
+      for (int u = 0; u < UN; ++u) cur[u] = q[u];
       // the next vectors - of this group, or the first of the workgroup's next group - while these multiply
-      if (s0 + UN < spw) request(group, s0 + UN);
+      if (batch + 1 < nbatch) request(group, batch + 1);
       else if (group + gridDim.x < groups) request(group + gridDim.x, 0);
 #pragma unroll
-      for (int u = 0; u < UN; ++u)
-        if (s0 + u < spw) {
-          union { uint4 u4; bf16x8 h; } xb;
-          xb.u4 = *(const uint4 *)(xrow + (s0 + u) * 32);
-          if (!live) xb.u4 = make_uint4(0u, 0u, 0u, 0u);
+      for (int w2 = 0; w2 < 2; ++w2) {
+        const uint32_t wk = (batch * 2 + w2) * 256;  // where the window starts in the wave's share of k
+        if (wk < kw) {
+          // (LDS serves a wave's accesses in order: these stores follow the previous window's reads)
+          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
 #pragma unroll
-          for (int e = 0; e < NM; ++e) {
-            union { VT v; bf16x8 h; } w;
+          for (int u = 0; u < 8; ++u) *(VT *)(mine + (2 * u + lrow) * GEMV_ROWS_TP + lk) = cur[w2 * 8 + u];
+          __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
 #pragma unroll
-            for (int c = 0; c < 4; ++c) w.v[c] = __builtin_amdgcn_ds_bpermute(from, cur[e][u][c]);
-            acc[e] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w.h, xb.h, acc[e], 0, 0, 0);
-          }
+          for (int s = 0; s < 8; ++s)
+            if (wk + s * 32 < kw) {
+              union { uint4 u4; bf16x8 h; } xb, w;
+              w.u4 = *(const uint4 *)(mine + r * GEMV_ROWS_TP + s * 32 + kb * 8);
+              xb.u4 = *(const uint4 *)(xrow + wk + s * 32);
+              if (!live) xb.u4 = make_uint4(0u, 0u, 0u, 0u);
+              acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w.h, xb.h, acc, 0, 0, 0);
+            }
         }
+      }
     }
     __syncthreads();  // the previous group's sums have been read
 #pragma unroll
-    for (int e = 0; e < NM; ++e)
-#pragma unroll
-      for (int v = 0; v < 4; ++v) red[e][wave][kb * 4 + v][r] = acc[e][v];
+    for (int v = 0; v < 4; ++v) red[wave][kb * 4 + v][r] = acc[v];
     __syncthreads();
-    const uint32_t m = tid >> 4, n = tid & 15, col = group * 16 + n;
-    if (m < rows && col < N) {
-      float v0 = (red[0][0][n][m] + red[0][1][n][m]) + (red[0][2][n][m] + red[0][3][n][m]);
+    const uint32_t m = tid >> 4, n = tid & 15, col = group * CG + n;
+    if (m < rows && n < (uint32_t)CG && col < N) {
+      float v0 = (red[0][n][m] + red[1][n][m]) + (red[2][n][m] + red[3][n][m]);
       if (GLUEPI) {
-        const float v1 = (red[NM - 1][0][n][m] + red[NM - 1][1][n][m]) + (red[NM - 1][2][n][m] + red[NM - 1][3][n][m]);
+        const float v1 = (red[0][n + 8][m] + red[1][n + 8][m]) + (red[2][n + 8][m] + red[3][n + 8][m]);
         v0 = (g.glu_epilogue == PRO_GEGLU ? gelu_ref(v0) : v0 * sigmoid_ref(v0)) * v1;
       } else if (Cadd) {
         v0 += Cadd[(uint64_t)m * cadd_rs + col];
@@ -1584,7 +1591,8 @@ __global__ void __launch_bounds__(256) gemv_rows_mfma_kernel(GemvProDesc g) {
 bool gemv_rows_mfma_ok(int b_stype, uint32_t rows, uint32_t K, int pro) {
   if (b_stype != ST_BF16 || rows < 2 || rows > GEMV_ROWS_MAX || K < 128 || K % 128) return false;
   if ((uint64_t)rows * (K + 8) > GEMV_ROWS_LDS) return false;
-  if (pro == PRO_RMSNORM && ((rows + 3) / 4) * ((K + 255) / 256) > 16) return false;
+  // RMSNorm keeps a wave's rows whole in registers: 16 pieces of 16 bytes per lane
+  if (pro == PRO_RMSNORM && (rows <= 4 ? 1u : rows <= 8 ? 2u : 4u) * ((K + 255) / 256) > 16) return false;
   return pro == PRO_NONE || pro == PRO_RMSNORM || pro == PRO_SWIGLU || pro == PRO_GEGLU;
 }
 
@@ -1594,20 +1602,22 @@ bool gemv_pro_rows_ok(int b_stype, uint32_t rows, uint32_t K, int pro) {
   return rows <= 4 && (uint64_t)rows * K <= GEMV_PRO_MAX_K && K <= gemv_pro_multi_row_max_k(b_stype);
 }
 
+template <bool GLUEPI>
+static void launch_gemv_rows_mfma_as(const LaunchCtx &lc, const GemvProDesc &g, dim3 grid) {
+  if (g.rows > 8) CG_LAUNCH(lc, (gemv_rows_mfma_kernel<GLUEPI, 4, 4>), grid, 256, g);
+  else if (g.rows > 4) CG_LAUNCH(lc, (gemv_rows_mfma_kernel<GLUEPI, 2, 8>), grid, 256, g);
+  else if (g.m.K > 2048) CG_LAUNCH(lc, (gemv_rows_mfma_kernel<GLUEPI, 1, 16>), grid, 256, g);
+  else CG_LAUNCH(lc, (gemv_rows_mfma_kernel<GLUEPI, 1, 8>), grid, 256, g);
+}
+
 static hipError_t launch_gemv_rows_mfma(const LaunchCtx &lc, const GemvProDesc &g, uint32_t max_n) {
-  const uint32_t groups = (max_n + 15) / 16;
-  // two workgroups (56 KB of LDS each) per CU; a workgroup stages the rows once and walks its groups
+  const uint32_t groups = g.glu_epilogue ? (max_n + 7) / 8 : (max_n + 15) / 16;
+  // two workgroups (77 KB of LDS each) per CU; a workgroup stages the rows once and walks its groups
   uint32_t cap = (uint32_t)lc.n_cus * 2 / (g.glu_epilogue ? 1 : g.m.n_prob);
   if (!cap) cap = 1;
   const uint32_t blocks = groups < cap ? groups : cap;
-  const uint32_t xv = ((g.rows + 3) / 4) * ((g.m.K + 255) / 256);
-  if (g.glu_epilogue) {
-    if (g.pro == PRO_RMSNORM && xv > 8) CG_LAUNCH(lc, (gemv_rows_mfma_kernel<true, 16>), dim3(blocks, 1, 1), 256, g);
-    else CG_LAUNCH(lc, (gemv_rows_mfma_kernel<true, 8>), dim3(blocks, 1, 1), 256, g);
-  } else {
-    if (g.pro == PRO_RMSNORM && xv > 8) CG_LAUNCH(lc, (gemv_rows_mfma_kernel<false, 16>), dim3(blocks, g.m.n_prob, 1), 256, g);
-    else CG_LAUNCH(lc, (gemv_rows_mfma_kernel<false, 8>), dim3(blocks, g.m.n_prob, 1), 256, g);
-  }
+  if (g.glu_epilogue) launch_gemv_rows_mfma_as<true>(lc, g, dim3(blocks, 1, 1));
+  else launch_gemv_rows_mfma_as<false>(lc, g, dim3(blocks, g.m.n_prob, 1));
   return hipGetLastError();
 }
 
