@@ -2238,6 +2238,14 @@ bool gemm_epilogue_ok(const GemmDesc &g) {
 }
 
 // A plain product of 2 to 16 rows with bf16 weights [N][K] that gemv_rows_mfma_kernel takes.
+// (any number of columns: the caller may group several narrow products into one launch)
+bool gemv_rows_group_ok(const GemmDesc &g) {
+  if (g.M < 2 || g.M > GEMV_ROWS_MAX || g.nb0 * g.nb1 != 1 || g.b_index || g.splits > 1 || g.K >= 4096) return false;
+  if (g.a_stype != ST_F32 || g.b_stype != ST_BF16 || !g.bf16_math || g.sak != 1 || g.sbk != 1 || g.N < 1) return false;
+  if (g.glu_gate || g.c16 || g.n_group || g.dual_b || (g.c_add && g.M > 8)) return false;
+  if ((uintptr_t)g.a % 16 || g.sam % 4 || (uintptr_t)g.b % 16 || (g.N > 1 && g.sbn % 8)) return false;
+  return gemv_rows_mfma_ok(ST_BF16, g.M, g.K, PRO_NONE);
+}
 bool gemv_rows_plain_ok(const LaunchCtx &lc, const GemmDesc &g) {
   // deep and narrow (down_proj of a wide MLP, 4 x 5632 x 2048): fewer 16-column groups than half the CUs, each
   // a chain of several trips to memory - the vector kernel splits k further and is faster there (12.6 against 16.7 us)

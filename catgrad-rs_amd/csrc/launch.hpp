@@ -351,9 +351,11 @@ uint32_t gemv_pro_multi_row_max_k(int b_stype);
 enum { GEMV_PRO_MAX_ROWS = 16 };
 // whether launch_gemv_pro takes `rows` input rows of K values with prologue `pro` against weights of this
 // storage type: one row; up to 4 on the vector ALUs; up to 16 against bf16 weights on the matrix cores
-// (K % 128 == 0, rows * (K + 8) <= 24576, inputs rounded to bf16)
+// (K % 128 == 0, rows * (K + 8) <= 20480, inputs rounded to bf16)
 bool gemv_pro_rows_ok(int b_stype, uint32_t rows, uint32_t K, int pro);
 bool gemv_rows_mfma_ok(int b_stype, uint32_t rows, uint32_t K, int pro);
+// a plain product of 2 to 16 rows that launch_gemv_pro's matrix-core form takes as one of up to four problems
+bool gemv_rows_group_ok(const GemmDesc &g);
 // The routed experts of a MoE layer over many tokens (a prefill; models/qwen3.rs:104-123), expert by
 // expert.  A slot is one of the k choices of every token: its index vector, its input rows and its
 // outputs.  A problem is one stacked weight tensor [E, N, K] (bf16): gate_proj and up_proj share

@@ -700,6 +700,73 @@ int realize_matmul(cg_backend *be, cg_tensor *n, cg_tensor *addend, bool *added,
         return CG_OK;
       }
     }
+    // The same for the few rows of a small batch against bf16 weights (the router and the shared expert's gate
+    // of a MoE block, both narrow: 60 and 1 columns): the matrix-core kernel takes up to four products, and a
+    // lone product of fewer than 64 columns too (the vector kernel needs 8 us for 4 x 60 x 2048).
+    if (M >= 2 && N < 64 && batch == 1 && n->gemv_candidate && gemv_rows_group_ok(g)) {
+      std::vector<cg_tensor *> members;
+      for (cg_tensor *c : std::vector<cg_tensor *>(be->gemv_candidates)) {
+        if (c == n || members.size() >= 3 || c->op != N_MATMUL || c->in[0] != n->in[0] || c->dtype != CG_F32) continue;
+        cg_tensor *w = c->in[1];
+        const int64_t nc = w->shape[w->rank - 1];
+        if (w->rank != n->rank || w->shape[w->rank - 2] != (int64_t)K || nc < 1 || nc >= 64 ||  // (wide ones have fusions of their own)
+            c->size() != (int64_t)M * nc)
+          continue;
+        TRY(realize(be, w));  // a view of the parameter
+        if (w->stype != ST_BF16 || w->strides[w->rank - 2] != 1) continue;
+        bool shared = true;  // one matrix for every row: batch axes of extent 1 or stride 0
+        for (int i = 0; i + 2 < w->rank; ++i) shared = shared && (w->shape[i] == 1 || w->strides[i] == 0);
+        // (the stride between columns of a single column is never used)
+        if (!shared || (uintptr_t)data_ptr(w) % 16 || (nc > 1 && w->strides[w->rank - 1] % 8)) continue;
+        members.push_back(c);
+      }
+      {
+        GemvProDesc d;
+        std::memset(&d, 0, sizeof(d));
+        d.pro = PRO_NONE;
+        d.a = (const float *)g.a;
+        d.rows = M;
+        d.a_rstride = g.sam;
+        d.m.K = K;
+        d.m.b_stype = ST_BF16;
+        d.m.n_prob = 1;
+        d.m.p[0].b = g.b;
+        d.m.p[0].c = g.c;
+        d.m.p[0].c_add = g.c_add;
+        d.m.p[0].sbn = N > 1 ? g.sbn : (int64_t)K;  // (the stride between columns of a single column is never used)
+        d.m.p[0].N = N;
+        double bytes = uniq(A, sao) + uniq(B, sbo) + (double)n->size() * 4, flops = 2.0 * M * N * K;
+        for (cg_tensor *c : members) {
+          cg_tensor *w = c->in[1];
+          TRY(alloc_result(be, c, ST_F32));
+          auto &pr = d.m.p[d.m.n_prob++];
+          pr.b = data_ptr(w);
+          pr.c = (float *)c->st->ptr;
+          pr.N = (uint32_t)w->shape[w->rank - 1];
+          pr.sbn = pr.N > 1 ? w->strides[w->rank - 1] : (int64_t)K;
+          bytes += (double)pr.N * K * 2 + (double)M * pr.N * 4;
+          flops += 2.0 * M * pr.N * K;
+        }
+        {
+          KernelScope ks(be, "gemv_rows_bf16", bytes, flops);
+          if (be->trace_shapes) {
+            char buf[96];
+            snprintf(buf, sizeof buf, "gemv_rows_bf16[multi%d,M%u,K%u,N%.0f]", d.m.n_prob, M, K, flops / (2.0 * M * K));
+            ks.rename(buf);
+          }
+          HIPCHK(be, launch_gemv_pro(be->lc(), d));
+        }
+        for (cg_tensor *c : members) {
+          forget_gemv_candidate(c);
+          c->op = N_REAL;
+          drop_inputs(c);
+        }
+        forget_gemv_candidate(n);
+        n->op = N_REAL;
+        drop_inputs(n);
+        return CG_OK;
+      }
+    }
     // q/k/v of a prefill: the other deferred many-row products on the same left operand join this
     // launch as further column ranges (their own weights, their own outputs)
     std::vector<cg_tensor *> group;

@@ -611,6 +611,32 @@ def test_few_rows_on_the_matrix_cores(hip_bf16, rows, K, N):
     assert np.max(np.abs(got.reshape(rows, N) - (want + r16.reshape(rows, N)))) <= 1e-5 * (scale + np.abs(res).max())
 
 
+@pytest.mark.parametrize("rows,K,widths", [(4, 2048, (60, 1)), (2, 256, (5, 13, 1, 16)), (16, 1024, (33,))])
+def test_narrow_products_of_a_few_rows_share_a_launch(hip_bf16, rows, K, widths):
+    """The router and the shared expert's gate of a MoE block (qwen_moe.py: 60 and 1 columns on the same
+    rows, each a plain linear over [1, rows, K]): one launch of the matrix-core kernel for up to four
+    such products, and no other product launch."""
+    g = np.random.default_rng(rows + K)
+    x = g.standard_normal((1, rows, K)).astype(np.float32)   # (the block sees the batch folded into the rows)
+    p = {f"w{i}.weight": (g.standard_normal((n, K)) * 0.05).astype(np.float32) for i, n in enumerate(widths)}
+
+    def f(b, xv):
+        xv = xv + xv - xv
+        return [nn.linear_no_bias(b, K, n, lang.path([f"w{i}"]), xv) for i, n in enumerate(widths)]
+    hip_bf16.trace(True)
+    hip_bf16.trace_reset()
+    got = vectors.run(hip_bf16, f, len(widths), x, params=p)
+    rep = hip_bf16.trace_report()
+    hip_bf16.trace(False)
+    launches = {k: v["launches"] for k, v in rep.items() if k.startswith("gem")}
+    assert launches == {"gemv_rows_bf16": 1}, launches
+    x16 = vectors.bf16_round(x.reshape(rows, K)).astype(np.float64)
+    for i, n in enumerate(widths):
+        want = x16 @ vectors.bf16_round(p[f"w{i}.weight"]).astype(np.float64).T
+        assert got[i].shape == (1, rows, n)
+        assert np.max(np.abs(got[i].reshape(rows, n) - want)) <= 1e-5 * max(np.abs(want).max(), 1.0)
+
+
 @pytest.mark.parametrize("rows,K,N", [(3, 1152, 520), (16, 1152, 96), (4, 4608, 130)])
 @pytest.mark.parametrize("act", ["silu", "gelu"])
 def test_glu_of_a_few_rows_in_the_prologue_of_the_matrix_core_kernel(oracle, hip_bf16, rows, K, N, act):
