@@ -712,6 +712,56 @@ __global__ void __launch_bounds__(256) glu_kernel(const float *gate, const float
   }
 }
 
+// ---- a sum of rows, each scaled by a value of its own ------------------------------------------------
+// One thread owns four consecutive columns of one row: it asks for its piece of every term and for every
+// term's scale at once, then adds them up in the order given.
+__global__ void __launch_bounds__(256) row_scaled_sum_kernel(RowSumDesc g) {
+  const uint32_t per_row = g.d / 4, total = g.rows * per_row;
+  for (uint32_t p = blockIdx.x * 256 + threadIdx.x; p < total; p += gridDim.x * 256) {
+    const uint32_t row = p / per_row, c = (p - row * per_row) * 4;
+    float4 xv[ROW_SUM_MAX_TERMS];
+    float sv[ROW_SUM_MAX_TERMS];
+#pragma unroll
+    for (int j = 0; j < ROW_SUM_MAX_TERMS; ++j)
+      if ((uint32_t)j < g.n_terms) {
+        xv[j] = *(const float4 *)(g.t[j].x + (int64_t)row * g.t[j].x_rs + c);
+        sv[j] = g.t[j].s ? g.t[j].s[(int64_t)row * g.t[j].s_rs] : 1.0f;
+      }
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+    for (int j = 0; j < ROW_SUM_MAX_TERMS; ++j)
+      if ((uint32_t)j < g.n_terms) {
+        float4 t = xv[j];
+        if (g.t[j].s) {
+          const float w = g.t[j].sigmoid ? sigmoid_ref(sv[j]) : sv[j];
+          t.x = __fmul_rn(t.x, w); t.y = __fmul_rn(t.y, w); t.z = __fmul_rn(t.z, w); t.w = __fmul_rn(t.w, w);
+        }
+        if (j == 0) {
+          acc = t;
+        } else {
+          acc.x = __fadd_rn(acc.x, t.x); acc.y = __fadd_rn(acc.y, t.y);
+          acc.z = __fadd_rn(acc.z, t.z); acc.w = __fadd_rn(acc.w, t.w);
+        }
+      }
+    *(float4 *)(g.out + (int64_t)row * g.out_rs + c) = acc;
+  }
+}
+
+hipError_t launch_row_scaled_sum(const LaunchCtx &lc, const RowSumDesc &g) {
+  if (!g.rows || !g.d) return hipSuccess;
+  if (g.n_terms < 1 || g.n_terms > ROW_SUM_MAX_TERMS || g.d % 4 || (uintptr_t)g.out % 16 || g.out_rs % 4 ||
+      (uint64_t)g.rows * (g.d / 4) >= (1ull << 32))
+    return hipErrorInvalidValue;
+  for (uint32_t j = 0; j < g.n_terms; ++j)
+    if (!g.t[j].x || (uintptr_t)g.t[j].x % 16 || g.t[j].x_rs % 4) return hipErrorInvalidValue;
+  const uint64_t total = (uint64_t)g.rows * (g.d / 4);
+  uint64_t blocks = (total + 255) / 256;
+  const uint64_t cap = (uint64_t)lc.n_cus * 8;
+  if (blocks > cap) blocks = cap;
+  CG_LAUNCH(lc, row_scaled_sum_kernel, (unsigned)blocks, 256, g);
+  return hipGetLastError();
+}
+
 hipError_t launch_glu(const LaunchCtx &lc, int gelu, const float *gate, const float *up, float *out,
                       uint64_t n, uint16_t *out16) {
   if (!n) return hipSuccess;

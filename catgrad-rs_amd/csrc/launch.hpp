@@ -143,6 +143,23 @@ hipError_t launch_rope(const LaunchCtx &lc, const RopeDesc &d);
 // two rotations (the queries and the keys of an attention) as one launch
 hipError_t launch_rope_pair(const LaunchCtx &lc, const RopeDesc &d0, const RopeDesc &d1);
 // out = silu(gate) * up (gelu = 0) or gelu(gate) * up (gelu = 1); contiguous, n % 4 == 0
+// out[r, :] = sum_j w_j[r] * x_j[r, :] in the order of the terms, w_j = 1 (s null), s_j[r] or sigmoid(s_j[r]):
+// how a MoE block ends (models/qwen3.rs:104-123, deepseek.rs:163-165: the routed experts' rows weighted by
+// their router values, the shared expert's row through its gate, the residual) as one launch.  Every product
+// and every sum is rounded on its own (no fused multiply-add), like the one-op-at-a-time evaluation.
+// rows of d floats, d % 4 == 0; x_j and out 16-byte aligned with row strides that are multiples of 4
+enum { ROW_SUM_MAX_TERMS = 8 };
+struct RowSumDesc {
+  float *out;
+  int64_t out_rs;
+  uint32_t rows, d, n_terms;
+  struct {
+    const float *x, *s;
+    int64_t x_rs, s_rs;
+    int32_t sigmoid;
+  } t[ROW_SUM_MAX_TERMS];
+};
+hipError_t launch_row_scaled_sum(const LaunchCtx &lc, const RowSumDesc &g);
 hipError_t launch_glu(const LaunchCtx &lc, int gelu, const float *gate, const float *up, float *out,
                       uint64_t n, uint16_t *out16 = nullptr);  // out16: optional bf16 copy of out
 // op: 0 add, 1 sub, 2 mul, 3 div; b is contiguous (b_period = 0) or a vector of b_period floats

@@ -113,6 +113,7 @@ bool match_rmsnorm(cg_tensor *root, RmsNormMatch *m);
 int gamma_row_vector(cg_backend *be, cg_tensor *gb, bool *ok);
 int try_rmsnorm_pair(cg_backend *be, cg_tensor *root, const RmsNormMatch &outer, bool *done);
 int try_rmsnorm(cg_backend *be, cg_tensor *root, bool *done);
+int try_row_scaled_sum(cg_backend *be, cg_tensor *root, bool *done);
 bool match_rope(cg_tensor *root, RopeMatch *m);
 int rope_operands(cg_backend *be, const RopeMatch &m, bool *ok);
 int rope_into(cg_backend *be, cg_tensor *root, const RopeMatch &m, float *out, const int64_t *o_strides,

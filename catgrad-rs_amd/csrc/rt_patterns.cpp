@@ -887,6 +887,150 @@ int try_gemv_add(cg_backend *be, cg_tensor *root, bool *done) {
 }
 
 
+// ---- a sum of rows, each scaled by a value of its own -------------------------------------------------
+// How a MoE block ends (llm/qwen_moe.py after deepseek.rs:163-165 and qwen3.rs:104-123):
+//   sum_k h_k * broadcast(value_k)  +  shared * broadcast(sigmoid(gate))  +  residual
+// with transposes and reshapes in between that only move axes of extent 1.  One op at a time that is four
+// launches of the generic evaluator (its operand limit, the views and the broadcast of a computed value each
+// end a program); launch_row_scaled_sum adds the terms in the same order, each product and sum rounded alone.
+namespace {
+struct SumTerm {
+  cg_tensor *x, *s;  // rows; one value per row (or null)
+  bool sigmoid;
+};
+
+// rows of `d` values with at most one leading axis longer than 1: views between such shapes keep the row order
+bool rows_shape(const cg_tensor *t, int64_t d) {
+  if (t->rank < 1 || t->shape[t->rank - 1] != d) return false;
+  int big = 0;
+  for (int i = 0; i + 1 < t->rank; ++i) big += t->shape[i] != 1;
+  return big <= 1;
+}
+
+// through deferred reshapes / transposes that nobody else reads and that only move axes of extent 1
+cg_tensor *under_unit_views(cg_tensor *n, const cg_tensor *root, int64_t d) {
+  while ((n->op == N_RESHAPE || n->op == N_TRANSPOSE) && (n == root || refs(n) == 1) && n->in[0] &&
+         n->in[0]->size() == n->size() && rows_shape(n, d) && rows_shape(n->in[0], d))
+    n = n->in[0];
+  return n;
+}
+
+// one value per row: a realised f32 view whose axes are broadcast (stride 0), of extent 1, or step through
+// `rows` values at one stride
+bool row_scalar_view(const cg_tensor *t, int64_t rows, int64_t *stride) {
+  if (t->op != N_REAL || t->stype != ST_F32) return false;
+  int64_t count = 1, st = 0, expect = -1;
+  for (int i = t->rank - 1; i >= 0; --i) {
+    if (t->shape[i] == 1 || t->strides[i] == 0) continue;
+    if (expect < 0) st = t->strides[i];
+    else if (t->strides[i] != expect) return false;
+    expect = t->strides[i] * t->shape[i];
+    count *= t->shape[i];
+  }
+  if (count != rows) return false;
+  *stride = st;
+  return true;
+}
+
+// x, or x * (one value per row), the value possibly through a sigmoid
+bool sum_term(cg_tensor *n, const cg_tensor *root, int64_t rows, int64_t d, SumTerm *out) {
+  n = under_unit_views(n, root, d);
+  out->x = n;
+  out->s = nullptr;
+  out->sigmoid = false;
+  if (n->op == N_REAL || !is_bin(n, E_MUL_F) || refs(n) != 1) return rows_shape(n, d) && n->size() == rows * d;
+  for (int side = 0; side < 2; ++side) {
+    cg_tensor *sc = under_unit_views(n->in[side], root, d), *x = under_unit_views(n->in[1 - side], root, d);
+    if (!rows_shape(x, d) || x->size() != rows * d || sc->size() != rows * d) continue;
+    int64_t st;
+    if (sc->op == N_REAL && sc->strides[sc->rank - 1] == 0 && row_scalar_view(sc, rows, &st)) {
+      out->x = x;
+      out->s = sc;  // a broadcast of values in memory is a view
+      return true;
+    }
+    const cg_tensor *arg = nullptr;
+    if (sc->op == N_BROADCAST && refs(sc) == 1 && sc->in[0]->size() == rows && is_sigmoid_of(sc->in[0], &arg) &&
+        arg->size() == rows) {
+      out->x = x;
+      out->s = const_cast<cg_tensor *>(arg);
+      out->sigmoid = true;
+      return true;
+    }
+  }
+  return rows_shape(n, d) && n->size() == rows * d;  // some other product: a term like any value
+}
+
+// the terms of a chain of additions, left to right (a + b == b + a exactly, so either side may be the chain)
+bool sum_chain(cg_tensor *n, const cg_tensor *root, int64_t rows, int64_t d, std::vector<SumTerm> &terms, int depth) {
+  n = under_unit_views(n, root, d);
+  if (depth < 16 && n->op != N_REAL && is_bin(n, E_ADD_F) && (n == root || refs(n) == 1) && n->size() == rows * d) {
+    for (int side = 0; side < 2; ++side) {
+      cg_tensor *chain = under_unit_views(n->in[side], root, d), *leaf = n->in[1 - side];
+      const bool zero = chain->op == N_CONST && is_constf(chain, 0u);  // the accumulator's first value: 0 + t = t
+      if (!zero && !(chain->op != N_REAL && is_bin(chain, E_ADD_F) && refs(chain) == 1)) continue;
+      if (!zero && !sum_chain(chain, root, rows, d, terms, depth + 1)) return false;
+      SumTerm t;
+      if (!sum_term(leaf, root, rows, d, &t)) return false;
+      terms.push_back(t);
+      return true;
+    }
+    // two values
+    SumTerm a, b;
+    if (!sum_term(n->in[0], root, rows, d, &a) || !sum_term(n->in[1], root, rows, d, &b)) return false;
+    terms.push_back(a);
+    terms.push_back(b);
+    return true;
+  }
+  SumTerm t;
+  if (!sum_term(n, root, rows, d, &t)) return false;
+  terms.push_back(t);
+  return true;
+}
+}  // namespace
+
+int try_row_scaled_sum(cg_backend *be, cg_tensor *root, bool *done) {
+  if (root->dtype != CG_F32 || !is_bin(root, E_ADD_F) || root->rank < 2) return CG_OK;
+  const int64_t d = root->shape[root->rank - 1];
+  if (d < 4 || d % 4 || !rows_shape(root, d)) return CG_OK;
+  const int64_t rows = root->size() / d;
+  if (rows < 1 || rows > 4096) return CG_OK;
+  std::vector<SumTerm> terms;
+  if (!sum_chain(root, root, rows, d, terms, 0)) return CG_OK;
+  int scaled = 0;
+  for (const SumTerm &t : terms) scaled += t.s != nullptr;
+  // (two terms, or none with a scale: the product epilogues and the plain kernels do those)
+  if (terms.size() < 3 || terms.size() > ROW_SUM_MAX_TERMS || !scaled) return CG_OK;
+  RowSumDesc g;
+  std::memset(&g, 0, sizeof(g));
+  g.rows = (uint32_t)rows;
+  g.d = (uint32_t)d;
+  g.n_terms = (uint32_t)terms.size();
+  for (size_t j = 0; j < terms.size(); ++j) {
+    cg_tensor *x = terms[j].x, *sc = terms[j].s;
+    TRY(realize(be, x));
+    if (sc) TRY(realize(be, sc));
+    int64_t rs = 0, ss = 0;
+    if (!rows_view(x, &rs) || x->strides[x->rank - 1] != 1 || rs % 4 || (uintptr_t)data_ptr(x) % 16) return CG_OK;
+    if (sc && !row_scalar_view(sc, rows, &ss)) return CG_OK;
+    g.t[j].x = (const float *)data_ptr(x);
+    g.t[j].x_rs = rs;
+    g.t[j].s = sc ? (const float *)data_ptr(sc) : nullptr;
+    g.t[j].s_rs = ss;
+    g.t[j].sigmoid = terms[j].sigmoid ? 1 : 0;
+  }
+  TRY(alloc_result(be, root, ST_F32));
+  g.out = (float *)root->st->ptr;
+  g.out_rs = d;
+  {
+    KernelScope ks(be, "row_scaled_sum", (double)rows * d * 4 * (terms.size() + 1), 2.0 * rows * d * terms.size());
+    HIPCHK(be, launch_row_scaled_sum(be->lc(), g));
+  }
+  finish_fused(root);
+  *done = true;
+  return CG_OK;
+}
+
+
 int try_binary(cg_backend *be, cg_tensor *root, bool *done) {
   if (root->dtype != CG_F32 || root->op != N_BIN || root->size() % 4 || root->rank == 0) return CG_OK;
   int op;
@@ -943,6 +1087,8 @@ int try_patterns(cg_backend *be, cg_tensor *root, bool *done) {
   TRY(try_rope(be, root, done));
   if (*done) return CG_OK;
   TRY(try_glu(be, root, done));
+  if (*done) return CG_OK;
+  TRY(try_row_scaled_sum(be, root, done));
   if (*done) return CG_OK;
   TRY(try_gemv_add(be, root, done));
   if (*done) return CG_OK;

@@ -733,6 +733,58 @@ def test_decoder_block_of_a_small_batch(oracle, hip, hip_bf16, hip_nopat, rows, 
         assert np.max(np.abs(a - r)) <= 2e-2 * np.abs(r).max()
 
 
+@pytest.mark.parametrize("rows,d,k", [(4, 2048, 4), (2, 64, 2), (37, 260, 6), (3, 8, 1)])
+def test_sum_of_rows_scaled_by_their_own_values(oracle, hip, hip_nopat, rows, d, k):
+    """How a MoE block ends (llm/qwen_moe.py): the k expert rows times their router values, summed from zero
+    in a [rows, 1, d] frame, transposed to [1, rows, d], plus the shared expert's rows through a sigmoid gate,
+    unfolded to [rows, 1, d], plus the residual - one launch, and the bits of the one-op-at-a-time evaluation
+    on the same device (every product and sum rounded on its own, in the same order; the oracle's exp differs
+    from the device's in the last place)."""
+    g = np.random.default_rng(rows * 7 + d + k)
+    hs = [g.standard_normal((rows, 1, d)).astype(np.float32) for _ in range(k)]
+    vals = g.random((rows, k)).astype(np.float32)
+    shared = g.standard_normal((1, rows, d)).astype(np.float32)
+    gate = g.standard_normal((1, rows, 1)).astype(np.float32)
+    res = g.standard_normal((rows, 1, d)).astype(np.float32)
+
+    def f(b, *a):
+        h, (v, sh, gt, rs) = a[:k], a[k:]
+        acc = lang.constant(b, 0.0, lang.shape(b, h[0]))
+        for i in range(k):
+            vi = helpers.unsqueeze(b, 2, 2, lang.get(b, 1, i, v))
+            acc = acc + h[i] * lang.broadcast(b, vi, lang.shape(b, h[i]))
+        acc = lang.transpose(b, 0, 1, acc)
+        out = acc + sh * lang.broadcast(b, nn.sigmoid(b, gt), lang.shape(b, sh))
+        out = lang.reshape(b, lang.shape(b, rs), out)
+        return out + rs
+    args = (*hs, vals, shared, gate, res)
+    (ref,) = vectors.run(oracle, f, 1, *args)
+    (got,), names = run_traced(hip, f, 1, *args)
+    (gen,) = vectors.run(hip_nopat, f, 1, *args)
+    assert names == {"row_scaled_sum"}, sorted(names)
+    assert got.shape == ref.shape and np.array_equal(got, gen), np.abs(got - gen).max()
+    assert np.allclose(got, ref, rtol=1e-6, atol=1e-6)
+
+
+def test_sums_the_row_kernel_leaves_alone(oracle, hip):
+    """Two terms, no scale, or a scale that is not one value per row: the usual kernels."""
+    g = np.random.default_rng(5)
+    a, b_, c = (g.standard_normal((3, 1, 64)).astype(np.float32) for _ in range(3))
+    col = g.standard_normal((1, 1, 64)).astype(np.float32)
+
+    def plain(b, x, y, z):
+        return x + y + z
+
+    def by_column(b, x, y, z, w):
+        return x + y + z * lang.broadcast(b, w, lang.shape(b, z))
+    (ref,) = vectors.run(oracle, plain, 1, a, b_, c)
+    (got,), names = run_traced(hip, plain, 1, a, b_, c)
+    assert "row_scaled_sum" not in names and np.array_equal(got, ref)
+    (ref,) = vectors.run(oracle, by_column, 1, a, b_, c, col)
+    (got,), names = run_traced(hip, by_column, 1, a, b_, c, col)
+    assert "row_scaled_sum" not in names and np.allclose(got, ref, rtol=1e-6, atol=1e-6)
+
+
 @pytest.mark.parametrize("order", ["res_first", "norm_first"])
 @pytest.mark.parametrize("shape", [(2, 33, 1152), (1, 7, 64)])
 def test_rmsnorm_plus_residual(oracle, hip, hip_nopat, shape, order):

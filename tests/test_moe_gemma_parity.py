@@ -496,8 +496,8 @@ def test_moe_cached_decode_hip_vs_oracle(oracle, hip, hip_bf16, mode):
 @pytest.mark.gpu
 def test_generic_program_launches_of_the_other_decoders(hip_bf16):
     """Which launches of a Gemma-3 prefill and of a Qwen-MoE-layout decode step are generic programs:
-    the embedding scale (one per Gemma run) and the weighted expert sum around the routed experts (three
-    per MoE layer); everything else is a pattern kernel."""
+    the embedding scale (one per Gemma run); everything else is a pattern kernel - the weighted sum of the
+    expert rows, the gated shared expert and the residual of a MoE layer are one `row_scaled_sum` launch."""
     be = hip_bf16
     gcfg = MU.gemma_config()
     P = MU.gemma_params(gcfg, seed=9, std=0.2)
@@ -523,5 +523,6 @@ def test_generic_program_launches_of_the_other_decoders(hip_bf16):
     tok, _ = r.step(t)
     be.to_vec(tok)
     counts = be.launch_counts(reset=True)
-    assert sum(counts.get(k, 0) for k in be.GENERIC_PROGRAMS) == 3 * qcfg.num_hidden_layers, counts
+    assert sum(counts.get(k, 0) for k in be.GENERIC_PROGRAMS) == 0, counts
+    assert counts.get("row_scaled_sum") == qcfg.num_hidden_layers, counts
     assert counts.get("softmax_topk") == qcfg.num_hidden_layers and counts.get("attn_decode") == qcfg.num_hidden_layers
