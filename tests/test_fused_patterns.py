@@ -766,6 +766,38 @@ def test_sum_of_rows_scaled_by_their_own_values(oracle, hip, hip_nopat, rows, d,
     assert np.allclose(got, ref, rtol=1e-6, atol=1e-6)
 
 
+@pytest.mark.parametrize("variant", ["right_nested", "shared_term", "two_chains", "scale_on_the_left", "nine_terms"])
+def test_sum_of_scaled_rows_in_other_arrangements(hip, hip_nopat, variant):
+    """Additions nested to the right, a term somebody else reads too, two chains under one addition, the scale as
+    the left factor, more terms than the kernel takes: whatever part the row kernel computes, the values are
+    those of the one-op-at-a-time evaluation, bit for bit."""
+    rows, d = 5, 128
+    g = np.random.default_rng(len(variant))
+    xs = [g.standard_normal((rows, 1, d)).astype(np.float32) for _ in range(9)]
+    sc = [g.random((rows, 1, 1)).astype(np.float32) for _ in range(3)]
+
+    def f(b, *a):
+        x, s = a[:9], [lang.broadcast(b, v, lang.shape(b, a[0])) for v in a[9:]]
+        if variant == "right_nested":
+            return [x[0] + (x[1] * s[0] + (x[2] + x[3] * s[1]))]
+        if variant == "shared_term":
+            t = x[1] * s[0]
+            return [x[0] + t + x[2] * s[1], t + x[3]]
+        if variant == "two_chains":
+            return [(x[0] + x[1] * s[0] + x[2]) + (x[3] * s[1] + x[4] + x[5] * s[2])]
+        if variant == "scale_on_the_left":
+            return [s[0] * x[0] + s[1] * x[1] + x[2]]
+        out = x[0] * s[0]
+        for i in range(1, 9):
+            out = out + x[i] * s[i % 3]
+        return [out]
+    n_out = 2 if variant == "shared_term" else 1
+    got = vectors.run(hip, f, n_out, *xs, *sc)
+    gen = vectors.run(hip_nopat, f, n_out, *xs, *sc)
+    for a, c in zip(got, gen):
+        assert a.shape == c.shape and np.array_equal(a, c), np.abs(a - c).max()
+
+
 def test_sums_the_row_kernel_leaves_alone(oracle, hip):
     """Two terms, no scale, or a scale that is not one value per row: the usual kernels."""
     g = np.random.default_rng(5)
