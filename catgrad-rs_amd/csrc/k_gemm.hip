@@ -2279,7 +2279,9 @@ uint32_t gemm_split_k(const LaunchCtx &lc, const GemmDesc &g) {
     while (tiles * splits * 2 <= (uint64_t)lc.n_cus && g.K / (splits * 2) >= 256 && splits < 16) splits *= 2;
     return splits;
   }
-  if (g.N <= 64) return 1;
+  // (a narrow product - the router of a MoE prefill, 1024 x 60 x 2048: 16 tiles of 64 x 64 walking all of k, 27 us -
+  // is split like any other when its slices stay 16-byte aligned for the summing pass)
+  if (g.N <= 64 && ((uint64_t)batch * g.M * g.N) % 4) return 1;
   while (tiles * splits * 2 <= (uint64_t)lc.n_cus && g.K / (splits * 2) >= 512 && splits < 8) splits *= 2;
   return splits;
 }
