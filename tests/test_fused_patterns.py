@@ -658,6 +658,24 @@ def test_glu_of_a_few_rows_in_the_prologue_of_the_matrix_core_kernel(oracle, hip
     assert np.max(np.abs(got - ref)) <= 1e-2 * np.abs(ref).max()
 
 
+@pytest.mark.parametrize("rows,K,N", [(4, 256, 96), (9, 512, 200)])
+def test_few_rows_that_are_a_slice_of_wider_rows(hip_bf16, rows, K, N):
+    """The input rows as the left half of rows twice as long (a row stride that is not K), and the weights as
+    the left half of a wider matrix: whichever kernel runs, the product of the rounded operands."""
+    g = np.random.default_rng(rows + K + N)
+    x2 = g.standard_normal((1, rows, 2 * K)).astype(np.float32)
+    p = {"w.weight": (g.standard_normal((N, 2 * K)) * 0.05).astype(np.float32)}
+
+    def f(b, xv):
+        xv = xv + xv - xv
+        xs = lang.slice(b, 2, 0, K, xv)
+        w = lang.slice(b, 1, 0, K, lang.param(b, lang.path(["w", "weight"])))
+        return nn.linear_no_bias_param(b, K, N, w, xs)
+    (got,) = vectors.run(hip_bf16, f, 1, x2, params=p)
+    want = vectors.bf16_round(x2[0, :, :K]).astype(np.float64) @ vectors.bf16_round(p["w.weight"][:, :K]).astype(np.float64).T
+    assert got.shape == (1, rows, N) and np.max(np.abs(got[0] - want)) <= 1e-5 * np.abs(want).max()
+
+
 @pytest.mark.parametrize("rows,K", [(17, 256), (16, 2048), (4, 320), (4, 5632)])
 def test_rows_the_matrix_core_kernel_does_not_take(oracle, hip_bf16, rows, K):
     """More than 16 rows, rows that do not fit its LDS, K that its four waves cannot split evenly, or a
