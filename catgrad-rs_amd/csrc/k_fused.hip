@@ -49,7 +49,22 @@ __global__ void __launch_bounds__(BLOCK * RPW) rmsnorm_kernel(RmsNormDesc d) {
   for (int e = 0; e < EPT; ++e) {
     const uint32_t c = (tid + e * BLOCK) * 4;
     if (c < d.n) {
-      v[e] = *(const float4 *)(x + c);
+      if (d.x_slices) {  // the row is still the k-slices of a split product: sum them, keep the sum
+        const uint64_t at = (uint64_t)row * d.n + c;
+        float4 s = *(const float4 *)(d.x_slices + at);
+        for (uint32_t k = 1; k < d.x_n_slices; ++k) {
+          const float4 t = *(const float4 *)(d.x_slices + k * d.x_slice_stride + at);
+          s.x += t.x; s.y += t.y; s.z += t.z; s.w += t.w;
+        }
+        if (d.x_add) {
+          const float4 t = *(const float4 *)(d.x_add + at);
+          s.x += t.x; s.y += t.y; s.z += t.z; s.w += t.w;
+        }
+        *(float4 *)(d.x_out + at) = s;
+        v[e] = s;
+      } else {
+        v[e] = *(const float4 *)(x + c);
+      }
       ss += v[e].x * v[e].x + v[e].y * v[e].y + v[e].z * v[e].z + v[e].w * v[e].w;
     }
   }
@@ -120,6 +135,9 @@ static void launch_rmsnorm_as(const LaunchCtx &lc, const RmsNormDesc &d) {
 
 hipError_t launch_rmsnorm(const LaunchCtx &lc, const RmsNormDesc &d) {
   if (!d.rows || !d.n) return hipSuccess;
+  if (d.x_slices && (!d.x_out || !d.x_n_slices || d.n % 4 || d.x_slice_stride % 4 || d.x_d1 > 1 || d.x_d2 > 1 ||
+                     (uintptr_t)d.x_slices % 16 || (uintptr_t)d.x_out % 16 || (uintptr_t)d.x_add % 16))
+    return hipErrorInvalidValue;
   if (d.y_mid) launch_rmsnorm_as<true>(lc, d);
   else launch_rmsnorm_as<false>(lc, d);
   return hipGetLastError();

@@ -2257,6 +2257,14 @@ bool gemv_rows_plain_ok(const LaunchCtx &lc, const GemmDesc &g) {
   return gemv_rows_mfma_ok(ST_BF16, g.M, g.K, PRO_NONE);
 }
 
+hipError_t launch_splitk_sum(const LaunchCtx &lc, const float *ws, float *c, uint64_t n, uint32_t splits, const float *cadd) {
+  if (!n || !splits) return hipSuccess;
+  if ((uintptr_t)ws % 16 || (uintptr_t)c % 16 || (cadd && (uintptr_t)cadd % 16) || (splits > 1 && n % 4)) return hipErrorInvalidValue;
+  uint64_t blocks = (n / 4 + 255) / 256, cap = (uint64_t)lc.n_cus * 16;
+  CG_LAUNCH(lc, (splitk_reduce_kernel), (unsigned)(blocks < cap ? (blocks ? blocks : 1) : cap), 256, ws, c, n, splits, cadd);
+  return hipGetLastError();
+}
+
 // Split-K factor for a problem too small to fill the CUs with 128x128 tiles (0/1 = none).
 // The caller provides g.workspace of splits * batch * M * N floats and sets g.splits/k_per_split.
 uint32_t gemm_split_k(const LaunchCtx &lc, const GemmDesc &g) {
@@ -2292,7 +2300,7 @@ hipError_t launch_matmul(const LaunchCtx &lc_in, const GemmDesc &g, const char *
   // A product split along k is two launches (the slices, then their sum): when the launch is timed, the
   // start event goes with the first and the stop event with the second, so the record covers both.
   LaunchCtx lc = lc_in, tail = lc_in;
-  if (g.splits > 1) {
+  if (g.splits > 1 && !g.defer_reduce) {
     lc.ev_stop = nullptr;
     tail.ev_start = nullptr;
   }
@@ -2435,7 +2443,7 @@ hipError_t launch_matmul(const LaunchCtx &lc_in, const GemmDesc &g, const char *
       else CG_LAUNCH(lc, (gemm_bf16_nt_kernel<64, 64, false>), gr, 256, gg);
     }
     }
-    if (splits > 1) {
+    if (splits > 1 && !g.defer_reduce) {
       const uint64_t n = (uint64_t)batch * g.M * g.N;
       uint64_t blocks = (n / 4 + 255) / 256, cap = (uint64_t)lc.n_cus * 16;
       CG_LAUNCH(tail, (splitk_reduce_kernel), (unsigned)(blocks < cap ? (blocks ? blocks : 1) : cap), 256,
@@ -2445,7 +2453,7 @@ hipError_t launch_matmul(const LaunchCtx &lc_in, const GemmDesc &g, const char *
   }
   const uint32_t gsplits = g.splits > 1 ? g.splits : 1;
   auto sum_slices = [&]() {
-    if (gsplits > 1) {
+    if (gsplits > 1 && !g.defer_reduce) {
       const uint64_t n = (uint64_t)batch * g.M * g.N;
       uint64_t blocks = (n / 4 + 255) / 256, cap = (uint64_t)lc.n_cus * 16;
       CG_LAUNCH(tail, (splitk_reduce_kernel), (unsigned)(blocks < cap ? (blocks ? blocks : 1) : cap), 256,

@@ -110,6 +110,13 @@ struct RmsNormDesc {
   uint32_t x_d1, x_d2;   // 0 counts as 1
   uint32_t rows, n;
   float n_as_float, eps, gamma_offset;  // gamma_offset: 0 (llama) or 1 (gemma's 1 + gamma)
+  // x as the sum of the k-slices of a split product (non-null x_slices: x_n_slices slices, x_slice_stride
+  // floats apart, each contiguous [rows, n]) plus x_add (contiguous [rows, n], or null), summed in the order
+  // of launch_splitk_sum and also stored to x_out (contiguous [rows, n]); x itself is not read
+  const float *x_slices, *x_add;
+  float *x_out;
+  uint32_t x_n_slices;
+  uint64_t x_slice_stride;
   // Two norms in a row (non-null y_mid): the first result (with its residual) goes to y_mid, contiguous
   // [rows, n], and is normed again with gamma2 (n floats, not null) into y / y16.
   float *y_mid;
@@ -117,6 +124,8 @@ struct RmsNormDesc {
   float eps2, gamma2_offset;
 };
 hipError_t launch_rmsnorm(const LaunchCtx &lc, const RmsNormDesc &d);
+// c[i] = ws[0][i] + ws[1][i] + ... + ws[splits - 1][i] (+ cadd[i]): the k-slices of a split product, n floats each
+hipError_t launch_splitk_sum(const LaunchCtx &lc, const float *ws, float *c, uint64_t n, uint32_t splits, const float *cadd);
 
 struct SoftmaxDesc {
   const float *x;        // row r at x + r * x_row_stride, unit stride along the row
@@ -260,6 +269,9 @@ struct GemmDesc {
   uint32_t splits, k_per_split;
   // optional epilogue of the one-row kernels: C = A . B + c_add (c_add laid out like C)
   const float *c_add;
+  // split along k (splits > 1): leave the slices in the workspace; the caller sums them (launch_splitk_sum, or
+  // the RMSNorm kernel on its way in)
+  int32_t defer_reduce;
   // expert-indirect batches (one-row kernels only): when b_index is set, batch z reads its B
   // matrix at b + b_index[z * b_index_stride] * sb_index instead of the batch strides; an
   // index >= b_index_limit raises ERRF_INDEX_OOB in *err and is clamped

@@ -57,7 +57,9 @@ enum NodeOp : uint8_t {
   N_MATMUL,
   N_REDUCE,     // p0 = ReduceKind
   N_CONCAT,     // p0 = dim
-  N_INDEX       // p0 = dim; in[0] = x, in[1] = indices
+  N_INDEX,      // p0 = dim; in[0] = x, in[1] = indices
+  N_KSUM        // the k-slices of a split product, still to be summed: in[0] = the slices ([p0, size] floats),
+                // in[1] = a value added to the sum (or null); the node already owns the storage of the result
 };
 
 struct TraceRec {
@@ -160,6 +162,12 @@ struct cg_backend {
   // a block-closing value (residual + linear over many rows) to realise at the next call, when its
   // creator has let go of the operands
   cg_tensor *flush_node = nullptr;
+  // A block-closing `residual + linear(x)` realised ahead of its readers (run_pending_flush) may stop at the
+  // k-slices of its product (N_KSUM): the RMSNorm that reads it next sums them on its way in.
+  cg_tensor *ksum_flush_node = nullptr;  // that add, while it is being realised (a weak reference)
+  bool ksum_request = false;   // set by try_gemv_add around its product
+  cgrt::Storage *ksum_ws = nullptr;  // handed back by realize_matmul: the slices (the caller owns them now)
+  uint32_t ksum_splits = 0;
   // set by try_gemv_add around realize_matmul when the addend it passes is a bias vector (one row added
   // to every row of the product) instead of a tensor shaped like the product
   bool addend_is_row = false;

@@ -144,6 +144,20 @@ int realize_arange(cg_backend *be, cg_tensor *n) {
 }
 
 
+// the k-slices of a split product (N_KSUM) that no norm took on its way in: summed by a pass of their own
+int realize_ksum(cg_backend *be, cg_tensor *n) {
+  const cg_tensor *slices = n->in[0], *add = n->in[1];
+  {
+    KernelScope ks(be, "splitk_sum", (double)n->size() * 4 * (n->p0 + (add ? 2 : 1)), 0);
+    HIPCHK(be, launch_splitk_sum(be->lc(), (const float *)data_ptr(slices), (float *)data_ptr(n), (uint64_t)n->size(), (uint32_t)n->p0,
+                                 add ? (const float *)data_ptr(add) : nullptr));
+  }
+  n->op = N_REAL;
+  drop_inputs(n);
+  return CG_OK;
+}
+
+
 int realize(cg_backend *be, cg_tensor *n) {
   switch (n->op) {
     case N_REAL: return CG_OK;
@@ -159,6 +173,7 @@ int realize(cg_backend *be, cg_tensor *n) {
     case N_REDUCE: return realize_reduce(be, n);
     case N_CONCAT: return realize_concat(be, n);
     case N_INDEX: return realize_index(be, n);
+    case N_KSUM: return realize_ksum(be, n);
   }
   return fail(be, CG_ERR_INTERNAL, "realize: unknown node");
 }
@@ -252,7 +267,10 @@ int run_pending_flush(cg_backend *be) {
   int st = CG_OK;
   if (f->rc.load() > 1 && f->op != N_REAL) {  // somebody still wants it
     hipError_t e = hipSetDevice(be->device);
+    // (a norm reads this value next: if its product is split along k, the norm sums the slices itself)
+    be->ksum_flush_node = f;
     st = e == hipSuccess ? realize(be, f) : fail(be, CG_ERR_DEVICE, hipGetErrorString(e));
+    be->ksum_flush_node = nullptr;
   }
   node_release(f);
   return st;
@@ -376,9 +394,14 @@ int binary(cg_backend *be, cg_tensor *a, cg_tensor *b, cg_tensor **out, EwOp f_o
       if (mm->op == N_RESHAPE) mm = mm->in[0];  // batch folded into the rows for the linear and unfolded again
       // the residual stream is a value in memory (the previous block end); anything still deferred
       // on the other side may be part of a pattern around the product (gelu's x + c x^3)
-      if (mm->op != N_MATMUL || other->op != N_REAL) continue;
+      // (or the previous block end still as the k-slices of its product: its strides are those of the sum;
+      // or, in the first block, the embedding rows not yet gathered, behind reshapes at most)
+      const cg_tensor *src = other;
+      while (src->op == N_RESHAPE && src->in[0]) src = src->in[0];
+      const bool in_memory = other->op == N_REAL || other->op == N_KSUM;
+      if (mm->op != N_MATMUL || !(in_memory || src->op == N_INDEX)) continue;
       bool dense = true;
-      for (int i = 0; i < other->rank; ++i) dense = dense && (other->shape[i] == 1 || other->strides[i] != 0);
+      for (int i = 0; in_memory && i < other->rank; ++i) dense = dense && (other->shape[i] == 1 || other->strides[i] != 0);
       // a few-row product with siblings on the same rows (q/k/v, each about to get its bias) is the
       // middle of a block: the siblings' adds are not recorded yet
       if (dense && mm->gemv_candidate)

@@ -500,6 +500,9 @@ int realize_matmul(cg_backend *be, cg_tensor *n, cg_tensor *addend, bool *added,
   }
   if (pb && !ex.w) split_heads(&A, B.shape[2]);
   if (pa) split_heads(&B, A.shape[2]);
+  // an addend that is still the k-slices of an earlier product: the norm among this product's operands has
+  // summed it by now; if there was none, it is summed here
+  if (addend && addend->op == N_KSUM) TRY(realize(be, addend));
   const int r = n->rank;
   const uint32_t M = (uint32_t)n->shape[r - 2], N = (uint32_t)n->shape[r - 1],
                  K = (uint32_t)A.shape[A.rank - 1];
@@ -822,6 +825,8 @@ int realize_matmul(cg_backend *be, cg_tensor *n, cg_tensor *addend, bool *added,
       if (addend && !be->addend_is_row && !g.c_add && !g.b_index) {  // the pass that sums the k-slices adds the residual too
         g.c_add = (const float *)data_ptr(addend);
         *added = true;
+        // ... and the caller may leave that pass to the norm that reads the sum
+        if (be->ksum_request && n->size() % 4 == 0 && n->offset == 0) g.defer_reduce = 1;
       }
     }
     if (dual) {
@@ -867,7 +872,12 @@ int realize_matmul(cg_backend *be, cg_tensor *n, cg_tensor *addend, bool *added,
       c->op = N_REAL;
       drop_inputs(c);
     }
-    storage_release(ws);
+    if (g.defer_reduce && e == hipSuccess) {  // the caller owns the slices now
+      be->ksum_ws = ws;
+      be->ksum_splits = splits;
+    } else {
+      storage_release(ws);
+    }
     storage_release(bt);
     HIPCHK(be, e);
   }

@@ -456,8 +456,18 @@ int try_rmsnorm(cg_backend *be, cg_tensor *root, bool *done) {
   cg_tensor *view = x;
   while (view->op == N_RESHAPE && view->in[0] && view->in[0]->rank >= 1 && view->in[0]->shape[view->in[0]->rank - 1] == n)
     view = view->in[0];
-  TRY(realize(be, view));
-  if (rows_map(view, &rmap) && (rmap.d1 > 1 || rmap.d2 > 1) && (uintptr_t)data_ptr(view) % 16 == 0 &&
+  // The value may still be the k-slices of a split product (plus a residual): the kernel sums them on its way
+  // in, in the order of the pass it replaces, and stores the sum where the value belongs.
+  cg_tensor *ksum = view->op == N_KSUM && n % 4 == 0 && view->size() / n <= UINT32_MAX && view->stype == ST_F32 &&
+                            (uintptr_t)data_ptr(view) % 16 == 0 && (uintptr_t)data_ptr(view->in[0]) % 16 == 0 &&
+                            (!view->in[1] || (uintptr_t)data_ptr(view->in[1]) % 16 == 0)
+                        ? view
+                        : nullptr;
+  if (!ksum) TRY(realize(be, view));
+  if (ksum) {
+    xs = retain(view);
+    row_stride = n;
+  } else if (rows_map(view, &rmap) && (rmap.d1 > 1 || rmap.d2 > 1) && (uintptr_t)data_ptr(view) % 16 == 0 &&
       root->size() / n <= UINT32_MAX) {
     xs = retain(view);
     row_stride = rmap.s0;
@@ -482,21 +492,31 @@ int try_rmsnorm(cg_backend *be, cg_tensor *root, bool *done) {
     d.rows = (uint32_t)(root->size() / n);
     d.n = (uint32_t)n;
     d.residual = rs ? (const float *)data_ptr(rs) : nullptr;
+    double in_bytes = rs ? 8 : 4;
+    if (ksum) {
+      d.x_slices = (const float *)data_ptr(ksum->in[0]);
+      d.x_n_slices = (uint32_t)ksum->p0;
+      d.x_slice_stride = (uint64_t)ksum->size();
+      d.x_add = ksum->in[1] ? (const float *)data_ptr(ksum->in[1]) : nullptr;
+      d.x_out = (float *)data_ptr(ksum);
+      in_bytes += 4.0 * ((double)d.x_n_slices + (d.x_add ? 1 : 0));  // (the 4 above: x_out, written)
+    }
     if (only_gemms) {
       d.y16 = (uint16_t *)root->st->ptr;
     } else {
       d.y = (float *)root->st->ptr;
       if (to_gemms) st = twin_for_result(be, root, &d.y16);
     }
-    KernelScope ks(be, "rmsnorm_fused", (double)root->size() * ((rs ? 8 : 4) + (d.y ? 4 : 0) + (d.y16 ? 2 : 0)) + n * 4, 0);
+    KernelScope ks(be, "rmsnorm_fused", (double)root->size() * (in_bytes + (d.y ? 4 : 0) + (d.y16 ? 2 : 0)) + n * 4, 0);
     if (be->trace_shapes) {  // per-shape records: rmsnorm_fused[16384x1152,+res,f32+bf16]
       char buf[96];
-      snprintf(buf, sizeof buf, "rmsnorm_fused[%ux%u%s%s,%s]", d.rows, d.n, rs ? ",+res" : "", rmap.d1 > 1 || rmap.d2 > 1 ? ",strided" : "",
-               !d.y ? "bf16" : d.y16 ? "f32+bf16" : "f32");
+      snprintf(buf, sizeof buf, "rmsnorm_fused[%ux%u%s%s%s,%s]", d.rows, d.n, ksum ? ",k-slices" : "", rs ? ",+res" : "",
+               rmap.d1 > 1 || rmap.d2 > 1 ? ",strided" : "", !d.y ? "bf16" : d.y16 ? "f32+bf16" : "f32");
       ks.rename(buf);
     }
     hipError_t e = launch_rmsnorm(be->lc(), d);
     if (e != hipSuccess) st = fail(be, CG_ERR_DEVICE, hipGetErrorString(e));
+    else if (ksum) finish_fused(ksum);  // the sum is in memory now
   }
   node_release(xs);
   if (st) return st;
@@ -867,9 +887,20 @@ int try_gemv_add(cg_backend *be, cg_tensor *root, bool *done) {
       be->addend_is_row = false;
       if (st) return st;
     } else {
-      TRY(realize(be, other));
+      // A residual that is itself the unsummed k-slices of the previous block's product stays that way for
+      // now: the norm under this many-row product sums it (realize_matmul sees to it that it is summed by
+      // the time it is added).
+      if (other->op != N_KSUM || mm->gemv_candidate) TRY(realize(be, other));
       if (other->stype != ST_F32 || !is_contiguous(other)) return CG_OK;
-      TRY(realize_matmul(be, mm, other, &added, nullptr));
+      be->ksum_request = be->ksum_flush_node == root;
+      be->ksum_ws = nullptr;
+      const int st = realize_matmul(be, mm, other, &added, nullptr);
+      be->ksum_request = false;
+      if (st) {
+        storage_release(be->ksum_ws);
+        be->ksum_ws = nullptr;
+        return st;
+      }
     }
     if (!added) return CG_OK;  // the product is realised; the generic add takes it from here
     // mm now holds the sum and nobody else can see it: root takes over its storage
@@ -879,6 +910,24 @@ int try_gemv_add(cg_backend *be, cg_tensor *root, bool *done) {
     root->offset = mm->offset;
     if (folded) contiguous_strides(root->rank, root->shape, root->strides);  // products are dense
     else std::copy(mm->strides, mm->strides + mm->rank, root->strides);
+    if (Storage *ws = be->ksum_ws) {
+      // the product was left as its k-slices: root becomes their pending sum (plus the residual)
+      be->ksum_ws = nullptr;
+      const int64_t len = (int64_t)be->ksum_splits * root->size();
+      cg_tensor *slices = new_node(be, CG_F32, 1, &len);
+      slices->st = ws;
+      slices->stype = ST_F32;
+      slices->strides[0] = 1;
+      cg_tensor *keep = retain(other);
+      drop_inputs(root);
+      root->op = N_KSUM;
+      root->ew = 0;
+      root->in[0] = slices;
+      root->in[1] = keep;
+      root->p0 = be->ksum_splits;
+      *done = true;
+      return CG_OK;
+    }
     finish_fused(root);
     *done = true;
     return CG_OK;

@@ -337,6 +337,52 @@ def test_residual_add_with_a_split_gemm(oracle, hip_bf16, shape):
     assert np.max(np.abs(got[0] - ref)) <= 2e-2 * np.abs(ref).max()
 
 
+@pytest.mark.parametrize("shape", [(512, 8192, 2048), (256, 2048, 512), (512, 2048, 2048), (100, 4096, 264)])  # M, K, N
+@pytest.mark.parametrize("mode", ["bf16", "f32"])
+def test_norm_that_sums_the_slices_of_a_split_gemm(hip, hip_bf16, shape, mode):
+    """`residual + linear(x)` over many rows closes a decoder block (models/llama.rs:166-186) and an RMSNorm
+    reads it next.  When the product is split along k, the block end stays the slices of the product and the
+    norm sums them (and the residual) on its way in, storing the sum for its other readers: the bits of the
+    same two blocks run as two programs, where the sum is a pass of its own."""
+    be = hip_bf16 if mode == "bf16" else hip
+    M, K, N = shape
+    g = np.random.default_rng(M + K + N)
+    x = vectors.bf16_round(g.standard_normal((1, M, K)).astype(np.float32))
+    p = {"a.weight": vectors.bf16_round((g.standard_normal((N, K)) * 0.05).astype(np.float32)),
+         "b.weight": vectors.bf16_round((g.standard_normal((N, N)) * 0.05).astype(np.float32)),
+         "n.weight": g.standard_normal(N).astype(np.float32)}
+    res = g.standard_normal(M * N).astype(np.float32)   # rank 1: stays f32 in bf16 mode
+
+    def first(b, xv, rv):
+        xv = xv + xv - xv
+        y = nn.linear_no_bias(b, K, N, lang.path(["a"]), xv)
+        return lang.reshape(b, lang.shape(b, y), rv) + y
+
+    def second(b, hv):
+        return hv + nn.linear_no_bias(b, N, N, lang.path(["b"]), helpers.rmsnorm(b, 1e-5, lang.path(["n"]), hv))
+
+    def second_alone(b, hv):
+        return second(b, lang.reshape(b, lang.make_shape(b, 1, M, N), hv))
+
+    def both(b, xv, rv):
+        h = first(b, xv, rv)
+        return second(b, h), h
+    (h_alone,) = vectors.run(be, first, 1, x, res, params=p)
+    (h2_alone,) = vectors.run(be, second_alone, 1, h_alone.reshape(-1), params=p)
+    be.launch_counts(reset=True)
+    h2, h = vectors.run(be, both, 2, x, res, params=p)
+    counts = be.launch_counts(reset=True)
+    assert np.array_equal(h, h_alone) and np.array_equal(h2, h2_alone)
+    assert counts.get("rmsnorm_fused") == 1, counts
+    be.trace(2)
+    be.trace_reset()
+    vectors.run(be, both, 2, x, res, params=p)
+    names = set(be.trace_report())
+    be.trace(False)
+    if shape[:2] in ((512, 8192), (256, 2048), (512, 2048)):  # split along k: the sum is the norm's
+        assert any(n.startswith("rmsnorm_fused[") and "k-slices" in n for n in names), sorted(names)
+
+
 @pytest.mark.parametrize("cfg", [(1, 32, 8, 513, 64), (1, 4, 4, 7, 16), (2, 8, 2, 100, 128), (1, 4, 1, 33, 256),
                                  (1, 16, 16, 1, 64), (1, 2, 1, 9000, 64), (1, 32, 8, 2049, 128),
                                  (3, 4, 2, 700, 256)])  # b, heads, kv heads, T, d
