@@ -852,6 +852,47 @@ hipError_t launch_ew(const LaunchCtx &lc, const Program &p, const OutDesc &o, ui
   return hipGetLastError();
 }
 
+// Thousands of argmax records (one per wave of the launch that stored the row): one workgroup of 1024 threads,
+// a thread's records requested four at a time before any is merged, then wave shuffles and one exchange in LDS.
+__global__ void __launch_bounds__(1024) argmax_records_kernel(const uint32_t *records, uint32_t *out, uint32_t n) {
+  __shared__ uint32_t part[16][3];
+  const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  Acc<R_ARGMAX_F> acc;
+  for (uint32_t base = 0; base < n; base += 4096) {
+    uint32_t w[4][3];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const uint32_t c = min(base + u * 1024 + tid, n - 1);  // (past the end: the last record again)
+#pragma unroll
+      for (int j = 0; j < 3; ++j) w[u][j] = records[(uint64_t)c * 3 + j];
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      Acc<R_ARGMAX_F> o;
+      o.set(w[u]);
+      acc.merge(o);
+    }
+  }
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) acc.merge(shfl_xor_acc<R_ARGMAX_F>(acc, m));
+  if (lane == 0) acc.get(part[wave]);
+  __syncthreads();
+  if (tid == 0) {
+    for (int w2 = 1; w2 < 16; ++w2) {
+      Acc<R_ARGMAX_F> o;
+      o.set(part[w2]);
+      acc.merge(o);
+    }
+    out[0] = acc.result();
+  }
+}
+
+hipError_t launch_argmax_merge(const LaunchCtx &lc, const uint32_t *records, uint32_t *out, uint32_t n_records) {
+  if (!n_records) return hipErrorInvalidValue;
+  CG_LAUNCH(lc, (argmax_records_kernel), 1, 1024, records, out, n_records);
+  return hipGetLastError();
+}
+
 template <int KIND>
 static hipError_t launch_reduce_kind(const LaunchCtx &lc, const Program &p, uint32_t *out,
                                      uint32_t rows, uint32_t n, bool vec4, uint32_t *scratch,

@@ -1077,7 +1077,11 @@ hipError_t launch_gemv_multi(const LaunchCtx &lc, const GemvMultiDesc &g) {
 // exp(max_s - max) / sum.  All of it is requested with the first loads, so the attention launch needs no
 // hand-over between its workgroups (acknowledged stores, a counter, a second pass over the partials:
 // 2.8 us of a 6.7 us kernel) and the merge costs this launch one LDS exchange.
-template <typename TB, bool KSPLIT, bool GLUEPI, int MR, int XV, bool MERGE = false>
+// AMAX (one row, one problem, no k-split): a wave also keeps the largest value it stores - in the order of
+// f32::total_cmp, the last of equal values winning, like Backend::argmax (ndarray.rs:469-480) - and leaves
+// (key, column, any) in g.amax_part[wave of the grid]: the argmax over the row then only merges these records
+// instead of reading the row back.
+template <typename TB, bool KSPLIT, bool GLUEPI, int MR, int XV, bool MERGE = false, bool AMAX = false>
 __global__ void __launch_bounds__(256) gemv_pro_kernel(GemvProDesc g) {
   typedef typename WVec<TB>::type VT;
   constexpr int EPL = WVec<TB>::EPL, UNROLL = 4, R = 2;
@@ -1086,6 +1090,9 @@ __global__ void __launch_bounds__(256) gemv_pro_kernel(GemvProDesc g) {
   __shared__ float part[4][R][MR];
   __shared__ float2 merge_ml[MERGE ? 256 : 1];
   static_assert(!MERGE || (MR == 1 && !GLUEPI && !KSPLIT), "the attention merge feeds one row to a plain product");
+  static_assert(!AMAX || (MR == 1 && !GLUEPI && !KSPLIT && !MERGE), "argmax records: one row, a plain product");
+  int32_t best_key = INT32_MIN;
+  uint32_t best_col = 0, best_any = 0;
   warm_kernel_arguments<sizeof(GemvProDesc)>();
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const uint32_t K = g.m.K, bz = blockIdx.z;
@@ -1342,24 +1349,54 @@ __global__ void __launch_bounds__(256) gemv_pro_kernel(GemvProDesc g) {
         for (int m = 0; m < MR; ++m)
           if ((uint32_t)m < rows && nb + r < N) {
             const uint64_t at = (uint64_t)m * N + nb + r;
-            C[at] = acc[r][m] + (Cadd ? Cadd[(uint64_t)m * cadd_rs + nb + r] : 0.f);
+            const float v = acc[r][m] + (Cadd ? Cadd[(uint64_t)m * cadd_rs + nb + r] : 0.f);
+            C[at] = v;
+            if (AMAX) {
+              const int32_t b = __float_as_int(v), key = b ^ (int32_t)(((uint32_t)(b >> 31)) >> 1);
+              if (!best_any || key > best_key || (key == best_key && nb + r > best_col)) {
+                best_key = key;
+                best_col = nb + r;
+                best_any = 1;
+              }
+            }
           }
     }
   }
+  if (AMAX && lane == 0) {  // (a wave without a column leaves any = 0)
+    uint32_t *rec = g.amax_part + (uint64_t)(blockIdx.x * 4 + wave) * 3;
+    rec[0] = (uint32_t)best_key;
+    rec[1] = best_col;
+    rec[2] = best_any;
+  }
+}
+
+// workgroups along x of the plain (no GLU epilogue, no attention merge) form
+static uint32_t gemv_pro_block_count(const LaunchCtx &lc, const GemvProDesc &g, uint32_t slots, bool ksplit, bool multi) {
+  // `slots` = column pairs per problem; 256-thread workgroups (wider ones stream worse).  Long input
+  // rows cost more to recompute, so fewer workgroups each take several column pairs.
+  const uint32_t per_wg = ksplit ? 1 : 4;
+  uint32_t blocks = (slots + per_wg - 1) / per_wg;
+  const uint32_t batch = g.batch ? g.batch : 1;
+  // (several rows: two workgroups fit a CU and staging the rows costs as much as a pass of columns - one round)
+  const uint32_t cap = (uint32_t)lc.n_cus * (multi || g.m.K >= 4096 ? 2 : 4) / (g.m.n_prob * batch);
+  if (blocks > cap) blocks = cap ? cap : 1;
+  return blocks;
 }
 
 template <typename TB, bool KSPLIT, int MR>
 static void launch_gemv_pro_block(const LaunchCtx &lc, const GemvProDesc &g, uint32_t slots) {
-  // `slots` = column pairs per problem; 256-thread workgroups (wider ones stream worse).  Long input
-  // rows cost more to recompute, so fewer workgroups each take several column pairs.
-  const uint32_t per_wg = KSPLIT ? 1 : 4;
-  uint32_t blocks = (slots + per_wg - 1) / per_wg;
+  const uint32_t blocks = gemv_pro_block_count(lc, g, slots, KSPLIT, MR > 1);
   const uint32_t batch = g.batch ? g.batch : 1;
-  // (several rows: two workgroups fit a CU and staging the rows costs as much as a pass of columns - one round)
-  const uint32_t cap = (uint32_t)lc.n_cus * (MR > 1 || g.m.K >= 4096 ? 2 : 4) / (g.m.n_prob * batch);
-  if (blocks > cap) blocks = cap ? cap : 1;
   dim3 grid(blocks, g.m.n_prob, batch);
   const uint32_t xv = ((MR > 1 ? g.rows : 1u) * g.m.K / 4 + 255) / 256;  // 16-byte pieces of the input rows per thread
+  if constexpr (!KSPLIT && MR == 1) {
+    if (g.amax_part) {  // (launch_gemv_pro has checked gemv_pro_amax_records)
+      if (xv <= 2) CG_LAUNCH(lc, (gemv_pro_kernel<TB, false, false, 1, 2, false, true>), grid, 256, g);
+      else if (xv <= 4) CG_LAUNCH(lc, (gemv_pro_kernel<TB, false, false, 1, 4, false, true>), grid, 256, g);
+      else CG_LAUNCH(lc, (gemv_pro_kernel<TB, false, false, 1, 8, false, true>), grid, 256, g);
+      return;
+    }
+  }
   if (xv <= 2) CG_LAUNCH(lc, (gemv_pro_kernel<TB, KSPLIT, false, MR, 2>), grid, 256, g);
   else if (xv <= 4) CG_LAUNCH(lc, (gemv_pro_kernel<TB, KSPLIT, false, MR, 4>), grid, 256, g);
   else CG_LAUNCH(lc, (gemv_pro_kernel<TB, KSPLIT, false, MR, 8>), grid, 256, g);
@@ -1622,10 +1659,22 @@ static hipError_t launch_gemv_rows_mfma(const LaunchCtx &lc, const GemvProDesc &
 }
 
 
+// Whether (and how finely) launch_gemv_pro can leave argmax records: the number of records the launch writes
+// to GemvProDesc::amax_part (3 words each), or 0 when this product takes another form.
+uint32_t gemv_pro_amax_records(const LaunchCtx &lc, const GemvProDesc &g) {
+  if (g.m.n_prob != 1 || g.rows > 1 || g.batch > 1 || g.b_index || g.slot_tokens || g.glu_epilogue || g.pro == PRO_ATTN_MERGE ||
+      !g.m.p[0].N || g.m.K > GEMV_PRO_MAX_K)
+    return 0;
+  const uint32_t slots = (g.m.p[0].N + 1) / 2;
+  if (g.m.K >= 4096 && slots <= (uint32_t)lc.n_cus * 8) return 0;  // k split over the waves
+  return gemv_pro_block_count(lc, g, slots, false, false) * 4;
+}
+
 hipError_t launch_gemv_pro(const LaunchCtx &lc, const GemvProDesc &g) {
   uint32_t max_n = 0;
   for (int i = 0; i < g.m.n_prob; ++i) max_n = g.m.p[i].N > max_n ? g.m.p[i].N : max_n;
   if (!max_n || !g.m.n_prob) return hipSuccess;
+  if (g.amax_part && !gemv_pro_amax_records(lc, g)) return hipErrorInvalidValue;
   if (g.pro == PRO_ATTN_MERGE) {
     if (!g.merge_part || g.merge_splits < 1 || g.merge_splits > ATTN_MERGE_MAX_SPLITS || g.merge_d % 4 || !g.merge_d ||
         g.merge_heads * g.merge_splits > 256 || g.m.K != g.merge_heads * g.merge_d || g.m.K > 2048 || g.m.K % 8 ||

@@ -372,8 +372,15 @@ struct GemvProDesc {
   // PRO_ATTN_MERGE: the attention's partials (AttnDecodeDesc::part with merge_later) and their geometry
   const float *merge_part;
   uint32_t merge_splits, merge_heads, merge_d;
+  // optional: gemv_pro_amax_records(lc, g) records of 3 words, the argmax of the stored row in pieces
+  // (launch_argmax_merge finishes it)
+  uint32_t *amax_part;
 };
 hipError_t launch_gemv_pro(const LaunchCtx &lc, const GemvProDesc &g);
+// the number of argmax records launch_gemv_pro would write for this product (0: it cannot)
+uint32_t gemv_pro_amax_records(const LaunchCtx &lc, const GemvProDesc &g);
+// out[0] = the argmax (Backend::argmax's order) over `records` records of (key, column, any)
+hipError_t launch_argmax_merge(const LaunchCtx &lc, const uint32_t *records, uint32_t *out, uint32_t n_records);
 // largest K the several-row form on the vector ALUs takes for weights of this storage type
 uint32_t gemv_pro_multi_row_max_k(int b_stype);
 // most input rows any several-row form takes

@@ -168,6 +168,12 @@ struct cg_backend {
   bool ksum_request = false;   // set by try_gemv_add around its product
   cgrt::Storage *ksum_ws = nullptr;  // handed back by realize_matmul: the slices (the caller owns them now)
   uint32_t ksum_splits = 0;
+  // argmax over the row a one-row product is about to store (the logits of a greedy decode step): realize_reduce
+  // names the product, try_gemv_prologue's launch leaves the argmax in pieces (GemvProDesc::amax_part) and hands
+  // the records back
+  cg_tensor *amax_want = nullptr;
+  cgrt::Storage *amax_records = nullptr;
+  uint32_t amax_n_records = 0;
   // set by try_gemv_add around realize_matmul when the addend it passes is a bias vector (one row added
   // to every row of the product) instead of a tensor shaped like the product
   bool addend_is_row = false;

@@ -386,6 +386,41 @@ bool rows_layout(const cg_tensor *t, int64_t *row_stride) {
 int realize_reduce(cg_backend *be, cg_tensor *n) {
   cg_tensor *x = n->in[0];
   const int kind = (int)n->p0;
+  // Greedy decoding (llm/utils.rs: argmax of the last position's logits): the row is a one-row product that is
+  // still deferred.  Its launch keeps, per wave, the largest value it stores; the argmax merges those records
+  // instead of reading 128 K logits back with two launches of its own.
+  if (kind == R_ARGMAX_F && !(be->flags & CG_FLAG_NO_PATTERNS) && x->rank >= 1 && x->size() == x->shape[x->rank - 1] &&
+      x->size() >= 4096) {
+    cg_tensor *mm = x;
+    while (mm->op == N_RESHAPE && mm->in[0] && mm->in[0]->size() == mm->size()) mm = mm->in[0];
+    if (mm->op == N_MATMUL && mm->gemv_candidate && mm->dtype == CG_F32) {
+      be->amax_want = mm;
+      be->amax_records = nullptr;
+      const int st = realize(be, mm);
+      be->amax_want = nullptr;
+      Storage *records = be->amax_records;
+      be->amax_records = nullptr;
+      if (st) {
+        storage_release(records);
+        return st;
+      }
+      if (records) {
+        int st2 = alloc_result(be, n, ST_U32);
+        hipError_t e = hipSuccess;
+        if (!st2) {
+          KernelScope ks(be, "reduce_argmax", (double)be->amax_n_records * 12 + 4, 0);
+          if (be->trace_shapes) ks.rename("reduce_argmax[records]");
+          e = launch_argmax_merge(be->lc(), (const uint32_t *)records->ptr, (uint32_t *)n->st->ptr, be->amax_n_records);
+        }
+        storage_release(records);
+        if (st2) return st2;
+        HIPCHK(be, e);
+        n->op = N_REAL;
+        drop_inputs(n);
+        return CG_OK;
+      }
+    }
+  }
   // a tensor that is (or has to be) in memory anyway, with enough rows to fill the device: stream it
   if (!(be->flags & CG_FLAG_NO_PATTERNS) && !((x->op == N_BIN || x->op == N_UN) && x->rc.load() == 1) &&
       x->rank >= 1 && x->size() > 0 && x->size() < ((int64_t)1 << 32)) {

@@ -363,8 +363,18 @@ int try_gemv_prologue(cg_backend *be, cg_tensor *n, cg_tensor *addend, bool *add
                d.m.n_prob, (long long)rows, (long long)K, flops / (2.0 * rows * K));
       ks.rename(buf);
     }
+    // the argmax over this row is wanted next: the launch leaves it in pieces
+    Storage *records = nullptr;
+    uint32_t n_records = be->amax_want == n && !bias_add[0] ? gemv_pro_amax_records(be->lc(), d) : 0;
+    if (n_records && dev_alloc(be, (size_t)n_records * 12, &records) == CG_OK) d.amax_part = (uint32_t *)records->ptr;
     hipError_t e = launch_gemv_pro(be->lc(), d);
     if (e != hipSuccess) st = fail(be, CG_ERR_DEVICE, hipGetErrorString(e));
+    if (!st && records) {
+      be->amax_records = records;
+      be->amax_n_records = n_records;
+    } else {
+      storage_release(records);
+    }
   }
   node_release(a0);
   node_release(a1);

@@ -797,6 +797,52 @@ def test_decoder_block_of_a_small_batch(oracle, hip, hip_bf16, hip_nopat, rows, 
         assert np.max(np.abs(a - r)) <= 2e-2 * np.abs(r).max()
 
 
+@pytest.mark.parametrize("K,N", [(2048, 128256), (2048, 4100), (512, 9001), (4096, 40000), (8192, 4096), (2048, 4095)])
+@pytest.mark.parametrize("mode", ["f32", "bf16"])
+def test_argmax_of_the_row_a_projection_stores(oracle, hip, hip_bf16, hip_nopat, K, N, mode):
+    """Greedy decoding: final norm, lm_head, argmax over the logits.  The product's launch keeps the largest
+    value each wave stores and the argmax merges those records (one small launch) instead of reading the row
+    back.  Equal maxima: the last one wins, as in the reference (ndarray.rs:469-480) - the matrix holds the same
+    row several times.  Same index as the op-at-a-time evaluation of the same logits."""
+    be = hip if mode == "f32" else hip_bf16
+    g = np.random.default_rng(K + N)
+    x = g.standard_normal((1, 1, K)).astype(np.float32)
+    w = vectors.bf16_round((g.standard_normal((N, K)) * 0.05).astype(np.float32))
+    p = {"n.weight": g.standard_normal(K).astype(np.float32), "l.weight": w}
+
+    def f(b, xv):
+        xv = xv + xv - xv      # a computed f32 row, like the residual stream
+        lg = nn.linear_no_bias(b, K, N, lang.path(["l"]), helpers.rmsnorm(b, 1e-5, lang.path(["n"]), xv))
+        return lang.argmax(b, lg), lg
+    tok, lg = vectors.run(be, f, 2, x, params=p)
+    # the winning row three more times, one of them in the last column: four equal maxima
+    top = int(np.argmax(lg.reshape(-1)))
+    for at in (7, N // 2 + 1, N - 1):
+        w[at] = w[top]
+    be.launch_counts(reset=True)
+    tok, lg = vectors.run(be, f, 2, x, params=p)
+    counts = be.launch_counts(reset=True)
+    flat = lg.reshape(-1)
+    assert flat[7] == flat[top] == flat[N - 1] == flat.max()
+    assert int(tok.reshape(-1)[0]) == N - 1
+    for other in (hip_nopat, oracle):   # the argmax op on its own, over the same logits
+        (alone,) = vectors.run(other, lambda b, v: lang.argmax(b, v), 1, lg.reshape(-1))
+        assert int(np.asarray(alone).reshape(-1)[0]) == N - 1
+    x16 = vectors.bf16_round(x) if mode == "bf16" else x
+    ref_tok, ref_lg = vectors.run(oracle, f, 2, x16, params=p)
+    assert np.max(np.abs(lg - ref_lg)) <= (1e-4 if mode == "f32" else 2e-2) * np.abs(ref_lg).max()
+    counts.pop("ew_to_bf16", None)   # (the parameters on their way in)
+    assert counts.get("reduce_argmax") == 1 and sum(counts.values()) == 3, counts   # x + x - x, product, argmax
+    be.trace(2)
+    be.trace_reset()
+    vectors.run(be, f, 2, x, params=p)
+    names = set(be.trace_report())
+    be.trace(False)
+    # the one-row kernel leaves the records unless it splits k over its waves (deep and narrow: (8192, 4096)):
+    # the argmax reads those, not the row
+    assert ("reduce_argmax[records]" in names) == (N >= 4096 and (K, N) != (8192, 4096)), sorted(names)
+
+
 @pytest.mark.parametrize("rows,d,k", [(4, 2048, 4), (2, 64, 2), (37, 260, 6), (3, 8, 1)])
 def test_sum_of_rows_scaled_by_their_own_values(oracle, hip, hip_nopat, rows, d, k):
     """How a MoE block ends (llm/qwen_moe.py): the k expert rows times their router values, summed from zero
