@@ -1877,7 +1877,11 @@ __global__ void __launch_bounds__(256) moe_gemm_kernel(MoeGemmDesc g) {
 // One workgroup of 1024 threads sorts the (slot, token) pairs by expert: a histogram in LDS, a scan,
 // and a scatter through per-expert cursors.  The order of an expert's pairs depends on the order
 // the atomics land in, which only decides the tile row a token occupies, never its result.
-__global__ void __launch_bounds__(1024) moe_route_kernel(MoeGemmDesc g, uint32_t *count, uint32_t *offset, uint32_t *list) {
+// tiles (optional): tiles[0] = the number of 128-pair row tiles over all experts, tiles[1 + t] = expert << 16 |
+// row tile within the expert, expert by expert - the work list of the GEMM, one workgroup per (row tile, column
+// tile), so that an expert most tokens chose is spread over the device instead of walked by one workgroup.
+__global__ void __launch_bounds__(1024) moe_route_kernel(MoeGemmDesc g, uint32_t *count, uint32_t *offset, uint32_t *list,
+                                                         uint32_t *tiles) {
   __shared__ uint32_t hist[MOE_ROUTE_MAX_EXPERTS], cursor[MOE_ROUTE_MAX_EXPERTS], scan[1024];
   const uint32_t tid = threadIdx.x, E = g.n_expert, S = g.S, pairs = S * g.n_slot;
   for (uint32_t i = tid; i < E; i += 1024) hist[i] = 0;
@@ -1916,12 +1920,32 @@ __global__ void __launch_bounds__(1024) moe_route_kernel(MoeGemmDesc g, uint32_t
     const uint32_t ix = min(g.slot[sl].idx[(int64_t)t * g.slot[sl].idx_stride], E - 1);
     list[atomicAdd(&cursor[ix], 1u)] = sl << 16 | t;
   }
+  if (!tiles) return;
+  // the same scan over row tiles per expert
+  uint32_t my_tiles = 0;
+  for (uint32_t i = first; i < min(E, first + per); ++i) my_tiles += (hist[i] + 127) / 128;
+  scan[tid] = my_tiles;
+  __syncthreads();
+  for (uint32_t d = 1; d < 1024; d <<= 1) {
+    const uint32_t v = tid >= d ? scan[tid - d] : 0u;
+    __syncthreads();
+    scan[tid] += v;
+    __syncthreads();
+  }
+  uint32_t tt = scan[tid] - my_tiles;
+  for (uint32_t i = first; i < min(E, first + per); ++i)
+    for (uint32_t j = 0; j < (hist[i] + 127) / 128; ++j) tiles[1 + tt++] = i << 16 | j;
+  if (tid == 1023) tiles[0] = scan[1023];
 }
 
-hipError_t launch_moe_route(const LaunchCtx &lc, const MoeGemmDesc &g, uint32_t *count, uint32_t *offset, uint32_t *list) {
+// most row tiles launch_moe_route can list for g: every expert may end in a partly filled one
+uint32_t moe_route_max_tiles(const MoeGemmDesc &g) { return (g.S * g.n_slot + 127) / 128 + g.n_expert; }
+
+hipError_t launch_moe_route(const LaunchCtx &lc, const MoeGemmDesc &g, uint32_t *count, uint32_t *offset, uint32_t *list,
+                            uint32_t *tiles) {
   if (!g.S || !g.n_slot || !g.n_expert) return hipSuccess;
   if (g.n_expert > MOE_ROUTE_MAX_EXPERTS || g.S > 65535 || g.n_slot > 8) return hipErrorInvalidValue;
-  CG_LAUNCH(lc, moe_route_kernel, 1, 1024, g, count, offset, list);
+  CG_LAUNCH(lc, moe_route_kernel, 1, 1024, g, count, offset, list, tiles);
   return hipGetLastError();
 }
 
@@ -1945,9 +1969,17 @@ __global__ void __launch_bounds__(256) moe_gemm_dma_kernel(MoeGemmDesc g) {
   // consecutive workgroups (dealt round-robin to the 8 XCDs) take the column tiles of one expert: giving an
   // XCD a contiguous range of experts instead measured 10 % slower
   const uint32_t id = blockIdx.x;
-  const uint32_t e = id / tiles_n, n0 = (id - e * tiles_n) * BN_;
+  uint32_t e = id / tiles_n, m_first = 0, m_last = UINT32_MAX;
+  const uint32_t n0 = (id - e * tiles_n) * BN_;
+  if (g.route_tiles) {  // one row tile of one expert
+    if (e >= g.route_tiles[0]) return;  // the grid is sized for the most tiles there can be
+    const uint32_t ent = g.route_tiles[1 + e];
+    e = ent >> 16;
+    m_first = (ent & 0xFFFFu) * BM_;
+    m_last = m_first + BM_;
+  }
   if (e >= g.n_expert) return;  // the grid is sized for the wider problem
-  const uint32_t cnt = g.route_count[e];
+  const uint32_t cnt = min(g.route_count[e], m_last);
   const uint32_t *list = g.route_list + g.route_offset[e];
   const uint16_t *W[NP];
   int64_t sbn[NP];
@@ -1959,7 +1991,7 @@ __global__ void __launch_bounds__(256) moe_gemm_dma_kernel(MoeGemmDesc g) {
   const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint16_t *)dma_smem;
   const int sw = (lane >> 1) & 7, half = lane >> 5;
   const int n_steps = (int)(K / BK);
-  for (uint32_t m0 = 0; m0 < cnt; m0 += BM_) {
+  for (uint32_t m0 = m_first; m0 < cnt; m0 += BM_) {
     const int live_tiles = (int)min((uint32_t)MT, (cnt - m0 + 31) / 32);  // wave-uniform
     f32x16 acc[NP][MT];
 #pragma unroll
@@ -2126,11 +2158,12 @@ hipError_t launch_moe_gemm(const LaunchCtx &lc, const MoeGemmDesc &g) {
   if (!max_n) return hipSuccess;
   if (g.fuse_glu) {
     if (g.n_prob != 2 || g.prob[0].N != g.prob[1].N || g.pro != PRO_NONE) return hipErrorInvalidValue;
-    if (moe_gemm_pipelined_ok(g)) return launch_moe_gemm_dma<2, 3>(lc, g, dim3((max_n + 127) / 128 * g.n_expert, 1, 1));
+    if (moe_gemm_pipelined_ok(g))
+      return launch_moe_gemm_dma<2, 3>(lc, g, dim3((max_n + 127) / 128 * (g.route_tiles ? moe_route_max_tiles(g) : g.n_expert), 1, 1));
     dim3 grid((max_n + 127) / 128, g.n_expert, 1);
     CG_LAUNCH(lc, moe_gemm_kernel<2>, grid, 256, g);
   } else if (moe_gemm_pipelined_ok(g)) {
-    return launch_moe_gemm_dma<1, 2>(lc, g, dim3((max_n + 127) / 128 * g.n_expert, g.n_prob, 1));
+    return launch_moe_gemm_dma<1, 2>(lc, g, dim3((max_n + 127) / 128 * (g.route_tiles ? moe_route_max_tiles(g) : g.n_expert), g.n_prob, 1));
   } else {
     dim3 grid((max_n + 127) / 128, g.n_expert, g.n_prob);
     CG_LAUNCH(lc, moe_gemm_kernel<1>, grid, 256, g);

@@ -424,6 +424,8 @@ struct MoeGemmDesc {
   // optional: the (slot, token) pairs already sorted by expert (launch_moe_route): pairs
   // route_list[route_offset[e] .. + route_count[e]) = slot << 16 | token chose expert e
   const uint32_t *route_count, *route_offset, *route_list;
+  // optional, with the above: the row tiles of all experts as a work list (launch_moe_route's `tiles`)
+  const uint32_t *route_tiles;
 };
 hipError_t launch_moe_gemm(const LaunchCtx &lc, const MoeGemmDesc &g);
 // Sorts the S * n_slot (slot, token) pairs of g by expert into count / offset (n_expert words each) and
@@ -431,7 +433,12 @@ hipError_t launch_moe_gemm(const LaunchCtx &lc, const MoeGemmDesc &g);
 // (slot[].a16 for every slot) and K % 64 == 0, launch_moe_gemm streams the weights through a
 // multi-stage direct-to-LDS pipeline.
 enum { MOE_ROUTE_MAX_EXPERTS = 4096 };
-hipError_t launch_moe_route(const LaunchCtx &lc, const MoeGemmDesc &g, uint32_t *count, uint32_t *offset, uint32_t *list);
+// tiles (optional, 1 + moe_route_max_tiles(g) words): the number of 128-pair row tiles over all experts, then
+// expert << 16 | row tile for each; with it in g.route_tiles a workgroup of launch_moe_gemm owns one row tile
+// of one expert, so the launch stays balanced when most tokens choose the same few experts.
+hipError_t launch_moe_route(const LaunchCtx &lc, const MoeGemmDesc &g, uint32_t *count, uint32_t *offset, uint32_t *list,
+                            uint32_t *tiles);
+uint32_t moe_route_max_tiles(const MoeGemmDesc &g);
 bool moe_gemm_pipelined_ok(const MoeGemmDesc &g);
 // wrapping u32 matmul (ndarray's generic dot); all operands contiguous
 hipError_t launch_matmul_u32(const LaunchCtx &lc, const uint32_t *a, const uint32_t *b, uint32_t *c,

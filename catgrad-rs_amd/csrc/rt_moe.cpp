@@ -200,17 +200,18 @@ int try_moe_gemm(cg_backend *be, cg_tensor *n, bool *done) {
         // the pairs sorted by expert once, for both launches: count, offset (one word per expert), list
         Storage *route = nullptr;
         if (d.n_expert <= MOE_ROUTE_MAX_EXPERTS && H % 64 == 0 && F % 64 == 0) {
-          const size_t words = 2 * (size_t)d.n_expert + (size_t)S * d.n_slot;
+          const size_t words = 2 * (size_t)d.n_expert + (size_t)S * d.n_slot + 1 + moe_route_max_tiles(d);
           st = dev_alloc(be, words * 4, &route);
           if (st) {
             drop_h();
             return st;
           }
-          uint32_t *rc = (uint32_t *)route->ptr, *ro = rc + d.n_expert, *rl = ro + d.n_expert;
+          uint32_t *rc = (uint32_t *)route->ptr, *ro = rc + d.n_expert, *rl = ro + d.n_expert, *rt = rl + (size_t)S * d.n_slot;
           {
             KernelScope ks(be, "experts_route", (double)S * d.n_slot * 8, 0);
-            e = launch_moe_route(be->lc(), d, rc, ro, rl);
+            e = launch_moe_route(be->lc(), d, rc, ro, rl, rt);
           }
+          f.route_tiles = d.route_tiles = rt;
           f.route_count = d.route_count = rc;
           f.route_offset = d.route_offset = ro;
           f.route_list = d.route_list = rl;

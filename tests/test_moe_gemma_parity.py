@@ -357,19 +357,25 @@ def test_expert_slots_of_a_decode_step(request, oracle, dev_name, S, k):
 
 
 @pytest.mark.gpu
-def test_expert_slots_sorted_by_expert(oracle, hip_bf16):
+@pytest.mark.parametrize("routing", ["skewed", "two experts take every token"])
+def test_expert_slots_sorted_by_expert(oracle, hip_bf16, routing):
     """The same block where both products have k a multiple of 64: the (slot, token) pairs are sorted by
-    expert once and both launches stream their operands through LDS stages.  A skewed routing: one
-    expert takes most pairs (several 128-row passes over its matrices, the last one partly filled), one
-    takes none, the others a few rows.  An index past the last expert is reported from there as well."""
+    expert once, cut into row tiles of 128 pairs - the launches' work list, so a crowded expert is spread over
+    the device - and both launches stream their operands through LDS stages.  A skewed routing: one
+    expert takes most pairs (several row tiles, the last one partly filled), one takes none, the others a few
+    rows; or two experts share all pairs, five full row tiles each, and seven experts have none.  An index past
+    the last expert is reported from there as well."""
     import vectors
     lang, nn = vectors.lang, vectors.nn
-    S, E, F, H, k = 600, 9, 192, 256, 2
+    S, E, F, H, k = (600 if routing == "skewed" else 640), 9, 192, 256, 2
     g = np.random.default_rng(8)
     x = g.standard_normal((S, 1, H)).astype(np.float32)
     wg, wu = (U_round((g.standard_normal((E, F, H)) * 0.1).astype(np.float32)) for _ in range(2))
     wd = U_round((g.standard_normal((E, H, F)) * 0.1).astype(np.float32))
-    idx = g.choice(np.array([0, 1, 2, 3, 4, 6, 7, 8]), size=(S, k), p=[.04, .04, .7, .04, .04, .04, .05, .05]).astype(np.uint32)
+    if routing == "skewed":
+        idx = g.choice(np.array([0, 1, 2, 3, 4, 6, 7, 8]), size=(S, k), p=[.04, .04, .7, .04, .04, .04, .05, .05]).astype(np.uint32)
+    else:
+        idx = np.tile(np.array([2, 7], np.uint32), (S, 1))
     assert (idx == 2).sum() > 3 * 128 and not (idx == 5).any()
     val = g.random((S, k)).astype(np.float32)
 
