@@ -26,7 +26,9 @@ int try_attn_prefill(cg_backend *be, cg_tensor *n, bool *done) {
     return CG_OK;
   // Below this the three-launch path (GEMM, softmax, GEMM) is as fast and the scores are small;
   // above it the scores of one layer run to hundreds of MB.  CG_FLAG_ATTN_ONE_PASS lifts the threshold.
-  if (T < 512 && !(be->flags & CG_FLAG_ATTN_ONE_PASS)) return CG_OK;
+  // (bf16 mode from 256 keys on: 4 x 16 heads x 256 x 256, d = 128 - two batched GEMMs, a softmax, the copy
+  // of the transposed result and two casts, 44 us - take 21 us in one pass)
+  if (T < (f32 ? 512 : 256) && !(be->flags & CG_FLAG_ATTN_ONE_PASS)) return CG_OK;
   if (nb > 65535 || heads > 65535) return CG_OK;
   cg_tensor *q = S->in[0];
   // queries and keys both still to be rotated: one launch for the two (each alone otherwise, below)

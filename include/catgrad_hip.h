@@ -76,7 +76,7 @@ enum {
    * RoPE, gated activations): everything goes through the generic fused-program kernels */
   CG_FLAG_NO_PATTERNS = 4u,
   /* use the one-pass attention kernels over many query rows for every sequence length (by default
-   * only from 512 keys on, where the score tensor they avoid is large); bf16 or f32 products, as
+   * only from 512 keys on - 256 with CG_FLAG_BF16 -, where the score tensor they avoid is large); bf16 or f32 products, as
    * CG_FLAG_BF16 says */
   CG_FLAG_ATTN_ONE_PASS = 8u
 };

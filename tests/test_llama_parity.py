@@ -130,9 +130,10 @@ def test_llama_prefill_of_many_rows(oracle, hip, hip_bf16):
     hip_bf16.trace(False)
     parity.assert_bf16(rl, gl, "prefill of 256 rows")
     launches = {k: v["launches"] for k, v in rep.items()}
-    # per layer: q/k/v grouped, o_proj, gate_proj with up_proj (and the activation), down_proj, and the two
-    # products of an attention this short (the one-pass kernel starts at 512 keys) = 6 GEMMs
-    assert launches.get("gemm_mfma_bf16") == 6 * cfg.num_hidden_layers, launches
+    # per layer: q/k/v grouped, o_proj, gate_proj with up_proj (and the activation), down_proj = 4 GEMMs, and
+    # the attention in one pass (in bf16 mode from 256 keys on)
+    assert launches.get("gemm_mfma_bf16") == 4 * cfg.num_hidden_layers, launches
+    assert launches.get("attn_prefill") == cfg.num_hidden_layers, launches
     assert "swiglu_fused" not in launches, launches
 
 
