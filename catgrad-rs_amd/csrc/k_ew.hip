@@ -508,6 +508,12 @@ __global__ void __launch_bounds__(256) reduce_plain_kernel(const T *x, int64_t r
   const uint32_t row = WPR == 4 ? blockIdx.x : blockIdx.x * 4 + wave;
   const uint32_t t_in_row = WPR == 4 ? threadIdx.x : lane, tpr = WPR * 64;
   Acc<KIND> acc;
+  // argmax over floats, the order of f32::total_cmp with the last of equal values winning (the Acc above), as one
+  // 64-bit maximum: ordered bits of the value << 32 | column.  A thread meets its columns in increasing order,
+  // so inside a thread "not smaller" replaces; 0 stands for "nothing seen" and loses to every element but
+  // (smallest value, column 0), which is the same answer.  A third of the instructions of the three-word form,
+  // which kept bf16 rows (half the bytes) from streaming at memory speed.
+  uint32_t best_u = 0, best_c = 0;
   if (row < rows) {
     const T *r = x + (int64_t)row * row_stride;
     for (uint32_t c0 = t_in_row * 4; c0 < n; c0 += tpr * 4 * U) {
@@ -530,10 +536,44 @@ __global__ void __launch_bounds__(256) reduce_plain_kernel(const T *x, int64_t r
         const uint32_t c = c0 + u * tpr * 4;
         if (c < n) {
 #pragma unroll
-          for (int j = 0; j < 4; ++j) acc.add(v[u][j], c + j);
+          for (int j = 0; j < 4; ++j) {
+            if constexpr (KIND == R_ARGMAX_F) {
+              const uint32_t b = v[u][j], o = b ^ ((uint32_t)((int32_t)b >> 31) | 0x80000000u);  // total_cmp order, unsigned
+              const bool take = o >= best_u;
+              best_u = take ? o : best_u;
+              best_c = take ? c + j : best_c;
+            } else {
+              acc.add(v[u][j], c + j);
+            }
+          }
         }
       }
     }
+  }
+  if constexpr (KIND == R_ARGMAX_F) {
+    uint64_t best = (uint64_t)best_u << 32 | best_c;
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) {
+      const uint64_t o = (uint64_t)(uint32_t)__shfl_xor((int)(best >> 32), m, 64) << 32 | (uint32_t)__shfl_xor((int)(uint32_t)best, m, 64);
+      best = o > best ? o : best;
+    }
+    if (WPR == 4) {
+      if (lane == 0) {
+        part[wave][0] = (uint32_t)(best >> 32);
+        part[wave][1] = (uint32_t)best;
+      }
+      __syncthreads();
+      if (threadIdx.x == 0) {
+        for (int w2 = 1; w2 < 4; ++w2) {
+          const uint64_t o = (uint64_t)part[w2][0] << 32 | part[w2][1];
+          best = o > best ? o : best;
+        }
+        out[row] = (uint32_t)best;
+      }
+    } else if (lane == 0 && row < rows) {
+      out[row] = (uint32_t)best;
+    }
+    return;
   }
 #pragma unroll
   for (int m = 32; m >= 1; m >>= 1) acc.merge(shfl_xor_acc<KIND>(acc, m));
