@@ -138,6 +138,31 @@ def test_llama_prefill_of_many_rows(oracle, hip, hip_bf16):
 
 
 @pytest.mark.gpu
+def test_llama_prefill_block_ends_at_full_width(oracle, hip, hip_bf16):
+    """Two layers at the 1B model's widths (hidden 2048, FFN 8192, 32 / 8 heads of 64) over a 128-token prompt:
+    o_proj and down_proj are split along k here, every `residual + linear(x)` is issued as soon as it is recorded
+    and left as the slices of its product, and the RMSNorm that reads it sums them.  Logits against the oracle at
+    the stated bars in both modes, and the bf16 trace shows the norms taking the slices."""
+    cfg = U.tiny_config(hidden_size=2048, intermediate_size=8192, num_hidden_layers=2, num_attention_heads=32,
+                        num_key_value_heads=8, vocab_size=512)
+    arrays = U.param_arrays(cfg, seed=3, std=0.02)
+    rounded = {k: (vectors.bf16_round(a) if a.ndim >= 2 else a) for k, a in arrays.items()}
+    prompt = list(np.random.default_rng(4).integers(0, cfg.vocab_size, 128))
+    for be, params, check in ((hip, arrays, parity.assert_f32), (hip_bf16, rounded, parity.assert_bf16)):
+        _, rl = U.CachedRunner(oracle, cfg, params, 160).prefill(prompt)
+        g = U.CachedRunner(be, cfg, arrays, 160)
+        be.trace(2)
+        be.trace_reset()
+        _, gl = g.prefill(prompt)
+        gl = be.to_vec(gl)
+        names = set(be.trace_report())
+        be.trace(False)
+        check(oracle.to_vec(rl), gl, "prefill of 128 rows at full width")
+        if be is hip_bf16:
+            assert any(n.startswith("rmsnorm_fused[") and "k-slices" in n for n in names), sorted(names)
+
+
+@pytest.mark.gpu
 def test_pipelined_decode_gives_the_same_tokens(hip, hip_bf16):
     """Token fed back on the device and read one step behind (cg_tensor_prefetch) == the loop that
     reads every token before the next step; also that a prefetched read returns the right data."""
