@@ -357,7 +357,7 @@ def test_expert_slots_of_a_decode_step(request, oracle, dev_name, S, k):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("routing", ["skewed", "two experts take every token"])
+@pytest.mark.parametrize("routing", ["skewed", "two experts take every token", "1500 experts"])
 def test_expert_slots_sorted_by_expert(oracle, hip_bf16, routing):
     """The same block where both products have k a multiple of 64: the (slot, token) pairs are sorted by
     expert once, cut into row tiles of 128 pairs - the launches' work list, so a crowded expert is spread over
@@ -368,15 +368,21 @@ def test_expert_slots_sorted_by_expert(oracle, hip_bf16, routing):
     import vectors
     lang, nn = vectors.lang, vectors.nn
     S, E, F, H, k = (600 if routing == "skewed" else 640), 9, 192, 256, 2
+    if routing == "1500 experts":      # more experts than the routing kernel has threads: two to a thread
+        S, E, F, H = 300, 1500, 64, 64
     g = np.random.default_rng(8)
     x = g.standard_normal((S, 1, H)).astype(np.float32)
     wg, wu = (U_round((g.standard_normal((E, F, H)) * 0.1).astype(np.float32)) for _ in range(2))
     wd = U_round((g.standard_normal((E, H, F)) * 0.1).astype(np.float32))
     if routing == "skewed":
         idx = g.choice(np.array([0, 1, 2, 3, 4, 6, 7, 8]), size=(S, k), p=[.04, .04, .7, .04, .04, .04, .05, .05]).astype(np.uint32)
+    elif routing == "1500 experts":
+        idx = g.integers(0, E, (S, k)).astype(np.uint32)
+        idx[:200, 0] = 1499             # a crowded expert at the very end: two row tiles
+        idx[idx == 5] = 6
     else:
         idx = np.tile(np.array([2, 7], np.uint32), (S, 1))
-    assert (idx == 2).sum() > 3 * 128 and not (idx == 5).any()
+    assert ((idx == 2).sum() > 3 * 128 or routing == "1500 experts") and not (idx == 5).any()
     val = g.random((S, k)).astype(np.float32)
 
     def f(b, xv, iv, vv, g_all, u_all, d_all):
