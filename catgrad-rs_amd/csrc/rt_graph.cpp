@@ -399,7 +399,11 @@ int binary(cg_backend *be, cg_tensor *a, cg_tensor *b, cg_tensor **out, EwOp f_o
       const cg_tensor *src = other;
       while (src->op == N_RESHAPE && src->in[0]) src = src->in[0];
       const bool in_memory = other->op == N_REAL || other->op == N_KSUM;
-      if (mm->op != N_MATMUL || !(in_memory || src->op == N_INDEX)) continue;
+      // (or a sum with other readers besides this add - the norm before the product reads it twice: the residual
+      // stream where the previous block ended in something else than a product, a MoE block's weighted sum; a
+      // value with several readers is computed on its own whatever follows)
+      const bool stream_sum = other->op == N_BIN && other->ew == E_ADD_F && other->rc.load() >= 3;
+      if (mm->op != N_MATMUL || !(in_memory || src->op == N_INDEX || stream_sum)) continue;
       bool dense = true;
       for (int i = 0; in_memory && i < other->rank; ++i) dense = dense && (other->shape[i] == 1 || other->strides[i] != 0);
       // a few-row product with siblings on the same rows (q/k/v, each about to get its bias) is the
