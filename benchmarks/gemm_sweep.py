@@ -43,10 +43,17 @@ def run(lib, shapes=SHAPES, iters=10):
         out.append({"shape": f"{b}x{m}x{n}x{k}", "us": ms * 1e3, "tflops": tf, "frac": tf / MFMA_PEAK_BF16_TFLOPS,
                     "kernels": {name: v["launches"] // iters for name, v in rep.items()}})
         del x, w, wt
+    be.close()
     return out
 
 
 if __name__ == "__main__":
-    for r in run(cg.load_library()):
+    import argparse
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--shapes", default=None, help="comma-separated BxMxNxK list (default: the whole sweep)")
+    ap.add_argument("--iters", type=int, default=10)
+    a = ap.parse_args()
+    shapes = SHAPES if not a.shapes else [tuple(int(v) for v in s.split("x")) for s in a.shapes.split(",")]
+    for r in run(cg.load_library(), shapes, a.iters):
         print(f"{r['shape']:>22s} {r['us']:9.1f} us {r['tflops']:8.1f} TFLOP/s  {100 * r['frac']:5.1f} % of 2.5 PFLOP/s  {r['kernels']}",
               flush=True)

@@ -106,11 +106,25 @@ def run_qwen_moe(lib, layers=24, batch=4, prompt=256, steps=64, warmup=2):
     launches = (be.stats()["launches"] - launches0) / steps
     toks = np.stack(toks)
     assert toks.max() < cfg.vocab_size
+    # the experts a step really reads: a few more steps through a term that also returns its routing
+    routed_term = qwen_moe.QwenMoeDecodeRouted(cfg).term()
+    n_kv = 2 * cfg.num_hidden_layers
+    distinct = []
+    for _ in range(4):
+        out = r.it.run(routed_term, [be.reshape(tok, [batch, 1]), r.pos, r.cos, r.sin] + r.kv,
+                       moved=range(4, 4 + n_kv))
+        tok, r.kv, routing = out[0], out[2:2 + n_kv], out[2 + n_kv:]
+        r.pos += 1
+        distinct.append([len(np.unique(be.to_vec(ix))) for ix in routing])
+    distinct_per_layer = float(np.mean(distinct))
     # bytes a decode step has to read: attention + shared expert + router + distinct routed experts
     h, f, sf, e = cfg.hidden_size, cfg.moe_intermediate_size, cfg.shared_expert_intermediate_size, cfg.num_experts
+    del r, P, out, routing, tok, nxt, lg, lg1, tok1
+    be.close()
     per_layer_fixed = (4 * h * h + 3 * sf * h + e * h) * 2
     expert_bytes = 3 * f * h * 2
     upper = layers * (per_layer_fixed + min(batch * cfg.num_experts_per_tok, e) * expert_bytes) + cfg.vocab_size * h * 2
+    actual = layers * (per_layer_fixed + distinct_per_layer * expert_bytes) + cfg.vocab_size * h * 2
     return {"workload": "BASELINE configs[3]: Qwen1.5-MoE-A2.7B layout, random init N(0,0.02) (large matrices drawn "
                         f"from a pool of two per shape), bf16 weights, {layers} layers, batch {batch} x {prompt}-token "
                         f"prompts, {steps} greedy steps with KV cache",
@@ -119,6 +133,9 @@ def run_qwen_moe(lib, layers=24, batch=4, prompt=256, steps=64, warmup=2):
             "prefill_tokens_per_s": batch * prompt / prefill_s, "kernel_launches_per_step": launches,
             "decode_weight_bytes_per_step_upper_bound": upper,
             "decode_hbm_fraction_at_upper_bound": upper * (steps / decode_s) / 8e12,
+            "distinct_experts_per_layer_and_step": distinct_per_layer,
+            "decode_weight_bytes_per_step": actual,
+            "decode_hbm_fraction": actual * (steps / decode_s) / 8e12,
             "row_independence_rel_err": rel, "setup_s": setup_s}
 
 
@@ -187,6 +204,8 @@ def run_gemma3(lib, layers=26, batch=8, prompt=2048, iters=3):
     flops = sum(v["flops"] for v in rep.values())
     share = {k: round(v["ms"] / total, 4) for k, v in sorted(rep.items(), key=lambda kv: -kv[1]["ms"])[:8]}
     gm = rep.get("gemm_mfma_bf16")
+    del it, P, tok, lg, lg1, dev_ids
+    be.close()
     return {"workload": f"BASELINE configs[4]: Gemma-3-1B shape, random init N(0,0.02), bf16 weights, {layers} layers, "
                         f"batch {batch} x {prompt}-token prompts, prefill only, logits of the last position, 5 local "
                         "(window 512) : 1 global layers",

@@ -203,11 +203,16 @@ class Backend:
         self.ptr = p
         self.flags = flags
 
-    def __del__(self):
-        # tensors may outlive the Python object; the library keeps the backend alive for them
+    def close(self):
+        """Give the backend up now (its launch thread is joined, its stream and pool released once the
+        last tensor of it is gone) instead of whenever the garbage collector finds the object."""
         if getattr(self, "ptr", None):
             self.lib.cg_backend_destroy(self.ptr)
             self.ptr = None
+
+    def __del__(self):
+        # tensors may outlive the Python object; the library keeps the backend alive for them
+        self.close()
 
     @property
     def name(self):

@@ -403,7 +403,17 @@ int try_gemv_prologue(cg_backend *be, cg_tensor *n, cg_tensor *addend, bool *add
 int try_gemv_attn_merge(cg_backend *be, cg_tensor *n, cg_tensor *addend, bool *added, bool *done) {
   if (!n->gemv_candidate) return CG_OK;
   cg_tensor *att = n->in[0];
-  while ((att->op == N_RESHAPE || att->op == N_TRANSPOSE) && refs(att) == 1) att = att->in[0];
+  // The merge prologue reads the partials in the attention's own (head, d) order, so every view on the
+  // way must keep the row-major element order: a reshape always does; a transpose does when at most one
+  // axis in the swapped range has an extent other than 1 (it then only moves unit axes).
+  auto keeps_order = [](const cg_tensor *t) {
+    if (t->op == N_RESHAPE) return true;
+    const int64_t lo = std::min(t->p0, t->p1), hi = std::max(t->p0, t->p1);
+    int wide = 0;
+    for (int64_t i = lo; i <= hi; ++i) wide += t->shape[i] != 1;
+    return wide <= 1;
+  };
+  while ((att->op == N_RESHAPE || att->op == N_TRANSPOSE) && refs(att) == 1 && keeps_order(att)) att = att->in[0];
   if (att == n->in[0] || att->op != N_MATMUL || att->dtype != CG_F32 || att->rank != 4 || refs(att) != 1) return CG_OK;
   if (att->shape[0] != 1 || att->shape[2] != 1) return CG_OK;
   const int64_t K = att->shape[1] * att->shape[3];

@@ -60,6 +60,8 @@ class QwenMoeParts:
         sh = make_shape(builder, seq_len, c.num_experts_per_tok)
         indices = reshape(builder, sh, indices)
         values = reshape(builder, sh, values)
+        if getattr(self, "routing_out", None) is not None:   # (a term that also returns its routing, below)
+            self.routing_out.append(indices)
         if c.norm_topk_prob:
             sv = broadcast(builder, sum(builder, values), sh)
             values = values / sv
@@ -184,3 +186,18 @@ class QwenMoePrefill(_QwenMoeCachedParts, _llama.LlamaPrefill):
 
 class QwenMoeDecode(_QwenMoeCachedParts, _llama.LlamaDecode):
     """ids[B,1], pos: Nat, cos, sin, k0, v0, ... -> token, logits, k0', v0', ..."""
+
+
+class QwenMoeDecodeRouted(QwenMoeDecode):
+    """QwenMoeDecode that also returns every layer's expert indices [B, k] after the caches (for counting
+    the distinct experts a step reads; not the term the benchmarks time)."""
+
+    def sort(self):
+        i, o = super().sort()
+        return i, o + [TENSOR] * self.config.num_hidden_layers
+
+    def def_(self, builder, args):
+        self.routing_out = []
+        out = super().def_(builder, args)
+        routing, self.routing_out = self.routing_out, None
+        return out + routing

@@ -66,27 +66,33 @@ class CachedRunner:
         self.pos += 1
         return out[0], out[1]
 
+    def _host_tokens(self, tok):
+        """The sampled token of every batch row: an int for one row, a list of ints for several."""
+        t = self.be.to_vec(tok).reshape(-1)
+        return int(t[0]) if self.batch == 1 else [int(v) for v in t]
+
     def generate_pipelined(self, prompt, steps):
         """Greedy tokens with the sampled token fed back on the device and read one step behind:
-        the host records and issues step t+1 while the device still runs step t."""
+        the host records and issues step t+1 while the device still runs step t.  Per step an int, or -
+        prompts of shape [B, S] - the list of the B rows' tokens."""
         tok, _ = self.prefill(prompt)
         self.be.prefetch(tok)
         toks, prev = [], tok
         for _ in range(steps - 1):
             tok, _ = self.step(prev)
             self.be.prefetch(tok)
-            toks.append(int(self.be.to_vec(prev)[0]))
+            toks.append(self._host_tokens(prev))
             prev = tok
-        toks.append(int(self.be.to_vec(prev)[0]))
+        toks.append(self._host_tokens(prev))
         return toks
 
     def generate(self, prompt, steps):
         """Returns (tokens, logits per step as numpy), reading every token before the next step like
-        the reference's loop."""
+        the reference's loop.  Per step an int, or - prompts of shape [B, S] - the list of the B rows' tokens."""
         tok, logits = self.prefill(prompt)
         toks, lg = [], []
         for _ in range(steps):
-            t = int(self.be.to_vec(tok)[0])
+            t = self._host_tokens(tok)
             toks.append(t)
             lg.append(self.be.to_vec(logits))
             tok, logits = self.step(t)

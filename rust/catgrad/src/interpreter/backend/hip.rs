@@ -13,14 +13,51 @@ use catgrad_hip_sys as sys;
 use std::ffi::CStr;
 use std::fmt;
 use std::ptr;
-use std::sync::Arc;
+use std::sync::{Arc, Mutex};
+use std::thread::{self, ThreadId};
 
-struct Handle(*mut sys::cg_backend);
+// The library is single-threaded per backend: recording a graph, releasing a tensor and every other
+// call edit unlocked per-backend state.  The trait's bounds still make the handles `Send + Sync`, so
+// the rule is enforced here instead of being left to the caller: a backend is used on the thread that
+// made it (`raw` panics elsewhere), a tensor dropped on another thread is parked in `GRAVEYARD` and
+// released by its owner's next call, and the only thing other threads really do - `clone` and
+// `shape` - is an atomic increment and a read of fields that never change.
+struct Handle {
+    be: *mut sys::cg_backend,
+    owner: ThreadId,
+}
 unsafe impl Send for Handle {}
 unsafe impl Sync for Handle {}
 impl Drop for Handle {
     fn drop(&mut self) {
-        unsafe { sys::cg_backend_destroy(self.0) }
+        // (the library keeps the backend alive until its last tensor is released)
+        unsafe { sys::cg_backend_destroy(self.be) }
+    }
+}
+
+/// tensors dropped away from their owner thread: (owner, pointer)
+static GRAVEYARD: Mutex<Vec<(ThreadId, usize)>> = Mutex::new(Vec::new());
+
+fn bury_or_release(owner: ThreadId, t: *mut sys::cg_tensor) {
+    if thread::current().id() == owner {
+        unsafe { sys::cg_tensor_release(t) }
+    } else {
+        GRAVEYARD.lock().unwrap().push((owner, t as usize));
+    }
+}
+
+fn release_buried(owner: ThreadId) {
+    let mine: Vec<usize> = {
+        let mut g = GRAVEYARD.lock().unwrap();
+        if g.is_empty() {
+            return;
+        }
+        let (mine, rest): (Vec<_>, Vec<_>) = g.drain(..).partition(|(o, _)| *o == owner);
+        *g = rest;
+        mine.into_iter().map(|(_, p)| p).collect()
+    };
+    for p in mine {
+        unsafe { sys::cg_tensor_release(p as *mut sys::cg_tensor) }
     }
 }
 
@@ -35,18 +72,19 @@ impl fmt::Debug for HipBackend {
     }
 }
 
-/// `BackendTensor`: an owned reference.  `Clone` = retain (O(1)), `Drop` = release.
-pub struct HipTensor(*mut sys::cg_tensor);
+/// `BackendTensor`: an owned reference.  `Clone` = retain (O(1), an atomic increment), `Drop` =
+/// release on the owner thread (parked for it otherwise).
+pub struct HipTensor(*mut sys::cg_tensor, ThreadId);
 unsafe impl Send for HipTensor {}
 unsafe impl Sync for HipTensor {}
 impl Clone for HipTensor {
     fn clone(&self) -> Self {
-        HipTensor(unsafe { sys::cg_tensor_retain(self.0) })
+        HipTensor(unsafe { sys::cg_tensor_retain(self.0) }, self.1)
     }
 }
 impl Drop for HipTensor {
     fn drop(&mut self) {
-        unsafe { sys::cg_tensor_release(self.0) }
+        bury_or_release(self.1, self.0)
     }
 }
 impl fmt::Debug for HipTensor {
@@ -82,11 +120,14 @@ impl HipBackend {
         let flags = if bf16 { sys::CG_FLAG_BF16 } else { 0 };
         let st = unsafe { sys::cg_backend_create(device, flags, &mut be) };
         assert_eq!(st, sys::CG_OK, "cg_backend_create: no usable gfx950 device");
-        HipBackend(Arc::new(Handle(be)))
+        HipBackend(Arc::new(Handle { be, owner: thread::current().id() }))
     }
 
+    /// the backend pointer for a call into the library: only on the thread that made the backend
     fn raw(&self) -> *mut sys::cg_backend {
-        (self.0).0
+        assert_eq!(thread::current().id(), self.0.owner, "HipBackend is used on the thread that created it");
+        release_buried(self.0.owner);
+        self.0.be
     }
 
     /// the reference panics where the C ABI returns a status
@@ -107,9 +148,9 @@ impl HipBackend {
 
     fn tag(f32_tag: bool, out: *mut sys::cg_tensor) -> TaggedTensor<Self> {
         if f32_tag {
-            TaggedTensorTuple::F32([HipTensor(out)])
+            TaggedTensorTuple::F32([HipTensor(out, thread::current().id())])
         } else {
-            TaggedTensorTuple::U32([HipTensor(out)])
+            TaggedTensorTuple::U32([HipTensor(out, thread::current().id())])
         }
     }
 

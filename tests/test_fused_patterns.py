@@ -464,6 +464,39 @@ def test_attention_decode_merged_by_the_output_projection(oracle, hip, hip_bf16,
     assert np.max(np.abs(got - ref)) <= tol * np.abs(ref).max(), np.max(np.abs(got - ref)) / np.abs(ref).max()
 
 
+def test_attention_decode_merge_needs_the_head_order(oracle, hip, cg):
+    """The same chain with a head merge that reorders: `transpose(1, 3)` of [1, H, 1, d] puts d before the
+    heads, so the row o_proj reads is (d, head)-ordered.  The projection's merging prologue reads partials in
+    (head, d) order and must not take this graph; the result is the oracle's either way."""
+    H, KV, d, N, T = 32, 8, 64, 384, 300
+    g = np.random.default_rng(77)
+    q = g.standard_normal((1, H, 1, d)).astype(np.float32)
+    k = g.standard_normal((1, KV, T, d)).astype(np.float32)
+    v = g.standard_normal((1, KV, T, d)).astype(np.float32)
+    res = g.standard_normal((1, 1, N)).astype(np.float32)
+    p = {"o.weight": (g.standard_normal((N, H * d)) * 0.05).astype(np.float32)}
+
+    def f(b, qv, kv, vv, rv):
+        qv, kv, vv, rv = qv + qv - qv, kv + kv - kv, vv + vv - vv, rv + rv - rv
+        kr = helpers.repeat_kv(b, H // KV, kv)
+        vr = helpers.repeat_kv(b, H // KV, vv)
+        attn = lang.matmul(b, qv, lang.transpose(b, 2, 3, kr))
+        sh = lang.shape(b, attn)
+        attn = attn / lang.constant(b, float(np.sqrt(np.float32(d))), sh)
+        attn = attn + lang.broadcast(b, helpers.causal_mask(b, lang.to_nat(b, 1)), sh)
+        out = lang.matmul(b, nn.softmax(b, attn), vr)
+        out = lang.reshape(b, lang.make_shape(b, 1, 1, H * d), lang.transpose(b, 1, 3, out))   # [1, d, 1, H]
+        return rv + nn.linear_no_bias(b, H * d, N, lang.path(["o"]), out)
+    (ref,) = vectors.run(oracle, f, 1, q, k, v, res, params=p)
+    hip.trace(2)
+    hip.trace_reset()
+    (got,) = vectors.run(hip, f, 1, q, k, v, res, params=p)
+    names = set(hip.trace_report())
+    hip.trace(False)
+    assert not any("attn-merge" in nm for nm in names), sorted(names)
+    assert np.max(np.abs(got - ref)) <= 1e-4 * np.abs(ref).max(), np.max(np.abs(got - ref)) / np.abs(ref).max()
+
+
 def test_attention_decode_that_cannot_be_fused_still_appends_its_rows(oracle, hip_bf16, cg):
     """A decode step whose caches qualify for the append inside the attention kernel, but whose query
     does not (an uploaded rank-4 tensor is bf16 storage in bf16 mode): the new key and value rows must
@@ -1043,7 +1076,8 @@ def test_attention_prefill_with_an_arbitrary_shared_mask(oracle, hip_bf16_flash,
 
 
 @pytest.mark.parametrize("cfg", [(1, 32, 8, 512, 64), (2, 4, 2, 100, 128), (2, 4, 2, 104, 128), (1, 4, 1, 200, 256),
-                                 (1, 8, 8, 33, 64), (1, 2, 1, 1024, 64)])
+                                 (1, 8, 8, 33, 64), (1, 2, 1, 1024, 64),
+                                 (1, 4, 1, 2048, 256)])  # the last: Gemma-3's heads at its prompt length, window 512
 @pytest.mark.parametrize("mask_kind", ["causal", "window"])
 def test_attention_prefill_bf16(oracle, hip_bf16_flash, hip_bf16, hip_nopat, cfg, mask_kind):
     """Attention over many query rows in bf16 mode: one launch with online softmax, scores never
@@ -1065,7 +1099,7 @@ def test_attention_prefill_bf16(oracle, hip_bf16_flash, hip_bf16, hip_nopat, cfg
         sh = lang.shape(b, attn)
         attn = attn / lang.constant(b, float(np.sqrt(np.float32(d))), sh)
         n = lang.to_nat(b, S)
-        mask = helpers.causal_mask(b, n) if mask_kind == "causal" else model.window_mask(b, n, 17)
+        mask = helpers.causal_mask(b, n) if mask_kind == "causal" else model.window_mask(b, n, 512 if S >= 2048 else 17)
         attn = attn + lang.broadcast(b, mask, sh)
         return lang.matmul(b, nn.softmax(b, attn), vr)
     (ref,) = vectors.run(oracle, f, 1, q, k, v)
@@ -1083,7 +1117,8 @@ def test_attention_prefill_bf16(oracle, hip_bf16_flash, hip_bf16, hip_nopat, cfg
 
 
 @pytest.mark.parametrize("cfg", [(1, 32, 8, 512, 64), (2, 4, 2, 100, 128), (2, 4, 2, 104, 128), (1, 4, 1, 200, 256),
-                                 (1, 8, 8, 40, 64), (1, 2, 1, 1024, 64), (1, 8, 2, 320, 128), (2, 2, 2, 72, 256)])
+                                 (1, 8, 8, 40, 64), (1, 2, 1, 1024, 64), (1, 8, 2, 320, 128), (2, 2, 2, 72, 256),
+                                 (1, 4, 1, 2048, 256)])  # the last: Gemma-3's heads at its prompt length, window 512
 @pytest.mark.parametrize("mask_kind", ["causal", "window", "none"])
 def test_attention_prefill_f32(oracle, hip_f32_flash, hip, cfg, mask_kind):
     """Attention over many query rows without the bf16 flag: the same single launch with every product
@@ -1106,7 +1141,7 @@ def test_attention_prefill_f32(oracle, hip_f32_flash, hip, cfg, mask_kind):
         attn = attn / lang.constant(b, float(np.sqrt(np.float32(d))), sh)
         if mask_kind != "none":
             n = lang.to_nat(b, S)
-            mask = helpers.causal_mask(b, n) if mask_kind == "causal" else model.window_mask(b, n, 17)
+            mask = helpers.causal_mask(b, n) if mask_kind == "causal" else model.window_mask(b, n, 512 if S >= 2048 else 17)
             attn = attn + lang.broadcast(b, mask, sh)
         return lang.matmul(b, nn.softmax(b, attn), vr)
     (ref,) = vectors.run(oracle, f, 1, q, k, v)

@@ -25,6 +25,10 @@ def test_reference_nn_vectors(dev):
     vectors.check_nn_vectors(dev)
 
 
+def test_reference_legacy_shape_vectors(dev):
+    vectors.check_legacy_shape_vectors(dev)
+
+
 @pytest.mark.parametrize("name", ["sigmoid", "exp", "sqrt", "tanh", "gelu", "silu", "softmax"])
 def test_stdlib_definitions_vs_oracle(oracle, dev, cg, name):
     mod = {m.name: m for m in vectors.nn.stdlib_definitions()}[name]

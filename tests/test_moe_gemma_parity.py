@@ -478,6 +478,22 @@ def test_moe_cached_equals_full_recompute_on_oracle(oracle):
         seqs = np.concatenate([seqs, toks[i][:, None]], axis=1)
 
 
+def test_runner_generate_feeds_back_every_batch_row(oracle):
+    """CachedRunner.generate / generate_pipelined with prompts [2, S]: every row's token is returned and fed
+    back (the loops above are the check: they pass all rows by hand)."""
+    cfg = MU.qwen_moe_config()
+    P = MU.qwen_moe_params(cfg, seed=11, std=0.15)
+    prompts = np.random.default_rng(12).integers(0, cfg.vocab_size, (2, 6))
+    toks, _ = moe_cached_generate(oracle, cfg, P, prompts, 4)
+
+    def runner():
+        return U.CachedRunner(oracle, cfg, P, 16, prefill_cls=llm.qwen_moe.QwenMoePrefill,
+                              decode_cls=llm.qwen_moe.QwenMoeDecode)
+    got, _ = runner().generate(prompts, 4)
+    assert got == [[int(v) for v in row] for row in toks]
+    assert runner().generate_pipelined(prompts, 4) == got
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("mode", ["f32", "bf16"])
 def test_moe_cached_decode_hip_vs_oracle(oracle, hip, hip_bf16, mode):

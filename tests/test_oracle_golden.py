@@ -18,6 +18,10 @@ def test_reference_nn_vectors(oracle):
     vectors.check_nn_vectors(oracle)
 
 
+def test_reference_legacy_shape_vectors(oracle):
+    vectors.check_legacy_shape_vectors(oracle)
+
+
 def bf(x):
     return np.asarray(x, np.float32)
 

@@ -169,6 +169,71 @@ def check_nn_vectors(be):
     assert np.array_equal(m.ravel(), f32(g["pattern"]) * fmin)       # 0 * MIN = -0.0 == 0
 
 
+def _points(a, pts, what):
+    for idx, v in pts:
+        assert a[tuple(idx)] == v, (what, idx, float(a[tuple(idx)]), v)
+
+
+def check_legacy_shape_vectors(be):
+    """The shape-op vectors of catgrad-llm/src/legacy/nn/layers.rs (repeat_kv, index, narrow, concat,
+    transpose + reshape, expand, arange, cast, batched linear), on the Backend methods they map to; the
+    reference asserts single elements (`get(&[..])`), so single elements are what is compared."""
+    def arange_f32(n):
+        return be.cast(be.arange(n), cg.abi.F32)
+    g = GOLDEN["legacy_repeat_kv"]
+    x = np.arange(g["x_arange"], dtype=np.float32).reshape(g["x_shape"])
+    (y,) = run(be, lambda b, v: helpers.repeat_kv(b, g["rep"], v), 1, x)
+    assert list(y.shape) == g["shape"]
+    _points(y, g["points"], "repeat_kv")
+    g = GOLDEN["legacy_index"]
+    x = be.broadcast(arange_f32(g["x_arange"]), g["x_expand"])
+    for c in g["cases"]:
+        y = be.numpy(be.index(x, c["dim"], be.tensor(u32(c["indices"]))))
+        assert list(y.shape) == c["shape"]
+        _points(y, c["points"], "index")
+    g = GOLDEN["legacy_narrow"]
+    x = be.reshape(arange_f32(g["x_arange"]), g["x_shape"])
+    for c in g["cases"]:
+        y = be.numpy(be.slice(x, c["dim"], c["start"], c["len"]))
+        assert list(y.shape) == c["shape"]
+        _points(y, c["points"], "narrow")
+    g = GOLDEN["legacy_concat"]
+    a, b_ = be.tensor(f32(g["x"]), g["shape"]), be.tensor(f32(g["y"]), g["shape"])
+    for dim in (0, 1):
+        y = be.numpy(be.concat(a, b_, dim))
+        assert list(y.shape) == g[f"dim{dim}_shape"] and np.array_equal(y.ravel(), f32(g[f"dim{dim}"]))
+    g = GOLDEN["legacy_transpose_reshape"]
+    b_ = be.reshape(arange_f32(g["x_arange"]), g["b_shape"])
+    assert np.array_equal(be.to_vec(b_), f32(g["b"]))
+    d = be.reshape(be.transpose(b_, 0, 1), g["d_shape"])   # a reshape of a transposed view reorders
+    m = be.numpy(be.matmul(d, b_))
+    assert list(m.shape) == g["m_shape"] and np.array_equal(m.ravel(), f32(g["m"]))
+    g = GOLDEN["legacy_expand"]
+    y = be.numpy(be.broadcast(arange_f32(g["x_arange"]), g["shape"]))
+    assert list(y.shape) == g["shape"]
+    _points(y, g["points"], "expand")
+    g = GOLDEN["legacy_arange_expand_reshape"]
+    e = be.broadcast(arange_f32(g["x_arange"]), g["expand"])
+    _points(be.numpy(e), g["e_points"], "arange/expand")
+    r = be.numpy(be.reshape(e, g["reshape"]))
+    assert list(r.shape) == g["reshape"]
+    _points(r, g["r_points"], "arange/reshape")
+    g = GOLDEN["legacy_cast"]
+    i = be.arange(g["n"])
+    assert np.array_equal(be.to_vec(be.cast(i, cg.abi.F32)), f32(g["int_to_f32"]))
+    assert np.array_equal(be.to_vec(be.cast(be.cast(i, cg.abi.F32), cg.abi.U32)), u32(g["f32_to_int"]))
+    g = GOLDEN["legacy_linear_batch"]
+    x = np.broadcast_to(f32(g["x"]).reshape(g["x_shape"]), [g["batch"]] + g["x_shape"]).copy()
+    params = {"l.weight": f32(g["w"]).reshape(g["w_shape"]), "l.bias": f32(g["b"])}
+
+    def batched_linear(b, v):  # the batch folded into the rows and back: the batch-correct reading of nn.linear
+        qm = importlib.import_module("catgrad-rs_amd.llm.qwen_moe")
+        f, bb, s = qm.fold_batch(b, v)
+        return qm.unfold_batch(b, bb, s, nn.linear(b, 3, 2, lang.path(["l"]), f))
+    (y,) = run(be, batched_linear, 1, x, params=params)
+    assert y.shape == (2, 2, 2) and np.array_equal(approx6(y.ravel()), f32(g["expected"]))
+
+
 def bf16_round(a):
     """f32 array rounded to the nearest bf16 (ties to even), as f32."""
     u = np.ascontiguousarray(a, np.float32).view(np.uint32).astype(np.uint64)
