@@ -70,7 +70,8 @@ def other_configs(lib, args):
         res["mlp_us"] = {"wall_us_per_run": mlp[0]["wall_us"], "kernel_us_per_run": mlp[0]["kernel_us"],
                          "launches": sum(mlp[0]["kernels"].values())}
     sweep = importlib.import_module("benchmarks.gemm_sweep")
-    res["gemm_bf16_sweep"] = {r["shape"]: {"achieved": r["tflops"], "unit": "TFLOP/s", "frac": r["frac"], "us": r["us"]}
+    res["gemm_bf16_sweep"] = {r["shape"]: {"achieved": r["tflops"], "unit": "TFLOP/s", "frac": r["frac"], "us": r["us"],
+                                           "clock_mhz": r.get("clock_mhz"), "frac_at_clock": r.get("frac_at_clock")}
                               for r in sweep.run(lib, iters=5)}
     q = mb.run_qwen_moe(lib, steps=16, warmup=2)
     res["qwen_moe"] = {"ms_per_step": q["ms_per_step"], "decode_tokens_per_s": q["decode_tokens_per_s"],
@@ -168,6 +169,16 @@ def measure_llama(cg, llm, lib, cfg, arrays, prompt, dtype, args, steps, warmup,
         out["measured_peaks"] = {"copy_gbs_read_plus_write": be.peak_copy_gbs(1 << 30, 10),
                                  "mfma_bf16_tflops": be.peak_mfma_tflops(cg.abi.U32, 20000),
                                  "mfma_f32_tflops": be.peak_mfma_tflops(cg.abi.F32, 20000)}
+        # the shader clock (read inside the kernels) under the bare MFMA loop and under the bf16 GEMM: the
+        # data-sheet 2.5 PFLOP/s is 2400 MHz; a GEMM is clocked lower by the power limit
+        loop_tf, loop_mhz = be.peak_gemm_clock(0, 0, 0, 2)
+        g4_tf, g4_mhz = be.peak_gemm_clock(4096, 4096, 4096, 5)
+        g8_tf, g8_mhz = be.peak_gemm_clock(8192, 8192, 8192, 3)
+        out["measured_peaks"]["shader_clock_mhz"] = {
+            "data_sheet": 2400, "mfma_loop": loop_mhz, "gemm_bf16_4096": g4_mhz, "gemm_bf16_8192": g8_mhz,
+            "gemm_bf16_4096_tflops": g4_tf, "gemm_bf16_8192_tflops": g8_tf,
+            "gemm_bf16_8192_frac_of_mfma_peak_at_its_clock": g8_tf / (MFMA_PEAK_TFLOPS["bf16"] * g8_mhz / 2400.0)
+            if g8_mhz else None}
     if not args.profile_only:
         # ---- traced pass: per-kernel durations from events on the backend's own stream ---------
         be.trace(True)

@@ -40,8 +40,15 @@ def run(lib, shapes=SHAPES, iters=10):
         be.trace(False)
         ms = sum(v["ms"] for v in rep.values()) / iters
         tf = 2.0 * b * m * n * k / (ms * 1e-3) / 1e12
-        out.append({"shape": f"{b}x{m}x{n}x{k}", "us": ms * 1e3, "tflops": tf, "frac": tf / MFMA_PEAK_BF16_TFLOPS,
-                    "kernels": {name: v["launches"] // iters for name, v in rep.items()}})
+        rec = {"shape": f"{b}x{m}x{n}x{k}", "us": ms * 1e3, "tflops": tf, "frac": tf / MFMA_PEAK_BF16_TFLOPS,
+               "kernels": {name: v["launches"] // iters for name, v in rep.items()}}
+        if b == 1 and m % 128 == 0 and n % 128 == 0 and k % 64 == 0:
+            # the same product through the clock probe: the shader clock its main loop ran at (the data-sheet
+            # peak is 2400 MHz) and the rate as a fraction of the matrix cores' peak at that clock
+            ptf, mhz = be.peak_gemm_clock(m, n, k, iters)
+            if mhz:
+                rec.update(clock_mhz=mhz, frac_at_clock=tf / (MFMA_PEAK_BF16_TFLOPS * mhz / 2400.0))
+        out.append(rec)
         del x, w, wt
     be.close()
     return out
@@ -55,5 +62,6 @@ if __name__ == "__main__":
     a = ap.parse_args()
     shapes = SHAPES if not a.shapes else [tuple(int(v) for v in s.split("x")) for s in a.shapes.split(",")]
     for r in run(cg.load_library(), shapes, a.iters):
-        print(f"{r['shape']:>22s} {r['us']:9.1f} us {r['tflops']:8.1f} TFLOP/s  {100 * r['frac']:5.1f} % of 2.5 PFLOP/s  {r['kernels']}",
+        clk = f"  clock {r['clock_mhz']:5.0f} MHz -> {100 * r['frac_at_clock']:5.1f} % at that clock" if "clock_mhz" in r else ""
+        print(f"{r['shape']:>22s} {r['us']:9.1f} us {r['tflops']:8.1f} TFLOP/s  {100 * r['frac']:5.1f} % of 2.5 PFLOP/s{clk}  {r['kernels']}",
               flush=True)

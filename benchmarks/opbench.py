@@ -158,5 +158,12 @@ def run_all(lib, dtypes=("f32", "bf16"), iters=50):
             rec = run_case(be, mlp_case(), iters=200, warmup=20)
             rec["dtype"] = dtype
             out.append(rec)
+            # a plain 16-byte copy of 1 GiB (peak_copy_kernel): what this device gives a read + write stream, and
+            # the launch of known size that calibrates FETCH_SIZE / WRITE_SIZE when this runs under rocprofv3
+            out.append({"op": "copy_1GiB", "dtype": dtype, "bound": "hbm", "gbs": be.peak_copy_gbs(1 << 30, 5),
+                        "algorithmic_bytes": 2 << 30, "kernels": {"peak_copy_kernel": 1}, "input_copies_rotated": 1,
+                        "kernel_us": 0.0, "wall_us": 0.0})
+            out[-1]["frac"] = out[-1]["gbs"] / HBM_PEAK_GBS
+            out[-1]["kernel_us"] = out[-1]["algorithmic_bytes"] / out[-1]["gbs"] / 1e3
         be.close()
     return out

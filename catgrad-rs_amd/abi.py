@@ -66,6 +66,7 @@ _SIGNATURES = {
     "cg_tensor_prefetch": (C.c_int, [_P, _P]),
     "cg_peak_copy_gbs": (C.c_int, [_P, _SZ, C.c_int, C.POINTER(C.c_double)]),
     "cg_peak_mfma_tflops": (C.c_int, [_P, C.c_int, C.c_int, C.POINTER(C.c_double)]),
+    "cg_peak_gemm_clock": (C.c_int, [_P, _SZ, _SZ, _SZ, C.c_int, C.POINTER(C.c_double), C.POINTER(C.c_double)]),
     "cg_backend_name": (C.c_char_p, [_P]),
     "cg_tensor_retain": (_P, [_P]),
     "cg_tensor_release": (None, [_P]),
@@ -241,6 +242,12 @@ class Backend:
         out = C.c_double()
         self._check(self.lib.cg_peak_mfma_tflops(self.ptr, U32 if operand is None else operand, iters, C.byref(out)))
         return out.value
+
+    def peak_gemm_clock(self, m, n, k, iters=5):
+        """(TFLOP/s, shader clock in MHz) of the bf16 GEMM m x n x k; m == 0: of the register-resident MFMA loop."""
+        tf, mhz = C.c_double(), C.c_double()
+        self._check(self.lib.cg_peak_gemm_clock(self.ptr, m, n, k, iters, C.byref(tf), C.byref(mhz)))
+        return tf.value, mhz.value
 
     def prefetch(self, x):
         """Realize and start an asynchronous copy of a small tensor to the host; `to_vec(x)` then

@@ -499,11 +499,15 @@ __device__ __forceinline__ Acc<KIND> shfl_xor_acc(const Acc<KIND> &a, int m) {
 // No program to interpret: rows of n unit-stride elements (f32 / u32 words, or bf16 widened to f32)
 // streamed with 16-byte (8-byte for bf16) loads, four in flight per lane.  One row per workgroup
 // (WPR = 4) or per wavefront (WPR = 1).
-template <int KIND, typename T, int WPR>
+// W: values per load - 4, or 8 for bf16 rows whose pieces of 16 bytes are aligned (n, row stride % 8 == 0):
+// with 8-byte requests a bf16 row has half the bytes in flight and - one short row per workgroup - the launch is
+// paced by workgroup turnover, not by memory; short bf16 rows therefore also go a wave per row.
+template <int KIND, typename T, int WPR, int W = 4>
 __global__ void __launch_bounds__(256) reduce_plain_kernel(const T *x, int64_t row_stride, uint32_t *out,
                                                            uint32_t rows, uint32_t n) {
   __shared__ uint32_t part[4][Acc<KIND>::W];
   constexpr int U = 4;
+  static_assert(W == 4 || (W == 8 && sizeof(T) == 2), "eight values per load: bf16 only");
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const uint32_t row = WPR == 4 ? blockIdx.x : blockIdx.x * 4 + wave;
   const uint32_t t_in_row = WPR == 4 ? threadIdx.x : lane, tpr = WPR * 64;
@@ -516,15 +520,23 @@ __global__ void __launch_bounds__(256) reduce_plain_kernel(const T *x, int64_t r
   uint32_t best_u = 0, best_c = 0;
   if (row < rows) {
     const T *r = x + (int64_t)row * row_stride;
-    for (uint32_t c0 = t_in_row * 4; c0 < n; c0 += tpr * 4 * U) {
-      uint32_t v[U][4];
+    for (uint32_t c0 = t_in_row * W; c0 < n; c0 += tpr * W * U) {
+      uint32_t v[U][W];
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-        const uint32_t c = c0 + u * tpr * 4;
+        const uint32_t c = c0 + u * tpr * W;
         if (c < n) {
           if (sizeof(T) == 4) {
             const uint4 q = *(const uint4 *)(r + c);
             v[u][0] = q.x; v[u][1] = q.y; v[u][2] = q.z; v[u][3] = q.w;
+          } else if (W == 8) {
+            const uint4 q = *(const uint4 *)(r + c);
+            const uint32_t h[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+              v[u][(2 * k) % W] = h[k] << 16;
+              v[u][(2 * k + 1) % W] = h[k] & 0xFFFF0000u;
+            }
           } else {
             const uint2 q = *(const uint2 *)(r + c);
             v[u][0] = q.x << 16; v[u][1] = q.x & 0xFFFF0000u; v[u][2] = q.y << 16; v[u][3] = q.y & 0xFFFF0000u;
@@ -533,10 +545,10 @@ __global__ void __launch_bounds__(256) reduce_plain_kernel(const T *x, int64_t r
       }
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-        const uint32_t c = c0 + u * tpr * 4;
+        const uint32_t c = c0 + u * tpr * W;
         if (c < n) {
 #pragma unroll
-          for (int j = 0; j < 4; ++j) {
+          for (int j = 0; j < W; ++j) {
             if constexpr (KIND == R_ARGMAX_F) {
               const uint32_t b = v[u][j], o = b ^ ((uint32_t)((int32_t)b >> 31) | 0x80000000u);  // total_cmp order, unsigned
               const bool take = o >= best_u;
@@ -596,6 +608,11 @@ __global__ void __launch_bounds__(256) reduce_plain_kernel(const T *x, int64_t r
 template <int KIND>
 static void launch_reduce_plain_kind(const LaunchCtx &lc, const void *x, int bf16, int64_t row_stride, uint32_t *out,
                                      uint32_t rows, uint32_t n) {
+  if (bf16 && n % 8 == 0 && row_stride % 8 == 0 && (uintptr_t)x % 16 == 0) {
+    if (n > 8192) CG_LAUNCH(lc, (reduce_plain_kernel<KIND, uint16_t, 4, 8>), rows, 256, (const uint16_t *)x, row_stride, out, rows, n);
+    else CG_LAUNCH(lc, (reduce_plain_kernel<KIND, uint16_t, 1, 8>), (rows + 3) / 4, 256, (const uint16_t *)x, row_stride, out, rows, n);
+    return;
+  }
   if (n >= 1024) {
     if (bf16) CG_LAUNCH(lc, (reduce_plain_kernel<KIND, uint16_t, 4>), rows, 256, (const uint16_t *)x, row_stride, out, rows, n);
     else CG_LAUNCH(lc, (reduce_plain_kernel<KIND, uint32_t, 4>), rows, 256, (const uint32_t *)x, row_stride, out, rows, n);

@@ -613,6 +613,13 @@ __global__ void __launch_bounds__(WR *WC * 64) gemm_bf16_dma_kernel(GemmDesc g) 
     __builtin_amdgcn_s_setprio(0);
   };
   const int n_steps = k_end > k_begin ? (int)((k_end - k_begin) / BK) : 0;
+  // (clock probe only) s_memtime ticks with the shader clock, s_memrealtime with a constant 100 MHz: their ratio
+  // over the main loop is the clock this kernel really ran at
+  unsigned long long tick0 = 0, real0 = 0;
+  if (g.clock_ticks) {
+    tick0 = __builtin_amdgcn_s_memtime();
+    real0 = __builtin_amdgcn_s_memrealtime();
+  }
 #pragma unroll
   for (int s0 = 0; s0 < NS - 1; ++s0)
     if (s0 < n_steps) issue(s0);
@@ -624,6 +631,10 @@ __global__ void __launch_bounds__(WR *WC * 64) gemm_bf16_dma_kernel(GemmDesc g) 
     __syncthreads();   // ... and everyone's; all waves are done reading the buffer refilled next
     if (step + NS - 1 < n_steps) issue((step + NS - 1) % NS);
     compute(step % NS);
+  }
+  if (g.clock_ticks && tid == 0) {
+    atomicAdd(g.clock_ticks, __builtin_amdgcn_s_memtime() - tick0);
+    atomicAdd(g.clock_ticks + 1, __builtin_amdgcn_s_memrealtime() - real0);
   }
   if constexpr (EPI) {
     constexpr int TP = BNO + 4;  // row pitch of the staged tile (floats)

@@ -71,8 +71,62 @@ __global__ void __launch_bounds__(256) gather_kernel(GatherDesc g, uint64_t n_gr
   }
 }
 
+// Rows of a matrix by index (an embedding lookup, helpers.rs:259-271: `index(0, ids, table)`): a wavefront owns
+// an output row, reads its index once and streams the row - four values per lane and load, U loads in flight,
+// 16-byte stores - instead of decomposing every element's position with 64-bit divisions.  bf16 rows are
+// widened on the way (8-byte loads, so twice as many of them in flight).
+template <typename T, int U>
+__global__ void __launch_bounds__(256) gather_rows_kernel(const T *x, int64_t x_row_stride, const uint32_t *idx,
+                                                          uint32_t x_rows, uint32_t *out, uint32_t rows, uint32_t n,
+                                                          uint32_t *err) {
+  const uint32_t lane = threadIdx.x & 63, row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;  // the whole wave
+  uint32_t ix = idx[row];
+  if (ix >= x_rows) {  // the reference panics; flag it and stay in bounds
+    if (lane == 0) atomicOr(err, ERRF_INDEX_OOB);
+    ix = x_rows - 1;
+  }
+  const T *src = x + (int64_t)ix * x_row_stride;
+  uint32_t *dst = out + (uint64_t)row * n;
+  // Rows start at multiples of the row size, so waves that all began with their row's first piece would ask the
+  // same few memory channels at the same moment (8 KB rows of f32: 19 us against 13 for the same bytes); every
+  // row starts with another piece instead.
+  const uint32_t rot = row % U;
+  for (uint32_t c0 = lane * 4; c0 < n; c0 += 64 * 4 * U) {
+    uint4 v[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const uint32_t c = c0 + ((u + rot) % U) * 256;
+      if (c < n) {
+        if (sizeof(T) == 4) {
+          v[u] = *(const uint4 *)(src + c);
+        } else {
+          const uint2 q = *(const uint2 *)(src + c);
+          v[u] = make_uint4(q.x << 16, q.x & 0xFFFF0000u, q.y << 16, q.y & 0xFFFF0000u);
+        }
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const uint32_t c = c0 + ((u + rot) % U) * 256;
+      if (c < n) *(uint4 *)(dst + c) = v[u];
+    }
+  }
+}
+
 hipError_t launch_gather(const LaunchCtx &lc, const GatherDesc &g, uint64_t n_out) {
   if (!n_out) return hipSuccess;
+  if (g.vec && g.n_dims == 2 && g.dim == 0 && g.x_stride[1] == 1 && g.out_dims[1] % 4 == 0 && g.out_dims[1] >= 256 &&
+      (uintptr_t)g.out % 16 == 0) {
+    const uint32_t rows = g.out_dims[0], n = g.out_dims[1];
+    if (g.x_stype == ST_BF16)
+      CG_LAUNCH(lc, (gather_rows_kernel<uint16_t, 8>), (rows + 3) / 4, 256, (const uint16_t *)g.x, g.x_stride[0], g.idx,
+                g.x_dim_size, (uint32_t *)g.out, rows, n, lc.err_flag);
+    else
+      CG_LAUNCH(lc, (gather_rows_kernel<uint32_t, 8>), (rows + 3) / 4, 256, (const uint32_t *)g.x, g.x_stride[0], g.idx,
+                g.x_dim_size, (uint32_t *)g.out, rows, n, lc.err_flag);
+    return hipGetLastError();
+  }
   const bool vec = g.vec && g.dim != g.n_dims - 1 && (g.out_dims[g.n_dims - 1] % 4 == 0);
   uint64_t groups = vec ? n_out / 4 : n_out;
   uint64_t blocks = (groups + 255) / 256, cap = (uint64_t)lc.n_cus * 8;
@@ -285,11 +339,59 @@ __global__ void __launch_bounds__(256) transpose_copy_kernel(TransposeDesc d) {
   }
 }
 
+// The same for 4-byte elements whose rows allow 16-byte moves on both sides (R, C, the strides and the bases
+// multiples of four elements): a lane loads four values of an input row and stores four values of an output
+// row; the 64 x 64 tile turns around in LDS word by word (pitch 65: two lanes per bank at worst).  Four times
+// the bytes per request of the kernel above, which left a transposed copy at 4.1 TB/s where a plain copy
+// reaches 4.9.
+__global__ void __launch_bounds__(256) transpose_copy_vec_kernel(TransposeDesc d) {
+  __shared__ uint32_t tile[64][65];
+  uint32_t rem = blockIdx.z;
+  int64_t xo = 0, oo = 0;
+  for (int i = d.n_other - 1; i >= 0; --i) {
+    const uint32_t c = rem % d.odims[i];
+    rem /= d.odims[i];
+    xo += (int64_t)c * d.x_so[i];
+    oo += (int64_t)c * d.o_so[i];
+  }
+  const uint32_t *x = (const uint32_t *)d.x + xo;
+  uint32_t *out = (uint32_t *)d.out + oo;
+  const uint32_t c0 = blockIdx.x * 64, j0 = blockIdx.y * 64;
+  const uint32_t q4 = (threadIdx.x & 15) * 4, rr = threadIdx.x >> 4;
+  uint4 v[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const uint32_t c = c0 + rr + i * 16, j = j0 + q4;
+    if (c < d.C && j < d.R) v[i] = *(const uint4 *)(x + (int64_t)c * d.x_sc + j);
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const uint32_t r = rr + i * 16;
+    tile[r][q4] = v[i].x; tile[r][q4 + 1] = v[i].y; tile[r][q4 + 2] = v[i].z; tile[r][q4 + 3] = v[i].w;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const uint32_t jr = rr + i * 16, j = j0 + jr, c = c0 + q4;
+    if (j < d.R && c < d.C)
+      *(uint4 *)(out + (int64_t)j * d.o_sj + c) = make_uint4(tile[q4][jr], tile[q4 + 1][jr], tile[q4 + 2][jr], tile[q4 + 3][jr]);
+  }
+}
+
 hipError_t launch_transpose_copy(const LaunchCtx &lc, const TransposeDesc &d) {
   uint64_t other = 1;
   for (int i = 0; i < d.n_other; ++i) other *= d.odims[i];
   if (!d.R || !d.C || !other) return hipSuccess;
   dim3 grid((d.C + 63) / 64, (d.R + 63) / 64, (unsigned)other);
+  if (d.x_stype != ST_BF16 && !d.out_bf16 && d.R % 4 == 0 && d.C % 4 == 0 && d.x_sc % 4 == 0 && d.o_sj % 4 == 0 &&
+      (uintptr_t)d.x % 16 == 0 && (uintptr_t)d.out % 16 == 0) {
+    bool ok = true;
+    for (int i = 0; i < d.n_other; ++i) ok = ok && d.x_so[i] % 4 == 0 && d.o_so[i] % 4 == 0;
+    if (ok) {
+      CG_LAUNCH(lc, (transpose_copy_vec_kernel), grid, 256, d);
+      return hipGetLastError();
+    }
+  }
   if (d.x_stype == ST_BF16 && d.out_bf16) CG_LAUNCH(lc, (transpose_copy_kernel<uint16_t, true>), grid, 256, d);
   else if (d.x_stype == ST_BF16) CG_LAUNCH(lc, (transpose_copy_kernel<uint16_t, false>), grid, 256, d);
   else CG_LAUNCH(lc, (transpose_copy_kernel<uint32_t, false>), grid, 256, d);
@@ -313,7 +415,9 @@ typedef __attribute__((ext_vector_type(8))) __bf16 pk_bf16x8;
 typedef __attribute__((ext_vector_type(16))) float pk_f32x16;
 
 template <bool BF16>
-__global__ void __launch_bounds__(256) peak_mfma_kernel(float *out, int iters) {
+__global__ void __launch_bounds__(256) peak_mfma_kernel(float *out, int iters, unsigned long long *clock_ticks) {
+  // (optional) shader-clock ticks and 100 MHz ticks of the loop, summed over the workgroups: the clock it ran at
+  const unsigned long long tick0 = __builtin_amdgcn_s_memtime(), real0 = __builtin_amdgcn_s_memrealtime();
   pk_f32x16 acc[4];
   for (int i = 0; i < 4; ++i)
     for (int e = 0; e < 16; ++e) acc[i][e] = 0.f;
@@ -334,12 +438,16 @@ __global__ void __launch_bounds__(256) peak_mfma_kernel(float *out, int iters) {
   for (int i = 0; i < 4; ++i)
     for (int e = 0; e < 16; ++e) s += acc[i][e];
   out[(uint64_t)blockIdx.x * 256 + threadIdx.x] = s;
+  if (clock_ticks && threadIdx.x == 0) {
+    atomicAdd(clock_ticks, __builtin_amdgcn_s_memtime() - tick0);
+    atomicAdd(clock_ticks + 1, __builtin_amdgcn_s_memrealtime() - real0);
+  }
 }
 
 // flops issued: grid * 4 waves * iters * 4 MFMAs * (2 * 32 * 32 * k), k = 16 (bf16) or 2 (f32)
-hipError_t launch_peak_mfma(const LaunchCtx &lc, int bf16, float *out, unsigned grid, int iters) {
-  if (bf16) CG_LAUNCH(lc, (peak_mfma_kernel<true>), grid, 256, out, iters);
-  else CG_LAUNCH(lc, (peak_mfma_kernel<false>), grid, 256, out, iters);
+hipError_t launch_peak_mfma(const LaunchCtx &lc, int bf16, float *out, unsigned grid, int iters, unsigned long long *clock_ticks) {
+  if (bf16) CG_LAUNCH(lc, (peak_mfma_kernel<true>), grid, 256, out, iters, clock_ticks);
+  else CG_LAUNCH(lc, (peak_mfma_kernel<false>), grid, 256, out, iters, clock_ticks);
   return hipGetLastError();
 }
 

@@ -95,7 +95,8 @@ struct TransposeDesc {
 hipError_t launch_transpose_copy(const LaunchCtx &lc, const TransposeDesc &d);
 // peak probes: plain 16-byte copy; MFMA issue loop (out: grid * 256 floats)
 hipError_t launch_peak_copy(const LaunchCtx &lc, const void *in, void *out, uint64_t bytes);
-hipError_t launch_peak_mfma(const LaunchCtx &lc, int bf16, float *out, unsigned grid, int iters);
+hipError_t launch_peak_mfma(const LaunchCtx &lc, int bf16, float *out, unsigned grid, int iters,
+                            unsigned long long *clock_ticks = nullptr);
 
 // ---- k_fused.hip
 struct RmsNormDesc {
@@ -297,6 +298,9 @@ struct GemmDesc {
   const void *grp_b[3];
   float *grp_c[3];
   uint32_t grp_n[3];
+  // optional (the direct-to-LDS bf16 GEMM, for the clock probe): every workgroup adds the shader-clock ticks and
+  // the 100 MHz ticks its main loop took to clock_ticks[0] and [1]
+  unsigned long long *clock_ticks;
 };
 // split factor launch_matmul should be given for this problem (1 = none)
 uint32_t gemm_split_k(const LaunchCtx &lc, const GemmDesc &g);

@@ -152,6 +152,7 @@ struct cg_backend {
   // arange(n) is immutable and models ask for the same few n over and over (masks, RoPE tables of
   // every layer): one node per n, realised once
   std::map<int64_t, cg_tensor *> arange_cache;
+  std::deque<int64_t> arange_order;  // the cached extents, oldest first (the oldest leaves when the cache is full)
   // deferred nodes built from constants and aranges only, by structure: every layer of a model asks
   // for the same causal mask, and gets the same node (weak references; an entry goes when its node is
   // realised or deleted)

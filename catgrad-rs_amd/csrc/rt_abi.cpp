@@ -75,6 +75,7 @@ void cg_backend_destroy(cg_backend *be) {
   // cached nodes hold references to the backend: drop them first
   std::map<int64_t, cg_tensor *> cache;
   cache.swap(be->arange_cache);
+  be->arange_order.clear();
   for (auto &kv : cache) node_release(kv.second);
   std::deque<cg_tensor *> keep;
   keep.swap(be->shared_keep);
@@ -615,17 +616,31 @@ int cg_arange(cg_backend *be, size_t end, cg_tensor **out) {
       *out = retain(it->second);
       return CG_OK;
     }
-    if (be->arange_cache.size() < 32) {
-      cg_tensor *n = new_node(be, CG_U32, 1, shape);
-      n->op = N_ARANGE;
-      n->const_like = true;
-      n->cse_key = new std::string("arange" + std::to_string(end));
-      be->arange_cache[(int64_t)end] = retain(n);
-      return finish(be, n, out);
+    // A backend lives through many sequence lengths: when the cache is full its oldest extent leaves (whoever
+    // still holds that node keeps it alive), so that the lengths in use now are always the cached ones.
+    if (be->arange_cache.size() >= 32 && !be->arange_order.empty()) {
+      auto old = be->arange_cache.find(be->arange_order.front());
+      be->arange_order.pop_front();
+      if (old != be->arange_cache.end()) {
+        cg_tensor *t = old->second;
+        be->arange_cache.erase(old);
+        node_release(t);
+      }
     }
+    cg_tensor *n = new_node(be, CG_U32, 1, shape);
+    n->op = N_ARANGE;
+    n->const_like = true;
+    n->cse_key = new std::string("arange" + std::to_string(end));
+    be->arange_cache[(int64_t)end] = retain(n);
+    be->arange_order.push_back((int64_t)end);
+    return finish(be, n, out);
   }
   cg_tensor *n = new_node(be, CG_U32, 1, shape);
   n->op = N_ARANGE;
+  if (!(be->flags & CG_FLAG_EAGER)) {  // not cached, but still a value any mask built from it can be shared by
+    n->const_like = true;
+    n->cse_key = new std::string("arange" + std::to_string(end));
+  }
   return finish(be, n, out);
 }
 
@@ -692,6 +707,80 @@ int cg_peak_mfma_tflops(cg_backend *be, cg_dtype operand, int iters, double *tfl
   if (e != hipSuccess) return fail(be, CG_ERR_DEVICE, hipGetErrorString(e));
   const double k = bf16 ? 16.0 : 2.0;
   *tflops = (double)grid * 4 * iters * 4 * (2.0 * 32 * 32 * k) / (ms * 1e-3) / 1e12;
+  return CG_OK;
+}
+
+int cg_peak_gemm_clock(cg_backend *be, size_t m, size_t n, size_t k, int iters, double *tflops, double *clock_mhz) {
+  if (!be || !tflops || !clock_mhz || iters < 1) return CG_ERR_ARG;
+  if (m && (m % 128 || n % 128 || k % 64 || !n || !k || m * k >= ((size_t)1 << 31) || n * k >= ((size_t)1 << 31)))
+    return fail(be, CG_ERR_ARG, "cg_peak_gemm_clock: m, n multiples of 128, k of 64");
+  HIPCHK(be, hipSetDevice(be->device));
+  LaunchCtx lc = be->lc();
+  lc.ev_start = lc.ev_stop = nullptr;
+  Storage *a = nullptr, *b = nullptr, *c = nullptr, *ticks = nullptr;
+  const unsigned grid = (unsigned)be->n_cus * 8;
+  int st = dev_alloc(be, 16, &ticks);
+  if (!st) st = dev_alloc(be, m ? m * n * 4 : (size_t)grid * 256 * 4, &c);
+  if (!st && m) st = dev_alloc(be, m * k * 2, &a);
+  if (!st && m) st = dev_alloc(be, n * k * 2, &b);
+  hipEvent_t e0 = nullptr, e1 = nullptr;
+  hipError_t e = hipSuccess;
+  GemmDesc g;
+  std::memset(&g, 0, sizeof(g));
+  if (!st) {
+    if (m) {
+      // operands that toggle like real data (a constant operand draws less power and clocks higher)
+      std::vector<uint16_t> h(std::max(m, n) * k);
+      uint32_t r = 12345u;
+      for (auto &v : h) {
+        r = r * 1664525u + 1013904223u;
+        const float f = (float)((r >> 8) & 0xffff) / 65536.f - 0.5f;
+        uint32_t u;
+        std::memcpy(&u, &f, 4);
+        v = (uint16_t)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
+      }
+      e = hipStreamSynchronize(be->ordered_stream());
+      if (e == hipSuccess) e = hipMemcpy(a->ptr, h.data(), m * k * 2, hipMemcpyHostToDevice);
+      if (e == hipSuccess) e = hipMemcpy(b->ptr, h.data(), n * k * 2, hipMemcpyHostToDevice);
+      g.a = a->ptr; g.b = b->ptr; g.c = (float *)c->ptr;
+      g.a_stype = g.b_stype = ST_BF16;
+      g.bf16_math = 1;
+      g.M = (uint32_t)m; g.N = (uint32_t)n; g.K = (uint32_t)k;
+      g.nb0 = g.nb1 = 1;
+      g.sam = (int64_t)k; g.sak = 1; g.sbn = (int64_t)k; g.sbk = 1;
+      g.splits = 1; g.k_per_split = (uint32_t)k;
+    }
+    auto once = [&](unsigned long long *t) -> hipError_t {
+      if (!m) return launch_peak_mfma(lc, 1, (float *)c->ptr, grid, 20000, t);
+      g.clock_ticks = t;
+      return launch_matmul(lc, g, nullptr);
+    };
+    if (e == hipSuccess) e = hipEventCreate(&e0);
+    if (e == hipSuccess) e = hipEventCreate(&e1);
+    if (e == hipSuccess) e = once(nullptr);  // warm-up
+    if (e == hipSuccess) e = launch_fill_u32(lc, (uint32_t *)ticks->ptr, 0u, 4);
+    if (e == hipSuccess) e = hipEventRecord(e0, be->ordered_stream());
+    for (int i = 0; i < iters && e == hipSuccess; ++i) e = once((unsigned long long *)ticks->ptr);
+    if (e == hipSuccess) e = hipEventRecord(e1, be->ordered_stream());
+    if (e == hipSuccess) e = hipStreamSynchronize(be->ordered_stream());
+    float ms = 0.f;
+    unsigned long long t[2] = {0, 0};
+    if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
+    if (e == hipSuccess) e = hipMemcpy(t, ticks->ptr, 16, hipMemcpyDeviceToHost);
+    if (e == hipSuccess) {
+      const double flops = m ? 2.0 * (double)m * (double)n * (double)k : (double)grid * 4 * 20000.0 * 4 * (2.0 * 32 * 32 * 16);
+      *tflops = flops * iters / (ms * 1e-3) / 1e12;
+      *clock_mhz = t[1] ? (double)t[0] / (double)t[1] * 100.0 : 0.0;
+    }
+  }
+  if (e0) (void)hipEventDestroy(e0);
+  if (e1) (void)hipEventDestroy(e1);
+  storage_release(a);
+  storage_release(b);
+  storage_release(c);
+  storage_release(ticks);
+  if (st) return st;
+  if (e != hipSuccess) return fail(be, CG_ERR_DEVICE, hipGetErrorString(e));
   return CG_OK;
 }
 

@@ -258,7 +258,11 @@ int try_softmax(cg_backend *be, cg_tensor *root, bool *done) {
   if (!st) {
     d.x = (const float *)data_ptr(xs);
     d.y = (float *)root->st->ptr;
-    st = twin_for_result(be, root, &d.y16);
+    // the bf16 copy is for a product that waits for these rows as its left operand: attention's p . V (a
+    // batched product over heads, rank 4) or a recorded many-row product; for anybody else it would be a
+    // third of the launch's traffic written for nobody
+    bool only_gemms = false;
+    if (root->rank >= 4 || gemm_readers(be, root, &only_gemms) > 0) st = twin_for_result(be, root, &d.y16);
     d.x_row_stride = row_stride;
     d.rows = (uint32_t)(root->size() / n);
     d.n = (uint32_t)n;

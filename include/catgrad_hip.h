@@ -192,6 +192,12 @@ int cg_trace_enable(cg_backend *be, int on);
  * Benchmarks report them beside the data-sheet peaks. */
 int cg_peak_copy_gbs(cg_backend *be, size_t bytes, int iters, double *gbs);
 int cg_peak_mfma_tflops(cg_backend *be, cg_dtype operand, int iters, double *tflops);
+/* Clock probe (no counterpart in the reference): `iters` launches of the bf16 product C[m, n] = A[m, k] . B[n, k]^T
+ * on pseudo-random operands (m, n multiples of 128, k of 64) through the library's own GEMM dispatch; *tflops is
+ * their rate and *clock_mhz the shader clock their main loops ran at (shader-clock ticks over 100 MHz ticks,
+ * read inside the kernel).  m == 0: the register-resident bf16 MFMA loop of cg_peak_mfma_tflops instead.  A
+ * GEMM draws more power than the bare loop and is clocked lower; its MFMA fraction is a fraction of that clock. */
+int cg_peak_gemm_clock(cg_backend *be, size_t m, size_t n, size_t k, int iters, double *tflops, double *clock_mhz);
 int cg_trace_reset(cg_backend *be);
 /* returns the number of bytes needed (including the NUL); writes at most cap bytes */
 size_t cg_trace_report(cg_backend *be, char *buf, size_t cap);

@@ -98,6 +98,7 @@ int cg_tensor_prefetch(cg_backend *, cg_tensor *) { return CG_OK; }
 // the probes measure a device; the oracle has none
 int cg_peak_copy_gbs(cg_backend *, size_t, int, double *) { return CG_ERR_DEVICE; }
 int cg_peak_mfma_tflops(cg_backend *, cg_dtype, int, double *) { return CG_ERR_DEVICE; }
+int cg_peak_gemm_clock(cg_backend *, size_t, size_t, size_t, int, double *, double *) { return CG_ERR_DEVICE; }
 const char *cg_backend_name(const cg_backend *) { return "ndarray-oracle"; }
 
 cg_tensor *cg_tensor_retain(cg_tensor *t) {

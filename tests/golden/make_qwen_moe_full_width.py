@@ -7,8 +7,8 @@ this width, so its results are kept as vectors:
                        step of four rows fed those tokens;
   rounded parameters (what bf16 mode stores): the full-recompute model's logits at every position, the
                        mask of positions exposed to a router near tie (k-th and (k+1)-th router logit closer
-                       than 2e-2 of the row's largest, for the token or an earlier one of its sequence), and
-                       the same decode step.
+                       than 2e-2 of the row's largest; with one layer no attention reads a routed result,
+                       so a near tie exposes its own position only), and the same decode step.
 Parameters and prompts are rebuilt by the test from the same seeds (tests/model_util.py).
 
 Run from the repository root after `make -C oracle`:  python tests/golden/make_qwen_moe_full_width.py
@@ -82,7 +82,8 @@ def main():
         lg = oracle.numpy(layer).reshape(prompts.shape + (cfg.num_experts,)).astype(np.float64)
         srt = np.sort(lg, axis=-1)
         near |= (srt[..., -k] - srt[..., -k - 1]) <= NEAR_TIE * np.abs(lg).max(axis=-1)
-    out["rounded_exposed"] = np.maximum.accumulate(near, axis=1)
+    assert cfg.num_hidden_layers == 1
+    out["rounded_exposed"] = near
     out["prompts"] = prompts
     np.savez_compressed(os.path.join(ROOT, "tests", "golden", "qwen_moe_full_width.npz"), **out)
     print("exposed", out["rounded_exposed"].sum(), "of", near.size)

@@ -75,3 +75,19 @@ def test_opbench_runs(hip):
     for case in opbench.cases("f32", scale=8):
         rec = opbench.run_case(hip, case, iters=3, warmup=1)
         assert rec["kernel_us"] > 0 and rec["wall_us"] > 0, rec
+
+
+@pytest.mark.gpu
+def test_peak_probes(hip_bf16):
+    """The measured denominators bench.py prints: a copy rate, the MFMA issue rates, and the shader clock read
+    inside the bare MFMA loop and inside the bf16 GEMM (a GEMM draws more power and may be clocked lower, never
+    higher than the data sheet's 2400 MHz by more than the boost margin)."""
+    be = hip_bf16
+    assert 500 < be.peak_copy_gbs(1 << 28, 3) < 8000
+    assert 100 < be.peak_mfma_tflops(iters=2000) < 2600
+    loop_tf, loop_mhz = be.peak_gemm_clock(0, 0, 0, 1)
+    tf, mhz = be.peak_gemm_clock(2048, 2048, 2048, 3)
+    assert 100 < loop_tf < 2600 and 50 < tf < 2600
+    assert 500 < loop_mhz < 2700 and 500 < mhz < 2700
+    with pytest.raises(vectors.cg.abi.BackendPanic):
+        be.peak_gemm_clock(100, 128, 64, 1)      # m not a multiple of 128
