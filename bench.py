@@ -23,19 +23,19 @@ HBM_PEAK_GBS = 8000.0
 MFMA_PEAK_TFLOPS = {"bf16": 2500.0, "f32": 157.3}
 # HBM bytes per launch of the decode GEMV kernels at the default workload come from two rocprofv3 --pmc
 # runs of this file (FETCH_SIZE, WRITE_SIZE; a profiler cannot run inside this process).  Their
-# summary, with the commands, is this file; its "traffic_bytes_per_launch" line is read, so the figure
+# summary, with the commands, is these files; their "traffic_bytes_per_launch" line is read, so the figure
 # reported is the one the committed counters show, for the workload they were taken on only.
-PMC_SUMMARY = os.path.join(ROOT, "profiles", "gemv_rowdot_bf16_llama1b_decode_pmc.txt")
+PMC_SUMMARY = {dt: os.path.join(ROOT, "profiles", f"gemv_rowdot_{dt}_llama1b_decode_pmc.txt") for dt in ("bf16", "f32")}
 
 
 def pmc_traffic_bytes_per_launch(dtype, layers, kernel):
     """The `traffic_bytes_per_launch[dtype,layers,kernel] = N` line of the PMC summary, or None."""
     key = f"traffic_bytes_per_launch[{dtype},{layers},{kernel}]"
     try:
-        for line in open(PMC_SUMMARY):
+        for line in open(PMC_SUMMARY[dtype]):
             if key in line:
                 return float(line.split("=")[1].split()[0])
-    except OSError:
+    except (OSError, KeyError):
         pass
     return None
 

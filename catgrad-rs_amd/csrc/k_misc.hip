@@ -5,6 +5,8 @@
 // Backend::compare(mod.rs:59,    ndarray.rs:337-343): shape and element equality
 // All HBM- or latency-bound; index moves 16 bytes per lane along the innermost axis.
 #include <hip/hip_runtime.h>
+#include <algorithm>
+#include <cstdlib>
 #include "launch.hpp"
 #include "dev_common.hpp"
 
@@ -71,60 +73,56 @@ __global__ void __launch_bounds__(256) gather_kernel(GatherDesc g, uint64_t n_gr
   }
 }
 
-// Rows of a matrix by index (an embedding lookup, helpers.rs:259-271: `index(0, ids, table)`): a wavefront owns
-// an output row, reads its index once and streams the row - four values per lane and load, U loads in flight,
-// 16-byte stores - instead of decomposing every element's position with 64-bit divisions.  bf16 rows are
-// widened on the way (8-byte loads, so twice as many of them in flight).
+// Rows of a bf16 matrix by index (an embedding lookup in bf16 mode, helpers.rs:259-271: `index(0, ids, table)`),
+// widened to f32: a wavefront owns an output row, reads its index once and streams the row - four values per lane
+// and 8-byte load, U loads in flight, 16-byte stores - instead of decomposing every element's position with
+// 64-bit divisions and keeping one short load in flight per lane.
 template <typename T, int U>
 __global__ void __launch_bounds__(256) gather_rows_kernel(const T *x, int64_t x_row_stride, const uint32_t *idx,
                                                           uint32_t x_rows, uint32_t *out, uint32_t rows, uint32_t n,
                                                           uint32_t *err) {
-  const uint32_t lane = threadIdx.x & 63, row = blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (row >= rows) return;  // the whole wave
-  uint32_t ix = idx[row];
-  if (ix >= x_rows) {  // the reference panics; flag it and stay in bounds
-    if (lane == 0) atomicOr(err, ERRF_INDEX_OOB);
-    ix = x_rows - 1;
-  }
-  const T *src = x + (int64_t)ix * x_row_stride;
-  uint32_t *dst = out + (uint64_t)row * n;
-  // Rows start at multiples of the row size, so waves that all began with their row's first piece would ask the
-  // same few memory channels at the same moment (8 KB rows of f32: 19 us against 13 for the same bytes); every
-  // row starts with another piece instead.
-  const uint32_t rot = row % U;
-  for (uint32_t c0 = lane * 4; c0 < n; c0 += 64 * 4 * U) {
-    uint4 v[U];
+  const uint32_t lane = threadIdx.x & 63;
+  for (uint32_t row = blockIdx.x * 4 + (threadIdx.x >> 6); row < rows; row += gridDim.x * 4) {  // (uniform per wave)
+    uint32_t ix = idx[row];
+    if (ix >= x_rows) {  // the reference panics; flag it and stay in bounds
+      if (lane == 0) atomicOr(err, ERRF_INDEX_OOB);
+      ix = x_rows - 1;
+    }
+    const T *src = x + (int64_t)ix * x_row_stride;
+    uint32_t *dst = out + (uint64_t)row * n;
+    for (uint32_t c0 = lane * 4; c0 < n; c0 += 64 * 4 * U) {
+      uint4 v[U];
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const uint32_t c = c0 + ((u + rot) % U) * 256;
-      if (c < n) {
-        if (sizeof(T) == 4) {
-          v[u] = *(const uint4 *)(src + c);
-        } else {
-          const uint2 q = *(const uint2 *)(src + c);
-          v[u] = make_uint4(q.x << 16, q.x & 0xFFFF0000u, q.y << 16, q.y & 0xFFFF0000u);
+      for (int u = 0; u < U; ++u) {
+        const uint32_t c = c0 + u * 256;
+        if (c < n) {
+          if (sizeof(T) == 4) {
+            v[u] = *(const uint4 *)(src + c);
+          } else {
+            const uint2 q = *(const uint2 *)(src + c);
+            v[u] = make_uint4(q.x << 16, q.x & 0xFFFF0000u, q.y << 16, q.y & 0xFFFF0000u);
+          }
         }
       }
-    }
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const uint32_t c = c0 + ((u + rot) % U) * 256;
-      if (c < n) *(uint4 *)(dst + c) = v[u];
+      for (int u = 0; u < U; ++u) {
+        const uint32_t c = c0 + u * 256;
+        if (c < n) *(uint4 *)(dst + c) = v[u];
+      }
     }
   }
 }
 
 hipError_t launch_gather(const LaunchCtx &lc, const GatherDesc &g, uint64_t n_out) {
   if (!n_out) return hipSuccess;
-  if (g.vec && g.n_dims == 2 && g.dim == 0 && g.x_stride[1] == 1 && g.out_dims[1] % 4 == 0 && g.out_dims[1] >= 256 &&
-      (uintptr_t)g.out % 16 == 0) {
+  // (rows of 4-byte values stay on the generic kernel: the same row kernel moved them at 3.3 TB/s whatever its
+  // grid, against 5 TB/s for the kernel below, whose consecutive waves take consecutive pieces of a row)
+  if (g.vec && g.x_stype == ST_BF16 && g.n_dims == 2 && g.dim == 0 && g.x_stride[1] == 1 && g.out_dims[1] % 4 == 0 &&
+      g.out_dims[1] >= 256 && g.out_dims[0] >= (uint32_t)lc.n_cus && (uintptr_t)g.out % 16 == 0) {  // (a wave per row: enough rows)
     const uint32_t rows = g.out_dims[0], n = g.out_dims[1];
-    if (g.x_stype == ST_BF16)
-      CG_LAUNCH(lc, (gather_rows_kernel<uint16_t, 8>), (rows + 3) / 4, 256, (const uint16_t *)g.x, g.x_stride[0], g.idx,
-                g.x_dim_size, (uint32_t *)g.out, rows, n, lc.err_flag);
-    else
-      CG_LAUNCH(lc, (gather_rows_kernel<uint32_t, 8>), (rows + 3) / 4, 256, (const uint32_t *)g.x, g.x_stride[0], g.idx,
-                g.x_dim_size, (uint32_t *)g.out, rows, n, lc.err_flag);
+    const uint32_t blocks = std::min((rows + 3) / 4, (uint32_t)lc.n_cus * 16u);
+    CG_LAUNCH(lc, (gather_rows_kernel<uint16_t, 8>), blocks, 256, (const uint16_t *)g.x, g.x_stride[0], g.idx,
+              g.x_dim_size, (uint32_t *)g.out, rows, n, lc.err_flag);
     return hipGetLastError();
   }
   const bool vec = g.vec && g.dim != g.n_dims - 1 && (g.out_dims[g.n_dims - 1] % 4 == 0);

@@ -8,9 +8,11 @@
 // in a fixed array in device memory that the library's code object carries.
 //
 // Every GPU the library runs on holds its own copy of that array, at its own address, until the
-// process ends.  All calls on one GPU share it and it keeps the last call's contents: the split pass
-// writes every word the merge pass reads, so nothing needs clearing, but two calls that overlap on
-// one GPU (two backends on two streams) race on it.
+// process ends.  The array is cut into SLOTS slices; a backend takes a free slice of its device at its
+// first call and keeps it until it is destroyed, so calls of different backends (different streams) never
+// share scratch memory, and the calls of one backend are ordered by its stream.  A slice keeps the last
+// call's contents: the split pass writes every word the merge pass reads, so nothing needs clearing.  When
+// every slice of a device is taken the call is refused.
 #include "rt.hpp"
 
 #include <mutex>
@@ -22,14 +24,15 @@ namespace {
 // 12 bytes per (row, chunk); rows are split into at most 2 x CUs / rows chunks, so 16 KiB covers every
 // shape on a device of up to 682 CUs.  Beyond it the call is refused.
 enum : size_t { SCRATCH_BYTES = 16 * 1024 };
-enum : int { MAX_DEVICES = 64 };
+enum : int { MAX_DEVICES = 64, SLOTS = 8 };
 
-// Device memory.  In host code this name is only a handle for hipGetSymbolAddress, never an address:
-// the pointers below are what host code passes to kernels.
-static __device__ __align__(256) unsigned char scratch[SCRATCH_BYTES];
+// Device memory (128 KiB per GPU).  In host code this name is only a handle for hipGetSymbolAddress, never an
+// address: the pointers below are what host code passes to kernels.
+static __device__ __align__(256) unsigned char scratch[SLOTS * SCRATCH_BYTES];
 
 std::mutex g_lock;
 void *g_scratch_ptr[MAX_DEVICES];
+uint32_t g_slots_taken[MAX_DEVICES];  // bit s: slice s of this device's array belongs to a live backend
 
 }  // namespace
 
@@ -46,6 +49,12 @@ int noalloc_init_device(int device) {
   }
   g_scratch_ptr[device] = ptr;
   return CG_OK;
+}
+
+void noalloc_release_slot(int device, int slot) {
+  if (device < 0 || device >= MAX_DEVICES || slot < 0 || slot >= SLOTS) return;
+  std::lock_guard<std::mutex> lk(g_lock);
+  g_slots_taken[device] &= ~(1u << slot);
 }
 
 }  // namespace cgrt
@@ -71,9 +80,21 @@ extern "C" int cg_argmax_into(cg_backend *be, cg_tensor *x, cg_tensor *out) {
   uint32_t *ptr = nullptr;
   {
     std::lock_guard<std::mutex> lk(g_lock);
-    if (be->device >= 0 && be->device < MAX_DEVICES) ptr = (uint32_t *)g_scratch_ptr[be->device];
+    if (be->device >= 0 && be->device < MAX_DEVICES) {
+      if (be->noalloc_slot < 0)
+        for (int s = 0; s < SLOTS; ++s)
+          if (!(g_slots_taken[be->device] & (1u << s))) {
+            g_slots_taken[be->device] |= 1u << s;
+            be->noalloc_slot = s;
+            break;
+          }
+      if (be->noalloc_slot >= 0 && g_scratch_ptr[be->device])
+        ptr = (uint32_t *)((unsigned char *)g_scratch_ptr[be->device] + (size_t)be->noalloc_slot * SCRATCH_BYTES);
+    }
   }
-  if (!ptr) return fail_with(be, CG_ERR_DEVICE, "cg_argmax_into: no scratch address for this device");
+  if (!ptr)
+    return fail_with(be, CG_ERR_DEVICE, "cg_argmax_into: every scratch slice of this device belongs to another live "
+                                        "backend (8 per device)");
   if (hipSetDevice(be->device) != hipSuccess) return fail_with(be, CG_ERR_DEVICE, "hipSetDevice failed");
   return cgrt::reduce_into(be, x->dtype == CG_F32 ? R_ARGMAX_F : R_ARGMAX_U, x, out, ptr, SCRATCH_BYTES);
 }

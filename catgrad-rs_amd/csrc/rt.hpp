@@ -77,6 +77,7 @@ struct PendingEvent {
 // Resolves, once per device and with that device current, the address of the library's fixed scratch
 // array; cg_backend_create calls it.
 int noalloc_init_device(int device);
+void noalloc_release_slot(int device, int slot);  // a destroyed backend's slice of the scratch array
 int reduce_into(cg_backend *be, int kind, cg_tensor *x, cg_tensor *out, uint32_t *scratch, size_t scratch_bytes);
 int fail_with(cg_backend *be, int code, const std::string &msg);
 bool tensor_is_contiguous(const cg_tensor *t);
@@ -137,6 +138,7 @@ struct cg_backend {
   // pattern kernels ran and how many launches fell to the generic programs ("ew_fused", "row_fused", ...)
   std::map<std::string, uint64_t> launch_counts;
   uint64_t uid = 0;  // distinct for every backend ever created in the process
+  int noalloc_slot = -1;  // cg_argmax_into: this backend's slice of its device's scratch array, taken at the first call
   // tracing
   bool trace = false;
   bool trace_shapes = false;  // cg_trace_enable(be, 2): matmul records carry their shape

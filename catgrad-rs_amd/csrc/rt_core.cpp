@@ -123,6 +123,7 @@ void backend_release(cg_backend *be) {
   if (be->h_words) (void)hipHostFree(be->h_words);
   delete be->queue;  // drains and joins its thread
   be->queue = nullptr;
+  noalloc_release_slot(be->device, be->noalloc_slot);
   if (be->stream) (void)hipStreamDestroy(be->stream);
   delete be;
 }

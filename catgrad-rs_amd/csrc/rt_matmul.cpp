@@ -426,12 +426,20 @@ int try_gemv_attn_merge(cg_backend *be, cg_tensor *n, cg_tensor *addend, bool *a
   if (w->stype != ST_F32 && w->stype != ST_BF16) return CG_OK;
   if ((uintptr_t)data_ptr(w) % 16 || w->strides[w->rank - 1] % (16 / esize(w->stype))) return CG_OK;
   if (addend && (addend->stype != ST_F32 || be->addend_is_row)) return CG_OK;
-  AttnMergeLater later;
-  bool att_done = false;
-  TRY(try_attn_decode(be, att, &att_done, &later));
-  if (!att_done || !later.deferred) return CG_OK;  // not an attention, or one that wrote its result: the usual path
+  if (att->shape[3] % 4) return CG_OK;  // (the merging prologue reads four values of a head at a time)
+  // Once the attention has stopped at its partials its own value is never written, so everything that can
+  // fail here comes first: the result's memory now; the launch's own checks are the conditions above plus the
+  // split count and geometry try_attn_decode only defers for.
   int st = alloc_result(be, n, ST_F32);
   if (st) return st;
+  AttnMergeLater later;
+  bool att_done = false;
+  st = try_attn_decode(be, att, &att_done, &later);
+  if (st || !att_done || !later.deferred) {  // not an attention, or one that wrote its result: the usual path
+    storage_release(n->st);
+    n->st = nullptr;
+    return st;
+  }
   GemvProDesc d;
   std::memset(&d, 0, sizeof(d));
   d.pro = PRO_ATTN_MERGE;

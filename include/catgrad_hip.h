@@ -160,10 +160,12 @@ int cg_argmax(cg_backend *be, cg_tensor *x, cg_tensor **out);
  * harnesses that forbid hipMalloc).  `x` must already be in memory (an uploaded tensor, or one passed
  * through cg_tensor_realize) and `out` a contiguous U32 tensor in memory shaped like x with a last
  * axis of 1; both stay the caller's.  The call makes no hipMalloc / hipFree and creates no handle: the
- * per-chunk accumulators of long rows that are split over workgroups go to a fixed 16 KiB array in the
- * library's device image (12 bytes per row and chunk; a shape needing more is refused with
- * CG_ERR_ARG).  Each GPU has one such array, shared by every backend on it and holding the last
- * call's contents: calls that overlap on one GPU race. */
+ * per-chunk accumulators of long rows that are split over workgroups go to a fixed 16 KiB slice of an
+ * array in the library's device image (12 bytes per row and chunk; a shape needing more is refused with
+ * CG_ERR_ARG).  Each GPU holds one such array of 8 slices (128 KiB); a backend takes a free slice of its
+ * device at its first call and keeps it until it is destroyed, so calls of different backends never share
+ * scratch memory and the calls of one backend are ordered by its stream; with all 8 slices of a device
+ * taken by live backends the call is refused (CG_ERR_DEVICE).  A slice keeps the last call's contents. */
 int cg_argmax_into(cg_backend *be, cg_tensor *x, cg_tensor *out);
 /* topk (mod.rs:58, ndarray.rs:248-257, 495-520): f32 only; values f32, indices u32 */
 int cg_topk(cg_backend *be, cg_tensor *x, size_t k, cg_tensor **values, cg_tensor **indices);

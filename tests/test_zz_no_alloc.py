@@ -69,3 +69,18 @@ def test_rejects_what_it_cannot_do_without_allocating(hip, cg):
         hip.argmax_into(x, hip.zeros((2, 1), cg.U32))                   # a constant, not memory
     hip.argmax_into(hip.realize(hip.add(x, x)), out)                    # realised beforehand: fine
     assert list(hip.to_vec(out)) == [63, 63]
+
+
+def test_two_backends_do_not_share_scratch(hip, hip_bf16, oracle):
+    """Every backend owns a slice of the device's scratch array: split reductions of two backends (two
+    streams), issued one behind the other without a wait in between, both give the right answer."""
+    rng = np.random.default_rng(9)
+    a_np = rng.standard_normal((1, 1, 128256)).astype(np.float32)
+    b_np = (rng.standard_normal((1, 1, 128256)).astype(np.float32).view(np.uint32) & 0xFFFF0000).view(np.float32)
+    a, b = hip.tensor(a_np), hip_bf16.tensor(b_np)
+    oa = hip.realize(hip.tensor(np.full((1, 1, 1), 0xFFFFFFFF, dtype=np.uint32) + np.zeros((1, 1, 1), np.uint32)))
+    ob = hip_bf16.realize(hip_bf16.tensor(np.full((1, 1, 1), 0xFFFFFFFF, dtype=np.uint32) + np.zeros((1, 1, 1), np.uint32)))
+    for _ in range(8):
+        hip.argmax_into(a, oa)
+        hip_bf16.argmax_into(b, ob)
+    assert hip.to_vec(oa)[0] == int(np.argmax(a_np)) and hip_bf16.to_vec(ob)[0] == int(np.argmax(b_np))
