@@ -63,6 +63,110 @@ __device__ __forceinline__ float wave_max(float v) {
   return v;
 }
 
+// The largest value over the 64 lanes of a wavefront (all active), in every lane: the exchanges of wave_sum
+// with a maximum in place of the sum (lanes a step does not write keep their own value).
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ int32_t dpp_max_i32(int32_t v) {
+  const int32_t o = __builtin_amdgcn_update_dpp(v, v, CTRL, ROW_MASK, 0xF, false);
+  return o > v ? o : v;
+}
+__device__ __forceinline__ int32_t wave_max_i32(int32_t v) {
+  v = dpp_max_i32<0xB1, 0xF>(v);
+  v = dpp_max_i32<0x4E, 0xF>(v);
+  v = dpp_max_i32<0x141, 0xF>(v);
+  v = dpp_max_i32<0x140, 0xF>(v);
+  v = dpp_max_i32<0x142, 0xA>(v);
+  v = dpp_max_i32<0x143, 0xC>(v);
+  return __builtin_amdgcn_readlane(v, 63);
+}
+
+// f32::total_cmp as an integer order
+__device__ __forceinline__ int32_t total_key_f(float v) {
+  int32_t b = __float_as_int(v);
+  return b ^ (int32_t)(((uint32_t)(b >> 31)) >> 1);
+}
+
+// topk(softmax(row)) by one wavefront (all 64 lanes active) over a row of n <= 64 * EPT values: the
+// probabilities exactly as softmax_kernel<64, EPT> computes them (same folds, same order), then k selection
+// rounds in the order of Backend::topk (ndarray.rs:495-520: descending, equal values by ascending index).
+// emit(t, value, index) is called in every lane, with the same arguments, for t = 0 .. k - 1.
+template <int EPT, typename Emit>
+__device__ __forceinline__ void softmax_topk_row(const float *xr, uint32_t n, uint32_t k, uint32_t lane, Emit emit) {
+  float v[EPT];
+  float mx = -3.40282347e+38f;  // max folds from f32::MIN (ndarray.rs:455-460)
+#pragma unroll
+  for (int e = 0; e < EPT; ++e) {
+    const uint32_t c = lane + e * 64;
+    if (c < n) {
+      v[e] = xr[c];
+      mx = fmaxf(mx, v[e]);
+    }
+  }
+  mx = wave_max(mx);
+  float sum = 0.f;
+#pragma unroll
+  for (int e = 0; e < EPT; ++e) {
+    const uint32_t c = lane + e * 64;
+    if (c < n) {
+      v[e] = expf(v[e] - mx);
+      sum += v[e];
+    }
+  }
+  sum = wave_sum(sum);
+#pragma unroll
+  for (int e = 0; e < EPT; ++e) v[e] = v[e] / sum;
+  int32_t prev_key = 0;
+  uint32_t prev_idx = 0;
+  if constexpr (EPT == 1) {
+    // a lane holds one value and its column is its lane: the largest eligible key by a wavefront maximum, the
+    // first lane that holds it by a ballot (no trips through the LDS crossbar)
+    const int32_t key = lane < n ? total_key_f(v[0]) : INT32_MIN;
+    for (uint32_t t = 0; t < k; ++t) {
+      const bool eligible = lane < n && (t == 0 || key < prev_key || (key == prev_key && lane > prev_idx));
+      const int32_t best = wave_max_i32(eligible ? key : INT32_MIN);
+      const unsigned long long holders = __ballot(eligible && key == best);
+      const uint32_t bi = holders ? (uint32_t)__builtin_ctzll(holders) : 0xFFFFFFFFu;
+      const float bv = holders ? __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v[0]), (int)(bi & 63u))) : 0.f;
+      prev_key = best;
+      prev_idx = bi;
+      emit(t, bv, bi);
+    }
+    return;
+  }
+  for (uint32_t t = 0; t < k; ++t) {
+    int32_t bk = 0;
+    uint32_t bi = 0xFFFFFFFFu;  // none
+    float bv = 0.f;
+#pragma unroll
+    for (int e = 0; e < EPT; ++e) {
+      const uint32_t c = lane + e * 64;
+      if (c < n) {
+        const int32_t key = total_key_f(v[e]);
+        const bool eligible = t == 0 || key < prev_key || (key == prev_key && c > prev_idx);
+        if (eligible && (bi == 0xFFFFFFFFu || key > bk || (key == bk && c < bi))) {
+          bk = key;
+          bi = c;
+          bv = v[e];
+        }
+      }
+    }
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) {
+      const int32_t ok = __shfl_xor(bk, m, 64);
+      const uint32_t oi = (uint32_t)__shfl_xor((int)bi, m, 64);
+      const float ov = __shfl_xor(bv, m, 64);
+      if (oi != 0xFFFFFFFFu && (bi == 0xFFFFFFFFu || ok > bk || (ok == bk && oi < bi))) {
+        bk = ok;
+        bi = oi;
+        bv = ov;
+      }
+    }
+    prev_key = bk;
+    prev_idx = bi;
+    emit(t, bv, bi);
+  }
+}
+
 // Sum over aligned groups of LANES lanes (a power of two, 2 .. 64); every lane of a group gets the sum.
 // The lanes of a group must be active together.
 template <int LANES>

@@ -1119,8 +1119,24 @@ __global__ void __launch_bounds__(256) gemv_pro_kernel(GemvProDesc g) {
   const TB *B2 = GLUEPI ? (const TB *)g.m.p[1].b : nullptr;
   const int64_t sbn2 = GLUEPI ? g.m.p[1].sbn : 0;
   if (g.b_index || g.slot_tokens) {
-    const uint32_t *bi = g.slot_tokens ? g.b_index_slot[sz] : g.b_index;
-    uint32_t ix = bi[(int64_t)tz * g.b_index_stride];
+    uint32_t ix = 0;
+    if (g.slot_tokens && g.router_logits) {
+      // the router's softmax and top-k for this token, by every wave alike
+      const bool writer = blockIdx.x == 0 && blockIdx.y == 0 && sz == 0 && wave == 0 && lane == 0;
+      const uint32_t want = g.router_col[sz];
+      softmax_topk_row<1>(g.router_logits + (int64_t)tz * g.router_stride, g.router_n, g.router_k, (uint32_t)lane,
+                          [&](uint32_t t, float bv, uint32_t bi) {
+                            if (t == want) ix = bi;
+                            if (writer) {
+                              g.router_values[(uint64_t)tz * g.router_k + t] = bv;
+                              g.router_indices[(uint64_t)tz * g.router_k + t] = bi;
+                            }
+                          });
+      ix = __builtin_amdgcn_readfirstlane(ix);
+    } else {
+      const uint32_t *bi = g.slot_tokens ? g.b_index_slot[sz] : g.b_index;
+      ix = bi[(int64_t)tz * g.b_index_stride];
+    }
     if (ix >= g.b_index_limit) {  // the reference's select() panics; flag it and stay in bounds
       atomicOr(g.err, ERRF_INDEX_OOB);
       ix = g.b_index_limit - 1;
@@ -1451,26 +1467,26 @@ uint32_t gemv_pro_multi_row_max_k(int b_stype) { return 64u * (b_stype == ST_BF1
 // of squares never leaves the wave - as PP 16-byte pieces per lane and row in registers; RMSNorm needs the
 // whole row at once (K <= 256 * PP), the elementwise prologues take K in several passes.
 enum { GEMV_ROWS_MAX = 16, GEMV_ROWS_LDS = 20480, GEMV_ROWS_TP = 264 };
+// The work of one workgroup: problem `prob` (GLUEPI: problems 0 and 1), groups first_group, first_group +
+// group_step, ...
 template <bool GLUEPI, int RS, int PP>
-__global__ void __launch_bounds__(256) gemv_rows_mfma_kernel(GemvProDesc g) {
+__device__ __forceinline__ void gemv_rows_mfma_body(const GemvProDesc &g, const uint32_t prob, const uint32_t first_group,
+                                                    const uint32_t group_step, uint16_t *xs,
+                                                    uint16_t (*turn)[16 * GEMV_ROWS_TP], float (*red)[16][17]) {
   typedef WVec<uint16_t>::type VT;
   constexpr int UN = 16;               // 16-byte loads in flight per lane: two windows of 8
   constexpr int CG = GLUEPI ? 8 : 16;  // output columns per group
-  __shared__ __attribute__((aligned(16))) uint16_t xs[GEMV_ROWS_LDS];  // [rows][K + 8] bf16
-  __shared__ __attribute__((aligned(16))) uint16_t turn[4][16 * GEMV_ROWS_TP];
-  __shared__ float red[4][16][17];
-  warm_kernel_arguments<sizeof(GemvProDesc)>();
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 15, kb = lane >> 4;
   const uint32_t K = g.m.K, rows = g.rows, pitch = K + 8;
-  const uint32_t N = g.m.p[blockIdx.y].N, groups = (N + CG - 1) / CG;
-  if (blockIdx.x >= groups) return;  // the narrower problems of a grouped launch
-  const uint16_t *B = (const uint16_t *)g.m.p[blockIdx.y].b;
+  const uint32_t N = g.m.p[prob].N, groups = (N + CG - 1) / CG;
+  if (first_group >= groups) return;  // the narrower problems of a grouped launch
+  const uint16_t *B = (const uint16_t *)g.m.p[prob].b;
   const uint16_t *B2 = GLUEPI ? (const uint16_t *)g.m.p[1].b : nullptr;
-  const int64_t sbn = g.m.p[blockIdx.y].sbn, sbn2 = GLUEPI ? g.m.p[1].sbn : 0;
-  float *C = g.m.p[blockIdx.y].c;
-  const float *Cadd = g.m.p[blockIdx.y].c_add;
-  const uint32_t cadd_rs = g.m.p[blockIdx.y].c_add_is_row ? 0u : N;
+  const int64_t sbn = g.m.p[prob].sbn, sbn2 = GLUEPI ? g.m.p[1].sbn : 0;
+  float *C = g.m.p[prob].c;
+  const float *Cadd = g.m.p[prob].c_add;
+  const uint32_t cadd_rs = g.m.p[prob].c_add_is_row ? 0u : N;
   const uint32_t kw = K / 4, k_begin = wave * kw;  // this wave's share of k
   const uint32_t nbatch = (kw + 511) / 512;        // requests (two windows of 256) per group
   const uint32_t lrow = lane >> 5, lk = (lane & 31) * 8;
@@ -1513,7 +1529,7 @@ __global__ void __launch_bounds__(256) gemv_rows_mfma_kernel(GemvProDesc g) {
 #pragma unroll
       for (int rs = 0; rs < RS; ++rs) xv[rs][i] = early_load(g.a + (int64_t)min(wave + 4u * rs, rows - 1) * g.a_rstride + k);
     }
-    request(blockIdx.x, 0);
+    request(first_group, 0);
     const float has_gamma = g.aux ? 1.f : 0.f, no_gamma = 1.f - has_gamma;
 #pragma unroll
     for (int rs = 0; rs < RS; ++rs) {
@@ -1575,7 +1591,7 @@ __global__ void __launch_bounds__(256) gemv_rows_mfma_kernel(GemvProDesc g) {
       }
     };
     load_pass(0);
-    request(blockIdx.x, 0);
+    request(first_group, 0);
     store_pass(0);
     for (uint32_t i0 = PP; i0 < ppr; i0 += PP) {
       load_pass(i0);
@@ -1587,7 +1603,7 @@ __global__ void __launch_bounds__(256) gemv_rows_mfma_kernel(GemvProDesc g) {
   const bool live = (uint32_t)r < rows;
   const uint16_t *xrow = xs + (size_t)min((uint32_t)r, rows - 1) * pitch + k_begin + kb * 8;
   uint16_t *mine = turn[wave];
-  for (uint32_t group = blockIdx.x; group < groups; group += gridDim.x) {
+  for (uint32_t group = first_group; group < groups; group += group_step) {
     f32x4n acc = {0.f, 0.f, 0.f, 0.f};
     for (uint32_t batch = 0; batch < nbatch; ++batch) {
       VT cur[UN];
@@ -1595,7 +1611,7 @@ __global__ void __launch_bounds__(256) gemv_rows_mfma_kernel(GemvProDesc g) {
       for (int u = 0; u < UN; ++u) cur[u] = q[u];
       // the next vectors - of this group, or the first of the workgroup's next group - while these multiply
       if (batch + 1 < nbatch) request(group, batch + 1);
-      else if (group + gridDim.x < groups) request(group + gridDim.x, 0);
+      else if (group + group_step < groups) request(group + group_step, 0);
 #pragma unroll
       for (int w2 = 0; w2 < 2; ++w2) {
         const uint32_t wk = (batch * 2 + w2) * 256;  // where the window starts in the wave's share of k
@@ -1635,6 +1651,31 @@ __global__ void __launch_bounds__(256) gemv_rows_mfma_kernel(GemvProDesc g) {
   }
 }
 
+// GLUEPI with glu_extra_blocks > 0: the first workgroups of the grid take one group each of the plain problems
+// 2, 3 (narrow products on the same input rows: a MoE block's router and the gate of its shared expert), with
+// the same prologue; the gated pair has as many workgroups fewer, so that the whole grid is resident at once.
+template <bool GLUEPI, int RS, int PP>
+__global__ void __launch_bounds__(256) gemv_rows_mfma_kernel(GemvProDesc g) {
+  __shared__ __attribute__((aligned(16))) uint16_t xs[GEMV_ROWS_LDS];  // [rows][K + 8] bf16
+  __shared__ __attribute__((aligned(16))) uint16_t turn[4][16 * GEMV_ROWS_TP];
+  __shared__ float red[4][16][17];
+  warm_kernel_arguments<sizeof(GemvProDesc)>();
+  if constexpr (GLUEPI) {
+    if (blockIdx.x >= g.glu_extra_blocks) {
+      gemv_rows_mfma_body<true, RS, PP>(g, 0u, blockIdx.x - g.glu_extra_blocks, gridDim.x - g.glu_extra_blocks, xs, turn, red);
+    } else {
+      uint32_t at = blockIdx.x, prob = 2;
+      while (prob + 1 < (uint32_t)g.m.n_prob && at >= (g.m.p[prob].N + 15) / 16) {
+        at -= (g.m.p[prob].N + 15) / 16;
+        ++prob;
+      }
+      gemv_rows_mfma_body<false, RS, PP>(g, prob, at, 0x40000000u, xs, turn, red);
+    }
+  } else {
+    gemv_rows_mfma_body<false, RS, PP>(g, blockIdx.y, blockIdx.x, gridDim.x, xs, turn, red);
+  }
+}
+
 // Whether the kernel above takes `rows` input rows of K values with prologue `pro`.
 bool gemv_rows_mfma_ok(int b_stype, uint32_t rows, uint32_t K, int pro) {
   if (b_stype != ST_BF16 || rows < 2 || rows > GEMV_ROWS_MAX || K < 128 || K % 128) return false;
@@ -1659,13 +1700,21 @@ static void launch_gemv_rows_mfma_as(const LaunchCtx &lc, const GemvProDesc &g, 
 }
 
 static hipError_t launch_gemv_rows_mfma(const LaunchCtx &lc, const GemvProDesc &g, uint32_t max_n) {
+  if (g.glu_epilogue) max_n = g.m.p[0].N;  // (further problems ride along as extra workgroups)
   const uint32_t groups = g.glu_epilogue ? (max_n + 7) / 8 : (max_n + 15) / 16;
   // two workgroups (77 KB of LDS each) per CU; a workgroup stages the rows once and walks its groups
   uint32_t cap = (uint32_t)lc.n_cus * 2 / (g.glu_epilogue ? 1 : g.m.n_prob);
   if (!cap) cap = 1;
   const uint32_t blocks = groups < cap ? groups : cap;
-  if (g.glu_epilogue) launch_gemv_rows_mfma_as<true>(lc, g, dim3(blocks, 1, 1));
-  else launch_gemv_rows_mfma_as<false>(lc, g, dim3(blocks, g.m.n_prob, 1));
+  if (g.glu_epilogue) {
+    GemvProDesc gg = g;
+    gg.glu_extra_blocks = 0;
+    for (int i = 2; i < g.m.n_prob; ++i) gg.glu_extra_blocks += (g.m.p[i].N + 15) / 16;
+    const uint32_t glu_blocks = blocks + gg.glu_extra_blocks > cap && blocks > gg.glu_extra_blocks ? cap - gg.glu_extra_blocks : blocks;
+    launch_gemv_rows_mfma_as<true>(lc, gg, dim3(glu_blocks + gg.glu_extra_blocks, 1, 1));
+  } else {
+    launch_gemv_rows_mfma_as<false>(lc, g, dim3(blocks, g.m.n_prob, 1));
+  }
   return hipGetLastError();
 }
 
@@ -1702,7 +1751,7 @@ hipError_t launch_gemv_pro(const LaunchCtx &lc, const GemvProDesc &g) {
   }
   const bool multi = g.rows > 1;  // several input rows share the weights
   if (multi && g.batch <= 1 && !g.b_index && !g.slot_tokens && gemv_rows_mfma_ok(g.m.b_stype, g.rows, g.m.K, g.pro)) {
-    if (g.glu_epilogue && (g.m.n_prob != 2 || g.m.p[0].N != g.m.p[1].N)) return hipErrorInvalidValue;
+    if (g.glu_epilogue && (g.m.n_prob < 2 || g.m.p[0].N != g.m.p[1].N)) return hipErrorInvalidValue;
     if ((uintptr_t)g.a % 16 || g.a_rstride % 4 || (g.aux && ((uintptr_t)g.aux % 16 || g.aux_rstride % 4))) return hipErrorInvalidValue;
     for (int i = 0; i < g.m.n_prob; ++i)
       if ((uintptr_t)g.m.p[i].b % 16 || g.m.p[i].sbn % 8) return hipErrorInvalidValue;

@@ -134,10 +134,6 @@ hipError_t launch_gather(const LaunchCtx &lc, const GatherDesc &g, uint64_t n_ou
   return hipGetLastError();
 }
 
-__device__ __forceinline__ int32_t total_key_f(float v) {
-  int32_t b = __float_as_int(v);
-  return b ^ (int32_t)(((uint32_t)(b >> 31)) >> 1);
-}
 
 // One wavefront per row.  Round t selects the t-th element of the order
 // (key descending, index ascending) = what a stable descending sort yields.
@@ -187,67 +183,12 @@ __global__ void __launch_bounds__(256) softmax_topk_kernel(const float *x, int64
                                                            uint32_t rows, uint32_t n, uint32_t k) {
   const uint32_t lane = threadIdx.x, row = blockIdx.x * 4 + threadIdx.y;
   if (row >= rows) return;  // the whole wave exits together
-  const float *xr = x + (int64_t)row * x_row_stride;
-  float v[EPT];
-  float mx = -3.40282347e+38f;  // max folds from f32::MIN (ndarray.rs:455-460)
-#pragma unroll
-  for (int e = 0; e < EPT; ++e) {
-    const uint32_t c = lane + e * 64;
-    if (c < n) {
-      v[e] = xr[c];
-      mx = fmaxf(mx, v[e]);
-    }
-  }
-  mx = wave_max(mx);
-  float sum = 0.f;
-#pragma unroll
-  for (int e = 0; e < EPT; ++e) {
-    const uint32_t c = lane + e * 64;
-    if (c < n) {
-      v[e] = expf(v[e] - mx);
-      sum += v[e];
-    }
-  }
-  sum = wave_sum(sum);
-#pragma unroll
-  for (int e = 0; e < EPT; ++e) v[e] = v[e] / sum;
-  int32_t prev_key = 0;
-  uint32_t prev_idx = 0;
-  for (uint32_t t = 0; t < k; ++t) {
-    int32_t bk = 0;
-    uint32_t bi = 0xFFFFFFFFu;  // none
-    float bv = 0.f;
-#pragma unroll
-    for (int e = 0; e < EPT; ++e) {
-      const uint32_t c = lane + e * 64;
-      if (c < n) {
-        const int32_t key = total_key_f(v[e]);
-        const bool eligible = t == 0 || key < prev_key || (key == prev_key && c > prev_idx);
-        if (eligible && (bi == 0xFFFFFFFFu || key > bk || (key == bk && c < bi))) {
-          bk = key;
-          bi = c;
-          bv = v[e];
-        }
-      }
-    }
-#pragma unroll
-    for (int m = 32; m >= 1; m >>= 1) {
-      const int32_t ok = __shfl_xor(bk, m, 64);
-      const uint32_t oi = (uint32_t)__shfl_xor((int)bi, m, 64);
-      const float ov = __shfl_xor(bv, m, 64);
-      if (oi != 0xFFFFFFFFu && (bi == 0xFFFFFFFFu || ok > bk || (ok == bk && oi < bi))) {
-        bk = ok;
-        bi = oi;
-        bv = ov;
-      }
-    }
-    prev_key = bk;
-    prev_idx = bi;
+  softmax_topk_row<EPT>(x + (int64_t)row * x_row_stride, n, k, lane, [&](uint32_t t, float bv, uint32_t bi) {
     if (lane == 0) {
       values[(uint64_t)row * k + t] = bv;
       indices[(uint64_t)row * k + t] = bi;
     }
-  }
+  });
 }
 
 hipError_t launch_softmax_topk(const LaunchCtx &lc, const float *x, int64_t x_row_stride, float *values, uint32_t *indices,

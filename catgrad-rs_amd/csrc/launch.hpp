@@ -354,7 +354,10 @@ struct GemvProDesc {
   float n_as_float, eps, gamma_offset;
   // 0, or PRO_SWIGLU / PRO_GEGLU: two problems of equal N (gate, up); a single output
   // p[0].c[n] = act(x . gate_n) * (x . up_n) replaces the two product vectors
+  // (several rows against bf16 weights on the matrix cores: problems 2 and 3, if any, are plain products of
+  // the same input rows, computed by glu_extra_blocks further workgroups - set by the launcher)
   int32_t glu_epilogue;
+  uint32_t glu_extra_blocks;
   uint32_t batch;   // 0 or 1: a single row
   int64_t a_bstride, aux_bstride;
   // 0 / 1, or several input rows that share the weights (gemv_pro_rows_ok; no batch, no b_index):
@@ -373,6 +376,16 @@ struct GemvProDesc {
   uint32_t slot_tokens;
   int32_t a_by_token;
   const uint32_t *b_index_slot[8];
+  // ... and the router's choice made here (router_logits != null: rows of router_n <= 64 logits, router_stride
+  // apart, one per token): every workgroup computes topk(softmax(row)) of its token - router_k <= 8 choices,
+  // as launch_softmax_topk would - and slot s reads choice router_col[s]; b_index_slot is unused.  One workgroup
+  // per token also stores the k values and indices (rows of router_k) for whoever reads them next.
+  const float *router_logits;
+  int64_t router_stride;
+  uint32_t router_n, router_k;
+  float *router_values;
+  uint32_t *router_indices;
+  uint8_t router_col[8];
   // PRO_ATTN_MERGE: the attention's partials (AttnDecodeDesc::part with merge_later) and their geometry
   const float *merge_part;
   uint32_t merge_splits, merge_heads, merge_d;

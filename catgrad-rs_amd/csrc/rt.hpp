@@ -58,8 +58,10 @@ enum NodeOp : uint8_t {
   N_REDUCE,     // p0 = ReduceKind
   N_CONCAT,     // p0 = dim
   N_INDEX,      // p0 = dim; in[0] = x, in[1] = indices
-  N_KSUM        // the k-slices of a split product, still to be summed: in[0] = the slices ([p0, size] floats),
+  N_KSUM,       // the k-slices of a split product, still to be summed: in[0] = the slices ([p0, size] floats),
                 // in[1] = a value added to the sum (or null); the node already owns the storage of the result
+  N_TOPK,       // p0 = k; in[0] = x: the k largest values of every row; `pair` is the node of their indices
+  N_TOPK_INDEX  // in[0] = the N_TOPK node: realised together with it
 };
 
 struct TraceRec {
@@ -106,6 +108,11 @@ struct cg_tensor {
   // `linear(x) + bias`: on a deferred few-row product, the add that reads it next to a broadcast bias
   // vector (a weak reference, cleared when that add lets go of its inputs); on the add, the product
   cg_tensor *bias_user = nullptr, *bias_of = nullptr;
+  // `act(gate_proj(x)) * up_proj(x)`: on a deferred few-row product, the multiplication that gates with it (a
+  // weak reference, cleared like bias_user); on that multiplication, the product
+  cg_tensor *glu_user = nullptr, *glu_of = nullptr;
+  // on a deferred N_TOPK node: its N_TOPK_INDEX node while that is alive (a weak reference)
+  cg_tensor *pair = nullptr;
   // a value that depends on nothing but constants and aranges (a causal mask, say); such nodes are
   // shared: cse_key is this node's entry in cg_backend::shared_nodes while it is still deferred
   bool const_like = false;

@@ -480,42 +480,25 @@ int cg_topk(cg_backend *be, cg_tensor *x, size_t k, cg_tensor **values, cg_tenso
   if (x->rank == 0) return fail(be, CG_ERR_SHAPE, "topk of a rank-0 tensor");
   const int64_t n = x->shape[x->rank - 1];
   if ((int64_t)k > n) return fail(be, CG_ERR_SHAPE, "topk: k larger than the last dimension");
-  HIPCHK(be, hipSetDevice(be->device));
-  // The router of a MoE layer: topk(softmax(logits)) where nobody else reads the probabilities (the
-  // caller's handle is the only reference) - both in one launch, the probabilities never stored.
-  cg_tensor *c = nullptr;
-  bool router = false;
-  SoftmaxMatch sm;
-  if (x->op != N_REAL && !(be->flags & (CG_FLAG_EAGER | CG_FLAG_NO_PATTERNS)) && refs(x) == 1 && n <= 256 && n > 0 &&
-      match_softmax(x, &sm) && !sm.has_scale && !sm.has_mask_const && !sm.mask && sm.src == sm.x) {
-    TRY(contiguous(be, sm.src, &c));
-    router = c->stype == ST_F32;
-    if (!router) {
-      node_release(c);
-      c = nullptr;
-    }
-  }
-  if (!router) TRY(contiguous(be, x, &c));
+  // Both results stay deferred (realize_topk) like any other value: what feeds the router - and what reads the
+  // chosen indices - is then realised with the whole block recorded.
   int64_t shape[CG_MAX_RANK];
   std::copy(x->shape, x->shape + x->rank, shape);
   shape[x->rank - 1] = (int64_t)k;
   cg_tensor *v = new_node(be, CG_F32, x->rank, shape), *ix = new_node(be, CG_U32, x->rank, shape);
-  int st = alloc_result(be, v, ST_F32);
-  if (!st) st = alloc_result(be, ix, ST_U32);
-  if (!st) {
-    const int64_t rows = n ? x->size() / n : 0;
-    KernelScope ks(be, router ? "softmax_topk" : "topk", (double)x->size() * 4, 0);
-    hipError_t e = router ? launch_softmax_topk(be->lc(), (const float *)data_ptr(c), n, (float *)v->st->ptr,
-                                                (uint32_t *)ix->st->ptr, (uint32_t)rows, (uint32_t)n, (uint32_t)k)
-                          : launch_topk(be->lc(), (const float *)data_ptr(c), (float *)v->st->ptr, (uint32_t *)ix->st->ptr,
-                                        (uint32_t)rows, (uint32_t)n, (uint32_t)k);
-    if (e != hipSuccess) st = fail(be, CG_ERR_DEVICE, hipGetErrorString(e));
-  }
-  node_release(c);
-  if (st) {
-    node_release(v);
-    node_release(ix);
-    return st;
+  v->op = N_TOPK;
+  v->p0 = (int64_t)k;
+  v->in[0] = retain(x);
+  ix->op = N_TOPK_INDEX;
+  ix->in[0] = retain(v);
+  v->pair = ix;
+  if (be->flags & CG_FLAG_EAGER) {
+    int st = realize(be, v);
+    if (st) {
+      node_release(ix);
+      node_release(v);
+      return st;
+    }
   }
   *values = v;
   *indices = ix;

@@ -177,6 +177,8 @@ void node_release(cg_tensor *t) {
     if (n->gemm_candidate) forget_gemm_candidate(n);
     forget_shared(n);
     if (n->bias_of && n->bias_of->bias_user == n) n->bias_of->bias_user = nullptr;  // its inputs are still alive here
+    if (n->glu_of && n->glu_of->glu_user == n) n->glu_of->glu_user = nullptr;
+    if (n->op == N_TOPK_INDEX && n->in[0] && n->in[0]->pair == n) n->in[0]->pair = nullptr;
     if (n->in[0]) stack.push_back(n->in[0]);
     if (n->in[1]) stack.push_back(n->in[1]);
     storage_release(n->st);
@@ -213,6 +215,10 @@ void drop_inputs(cg_tensor *n) {
   if (n->bias_of) {
     if (n->bias_of->bias_user == n) n->bias_of->bias_user = nullptr;
     n->bias_of = nullptr;
+  }
+  if (n->glu_of) {
+    if (n->glu_of->glu_user == n) n->glu_of->glu_user = nullptr;
+    n->glu_of = nullptr;
   }
   cg_tensor *a = n->in[0], *b = n->in[1];
   n->in[0] = n->in[1] = nullptr;

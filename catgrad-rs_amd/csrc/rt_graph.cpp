@@ -158,6 +158,60 @@ int realize_ksum(cg_backend *be, cg_tensor *n) {
 }
 
 
+// ndarray.rs:495-520.  The values node computes both results; the index node is filled with it.
+int realize_topk(cg_backend *be, cg_tensor *v) {
+  if (v->op == N_TOPK_INDEX) {
+    cg_tensor *vals = retain(v->in[0]);  // (letting go of the inputs below must not delete it mid-way)
+    int st = vals->op == N_TOPK ? realize_topk(be, vals) : CG_OK;
+    node_release(vals);
+    if (st) return st;
+    return v->op == N_REAL ? CG_OK : fail(be, CG_ERR_INTERNAL, "topk: indices without their values");
+  }
+  cg_tensor *x = v->in[0], *ix = v->pair;
+  const int64_t n = x->shape[x->rank - 1], k = v->p0;
+  HIPCHK(be, hipSetDevice(be->device));
+  // The router of a MoE layer: topk(softmax(logits)) where nobody else reads the probabilities - both in one
+  // launch, the probabilities never stored.
+  cg_tensor *c = nullptr;
+  bool router = false;
+  SoftmaxMatch sm;
+  if (x->op != N_REAL && !(be->flags & (CG_FLAG_EAGER | CG_FLAG_NO_PATTERNS)) && refs(x) == 1 && n <= 256 && n > 0 &&
+      match_softmax(x, &sm) && !sm.has_scale && !sm.has_mask_const && !sm.mask && sm.src == sm.x) {
+    TRY(contiguous(be, sm.src, &c));
+    router = c->stype == ST_F32;
+    if (!router) {
+      node_release(c);
+      c = nullptr;
+    }
+  }
+  if (!router) TRY(contiguous(be, x, &c));
+  Storage *spare = nullptr;  // nobody holds the indices any more
+  int st = alloc_result(be, v, ST_F32);
+  if (!st) st = ix ? alloc_result(be, ix, ST_U32) : dev_alloc(be, (size_t)std::max<int64_t>(v->size(), 1) * 4, &spare);
+  if (!st && v->size()) {
+    const int64_t rows = n ? x->size() / n : 0;
+    KernelScope ks(be, router ? "softmax_topk" : "topk", (double)x->size() * 4, 0);
+    uint32_t *ip = (uint32_t *)(ix ? ix->st->ptr : spare->ptr);
+    hipError_t e = router ? launch_softmax_topk(be->lc(), (const float *)data_ptr(c), n, (float *)v->st->ptr, ip, (uint32_t)rows,
+                                                (uint32_t)n, (uint32_t)k)
+                          : launch_topk(be->lc(), (const float *)data_ptr(c), (float *)v->st->ptr, ip, (uint32_t)rows, (uint32_t)n,
+                                        (uint32_t)k);
+    if (e != hipSuccess) st = fail(be, CG_ERR_DEVICE, hipGetErrorString(e));
+  }
+  node_release(c);
+  storage_release(spare);
+  if (st) return st;
+  v->op = N_REAL;
+  v->pair = nullptr;
+  drop_inputs(v);
+  if (ix) {
+    ix->op = N_REAL;
+    drop_inputs(ix);
+  }
+  return CG_OK;
+}
+
+
 int realize(cg_backend *be, cg_tensor *n) {
   switch (n->op) {
     case N_REAL: return CG_OK;
@@ -174,6 +228,8 @@ int realize(cg_backend *be, cg_tensor *n) {
     case N_CONCAT: return realize_concat(be, n);
     case N_INDEX: return realize_index(be, n);
     case N_KSUM: return realize_ksum(be, n);
+    case N_TOPK:
+    case N_TOPK_INDEX: return realize_topk(be, n);
   }
   return fail(be, CG_ERR_INTERNAL, "realize: unknown node");
 }
@@ -423,6 +479,16 @@ int binary(cg_backend *be, cg_tensor *a, cg_tensor *b, cg_tensor **out, EwOp f_o
         n->bias_of = mm;
         break;
       }
+    }
+  }
+  // `act(gate_proj(x)) * up_proj(x)` on a few rows: the gate's product can be asked which multiplication it
+  // gates (the launch of a sibling product on the same rows may take the pair along)
+  if (n->ew == E_MUL_F && !(be->flags & (CG_FLAG_EAGER | CG_FLAG_NO_PATTERNS))) {
+    cg_tensor *g = glu_gate_of(n);
+    if (g && g->op == N_RESHAPE && g->in[0]) g = g->in[0];
+    if (g && g->op == N_MATMUL && g->gemv_candidate && !g->glu_user) {
+      g->glu_user = n;
+      n->glu_of = g;
     }
   }
   TRY(finish(be, n, out));

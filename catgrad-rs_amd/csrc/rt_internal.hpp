@@ -126,6 +126,7 @@ cg_tensor *node_under_repeat_kv(cg_tensor *t);
 bool is_sigmoid_of(const cg_tensor *s, const cg_tensor **arg);
 bool is_gelu_of(const cg_tensor *g, const cg_tensor **arg);
 bool match_glu(cg_tensor *root, cg_tensor **gate, cg_tensor **up, int *gelu);
+cg_tensor *glu_gate_of(const cg_tensor *root);
 bool same_rows(const cg_tensor *a, const cg_tensor *b);
 int try_glu(cg_backend *be, cg_tensor *root, bool *done);
 int try_gemv_add(cg_backend *be, cg_tensor *root, bool *done);
@@ -161,6 +162,7 @@ int try_attn_decode(cg_backend *be, cg_tensor *n, bool *done, AttnMergeLater *la
 int try_gemv_attn_merge(cg_backend *be, cg_tensor *n, cg_tensor *addend, bool *added, bool *done);
 cg_tensor *rows_base(cg_tensor *t);
 int try_gate_up_glu(cg_backend *be, cg_tensor *glu, cg_tensor *g, cg_tensor *u, int gelu, bool *done);
+bool norm_row_readers_ok(cg_backend *be, cg_tensor *base, cg_tensor *view, RmsNormMatch *rm);
 int try_gemv_prologue(cg_backend *be, cg_tensor *n, cg_tensor *addend, bool *added, bool *done);
 bool match_expert_operand(const cg_tensor *t, int64_t S, ExpertOperand *o);
 int try_moe_gemm(cg_backend *be, cg_tensor *n, bool *done);

@@ -150,6 +150,82 @@ cg_tensor *rows_base(cg_tensor *t) {
 }
 
 
+// A deferred RMSNorm row A (or a reshape of one that regroups its rows) whose every reader can compute the norm
+// on its own way in, so that the norm needs no launch and its value is never stored: few-row products reading
+// A directly - at most one gated pair (`glu`, with its gate and up products) and narrow plain ones - and
+// expert-indexed products reading it through one view (a MoE block's post-attention norm: router, shared
+// expert, routed experts; models/qwen3.rs:64-133, models/deepseek.rs:163-165).  A reader that does not take
+// the prologue after all realises A like any other value; the others still compute the same numbers.
+struct NormReaders {
+  cg_tensor *norm = nullptr;
+  RmsNormMatch rm;
+  std::vector<cg_tensor *> plain;
+  cg_tensor *glu = nullptr, *gate = nullptr, *up = nullptr;
+  int gelu = 0;
+  cg_tensor *view = nullptr;
+};
+static bool keeps_rows(const cg_tensor *v, const cg_tensor *of) {
+  if (!v->in[0] || v->in[0] != of || v->rank < 1 || of->rank < 1 || v->size() != of->size() ||
+      v->shape[v->rank - 1] != of->shape[of->rank - 1])
+    return false;
+  if (v->op == N_RESHAPE) return true;
+  // a transpose that moves an axis of extent 1 among the leading axes
+  if (v->op != N_TRANSPOSE || v->p0 == v->rank - 1 || v->p1 == v->rank - 1) return false;
+  return of->shape[v->p0] == 1 || of->shape[v->p1] == 1;
+}
+static bool norm_readers(cg_backend *be, cg_tensor *A, NormReaders *o) {
+  if (A->op == N_REAL || A->dtype != CG_F32 || A->rank < 1) return false;
+  cg_tensor *norm = A;
+  if (A->op == N_RESHAPE && A->in[0] && A->in[0]->op != N_REAL && refs(A->in[0]) == 1 && keeps_rows(A, A->in[0])) norm = A->in[0];
+  if (!match_rmsnorm(norm, &o->rm)) return false;
+  o->norm = norm;
+  int accounted = 0, view_readers = 0;
+  for (cg_tensor *c : be->gemv_candidates) {
+    if (c->op != N_MATMUL || !c->in[0]) continue;
+    cg_tensor *in = c->in[0];
+    if (rows_base(in) == A) {
+      ++accounted;
+      if (c->glu_user) {
+        if (o->glu) return false;
+        o->glu = c->glu_user;
+      } else {
+        o->plain.push_back(c);
+      }
+    } else if (in->op != N_REAL && keeps_rows(in, A)) {
+      ExpertOperand eo;
+      if ((o->view && o->view != in) || c->rank != 3 || !match_expert_operand(c->in[1], c->shape[0], &eo)) return false;
+      if (!o->view) ++accounted;
+      o->view = in;
+      ++view_readers;
+    }
+  }
+  if (o->view && refs(o->view) != view_readers) return false;
+  if (o->glu) {
+    if (!match_glu(o->glu, &o->gate, &o->up, &o->gelu)) return false;
+    cg_tensor *um = rows_base(o->up);
+    bool found = false;
+    for (size_t i = 0; i < o->plain.size(); ++i)
+      if (o->plain[i] == um) {
+        o->plain.erase(o->plain.begin() + i);
+        found = true;
+        break;
+      }
+    if (!found) return false;
+  }
+  return accounted == refs(A);
+}
+
+
+// `view` (of `base`) is read by expert-indexed products only, and every other reader of `base` computes the
+// RMSNorm that `base` is on its own way in: so may these products.
+bool norm_row_readers_ok(cg_backend *be, cg_tensor *base, cg_tensor *view, RmsNormMatch *rm) {
+  NormReaders nr;
+  if (!norm_readers(be, base, &nr) || nr.view != view) return false;
+  *rm = nr.rm;
+  return true;
+}
+
+
 // h = act(gate_proj(x)) * up_proj(x) with one input row (models/llama.rs:11-35): both products and the
 // activation in one launch, a wave computing column n of gate and of up (and x itself from its
 // RMSNorm when nothing else reads the normed row).  `glu` is the deferred act(g) * u node; on
@@ -182,8 +258,33 @@ int try_gate_up_glu(cg_backend *be, cg_tensor *glu, cg_tensor *g, cg_tensor *u, 
   std::memset(&d, 0, sizeof(d));
   RmsNormMatch rm;
   cg_tensor *a0 = nullptr, *a1 = nullptr;
-  if (X->op != N_REAL && refs(X) == 2 && gemv_pro_rows_ok(ws[0]->stype, (uint32_t)rows, (uint32_t)K, PRO_RMSNORM) &&
-      match_rmsnorm(X, &rm)) {
+  // narrow plain products on the same rows ride along (the matrix-core form only), and with them the norm may
+  // have further readers that compute it themselves
+  std::vector<cg_tensor *> extras;
+  bool shared_norm = false;
+  if (X->op != N_REAL && refs(X) > 2 && rows > 1 && ws[0]->stype == ST_BF16 &&
+      gemv_rows_mfma_ok(ST_BF16, (uint32_t)rows, (uint32_t)K, PRO_RMSNORM)) {
+    NormReaders nr;
+    if (norm_readers(be, X, &nr) && nr.glu == glu && nr.plain.size() <= 2) {
+      shared_norm = true;
+      for (cg_tensor *c : nr.plain) {
+        cg_tensor *w = c->in[1];
+        const int64_t nc = w->rank >= 2 ? w->shape[w->rank - 1] : 0;
+        TRY(realize(be, w));
+        bool ok = w->rank >= 2 && w->shape[w->rank - 2] == K && nc >= 1 && nc < 64 && c->size() == rows * nc && c->dtype == CG_F32 &&
+                  w->stype == ST_BF16 && w->strides[w->rank - 2] == 1 && (uintptr_t)data_ptr(w) % 16 == 0 &&
+                  (nc == 1 || w->strides[w->rank - 1] % 8 == 0) && !c->bias_user;
+        for (int i = 0; ok && i + 2 < w->rank; ++i) ok = w->shape[i] == 1 || w->strides[i] == 0;
+        shared_norm = shared_norm && ok;
+      }
+      if (shared_norm) {
+        extras = nr.plain;
+        rm = nr.rm;
+      }
+    }
+  }
+  if (X->op != N_REAL && (shared_norm || refs(X) == 2) && gemv_pro_rows_ok(ws[0]->stype, (uint32_t)rows, (uint32_t)K, PRO_RMSNORM) &&
+      (shared_norm || match_rmsnorm(X, &rm))) {
     bool vec = true;
     if (rm.gamma) TRY(gamma_row_vector(be, rm.gamma, &vec));
     TRY(realize(be, rm.x));
@@ -196,6 +297,7 @@ int try_gate_up_glu(cg_backend *be, cg_tensor *glu, cg_tensor *g, cg_tensor *u, 
       d.gamma_offset = rm.gamma_offset;
     }
   }
+  if (!a0) extras.clear();  // (the row is realised below, for every reader)
   if (!a0) {
     TRY(contiguous(be, X, &a0));
     if (a0->stype != ST_F32 || (uintptr_t)data_ptr(a0) % 16) {
@@ -205,6 +307,7 @@ int try_gate_up_glu(cg_backend *be, cg_tensor *glu, cg_tensor *g, cg_tensor *u, 
     d.pro = PRO_NONE;
   }
   int st = alloc_result(be, glu, ST_F32);
+  for (size_t i = 0; i < extras.size() && !st; ++i) st = alloc_result(be, extras[i], ST_F32);
   if (!st) {
     d.a = (const float *)data_ptr(a0);
     d.aux = a1 ? (const float *)data_ptr(a1) : nullptr;
@@ -220,14 +323,26 @@ int try_gate_up_glu(cg_backend *be, cg_tensor *glu, cg_tensor *g, cg_tensor *u, 
       d.m.p[i].sbn = ws[i]->strides[ws[i]->rank - 1];
       d.m.p[i].N = (uint32_t)N;
     }
+    double extra_bytes = 0, extra_flops = 0;
+    for (cg_tensor *c : extras) {
+      cg_tensor *w = c->in[1];
+      auto &pr = d.m.p[d.m.n_prob++];
+      pr.b = data_ptr(w);
+      pr.c = (float *)c->st->ptr;
+      pr.N = (uint32_t)w->shape[w->rank - 1];
+      pr.sbn = pr.N > 1 ? w->strides[w->rank - 1] : K;  // (the stride between columns of a single column is never used)
+      extra_bytes += (double)pr.N * K * 2 + (double)rows * pr.N * 4;
+      extra_flops += 2.0 * rows * pr.N * K;
+    }
     const char *base = rows > 1 && gemv_rows_mfma_ok(ws[0]->stype, (uint32_t)rows, (uint32_t)K, d.pro) ? "gemv_rows_bf16"
                        : ws[0]->stype == ST_BF16                                                          ? "gemv_rowdot_bf16"
                                                                                                           : "gemv_rowdot_f32";
-    KernelScope ks(be, base, 2.0 * N * K * esize(ws[0]->stype) + (double)rows * (K * 8 + N * 4), 4.0 * rows * N * K);
+    KernelScope ks(be, base, 2.0 * N * K * esize(ws[0]->stype) + (double)rows * (K * 8 + N * 4) + extra_bytes,
+                   4.0 * rows * N * K + extra_flops);
     if (be->trace_shapes) {
       char buf[96];
-      snprintf(buf, sizeof buf, "%s[%sgate*up,M%lld,K%lld,N%lld]", base, d.pro == PRO_RMSNORM ? "rmsnorm+" : "", (long long)rows,
-               (long long)K, (long long)(2 * N));
+      snprintf(buf, sizeof buf, "%s[%sgate*up%s,M%lld,K%lld,N%lld]", base, d.pro == PRO_RMSNORM ? "rmsnorm+" : "",
+               extras.empty() ? "" : "+narrow", (long long)rows, (long long)K, (long long)(2 * N));
       ks.rename(buf);
     }
     hipError_t e = launch_gemv_pro(be->lc(), d);
@@ -236,8 +351,29 @@ int try_gate_up_glu(cg_backend *be, cg_tensor *glu, cg_tensor *g, cg_tensor *u, 
   node_release(a0);
   node_release(a1);
   if (st) return st;
+  for (cg_tensor *c : extras) {
+    forget_gemv_candidate(c);
+    c->op = N_REAL;
+    drop_inputs(c);
+  }
   finish_fused(glu);  // releases the activation chain and with it g and u
   *done = true;
+  return CG_OK;
+}
+
+
+// A narrow product on the rows of a norm that a gated pair reads too (a MoE block's router, reached before its
+// shared expert): the pair's launch takes it along.
+int try_norm_reader_group(cg_backend *be, cg_tensor *n, bool *done) {
+  if (!n->gemv_candidate || !n->in[0] || !(be->flags & CG_FLAG_BF16)) return CG_OK;
+  cg_tensor *A = rows_base(n->in[0]);
+  if (A->op == N_REAL || refs(A) < 3) return CG_OK;
+  NormReaders nr;
+  if (!norm_readers(be, A, &nr) || !nr.glu) return CG_OK;
+  if (std::find(nr.plain.begin(), nr.plain.end(), n) == nr.plain.end()) return CG_OK;
+  bool fused = false;
+  TRY(try_gate_up_glu(be, nr.glu, nr.gate, nr.up, nr.gelu, &fused));
+  *done = fused && n->op == N_REAL;
   return CG_OK;
 }
 
@@ -494,6 +630,8 @@ int realize_matmul(cg_backend *be, cg_tensor *n, cg_tensor *addend, bool *added,
   if (n->dtype == CG_F32 && n->gemv_candidate && !(be->flags & CG_FLAG_NO_PATTERNS)) {
     bool done = false;
     if (!addend) TRY(try_moe_gemv(be, n, &done));
+    if (done) return CG_OK;
+    if (!addend) TRY(try_norm_reader_group(be, n, &done));
     if (done) return CG_OK;
     TRY(try_gemv_prologue(be, n, addend, added, &done));
     if (done) return CG_OK;

@@ -399,9 +399,45 @@ int try_moe_gemv_slots(cg_backend *be, cg_tensor *n, bool *done) {
   if (!has_n) return CG_OK;
   GemvProDesc d;
   std::memset(&d, 0, sizeof(d));
+  // The indices may be the router's choice that nothing has computed yet - column i of topk(softmax(logits))
+  // for slot i (models/qwen3.rs:64-80) - and then this launch makes the choice itself, token by token, and
+  // leaves values and indices in memory for their other readers: the router needs no launch of its own.
+  cg_tensor *topk_ix = nullptr;
+  SoftmaxMatch rsm;
+  if (!glu) {
+    bool fold = true;
+    for (const Member &m : members) {
+      cg_tensor *t = m.idx;
+      int64_t col = -1;
+      while (fold && t->op != N_TOPK_INDEX) {
+        if (t->op == N_RESHAPE && t->in[0] && t->in[0]->size() == t->size()) {
+          t = t->in[0];
+        } else if (t->op == N_SLICE && col < 0 && t->in[0] && t->p0 == t->rank - 1 && t->shape[t->rank - 1] == 1 && t->size() == S) {
+          col = t->p1;  // one column of rows of choices
+          t = t->in[0];
+        } else {
+          fold = false;
+        }
+      }
+      if (!fold) break;
+      if (topk_ix && t != topk_ix) fold = false;
+      topk_ix = t;
+      const int64_t k = t->shape[t->rank - 1];
+      if (col < 0 || col >= k || k > 8 || t->size() != S * k || m.slot >= 8) fold = false;
+      else d.router_col[m.slot] = (uint8_t)col;
+    }
+    if (fold && topk_ix) {
+      cg_tensor *v = topk_ix->in[0], *x = v && v->op == N_TOPK ? v->in[0] : nullptr;
+      const int64_t ne = x ? x->shape[x->rank - 1] : 0;
+      fold = x && x->op != N_REAL && refs(x) == 1 && ne >= 1 && ne <= 64 && x->size() == S * ne && match_softmax(x, &rsm) &&
+             !rsm.has_scale && !rsm.has_mask_const && !rsm.mask && rsm.src == rsm.x;
+    }
+    if (!fold) topk_ix = nullptr;
+  }
   // indices: u32, one stride between consecutive tokens, the same stride in every slot
   int64_t istride0 = -1;
   for (const Member &m : members) {
+    if (topk_ix) break;
     cg_tensor *idx = m.idx;
     TRY(realize(be, idx));
     if (idx->dtype != CG_U32) return CG_OK;
@@ -426,14 +462,36 @@ int try_moe_gemv_slots(cg_backend *be, cg_tensor *n, bool *done) {
     const int q = 16 / esize(w->stype);
     if ((uintptr_t)data_ptr(w) % 16 || w->strides[1] % q || w->strides[0] % q) return CG_OK;
   }
+  cg_tensor *norm_x = nullptr;
   if (!glu) {
+    // the rows are an RMSNorm that every reader computes on its way in (norm_row_readers_ok): so does this launch
+    RmsNormMatch rm;
+    if (A->op != N_REAL && A->in[0] && norm_row_readers_ok(be, A->in[0], A, &rm) && gemv_pro_rows_ok(b_stype, 1, (uint32_t)K, PRO_RMSNORM)) {
+      bool vec = true;
+      if (rm.gamma) TRY(gamma_row_vector(be, rm.gamma, &vec));
+      TRY(realize(be, rm.x));
+      if (vec && rm.x->stype == ST_F32 && is_contiguous(rm.x) && (uintptr_t)data_ptr(rm.x) % 16 == 0 && rm.x->size() == S * K) {
+        norm_x = rm.x;
+        d.pro = PRO_RMSNORM;
+        d.a = (const float *)data_ptr(rm.x);
+        d.aux = rm.gamma ? (const float *)data_ptr(rm.gamma) : nullptr;
+        d.a_bstride = K;
+        d.aux_bstride = 0;
+        d.a_by_token = 1;
+        d.n_as_float = rm.n_as_float;
+        d.eps = rm.eps;
+        d.gamma_offset = rm.gamma_offset;
+      }
+    }
+  }
+  if (!glu && !norm_x) {
     TRY(realize(be, A));
     if (A->stype != ST_F32 || A->strides[2] != 1 || A->strides[0] % 4 || (uintptr_t)data_ptr(A) % 16) return CG_OK;
     d.pro = PRO_NONE;
     d.a = (const float *)data_ptr(A);
     d.a_bstride = A->strides[0];
     d.a_by_token = 1;
-  } else {
+  } else if (glu) {
     if ((uintptr_t)gs->ptr % 16 || (uintptr_t)us->ptr % 16) return CG_OK;
     d.pro = gelu ? PRO_GEGLU : PRO_SWIGLU;
     d.a = (const float *)gs->ptr;
@@ -470,11 +528,40 @@ int try_moe_gemv_slots(cg_backend *be, cg_tensor *n, bool *done) {
     bytes += (double)n_slot * S * N * (K * esize(w->stype) + 4);
     flops += 2.0 * n_slot * S * N * K;
   }
+  cg_tensor *logits = nullptr;
+  if (topk_ix) {
+    // the logits (their launch comes first), then both results of the top-k as values in memory that the launch
+    // below fills
+    cg_tensor *v = retain(topk_ix->in[0]);
+    int st = contiguous(be, rsm.src, &logits);
+    if (!st && logits->stype != ST_F32) st = fail(be, CG_ERR_INTERNAL, "router logits are not f32");
+    if (!st) st = alloc_result(be, v, ST_F32);
+    if (!st) st = alloc_result(be, topk_ix, ST_U32);
+    if (st) {
+      node_release(logits);
+      node_release(v);
+      drop_outs();
+      return st;
+    }
+    d.router_logits = (const float *)data_ptr(logits);
+    d.router_n = (uint32_t)logits->shape[logits->rank - 1];
+    d.router_stride = d.router_n;
+    d.router_k = (uint32_t)v->p0;
+    d.router_values = (float *)v->st->ptr;
+    d.router_indices = (uint32_t *)topk_ix->st->ptr;
+    v->op = N_REAL;
+    v->pair = nullptr;
+    drop_inputs(v);
+    topk_ix->op = N_REAL;
+    drop_inputs(topk_ix);
+    node_release(v);
+  }
   hipError_t e;
   {
     KernelScope ks(be, b_stype == ST_BF16 ? "gemv_experts_bf16" : "gemv_experts_f32", bytes, flops);
     e = launch_gemv_pro(be->lc(), d);
   }
+  node_release(logits);
   if (e != hipSuccess) {
     drop_outs();
     return fail(be, CG_ERR_DEVICE, hipGetErrorString(e));

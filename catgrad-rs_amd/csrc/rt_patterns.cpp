@@ -767,6 +767,17 @@ bool match_glu(cg_tensor *root, cg_tensor **gate, cg_tensor **up, int *gelu) {
 }
 
 
+// The gate of `act(gate) * up` by structure alone (no reference counts: while a term is being recorded the
+// caller still holds values that it lets go of before anything is realised), or null.
+cg_tensor *glu_gate_of(const cg_tensor *root) {
+  if (root->dtype != CG_F32 || !is_bin(root, E_MUL_F)) return nullptr;
+  const cg_tensor *act = root->in[0], *g = nullptr;
+  if (is_bin(act, E_MUL_F) && is_sigmoid_of(act->in[1], &g) && g == act->in[0]) return const_cast<cg_tensor *>(g);
+  if (is_gelu_of(act, &g)) return const_cast<cg_tensor *>(g);
+  return nullptr;
+}
+
+
 // the same tensor, or two reshapes of one tensor to one shape (each linear folds the batch into its rows itself)
 bool same_rows(const cg_tensor *a, const cg_tensor *b) {
   if (a == b) return true;
@@ -1000,6 +1011,18 @@ bool sum_term(cg_tensor *n, const cg_tensor *root, int64_t rows, int64_t d, SumT
       out->x = x;
       out->s = sc;  // a broadcast of values in memory is a view
       return true;
+    }
+    // the same still deferred: views, ending in a broadcast, of a value that takes a launch of its own whoever
+    // reads it (the values a top-k chose); the caller checks the strides once the views are realised
+    if (sc->op == N_BROADCAST && refs(sc) == 1) {
+      const cg_tensor *src = sc->in[0];
+      while ((src->op == N_RESHAPE || src->op == N_SLICE || src->op == N_TRANSPOSE || src->op == N_BROADCAST) && src->in[0])
+        src = src->in[0];
+      if ((src->op == N_TOPK || src->op == N_REAL) && src->dtype == CG_F32 && sc->in[0]->size() == rows) {
+        out->x = x;
+        out->s = sc;
+        return true;
+      }
     }
     const cg_tensor *arg = nullptr;
     if (sc->op == N_BROADCAST && refs(sc) == 1 && sc->in[0]->size() == rows && is_sigmoid_of(sc->in[0], &arg) &&

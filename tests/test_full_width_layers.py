@@ -73,9 +73,22 @@ def test_qwen_moe_full_width_bf16(hip_bf16, qwen_full):
     # a decode step of four rows after the cached prefill, fed the oracle's tokens
     g = qwen_runner(hip_bf16, cfg, P)
     g.prefill(prompts)
+    hip_bf16.launch_counts(reset=True)
     _, gl = g.step(gold["rounded_tokens"])
     e = parity.per_row_bf16(gold["rounded_step_logits"], hip_bf16.numpy(gl))
     assert np.all((e <= parity.RTOL_BF16) | exposed[:, -1]), e
+    # the launches of that step: eight per layer - q/k/v (with the input norm), attention, o_proj + residual,
+    # the shared expert's gate * up with the router and its gate riding along (each reader of the post-attention
+    # norm computes it itself), the shared down_proj, the routed experts' two stages (the first makes the router's
+    # softmax and top-k), the weighted sum - plus embedding rows, lm_head (with the final norm) and argmax
+    # (counted on a second step: the first one after a prefill moves the caches to storage with room to grow)
+    hip_bf16.launch_counts(reset=True)
+    tok, _ = g.step(gold["rounded_tokens"])
+    hip_bf16.to_vec(tok)
+    counts = hip_bf16.launch_counts(reset=True)
+    assert counts.get("softmax_topk", 0) == 0 and counts.get("rmsnorm_fused", 0) == 0, counts
+    assert counts.get("gemv_experts_bf16") == 2 * cfg.num_hidden_layers and counts.get("row_scaled_sum") == cfg.num_hidden_layers, counts
+    assert sum(counts.values()) == 8 * cfg.num_hidden_layers + 3, counts
 
 
 @pytest.fixture(scope="module")

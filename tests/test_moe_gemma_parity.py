@@ -553,4 +553,6 @@ def test_generic_program_launches_of_the_other_decoders(hip_bf16):
     counts = be.launch_counts(reset=True)
     assert sum(counts.get(k, 0) for k in be.GENERIC_PROGRAMS) == 0, counts
     assert counts.get("row_scaled_sum") == qcfg.num_hidden_layers, counts
-    assert counts.get("softmax_topk") == qcfg.num_hidden_layers and counts.get("attn_decode") == qcfg.num_hidden_layers
+    # (the router's softmax and top-k are made by the routed experts' first launch, the post-attention norm by
+    # each of its readers)
+    assert counts.get("softmax_topk", 0) == 0 and counts.get("attn_decode") == qcfg.num_hidden_layers, counts
