@@ -648,8 +648,10 @@ __global__ void __launch_bounds__(WR *WC * 64) gemm_bf16_dma_kernel(GemmDesc g) 
 #pragma unroll
           for (int e = 0; e < 16; ++e) {
             const float gt = acc[i][j][e];
+            // (the activation as the stdlib defines it when the f32 tile is stored too)
+            const float act = g.c ? (g.glu_kind ? gelu_ref(gt) : gt * sigmoid_ref(gt)) : (g.glu_kind ? gelu_fast(gt) : silu_fast(gt));
             T[(wm * WM + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3)) * TP + wn * OC + j * 32 + (lane & 31)] =
-                (g.glu_kind ? gelu_ref(gt) : gt * sigmoid_ref(gt)) * acc[i][TNH + j][e];
+                act * acc[i][TNH + j][e];
           }
     } else {
 #pragma unroll
@@ -1920,7 +1922,7 @@ __global__ void __launch_bounds__(256) moe_gemm_kernel(MoeGemmDesc g) {
             const uint64_t at = (uint64_t)(ent & 0xFFFFu) * N + col;
             if (NP == 2) {
               const float gt = acc[0][h][i];
-              const float hv = (g.fuse_glu == PRO_GEGLU ? gelu_ref(gt) : gt * sigmoid_ref(gt)) * acc[NP - 1][h][i];
+              const float hv = (g.fuse_glu == PRO_GEGLU ? gelu_fast(gt) : silu_fast(gt)) * acc[NP - 1][h][i];  // (leaves as bf16)
               g.slot[ent >> 16].h16[at] = (uint16_t)bf16_bits(hv);
             } else {
               g.slot[ent >> 16].c[prob][at] = acc[0][h][i];
@@ -2140,7 +2142,7 @@ __global__ void __launch_bounds__(256) moe_gemm_dma_kernel(MoeGemmDesc g) {
 #pragma unroll
           for (int i = 0; i < 16; ++i) {
             const float gt = acc[0][h][i];
-            const float hv = (g.fuse_glu == PRO_GEGLU ? gelu_ref(gt) : gt * sigmoid_ref(gt)) * acc[NP - 1][h][i];
+            const float hv = (g.fuse_glu == PRO_GEGLU ? gelu_fast(gt) : silu_fast(gt)) * acc[NP - 1][h][i];  // (leaves as bf16)
             T[(h * 32 + (i >> 2) * 8 + (lane >> 5) * 4 + (i & 3)) * TP + wave * 32 + (lane & 31)] = (uint16_t)bf16_bits(hv);
           }
     } else {
@@ -2559,6 +2561,26 @@ hipError_t launch_matmul(const LaunchCtx &lc_in, const GemmDesc &g, const char *
         // 256 x 256 tiles run one to a CU, 128 x 128 two to a CU: when the big tiles leave the last round of
         // workgroups mostly empty (320 tiles on 256 CUs), the small ones fill the machine better
         auto fill = [&](uint64_t tiles, uint64_t slots) { return (double)tiles / (double)((tiles + slots - 1) / slots * slots); };
+        // A deep product whose last round of big tiles would leave most CUs idle (Gemma's down_proj,
+        // 16384 x 1152 x 6912: 320 tiles): whole rounds over the leading rows, the remaining rows as a product of
+        // their own with the tiling that suits them (347 -> 307 us; with K = 1024 the second launch costs what
+        // the idle CUs did)
+        const uint64_t tiles_n = (g.N + 255) / 256, tiles_m = (g.M + 255) / 256;
+        const uint64_t lead_m = t256 / (uint64_t)lc.n_cus * (uint64_t)lc.n_cus / tiles_n;  // tile rows of the whole rounds
+        if (!g.n_group && batch == 1 && splits == 1 && g.K >= 2048 && fill(t256, (uint64_t)lc.n_cus) < 0.8 && lead_m >= 1 &&
+            lead_m < tiles_m && g.a_stype == ST_BF16) {
+          GemmDesc lead = gg, rest = g;
+          lead.M = (uint32_t)(lead_m * 256);
+          rest.M = g.M - lead.M;
+          rest.a = (const uint16_t *)g.a + (int64_t)lead.M * g.sam;
+          rest.c = g.c + (uint64_t)lead.M * g.N;
+          LaunchCtx first = lc, second = lc_in;
+          first.ev_stop = nullptr;
+          second.ev_start = nullptr;
+          e = launch_gemm_dma<256, 256, 2, 4>(first, lead, (uint32_t)(lead_m * tiles_n));
+          if (e != hipSuccess) return e;
+          return launch_matmul(second, rest, nullptr);
+        }
         if (!g.n_group && fill(t128, 2 * (uint64_t)lc.n_cus) > 1.15 * fill(t256, (uint64_t)lc.n_cus))
           e = launch_gemm_dma<128, 128, 2, 2>(lc, gg, (uint32_t)t128);
         else
