@@ -79,6 +79,8 @@ struct KeyTiles {
   }
 };
 
+constexpr float ATTN_MAX_SLACK = 8.0f;
+
 // BN keys per step; the K / V rows and the mask values of step i+1 are fetched into registers while
 // step i is being computed, so global latency is paid once per workgroup, not once per step.
 // NW waves of 32 queries each per workgroup (4, or 2 when that is what it takes to occupy the CUs).
@@ -238,7 +240,10 @@ __global__ void __launch_bounds__(NW * 64) attn_prefill_kernel(AttnPrefillDesc a
         }
       }
     tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-    const float m_new = fmaxf(m_run, tmax);
+    // The reference point of the exponentials only follows the maximum when that has moved by more than
+    // ATTN_MAX_SLACK: the quotient O / l at the end does not depend on it, weights of up to e^slack are as
+    // exact in f32 and bf16 as weights of up to 1, and O is rescaled on a few steps instead of on most.
+    const float m_new = tmax > m_run + ATTN_MAX_SLACK ? tmax : m_run;
     const float alpha = __expf(m_run - m_new);
     float psum = 0.f;
     a_bf16x8 pf[KT * 2];  // P^T as B fragments of the 16-key blocks
@@ -471,7 +476,10 @@ attn_prefill_keysplit_kernel(AttnPrefillDesc a) {
         }
       }
     tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-    const float m_new = fmaxf(m_run, tmax);
+    // The reference point of the exponentials only follows the maximum when that has moved by more than
+    // ATTN_MAX_SLACK: the quotient O / l at the end does not depend on it, weights of up to e^slack are as
+    // exact in f32 and bf16 as weights of up to 1, and O is rescaled on a few steps instead of on most.
+    const float m_new = tmax > m_run + ATTN_MAX_SLACK ? tmax : m_run;
     const float alpha = __expf(m_run - m_new);
     float psum = 0.f;
     a_bf16x8 pf[KT * 2];
