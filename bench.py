@@ -259,7 +259,7 @@ def main():
     if args.workload in ("qwen_moe", "gemma3"):
         mb = importlib.import_module("benchmarks.modelbench")
         if args.workload == "qwen_moe":
-            rec = mb.run_qwen_moe(lib, layers=args.layers or 24, steps=args.steps, warmup=args.warmup)
+            rec = mb.run_qwen_moe(lib, layers=args.layers or 24, steps=args.steps, warmup=args.warmup, count_experts=not args.profile_only)
         else:
             rec = mb.run_gemma3(lib, layers=args.layers or 26)
         print(json.dumps({"metric": rec.pop("workload"), "n_gpus": 1, "dtype": "bf16", "data": "synthetic", **rec}))

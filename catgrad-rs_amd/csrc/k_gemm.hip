@@ -1094,7 +1094,9 @@ hipError_t launch_gemv_multi(const LaunchCtx &lc, const GemvMultiDesc &g) {
 // f32::total_cmp, the last of equal values winning, like Backend::argmax (ndarray.rs:469-480) - and leaves
 // (key, column, any) in g.amax_part[wave of the grid]: the argmax over the row then only merges these records
 // instead of reading the row back.
-template <typename TB, bool KSPLIT, bool GLUEPI, int MR, int XV, bool MERGE = false, bool AMAX = false>
+// ROUTER (batched over MoE slots, one row, a plain product): the expert of a (slot, token) pair is chosen here, by
+// the softmax and top-k of the token's router logits (GemvProDesc::router_logits).
+template <typename TB, bool KSPLIT, bool GLUEPI, int MR, int XV, bool MERGE = false, bool AMAX = false, bool ROUTER = false>
 __global__ void __launch_bounds__(256) gemv_pro_kernel(GemvProDesc g) {
   typedef typename WVec<TB>::type VT;
   constexpr int EPL = WVec<TB>::EPL, UNROLL = 4, R = 2;
@@ -1122,7 +1124,7 @@ __global__ void __launch_bounds__(256) gemv_pro_kernel(GemvProDesc g) {
   const int64_t sbn2 = GLUEPI ? g.m.p[1].sbn : 0;
   if (g.b_index || g.slot_tokens) {
     uint32_t ix = 0;
-    if (g.slot_tokens && g.router_logits) {
+    if constexpr (ROUTER) {
       // the router's softmax and top-k for this token, by every wave alike
       const bool writer = blockIdx.x == 0 && blockIdx.y == 0 && sz == 0 && wave == 0 && lane == 0;
       const uint32_t want = g.router_col[sz];
@@ -1419,6 +1421,12 @@ static void launch_gemv_pro_block(const LaunchCtx &lc, const GemvProDesc &g, uin
   dim3 grid(blocks, g.m.n_prob, batch);
   const uint32_t xv = ((MR > 1 ? g.rows : 1u) * g.m.K / 4 + 255) / 256;  // 16-byte pieces of the input rows per thread
   if constexpr (!KSPLIT && MR == 1) {
+    if (g.router_logits) {  // (launch_gemv_pro has checked the form)
+      if (xv <= 2) CG_LAUNCH(lc, (gemv_pro_kernel<TB, false, false, 1, 2, false, false, true>), grid, 256, g);
+      else if (xv <= 4) CG_LAUNCH(lc, (gemv_pro_kernel<TB, false, false, 1, 4, false, false, true>), grid, 256, g);
+      else CG_LAUNCH(lc, (gemv_pro_kernel<TB, false, false, 1, 8, false, false, true>), grid, 256, g);
+      return;
+    }
     if (g.amax_part) {  // (launch_gemv_pro has checked gemv_pro_amax_records)
       if (xv <= 2) CG_LAUNCH(lc, (gemv_pro_kernel<TB, false, false, 1, 2, false, true>), grid, 256, g);
       else if (xv <= 4) CG_LAUNCH(lc, (gemv_pro_kernel<TB, false, false, 1, 4, false, true>), grid, 256, g);
@@ -1771,6 +1779,9 @@ hipError_t launch_gemv_pro(const LaunchCtx &lc, const GemvProDesc &g) {
   }
   const uint32_t slots = (max_n + 1) / 2;
   const bool ksplit = g.m.K >= 4096 && slots * (uint32_t)g.m.n_prob <= (uint32_t)lc.n_cus * 8;
+  if (g.router_logits && (multi || ksplit || !g.slot_tokens || g.amax_part || g.router_n < 1 || g.router_n > 64 || g.router_k < 1 ||
+                          g.router_k > 8 || g.router_k > g.router_n || !g.router_values || !g.router_indices))
+    return hipErrorInvalidValue;
   if (g.m.b_stype == ST_BF16) {
     if (multi) launch_gemv_pro_block<uint16_t, false, 4>(lc, g, slots);  // rows * K <= 8192: K < 4096
     else if (ksplit) launch_gemv_pro_block<uint16_t, true, 1>(lc, g, slots);

@@ -405,7 +405,7 @@ int try_moe_gemv_slots(cg_backend *be, cg_tensor *n, bool *done) {
   cg_tensor *topk_ix = nullptr;
   SoftmaxMatch rsm;
   if (!glu) {
-    bool fold = true;
+    bool fold = K < 4096;  // (deeper rows split k over the waves: another form of the kernel)
     for (const Member &m : members) {
       cg_tensor *t = m.idx;
       int64_t col = -1;
