@@ -483,8 +483,9 @@ template <int N> __device__ __forceinline__ void wait_vmcnt() {
   __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
 }
 
-// EPI: the product goes through LDS on its way out, so that the optional gate (C = act(gate) * product)
-// is read, and C and its bf16 copy are written, 16 bytes per lane along rows.
+// EPI: the MFMA operands change places, so that a lane holds four consecutive columns of a row of C: the optional
+// gate (C = act(gate) * product) is read, and C and its bf16 copy are written, 16 / 8 bytes per lane along rows,
+// straight from the accumulators.
 // NS stages of operand tiles in LDS: two when several workgroups share a CU (large problems, bound by
 // the L2 -> LDS rate), four when a CU holds one workgroup and every k-step would otherwise wait out a
 // full trip to HBM (few tiles, cold weights: the prefill-sized products).
@@ -595,7 +596,10 @@ __global__ void __launch_bounds__(WR *WC * 64) gemm_bf16_dma_kernel(GemmDesc g) 
       for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[ks & 1][i], bfr[ks & 1][j], acc[i][j], 0, 0, 0);
+          // (EPI: the product transposed - a lane then holds four consecutive columns of one row of C, which
+          // is what the epilogue stores, 16 bytes at a time, without a trip through LDS)
+          acc[i][j] = EPI ? __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[ks & 1][j], af[ks & 1][i], acc[i][j], 0, 0, 0)
+                          : __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[ks & 1][i], bfr[ks & 1][j], acc[i][j], 0, 0, 0);
       // Issue order within the slice: one LDS read behind each of the first MFMAs, so that the reads of
       // the next slice go out while the matrix pipe is busy instead of in a block during which it drains
       // (measured on 4096^3: 0.93 -> 1.06 PFLOP/s).
@@ -637,64 +641,49 @@ __global__ void __launch_bounds__(WR *WC * 64) gemm_bf16_dma_kernel(GemmDesc g) 
     atomicAdd(g.clock_ticks + 1, __builtin_amdgcn_s_memrealtime() - real0);
   }
   if constexpr (EPI) {
-    constexpr int TP = BNO + 4;  // row pitch of the staged tile (floats)
-    float *T = (float *)dma_smem;
-    __syncthreads();  // every wave is done with the operand stages
-    if constexpr (DUAL) {
+    // acc[i][j][e] = C[m0 + wm * WM + i * 32 + (lane & 31)][n0 + (this fragment's columns) + (e >> 2) * 8 + half * 4 + (e & 3)]:
+    // pieces of four columns (N % 4 == 0: a piece is inside or outside), the optional gate read the same way
+    constexpr int TJ = DUAL ? TNH : TN;
 #pragma unroll
-      for (int i = 0; i < TM; ++i)
+    for (int i = 0; i < TM; ++i) {
+      const uint32_t row = m0 + wm * WM + i * 32 + (lane & 31);
 #pragma unroll
-        for (int j = 0; j < TNH; ++j)
+      for (int j = 0; j < TJ; ++j) {
+        float4 gt[4];
+        uint64_t at[4];
+        bool live[4];
 #pragma unroll
-          for (int e = 0; e < 16; ++e) {
-            const float gt = acc[i][j][e];
-            // (the activation as the stdlib defines it when the f32 tile is stored too)
-            const float act = g.c ? (g.glu_kind ? gelu_ref(gt) : gt * sigmoid_ref(gt)) : (g.glu_kind ? gelu_fast(gt) : silu_fast(gt));
-            T[(wm * WM + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3)) * TP + wn * OC + j * 32 + (lane & 31)] =
-                act * acc[i][TNH + j][e];
-          }
-    } else {
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-#pragma unroll
-          for (int e = 0; e < 16; ++e)
-            T[(wm * WM + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3)) * TP + wn * WN + j * 32 + (lane & 31)] =
-                acc[i][j][e];
-    }
-    __syncthreads();
-    // four 16-byte pieces per thread and round: the gate values of a round are requested together, so a
-    // round waits for memory once (a store to C could alias Gate as far as the compiler knows, which
-    // would otherwise order every load behind the previous piece's stores)
-    constexpr int PIECES = BM_ * BNO / 4, ROUND = NW * 64 * 4;
-    for (int base = 0; base < PIECES; base += ROUND) {
-      float4 gt[4];
-      uint64_t at[4];
-      bool live[4];
-#pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const int idx = base + u * NW * 64 + tid, r = idx / (BNO / 4), c4 = (idx % (BNO / 4)) * 4;
-        const uint32_t row = m0 + r, col = n0 + c4;
-        live[u] = idx < PIECES && row < g.M && col < Nl;  // N % 4 == 0: a group of four columns is inside or outside
-        at[u] = (uint64_t)row * Nl + col;
-        if (!DUAL && Gate && live[u]) gt[u] = *(const float4 *)(Gate + at[u]);
-      }
-#pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        if (!live[u]) continue;
-        const int idx = base + u * NW * 64 + tid, r = idx / (BNO / 4), c4 = (idx % (BNO / 4)) * 4;
-        float4 v = *(const float4 *)(&T[r * TP + c4]);
-        if (!DUAL && Gate) {
-          if (g.glu_kind) {
-            v.x *= gelu_ref(gt[u].x); v.y *= gelu_ref(gt[u].y); v.z *= gelu_ref(gt[u].z); v.w *= gelu_ref(gt[u].w);
-          } else {
-            v.x *= gt[u].x * sigmoid_ref(gt[u].x); v.y *= gt[u].y * sigmoid_ref(gt[u].y);
-            v.z *= gt[u].z * sigmoid_ref(gt[u].z); v.w *= gt[u].w * sigmoid_ref(gt[u].w);
-          }
+        for (int q = 0; q < 4; ++q) {
+          const uint32_t col = n0 + (DUAL ? wn * OC : wn * WN) + j * 32 + q * 8 + half * 4;
+          live[q] = row < g.M && col < Nl;
+          at[q] = (uint64_t)row * Nl + col;
+          if (!DUAL && Gate && live[q]) gt[q] = *(const float4 *)(Gate + at[q]);
         }
-        if (!DUAL || g.c) *(float4 *)(C + at[u]) = v;
-        if (C16) *(uint2 *)(C16 + at[u]) = bf16_pack4(v);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          if (!live[q]) continue;
+          float4 v = make_float4(acc[i][j][q * 4], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3]);
+          if constexpr (DUAL) {
+            const float u0 = acc[i][TNH + j][q * 4], u1 = acc[i][TNH + j][q * 4 + 1], u2 = acc[i][TNH + j][q * 4 + 2],
+                        u3 = acc[i][TNH + j][q * 4 + 3];
+            if (g.c) {  // (the activation as the stdlib defines it when the f32 tile is stored too)
+              if (g.glu_kind) v = make_float4(gelu_ref(v.x) * u0, gelu_ref(v.y) * u1, gelu_ref(v.z) * u2, gelu_ref(v.w) * u3);
+              else v = make_float4(v.x * sigmoid_ref(v.x) * u0, v.y * sigmoid_ref(v.y) * u1, v.z * sigmoid_ref(v.z) * u2, v.w * sigmoid_ref(v.w) * u3);
+            } else {
+              if (g.glu_kind) v = make_float4(gelu_fast(v.x) * u0, gelu_fast(v.y) * u1, gelu_fast(v.z) * u2, gelu_fast(v.w) * u3);
+              else v = make_float4(silu_fast(v.x) * u0, silu_fast(v.y) * u1, silu_fast(v.z) * u2, silu_fast(v.w) * u3);
+            }
+          } else if (Gate) {
+            if (g.glu_kind) {
+              v.x *= gelu_ref(gt[q].x); v.y *= gelu_ref(gt[q].y); v.z *= gelu_ref(gt[q].z); v.w *= gelu_ref(gt[q].w);
+            } else {
+              v.x *= gt[q].x * sigmoid_ref(gt[q].x); v.y *= gt[q].y * sigmoid_ref(gt[q].y);
+              v.z *= gt[q].z * sigmoid_ref(gt[q].z); v.w *= gt[q].w * sigmoid_ref(gt[q].w);
+            }
+          }
+          if (!DUAL || g.c) *(float4 *)(C + at[q]) = v;
+          if (C16) *(uint2 *)(C16 + at[q]) = bf16_pack4(v);
+        }
       }
     }
     return;
@@ -714,8 +703,7 @@ __global__ void __launch_bounds__(WR *WC * 64) gemm_bf16_dma_kernel(GemmDesc g) 
 
 template <int BM_, int BN_, int WR, int WC, bool EPI = false, int NS = 2, bool DUAL = false>
 static hipError_t launch_gemm_dma(const LaunchCtx &lc, const GemmDesc &g, uint32_t grid) {
-  constexpr int stages = NS * (BM_ + BN_) * 64 * 2, staged_tile = EPI ? BM_ * ((DUAL ? BN_ / 2 : BN_) + 4) * 4 : 0;
-  constexpr int smem = stages > staged_tile ? stages : staged_tile;
+  constexpr int smem = NS * (BM_ + BN_) * 64 * 2;
   static bool configured = false;  // one attribute call per kernel and process
   if (!configured) {
     hipError_t e = hipFuncSetAttribute((const void *)gemm_bf16_dma_kernel<BM_, BN_, WR, WC, EPI, NS, DUAL>,
