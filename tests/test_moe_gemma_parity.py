@@ -357,6 +357,99 @@ def test_expert_slots_of_a_decode_step(request, oracle, dev_name, S, k):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("dev_name", ["hip", "hip_bf16"])
+@pytest.mark.parametrize("S,E,k", [(4, 60, 4), (1, 8, 2), (7, 64, 8), (3, 5, 5)])
+def test_router_choice_made_by_the_experts_launch(request, oracle, dev_name, S, E, k):
+    """The same block with its router (models/qwen3.rs:64-80): slot i reads column i of topk(softmax(logits)),
+    and the weights are the chosen probabilities.  With at most 64 experts the first expert launch makes the
+    choice itself - no router launch - and leaves values and indices for their other readers; both must be the
+    oracle's (exact ties between logits go to the lower index), whatever else reads them."""
+    import vectors
+    lang, nn = vectors.lang, vectors.nn
+    dev = request.getfixturevalue(dev_name)
+    F, H = 64, 128
+    g = np.random.default_rng(S * 100 + E + k)
+    x = g.standard_normal((S, 1, H)).astype(np.float32)
+    logits = (g.standard_normal((1, S, E)) * 2).astype(np.float32)
+    logits[0, 0, 1] = logits[0, 0, 3] = logits[0, 0].max() + 0.5        # a tie for the first choice of token 0
+    wg, wu = ((g.standard_normal((E, F, H)) * 0.1).astype(np.float32) for _ in range(2))
+    wd = (g.standard_normal((E, H, F)) * 0.1).astype(np.float32)
+    if dev_name == "hip_bf16":   # (arrays of two or more axes are stored as bf16 in this mode: the oracle gets the same values)
+        wg, wu, wd, logits = U_round(wg), U_round(wu), U_round(wd), U_round(logits)
+
+    def f(b, xv, lv, g_all, u_all, d_all):
+        xv = xv + xv - xv
+        lv = lv + lv - lv
+        vv, iv = lang.topk(b, k, nn.softmax(b, lv))
+        sh = lang.make_shape(b, S, k)
+        iv, vv = lang.reshape(b, sh, iv), lang.reshape(b, sh, vv)
+        total = None
+        for i in range(k):
+            slot = lang.get(b, 1, i, iv)
+            sel = lambda w: lang.transpose(b, 1, 2, lang.index(b, 0, slot, w))
+            gate = lang.matmul(b, xv, sel(g_all))
+            up = lang.matmul(b, xv, sel(u_all))
+            y = lang.matmul(b, nn.silu(b, gate) * up, sel(d_all))
+            wgt = lang.reshape(b, lang.shape(b, lang.get(b, 2, 0, y)), lang.get(b, 1, i, vv))
+            y = y * lang.broadcast(b, wgt, lang.shape(b, y))
+            total = y if total is None else total + y
+        return total, iv, vv
+    ref, ri, rv = vectors.run(oracle, f, 3, x, logits, wg, wu, wd)
+    dev.trace(True)
+    dev.trace_reset()
+    got, gi, gv = vectors.run(dev, f, 3, x, logits, wg, wu, wd)
+    rep = dev.trace_report()
+    dev.trace(False)
+    name = "gemv_experts_bf16" if dev_name == "hip_bf16" else "gemv_experts_f32"
+    launches = {n: v["launches"] for n, v in rep.items()}
+    assert launches.get(name) == 2 and "softmax_topk" not in launches and "topk" not in launches, launches
+    assert np.array_equal(gi, ri) and ri[0, 0] == 1 and ri[0, 1] == 3
+    assert np.allclose(gv, rv, rtol=1e-4, atol=1e-7)
+    tol = 2e-2 if dev_name == "hip_bf16" else 1e-4
+    assert np.max(np.abs(got - ref)) <= tol * np.abs(ref).max()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("norm_is_read_elsewhere", [False, True])
+def test_norm_computed_by_each_reader_of_a_moe_block(oracle, hip_bf16, norm_is_read_elsewhere):
+    """post-attention RMSNorm -> MoE block (qwen_moe.py `layer`) on the four rows of a decode step: when the router,
+    the shared expert's gate, the shared expert's gated pair and the routed experts are the norm's only readers,
+    each computes it on its way in and the norm has no launch; when anything else reads it too it is computed
+    once, in memory.  The same numbers either way."""
+    import vectors
+    lang = vectors.lang
+    cfg = MU.qwen_moe_config(num_hidden_layers=1, hidden_size=256, moe_intermediate_size=128,
+                             shared_expert_intermediate_size=256)
+    P = MU.qwen_moe_params(cfg, seed=31, std=0.2)
+    pre = "qwen_moe.model.layers.0."
+    P = {k: v for k, v in P.items() if k.startswith(pre + "mlp.") or k == pre + "post_attention_layernorm.weight"}
+    P[pre + "post_attention_layernorm.weight"] = (1 + 0.1 * np.random.default_rng(5).standard_normal(cfg.hidden_size)).astype(np.float32)
+    P16 = {k: (llm.random_init.bf16_round(v) if v.ndim >= 2 else v) for k, v in P.items()}
+    model = llm.qwen_moe.QwenMoeModel(cfg, 8)
+    x = np.random.default_rng(32).standard_normal((4, 1, cfg.hidden_size)).astype(np.float32)
+    root = lang.path(["qwen_moe", "model", "layers", 0])
+
+    def f(b, xv):
+        xv = xv + xv - xv
+        h = llm.helpers.rmsnorm(b, cfg.rms_norm_eps, root.extend(["post_attention_layernorm"]), xv)
+        folded, bb, ss = llm.qwen_moe.fold_batch(b, h)
+        y = llm.qwen_moe.unfold_batch(b, bb, ss, model.moe(b, root.extend(["mlp"]), folded)) + xv
+        return [y, h] if norm_is_read_elsewhere else [y]
+    n_out = 2 if norm_is_read_elsewhere else 1
+    ref = vectors.run(oracle, f, n_out, x, params=P16)
+    hip_bf16.launch_counts(reset=True)
+    got = vectors.run(hip_bf16, f, n_out, x, params=P)
+    counts = hip_bf16.launch_counts(reset=True)
+    for r, a in zip(ref, got):
+        assert a.shape == r.shape and np.max(np.abs(a - r)) <= 2e-2 * np.abs(r).max()
+    assert counts.get("rmsnorm_fused", 0) == (1 if norm_is_read_elsewhere else 0), counts
+    assert counts.get("gemv_experts_bf16") == 2 and counts.get("row_scaled_sum") == 1, counts
+    # the router and the shared expert's gate ride in the launch of the shared expert's gate * up, or - when the rows
+    # are in memory anyway - share a launch of their own; the router's choice is made by the first expert launch
+    assert counts.get("softmax_topk", 0) == 0 and counts.get("gemv_rows_bf16") == (2 if norm_is_read_elsewhere else 1), counts
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("routing", ["skewed", "two experts take every token", "1500 experts"])
 def test_expert_slots_sorted_by_expert(oracle, hip_bf16, routing):
     """The same block where both products have k a multiple of 64: the (slot, token) pairs are sorted by
