@@ -894,6 +894,20 @@ __global__ void __launch_bounds__(256) gemv_rowdot_kernel(GemmDesc g, int b_vec,
     for (int r = 0; r < R; ++r)
 #pragma unroll
       for (int m = 0; m < MROWS; ++m) acc[r][m] = 0.f;
+    // What is added at the end (a residual) is requested now, by every lane with its position clamped, so that
+    // it is there when the sums are: loaded where it is used it costs the launch one more trip to memory.
+    float cpre[R][MROWS];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+      for (int m = 0; m < MROWS; ++m) cpre[r][m] = 0.f;
+    if (Cadd) {
+#pragma unroll
+      for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int m = 0; m < MROWS; ++m)
+          cpre[r][m] = Cadd[(uint64_t)min((uint32_t)m, g.M - 1) * g.N + min(nb + r * CPW + col_in_wave, g.N - 1)];
+    }
     if (fast) {
       for (uint32_t k0 = k_begin + sub * EPL; k0 < k_end; k0 += LPR * EPL * UNROLL) {
         VT q[R][UNROLL];
@@ -972,7 +986,7 @@ __global__ void __launch_bounds__(256) gemv_rowdot_kernel(GemmDesc g, int b_vec,
             if (n < g.N && (uint32_t)m < g.M)
               C[(uint64_t)m * g.N + n] = ((red[0][r][m][col_in_wave] + red[1][r][m][col_in_wave]) +
                                           (red[2][r][m][col_in_wave] + red[3][r][m][col_in_wave])) +
-                                         (Cadd ? Cadd[(uint64_t)m * g.N + n] : 0.f);
+                                         cpre[r][m];
         }
       }
     } else if (sub == 0) {
@@ -982,7 +996,7 @@ __global__ void __launch_bounds__(256) gemv_rowdot_kernel(GemmDesc g, int b_vec,
 #pragma unroll
         for (int m = 0; m < MROWS; ++m)
           if (n < g.N && (uint32_t)m < g.M)
-            C[(uint64_t)m * g.N + n] = acc[r][m] + (Cadd ? Cadd[(uint64_t)m * g.N + n] : 0.f);
+            C[(uint64_t)m * g.N + n] = acc[r][m] + cpre[r][m];
       }
     }
   }
@@ -1300,6 +1314,18 @@ __global__ void __launch_bounds__(256) gemv_pro_kernel(GemvProDesc g) {
   }
   // ---- the products
   for (uint32_t nb = slot * CPS; nb < N; nb += n_slots * CPS) {  // uniform per workgroup when KSPLIT
+    // (what is added at the end is requested now, positions clamped: see gemv_rowdot_kernel)
+    float cpre[R][MR];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+      for (int m = 0; m < MR; ++m) cpre[r][m] = 0.f;
+    if (Cadd && !KSPLIT && !GLUEPI) {
+#pragma unroll
+      for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int m = 0; m < MR; ++m) cpre[r][m] = Cadd[(uint64_t)min((uint32_t)m, rows - 1) * cadd_rs + min(nb + r, N - 1)];
+    }
     float acc[R][MR];
 #pragma unroll
     for (int r = 0; r < R; ++r)
@@ -1368,7 +1394,7 @@ __global__ void __launch_bounds__(256) gemv_pro_kernel(GemvProDesc g) {
         for (int m = 0; m < MR; ++m)
           if ((uint32_t)m < rows && nb + r < N) {
             const uint64_t at = (uint64_t)m * N + nb + r;
-            const float v = acc[r][m] + (Cadd ? Cadd[(uint64_t)m * cadd_rs + nb + r] : 0.f);
+            const float v = acc[r][m] + cpre[r][m];
             C[at] = v;
             if (AMAX) {
               const int32_t b = __float_as_int(v), key = b ^ (int32_t)(((uint32_t)(b >> 31)) >> 1);
