@@ -493,9 +493,16 @@ template <int N> __device__ __forceinline__ void wait_vmcnt() {
 // wavefront holds the same columns of both products, and the tile that leaves is act(gate) * up,
 // 128 columns wide (BN_ = 256 counts the stacked rows): the gated MLP's two products and its
 // activation in one pass over the activations, neither product ever stored.
-template <int BM_, int BN_, int WR, int WC, bool EPI, int NS, bool DUAL = false>
+// BKM: B is k-major - [K, N] with unit stride along n, rows g.sbk apart (the right operand of a product of two
+// activations, ndarray.rs:549-615) - and is used where it lies: its tile travels as 64 k-rows of BN_ columns
+// (16-byte pieces of a row swizzled by (k & 3) << 2, so that the four rows a fragment read touches fall on
+// different banks), and the MFMA operand - eight consecutive k of one column per lane - comes out of LDS through
+// the transposing read (ds_read_b64_tr_b16: the 16 lanes of a group hand in four rows of 16 columns, lane c
+// receives column c of the four rows), two reads per fragment.
+template <int BM_, int BN_, int WR, int WC, bool EPI, int NS, bool DUAL = false, bool BKM = false>
 __global__ void __launch_bounds__(WR *WC * 64) gemm_bf16_dma_kernel(GemmDesc g) {
   constexpr int NW = WR * WC, BK = 64;
+  static_assert(!BKM || (!EPI && !DUAL && (BM_ / 8) % ((BM_ + BN_) / 8 / (WR * WC)) == 0), "k-major B: the plain product");
   constexpr int WM = BM_ / WR, WN = BN_ / WC, TM = WM / 32, TN = WN / 32;
   constexpr int BNO = DUAL ? BN_ / 2 : BN_;    // output columns of a tile
   constexpr int OC = BNO / WC, TNH = OC / 32;  // DUAL: output columns per wave, fragments per product
@@ -559,15 +566,23 @@ __global__ void __launch_bounds__(WR *WC * 64) gemm_bf16_dma_kernel(GemmDesc g) 
     const int q = wave * LPW + i;  // 8-row block of the stacked [A; B] tile
     const int R = q * 8 + (lane >> 3);
     const int c = (lane & 7) ^ ((R >> 1) & 7);
-    if (q * 8 < BM_) gp[i] = A + (int64_t)min(m0 + R, g.M - 1) * g.sam + k_begin + c * 8;
-    else if (DUAL) gp[i] = (R - BM_ < BNO ? B : B2) + (int64_t)min(n0 + (uint32_t)((R - BM_) % BNO), Nl - 1) * g.sbn + k_begin + c * 8;
+    if (q * 8 < BM_) {
+      gp[i] = A + (int64_t)min(m0 + R, g.M - 1) * g.sam + k_begin + c * 8;
+    } else if (BKM) {
+      // 1 KB of the B tile = 1024 / (2 BN_) k-rows; this lane's 16 bytes: row kr, physical piece pc
+      const int qb = q - BM_ / 8, kr = qb * (512 / BN_) + lane / (BN_ / 8), pc = lane % (BN_ / 8);
+      const uint32_t n = n0 + (uint32_t)((pc ^ ((kr & 3) << 2)) * 8);
+      gp[i] = B + (int64_t)(k_begin + kr) * g.sbk + min(n, Nl - 8);
+    } else if (DUAL) gp[i] = (R - BM_ < BNO ? B : B2) + (int64_t)min(n0 + (uint32_t)((R - BM_) % BNO), Nl - 1) * g.sbn + k_begin + c * 8;
     else gp[i] = B + (int64_t)min(n0 + (R - BM_), Nl - 1) * g.sbn + k_begin + c * 8;
   }
+  // (k-major B: a wave's loads are all A's or all B's, and B's step down 64 rows per stage)
+  const int64_t gp_step = BKM && wave * LPW * 8 >= BM_ ? (int64_t)BK * g.sbk : (int64_t)BK;
   auto issue = [&](int buf) {
 #pragma unroll
     for (int i = 0; i < LPW; ++i) {
       lds_dma16(gp[i], lds0 + buf * STAGE + (wave * LPW + i) * 1024);
-      gp[i] += BK;
+      gp[i] += gp_step;
     }
   };
   const int sw = (lane >> 1) & 7, half = lane >> 5;
@@ -581,9 +596,22 @@ __global__ void __launch_bounds__(WR *WC * 64) gemm_bf16_dma_kernel(GemmDesc g) 
         af[set][i] = *(const bf16x8 *)(&As[(wm * WM + i * 32 + (lane & 31)) * BK + p]);
 #pragma unroll
       for (int j = 0; j < TN; ++j) {
-        // DUAL: fragments [0, TNH) are this wave's gate columns, [TNH, TN) the same columns of up
-        const int brow = DUAL ? (j / TNH) * BNO + wn * OC + (j % TNH) * 32 : wn * WN + j * 32;
-        bfr[set][j] = *(const bf16x8 *)(&Bs[(brow + (lane & 31)) * BK + p]);
+        if constexpr (BKM) {
+          typedef short v4s __attribute__((ext_vector_type(4)));
+          const int r = (lane & 15) >> 2, col = wn * WN + j * 32 + ((lane >> 4) & 1) * 16 + (lane & 3) * 4;
+          const int at = (ks * 16 + half * 8 + r) * BN_ + (((col >> 3) ^ (r << 2)) << 3) + (col & 7);
+          union {
+            v4s q[2];
+            bf16x8 f;
+          } u;
+          u.q[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s *)(Bs + at));
+          u.q[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s *)(Bs + at + 4 * BN_));
+          bfr[set][j] = u.f;
+        } else {
+          // DUAL: fragments [0, TNH) are this wave's gate columns, [TNH, TN) the same columns of up
+          const int brow = DUAL ? (j / TNH) * BNO + wn * OC + (j % TNH) * 32 : wn * WN + j * 32;
+          bfr[set][j] = *(const bf16x8 *)(&Bs[(brow + (lane & 31)) * BK + p]);
+        }
       }
     };
     frags(0, 0);
@@ -701,17 +729,17 @@ __global__ void __launch_bounds__(WR *WC * 64) gemm_bf16_dma_kernel(GemmDesc g) 
     }
 }
 
-template <int BM_, int BN_, int WR, int WC, bool EPI = false, int NS = 2, bool DUAL = false>
+template <int BM_, int BN_, int WR, int WC, bool EPI = false, int NS = 2, bool DUAL = false, bool BKM = false>
 static hipError_t launch_gemm_dma(const LaunchCtx &lc, const GemmDesc &g, uint32_t grid) {
   constexpr int smem = NS * (BM_ + BN_) * 64 * 2;
   static bool configured = false;  // one attribute call per kernel and process
   if (!configured) {
-    hipError_t e = hipFuncSetAttribute((const void *)gemm_bf16_dma_kernel<BM_, BN_, WR, WC, EPI, NS, DUAL>,
+    hipError_t e = hipFuncSetAttribute((const void *)gemm_bf16_dma_kernel<BM_, BN_, WR, WC, EPI, NS, DUAL, BKM>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return e;
     configured = true;
   }
-  cg_launch(lc, gemm_bf16_dma_kernel<BM_, BN_, WR, WC, EPI, NS, DUAL>, dim3(grid), dim3(WR * WC * 64), smem, g);
+  cg_launch(lc, gemm_bf16_dma_kernel<BM_, BN_, WR, WC, EPI, NS, DUAL, BKM>, dim3(grid), dim3(WR * WC * 64), smem, g);
   return hipGetLastError();
 }
 
@@ -2394,6 +2422,14 @@ static bool gemm_dma_ok(const GemmDesc &g) {
   return g.sak == 1 && g.sbk == 1 && g.K % 64 == 0 && g.K >= 64 && g.M >= 64 && g.N >= 64;
 }
 
+// B [K, N] with unit stride along n, used as it lies by the k-major form of the direct-to-LDS kernel
+bool gemm_dma_bkm_ok(const GemmDesc &g) {
+  return g.bf16_math && g.a_stype == ST_BF16 && g.b_stype == ST_BF16 && g.sak == 1 && g.sbn == 1 && g.sbk != 1 && g.sbk % 8 == 0 &&
+         g.K % 64 == 0 && g.K >= 64 && g.M >= 64 && g.N >= 64 && g.N % 8 == 0 && ((uintptr_t)g.a & 15) == 0 &&
+         ((uintptr_t)g.b & 15) == 0 && g.sam % 8 == 0 && g.sa_b0 % 8 == 0 && g.sa_b1 % 8 == 0 && g.sb_b0 % 8 == 0 &&
+         g.sb_b1 % 8 == 0 && !g.b_index && !g.n_group && !g.glu_gate && !g.c16 && !g.dual_b && !g.c_add;
+}
+
 static bool gemm_fast_path(const GemmDesc &g, int av, int bv) {
   return g.bf16_math && g.M > 8 && g.a_stype == ST_BF16 && g.b_stype == ST_BF16 && g.sak == 1 &&
          (g.sbk == 1 || g.sbn == 1) && g.K % 8 == 0 && (g.sbk == 1 || g.N % 8 == 0) && av && bv;
@@ -2618,6 +2654,12 @@ hipError_t launch_matmul(const LaunchCtx &lc_in, const GemmDesc &g, const char *
       } else {
         e = launch_gemm_dma<128, 128, 2, 2>(lc, gg, (uint32_t)t128);
       }
+      if (e != hipSuccess) return e;
+    } else if (gemm_dma_bkm_ok(g)) {
+      const uint64_t t256 = (uint64_t)((g.M + 255) / 256) * ((g.N + 255) / 256) * batch * splits;
+      const uint64_t t128 = (uint64_t)((g.M + 127) / 128) * ((g.N + 127) / 128) * batch * splits;
+      hipError_t e = t256 >= (uint64_t)lc.n_cus ? launch_gemm_dma<256, 256, 2, 4, false, 2, false, true>(lc, gg, (uint32_t)t256)
+                                                : launch_gemm_dma<128, 128, 2, 2, false, 2, false, true>(lc, gg, (uint32_t)t128);
       if (e != hipSuccess) return e;
     } else {
     if (g.n_group) return hipErrorInvalidValue;

@@ -409,6 +409,9 @@ bool gemv_pro_rows_ok(int b_stype, uint32_t rows, uint32_t K, int pro);
 bool gemv_rows_mfma_ok(int b_stype, uint32_t rows, uint32_t K, int pro);
 // a plain product of 2 to 16 rows that launch_gemv_pro's matrix-core form takes as one of up to four problems
 bool gemv_rows_group_ok(const GemmDesc &g);
+// a bf16 product whose right operand is [K, N] with unit stride along n and that the direct-to-LDS kernel takes
+// as it lies (no transposed copy of B)
+bool gemm_dma_bkm_ok(const GemmDesc &g);
 // The routed experts of a MoE layer over many tokens (a prefill; models/qwen3.rs:104-123), expert by
 // expert.  A slot is one of the k choices of every token: its index vector, its input rows and its
 // outputs.  A problem is one stacked weight tensor [E, N, K] (bf16): gate_proj and up_proj share

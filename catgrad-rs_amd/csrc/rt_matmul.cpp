@@ -762,8 +762,13 @@ int realize_matmul(cg_backend *be, cg_tensor *n, cg_tensor *addend, bool *added,
     // B with unit stride along n (bmm of row-major matrices, p . V): re-laid out once as bf16 [N, K]
     // so that the product takes the direct-to-LDS kernel (one pass over B against K/64 strided ones)
     Storage *bt = nullptr;
+    // (a bf16 B that the k-major form of that kernel reads where it lies needs no copy at all)
+    GemmDesc probe = g;
+    probe.nb0 = nbo[0]; probe.nb1 = nbo[1];
+    probe.sa_b0 = sao[0]; probe.sa_b1 = sao[1]; probe.sb_b0 = sbo[0]; probe.sb_b1 = sbo[1];
+    probe.bf16_math = (be->flags & CG_FLAG_BF16) ? 1 : 0;
     if (g.bf16_math && M >= 64 && N >= 64 && K % 64 == 0 && g.a_stype == ST_BF16 && g.sak == 1 && g.sbn == 1 &&
-        g.sbk != 1 && !ex.w && (g.b_stype == ST_F32 || g.b_stype == ST_BF16)) {
+        g.sbk != 1 && !ex.w && (g.b_stype == ST_F32 || g.b_stype == ST_BF16) && !gemm_dma_bkm_ok(probe)) {
       // batches that only repeat (stride 0) are transposed once
       const uint32_t tb0 = g.sb_b0 ? g.nb0 : 1, tb1 = g.sb_b1 ? g.nb1 : 1;
       TRY(dev_alloc(be, (size_t)tb0 * tb1 * N * K * 2, &bt));

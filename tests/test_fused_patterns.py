@@ -690,6 +690,21 @@ def test_few_rows_on_the_matrix_cores(hip_bf16, rows, K, N):
     assert np.max(np.abs(got.reshape(rows, N) - (want + r16.reshape(rows, N)))) <= 1e-5 * (scale + np.abs(res).max())
 
 
+@pytest.mark.parametrize("b,m,n,k", [(1, 1024, 1024, 1024), (8, 256, 384, 512), (1, 4096, 4104, 256), (2, 192, 200, 128),
+                                     (1, 130, 72, 64), (3, 64, 64, 64), (1, 512, 136, 4096)])
+def test_product_of_two_activations_reads_the_right_operand_where_it_lies(hip_bf16, b, m, n, k):
+    """matmul(x [b, m, k], w [b, k, n]) with both operands as they are stored (ndarray.rs:549-615: any layout): in
+    bf16 mode the right operand, k-major, goes from memory into LDS as it lies and reaches the MFMA through the
+    transposing LDS read - no transposed copy is made first.  Checked against float64 on the rounded operands."""
+    g = np.random.default_rng(b * 1000 + m + n + k)
+    x = vectors.bf16_round(g.standard_normal((b, m, k)).astype(np.float32))
+    w = vectors.bf16_round(g.standard_normal((b, k, n)).astype(np.float32))
+    (got,), names = run_traced(hip_bf16, lambda bb, xv, wv: lang.matmul(bb, xv, wv), 1, x, w)
+    assert "gemm_mfma_bf16" in names and "transpose_cast_bf16" not in names, sorted(names)
+    want = np.einsum("bmk,bkn->bmn", x.astype(np.float64), w.astype(np.float64))
+    assert got.shape == want.shape and np.max(np.abs(got - want)) <= 2e-6 * np.abs(want).max() * np.sqrt(k / 64)
+
+
 @pytest.mark.parametrize("rows,K,widths", [(4, 2048, (60, 1)), (2, 256, (5, 13, 1, 16)), (16, 1024, (33,))])
 def test_narrow_products_of_a_few_rows_share_a_launch(hip_bf16, rows, K, widths):
     """The router and the shared expert's gate of a MoE block (qwen_moe.py: 60 and 1 columns on the same
