@@ -21,14 +21,17 @@ SHAPES = [(1, 8192, 8192, 8192), (1, 4096, 4096, 4096), (8, 1024, 1024, 1024), (
           (1, 16384, 1152, 6912)]
 
 
-def run(lib, shapes=SHAPES, iters=10):
+def run(lib, shapes=SHAPES, iters=10, k_major=False):
     be = cg.Backend(lib, flags=cg.FLAG_BF16)
     g = np.random.default_rng(0)
     out = []
     for b, m, n, k in shapes:
         x = be.tensor(g.standard_normal((b, m, k), dtype=np.float32))
-        w = be.tensor(g.standard_normal((b, n, k), dtype=np.float32))
-        wt = be.transpose(w, 1, 2)                       # [b, K, N] view, unit stride along k
+        if k_major:                                      # the right operand of a product of two activations: [b, K, N] as stored
+            wt = be.tensor(g.standard_normal((b, k, n), dtype=np.float32))
+        else:
+            w = be.tensor(g.standard_normal((b, n, k), dtype=np.float32))
+            wt = be.transpose(w, 1, 2)                   # [b, K, N] view, unit stride along k
         be.realize(be.matmul(x, wt))
         be.sync()
         be.trace(True)
@@ -42,14 +45,14 @@ def run(lib, shapes=SHAPES, iters=10):
         tf = 2.0 * b * m * n * k / (ms * 1e-3) / 1e12
         rec = {"shape": f"{b}x{m}x{n}x{k}", "us": ms * 1e3, "tflops": tf, "frac": tf / MFMA_PEAK_BF16_TFLOPS,
                "kernels": {name: v["launches"] // iters for name, v in rep.items()}}
-        if b == 1 and m % 128 == 0 and n % 128 == 0 and k % 64 == 0:
+        if b == 1 and m % 128 == 0 and n % 128 == 0 and k % 64 == 0 and not k_major:
             # the same product through the clock probe: the shader clock its main loop ran at (the data-sheet
             # peak is 2400 MHz) and the rate as a fraction of the matrix cores' peak at that clock
             ptf, mhz = be.peak_gemm_clock(m, n, k, iters)
             if mhz:
                 rec.update(clock_mhz=mhz, frac_at_clock=tf / (MFMA_PEAK_BF16_TFLOPS * mhz / 2400.0))
         out.append(rec)
-        del x, w, wt
+        del x, wt
     be.close()
     return out
 
@@ -59,9 +62,10 @@ if __name__ == "__main__":
     ap = argparse.ArgumentParser()
     ap.add_argument("--shapes", default=None, help="comma-separated BxMxNxK list (default: the whole sweep)")
     ap.add_argument("--iters", type=int, default=10)
+    ap.add_argument("--k-major", action="store_true", help="B stored [K, N] (unit stride along n) instead of [N, K]")
     a = ap.parse_args()
     shapes = SHAPES if not a.shapes else [tuple(int(v) for v in s.split("x")) for s in a.shapes.split(",")]
-    for r in run(cg.load_library(), shapes, a.iters):
+    for r in run(cg.load_library(), shapes, a.iters, a.k_major):
         clk = f"  clock {r['clock_mhz']:5.0f} MHz -> {100 * r['frac_at_clock']:5.1f} % at that clock" if "clock_mhz" in r else ""
         print(f"{r['shape']:>22s} {r['us']:9.1f} us {r['tflops']:8.1f} TFLOP/s  {100 * r['frac']:5.1f} % of 2.5 PFLOP/s{clk}  {r['kernels']}",
               flush=True)
