@@ -499,9 +499,11 @@ template <int N> __device__ __forceinline__ void wait_vmcnt() {
 // different banks), and the MFMA operand - eight consecutive k of one column per lane - comes out of LDS through
 // the transposing read (ds_read_b64_tr_b16: the 16 lanes of a group hand in four rows of 16 columns, lane c
 // receives column c of the four rows), two reads per fragment.
-template <int BM_, int BN_, int WR, int WC, bool EPI, int NS, bool DUAL = false, bool BKM = false>
+template <int BM_, int BN_, int WR, int WC, bool EPI, int NS, bool DUAL = false, bool BKM = false, bool ROPE = false>
 __global__ void __launch_bounds__(WR *WC * 64) gemm_bf16_dma_kernel(GemmDesc g) {
   constexpr int NW = WR * WC, BK = 64;
+  static_assert(!ROPE || (BN_ == 64 && WC == 2 && BM_ / WR == 32 && !EPI && !DUAL && !BKM && NS * (BM_ + BN_) * 128 >= BM_ * 72 * 4),
+                "rotated heads: one head of 64 columns per tile, its halves in the two waves of a row");
   static_assert(!BKM || (!EPI && !DUAL && (BM_ / 8) % ((BM_ + BN_) / 8 / (WR * WC)) == 0), "k-major B: the plain product");
   constexpr int WM = BM_ / WR, WN = BN_ / WC, TM = WM / 32, TN = WN / 32;
   constexpr int BNO = DUAL ? BN_ / 2 : BN_;    // output columns of a tile
@@ -535,7 +537,7 @@ __global__ void __launch_bounds__(WR *WC * 64) gemm_bf16_dma_kernel(GemmDesc g) 
   float *C = (g.splits > 1 ? g.workspace + (uint64_t)split * batch * g.M * g.N : g.c) +
              (uint64_t)bz * g.M * g.N;
   // grouped products: this tile's columns belong to one of them (tiles never straddle two)
-  uint32_t n0 = n0_all, Nl = g.N;
+  uint32_t n0 = n0_all, Nl = g.N, grp = 0;
   if (g.n_group) {
     uint32_t p = 0;
     while (p + 1 < g.n_group && n0 >= g.grp_n[p]) {
@@ -545,6 +547,7 @@ __global__ void __launch_bounds__(WR *WC * 64) gemm_bf16_dma_kernel(GemmDesc g) 
     B = (const uint16_t *)g.grp_b[p];
     C = g.grp_c[p];
     Nl = g.grp_n[p];
+    grp = p;
   }
   const float *Gate = g.glu_gate ? g.glu_gate + (uint64_t)bz * g.M * g.N : nullptr;  // only without split-K
   uint16_t *C16 = g.c16 ? g.c16 + (uint64_t)bz * g.M * g.N : nullptr;
@@ -716,6 +719,62 @@ __global__ void __launch_bounds__(WR *WC * 64) gemm_bf16_dma_kernel(GemmDesc g) 
     }
     return;
   }
+  if constexpr (ROPE) {
+    // The tile is one head: this wave holds 32 of its columns (lane & 31) for 32 rows, the wave beside it the
+    // other half of the same rows, element for element in the same lanes.
+    const uint32_t role = g.rope_s ? g.rope_role[grp] : 0;
+    const uint32_t colh = wn * 32 + (lane & 31), head = n0 / 64;
+    if (role == 1) {
+      // apply_rope_embedding (catgrad-llm/src/helpers.rs:195-221) on the tile while it is still on the chip, the
+      // arithmetic of rope_kernel: out = cos * x + sin * rot, rot = -x[j + 32] in the lower half, x[j - 32] in the
+      // upper.  The tile goes through LDS once, so that a thread holds four consecutive columns of a row and their
+      // partners, the tables come in 16 bytes at a time, and the head's rows (contiguous in the result) leave as
+      // whole lines.
+      constexpr int P = 72;  // floats per tile row: rows four apart, which a wave writes together, fall on different banks
+      const float *cs = g.rope_cos[grp], *sn = g.rope_sin[grp];
+      const int64_t ss = g.rope_cs_ss[grp];
+      float4 cv[BM_ * 16 / (NW * 64)], sv[BM_ * 16 / (NW * 64)];
+#pragma unroll
+      for (int it = 0; it < BM_ * 16 / (NW * 64); ++it) {
+        const int idx = it * NW * 64 + tid, r = idx >> 4, c4 = (idx & 15) * 4;
+        const uint32_t row = min(m0 + r, g.M - 1);
+        cv[it] = *(const float4 *)(cs + (int64_t)row * ss + c4);
+        sv[it] = *(const float4 *)(sn + (int64_t)row * ss + c4);
+      }
+      float *tile = (float *)dma_smem;
+      __syncthreads();  // every wave is done with the last stage
+#pragma unroll
+      for (int e = 0; e < 16; ++e) tile[(wm * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3)) * P + colh] = acc[0][0][e];
+      __syncthreads();
+      float *out = g.rope_out[grp] + (uint64_t)head * g.rope_s * 64;
+      uint16_t *out16 = g.rope_out16[grp] ? g.rope_out16[grp] + (uint64_t)head * g.rope_s * 64 : nullptr;
+#pragma unroll
+      for (int it = 0; it < BM_ * 16 / (NW * 64); ++it) {
+        const int idx = it * NW * 64 + tid, r = idx >> 4, c4 = (idx & 15) * 4;
+        const uint32_t row = m0 + r;
+        const float4 xv = *(const float4 *)(tile + r * P + c4);
+        float4 pv = *(const float4 *)(tile + r * P + (c4 ^ 32));
+        if (c4 < 32) { pv.x = -pv.x; pv.y = -pv.y; pv.z = -pv.z; pv.w = -pv.w; }
+        float4 o;
+        o.x = cv[it].x * xv.x + sv[it].x * pv.x; o.y = cv[it].y * xv.y + sv[it].y * pv.y;
+        o.z = cv[it].z * xv.z + sv[it].z * pv.z; o.w = cv[it].w * xv.w + sv[it].w * pv.w;
+        if (row < g.M) {
+          *(float4 *)(out + (uint64_t)row * 64 + c4) = o;
+          if (out16) *(uint2 *)(out16 + (uint64_t)row * 64 + c4) = bf16_pack4(o);
+        }
+      }
+      return;
+    }
+    if (role == 2) {  // the values: also as bf16 [head][64][position], four consecutive positions per store
+      uint16_t *vt = g.rope_out16[grp] + ((uint64_t)head * 64 + colh) * g.rope_s;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const uint32_t r0 = m0 + wm * 32 + q * 8 + (lane >> 5) * 4;
+        if (r0 < g.M)
+          *(uint2 *)(vt + r0) = bf16_pack4(make_float4(acc[0][0][q * 4], acc[0][0][q * 4 + 1], acc[0][0][q * 4 + 2], acc[0][0][q * 4 + 3]));
+      }
+    }
+  }
 #pragma unroll
   for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -729,17 +788,17 @@ __global__ void __launch_bounds__(WR *WC * 64) gemm_bf16_dma_kernel(GemmDesc g) 
     }
 }
 
-template <int BM_, int BN_, int WR, int WC, bool EPI = false, int NS = 2, bool DUAL = false, bool BKM = false>
+template <int BM_, int BN_, int WR, int WC, bool EPI = false, int NS = 2, bool DUAL = false, bool BKM = false, bool ROPE = false>
 static hipError_t launch_gemm_dma(const LaunchCtx &lc, const GemmDesc &g, uint32_t grid) {
   constexpr int smem = NS * (BM_ + BN_) * 64 * 2;
   static bool configured = false;  // one attribute call per kernel and process
   if (!configured) {
-    hipError_t e = hipFuncSetAttribute((const void *)gemm_bf16_dma_kernel<BM_, BN_, WR, WC, EPI, NS, DUAL, BKM>,
+    hipError_t e = hipFuncSetAttribute((const void *)gemm_bf16_dma_kernel<BM_, BN_, WR, WC, EPI, NS, DUAL, BKM, ROPE>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return e;
     configured = true;
   }
-  cg_launch(lc, gemm_bf16_dma_kernel<BM_, BN_, WR, WC, EPI, NS, DUAL, BKM>, dim3(grid), dim3(WR * WC * 64), smem, g);
+  cg_launch(lc, gemm_bf16_dma_kernel<BM_, BN_, WR, WC, EPI, NS, DUAL, BKM, ROPE>, dim3(grid), dim3(WR * WC * 64), smem, g);
   return hipGetLastError();
 }
 
@@ -2442,6 +2501,28 @@ bool gemm_epilogue_ok(const GemmDesc &g) {
   return gemm_fast_path(g, av, bv) && gemm_dma_ok(g) && g.splits <= 1 && !g.b_index && !g.c_add && g.N % 4 == 0;
 }
 
+bool gemm_rope_epilogue_ok(const LaunchCtx &lc, const GemmDesc &g) {
+  if (!g.rope_s || !g.n_group || !gemm_epilogue_ok(g)) return false;
+  if (g.nb0 * g.nb1 != 1 || g.glu_gate || g.c16 || g.dual_b || g.M != g.rope_s || g.M % 4 || g.M < 64) return false;
+  bool grp256 = true;
+  for (uint32_t p = 0; p < g.n_group; ++p) {
+    if (g.grp_n[p] % 64) return false;
+    grp256 = grp256 && g.grp_n[p] % 256 == 0;
+    if (g.rope_role[p] == 1) {
+      if (!g.rope_out[p] || !g.rope_cos[p] || !g.rope_sin[p]) return false;
+    } else if (g.rope_role[p] == 2) {
+      if (!g.rope_out16[p] || (uintptr_t)g.rope_out16[p] % 8 || !g.grp_c[p]) return false;
+    } else if (g.rope_role[p] != 0 || !g.grp_c[p]) {
+      return false;
+    }
+  }
+  // the tile launch_matmul picks for this problem must be the one of one head per tile
+  const uint64_t t256 = (uint64_t)((g.M + 255) / 256) * ((g.N + 255) / 256);
+  const uint64_t t128 = (uint64_t)((g.M + 127) / 128) * ((g.N + 127) / 128);
+  if (t256 >= (uint64_t)lc.n_cus && grp256) return false;
+  return t128 * 2 <= (uint64_t)lc.n_cus && g.N >= 128;
+}
+
 // A plain product of 2 to 16 rows with bf16 weights [N][K] that gemv_rows_mfma_kernel takes.
 // (any number of columns: the caller may group several narrow products into one launch)
 bool gemv_rows_group_ok(const GemmDesc &g) {
@@ -2521,6 +2602,7 @@ hipError_t launch_matmul(const LaunchCtx &lc_in, const GemmDesc &g, const char *
   if (g.b_index && !one_row) return hipErrorInvalidValue;
   if (g.c_add && !one_row && g.splits <= 1) return hipErrorInvalidValue;
   if ((g.glu_gate || g.c16 || g.n_group || g.dual_b) && !gemm_epilogue_ok(g)) return hipErrorInvalidValue;
+  if (g.rope_s && !gemm_rope_epilogue_ok(lc_in, g)) return hipErrorInvalidValue;
 
   if (gemv_rows_plain_ok(lc_in, g)) {
     // a few rows against bf16 weights: the matrix-core kernel, without a prologue
@@ -2648,7 +2730,9 @@ hipError_t launch_matmul(const LaunchCtx &lc_in, const GemmDesc &g, const char *
           e = launch_gemm_dma<256, 256, 2, 4>(lc, gg, (uint32_t)t256);
       } else if (splits == 1 && t128 * 2 <= (uint64_t)lc.n_cus && g.N >= 128) {
         // too few 128 x 128 tiles for the CUs and no split-K to multiply them: halve the tile
-        e = launch_gemm_dma<128, 64, 4, 2, false, 4>(lc, gg, (uint32_t)((uint64_t)((g.M + 127) / 128) * ((g.N + 63) / 64) * batch));
+        const uint32_t t64 = (uint32_t)((uint64_t)((g.M + 127) / 128) * ((g.N + 63) / 64) * batch);
+        if (g.rope_s) e = launch_gemm_dma<128, 64, 4, 2, false, 4, false, false, true>(lc, gg, t64);
+        else e = launch_gemm_dma<128, 64, 4, 2, false, 4>(lc, gg, t64);
       } else if (deep) {
         e = launch_gemm_dma<128, 128, 2, 4, false, 4>(lc, gg, (uint32_t)t128);
       } else {

@@ -298,6 +298,17 @@ struct GemmDesc {
   const void *grp_b[3];
   float *grp_c[3];
   uint32_t grp_n[3];
+  // optional, with n_group (gemm_rope_epilogue_ok): the products are the q / k / v projections of one batch of
+  // rope_s positions with heads of 64 columns, row m being position m.  A group with rope_role 1 leaves the
+  // kernel rotated (apply_rope_embedding, cos / sin rows of 64 at rope_cs_ss apart) as [head][position][64] at
+  // rope_out (f32) and rope_out16 (bf16, optional) instead of grp_c; a group with rope_role 2 is stored as usual
+  // and also transposed, as bf16 [head][64][position], at rope_out16.
+  uint32_t rope_s;
+  uint32_t rope_role[3];
+  float *rope_out[3];
+  uint16_t *rope_out16[3];
+  const float *rope_cos[3], *rope_sin[3];
+  int64_t rope_cs_ss[3];
   // optional (the direct-to-LDS bf16 GEMM, for the clock probe): every workgroup adds the shader-clock ticks and
   // the 100 MHz ticks its main loop took to clock_ticks[0] and [1]
   unsigned long long *clock_ticks;
@@ -307,6 +318,8 @@ uint32_t gemm_split_k(const LaunchCtx &lc, const GemmDesc &g);
 // whether launch_matmul would run this problem (splits as given) on the kernel that honours
 // glu_gate / c16
 bool gemm_epilogue_ok(const GemmDesc &g);
+// whether launch_matmul would run this grouped problem on the tile whose epilogue honours rope_role
+bool gemm_rope_epilogue_ok(const LaunchCtx &lc, const GemmDesc &g);
 hipError_t launch_matmul(const LaunchCtx &lc, const GemmDesc &g, const char **kernel_name);
 // contiguous f32 -> bf16 (RNE); n % 8 == 0, 16-byte aligned
 hipError_t launch_cast_bf16(const LaunchCtx &lc, const float *in, void *out, uint64_t n);

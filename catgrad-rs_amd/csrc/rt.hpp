@@ -22,6 +22,8 @@
 
 namespace cgrt {
 
+struct RopeGemmRequest;
+
 struct Storage {
   std::atomic<int> rc{1};
   void *ptr = nullptr;
@@ -176,6 +178,9 @@ struct cg_backend {
   // k-slices of its product (N_KSUM): the RMSNorm that reads it next sums them on its way in.
   cg_tensor *ksum_flush_node = nullptr;  // that add, while it is being realised (a weak reference)
   bool ksum_request = false;   // set by try_gemv_add around its product
+  // set by try_qkv_rope_gemm around the realisation of a q projection: the grouped q / k / v launch may rotate
+  // the queries and keys and transpose the values in its epilogue
+  cgrt::RopeGemmRequest *rope_request = nullptr;
   cgrt::Storage *ksum_ws = nullptr;  // handed back by realize_matmul: the slices (the caller owns them now)
   uint32_t ksum_splits = 0;
   // argmax over the row a one-row product is about to store (the logits of a greedy decode step): realize_reduce

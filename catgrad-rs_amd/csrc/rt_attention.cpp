@@ -32,9 +32,17 @@ int try_attn_prefill(cg_backend *be, cg_tensor *n, bool *done) {
   if (nb > 65535 || heads > 65535) return CG_OK;
   cg_tensor *q = S->in[0];
   // queries and keys both still to be rotated: one launch for the two (each alone otherwise, below)
+  // (the transposed bf16 values, when the projections' own launch has made them: released on every way out)
+  struct Held {
+    Storage *s = nullptr;
+    ~Held() { storage_release(s); }
+  } vt_made;
+  const Storage *vt_of = nullptr;
   if (cg_tensor *kr = node_under_repeat_kv(S->in[1])) {
     bool paired = false;
-    TRY(try_rope_pair(be, q, kr, &paired));
+    // ... or none at all: the projections still deferred rotate q and k in their epilogue
+    if (!f32 && d == 64 && nb == 1) TRY(try_qkv_rope_gemm(be, q, kr, node_under_repeat_kv(n->in[1]), &vt_made.s, &vt_of, &paired));
+    if (!paired) TRY(try_rope_pair(be, q, kr, &paired));
   }
   MatOperand Kop, Vop;
   bool pk = false, pv = false;
@@ -93,6 +101,7 @@ int try_attn_prefill(cg_backend *be, cg_tensor *n, bool *done) {
     return CG_OK;
   }
   Storage *vt = nullptr;
+  bool vt_ready = false;
   const int64_t kvh = Kop.shape[1];
   if (f32) {
     a.f32 = 1;
@@ -100,9 +109,17 @@ int try_attn_prefill(cg_backend *be, cg_tensor *n, bool *done) {
   } else {
     TRY(bf16_shadow(be, Kop.t->st, &ksh));
     a.k16 = (const uint16_t *)ksh->ptr + Kop.t->offset;
-    TRY(dev_alloc(be, (size_t)nb * kvh * d * T * 2, &vt));
+    // the values as the projections left them, [T, kv heads * d] read as [kv heads][T][d]: their transposed copy is there
+    if (vt_made.s && vt_of == Vop.t->st && Vop.t->offset == 0 && Vop.strides[1] == d && Vop.strides[3] == kvh * d &&
+        Vop.strides[4] == 1 && (size_t)kvh * d * T * 2 <= vt_made.s->bytes) {
+      vt = vt_made.s;
+      vt_made.s = nullptr;
+      vt_ready = true;
+    } else {
+      TRY(dev_alloc(be, (size_t)nb * kvh * d * T * 2, &vt));
+    }
   }
-  if (!f32) {
+  if (!f32 && !vt_ready) {
     KernelScope ks(be, "transpose_cast_bf16", (double)nb * kvh * d * T * 6, 0);
     hipError_t te = launch_transpose_cast_bf16(be->lc(), data_ptr(Vop.t), ST_F32, vt->ptr, (uint32_t)T, (uint32_t)d,
                                                Vop.strides[3], (uint32_t)nb, (uint32_t)kvh, Vop.strides[0], Vop.strides[1]);

@@ -115,6 +115,7 @@ int try_rmsnorm_pair(cg_backend *be, cg_tensor *root, const RmsNormMatch &outer,
 int try_rmsnorm(cg_backend *be, cg_tensor *root, bool *done);
 int try_row_scaled_sum(cg_backend *be, cg_tensor *root, bool *done);
 bool match_rope(cg_tensor *root, RopeMatch *m);
+int rope_tables(cg_backend *be, const RopeMatch &m, bool *ok);
 int rope_operands(cg_backend *be, const RopeMatch &m, bool *ok);
 int rope_into(cg_backend *be, cg_tensor *root, const RopeMatch &m, float *out, const int64_t *o_strides,
               const char *name, bool *done, uint16_t *out16 = nullptr);
@@ -122,6 +123,8 @@ int try_rope(cg_backend *be, cg_tensor *root, bool *done);
 int rope_describe(cg_backend *be, cg_tensor *root, const RopeMatch &m, float *out, const int64_t *o_strides,
                   uint16_t *out16, RopeDesc *dsc, cg_tensor **xs_out, bool *ok);
 int try_rope_pair(cg_backend *be, cg_tensor *rq, cg_tensor *rk, bool *done);
+int try_qkv_rope_gemm(cg_backend *be, cg_tensor *rq, cg_tensor *rk, cg_tensor *v, Storage **vt, const Storage **v_st,
+                      bool *done);
 cg_tensor *node_under_repeat_kv(cg_tensor *t);
 bool is_sigmoid_of(const cg_tensor *s, const cg_tensor **arg);
 bool is_gelu_of(const cg_tensor *g, const cg_tensor **arg);
@@ -499,6 +502,19 @@ struct RmsNormMatch {
 // apply_rope_embedding (catgrad-llm/src/helpers.rs:195-221): cos * x + sin * rotate_half(x)
 struct RopeMatch {
   cg_tensor *cb = nullptr, *sb = nullptr, *x = nullptr;  // cos / sin broadcasts, the rotated tensor
+};
+
+// What the q / k / v projections of a prefill are asked to do in the epilogue of their grouped launch: leave the
+// queries and keys rotated, head-major, and a transposed bf16 copy of the values (GemmDesc::rope_role).  The
+// launch sets `applied` when it did.
+struct RopeGemmRequest {
+  cg_tensor *mm[3] = {nullptr, nullptr, nullptr};  // the products: q, k, v
+  float *out[2] = {nullptr, nullptr};              // rotated q, k: [heads][positions][64]
+  uint16_t *out16[3] = {nullptr, nullptr, nullptr};  // their bf16 copies (optional); [2]: v as [heads][64][positions]
+  const float *cos[2] = {nullptr, nullptr}, *sin[2] = {nullptr, nullptr};
+  int64_t cs_ss[2] = {0, 0};
+  uint32_t positions = 0;
+  bool applied = false;
 };
 
 

@@ -985,6 +985,33 @@ int realize_matmul(cg_backend *be, cg_tensor *n, cg_tensor *addend, bool *added,
         ++g.n_group;
       }
     }
+    // q / k / v of an attention that asked for its rotation and transposition in this launch's epilogue
+    if (RopeGemmRequest *rq = be->rope_request; rq && group.size() == 2) {
+      cg_tensor *members[3] = {n, group[0], group[1]};
+      GemmDesc t = g;
+      bool all = true;
+      for (int i = 0; i < 3 && all; ++i) {
+        int j = 0;
+        while (j < 3 && rq->mm[j] != members[i]) ++j;
+        if (j == 3) all = false;
+        else if (j < 2) {
+          t.rope_role[i] = 1;
+          t.rope_out[i] = rq->out[j];
+          t.rope_out16[i] = rq->out16[j];
+          t.rope_cos[i] = rq->cos[j];
+          t.rope_sin[i] = rq->sin[j];
+          t.rope_cs_ss[i] = rq->cs_ss[j];
+        } else {
+          t.rope_role[i] = 2;
+          t.rope_out16[i] = rq->out16[2];
+        }
+      }
+      t.rope_s = rq->positions;
+      if (all && gemm_rope_epilogue_ok(be->lc(), t)) {
+        g = t;
+        rq->applied = true;
+      }
+    }
     Storage *ws = nullptr;
     const bool dual = ep && ep->dual_w;  // twice the work per tile: no k-slices on top
     const uint32_t splits = group.empty() && !dual ? gemm_split_k(be->lc(), g) : 1;
@@ -1034,7 +1061,7 @@ int realize_matmul(cg_backend *be, cg_tensor *n, cg_tensor *addend, bool *added,
       if (be->trace_shapes) {  // per-shape records: gemm_mfma_bf16[b32,512x512x64,s1]
         char buf[96];
         snprintf(buf, sizeof buf, "%s[b%lld,%ux%ux%u,s%u%s]", kname, (long long)batch, M, g.N, K, splits,
-                 g.dual_b ? ",gate*up" : group.empty() ? "" : ",grouped");
+                 g.dual_b ? ",gate*up" : group.empty() ? "" : g.rope_s ? ",grouped,rope" : ",grouped");
         ks.rename(buf);
       }
     }

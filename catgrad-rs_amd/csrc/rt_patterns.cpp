@@ -560,11 +560,10 @@ bool match_rope(cg_tensor *root, RopeMatch *m) {
 }
 
 
-// realises the operands of a matched rope; *ok = the kernel's layout requirements hold
-int rope_operands(cg_backend *be, const RopeMatch &m, bool *ok) {
+// realises the cos / sin tables of a matched rope; *ok = the kernels' layout requirements hold
+int rope_tables(cg_backend *be, const RopeMatch &m, bool *ok) {
   TRY(realize(be, m.cb));
   TRY(realize(be, m.sb));
-  TRY(realize(be, m.x));
   auto table_ok = [&](const cg_tensor *t) {
     return t->stype == ST_F32 && t->strides[0] * (t->shape[0] != 1) == 0 &&
            t->strides[1] * (t->shape[1] != 1) == 0 && t->strides[3] == 1 && t->strides[2] % 4 == 0 &&
@@ -572,6 +571,12 @@ int rope_operands(cg_backend *be, const RopeMatch &m, bool *ok) {
   };
   *ok = table_ok(m.cb) && table_ok(m.sb) && m.cb->strides[2] == m.sb->strides[2];
   return CG_OK;
+}
+
+// ... and the rotated tensor too
+int rope_operands(cg_backend *be, const RopeMatch &m, bool *ok) {
+  TRY(realize(be, m.x));
+  return rope_tables(be, m, ok);
 }
 
 
@@ -680,6 +685,84 @@ int try_rope_pair(cg_backend *be, cg_tensor *rq, cg_tensor *rk, bool *done) {
   }
   finish_fused(rq);
   finish_fused(rk);
+  *done = true;
+  return CG_OK;
+}
+
+// The queries, keys and values of a prefill attention whose projections are all still deferred (models/llama.rs:77-94:
+// three linears on one input, `reshape [b, s, heads, d]`, `transpose(1, 2)`, then apply_rope_embedding on q and k):
+// the grouped launch of the three products rotates q and k where they are still accumulators and stores a
+// transposed bf16 copy of v beside v itself, so neither the rotation nor the transposition is a launch of its own.
+// Heads of 64 columns, one batch.  *done = false: nothing was changed beyond realising the products.
+// On success *vt owns the transposed values ([kv heads][64][positions], bf16) of the storage *v_st.
+int try_qkv_rope_gemm(cg_backend *be, cg_tensor *rq, cg_tensor *rk, cg_tensor *v, Storage **vt, const Storage **v_st,
+                      bool *done) {
+  *done = false;
+  *vt = nullptr;
+  *v_st = nullptr;
+  if (!(be->flags & CG_FLAG_BF16) || (be->flags & CG_FLAG_NO_PATTERNS)) return CG_OK;
+  if (rq == rk || rq->op == N_REAL || rk->op == N_REAL || !v || v->op == N_REAL) return CG_OK;
+  RopeMatch mq, mk;
+  if (!match_rope(rq, &mq) || !match_rope(rk, &mk)) return CG_OK;
+  // x = transpose(1, 2) of reshapes of a deferred product [1, s, heads * 64]; `readers`: the references x must
+  // have (the rotation reads it three times and nobody else may: its product is never stored as such), 0 = any
+  auto product_under = [](cg_tensor *x, int readers) -> cg_tensor * {
+    if (x->op != N_TRANSPOSE || x->rank != 4 || (readers && refs(x) != readers)) return nullptr;
+    if (!((x->p0 == 1 && x->p1 == 2) || (x->p0 == 2 && x->p1 == 1)) || x->shape[0] != 1 || x->shape[3] != 64) return nullptr;
+    cg_tensor *t = x->in[0];
+    while (t->op == N_RESHAPE && (!readers || refs(t) == 1)) t = t->in[0];
+    if (t->op != N_MATMUL || (readers && refs(t) != 1) || !t->gemm_candidate || t->dtype != CG_F32 || t->rank != 3) return nullptr;
+    if (t->shape[0] != 1 || t->shape[1] != x->shape[2] || t->shape[2] != x->shape[1] * 64) return nullptr;
+    return t;
+  };
+  cg_tensor *pq = product_under(mq.x, 3), *pk = product_under(mk.x, 3), *pv = product_under(v, 0);
+  if (!pq || !pk || !pv || pq == pk || pq == pv || pk == pv) return CG_OK;
+  const int64_t positions = pq->shape[1];
+  if (pk->shape[1] != positions || pv->shape[1] != positions || pk->shape[2] != pv->shape[2] || positions % 4) return CG_OK;
+  bool tq = false, tk = false;
+  TRY(rope_tables(be, mq, &tq));
+  TRY(rope_tables(be, mk, &tk));
+  if (!tq || !tk) return CG_OK;
+  RopeGemmRequest req;
+  cg_tensor *roots[2] = {rq, rk};
+  const RopeMatch *ms[2] = {&mq, &mk};
+  int st = CG_OK;
+  for (int i = 0; i < 2 && !st; ++i) {
+    st = alloc_result(be, roots[i], ST_F32);
+    if (!st) st = twin_for_result(be, roots[i], &req.out16[i]);
+    if (!st) {
+      req.out[i] = (float *)roots[i]->st->ptr;
+      req.cos[i] = (const float *)data_ptr(ms[i]->cb);
+      req.sin[i] = (const float *)data_ptr(ms[i]->sb);
+      req.cs_ss[i] = ms[i]->cb->strides[2];
+    }
+  }
+  Storage *t = nullptr;
+  if (!st) st = dev_alloc(be, (size_t)pv->shape[2] * positions * 2, &t);
+  if (!st) {
+    req.out16[2] = (uint16_t *)t->ptr;
+    req.mm[0] = pq;
+    req.mm[1] = pk;
+    req.mm[2] = pv;
+    req.positions = (uint32_t)positions;
+    cg_tensor *keep = retain(pv);  // (the products leave the graph as they are realised)
+    be->rope_request = &req;
+    st = realize(be, pq);
+    be->rope_request = nullptr;
+    if (!st && req.applied && keep->op == N_REAL) *v_st = keep->st;
+    node_release(keep);
+  }
+  if (st || !req.applied) {  // the rotation and the transposition stay with their own kernels
+    for (int i = 0; i < 2; ++i) {
+      storage_release(roots[i]->st);
+      roots[i]->st = nullptr;
+    }
+    storage_release(t);
+    return st;
+  }
+  finish_fused(rq);
+  finish_fused(rk);
+  *vt = t;
   *done = true;
   return CG_OK;
 }

@@ -138,6 +138,42 @@ def test_llama_prefill_of_many_rows(oracle, hip, hip_bf16):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("tokens,heads,kv_heads", [(256, 8, 2), (320, 4, 4), (300, 4, 2), (512, 16, 2)])
+def test_llama_prefill_rotates_in_the_projections_launch(oracle, hip_bf16, tokens, heads, kv_heads):
+    """bf16 prefill with heads of 64 (models/llama.rs:77-94, helpers.rs:195-221): the grouped q/k/v launch leaves the
+    queries and keys rotated and a transposed bf16 copy of the values, so the trace holds neither a rotation nor a
+    transposition of its own.  The caches it returns (rotated keys, values) and the logits of the prefill and of a
+    decode step that reads those caches are held to the bf16 bar against the oracle on rounded parameters."""
+    cfg = U.tiny_config(hidden_size=64 * heads, intermediate_size=512, num_hidden_layers=2,
+                        num_attention_heads=heads, num_key_value_heads=kv_heads, vocab_size=300)
+    arrays = U.param_arrays(cfg, seed=21, std=0.05)
+    rounded = {k: (vectors.bf16_round(a) if a.ndim >= 2 else a) for k, a in arrays.items()}
+    prompt = list(np.random.default_rng(tokens).integers(0, cfg.vocab_size, tokens))
+    ref = U.CachedRunner(oracle, cfg, rounded, tokens + 8)
+    rt, rl = ref.prefill(prompt)
+    g = U.CachedRunner(hip_bf16, cfg, arrays, tokens + 8)
+    hip_bf16.trace(2)
+    hip_bf16.trace_reset()
+    gt, gl = g.prefill(prompt)
+    gl = hip_bf16.to_vec(gl)
+    names = sorted(hip_bf16.trace_report())
+    hip_bf16.trace(False)
+    parity.assert_bf16(oracle.to_vec(rl), gl, "prefill logits")
+    assert sum("grouped,rope" in n for n in names) >= 1, names
+    # (300 keys are not a multiple of 8: that attention runs as two products and a softmax, which lay out the
+    # values for themselves)
+    assert not any(n.startswith(("rope_fused", "transpose_cast_bf16")) for n in names) or tokens % 8, names
+    for layer in range(cfg.num_hidden_layers):
+        for which, what in ((0, "rotated keys"), (1, "values")):
+            parity.assert_bf16(oracle.to_vec(ref.kv[2 * layer + which]), hip_bf16.to_vec(g.kv[2 * layer + which]),
+                               f"layer {layer} {what}")
+    tok = int(oracle.to_vec(rt).reshape(-1)[0])
+    _, rl = ref.step(tok)
+    _, gl = g.step(tok)
+    parity.assert_bf16(oracle.to_vec(rl), hip_bf16.to_vec(gl), "decode step on the prefill's caches")
+
+
+@pytest.mark.gpu
 def test_llama_prefill_block_ends_at_full_width(oracle, hip, hip_bf16):
     """Two layers at the 1B model's widths (hidden 2048, FFN 8192, 32 / 8 heads of 64) over a 128-token prompt:
     o_proj and down_proj are split along k here, every `residual + linear(x)` is issued as soon as it is recorded
