@@ -502,8 +502,8 @@ template <int N> __device__ __forceinline__ void wait_vmcnt() {
 template <int BM_, int BN_, int WR, int WC, bool EPI, int NS, bool DUAL = false, bool BKM = false, bool ROPE = false>
 __global__ void __launch_bounds__(WR *WC * 64) gemm_bf16_dma_kernel(GemmDesc g) {
   constexpr int NW = WR * WC, BK = 64;
-  static_assert(!ROPE || (BN_ == 64 && WC == 2 && BM_ / WR == 32 && !EPI && !DUAL && !BKM && NS * (BM_ + BN_) * 128 >= BM_ * 72 * 4),
-                "rotated heads: one head of 64 columns per tile, its halves in the two waves of a row");
+  static_assert(!ROPE || (BN_ % 64 == 0 && !EPI && !DUAL && !BKM && (BM_ * BN_ / 4) % (WR * WC * 64) == 0),
+                "rotated heads: whole heads of 64 columns per tile");
   static_assert(!BKM || (!EPI && !DUAL && (BM_ / 8) % ((BM_ + BN_) / 8 / (WR * WC)) == 0), "k-major B: the plain product");
   constexpr int WM = BM_ / WR, WN = BN_ / WC, TM = WM / 32, TN = WN / 32;
   constexpr int BNO = DUAL ? BN_ / 2 : BN_;    // output columns of a tile
@@ -720,59 +720,72 @@ __global__ void __launch_bounds__(WR *WC * 64) gemm_bf16_dma_kernel(GemmDesc g) 
     return;
   }
   if constexpr (ROPE) {
-    // The tile is one head: this wave holds 32 of its columns (lane & 31) for 32 rows, the wave beside it the
-    // other half of the same rows, element for element in the same lanes.
+    // The tile holds BN_ / 64 whole heads of 64 columns.
     const uint32_t role = g.rope_s ? g.rope_role[grp] : 0;
-    const uint32_t colh = wn * 32 + (lane & 31), head = n0 / 64;
     if (role == 1) {
       // apply_rope_embedding (catgrad-llm/src/helpers.rs:195-221) on the tile while it is still on the chip, the
-      // arithmetic of rope_kernel: out = cos * x + sin * rot, rot = -x[j + 32] in the lower half, x[j - 32] in the
-      // upper.  The tile goes through LDS once, so that a thread holds four consecutive columns of a row and their
-      // partners, the tables come in 16 bytes at a time, and the head's rows (contiguous in the result) leave as
-      // whole lines.
-      constexpr int P = 72;  // floats per tile row: rows four apart, which a wave writes together, fall on different banks
+      // arithmetic of rope_kernel: out = cos * x + sin * rot, rot = -x[j + 32] in the lower half of a head,
+      // x[j - 32] in the upper.  The tile goes through LDS once, so that a thread holds four consecutive columns
+      // of a row and their partners, the tables come in 16 bytes at a time, and the rows of a head (contiguous
+      // in the result) leave as whole lines.
+      constexpr int P = BN_ + 8;  // floats per tile row: rows four apart, which a wave writes together, fall on different banks
+      constexpr int F4 = BN_ / 4, ITERS = BM_ * F4 / (NW * 64), AHEAD = ITERS < 4 ? ITERS : 4;
       const float *cs = g.rope_cos[grp], *sn = g.rope_sin[grp];
       const int64_t ss = g.rope_cs_ss[grp];
-      float4 cv[BM_ * 16 / (NW * 64)], sv[BM_ * 16 / (NW * 64)];
+      auto table = [&](const float *tb, int it) {
+        const int idx = it * NW * 64 + tid, r = idx / F4, c4 = (idx % F4) * 4;
+        return *(const float4 *)(tb + (int64_t)min(m0 + r, g.M - 1) * ss + (c4 & 63));
+      };
+      float4 cv[AHEAD], sv[AHEAD];  // the first rows of the tables are requested before the tile is exchanged
 #pragma unroll
-      for (int it = 0; it < BM_ * 16 / (NW * 64); ++it) {
-        const int idx = it * NW * 64 + tid, r = idx >> 4, c4 = (idx & 15) * 4;
-        const uint32_t row = min(m0 + r, g.M - 1);
-        cv[it] = *(const float4 *)(cs + (int64_t)row * ss + c4);
-        sv[it] = *(const float4 *)(sn + (int64_t)row * ss + c4);
+      for (int it = 0; it < AHEAD; ++it) {
+        cv[it] = table(cs, it);
+        sv[it] = table(sn, it);
       }
       float *tile = (float *)dma_smem;
       __syncthreads();  // every wave is done with the last stage
 #pragma unroll
-      for (int e = 0; e < 16; ++e) tile[(wm * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3)) * P + colh] = acc[0][0][e];
-      __syncthreads();
-      float *out = g.rope_out[grp] + (uint64_t)head * g.rope_s * 64;
-      uint16_t *out16 = g.rope_out16[grp] ? g.rope_out16[grp] + (uint64_t)head * g.rope_s * 64 : nullptr;
+      for (int i = 0; i < TM; ++i)
 #pragma unroll
-      for (int it = 0; it < BM_ * 16 / (NW * 64); ++it) {
-        const int idx = it * NW * 64 + tid, r = idx >> 4, c4 = (idx & 15) * 4;
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+          for (int e = 0; e < 16; ++e)
+            tile[(wm * WM + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3)) * P + wn * WN + j * 32 + (lane & 31)] = acc[i][j][e];
+      __syncthreads();
+#pragma unroll
+      for (int it = 0; it < ITERS; ++it) {
+        const int idx = it * NW * 64 + tid, r = idx / F4, c4 = (idx % F4) * 4;
         const uint32_t row = m0 + r;
+        const float4 c = it < AHEAD ? cv[it < AHEAD ? it : 0] : table(cs, it);
+        const float4 sn4 = it < AHEAD ? sv[it < AHEAD ? it : 0] : table(sn, it);
         const float4 xv = *(const float4 *)(tile + r * P + c4);
         float4 pv = *(const float4 *)(tile + r * P + (c4 ^ 32));
-        if (c4 < 32) { pv.x = -pv.x; pv.y = -pv.y; pv.z = -pv.z; pv.w = -pv.w; }
+        if (!(c4 & 32)) { pv.x = -pv.x; pv.y = -pv.y; pv.z = -pv.z; pv.w = -pv.w; }
         float4 o;
-        o.x = cv[it].x * xv.x + sv[it].x * pv.x; o.y = cv[it].y * xv.y + sv[it].y * pv.y;
-        o.z = cv[it].z * xv.z + sv[it].z * pv.z; o.w = cv[it].w * xv.w + sv[it].w * pv.w;
+        o.x = c.x * xv.x + sn4.x * pv.x; o.y = c.y * xv.y + sn4.y * pv.y;
+        o.z = c.z * xv.z + sn4.z * pv.z; o.w = c.w * xv.w + sn4.w * pv.w;
         if (row < g.M) {
-          *(float4 *)(out + (uint64_t)row * 64 + c4) = o;
-          if (out16) *(uint2 *)(out16 + (uint64_t)row * 64 + c4) = bf16_pack4(o);
+          const uint64_t at = ((uint64_t)((n0 + c4) / 64) * g.rope_s + row) * 64 + (c4 & 63);
+          *(float4 *)(g.rope_out[grp] + at) = o;
+          if (g.rope_out16[grp]) *(uint2 *)(g.rope_out16[grp] + at) = bf16_pack4(o);
         }
       }
       return;
     }
     if (role == 2) {  // the values: also as bf16 [head][64][position], four consecutive positions per store
-      uint16_t *vt = g.rope_out16[grp] + ((uint64_t)head * 64 + colh) * g.rope_s;
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const uint32_t r0 = m0 + wm * 32 + q * 8 + (lane >> 5) * 4;
-        if (r0 < g.M)
-          *(uint2 *)(vt + r0) = bf16_pack4(make_float4(acc[0][0][q * 4], acc[0][0][q * 4 + 1], acc[0][0][q * 4 + 2], acc[0][0][q * 4 + 3]));
-      }
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          const uint32_t col = n0 + wn * WN + j * 32 + (lane & 31);  // = head * 64 + column of the head
+          uint16_t *vt = g.rope_out16[grp] + (uint64_t)col * g.rope_s;
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const uint32_t r0 = m0 + wm * WM + i * 32 + q * 8 + (lane >> 5) * 4;
+            if (r0 < g.M)
+              *(uint2 *)(vt + r0) = bf16_pack4(make_float4(acc[i][j][q * 4], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3]));
+          }
+        }
     }
   }
 #pragma unroll
@@ -790,7 +803,8 @@ __global__ void __launch_bounds__(WR *WC * 64) gemm_bf16_dma_kernel(GemmDesc g) 
 
 template <int BM_, int BN_, int WR, int WC, bool EPI = false, int NS = 2, bool DUAL = false, bool BKM = false, bool ROPE = false>
 static hipError_t launch_gemm_dma(const LaunchCtx &lc, const GemmDesc &g, uint32_t grid) {
-  constexpr int smem = NS * (BM_ + BN_) * 64 * 2;
+  // (ROPE: the f32 tile is exchanged through LDS at the end, BN_ + 8 floats per row)
+  constexpr int stages = NS * (BM_ + BN_) * 64 * 2, smem = ROPE && BM_ * (BN_ + 8) * 4 > stages ? BM_ * (BN_ + 8) * 4 : stages;
   static bool configured = false;  // one attribute call per kernel and process
   if (!configured) {
     hipError_t e = hipFuncSetAttribute((const void *)gemm_bf16_dma_kernel<BM_, BN_, WR, WC, EPI, NS, DUAL, BKM, ROPE>,
@@ -2516,11 +2530,13 @@ bool gemm_rope_epilogue_ok(const LaunchCtx &lc, const GemmDesc &g) {
       return false;
     }
   }
-  // the tile launch_matmul picks for this problem must be the one of one head per tile
+  // launch_matmul's tiles of 128 rows have this epilogue (128 columns, or 64 where those are too few for the
+  // CUs); the 256 x 256 tile of the largest problems has not
   const uint64_t t256 = (uint64_t)((g.M + 255) / 256) * ((g.N + 255) / 256);
-  const uint64_t t128 = (uint64_t)((g.M + 127) / 128) * ((g.N + 127) / 128);
   if (t256 >= (uint64_t)lc.n_cus && grp256) return false;
-  return t128 * 2 <= (uint64_t)lc.n_cus && g.N >= 128;
+  for (uint32_t p = 0; p < g.n_group; ++p)
+    if (g.grp_n[p] % 128) return false;
+  return g.N >= 128;
 }
 
 // A plain product of 2 to 16 rows with bf16 weights [N][K] that gemv_rows_mfma_kernel takes.
@@ -2734,9 +2750,11 @@ hipError_t launch_matmul(const LaunchCtx &lc_in, const GemmDesc &g, const char *
         if (g.rope_s) e = launch_gemm_dma<128, 64, 4, 2, false, 4, false, false, true>(lc, gg, t64);
         else e = launch_gemm_dma<128, 64, 4, 2, false, 4>(lc, gg, t64);
       } else if (deep) {
-        e = launch_gemm_dma<128, 128, 2, 4, false, 4>(lc, gg, (uint32_t)t128);
+        if (g.rope_s) e = launch_gemm_dma<128, 128, 2, 4, false, 4, false, false, true>(lc, gg, (uint32_t)t128);
+        else e = launch_gemm_dma<128, 128, 2, 4, false, 4>(lc, gg, (uint32_t)t128);
       } else {
-        e = launch_gemm_dma<128, 128, 2, 2>(lc, gg, (uint32_t)t128);
+        if (g.rope_s) e = launch_gemm_dma<128, 128, 2, 2, false, 2, false, false, true>(lc, gg, (uint32_t)t128);
+        else e = launch_gemm_dma<128, 128, 2, 2>(lc, gg, (uint32_t)t128);
       }
       if (e != hipSuccess) return e;
     } else if (gemm_dma_bkm_ok(g)) {
