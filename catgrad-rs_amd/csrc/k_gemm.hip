@@ -549,6 +549,7 @@ __global__ void __launch_bounds__(WR *WC * 64) gemm_bf16_dma_kernel(GemmDesc g) 
     Nl = g.grp_n[p];
     grp = p;
   }
+  const float *Bias = g.n_group ? g.grp_bias[grp] : nullptr;
   const float *Gate = g.glu_gate ? g.glu_gate + (uint64_t)bz * g.M * g.N : nullptr;  // only without split-K
   uint16_t *C16 = g.c16 ? g.c16 + (uint64_t)bz * g.M * g.N : nullptr;
   const uint32_t k_begin = split * g.k_per_split;
@@ -720,70 +721,88 @@ __global__ void __launch_bounds__(WR *WC * 64) gemm_bf16_dma_kernel(GemmDesc g) 
     return;
   }
   if constexpr (ROPE) {
-    // The tile holds BN_ / 64 whole heads of 64 columns.
+    // The tile holds whole heads of hd = 64 or 128 columns (BN_ is a multiple of hd).
     const uint32_t role = g.rope_s ? g.rope_role[grp] : 0;
+    const uint32_t hd = g.rope_hd, S = g.rope_s, heads = Nl / hd;
     if (role == 1) {
       // apply_rope_embedding (catgrad-llm/src/helpers.rs:195-221) on the tile while it is still on the chip, the
-      // arithmetic of rope_kernel: out = cos * x + sin * rot, rot = -x[j + 32] in the lower half of a head,
-      // x[j - 32] in the upper.  The tile goes through LDS once, so that a thread holds four consecutive columns
-      // of a row and their partners, the tables come in 16 bytes at a time, and the rows of a head (contiguous
-      // in the result) leave as whole lines.
+      // arithmetic of rope_kernel: out = cos * x + sin * rot, rot = -x[j + hd / 2] in the lower half of a head,
+      // x[j - hd / 2] in the upper.  The tile goes through LDS once, so that a thread holds four consecutive
+      // columns of a row and their partners, the tables come in 16 bytes at a time, and the rows of a head
+      // (contiguous in the result) leave as whole lines.
       constexpr int P = BN_ + 8;  // floats per tile row: rows four apart, which a wave writes together, fall on different banks
-      constexpr int F4 = BN_ / 4, ITERS = BM_ * F4 / (NW * 64), AHEAD = ITERS < 4 ? ITERS : 4;
+      constexpr int F4 = BN_ / 4, ITERS = BM_ * F4 / (NW * 64), CH = ITERS < 4 ? ITERS : 4;
+      static_assert(ITERS % CH == 0, "table rows are requested a chunk of iterations ahead");
       const float *cs = g.rope_cos[grp], *sn = g.rope_sin[grp];
       const int64_t ss = g.rope_cs_ss[grp];
       auto table = [&](const float *tb, int it) {
         const int idx = it * NW * 64 + tid, r = idx / F4, c4 = (idx % F4) * 4;
-        return *(const float4 *)(tb + (int64_t)min(m0 + r, g.M - 1) * ss + (c4 & 63));
+        return *(const float4 *)(tb + (int64_t)(min(m0 + r, g.M - 1) % S) * ss + (c4 & (hd - 1)));
       };
-      float4 cv[AHEAD], sv[AHEAD];  // the first rows of the tables are requested before the tile is exchanged
+      // Table rows are requested a chunk of iterations ahead of their use (the first chunk before the tile is
+      // exchanged): behind the stores of the iteration before, each would cost a trip to L2 of its own.
+      float4 cv[2][CH], sv[2][CH];
 #pragma unroll
-      for (int it = 0; it < AHEAD; ++it) {
-        cv[it] = table(cs, it);
-        sv[it] = table(sn, it);
+      for (int u = 0; u < CH; ++u) {
+        cv[0][u] = table(cs, u);
+        sv[0][u] = table(sn, u);
       }
       float *tile = (float *)dma_smem;
       __syncthreads();  // every wave is done with the last stage
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
+        for (int j = 0; j < TN; ++j) {
+          const int cl = wn * WN + j * 32 + (lane & 31);
+          const float bv = Bias ? Bias[min(n0 + cl, Nl - 1)] : 0.f;
 #pragma unroll
           for (int e = 0; e < 16; ++e)
-            tile[(wm * WM + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3)) * P + wn * WN + j * 32 + (lane & 31)] = acc[i][j][e];
+            tile[(wm * WM + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3)) * P + cl] = acc[i][j][e] + bv;
+        }
       __syncthreads();
+      const int half = (int)hd / 2;
 #pragma unroll
       for (int it = 0; it < ITERS; ++it) {
+        if (it % CH == 0 && it + CH < ITERS) {
+#pragma unroll
+          for (int u = 0; u < CH; ++u) {
+            cv[(it / CH + 1) & 1][u] = table(cs, it + CH + u);
+            sv[(it / CH + 1) & 1][u] = table(sn, it + CH + u);
+          }
+        }
         const int idx = it * NW * 64 + tid, r = idx / F4, c4 = (idx % F4) * 4;
         const uint32_t row = m0 + r;
-        const float4 c = it < AHEAD ? cv[it < AHEAD ? it : 0] : table(cs, it);
-        const float4 sn4 = it < AHEAD ? sv[it < AHEAD ? it : 0] : table(sn, it);
+        const float4 c = cv[(it / CH) & 1][it % CH], sn4 = sv[(it / CH) & 1][it % CH];
         const float4 xv = *(const float4 *)(tile + r * P + c4);
-        float4 pv = *(const float4 *)(tile + r * P + (c4 ^ 32));
-        if (!(c4 & 32)) { pv.x = -pv.x; pv.y = -pv.y; pv.z = -pv.z; pv.w = -pv.w; }
+        float4 pv = *(const float4 *)(tile + r * P + (c4 ^ half));
+        if (!(c4 & half)) { pv.x = -pv.x; pv.y = -pv.y; pv.z = -pv.z; pv.w = -pv.w; }
         float4 o;
         o.x = c.x * xv.x + sn4.x * pv.x; o.y = c.y * xv.y + sn4.y * pv.y;
         o.z = c.z * xv.z + sn4.z * pv.z; o.w = c.w * xv.w + sn4.w * pv.w;
         if (row < g.M) {
-          const uint64_t at = ((uint64_t)((n0 + c4) / 64) * g.rope_s + row) * 64 + (c4 & 63);
+          const uint32_t sq = row / S, pos = row - sq * S, head = (n0 + c4) / hd;
+          const uint64_t at = (((uint64_t)sq * heads + head) * S + pos) * hd + (c4 & (hd - 1));
           *(float4 *)(g.rope_out[grp] + at) = o;
           if (g.rope_out16[grp]) *(uint2 *)(g.rope_out16[grp] + at) = bf16_pack4(o);
         }
       }
       return;
     }
-    if (role == 2) {  // the values: also as bf16 [head][64][position], four consecutive positions per store
+    if (role == 2) {  // the values: also as bf16 [sequence][head][hd][position], four consecutive positions per store
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
-          const uint32_t col = n0 + wn * WN + j * 32 + (lane & 31);  // = head * 64 + column of the head
-          uint16_t *vt = g.rope_out16[grp] + (uint64_t)col * g.rope_s;
+          const uint32_t col = n0 + wn * WN + j * 32 + (lane & 31);  // = head * hd + column of the head
+          const float bv = Bias ? Bias[min(col, Nl - 1)] : 0.f;
 #pragma unroll
           for (int q = 0; q < 4; ++q) {
-            const uint32_t r0 = m0 + wm * WM + i * 32 + q * 8 + (lane >> 5) * 4;
-            if (r0 < g.M)
-              *(uint2 *)(vt + r0) = bf16_pack4(make_float4(acc[i][j][q * 4], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3]));
+            const uint32_t r0 = m0 + wm * WM + i * 32 + q * 8 + (lane >> 5) * 4;  // S % 4 == 0: the four share a sequence
+            if (r0 < g.M && col < Nl) {
+              const uint32_t sq = r0 / S, pos = r0 - sq * S;
+              *(uint2 *)(g.rope_out16[grp] + ((uint64_t)sq * Nl + col) * S + pos) =
+                  bf16_pack4(make_float4(acc[i][j][q * 4] + bv, acc[i][j][q * 4 + 1] + bv, acc[i][j][q * 4 + 2] + bv, acc[i][j][q * 4 + 3] + bv));
+            }
           }
         }
     }
@@ -793,10 +812,11 @@ __global__ void __launch_bounds__(WR *WC * 64) gemm_bf16_dma_kernel(GemmDesc g) 
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
       const uint32_t col = n0 + wn * WN + j * 32 + (lane & 31);
+      const float bv = Bias ? Bias[min(col, Nl - 1)] : 0.f;
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
         const uint32_t row = m0 + wm * WM + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
-        if (row < g.M && col < Nl) C[(uint64_t)row * Nl + col] = acc[i][j][e];
+        if (row < g.M && col < Nl) C[(uint64_t)row * Nl + col] = acc[i][j][e] + bv;
       }
     }
 }
@@ -2517,10 +2537,11 @@ bool gemm_epilogue_ok(const GemmDesc &g) {
 
 bool gemm_rope_epilogue_ok(const LaunchCtx &lc, const GemmDesc &g) {
   if (!g.rope_s || !g.n_group || !gemm_epilogue_ok(g)) return false;
-  if (g.nb0 * g.nb1 != 1 || g.glu_gate || g.c16 || g.dual_b || g.M != g.rope_s || g.M % 4 || g.M < 64) return false;
+  if (g.rope_hd != 64 && g.rope_hd != 128) return false;
+  if (g.nb0 * g.nb1 != 1 || g.glu_gate || g.c16 || g.dual_b || g.M % g.rope_s || g.rope_s % 4 || g.M < 64) return false;
   bool grp256 = true;
   for (uint32_t p = 0; p < g.n_group; ++p) {
-    if (g.grp_n[p] % 64) return false;
+    if (g.grp_n[p] % 128) return false;
     grp256 = grp256 && g.grp_n[p] % 256 == 0;
     if (g.rope_role[p] == 1) {
       if (!g.rope_out[p] || !g.rope_cos[p] || !g.rope_sin[p]) return false;
@@ -2530,12 +2551,10 @@ bool gemm_rope_epilogue_ok(const LaunchCtx &lc, const GemmDesc &g) {
       return false;
     }
   }
-  // launch_matmul's tiles of 128 rows have this epilogue (128 columns, or 64 where those are too few for the
-  // CUs); the 256 x 256 tile of the largest problems has not
+  // launch_matmul's tiles of 128 rows have this epilogue (128 columns, or 64 - for heads of 64 - where those are
+  // too few for the CUs); the 256 x 256 tile of the largest problems has not
   const uint64_t t256 = (uint64_t)((g.M + 255) / 256) * ((g.N + 255) / 256);
   if (t256 >= (uint64_t)lc.n_cus && grp256) return false;
-  for (uint32_t p = 0; p < g.n_group; ++p)
-    if (g.grp_n[p] % 128) return false;
   return g.N >= 128;
 }
 
@@ -2747,7 +2766,9 @@ hipError_t launch_matmul(const LaunchCtx &lc_in, const GemmDesc &g, const char *
       } else if (splits == 1 && t128 * 2 <= (uint64_t)lc.n_cus && g.N >= 128) {
         // too few 128 x 128 tiles for the CUs and no split-K to multiply them: halve the tile
         const uint32_t t64 = (uint32_t)((uint64_t)((g.M + 127) / 128) * ((g.N + 63) / 64) * batch);
-        if (g.rope_s) e = launch_gemm_dma<128, 64, 4, 2, false, 4, false, false, true>(lc, gg, t64);
+        // (heads of 128 columns need the whole head in one tile)
+        if (g.rope_s && g.rope_hd > 64) e = launch_gemm_dma<128, 128, 2, 4, false, 4, false, false, true>(lc, gg, (uint32_t)t128);
+        else if (g.rope_s) e = launch_gemm_dma<128, 64, 4, 2, false, 4, false, false, true>(lc, gg, t64);
         else e = launch_gemm_dma<128, 64, 4, 2, false, 4>(lc, gg, t64);
       } else if (deep) {
         if (g.rope_s) e = launch_gemm_dma<128, 128, 2, 4, false, 4, false, false, true>(lc, gg, (uint32_t)t128);

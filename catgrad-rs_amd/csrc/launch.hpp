@@ -298,12 +298,15 @@ struct GemmDesc {
   const void *grp_b[3];
   float *grp_c[3];
   uint32_t grp_n[3];
-  // optional, with n_group (gemm_rope_epilogue_ok): the products are the q / k / v projections of one batch of
-  // rope_s positions with heads of 64 columns, row m being position m.  A group with rope_role 1 leaves the
-  // kernel rotated (apply_rope_embedding, cos / sin rows of 64 at rope_cs_ss apart) as [head][position][64] at
+  // optional, with n_group: a vector of grp_n[p] floats added to every row of product p (the bias of a linear)
+  const float *grp_bias[3];
+  // optional, with n_group (gemm_rope_epilogue_ok): the products are the q / k / v projections of M / rope_s
+  // sequences of rope_s positions each (row m = sequence m / rope_s, position m % rope_s) with heads of rope_hd
+  // (64 or 128) columns.  A group with rope_role 1 leaves the kernel rotated (apply_rope_embedding, cos / sin
+  // rows of rope_hd floats at rope_cs_ss apart, indexed by position) as [sequence][head][position][rope_hd] at
   // rope_out (f32) and rope_out16 (bf16, optional) instead of grp_c; a group with rope_role 2 is stored as usual
-  // and also transposed, as bf16 [head][64][position], at rope_out16.
-  uint32_t rope_s;
+  // and also transposed, as bf16 [sequence][head][rope_hd][position], at rope_out16.
+  uint32_t rope_s, rope_hd;
   uint32_t rope_role[3];
   float *rope_out[3];
   uint16_t *rope_out16[3];

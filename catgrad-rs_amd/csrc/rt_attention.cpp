@@ -41,7 +41,7 @@ int try_attn_prefill(cg_backend *be, cg_tensor *n, bool *done) {
   if (cg_tensor *kr = node_under_repeat_kv(S->in[1])) {
     bool paired = false;
     // ... or none at all: the projections still deferred rotate q and k in their epilogue
-    if (!f32 && d == 64 && nb == 1) TRY(try_qkv_rope_gemm(be, q, kr, node_under_repeat_kv(n->in[1]), &vt_made.s, &vt_of, &paired));
+    if (!f32 && (d == 64 || d == 128)) TRY(try_qkv_rope_gemm(be, q, kr, node_under_repeat_kv(n->in[1]), &vt_made.s, &vt_of, &paired));
     if (!paired) TRY(try_rope_pair(be, q, kr, &paired));
   }
   MatOperand Kop, Vop;
@@ -111,7 +111,7 @@ int try_attn_prefill(cg_backend *be, cg_tensor *n, bool *done) {
     a.k16 = (const uint16_t *)ksh->ptr + Kop.t->offset;
     // the values as the projections left them, [T, kv heads * d] read as [kv heads][T][d]: their transposed copy is there
     if (vt_made.s && vt_of == Vop.t->st && Vop.t->offset == 0 && Vop.strides[1] == d && Vop.strides[3] == kvh * d &&
-        Vop.strides[4] == 1 && (size_t)kvh * d * T * 2 <= vt_made.s->bytes) {
+        Vop.strides[4] == 1 && (nb == 1 || Vop.strides[0] == T * kvh * d) && (size_t)nb * kvh * d * T * 2 <= vt_made.s->bytes) {
       vt = vt_made.s;
       vt_made.s = nullptr;
       vt_ready = true;

@@ -470,11 +470,12 @@ int binary(cg_backend *be, cg_tensor *a, cg_tensor *b, cg_tensor **out, EwOp f_o
       block_end = dense;
     }
   }
-  // `linear(x) + bias` on a few rows: the product's launch can add the bias itself (try_gemv_prologue)
+  // `linear(x) + bias`: the product's launch can add the bias itself (a few rows: try_gemv_prologue; many rows
+  // in bf16 mode: the grouped q / k / v launch of realize_matmul)
   if (n->ew == E_ADD_F && !(be->flags & (CG_FLAG_EAGER | CG_FLAG_NO_PATTERNS))) {
     for (int side = 0; side < 2; ++side) {
       cg_tensor *mm = n->in[side], *other = n->in[1 - side];
-      if (mm->op == N_MATMUL && mm->gemv_candidate && !mm->bias_user && bias_vector_of(other, n) != nullptr) {
+      if (mm->op == N_MATMUL && (mm->gemv_candidate || mm->gemm_candidate) && !mm->bias_user && bias_vector_of(other, n) != nullptr) {
         mm->bias_user = n;
         n->bias_of = mm;
         break;

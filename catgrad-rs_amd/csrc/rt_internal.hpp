@@ -509,11 +509,11 @@ struct RopeMatch {
 // launch sets `applied` when it did.
 struct RopeGemmRequest {
   cg_tensor *mm[3] = {nullptr, nullptr, nullptr};  // the products: q, k, v
-  float *out[2] = {nullptr, nullptr};              // rotated q, k: [heads][positions][64]
-  uint16_t *out16[3] = {nullptr, nullptr, nullptr};  // their bf16 copies (optional); [2]: v as [heads][64][positions]
+  float *out[2] = {nullptr, nullptr};              // rotated q, k: [sequences][heads][positions][head_dim]
+  uint16_t *out16[3] = {nullptr, nullptr, nullptr};  // their bf16 copies (optional); [2]: v as [sequences][heads][head_dim][positions]
   const float *cos[2] = {nullptr, nullptr}, *sin[2] = {nullptr, nullptr};
   int64_t cs_ss[2] = {0, 0};
-  uint32_t positions = 0;
+  uint32_t positions = 0, head_dim = 0;
   bool applied = false;
 };
 

@@ -943,8 +943,9 @@ int realize_matmul(cg_backend *be, cg_tensor *n, cg_tensor *addend, bool *added,
     }
     // q/k/v of a prefill: the other deferred many-row products on the same left operand join this
     // launch as further column ranges (their own weights, their own outputs)
-    std::vector<cg_tensor *> group;
-    if (n->gemm_candidate && !addend && !ep && !ex.w && batch == 1 && g.bf16_math && g.a_stype == ST_BF16 &&
+    std::vector<cg_tensor *> group, group_add, group_bias;  // a member, the add that takes its value, its bias vector
+    const bool bias_row = addend && be->addend_is_row;  // `addend` is a vector added to every row
+    if (n->gemm_candidate && (!addend || bias_row) && !ep && !ex.w && batch == 1 && g.bf16_math && g.a_stype == ST_BF16 &&
         g.b_stype == ST_BF16 && g.sbk == 1 && N % 128 == 0 && gemm_epilogue_ok(g)) {
       // the same rows: one node, or - each linear folding the batch itself - dense reshapes of one value
       auto dense_view = [](const cg_tensor *t, const Storage **st, int64_t *off) {
@@ -967,7 +968,18 @@ int realize_matmul(cg_backend *be, cg_tensor *n, cg_tensor *addend, bool *added,
         if (w->op != N_REAL || w->rank != 3 || w->stype != ST_BF16 || w->shape[0] != 1) continue;
         if (w->shape[1] != (int64_t)K || w->strides[1] != 1 || w->strides[2] != g.sbn) continue;
         if (w->shape[2] % 128 || (uintptr_t)data_ptr(w) % 16) continue;
+        // a sibling whose only reader adds a bias vector to it: the launch stores the sum, as that add's value
+        cg_tensor *add = c->bias_user, *bv = nullptr;
+        if (add) {
+          if (refs(c) != 1 || add->op != N_BIN || add->bias_of != c || add->size() != c->size()) continue;
+          bv = bias_vector_of(add->in[add->in[0] == c ? 1 : 0], add);
+          if (!bv) continue;
+          TRY(realize(be, bv));
+          if (!bias_vector_ready(bv)) continue;
+        }
         group.push_back(c);
+        group_add.push_back(add);
+        group_bias.push_back(bv);
       }
       if (group.size() < 2) group.clear();  // pairs (gate / up) keep their own launches and epilogues
     }
@@ -976,10 +988,16 @@ int realize_matmul(cg_backend *be, cg_tensor *n, cg_tensor *addend, bool *added,
       g.grp_b[0] = g.b;
       g.grp_c[0] = g.c;
       g.grp_n[0] = N;
-      for (cg_tensor *c : group) {
-        TRY(alloc_result(be, c, ST_F32));
+      if (bias_row) {
+        g.grp_bias[0] = (const float *)data_ptr(addend);
+        *added = true;
+      }
+      for (size_t i = 0; i < group.size(); ++i) {
+        cg_tensor *c = group[i], *dest = group_add[i] ? group_add[i] : c;
+        TRY(alloc_result(be, dest, ST_F32));
         g.grp_b[g.n_group] = data_ptr(c->in[1]);
-        g.grp_c[g.n_group] = (float *)c->st->ptr;
+        g.grp_c[g.n_group] = (float *)dest->st->ptr;
+        g.grp_bias[g.n_group] = group_bias[i] ? (const float *)data_ptr(group_bias[i]) : nullptr;
         g.grp_n[g.n_group] = (uint32_t)c->in[1]->shape[2];
         g.N += g.grp_n[g.n_group];
         ++g.n_group;
@@ -1007,6 +1025,7 @@ int realize_matmul(cg_backend *be, cg_tensor *n, cg_tensor *addend, bool *added,
         }
       }
       t.rope_s = rq->positions;
+      t.rope_hd = rq->head_dim;
       if (all && gemm_rope_epilogue_ok(be->lc(), t)) {
         g = t;
         rq->applied = true;
@@ -1065,7 +1084,17 @@ int realize_matmul(cg_backend *be, cg_tensor *n, cg_tensor *addend, bool *added,
         ks.rename(buf);
       }
     }
-    for (cg_tensor *c : group) {
+    for (size_t i = 0; i < group.size(); ++i) {
+      if (group_add[i]) {  // the add holds the value; letting go of its inputs deletes the product node
+        if (e == hipSuccess) {
+          finish_fused(group_add[i]);
+        } else {
+          storage_release(group_add[i]->st);
+          group_add[i]->st = nullptr;
+        }
+        continue;
+      }
+      cg_tensor *c = group[i];
       forget_gemm_candidate(c);
       c->op = N_REAL;
       drop_inputs(c);

@@ -690,11 +690,12 @@ int try_rope_pair(cg_backend *be, cg_tensor *rq, cg_tensor *rk, bool *done) {
 }
 
 // The queries, keys and values of a prefill attention whose projections are all still deferred (models/llama.rs:77-94:
-// three linears on one input, `reshape [b, s, heads, d]`, `transpose(1, 2)`, then apply_rope_embedding on q and k):
-// the grouped launch of the three products rotates q and k where they are still accumulators and stores a
-// transposed bf16 copy of v beside v itself, so neither the rotation nor the transposition is a launch of its own.
-// Heads of 64 columns, one batch.  *done = false: nothing was changed beyond realising the products.
-// On success *vt owns the transposed values ([kv heads][64][positions], bf16) of the storage *v_st.
+// three linears on one input - with or without a bias -, `reshape [b, s, heads, d]`, `transpose(1, 2)`, then
+// apply_rope_embedding on q and k): the grouped launch of the three products rotates q and k where they are still
+// accumulators and stores a transposed bf16 copy of v beside v itself, so neither the rotation nor the
+// transposition is a launch of its own.  Heads of 64 or 128 columns; the linears see the batch folded into the rows.
+// *done = false: nothing was changed beyond realising the products.  On success *vt owns the transposed values
+// ([sequences][kv heads][d][positions], bf16) of the storage *v_st.
 int try_qkv_rope_gemm(cg_backend *be, cg_tensor *rq, cg_tensor *rk, cg_tensor *v, Storage **vt, const Storage **v_st,
                       bool *done) {
   *done = false;
@@ -704,21 +705,29 @@ int try_qkv_rope_gemm(cg_backend *be, cg_tensor *rq, cg_tensor *rk, cg_tensor *v
   if (rq == rk || rq->op == N_REAL || rk->op == N_REAL || !v || v->op == N_REAL) return CG_OK;
   RopeMatch mq, mk;
   if (!match_rope(rq, &mq) || !match_rope(rk, &mk)) return CG_OK;
-  // x = transpose(1, 2) of reshapes of a deferred product [1, s, heads * 64]; `readers`: the references x must
-  // have (the rotation reads it three times and nobody else may: its product is never stored as such), 0 = any
-  auto product_under = [](cg_tensor *x, int readers) -> cg_tensor * {
+  const int64_t hd = rq->shape[3];
+  if (hd != 64 && hd != 128) return CG_OK;
+  // x = transpose(1, 2) of reshapes of a deferred product [1, b * s, heads * hd], or of that product plus its bias
+  // vector; `readers`: the references x must have (the rotation reads it three times and nobody else may: its
+  // product is never stored as such), 0 = any.  *top: the node whose realisation launches the product.
+  auto product_under = [hd](cg_tensor *x, int readers, cg_tensor **top) -> cg_tensor * {
     if (x->op != N_TRANSPOSE || x->rank != 4 || (readers && refs(x) != readers)) return nullptr;
-    if (!((x->p0 == 1 && x->p1 == 2) || (x->p0 == 2 && x->p1 == 1)) || x->shape[0] != 1 || x->shape[3] != 64) return nullptr;
+    if (!((x->p0 == 1 && x->p1 == 2) || (x->p0 == 2 && x->p1 == 1)) || x->shape[3] != hd) return nullptr;
     cg_tensor *t = x->in[0];
     while (t->op == N_RESHAPE && (!readers || refs(t) == 1)) t = t->in[0];
+    *top = t;
+    if (t->op == N_BIN && t->bias_of && (!readers || refs(t) == 1) && (t->in[0] == t->bias_of || t->in[1] == t->bias_of)) t = t->bias_of;
     if (t->op != N_MATMUL || (readers && refs(t) != 1) || !t->gemm_candidate || t->dtype != CG_F32 || t->rank != 3) return nullptr;
-    if (t->shape[0] != 1 || t->shape[1] != x->shape[2] || t->shape[2] != x->shape[1] * 64) return nullptr;
+    if (t->shape[0] != 1 || t->shape[1] != x->shape[0] * x->shape[2] || t->shape[2] != x->shape[1] * hd) return nullptr;
     return t;
   };
-  cg_tensor *pq = product_under(mq.x, 3), *pk = product_under(mk.x, 3), *pv = product_under(v, 0);
+  cg_tensor *top_q = nullptr, *top_k = nullptr, *top_v = nullptr;
+  cg_tensor *pq = product_under(mq.x, 3, &top_q), *pk = product_under(mk.x, 3, &top_k), *pv = product_under(v, 0, &top_v);
   if (!pq || !pk || !pv || pq == pk || pq == pv || pk == pv) return CG_OK;
-  const int64_t positions = pq->shape[1];
-  if (pk->shape[1] != positions || pv->shape[1] != positions || pk->shape[2] != pv->shape[2] || positions % 4) return CG_OK;
+  const int64_t positions = rq->shape[2], seqs = rq->shape[0];
+  if (rk->shape[2] != positions || rk->shape[0] != seqs || v->shape[2] != positions || v->shape[0] != seqs ||
+      pk->shape[2] != pv->shape[2] || positions % 4)
+    return CG_OK;
   bool tq = false, tk = false;
   TRY(rope_tables(be, mq, &tq));
   TRY(rope_tables(be, mk, &tk));
@@ -734,20 +743,21 @@ int try_qkv_rope_gemm(cg_backend *be, cg_tensor *rq, cg_tensor *rk, cg_tensor *v
       req.out[i] = (float *)roots[i]->st->ptr;
       req.cos[i] = (const float *)data_ptr(ms[i]->cb);
       req.sin[i] = (const float *)data_ptr(ms[i]->sb);
-      req.cs_ss[i] = ms[i]->cb->strides[2];
+      req.cs_ss[i] = positions == 1 ? 0 : ms[i]->cb->strides[2];
     }
   }
   Storage *t = nullptr;
-  if (!st) st = dev_alloc(be, (size_t)pv->shape[2] * positions * 2, &t);
+  if (!st) st = dev_alloc(be, (size_t)pv->shape[1] * pv->shape[2] * 2, &t);
   if (!st) {
     req.out16[2] = (uint16_t *)t->ptr;
     req.mm[0] = pq;
     req.mm[1] = pk;
     req.mm[2] = pv;
     req.positions = (uint32_t)positions;
-    cg_tensor *keep = retain(pv);  // (the products leave the graph as they are realised)
+    req.head_dim = (uint32_t)hd;
+    cg_tensor *keep = retain(top_v);  // (the products leave the graph as they are realised)
     be->rope_request = &req;
-    st = realize(be, pq);
+    st = realize(be, top_q);
     be->rope_request = nullptr;
     if (!st && req.applied && keep->op == N_REAL) *v_st = keep->st;
     node_release(keep);
@@ -976,8 +986,11 @@ int try_gemv_add(cg_backend *be, cg_tensor *root, bool *done) {
     bool added = false;
     // (a single row in memory goes the residual's way below: every one-row kernel can add that)
     const bool plain_row = other->op == N_REAL && other->stype == ST_F32 && is_contiguous(other);
-    if (cg_tensor *bv = (!folded && !plain_row && mm->gemv_candidate) ? bias_vector_of(other, root) : nullptr) {
-      // linear(x) + bias on a few rows: the grouped product launch adds the vector to every row
+    if (cg_tensor *bv = (!folded && !plain_row && (mm->gemv_candidate || (mm->gemm_candidate && mm->bias_user == root)))
+                            ? bias_vector_of(other, root)
+                            : nullptr) {
+      // linear(x) + bias: the grouped product launch adds the vector to every row (few rows: always; many rows:
+      // where q / k / v go out as one launch - otherwise *added stays false and the add runs as an op of its own)
       TRY(realize(be, bv));
       if (!bias_vector_ready(bv)) return CG_OK;
       be->addend_is_row = true;

@@ -615,6 +615,51 @@ def test_moe_cached_decode_hip_vs_oracle(oracle, hip, hip_bf16, mode):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("batch,tokens,heads,kv_heads,head_dim", [(2, 256, 2, 2, 128), (1, 320, 4, 2, 128), (3, 256, 4, 4, 64)])
+def test_qwen_prefill_biases_and_rotation_in_the_projections_launch(oracle, hip_bf16, batch, tokens, heads, kv_heads, head_dim):
+    """bf16 prefill of the Qwen layout (q/k/v linears with biases on the batch folded into the rows, qwen3.rs:64-133 /
+    models/llama.rs:77-94): one grouped launch adds the three biases, rotates q and k and leaves the transposed bf16
+    values - the trace has no bias add, rotation or transposition of its own.  Every token goes to every expert
+    (k = E), so the routing has no ties to flip and the caches, the prefill's logits and a decode step's are held
+    to the bf16 bar against the oracle on rounded parameters."""
+    cfg = MU.qwen_moe_config(hidden_size=heads * head_dim, num_hidden_layers=2, num_attention_heads=heads,
+                             num_key_value_heads=kv_heads, head_dim=head_dim, num_experts=4, num_experts_per_tok=4, vocab_size=211)
+    P = MU.qwen_moe_params(cfg, seed=31, std=0.04)
+    P_ref = {k: (U_round(v) if v.ndim >= 2 else v) for k, v in P.items()}
+    prompts = np.random.default_rng(32).integers(0, cfg.vocab_size, (batch, tokens))
+    runners = [U.CachedRunner(be, cfg, arrays, tokens + 8, prefill_cls=llm.qwen_moe.QwenMoePrefill,
+                              decode_cls=llm.qwen_moe.QwenMoeDecode) for be, arrays in ((oracle, P_ref), (hip_bf16, P))]
+    rt, rl = runners[0].prefill(prompts)
+    hip_bf16.trace(2)
+    hip_bf16.trace_reset()
+    gt, gl = runners[1].prefill(prompts)
+    gl = hip_bf16.numpy(gl)
+    rep = hip_bf16.trace_report()
+    names = sorted(rep)
+    hip_bf16.trace(False)
+    parity.assert_bf16(oracle.numpy(rl), gl, "prefill logits")
+    assert sum("grouped,rope" in n for n in names) == 1, names
+    assert not any(n.startswith(("rope_fused", "transpose_cast_bf16")) for n in names), names
+    # (at most the two residual adds of a layer are launches of their own at this size; the three bias adds are not)
+    assert rep.get("binary_f32", {"launches": 0})["launches"] <= 2 * cfg.num_hidden_layers, {k: v["launches"] for k, v in rep.items()}
+    # The first layer's caches are that launch's own output on exact inputs: the bar.  Deeper layers see the bf16
+    # rounding of a whole block first (the rounded queries and keys move the attention's scores by absolute amounts,
+    # which positions with a sharp softmax amplify past the bar; f32 mode agrees to 1e-4, and the unfused kernels
+    # give the same values bit for bit): there the typical position is held to it.
+    for layer in range(cfg.num_hidden_layers):
+        for which, what in ((0, "rotated keys"), (1, "values")):
+            ref, got = oracle.numpy(runners[0].kv[2 * layer + which]), hip_bf16.numpy(runners[1].kv[2 * layer + which])
+            if layer == 0:
+                parity.assert_bf16(ref, got, f"layer {layer} {what}")
+            else:
+                assert np.median(parity.per_row_bf16(ref, got)) <= parity.RTOL_BF16, (layer, what)
+    tok = oracle.to_vec(rt).reshape(-1)
+    _, rl = runners[0].step(tok)
+    _, gl = runners[1].step(tok)
+    parity.assert_bf16(oracle.numpy(rl), hip_bf16.numpy(gl), "decode step on the prefill's caches")
+
+
+@pytest.mark.gpu
 def test_generic_program_launches_of_the_other_decoders(hip_bf16):
     """Which launches of a Gemma-3 prefill and of a Qwen-MoE-layout decode step are generic programs:
     the embedding scale (one per Gemma run); everything else is a pattern kernel - the weighted sum of the
