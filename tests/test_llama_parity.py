@@ -139,14 +139,14 @@ def test_llama_prefill_of_many_rows(oracle, hip, hip_bf16):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("tokens,heads,kv_heads,layers", [(256, 8, 2, 2), (320, 4, 4, 2), (300, 4, 2, 2), (512, 16, 2, 2),
-                                                         (1280, 16, 8, 1), (2048, 32, 16, 1)])
+                                                         (1280, 16, 8, 1), (2048, 16, 16, 1), (2048, 32, 16, 1)])
 def test_llama_prefill_rotates_in_the_projections_launch(oracle, hip_bf16, tokens, heads, kv_heads, layers):
     """bf16 prefill with heads of 64 (models/llama.rs:77-94, helpers.rs:195-221): the grouped q/k/v launch leaves the
     queries and keys rotated and a transposed bf16 copy of the values, so the trace holds neither a rotation nor a
     transposition of its own.  The caches it returns (rotated keys, values) and the logits of the prefill and of a
     decode step that reads those caches are held to the bf16 bar against the oracle on rounded parameters.  The
-    sizes cover the three tiles the launch may choose (128 x 64, and 128 x 128 with eight or four waves) and a
-    prompt that ends inside a tile."""
+    sizes cover the tiles the launch may choose (128 x 64; 128 x 128 with eight waves, one or two workgroups to a
+    CU, or with four waves) and a prompt that ends inside a tile."""
     cfg = U.tiny_config(hidden_size=64 * heads, intermediate_size=512, num_hidden_layers=layers,
                         num_attention_heads=heads, num_key_value_heads=kv_heads, vocab_size=300)
     arrays = U.param_arrays(cfg, seed=21, std=0.05)

@@ -615,7 +615,8 @@ def test_moe_cached_decode_hip_vs_oracle(oracle, hip, hip_bf16, mode):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("batch,tokens,heads,kv_heads,head_dim", [(2, 256, 2, 2, 128), (1, 320, 4, 2, 128), (3, 256, 4, 4, 64)])
+@pytest.mark.parametrize("batch,tokens,heads,kv_heads,head_dim", [(2, 256, 2, 2, 128), (1, 320, 4, 2, 128), (3, 256, 4, 4, 64),
+                                                                  (4, 512, 8, 8, 128)])
 def test_qwen_prefill_biases_and_rotation_in_the_projections_launch(oracle, hip_bf16, batch, tokens, heads, kv_heads, head_dim):
     """bf16 prefill of the Qwen layout (q/k/v linears with biases on the batch folded into the rows, qwen3.rs:64-133 /
     models/llama.rs:77-94): one grouped launch adds the three biases, rotates q and k and leaves the transposed bf16
