@@ -679,14 +679,60 @@ __device__ __forceinline__ void rope_rows(const RopeDesc &d, uint32_t block, uin
   }
 }
 
+// The same with every row normed on its way in (gemma3.rs:99-117: q and k are RMS-normed per head between the head
+// transpose and the rotation): LPR = dim / 4 lanes hold a row, sum its squares among themselves, and a lane
+// gets its partner half a row away from lane ^ (LPR / 2).  The normed rows are never stored.
+template <int LPR>
+__device__ __forceinline__ void rope_norm_rows(const RopeDesc &d, uint32_t block, uint32_t n_blocks) {
+  const uint64_t total = (uint64_t)d.b * d.h * d.s * LPR;  // a multiple of LPR, as 256 is: a row's lanes stay together
+  for (uint64_t i = (uint64_t)block * 256 + threadIdx.x; i < total; i += (uint64_t)n_blocks * 256) {
+    const uint32_t j = (uint32_t)(i % LPR) * 4;
+    uint64_t r = i / LPR;
+    const uint32_t s = (uint32_t)(r % d.s);
+    r /= d.s;
+    const uint32_t h = (uint32_t)(r % d.h), b = (uint32_t)(r / d.h);
+    const float4 xv = *(const float4 *)(d.x + (int64_t)b * d.x_sb + (int64_t)h * d.x_sh + (int64_t)s * d.x_ss + j);
+    const float4 c = *(const float4 *)(d.cos + (int64_t)s * d.cs_ss + j);
+    const float4 sn = *(const float4 *)(d.sin + (int64_t)s * d.cs_ss + j);
+    float4 g = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (d.gamma) g = *(const float4 *)(d.gamma + j);
+    float ss = xv.x * xv.x + xv.y * xv.y + xv.z * xv.z + xv.w * xv.w;
+    ss = group_sum<LPR>(ss);
+    const float rms = sqrtf(ss / d.n_as_float + d.eps);  // (a true square root and true divisions, as in rmsnorm_kernel)
+    float4 y;
+    y.x = xv.x / rms; y.y = xv.y / rms; y.z = xv.z / rms; y.w = xv.w / rms;
+    if (d.gamma) {
+      y.x *= d.gamma_offset + g.x; y.y *= d.gamma_offset + g.y;
+      y.z *= d.gamma_offset + g.z; y.w *= d.gamma_offset + g.w;
+    }
+    float4 pv;
+    pv.x = __shfl_xor(y.x, LPR / 2); pv.y = __shfl_xor(y.y, LPR / 2);
+    pv.z = __shfl_xor(y.z, LPR / 2); pv.w = __shfl_xor(y.w, LPR / 2);
+    if (j < d.half) { pv.x = -pv.x; pv.y = -pv.y; pv.z = -pv.z; pv.w = -pv.w; }
+    float4 o;
+    o.x = c.x * y.x + sn.x * pv.x; o.y = c.y * y.y + sn.y * pv.y;
+    o.z = c.z * y.z + sn.z * pv.z; o.w = c.w * y.w + sn.w * pv.w;
+    const int64_t oo = (int64_t)b * d.o_sb + (int64_t)h * d.o_sh + (int64_t)s * d.o_ss + j;
+    *(float4 *)(d.out + oo) = o;
+    if (d.out16) *(uint2 *)(d.out16 + oo) = bf16_pack4(o);
+  }
+}
+
+__device__ __forceinline__ void rope_any_rows(const RopeDesc &d, uint32_t block, uint32_t n_blocks) {
+  if (!d.norm) rope_rows(d, block, n_blocks);
+  else if (d.dim == 256) rope_norm_rows<64>(d, block, n_blocks);
+  else if (d.dim == 128) rope_norm_rows<32>(d, block, n_blocks);
+  else rope_norm_rows<16>(d, block, n_blocks);
+}
+
 __global__ void __launch_bounds__(256) rope_kernel(RopeDesc d) {
-  rope_rows(d, blockIdx.x, gridDim.x);
+  rope_any_rows(d, blockIdx.x, gridDim.x);
 }
 
 // queries and keys of one attention in one launch: the first blocks0 workgroups rotate d0, the rest d1
 __global__ void __launch_bounds__(256) rope_pair_kernel(RopeDesc d0, RopeDesc d1, uint32_t blocks0) {
-  if (blockIdx.x < blocks0) rope_rows(d0, blockIdx.x, blocks0);
-  else rope_rows(d1, blockIdx.x - blocks0, gridDim.x - blocks0);
+  if (blockIdx.x < blocks0) rope_any_rows(d0, blockIdx.x, blocks0);
+  else rope_any_rows(d1, blockIdx.x - blocks0, gridDim.x - blocks0);
 }
 
 static unsigned rope_blocks(const LaunchCtx &lc, const RopeDesc &d) {
@@ -696,6 +742,7 @@ static unsigned rope_blocks(const LaunchCtx &lc, const RopeDesc &d) {
 }
 
 hipError_t launch_rope(const LaunchCtx &lc, const RopeDesc &d) {
+  if (d.norm && d.dim != 64 && d.dim != 128 && d.dim != 256) return hipErrorInvalidValue;
   const unsigned blocks = rope_blocks(lc, d);
   if (!blocks) return hipSuccess;
   CG_LAUNCH(lc, (rope_kernel), blocks, 256, d);
@@ -703,6 +750,8 @@ hipError_t launch_rope(const LaunchCtx &lc, const RopeDesc &d) {
 }
 
 hipError_t launch_rope_pair(const LaunchCtx &lc, const RopeDesc &d0, const RopeDesc &d1) {
+  for (const RopeDesc *d : {&d0, &d1})
+    if (d->norm && d->dim != 64 && d->dim != 128 && d->dim != 256) return hipErrorInvalidValue;
   const unsigned b0 = rope_blocks(lc, d0), b1 = rope_blocks(lc, d1);
   if (!b0) return launch_rope(lc, d1);
   if (!b1) return launch_rope(lc, d0);

@@ -812,11 +812,19 @@ __global__ void __launch_bounds__(WR *WC * 64) gemm_bf16_dma_kernel(GemmDesc g) 
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
       const uint32_t col = n0 + wn * WN + j * 32 + (lane & 31);
-      const float bv = Bias ? Bias[min(col, Nl - 1)] : 0.f;
+      if (Bias) {
+        const float bv = Bias[min(col, Nl - 1)];
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const uint32_t row = m0 + wm * WM + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
+          if (row < g.M && col < Nl) C[(uint64_t)row * Nl + col] = acc[i][j][e] + bv;
+        }
+        continue;
+      }
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
         const uint32_t row = m0 + wm * WM + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
-        if (row < g.M && col < Nl) C[(uint64_t)row * Nl + col] = acc[i][j][e] + bv;
+        if (row < g.M && col < Nl) C[(uint64_t)row * Nl + col] = acc[i][j][e];
       }
     }
 }

@@ -148,6 +148,11 @@ struct RopeDesc {
   int64_t o_sb, o_sh, o_ss;
   uint16_t *out16;       // optional bf16 copy, same layout as out, or null
   uint32_t b, h, s, dim, half;
+  // optional (norm != 0, dim 64, 128 or 256): every row of x is RMS-normed first, the arithmetic of rmsnorm_kernel -
+  // x / sqrt(sum(x * x) / n_as_float + eps) * (gamma_offset + gamma), gamma: dim floats or null
+  int32_t norm;
+  const float *gamma;
+  float n_as_float, eps, gamma_offset;
 };
 hipError_t launch_rope(const LaunchCtx &lc, const RopeDesc &d);
 // two rotations (the queries and the keys of an attention) as one launch

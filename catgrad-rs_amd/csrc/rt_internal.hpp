@@ -48,6 +48,7 @@ struct RowMap;
 struct SoftmaxMatch;
 struct RmsNormMatch;
 struct RopeMatch;
+struct RopeNormed;
 struct MatmulEpilogue;
 struct MatOperand;
 struct ExpertPeel;
@@ -121,7 +122,7 @@ int rope_into(cg_backend *be, cg_tensor *root, const RopeMatch &m, float *out, c
               const char *name, bool *done, uint16_t *out16 = nullptr);
 int try_rope(cg_backend *be, cg_tensor *root, bool *done);
 int rope_describe(cg_backend *be, cg_tensor *root, const RopeMatch &m, float *out, const int64_t *o_strides,
-                  uint16_t *out16, RopeDesc *dsc, cg_tensor **xs_out, bool *ok);
+                  uint16_t *out16, RopeDesc *dsc, cg_tensor **xs_out, bool *ok, const RopeNormed *normed = nullptr);
 int try_rope_pair(cg_backend *be, cg_tensor *rq, cg_tensor *rk, bool *done);
 int try_qkv_rope_gemm(cg_backend *be, cg_tensor *rq, cg_tensor *rk, cg_tensor *v, Storage **vt, const Storage **v_st,
                       bool *done);
@@ -502,6 +503,15 @@ struct RmsNormMatch {
 // apply_rope_embedding (catgrad-llm/src/helpers.rs:195-221): cos * x + sin * rotate_half(x)
 struct RopeMatch {
   cg_tensor *cb = nullptr, *sb = nullptr, *x = nullptr;  // cos / sin broadcasts, the rotated tensor
+};
+
+// The rotated tensor of a RopeMatch as the RMS norm of `view` ([b, h, s, d], realised), read by nothing but the
+// rotation: the rotation's kernel norms each row on its way in (rope_normed_input).
+struct RopeNormed {
+  bool on = false;
+  RmsNormMatch rm;
+  cg_tensor *view = nullptr;  // not retained: the graph under the rotation holds it
+  const float *gamma = nullptr;
 };
 
 // What the q / k / v projections of a prefill are asked to do in the epilogue of their grouped launch: leave the

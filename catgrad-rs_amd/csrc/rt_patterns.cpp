@@ -580,17 +580,56 @@ int rope_operands(cg_backend *be, const RopeMatch &m, bool *ok) {
 }
 
 
+// gemma3.rs:99-117: q and k are RMS-normed per head - folded to [b * heads * s, head_dim] - between the head
+// transpose and the rotation.  When the rotated tensor of `m` is such a norm, still deferred and read by nothing
+// but the rotation, the rotation's kernel can norm each row on its way in: *out says so and holds what it reads
+// (the norm's input as a [b, h, s, d] view, realised here, and gamma).  out->on = false: not that shape.
+static int rope_normed_input(cg_backend *be, cg_tensor *root, const RopeMatch &m, RopeNormed *out) {
+  *out = RopeNormed();
+  if (be->flags & CG_FLAG_NO_PATTERNS) return CG_OK;
+  const int64_t n = root->shape[3];
+  if ((n != 64 && n != 128 && n != 256) || m.x->op == N_REAL || refs(m.x) != 3) return CG_OK;
+  cg_tensor *t = m.x;
+  while (t->op == N_RESHAPE && t->in[0] && (t == m.x || refs(t) == 1) && t->in[0]->rank >= 1 &&
+         t->in[0]->shape[t->in[0]->rank - 1] == n)
+    t = t->in[0];
+  if (t->op == N_REAL || (t != m.x && refs(t) != 1)) return CG_OK;
+  RmsNormMatch rm;
+  if (!match_rmsnorm(t, &rm)) return CG_OK;
+  cg_tensor *v = rm.x;
+  while (v->op == N_RESHAPE && v->in[0] && v->in[0]->rank >= 1 && v->in[0]->shape[v->in[0]->rank - 1] == n) v = v->in[0];
+  if (v->rank != 4 || !std::equal(v->shape, v->shape + 4, root->shape) || v->dtype != CG_F32) return CG_OK;
+  if (rm.gamma) {
+    bool vec = false;
+    TRY(gamma_row_vector(be, rm.gamma, &vec));
+    if (!vec) return CG_OK;
+  }
+  TRY(realize(be, v));
+  bool fits = v->stype == ST_F32 && v->strides[3] == 1 && (uintptr_t)data_ptr(v) % 16 == 0;
+  for (int i = 0; i < 3; ++i)
+    if (v->strides[i] % 4) fits = false;
+  if (!fits) return CG_OK;
+  out->on = true;
+  out->rm = rm;
+  out->view = v;
+  out->gamma = rm.gamma ? (const float *)data_ptr(rm.gamma) : nullptr;
+  return CG_OK;
+}
+
+
 // Fills the rope kernel's descriptor for `root` (matched as m) writing to `out` with the given element
 // strides.  *xs receives a retained tensor the descriptor reads from (release it after the launch);
 // *ok = false: layout requirements not met, nothing to launch.
 int rope_describe(cg_backend *be, cg_tensor *root, const RopeMatch &m, float *out, const int64_t *o_strides,
-                  uint16_t *out16, RopeDesc *dsc, cg_tensor **xs_out, bool *ok) {
+                  uint16_t *out16, RopeDesc *dsc, cg_tensor **xs_out, bool *ok, const RopeNormed *normed) {
   *ok = false;
   *xs_out = nullptr;
   bool tables = false;
-  TRY(rope_operands(be, m, &tables));
+  const bool nrm = normed && normed->on;
+  if (nrm) TRY(rope_tables(be, m, &tables));  // (the rotated tensor itself stays deferred: the kernel norms its input)
+  else TRY(rope_operands(be, m, &tables));
   if (!tables) return CG_OK;
-  cg_tensor *x = m.x, *cb = m.cb, *sb = m.sb;
+  cg_tensor *x = nrm ? normed->view : m.x, *cb = m.cb, *sb = m.sb;
   cg_tensor *xs = retain(x);
   bool fits = x->stype == ST_F32 && x->strides[3] == 1 && (uintptr_t)data_ptr(x) % 16 == 0;
   for (int i = 0; i < 3; ++i)
@@ -620,6 +659,13 @@ int rope_describe(cg_backend *be, cg_tensor *root, const RopeMatch &m, float *ou
   d.s = (uint32_t)root->shape[2];
   d.dim = (uint32_t)dim;
   d.half = (uint32_t)(dim / 2);
+  if (nrm) {
+    d.norm = 1;
+    d.gamma = normed->gamma;
+    d.n_as_float = normed->rm.n_as_float;
+    d.eps = normed->rm.eps;
+    d.gamma_offset = normed->rm.gamma_offset;
+  }
   *xs_out = xs;
   *ok = true;
   return CG_OK;
@@ -655,8 +701,13 @@ int try_rope_pair(cg_backend *be, cg_tensor *rq, cg_tensor *rk, bool *done) {
   RopeMatch mq, mk;
   if (!match_rope(rq, &mq) || !match_rope(rk, &mk)) return CG_OK;
   bool tq = false, tk = false;
-  TRY(rope_operands(be, mq, &tq));
-  TRY(rope_operands(be, mk, &tk));
+  RopeNormed norms[2];
+  TRY(rope_normed_input(be, rq, mq, &norms[0]));
+  TRY(rope_normed_input(be, rk, mk, &norms[1]));
+  if (norms[0].on) TRY(rope_tables(be, mq, &tq));
+  else TRY(rope_operands(be, mq, &tq));
+  if (norms[1].on) TRY(rope_tables(be, mk, &tk));
+  else TRY(rope_operands(be, mk, &tk));
   if (!tq || !tk) return CG_OK;
   cg_tensor *roots[2] = {rq, rk};
   const RopeMatch *ms[2] = {&mq, &mk};
@@ -668,10 +719,11 @@ int try_rope_pair(cg_backend *be, cg_tensor *rq, cg_tensor *rk, bool *done) {
     st = alloc_result(be, roots[i], ST_F32);
     uint16_t *y16 = nullptr;
     if (!st) st = twin_for_result(be, roots[i], &y16);
-    if (!st) st = rope_describe(be, roots[i], *ms[i], (float *)roots[i]->st->ptr, roots[i]->strides, y16, &d[i], &xs[i], &ok);
+    if (!st) st = rope_describe(be, roots[i], *ms[i], (float *)roots[i]->st->ptr, roots[i]->strides, y16, &d[i], &xs[i], &ok, &norms[i]);
   }
   if (!st && ok) {
     KernelScope ks(be, "rope_fused", (double)(rq->size() + rk->size()) * 8, 0);
+    if (be->trace_shapes && (norms[0].on || norms[1].on)) ks.rename("rope_fused[normed]");
     hipError_t e = launch_rope_pair(be->lc(), d[0], d[1]);
     if (e != hipSuccess) st = fail(be, CG_ERR_DEVICE, hipGetErrorString(e));
   }

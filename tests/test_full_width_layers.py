@@ -115,4 +115,8 @@ def test_gemma3_full_width(oracle, hip, hip_bf16, gemma_full, mode):
     gl = dev.numpy(gl)
     counts = dev.launch_counts(reset=True)
     assert counts.get("attn_prefill") == cfg.num_hidden_layers, counts
+    # q and k are normed per head by the launch that rotates them (one per layer for both): what is left of the
+    # norms is the input norm of the first layer, two sandwich pairs per layer and the final norm
+    assert counts.get("rope_fused") == cfg.num_hidden_layers, counts
+    assert counts.get("rmsnorm_fused") <= 2 * cfg.num_hidden_layers + 2, counts
     parity.assert_logits(rl, gl, mode, "Gemma-3 at full width")
