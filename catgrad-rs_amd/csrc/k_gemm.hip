@@ -98,7 +98,9 @@ template <> struct Tile<true> {
   typedef uint16_t LT;
 };
 template <> struct Tile<false> {
-  enum { BK = 16, LD = 20 };  // row pitch 80 bytes
+  // row pitch 136 bytes: the 32 rows a wave reads for one k land on the 32 even banks, the rows of k + 1 (the upper
+  // half of the wave) on the odd ones; rows are 8-byte aligned
+  enum { BK = 32, LD = 34 };
   typedef float LT;
 };
 
@@ -110,8 +112,9 @@ __global__ void __launch_bounds__(256) gemm_kernel(GemmDesc g, int a_vec, int b_
   typedef typename TL::LT LT;
   constexpr int BK = TL::BK, LD = TL::LD;
   constexpr int CPT = BM * BK / 8 / 256;  // 8-element chunks per thread per operand tile
-  __shared__ __attribute__((aligned(16))) LT As[BM * LD];
-  __shared__ __attribute__((aligned(16))) LT Bs[BN * LD];
+  // two stages: the tile of step s + 1 is written while the MFMAs of step s read the other one
+  __shared__ __attribute__((aligned(16))) LT As2[2][BM * LD];
+  __shared__ __attribute__((aligned(16))) LT Bs2[2][BN * LD];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
@@ -168,8 +171,10 @@ __global__ void __launch_bounds__(256) gemm_kernel(GemmDesc g, int a_vec, int b_
         q.w = bf16_rne(v[6]) | (bf16_rne(v[7]) << 16);
         *(uint4 *)d = q;
       } else {
-        *(float4 *)d = make_float4(v[0], v[1], v[2], v[3]);
-        *(float4 *)(d + 4) = make_float4(v[4], v[5], v[6], v[7]);
+        *(float2 *)d = make_float2(v[0], v[1]);
+        *(float2 *)(d + 2) = make_float2(v[2], v[3]);
+        *(float2 *)(d + 4) = make_float2(v[4], v[5]);
+        *(float2 *)(d + 6) = make_float2(v[6], v[7]);
       }
     } else {
       const int kk = chunk / (rows_total / 8), rc = (chunk % (rows_total / 8)) * 8;
@@ -181,21 +186,30 @@ __global__ void __launch_bounds__(256) gemm_kernel(GemmDesc g, int a_vec, int b_
     }
   };
 
-  auto stash = [&]() {
+  auto stash = [&](int buf) {
 #pragma unroll
     for (int c = 0; c < CPT; ++c) {
-      put(As, ra[c], tid + c * 256, A_KC, BM);
-      put(Bs, rb[c], tid + c * 256, B_KC, BN);
+      put(As2[buf], ra[c], tid + c * 256, A_KC, BM);
+      put(Bs2[buf], rb[c], tid + c * 256, B_KC, BN);
     }
   };
 
+  // Step s: the registers hold tile s + 1 (asked for a whole step ago); it goes into the stage that step s - 1
+  // read - every wave is past that step's barrier -, tile s + 2 is asked for, and the MFMAs of step s run on the
+  // other stage with those loads and LDS writes under them.  One barrier per step.
   const uint32_t n_steps = (k_end - k_begin + BK - 1) / BK;
-  if (n_steps) fetch(k_begin);
+  if (n_steps) {
+    fetch(k_begin);
+    stash(0);
+    if (n_steps > 1) fetch(k_begin + BK);
+  }
+  __syncthreads();
   for (uint32_t s = 0; s < n_steps; ++s) {
-    __syncthreads();  // previous step's MFMA reads are done
-    stash();
-    __syncthreads();
-    if (s + 1 < n_steps) fetch(k_begin + (s + 1) * BK);
+    if (s + 1 < n_steps) {
+      stash((s + 1) & 1);
+      if (s + 2 < n_steps) fetch(k_begin + (s + 2) * BK);
+    }
+    const LT *As = As2[s & 1], *Bs = Bs2[s & 1];
     if (BF16) {
 #pragma unroll
       for (int kk = 0; kk < BK; kk += 16) {
@@ -227,6 +241,7 @@ __global__ void __launch_bounds__(256) gemm_kernel(GemmDesc g, int a_vec, int b_
             acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i], bfr[j], acc[i][j], 0, 0, 0);
       }
     }
+    __syncthreads();  // stage (s + 1) & 1 is complete, and every wave is done reading stage s & 1
   }
 
   // 32x32 accumulator layout: element e of a lane sits at
