@@ -694,7 +694,7 @@ int cg_slice(cg_backend *be, cg_tensor *x, size_t dim, size_t start, size_t len,
   for (size_t i = dim + 1; i < r; ++i) inner *= os[i];
   cg_tensor *t = make(x->dtype, os);
   for (size_t o = 0; o < outer; ++o)
-    if (len * inner)
+    if (len * inner != 0)
       std::memcpy(&t->bits[o * len * inner], &x->bits[(o * nd + start) * inner], len * inner * 4);
   *out = t;
   return CG_OK;
