@@ -2522,6 +2522,13 @@ static void launch_rowdot(const LaunchCtx &lc, const GemmDesc &g, int bv, int av
   if (blocks < 1) blocks = 1;
   dim3 grid(blocks, batch);
   if (ksplit) {
+    // Up to four rows (the shared expert's down_proj of a MoE decode step, 4 x 5632 x 2048): a wave reads its share of
+    // every input row from L2 once per column group - with one column in a group that is eight times the weights'
+    // bytes.  Two columns share it (10.7 us against 14.0; four columns 12.3, eight 16.2: too few workgroups).
+    if constexpr (MROWS == 4) {
+      CG_LAUNCH(lc, (gemv_rowdot_kernel<TB, 64, 4, 2, 4>), dim3((g.N + 1) / 2, batch), 256, g, bv, av);
+      return;
+    }
     CG_LAUNCH(lc, (gemv_rowdot_kernel<TB, 64, MROWS, R, 4>), grid, 256, g, bv, av);
     return;
   }
