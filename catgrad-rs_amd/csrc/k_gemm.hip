@@ -1661,19 +1661,20 @@ __device__ __forceinline__ void gemv_rows_mfma_body(const GemvProDesc &g, const 
   // Every request is UN loads, no fewer (pieces past the end of the wave's share repeat its last and are not
   // used), so the prologue's wait for its own, older loads is a count that leaves these in flight.
   VT q[UN];
-  auto request = [&](uint32_t group, uint32_t batch) {
+  auto request_window = [&](uint32_t group, uint32_t batch, int w2) {
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
       const uint32_t v = 2 * u + lrow;  // row of the operand
       const uint16_t *row;
       if (GLUEPI) row = u < 4 ? B + (int64_t)min(group * 8 + v, N - 1) * sbn : B2 + (int64_t)min(group * 8 + v - 8, N - 1) * sbn2;
       else row = B + (int64_t)min(group * 16 + v, N - 1) * sbn;
-#pragma unroll
-      for (int w2 = 0; w2 < 2; ++w2) {
-        const uint32_t kl = min((batch * 2 + w2) * 256 + lk, kw - 8);
-        q[w2 * 8 + u] = __builtin_nontemporal_load((const VT *)(row + k_begin + kl));
-      }
+      const uint32_t kl = min((batch * 2 + w2) * 256 + lk, kw - 8);
+      q[w2 * 8 + u] = __builtin_nontemporal_load((const VT *)(row + k_begin + kl));
     }
+  };
+  auto request = [&](uint32_t group, uint32_t batch) {
+    request_window(group, batch, 0);
+    request_window(group, batch, 1);
   };
   // Everything the prologue loads is used in straight-line code, down to the LDS store (pieces past the end of
   // a row or of the rows go to a spare location): a load whose only use sits inside a branch - gamma under
@@ -1774,12 +1775,6 @@ __device__ __forceinline__ void gemv_rows_mfma_body(const GemvProDesc &g, const 
   for (uint32_t group = first_group; group < groups; group += group_step) {
     f32x4n acc = {0.f, 0.f, 0.f, 0.f};
     for (uint32_t batch = 0; batch < nbatch; ++batch) {
-      VT cur[UN];
-#pragma unroll
-      for (int u = 0; u < UN; ++u) cur[u] = q[u];
-      // the next vectors - of this group, or the first of the workgroup's next group - while these multiply
-      if (batch + 1 < nbatch) request(group, batch + 1);
-      else if (group + group_step < groups) request(group + group_step, 0);
 #pragma unroll
       for (int w2 = 0; w2 < 2; ++w2) {
         const uint32_t wk = (batch * 2 + w2) * 256;  // where the window starts in the wave's share of k
@@ -1787,8 +1782,14 @@ __device__ __forceinline__ void gemv_rows_mfma_body(const GemvProDesc &g, const 
           // (LDS serves a wave's accesses in order: these stores follow the previous window's reads)
           __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
 #pragma unroll
-          for (int u = 0; u < 8; ++u) *(VT *)(mine + (2 * u + lrow) * GEMV_ROWS_TP + lk) = cur[w2 * 8 + u];
+          for (int u = 0; u < 8; ++u) *(VT *)(mine + (2 * u + lrow) * GEMV_ROWS_TP + lk) = q[w2 * 8 + u];
           __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        }
+        // The window's registers are free again: the same window of the next vectors - of this group, or the first
+        // of the workgroup's next group - is requested into them while this one multiplies.
+        if (batch + 1 < nbatch) request_window(group, batch + 1, w2);
+        else if (group + group_step < groups) request_window(group + group_step, 0, w2);
+        if (wk < kw) {
 #pragma unroll
           for (int s = 0; s < 8; ++s)
             if (wk + s * 32 < kw) {
@@ -1870,11 +1871,12 @@ static void launch_gemv_rows_mfma_as(const LaunchCtx &lc, const GemvProDesc &g, 
 static hipError_t launch_gemv_rows_mfma(const LaunchCtx &lc, const GemvProDesc &g, uint32_t max_n) {
   if (g.glu_epilogue) max_n = g.m.p[0].N;  // (further problems ride along as extra workgroups)
   const uint32_t groups = g.glu_epilogue ? (max_n + 7) / 8 : (max_n + 15) / 16;
-  // One workgroup per CU - the kernel's 270-280 registers per lane leave room for one wave per SIMD, so a larger
-  // grid only queues behind the first 256 workgroups and stages the rows again; a workgroup stages the rows once
-  // and walks its groups, the next group's vectors requested while the current ones multiply (with twice the
-  // workgroups: q/k/v of a four-row step 11.1 -> 9.5 us, gate * up 15.0 -> 13.2 us)
-  uint32_t cap = (uint32_t)lc.n_cus / (g.glu_epilogue ? 1 : g.m.n_prob);
+  // Two workgroups per CU is what the kernel's registers (under 256 per lane) and its 77 KB of LDS allow: a larger
+  // grid only queues behind the resident workgroups and stages the rows again.  A workgroup stages the rows once and
+  // walks its groups, the next group's vectors requested while the current ones multiply.  (While the kernel kept a
+  // register copy of the vectors in flight it held 270-280 registers, one workgroup per CU, and a grid sized for
+  // two cost q/k/v of a four-row step 11.1 us instead of 9.5; without the copy and with two resident: 8.7 us.)
+  uint32_t cap = (uint32_t)lc.n_cus * 2 / (g.glu_epilogue ? 1 : g.m.n_prob);
   if (!cap) cap = 1;
   const uint32_t blocks = groups < cap ? groups : cap;
   if (g.glu_epilogue) {
